@@ -1,0 +1,752 @@
+// CPU oracle for the quantized MoE expert-FFN path.
+//
+// THIS FILE IS TEST INFRASTRUCTURE. It restates, in plain scalar C++, the arithmetic of the
+// reference (GreatV/flyingfish) for the router, the expert SwiGLU FFN, the block-scaled linears
+// and the combine, so that the HIP kernels can be checked against it. Nothing in the shipped
+// library links, loads or calls it; only tests, the smoke check and the CPU-baseline leg of the
+// benchmark do.
+//
+// Every function cites the reference lines it follows (paths relative to the reference root).
+// Parity status per function group:
+//   * codecs, BF16 rounding, effective weights ............ pinned (exhaustive closed forms, spot values)
+//   * noaux / sigmoid / softmax top-k ...................... pinned (golden router vectors, brute force)
+//   * SwiGLU boundaries ..................................... pinned (golden BF16 bit patterns)
+//   * expert FFN on BF16 / per-channel FP8 weights .......... pinned (FP64 boundary oracle at 0 BF16 steps)
+//   * W8A8 quantizer + block dot ............................ pinned (FP64 gamma bound, wrong-cell mutant)
+//   * NVFP4 / BF16-scale skinny linear orders ............... pinned (closed-form dequant table, FP64 bound)
+//   * combine variants ...................................... pinned (order-spread constants of the fixture)
+//   * expert FFN composed over 128x128-f32 block scales or
+//     NVFP4 weights, grouped routing with n_group > 1,
+//     FP32-logit dot order, last-bit behaviour of expf ....... parity unpinned (no reference code or vectors)
+#include <cmath>
+#include <cstdint>
+#include <cstring>
+#include <algorithm>
+#include <vector>
+
+#define ORC_API extern "C" __attribute__((visibility("default")))
+
+namespace {
+
+inline uint32_t f2u(float f) { uint32_t u; std::memcpy(&u, &f, 4); return u; }
+inline float u2f(uint32_t u) { float f; std::memcpy(&f, &u, 4); return f; }
+
+// BF16 round-to-nearest-even; crate `half` 2.7.1 `bf16::from_f32`, restated by the reference in
+// src/cpu/expert_ffn.rs:1072-1080. NaN keeps its sign and gains the quiet bit.
+inline uint16_t bf16_rne(float f) {
+  uint32_t b = f2u(f);
+  if ((b & 0x7fffffffu) > 0x7f800000u) return uint16_t((b >> 16) | 0x40u);
+  b += 0x7fffu + ((b >> 16) & 1u);
+  return uint16_t(b >> 16);
+}
+inline float bf16_f32(uint16_t h) { return u2f(uint32_t(h) << 16); }
+inline float bround(float f) { return bf16_f32(bf16_rne(f)); }
+
+// src/fp8.rs:69-82
+inline float decode_e4m3(uint8_t code) {
+  const uint32_t sign = uint32_t(code & 0x80u) << 24;
+  const uint32_t mag = code & 0x7fu;
+  if (mag == 0x7fu) return u2f(sign | 0x7fc00000u);
+  const uint32_t e = mag >> 3, m = mag & 7u;
+  if (e == 0) return u2f(f2u(float(m) * (1.0f / 512.0f)) | sign);
+  return u2f(sign | ((e + 120u) << 23) | (m << 20));
+}
+
+// src/fp8.rs:85-121 (value already clamped to [-448, 448]).
+inline uint8_t encode_e4m3(float value) {
+  const uint32_t bits = f2u(value);
+  const uint8_t sign = uint8_t((bits >> 31) & 1u);
+  const uint32_t magnitude = bits & 0x7fffffffu;
+  if (magnitude == 0) return uint8_t(sign << 7);
+  const int exponent = int((magnitude >> 23) & 0xffu) - 127;
+  const uint32_t mantissa = magnitude & 0x7fffffu;
+  if (exponent < -6) {
+    const double scaled = double(std::fabs(value)) * 512.0;
+    uint64_t m = uint64_t(std::floor(scaled));
+    const double fraction = scaled - double(m);
+    if (fraction > 0.5 || (fraction == 0.5 && (m & 1u) == 1u)) m += 1;
+    if (m >= 8) return uint8_t((sign << 7) | 0x08u);
+    return uint8_t((sign << 7) | uint8_t(m));
+  }
+  int e = exponent + 7;
+  uint32_t m = mantissa >> 20;
+  const uint32_t rest = mantissa & 0xfffffu;
+  if (rest > 0x80000u || (rest == 0x80000u && (m & 1u) == 1u)) {
+    m += 1;
+    if (m == 8) { m = 0; e += 1; }
+  }
+  if (e > 15) return uint8_t((sign << 7) | 0x7eu);
+  // exponent field 15 with mantissa 7 is the NaN code; the reference clamps its input to 448
+  // (mantissa 6) before calling, so that pattern never forms.
+  return uint8_t((sign << 7) | (uint8_t(e) << 3) | uint8_t(m));
+}
+
+// src/fp8.rs:124-136; kernels/q38_contract.cuh:172-178 keeps the sign of zero.
+inline float decode_e2m1(uint8_t code) {
+  static const float mags[8] = {0.0f, 0.5f, 1.0f, 1.5f, 2.0f, 3.0f, 4.0f, 6.0f};
+  if ((code & 7u) == 0) return 0.0f;  // fp8.rs:126 returns +0 for both zero codes
+  return u2f(f2u(mags[code & 7u]) | (uint32_t(code & 8u) << 28));
+}
+
+// kernels/q38_contract.cuh:180-187
+inline uint8_t encode_e2m1(float value) {
+  const float m = std::fabs(value);
+  const uint8_t code = m <= 0.25f ? 0 : m < 0.75f ? 1 : m <= 1.25f ? 2 : m < 1.75f ? 3
+                     : m <= 2.5f ? 4 : m < 3.5f ? 5 : m <= 5.0f ? 6 : 7;
+  return uint8_t(code | uint8_t((f2u(value) >> 28) & 8u));
+}
+
+// ---------------------------------------------------------------------------------------------
+// expf / log1pf built from IEEE +,-,*,/ and fused multiply-add only, so that host and device
+// produce the same bits. The reference takes expf from libm (CPU) or the CUDA math library (GPU)
+// and pins neither; this oracle therefore fixes one definition and checks it to <= 2 ulp of the
+// exact function (see tests). Range reduction x = n ln2 + r, degree-5 polynomial in r for
+// (e^r - 1 - r)/r^2 (Cephes expf coefficients), two-step scaling so subnormal results round once.
+inline float det_expf(float x) {
+  if (x != x) return x;
+  if (!(x > -104.0f)) return 0.0f;
+  if (x > 88.72283935546875f) return u2f(0x7f800000u);
+  const float magic = 12582912.0f;  // 1.5 * 2^23: adding it rounds to the nearest integer
+  const float t = std::fmaf(x, 1.44269502162933349609375f, magic);
+  const float n = t - magic;
+  float r = std::fmaf(n, -0.693145751953125f, x);
+  r = std::fmaf(n, -1.428606765330187045037746429443359375e-06f, r);
+  float p = 1.9875691500e-4f;
+  p = std::fmaf(p, r, 1.3981999507e-3f);
+  p = std::fmaf(p, r, 8.3334519073e-3f);
+  p = std::fmaf(p, r, 4.1665795894e-2f);
+  p = std::fmaf(p, r, 1.6666665459e-1f);
+  p = std::fmaf(p, r, 5.0000001201e-1f);
+  const float r2 = r * r;
+  float y = std::fmaf(p, r2, r);
+  y = y + 1.0f;
+  const int ni = int(n);
+  const int a = ni >> 1, b = ni - a;
+  y = y * u2f(uint32_t(a + 127) << 23);
+  y = y * u2f(uint32_t(b + 127) << 23);
+  return y;
+}
+
+// log(1+u) for 0 <= u <= 1 (the only range sqrt-softplus needs): w = 1+u rounded, Cephes logf
+// polynomial on the reduced argument, then the first-order correction for the rounding of w.
+inline float det_log1pf_unit(float u) {
+  const float w = 1.0f + u;
+  if (w == 1.0f) return u;
+  float m = w;
+  float e = 0.0f;
+  if (m > 1.41421353816986083984375f) { m = m * 0.5f; e = 1.0f; }
+  const float f = m - 1.0f;
+  const float z = f * f;
+  float p = 7.0376836292e-2f;
+  p = std::fmaf(p, f, -1.1514610310e-1f);
+  p = std::fmaf(p, f, 1.1676998740e-1f);
+  p = std::fmaf(p, f, -1.2420140846e-1f);
+  p = std::fmaf(p, f, 1.4249322787e-1f);
+  p = std::fmaf(p, f, -1.6668057665e-1f);
+  p = std::fmaf(p, f, 2.0000714765e-1f);
+  p = std::fmaf(p, f, -2.4999993993e-1f);
+  p = std::fmaf(p, f, 3.3333331174e-1f);
+  float y = (f * z) * p;
+  y = std::fmaf(-0.5f, z, y);
+  float lg = f + y;
+  lg = std::fmaf(e, 0.693147182464599609375f, lg);
+  // log1p(u) = log(w) + (u - (w - 1)) / w
+  const float c = (u - (w - 1.0f)) / w;
+  return lg + c;
+}
+
+inline float sigmoid1(float l) { return 1.0f / (1.0f + det_expf(-l)); }  // moe_route.cu:255,330
+
+// moe_route.cu:332-335 (non-literal form) / moe/reference.rs:73-76
+inline float sqrt_softplus(float l) {
+  const float softplus = std::fmax(l, 0.0f) + det_log1pf_unit(det_expf(-std::fabs(l)));
+  return std::sqrt(softplus);
+}
+
+// ---------------------------------------------------------------------------------------------
+// reductions of src/cpu/expert_ffn.rs
+enum Form { LANE16 = 0, LANE8 = 1, F64 = 2 };
+
+// expert_ffn.rs:681-687
+inline float pairwise16(const float* l) {
+  const float low = ((l[0] + l[1]) + (l[2] + l[3])) + ((l[4] + l[5]) + (l[6] + l[7]));
+  const float high = ((l[8] + l[9]) + (l[10] + l[11])) + ((l[12] + l[13]) + (l[14] + l[15]));
+  return low + high;
+}
+// expert_ffn.rs:37-41
+inline float group_sum8(const float* l) {
+  return ((l[0] + l[4]) + (l[2] + l[6])) + ((l[1] + l[5]) + (l[3] + l[7]));
+}
+
+// expert_ffn.rs:689-732 (scalar_dot); weights are already BF16-rounded effective weights, which
+// makes scalar_dot_e4m3 (:734-776) the same function. F64 is the reference's test oracle
+// accumulation (:3290-3299): double sum in index order, one cast to f32.
+float dot_form(const float* x, const uint16_t* w, int n, int form) {
+  if (form == F64) {
+    double acc = 0.0;
+    for (int k = 0; k < n; ++k) acc += double(x[k]) * double(bf16_f32(w[k]));
+    return float(acc);
+  }
+  float lanes[16] = {0};
+  if (form == LANE16) {
+    int k = 0;
+    for (; k + 16 <= n; k += 16)
+      for (int l = 0; l < 16; ++l) lanes[l] = std::fmaf(x[k + l], bf16_f32(w[k + l]), lanes[l]);
+    for (; k < n; ++k) lanes[k % 16] = std::fmaf(x[k], bf16_f32(w[k]), lanes[k % 16]);
+    return pairwise16(lanes);
+  }
+  const int vectors = n / 8;
+  for (int v = 0; v < vectors; ++v) {
+    float inner = 0.0f;
+    for (int s = 0; s < 8; ++s) inner = std::fmaf(x[v * 8 + s], bf16_f32(w[v * 8 + s]), inner);
+    lanes[v % 8] += inner;
+  }
+  for (int k = vectors * 8; k < n; ++k) lanes[k % 8] = std::fmaf(x[k], bf16_f32(w[k]), lanes[k % 8]);
+  return group_sum8(lanes);
+}
+
+enum Swiglu { TWICE = 0, ONCE = 1, CLAMPED_TWICE = 2, CLAMPED_ONCE = 3 };
+enum Boundary { AFTER_DOWN_BF16 = 0, BEFORE_CONTRIBUTION_BF16 = 1 };
+
+// expert_ffn.rs:58-100 (silu_mul_value) followed by the BF16 store of :103-114.
+// silu_kind 0: g / (1 + exp(-g))      (Lane8, and Lane16 with Once; moe_ffn.cu:58)
+//           1: g * (1 / (1 + exp(-g))) (Lane16 with Twice; moe_ffn.cu:201-203)
+//           2: g * sigmoid2(g)         (two-branch sigmoid of q38_contract.cuh:17-21, act.cu:152-156)
+inline float silu_kind(float g, int kind) {
+  if (kind == 0) return g / (1.0f + det_expf(-g));
+  if (kind == 1) return g * (1.0f / (1.0f + det_expf(-g)));
+  float s;
+  if (g >= 0.0f) s = 1.0f / (1.0f + det_expf(-g));
+  else { const float e = det_expf(g); s = e / (1.0f + e); }
+  return g * s;
+}
+inline uint16_t silu_mul_bits(uint16_t gate, uint16_t up, int rounding, float limit, int kind) {
+  float g = bf16_f32(gate), u = bf16_f32(up);
+  if (rounding == CLAMPED_TWICE || rounding == CLAMPED_ONCE) {
+    g = std::fmin(g, limit);
+    u = std::fmin(std::fmax(u, -limit), limit);
+  }
+  const float act = silu_kind(g, kind);
+  const float prod = (rounding == TWICE || rounding == CLAMPED_TWICE) ? bround(act) * u : act * u;
+  return bf16_rne(prod);
+}
+
+// 32-lane shuffle-down tree (offsets 16,8,4,2,1): lane 0 ends with the full pairwise sum.
+inline float warp_tree32(float* v) {
+  for (int off = 16; off > 0; off >>= 1)
+    for (int l = 0; l + off < 32; ++l) v[l] = v[l] + v[l + off];  // ascending l reads unmodified v[l+off]
+  return v[0];
+}
+
+}  // namespace
+
+// =============================================================================================
+// codecs
+ORC_API float orc_decode_e4m3(uint8_t c) { return decode_e4m3(c); }
+ORC_API uint8_t orc_encode_e4m3(float v) { return encode_e4m3(v); }
+ORC_API float orc_decode_e2m1(uint8_t c) { return decode_e2m1(c); }
+ORC_API uint8_t orc_encode_e2m1(float v) { return encode_e2m1(v); }
+ORC_API uint16_t orc_bf16_rne(float v) { return bf16_rne(v); }
+ORC_API float orc_expf(float v) { return det_expf(v); }
+ORC_API float orc_log1pf_unit(float v) { return det_log1pf_unit(v); }
+ORC_API void orc_expf_array(const float* x, float* y, long n) { for (long i = 0; i < n; ++i) y[i] = det_expf(x[i]); }
+ORC_API void orc_bf16_rne_array(const float* x, uint16_t* y, long n) { for (long i = 0; i < n; ++i) y[i] = bf16_rne(x[i]); }
+
+// src/fp8.rs:138-140 with an f32 scale: bf16(decode(code) * scale).
+ORC_API uint16_t orc_effective_weight(uint8_t code, float scale) { return bf16_rne(decode_e4m3(code) * scale); }
+// src/fp8.rs:143-145: bf16(e2m1 * (e4m3(scale) * global)); kernels/nvfp4_linear.cu:12-14 zero rule.
+ORC_API uint16_t orc_nvfp4_effective_weight(uint8_t code, uint8_t scale_code, float global) {
+  return bf16_rne(decode_e2m1(code & 15u) * (decode_e4m3(scale_code) * global));
+}
+
+// Materialise BF16 effective weights of an [n,k] FP8 matrix with [ceil(n/bn), ceil(k/bk)] f32 scales
+// (scale geometry: src/fp8.rs:31-36).
+ORC_API void orc_dequant_fp8_block(const uint8_t* codes, const float* scales, int n, int k, int bn, int bk,
+                                   uint16_t* out) {
+  const int gk = (k + bk - 1) / bk;
+  for (int r = 0; r < n; ++r)
+    for (int c = 0; c < k; ++c)
+      out[size_t(r) * k + c] = bf16_rne(decode_e4m3(codes[size_t(r) * k + c]) * scales[size_t(r / bn) * gk + c / bk]);
+}
+// per-output-channel BF16 scales (src/cpu/expert_ffn.rs:542-545,734-737)
+ORC_API void orc_dequant_fp8_channel(const uint8_t* codes, const uint16_t* scales, int n, int k, uint16_t* out) {
+  for (int r = 0; r < n; ++r)
+    for (int c = 0; c < k; ++c)
+      out[size_t(r) * k + c] = bf16_rne(decode_e4m3(codes[size_t(r) * k + c]) * bf16_f32(scales[r]));
+}
+// kernels/nvfp4_linear.cu:17-47: low nibble = even column.
+ORC_API void orc_dequant_nvfp4(const uint8_t* codes, const uint8_t* scales, float global, int n, int k, uint16_t* out) {
+  for (int r = 0; r < n; ++r)
+    for (int c = 0; c < k; ++c) {
+      const uint8_t b = codes[size_t(r) * (k / 2) + c / 2];
+      const uint8_t nib = (c & 1) ? uint8_t(b >> 4) : uint8_t(b & 15u);
+      const float s = decode_e4m3(scales[size_t(r) * (k / 16) + c / 16]) * global;
+      out[size_t(r) * k + c] = bf16_rne(decode_e2m1(nib) * s);
+    }
+}
+
+// =============================================================================================
+// quantizers for synthetic weights (absmax block scales; the layout rules are the reference's,
+// the recipe is the benchmark's: s = amax/448 per 128x128 block, code = encode(clamp(w/s))).
+ORC_API void orc_quant_weight_fp8_block(const float* w, int n, int k, int bn, int bk, uint8_t* codes, float* scales) {
+  const int gn = (n + bn - 1) / bn, gk = (k + bk - 1) / bk;
+  for (int br = 0; br < gn; ++br)
+    for (int bc = 0; bc < gk; ++bc) {
+      float amax = 0.0f;
+      for (int r = br * bn; r < std::min(n, (br + 1) * bn); ++r)
+        for (int c = bc * bk; c < std::min(k, (bc + 1) * bk); ++c) amax = std::fmax(amax, std::fabs(w[size_t(r) * k + c]));
+      const float s = amax * (1.0f / 448.0f);
+      scales[size_t(br) * gk + bc] = s;
+      const float d = std::fmax(s, 1.0e-12f);
+      for (int r = br * bn; r < std::min(n, (br + 1) * bn); ++r)
+        for (int c = bc * bk; c < std::min(k, (bc + 1) * bk); ++c)
+          codes[size_t(r) * k + c] = encode_e4m3(std::fmin(448.0f, std::fmax(-448.0f, w[size_t(r) * k + c] / d)));
+    }
+}
+
+// NVFP4: s16 = amax16/6, global = max(s16)/448, stored scale = e4m3(s16/global) floored at code 1
+// (kernels/q38_contract.cuh:207-209), code = e2m1(w / (e4m3(scale) * global)) (:180-187).
+ORC_API void orc_quant_weight_nvfp4(const float* w, int n, int k, uint8_t* codes, uint8_t* scales, float* global_out) {
+  float smax = 0.0f;
+  const int g = k / 16;
+  std::vector<float> s16(size_t(n) * g);
+  for (int r = 0; r < n; ++r)
+    for (int j = 0; j < g; ++j) {
+      float amax = 0.0f;
+      for (int c = 0; c < 16; ++c) amax = std::fmax(amax, std::fabs(w[size_t(r) * k + j * 16 + c]));
+      s16[size_t(r) * g + j] = amax / 6.0f;
+      smax = std::fmax(smax, amax / 6.0f);
+    }
+  float global = smax / 448.0f;
+  if (!(global > 0.0f)) global = 1.0f;
+  *global_out = global;
+  for (int r = 0; r < n; ++r)
+    for (int j = 0; j < g; ++j) {
+      uint8_t sc = encode_e4m3(std::fmin(448.0f, s16[size_t(r) * g + j] / global));
+      if (sc == 0) sc = 1;
+      scales[size_t(r) * g + j] = sc;
+      const float s = decode_e4m3(sc) * global;
+      for (int c = 0; c < 16; c += 2) {
+        const uint8_t lo = encode_e2m1(w[size_t(r) * k + j * 16 + c] / s);
+        const uint8_t hi = encode_e2m1(w[size_t(r) * k + j * 16 + c + 1] / s);
+        codes[size_t(r) * (k / 2) + (j * 16 + c) / 2] = uint8_t(lo | (hi << 4));
+      }
+    }
+}
+
+// kernels/fp8_linear.cu:12-48 (fp8_quant_f32_128): per (row, 128-group) scale = amax * (1/448) as
+// an f32 multiply, divisor max(scale, 1e-12), code = encode(clamp(x / divisor, +-448)).
+ORC_API void orc_quant_act_fp8_128(const uint16_t* x, int m, int k, uint8_t* codes, float* scales) {
+  const int groups = (k + 127) / 128;
+  for (int r = 0; r < m; ++r)
+    for (int g = 0; g < groups; ++g) {
+      float amax = 0.0f;
+      const int end = std::min(k, (g + 1) * 128);
+      for (int c = g * 128; c < end; ++c) amax = std::fmax(amax, std::fabs(bf16_f32(x[size_t(r) * k + c])));
+      const float scale = amax * (1.0f / 448.0f);
+      scales[size_t(r) * groups + g] = scale;
+      const float divisor = std::fmax(scale, 1.0e-12f);
+      for (int c = g * 128; c < end; ++c)
+        codes[size_t(r) * k + c] = encode_e4m3(std::fmin(448.0f, std::fmax(-448.0f, bf16_f32(x[size_t(r) * k + c]) / divisor)));
+    }
+}
+
+// =============================================================================================
+// router
+// kernels/moe_route.cu:392-403,496-560: one ascending FP32 fma chain per (row, expert), BF16 store.
+ORC_API void orc_route_logits_bf16(const uint16_t* x, const uint16_t* w, uint16_t* logits, int rows, int experts, int hidden) {
+  for (int r = 0; r < rows; ++r)
+    for (int e = 0; e < experts; ++e) {
+      float acc = 0.0f;
+      for (int k = 0; k < hidden; ++k) acc = std::fmaf(bf16_f32(x[size_t(r) * hidden + k]), bf16_f32(w[size_t(e) * hidden + k]), acc);
+      logits[size_t(r) * experts + e] = bf16_rne(acc);
+    }
+}
+
+// FP32 logits. The reference takes these from a BLAS GEMM whose summation order is undefined
+// (src/backend/cuda/moe/route.rs:505-562), so any order is within its contract; the order fixed
+// here is the one the HIP kernel uses, so ids can be compared bit for bit: 64 lanes, lane L owns
+// the 8-element vectors v = L, L+64, ... and chains fma over them in ascending order; the lane
+// partials are summed by a shuffle-down tree with offsets 32,16,8,4,2,1. PARITY UNPINNED at bit
+// level (tolerance-checked against float64 in the tests, as the reference's own tests do).
+ORC_API void orc_route_logits_f32(const uint16_t* x, const uint16_t* w, float* logits, int rows, int experts, int hidden) {
+  const int vectors = hidden / 8;
+  for (int r = 0; r < rows; ++r)
+    for (int e = 0; e < experts; ++e) {
+      float lanes[64];
+      for (int l = 0; l < 64; ++l) {
+        float acc = 0.0f;
+        for (int v = l; v < vectors; v += 64)
+          for (int s = 0; s < 8; ++s)
+            acc = std::fmaf(bf16_f32(x[size_t(r) * hidden + v * 8 + s]), bf16_f32(w[size_t(e) * hidden + v * 8 + s]), acc);
+        lanes[l] = acc;
+      }
+      for (int off = 32; off > 0; off >>= 1)
+        for (int l = 0; l + off < 64; ++l) lanes[l] = lanes[l] + lanes[l + off];
+      logits[size_t(r) * experts + e] = lanes[0];
+    }
+}
+
+namespace {
+// K rounds of arg-max under (score desc, id asc) over not-yet-taken experts
+// (kernels/moe_route.cu:205-235); returns ids in selection order.
+void select_topk(const float* score, const bool* allowed, int experts, int top_k, int* out) {
+  std::vector<char> taken(experts, 0);
+  for (int r = 0; r < top_k; ++r) {
+    int best = -1;
+    for (int e = 0; e < experts; ++e) {
+      if (taken[e] || (allowed && !allowed[e])) continue;
+      if (best < 0 || score[e] > score[best]) best = e;  // strict > keeps the lower id on ties
+    }
+    out[r] = best;
+    if (best >= 0) taken[best] = 1;
+  }
+}
+}  // namespace
+
+// kernels/moe_route.cu:154-242 (moe_route_select): FP32 softmax over BF16 logits with the max and
+// the sum taken by 32-lane shuffle-down trees per warp and again over the per-warp partials;
+// weights = p / (sum of selected p in selection order), BF16 store.
+ORC_API void orc_route_topk_softmax(const uint16_t* logits, int* ids, uint16_t* weights, int rows, int experts, int top_k) {
+  const int nthr = (experts + 31) & ~31, nw = nthr / 32;
+  std::vector<float> ev(nthr), prob(experts);
+  for (int r = 0; r < rows; ++r) {
+    float mx = -INFINITY;
+    for (int e = 0; e < experts; ++e) mx = std::fmax(mx, bf16_f32(logits[size_t(r) * experts + e]));
+    for (int e = 0; e < nthr; ++e) ev[e] = e < experts ? det_expf(bf16_f32(logits[size_t(r) * experts + e]) - mx) : 0.0f;
+    float partial[32];
+    for (int w = 0; w < 32; ++w) partial[w] = 0.0f;
+    for (int w = 0; w < nw; ++w) {
+      float lanes[32];
+      for (int l = 0; l < 32; ++l) lanes[l] = ev[w * 32 + l];
+      partial[w] = warp_tree32(lanes);
+    }
+    const float sum = warp_tree32(partial);
+    for (int e = 0; e < experts; ++e) prob[e] = ev[e] / sum;
+    std::vector<int> sel(top_k);
+    select_topk(prob.data(), nullptr, experts, top_k, sel.data());
+    float tsum = 0.0f;
+    for (int j = 0; j < top_k; ++j) tsum += prob[sel[j]];
+    for (int j = 0; j < top_k; ++j) {
+      ids[size_t(r) * top_k + j] = sel[j];
+      weights[size_t(r) * top_k + j] = bf16_rne(prob[sel[j]] / tsum);
+    }
+  }
+}
+
+// kernels/moe_route.cu:244-301 (moe_route_select_sigmoid)
+ORC_API void orc_route_topk_sigmoid(const uint16_t* logits, int* ids, uint16_t* weights, int rows, int experts, int top_k) {
+  std::vector<float> score(experts);
+  std::vector<int> sel(top_k);
+  for (int r = 0; r < rows; ++r) {
+    for (int e = 0; e < experts; ++e) score[e] = sigmoid1(bf16_f32(logits[size_t(r) * experts + e]));
+    select_topk(score.data(), nullptr, experts, top_k, sel.data());
+    float tsum = 0.0f;
+    for (int j = 0; j < top_k; ++j) tsum += score[sel[j]];
+    for (int j = 0; j < top_k; ++j) {
+      ids[size_t(r) * top_k + j] = sel[j];
+      weights[size_t(r) * top_k + j] = bf16_rne(score[sel[j]] / (tsum + 1.0e-20f));
+    }
+  }
+}
+
+// kernels/moe_route.cu:315-390 (moe_route_select_noaux) and its host twin
+// src/backend/cuda/moe/reference.rs:79-131: select on score+bias, weight = score / (sum + 1e-20) *
+// routed_scaling with the sum accumulated in selection order. score_mode 0 sigmoid, 1 sqrt-softplus.
+// n_group > 1 adds the DeepSeek-V3 group filter, which the reference does not implement
+// (src/model_spec.rs:3832-3841 requires n_group == topk_group == 1): group score = sum of the two
+// largest score+bias values of the group, keep the topk_group best groups under (score desc,
+// group id asc), drop the other experts. PARITY UNPINNED for n_group > 1; n_group == 1 is the
+// reference path exactly.
+ORC_API void orc_route_topk_noaux(const float* logits, const float* bias, int* ids, float* weights, int rows, int experts,
+                                  int top_k, int score_mode, float routed_scaling, int n_group, int topk_group) {
+  std::vector<float> score(experts), sel_score(experts);
+  std::vector<int> sel(top_k);
+  std::vector<char> allowed_c(experts);
+  for (int r = 0; r < rows; ++r) {
+    for (int e = 0; e < experts; ++e) {
+      const float l = logits[size_t(r) * experts + e];
+      score[e] = score_mode == 0 ? sigmoid1(l) : sqrt_softplus(l);
+      sel_score[e] = score[e] + (bias ? bias[size_t(r) * experts + e] : 0.0f);
+    }
+    const bool* allowed = nullptr;
+    std::vector<char> keep;
+    if (n_group > 1) {
+      const int per = experts / n_group;
+      std::vector<float> gscore(n_group);
+      for (int g = 0; g < n_group; ++g) {
+        float a = -INFINITY, b = -INFINITY;  // largest, second largest
+        for (int e = g * per; e < (g + 1) * per; ++e) {
+          const float v = sel_score[e];
+          if (v > a) { b = a; a = v; } else if (v > b) { b = v; }
+        }
+        gscore[g] = a + b;
+      }
+      std::vector<int> gsel(topk_group);
+      select_topk(gscore.data(), nullptr, n_group, topk_group, gsel.data());
+      std::fill(allowed_c.begin(), allowed_c.end(), 0);
+      for (int j = 0; j < topk_group; ++j)
+        for (int e = gsel[j] * per; e < (gsel[j] + 1) * per; ++e) allowed_c[e] = 1;
+      allowed = reinterpret_cast<const bool*>(allowed_c.data());
+    }
+    select_topk(sel_score.data(), allowed, experts, top_k, sel.data());
+    float tsum = 0.0f;
+    for (int j = 0; j < top_k; ++j) tsum += score[sel[j]];
+    for (int j = 0; j < top_k; ++j) {
+      ids[size_t(r) * top_k + j] = sel[j];
+      weights[size_t(r) * top_k + j] = (score[sel[j]] / (tsum + 1.0e-20f)) * routed_scaling;
+    }
+  }
+}
+
+// Plain descending top-k with lower-id tie break (src/backend/cuda/moe/reference.rs:35-71).
+ORC_API void orc_topk_ids(const float* scores, int n, int k, int* ids) { select_topk(scores, nullptr, n, k, ids); }
+
+// =============================================================================================
+// SwiGLU boundary (expert_ffn.rs:58-114; act.cu:24-159)
+ORC_API uint16_t orc_silu_mul(uint16_t gate, uint16_t up, int rounding, float limit, int kind) {
+  return silu_mul_bits(gate, up, rounding, limit, kind);
+}
+ORC_API void orc_silu_mul_array(const uint16_t* gate, const uint16_t* up, uint16_t* out, long n, int rounding, float limit, int kind) {
+  for (long i = 0; i < n; ++i) out[i] = silu_mul_bits(gate[i], up[i], rounding, limit, kind);
+}
+
+ORC_API float orc_dot(const float* x, const uint16_t* w, int n, int form) { return dot_form(x, w, n, form); }
+
+// One (row, choice) contribution over BF16 effective weights: src/cpu/expert_ffn.rs:431-497
+// (compute) and :592-679 (compute_fp8, identical once weights are BF16-rounded effective weights).
+// form F64 restates the reference's own test oracle (:3281-3320, :3725-3790): FP64 accumulation,
+// SiLU in FP64 as g * (1/(1+exp(-g))), the same BF16 boundaries.
+// gate/up [I,H], down [H,I] row-major BF16; act_out (optional) receives the BF16 activation [I];
+// apply_weight 0 leaves the down output as bf16(d) (shared expert, moe_ffn.cu:300).
+ORC_API void orc_expert_ffn(const uint16_t* x, const uint16_t* gate, const uint16_t* up, const uint16_t* down, int H, int I,
+                            float routing, int rounding, float limit, int boundary, int form, int silu_k, int apply_weight,
+                            uint16_t* out, uint16_t* act_out) {
+  std::vector<float> xf(H), af(I);
+  for (int k = 0; k < H; ++k) xf[k] = bf16_f32(x[k]);
+  for (int j = 0; j < I; ++j) {
+    const uint16_t g = bf16_rne(dot_form(xf.data(), gate + size_t(j) * H, H, form));
+    const uint16_t u = bf16_rne(dot_form(xf.data(), up + size_t(j) * H, H, form));
+    uint16_t a;
+    if (form == F64) {
+      const double gd = double(bf16_f32(g)), ud = double(bf16_f32(u));
+      const double silu = double(bround(float(gd * (1.0 / (1.0 + std::exp(-gd))))));
+      a = bf16_rne(float(silu * ud));
+    } else {
+      a = silu_mul_bits(g, u, rounding, limit, silu_k);
+    }
+    af[j] = bf16_f32(a);
+    if (act_out) act_out[j] = a;
+  }
+  for (int d = 0; d < H; ++d) {
+    const float lin = dot_form(af.data(), down + size_t(d) * I, I, form);
+    float v;
+    if (!apply_weight) v = bround(lin);
+    else if (boundary == AFTER_DOWN_BF16) v = bround(lin) * routing;
+    else v = lin * routing;
+    out[d] = bf16_rne(v);
+  }
+}
+
+// =============================================================================================
+// W8A8 block linear: kernels/q38_contract.cuh:239-279 (fp8_block_decode<float,128>): per output
+// and per 128-group, lane L of 32 chains fma over elements L, L+32, L+64, L+96, a shuffle-down
+// tree 16..1 gives the group sum, then total = fma(sum, sw*sx, total); BF16 store.
+// order 1 = FP64 reference (src/backend/cuda/linear.rs:2105-2142) rounded f64 -> f32 -> bf16.
+ORC_API void orc_linear_fp8_block_w8a8(const uint8_t* w, const float* sw, const uint8_t* xq, const float* sx, int m, int n,
+                                       int k, int order, uint16_t* y, float* y_f32) {
+  const int groups = (k + 127) / 128;
+  for (int r = 0; r < m; ++r)
+    for (int c = 0; c < n; ++c) {
+      float result;
+      if (order == 1) {
+        double sum = 0.0;
+        for (int i = 0; i < k; ++i)
+          sum += (double(decode_e4m3(w[size_t(c) * k + i])) * double(sw[size_t(c / 128) * groups + i / 128])) *
+                 (double(decode_e4m3(xq[size_t(r) * k + i])) * double(sx[size_t(r) * groups + i / 128]));
+        result = float(sum);
+      } else {
+        float total = 0.0f;
+        for (int g = 0; g < groups; ++g) {
+          float lanes[32];
+          for (int l = 0; l < 32; ++l) {
+            float s = 0.0f;
+            for (int off = l; off < 128; off += 32) {
+              const int i = g * 128 + off;
+              if (i < k) s = std::fmaf(decode_e4m3(w[size_t(c) * k + i]), decode_e4m3(xq[size_t(r) * k + i]), s);
+            }
+            lanes[l] = s;
+          }
+          const float sum = warp_tree32(lanes);
+          const float scale = sw[size_t(c / 128) * groups + g] * sx[size_t(r) * groups + g];
+          total = std::fmaf(sum, scale, total);
+        }
+        result = total;
+      }
+      if (y) y[size_t(r) * n + c] = bf16_rne(result);
+      if (y_f32) y_f32[size_t(r) * n + c] = result;
+    }
+}
+
+// W8A16 skinny linear with the reduction of src/fp8.rs:245-287 (host mirror of
+// kernels/fp8_linear.cu:407-487) over BF16 effective weights [n,k]; the NVFP4 twin is
+// src/fp8.rs:290-340 (kernels/nvfp4_linear.cu:50-229). kind 0 = FP8 order, 1 = NVFP4 order,
+// 2 = FP64 accumulate.
+ORC_API void orc_linear_skinny(const uint16_t* weight, const uint16_t* x, int m, int n, int k, int kind, uint16_t* y) {
+  for (int r = 0; r < m; ++r) {
+    const uint16_t* in = x + size_t(r) * k;
+    for (int c = 0; c < n; ++c) {
+      const uint16_t* row = weight + size_t(c) * k;
+      if (kind == 2) {
+        double acc = 0.0;
+        for (int i = 0; i < k; ++i) acc += double(bf16_f32(row[i])) * double(bf16_f32(in[i]));
+        y[size_t(r) * n + c] = bf16_rne(float(acc));
+        continue;
+      }
+      float lanes[32];
+      for (int lane = 0; lane < 32; ++lane) {
+        float sums[4] = {0, 0, 0, 0};
+        if (k % 1024 == 0) {
+          for (int base = 0; base < k; base += 1024) {
+            if (kind == 0) {
+              for (int word = 0; word < 4; ++word)
+                for (int byte = 0; byte < 4; ++byte) {
+                  int col = base + lane * 16 + word * 4 + byte;
+                  sums[byte] = std::fmaf(bf16_f32(row[col]), bf16_f32(in[col]), sums[byte]);
+                  col += 512;
+                  const int idx = (byte + 2) & 3;
+                  sums[idx] = std::fmaf(bf16_f32(row[col]), bf16_f32(in[col]), sums[idx]);
+                }
+            } else {
+              const int col = base + lane * 32;
+              for (int word = 0; word < 4; ++word)
+                for (int byte = 0; byte < 4; ++byte) {
+                  const int lo = col + 8 * word + 2 * byte, hi = lo + 1;
+                  const float acc = std::fmaf(bf16_f32(row[lo]), bf16_f32(in[lo]), sums[byte]);
+                  sums[byte] = std::fmaf(bf16_f32(row[hi]), bf16_f32(in[hi]), acc);
+                }
+            }
+          }
+        } else if (kind == 0) {
+          for (int col = lane; col < k; col += 32) sums[0] = std::fmaf(bf16_f32(row[col]), bf16_f32(in[col]), sums[0]);
+        } else {
+          for (int pair = lane; pair < k / 2; pair += 32) {
+            const int lo = 2 * pair, hi = lo + 1;
+            const float acc = std::fmaf(bf16_f32(row[lo]), bf16_f32(in[lo]), sums[0]);
+            sums[0] = std::fmaf(bf16_f32(row[hi]), bf16_f32(in[hi]), acc);
+          }
+        }
+        lanes[lane] = (sums[0] + sums[1]) + (sums[2] + sums[3]);
+      }
+      y[size_t(r) * n + c] = bf16_rne(warp_tree32(lanes));
+    }
+  }
+}
+
+// =============================================================================================
+// combine (kernels/moe_combine.cu)
+namespace {
+// moe_combine.cu:51-69: stable insertion sort of the active choices by ascending expert id.
+int order_row(const int* ids, const uint32_t* active, int a0, int top_k, int* order) {
+  int live = 0;
+  for (int c = 0; c < top_k; ++c) {
+    if (active && active[a0 + c] == 0u) continue;
+    int p = live;
+    while (p > 0 && ids[a0 + order[p - 1]] > ids[a0 + c]) { order[p] = order[p - 1]; --p; }
+    order[p] = c;
+    ++live;
+  }
+  return live;
+}
+}  // namespace
+
+// moe_combine.cu:21-49: scale[r] = bf16(sigmoid(bf16(dot))) with the dot strided over 256 threads,
+// products added (not fused), 32-lane trees per warp then over the 8 warp partials.
+ORC_API void orc_shared_scale(const uint16_t* x, const uint16_t* seg, uint16_t* scale, int rows, int hidden) {
+  for (int r = 0; r < rows; ++r) {
+    float part[256];
+    for (int t = 0; t < 256; ++t) {
+      float p = 0.0f;
+      for (int c = t; c < hidden; c += 256) p += bf16_f32(x[size_t(r) * hidden + c]) * bf16_f32(seg[c]);
+      part[t] = p;
+    }
+    float red[32];
+    for (int w = 0; w < 32; ++w) red[w] = 0.0f;
+    for (int w = 0; w < 8; ++w) red[w] = warp_tree32(part + w * 32);
+    const float v = warp_tree32(red);
+    scale[r] = bf16_rne(1.0f / (1.0f + det_expf(-bround(v))));
+  }
+}
+
+// mode 0: moe_combine (:71-93) FP32 sum ascending id -> bf16, + bf16(scale*shared) in BF16
+// mode 1: moe_combine_ungated (:95-116) same, + shared in BF16
+// mode 2: moe_combine_bf16 (:592-613) BF16 running sum ascending id, + shared in BF16
+// mode 3: moe_combine_accum fp32_accum=1 (:541-591) choice order, shared added in FP32, one round
+// mode 4: moe_combine_accum fp32_accum=0: choice order FP32 -> bf16, + shared -> bf16
+// mode 5: moe_combine_routed (:176-196) FP32 sum ascending id -> bf16, no shared
+// mode 6: descending-id BF16 running sum + gated shared (reference.rs:559-573, order-noise control)
+// mode 7: ascending-id BF16 running sum + gated shared (reference.rs:559-573 AscendingBf16)
+ORC_API void orc_combine(const uint16_t* contributions, const uint16_t* shared, const uint16_t* scale, const int* ids,
+                         const uint32_t* active, uint16_t* y, int rows, int top_k, int hidden, int mode) {
+  std::vector<int> order(top_k);
+  for (int r = 0; r < rows; ++r) {
+    const int a0 = r * top_k;
+    int live;
+    if (mode == 3 || mode == 4) { live = top_k; for (int c = 0; c < top_k; ++c) order[c] = c; }
+    else live = order_row(ids, active, a0, top_k, order.data());
+    if (mode == 6) std::reverse(order.begin(), order.begin() + live);
+    for (int d = 0; d < hidden; ++d) {
+      const float sh = shared ? bf16_f32(shared[size_t(r) * hidden + d]) : 0.0f;
+      auto c = [&](int k) { return bf16_f32(contributions[(size_t(a0) + order[k]) * hidden + d]); };
+      float out;
+      if (mode == 2 || mode == 6 || mode == 7) {
+        float acc = 0.0f;
+        for (int k = 0; k < live; ++k) acc = bround(acc + c(k));
+        const float add = mode == 2 ? sh : bround(bf16_f32(scale[r]) * sh);
+        out = bround(acc + add);
+      } else {
+        float acc = 0.0f;
+        for (int k = 0; k < live; ++k) acc += c(k);
+        if (mode == 0) out = bround(bround(acc) + bround(bf16_f32(scale[r]) * sh));
+        else if (mode == 1 || mode == 4) out = bround(bround(acc) + sh);
+        else if (mode == 3) out = bround(acc + sh);
+        else out = bround(acc);
+      }
+      y[size_t(r) * hidden + d] = bf16_rne(out);
+    }
+  }
+}
+
+// kernels/moe_ffn.cu:894-908 (moe_ffn_weight_f32): contrib = bf16(float(down_bf16) * w_f32)
+ORC_API void orc_weight_f32(const uint16_t* down, const float* w, uint16_t* contrib, int assignments, int hidden) {
+  for (int a = 0; a < assignments; ++a)
+    for (int d = 0; d < hidden; ++d) contrib[size_t(a) * hidden + d] = bf16_rne(bf16_f32(down[size_t(a) * hidden + d]) * w[a]);
+}
+
+// =============================================================================================
+// reference fixture generator (src/backend/cuda/moe/reference.rs:204-224)
+namespace {
+uint64_t mix(uint64_t salt, uint64_t a, uint64_t b, uint64_t c) {
+  uint64_t z = salt + a * 0x9E3779B1ull + b * 0x85EBCA77ull + c * 0xC2B2AE3Dull;
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  return z ^ (z >> 31);
+}
+}  // namespace
+ORC_API float orc_fixture_unit(uint64_t salt, uint64_t a, uint64_t b, uint64_t c) {
+  return float(mix(salt, a, b, c) >> 40) / 8388608.0f - 1.0f;
+}
+ORC_API uint64_t orc_fixture_seed(uint32_t variant, uint64_t slot) {
+  return uint64_t(variant) * 0x9E3779B97F4A7C15ull ^ slot * 0xC2B2AE3D27D4EB4Full;
+}
+// out[i0*n1*n2 + i1*n2 + i2] = bf16(unit(salt, a0+i0, i1, i2) * scale)
+ORC_API void orc_fixture_fill(uint64_t salt, uint64_t a0, int n0, int n1, int n2, float scale, uint16_t* out) {
+  for (int i0 = 0; i0 < n0; ++i0)
+    for (int i1 = 0; i1 < n1; ++i1)
+      for (int i2 = 0; i2 < n2; ++i2)
+        out[(size_t(i0) * n1 + i1) * n2 + i2] = bf16_rne(orc_fixture_unit(salt, a0 + i0, i1, i2) * scale);
+}
+// sine fixture of src/cpu/expert_ffn.rs:3077-3079
+ORC_API void orc_pattern_fill(uint64_t seed0, double phase, long n, uint16_t* out) {
+  for (long i = 0; i < n; ++i) out[i] = bf16_rne(float(std::sin(double(seed0 + uint64_t(i)) * 0.6180339887498949 + phase) * 0.75));
+}

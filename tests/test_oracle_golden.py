@@ -1,0 +1,604 @@
+"""Pins the CPU oracle against the reference's own golden vectors, known-answer values and the
+closed forms / invariants its unit tests assert. No GPU, no product code."""
+import json
+import math
+import os
+
+import numpy as np
+import pytest
+
+import oracle as orc
+
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden", "shared-ops.json")
+
+
+@pytest.fixture(scope="module")
+def shared_ops():
+    with open(GOLDEN) as f:
+        return json.load(f)
+
+
+def f32(x):
+    return np.float32(x)
+
+
+# ------------------------------------------------------------------------------------------------
+# codecs
+def test_e4m3_decode_closed_form_all_codes():
+    # src/fp8.rs:69-82: bias 7, subnormal m/512, max 448, 0x7f/0xff NaN, no infinity
+    L = orc.lib()
+    for code in range(256):
+        v = L.orc_decode_e4m3(code)
+        mag = code & 0x7F
+        if mag == 0x7F:
+            assert math.isnan(v)
+            continue
+        e, m = mag >> 3, mag & 7
+        want = (m / 512.0) if e == 0 else (1 + m / 8.0) * 2.0 ** (e - 7)
+        if code & 0x80:
+            want = -want
+        assert v == want and math.copysign(1, v) == (-1 if code & 0x80 else 1), code
+    assert L.orc_decode_e4m3(0x7E) == 448.0 and L.orc_decode_e4m3(0x08) == 2.0 ** -6
+
+
+def test_e4m3_encode_spot_values_and_round_trip():
+    # src/backend/cuda/moe/decode_tests.rs:52-66
+    L = orc.lib()
+    cases = [(0.0, 0x00), (448.0, 0x7E), (449.0, 0x7E), (1.5 * 2.0 ** -9, 0x02), (2.5 * 2.0 ** -9, 0x02),
+             (1.1875, 0x3A), (-0.0, 0x80), (-448.0, 0xFE)]
+    for value, code in cases:
+        assert L.orc_encode_e4m3(value) == code, value
+    for code in range(256):
+        if code & 0x7F == 0x7F:
+            continue
+        assert L.orc_encode_e4m3(L.orc_decode_e4m3(code)) == code
+    # round to nearest even between every adjacent pair of positive codes
+    for code in range(0, 0x7E):
+        lo, hi = L.orc_decode_e4m3(code), L.orc_decode_e4m3(code + 1)
+        mid = (lo + hi) / 2
+        assert L.orc_encode_e4m3(mid) == (code if code % 2 == 0 else code + 1)
+        assert L.orc_encode_e4m3(np.nextafter(f32(mid), f32(0))) == code
+        assert L.orc_encode_e4m3(np.nextafter(f32(mid), f32(1e9))) == code + 1
+
+
+def test_e4m3_encode_is_nearest_grid_point_random():
+    L = orc.lib()
+    rng = np.random.default_rng(7)
+    grid = np.array([L.orc_decode_e4m3(c) for c in range(0x7F)], dtype=np.float64)
+    vals = np.concatenate([rng.uniform(-448, 448, 4000), rng.normal(0, 1, 4000), rng.normal(0, 0.01, 4000)]).astype(np.float32)
+    for v in vals:
+        c = L.orc_encode_e4m3(float(v))
+        d = np.abs(grid - abs(float(v)))
+        assert abs(L.orc_decode_e4m3(c & 0x7F) - abs(float(v))) <= d.min() + 0.0
+        assert (c >> 7) == (1 if np.signbit(v) else 0)
+
+
+def test_effective_weight_rounds_to_bf16_before_the_dot():
+    # src/cpu/expert_ffn.rs:3703-3709
+    L = orc.lib()
+    scale = 1.0078125
+    product = f32(L.orc_decode_e4m3(0x3F)) * f32(scale)
+    assert product == f32(1.8896484)
+    w = orc.bf16_to_f32(np.array([L.orc_effective_weight(0x3F, scale)], dtype=np.uint16))[0]
+    assert w == f32(1.890625) and w != product
+
+
+def test_nvfp4_e2m1_and_effective_weight_contract():
+    # src/fp8.rs:347-375 (exhaustive): both zero codes decode to +0, sign preserved otherwise
+    L = orc.lib()
+    mags = [0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0]
+    for code in range(16):
+        mag = mags[code & 7]
+        v = L.orc_decode_e2m1(code)
+        want = mag if (mag == 0.0 or not code & 8) else -mag
+        assert v == want and (mag != 0.0 or math.copysign(1, v) == 1)
+        assert L.orc_decode_e2m1(code | 0xF0) == v
+        for s_code in range(256):
+            bs = L.orc_decode_e4m3(s_code)
+            if math.isnan(bs):
+                continue
+            for g in [0.0, 1.0, 0.0029296875, 0.013183594]:
+                want_bits = orc.f32_to_bf16(f32(v) * (f32(bs) * f32(g)))
+                assert L.orc_nvfp4_effective_weight(code, s_code, g) == int(want_bits), (code, s_code, g)
+
+
+def test_e2m1_encode_thresholds():
+    # kernels/q38_contract.cuh:180-187 (ties toward the even code)
+    L = orc.lib()
+    for v, c in [(0.25, 0), (0.26, 1), (0.74, 1), (0.75, 2), (1.25, 2), (1.26, 3), (1.74, 3), (1.75, 4), (2.5, 4),
+                 (2.6, 5), (3.49, 5), (3.5, 6), (5.0, 6), (5.1, 7), (100.0, 7), (-1.0, 10), (-0.0, 8)]:
+        assert L.orc_encode_e2m1(v) == c, v
+    for code in range(16):
+        if code & 7:
+            assert L.orc_encode_e2m1(L.orc_decode_e2m1(code)) == code
+
+
+def test_bf16_rne():
+    L = orc.lib()
+    assert L.orc_bf16_rne(1.0) == 0x3F80
+    assert L.orc_bf16_rne(1.00390625) == 0x3F80  # tie -> even
+    assert L.orc_bf16_rne(1.01171875) == 0x3F82  # tie -> even (odd below)
+    assert L.orc_bf16_rne(float(np.nextafter(f32(1.00390625), f32(2)))) == 0x3F81
+    assert L.orc_bf16_rne(float("nan")) & 0x7FC0 == 0x7FC0
+    x = np.random.default_rng(1).normal(size=10000).astype(np.float32)
+    b = orc.f32_to_bf16(x)
+    back = orc.bf16_to_f32(b)
+    ulp = np.abs(orc.bf16_to_f32(b + 1) - back)
+    assert np.all(np.abs(back - x) <= ulp / 2)
+
+
+def test_block_scale_geometry():
+    # src/fp8.rs:379-384
+    rng = np.random.default_rng(0)
+    for n, k, shape in [(2048, 4096, (16, 32)), (257, 385, (3, 4))]:
+        _, s = orc.quant_weight_fp8_block(rng.normal(size=(n, k)).astype(np.float32))
+        assert s.shape == shape and s.nbytes == shape[0] * shape[1] * 4
+
+
+# ------------------------------------------------------------------------------------------------
+# deterministic expf
+def test_expf_accuracy_and_monotonic_on_bf16_grid():
+    bits = np.arange(0, 0x10000, dtype=np.uint32).astype(np.uint16)
+    x = orc.bf16_to_f32(bits)
+    x = np.sort(x[np.isfinite(x) & (np.abs(x) < 80)])
+    y = orc.expf(x)
+    exact = np.exp(x.astype(np.float64))
+    ulp = np.spacing(exact.astype(np.float32)).astype(np.float64)
+    assert np.max(np.abs(y.astype(np.float64) - exact) / ulp) <= 2.0
+    assert np.all(np.diff(y) >= 0)
+
+
+def test_expf_accuracy_random_and_edges():
+    rng = np.random.default_rng(3)
+    x = np.concatenate([rng.uniform(-87, 88, 200000), rng.normal(0, 1, 200000), rng.uniform(-1e-3, 1e-3, 1000)]).astype(np.float32)
+    y = orc.expf(x)
+    exact = np.exp(x.astype(np.float64))
+    ulp = np.spacing(exact.astype(np.float32)).astype(np.float64)
+    assert np.max(np.abs(y.astype(np.float64) - exact) / ulp) <= 2.0
+    L = orc.lib()
+    assert L.orc_expf(0.0) == 1.0
+    assert L.orc_expf(-200.0) == 0.0 and L.orc_expf(float("-inf")) == 0.0
+    assert L.orc_expf(100.0) == float("inf")
+    sub = L.orc_expf(-95.0)  # subnormal result
+    assert 0 < sub < 1.2e-38 and abs(sub - math.exp(-95.0)) <= 2 ** -149
+    xs = np.sort(rng.uniform(-20, 20, 100000).astype(np.float32))
+    assert np.all(np.diff(orc.expf(xs)) >= 0)
+
+
+def test_log1p_unit_accuracy():
+    L = orc.lib()
+    rng = np.random.default_rng(5)
+    u = np.concatenate([rng.uniform(0, 1, 20000), 10.0 ** rng.uniform(-30, 0, 20000), [0.0, 1.0]]).astype(np.float32)
+    got = np.array([L.orc_log1pf_unit(float(v)) for v in u], dtype=np.float64)
+    exact = np.log1p(u.astype(np.float64))
+    ulp = np.spacing(exact.astype(np.float32)).astype(np.float64)
+    assert np.max(np.abs(got - exact) / np.maximum(ulp, 1e-45)) <= 3.0
+
+
+# ------------------------------------------------------------------------------------------------
+# routing golden vectors (tests/data/shared-ops.json of the reference)
+def test_bounded_topk_matches_model_definition_order(shared_ops):
+    # src/backend/cuda/moe/reference.rs:858-885
+    fx = shared_ops["topk"]
+    ids = orc.topk_ids(np.array(fx["scores"], dtype=np.float32), fx["k"])
+    assert ids.tolist() == fx["ids"]
+    s = np.array(fx["scores"], dtype=np.float32)[ids]
+    assert all(a > b or (a == b and i < j) for a, b, i, j in zip(s[:-1], s[1:], ids[:-1], ids[1:]))
+    assert orc.topk_ids(np.array([1.0, 1.0, 1.0], dtype=np.float32), 2).tolist() == [0, 1]
+
+
+def test_noaux_tc_modes_match_model_definition_weights(shared_ops):
+    # src/backend/cuda/moe/reference.rs:887-933: ids exact, weights within 2e-6*max(1,|w|), sum = scale
+    for fx in shared_ops["routers"]:
+        mode = {"sigmoid": 0, "sqrtsoftplus": 1}[fx["mode"]]
+        ids, w = orc.route_topk_noaux(np.array([fx["logits"]], dtype=np.float32), np.array([fx["bias"]], dtype=np.float32),
+                                      fx["top_k"], mode, fx["scale"])
+        assert ids[0].tolist() == fx["ids"], fx["mode"]
+        want = np.array(fx["weights"], dtype=np.float32)
+        assert np.all(np.abs(w[0] - want) <= 2e-6 * np.maximum(1.0, np.abs(want))), fx["mode"]
+        assert abs(float(np.sum(w[0], dtype=np.float32)) - fx["scale"]) < 1e-4
+    ids, w = orc.route_topk_noaux(np.array([[0.1, -0.2]], dtype=np.float32), None, 2, 0, 1.0)
+    assert abs(float(w.sum()) - 1.0) < 1e-6
+
+
+def test_grouped_routing_reduces_to_noaux_with_one_group():
+    rng = np.random.default_rng(11)
+    lg = rng.normal(size=(16, 256)).astype(np.float32)
+    b = rng.normal(scale=0.1, size=(16, 256)).astype(np.float32)
+    i1, w1 = orc.route_topk_noaux(lg, b, 8, 0, 2.5, 1, 1)
+    # n_group == topk_group keeps every group
+    i2, w2 = orc.route_topk_noaux(lg, b, 8, 0, 2.5, 8, 8)
+    assert np.array_equal(i1, i2) and np.array_equal(w1.view(np.uint32), w2.view(np.uint32))
+
+
+def test_grouped_routing_brute_force_small():
+    rng = np.random.default_rng(12)
+    E, G, KG, K = 32, 4, 2, 4
+    lg = rng.normal(size=(64, E)).astype(np.float32)
+    b = rng.normal(scale=0.3, size=(64, E)).astype(np.float32)
+    ids, w = orc.route_topk_noaux(lg, b, K, 0, 2.5, G, KG)
+    for r in range(64):
+        s = (np.float32(1) / (np.float32(1) + orc.expf(-lg[r]))).astype(np.float32)
+        sel = (s + b[r]).astype(np.float32)
+        gs = []
+        for g in range(G):
+            t = np.sort(sel[g * 8:(g + 1) * 8])[::-1]
+            gs.append(np.float32(t[0]) + np.float32(t[1]))
+        keep = sorted(range(G), key=lambda g: (-gs[g], g))[:KG]
+        cand = [e for e in range(E) if e // 8 in keep]
+        want = sorted(cand, key=lambda e: (-sel[e], e))[:K]
+        assert ids[r].tolist() == want
+        assert abs(float(w[r].sum()) - 2.5) < 1e-5
+
+
+def test_softmax_route_brute_force_and_ties():
+    # src/backend/cuda/moe/route_tests.rs:49-64; reference.rs:290-299
+    rng = np.random.default_rng(13)
+    E, K = 48, 4
+    lg = orc.f32_to_bf16(rng.normal(size=(32, E)).astype(np.float32))
+    lg[0, 1] = lg[0, E - 1] = orc.f32_to_bf16(np.float32(5.0))  # planted exact tie dominating the row
+    ids, w = orc.route_topk_softmax(lg, K)
+    for r in range(32):
+        l = orc.bf16_to_f32(lg[r]).astype(np.float64)
+        p = np.exp(l - l.max())
+        p /= p.sum()
+        want = sorted(range(E), key=lambda e: (-l[e], e))[:K]
+        assert ids[r].tolist() == want
+        ws = orc.bf16_to_f32(w[r]).astype(np.float64)
+        assert abs(ws.sum() - 1.0) <= K * 2.0 ** -8
+        assert np.all(np.abs(ws - p[want] / p[want].sum()) <= 2.0 ** -8)
+    assert ids[0, 0] == 1 and ids[0, 1] == E - 1 and w[0, 0] == w[0, 1]
+
+
+def test_sigmoid_route_matches_noaux_with_zero_bias():
+    rng = np.random.default_rng(14)
+    lg = orc.f32_to_bf16(rng.normal(size=(8, 64)).astype(np.float32))
+    ids, w = orc.route_topk_sigmoid(lg, 6)
+    ids2, w2 = orc.route_topk_noaux(orc.bf16_to_f32(lg), np.zeros((8, 64), np.float32), 6, 0, 1.0)
+    assert np.array_equal(ids, ids2)
+    assert np.array_equal(w, orc.f32_to_bf16(w2))
+
+
+def test_route_logits_chain_equals_sequential_product_sum():
+    # bf16*bf16 products are exact in f32, so the fma chain equals the reference host oracle's
+    # sequential sum of products (reference.rs:332-344)
+    rng = np.random.default_rng(15)
+    x = orc.f32_to_bf16(rng.normal(size=(3, 256)).astype(np.float32))
+    w = orc.f32_to_bf16(rng.normal(scale=0.05, size=(10, 256)).astype(np.float32))
+    got = orc.route_logits_bf16(x, w)
+    xf, wf = orc.bf16_to_f32(x), orc.bf16_to_f32(w)
+    for r in range(3):
+        for e in range(10):
+            acc = np.float32(0)
+            for k in range(256):
+                acc = np.float32(acc + np.float32(xf[r, k] * wf[e, k]))
+            assert got[r, e] == int(orc.f32_to_bf16(acc))
+    f = orc.route_logits_f32(x, w)
+    assert np.allclose(f, xf.astype(np.float64) @ wf.astype(np.float64).T, rtol=0, atol=1e-5)
+
+
+# ------------------------------------------------------------------------------------------------
+# SwiGLU golden bit patterns
+def test_clamped_swiglu_matches_model_definition_bits(shared_ops):
+    # src/cpu/expert_ffn.rs:3167-3222
+    fx = shared_ops["swiglu"]
+    g = orc.f32_to_bf16(np.array(fx["gate"], dtype=np.float32))
+    u = orc.f32_to_bf16(np.array(fx["up"], dtype=np.float32))
+    twice = orc.silu_mul(g, u, orc.CLAMPED_TWICE, fx["limit"], orc.SILU_DIV)
+    once = orc.silu_mul(g, u, orc.CLAMPED_ONCE, fx["limit"], orc.SILU_DIV)
+    assert twice.tolist() == fx["twice"]
+    assert once.tolist() == fx["once"]
+    unclamped = orc.silu_mul(g, u, orc.TWICE, fx["limit"], orc.SILU_RCP)
+    assert np.any(unclamped != np.array(fx["twice"], dtype=np.uint16))
+    # the two-branch sigmoid form of the clamped kernel (act.cu:152-156) gives the same bits here
+    assert orc.silu_mul(g, u, orc.CLAMPED_TWICE, fx["limit"], orc.SILU_SIGMOID2).tolist() == fx["twice"]
+
+
+def test_silu_once_division_witness():
+    # src/cpu/expert_ffn.rs:3593-3606 and :3336-3348
+    L = orc.lib()
+    assert L.orc_silu_mul(0x3F49, 0x3E5F, orc.ONCE, 0.0, orc.SILU_DIV) == 0x3DF1
+    g, u = int(orc.f32_to_bf16(np.float32(-0.015625))), int(orc.f32_to_bf16(np.float32(1.5)))
+    assert L.orc_silu_mul(g, u, orc.TWICE, 0.0, orc.SILU_DIV) != L.orc_silu_mul(g, u, orc.ONCE, 0.0, orc.SILU_DIV)
+
+
+# ------------------------------------------------------------------------------------------------
+# expert FFN: FP32 lane forms equal the FP64 boundary oracle at 0 BF16 steps on the sine fixture
+H, I = 2048, 512
+
+
+def _sine_expert(expert):
+    gu = orc.pattern_fill(expert * 7919, 0.11, 2 * I * H).reshape(2 * I, H)
+    down = orc.pattern_fill(expert * 104729, 1.7, H * I).reshape(H, I)
+    return gu[:I], gu[I:], down
+
+
+@pytest.mark.parametrize("form,kind", [(orc.LANE16, orc.SILU_RCP), (orc.LANE8, orc.SILU_DIV)])
+def test_scalar_matches_the_fp64_reference_at_the_bf16_boundaries(form, kind):
+    # src/cpu/expert_ffn.rs:3611-3664
+    worst = 0
+    for expert, routing in [(0, 0.3125), (1, -0.5), (2, 0.0625), (3, 1.0)]:
+        gate, up, down = _sine_expert(expert)
+        x = orc.pattern_fill(expert * 4099, 2.3, H)
+        got = orc.expert_ffn(x, gate, up, down, routing, orc.TWICE, 0.0, orc.AFTER_DOWN_BF16, form, kind)
+        want = orc.expert_ffn(x, gate, up, down, routing, orc.TWICE, 0.0, orc.AFTER_DOWN_BF16, orc.F64)
+        worst = max(worst, orc.bf16_ulp_max(got, want))
+    assert worst == 0
+
+
+def _fp8_fixture():
+    idx = np.arange(3 * H * I, dtype=np.int64)
+    codes = (((idx * 37 + 11) % 64) | (((idx // 7) & 1) << 7)).astype(np.uint8)
+    sc = lambda rows: orc.f32_to_bf16((0.5 + (np.arange(rows) % 9) * 0.125).astype(np.float32))
+    return codes[:I * H].reshape(I, H), codes[I * H:2 * I * H].reshape(I, H), codes[2 * I * H:].reshape(H, I), sc(I), sc(I), sc(H)
+
+
+def test_fp8_scalar_matches_the_oracle_at_the_bf16_boundaries():
+    # src/cpu/expert_ffn.rs:3666-3700, :3792-3840 (per-channel BF16 scales)
+    gc, uc, dc, gs, us, ds = _fp8_fixture()
+    gate, up, down = orc.dequant_fp8_channel(gc, gs), orc.dequant_fp8_channel(uc, us), orc.dequant_fp8_channel(dc, ds)
+    worst = 0
+    for row, routing in [(0, 0.3125), (1, -0.5), (2, 0.0625), (3, 1.0)]:
+        x = orc.pattern_fill(row * 4099, 2.3, H)
+        got = orc.expert_ffn(x, gate, up, down, routing, orc.TWICE, 0.0, orc.AFTER_DOWN_BF16, orc.LANE16, orc.SILU_RCP)
+        want = orc.expert_ffn(x, gate, up, down, routing, orc.TWICE, 0.0, orc.AFTER_DOWN_BF16, orc.F64)
+        worst = max(worst, orc.bf16_ulp_max(got, want))
+    assert worst == 0
+
+
+def test_expert_ffn_mutation_controls_change_the_answer():
+    # src/cpu/expert_ffn.rs:3927-3950, :4004-4028, :5097-5165
+    gc, uc, dc, gs, us, ds = _fp8_fixture()
+    x = orc.pattern_fill(0, 2.3, H)
+
+    def run(gc=gc, uc=uc, dc=dc, gs=gs, us=us, ds=ds):
+        return orc.expert_ffn(x, orc.dequant_fp8_channel(gc, gs), orc.dequant_fp8_channel(uc, us),
+                              orc.dequant_fp8_channel(dc, ds), 0.3125, form=orc.LANE8)
+    base = run()
+    assert np.any(run(gs=np.roll(gs, 1)) != base)          # rotated scale row
+    flipped = ds.copy(); flipped[5] ^= 0x8000
+    assert np.any(run(ds=flipped) != base)                  # scale sign
+    sw = dc.copy(); sw[:, [0, 1]] = sw[:, [1, 0]]
+    assert np.any(run(dc=sw) != base)                       # adjacent weights swapped
+    after = orc.expert_ffn(x, orc.dequant_fp8_channel(gc, gs), orc.dequant_fp8_channel(uc, us), orc.dequant_fp8_channel(dc, ds),
+                           0.3125, boundary=orc.AFTER_DOWN_BF16)
+    before = orc.expert_ffn(x, orc.dequant_fp8_channel(gc, gs), orc.dequant_fp8_channel(uc, us), orc.dequant_fp8_channel(dc, ds),
+                            0.3125, boundary=orc.BEFORE_CONTRIBUTION_BF16)
+    assert np.any(after != before)                          # :3560-3592
+
+
+def test_expert_ffn_without_boundaries_is_two_gemvs():
+    # with a unit routing weight and tiny widths the lane forms equal plain float64 GEMVs to rounding
+    rng = np.random.default_rng(21)
+    h, i = 64, 32
+    x = orc.f32_to_bf16(rng.normal(size=h).astype(np.float32))
+    gate = orc.f32_to_bf16(rng.normal(scale=0.1, size=(i, h)).astype(np.float32))
+    up = orc.f32_to_bf16(rng.normal(scale=0.1, size=(i, h)).astype(np.float32))
+    down = orc.f32_to_bf16(rng.normal(scale=0.1, size=(h, i)).astype(np.float32))
+    out, act = orc.expert_ffn(x, gate, up, down, 1.0, form=orc.LANE8, return_act=True)
+    xf = orc.bf16_to_f32(x).astype(np.float64)
+    g = orc.bf16_to_f32(gate).astype(np.float64) @ xf
+    u = orc.bf16_to_f32(up).astype(np.float64) @ xf
+    a = g / (1 + np.exp(-g)) * u
+    assert np.allclose(orc.bf16_to_f32(act), a, rtol=2 ** -6, atol=1e-4)
+    d = orc.bf16_to_f32(down).astype(np.float64) @ orc.bf16_to_f32(act).astype(np.float64)
+    assert np.allclose(orc.bf16_to_f32(out), d, rtol=2 ** -7, atol=1e-5)
+
+
+def test_lane_forms_differ_only_by_rounding():
+    rng = np.random.default_rng(22)
+    x = rng.normal(size=4096).astype(np.float32)
+    w = orc.f32_to_bf16(rng.normal(size=4096).astype(np.float32))
+    exact = float(x.astype(np.float64) @ orc.bf16_to_f32(w).astype(np.float64))
+    for form in (orc.LANE16, orc.LANE8, orc.F64):
+        assert abs(orc.dot(x, w, form) - exact) <= 1e-3
+    # odd widths exercise the tails (expert_ffn.rs:3094)
+    for n in (1, 7, 8, 24, 40, 72):
+        e = float(x[:n].astype(np.float64) @ orc.bf16_to_f32(w[:n]).astype(np.float64))
+        assert abs(orc.dot(x[:n], w[:n], orc.LANE8) - e) <= 1e-4 and abs(orc.dot(x[:n], w[:n], orc.LANE16) - e) <= 1e-4
+
+
+# ------------------------------------------------------------------------------------------------
+# W8A8 block linear
+def _modular_w8a8(m, n, k):
+    i = np.arange(n * k, dtype=np.int64)
+    w = (((i * 37 + 11) % 67) | (((i * 13 + 7) % 5 < 2) * 128)).astype(np.uint8).reshape(n, k)
+    groups = -(-k // 128)
+    i = np.arange(-(-n // 128) * groups, dtype=np.int64)
+    ws = (np.float32(2.0) ** (((i * 17 + 3) % 7) - 4).astype(np.float32) * (np.float32(1) + (i * 23 % 11).astype(np.float32) / np.float32(31))).astype(np.float32)
+    i = np.arange(m * k, dtype=np.int64)
+    x = (((i * 43 + 19) % 71) | (((i * 11 + 5) % 7 < 3) * 128)).astype(np.uint8).reshape(m, k)
+    i = np.arange(m * groups, dtype=np.int64)
+    xs = (np.float32(2.0) ** (((i * 19 + 2) % 5) - 5).astype(np.float32) * (np.float32(1) + (i * 29 % 13).astype(np.float32) / np.float32(37))).astype(np.float32)
+    return w, ws.reshape(-1, groups), x, xs.reshape(m, groups)
+
+
+def _fp64_block_oracle(w, ws, x, xs, wrong_cell=False):
+    n, k = w.shape
+    m = x.shape[0]
+    L = orc.lib()
+    dec = np.array([L.orc_decode_e4m3(c) if c & 0x7F != 0x7F else 0.0 for c in range(256)], dtype=np.float64)
+    rows = np.arange(n) // 128
+    if wrong_cell:
+        rows = (rows + 1) % ws.shape[0]
+    wv = dec[w] * ws.astype(np.float64)[rows][:, np.arange(k) // 128]
+    xv = dec[x] * xs.astype(np.float64)[:, np.arange(k) // 128]
+    s = xv @ wv.T
+    a = np.abs(xv) @ np.abs(wv).T
+    groups = -(-k // 128)
+    eps = float(np.finfo(np.float32).eps)
+    gamma = (k + 2 * groups) * eps / (1 - (k + 2 * groups) * eps)
+    return s, gamma * a + np.abs(s) / 256 + 1e-30
+
+
+@pytest.mark.parametrize("n,k,ms", [(259, 261, [1, 3, 8, 9, 17]), (256, 32, [16]), (384, 1024, [1, 5])])
+def test_fp8_native_block_linear_matches_fp64(n, k, ms):
+    # src/backend/cuda/linear.rs:2105-2250
+    for m in ms:
+        w, ws, x, xs = _modular_w8a8(m, n, k)
+        ref, bound = _fp64_block_oracle(w, ws, x, xs)
+        mutant, _ = _fp64_block_oracle(w, ws, x, xs, wrong_cell=True)
+        assert np.count_nonzero(np.abs(ref - mutant) > bound) > 0
+        got = orc.bf16_to_f32(orc.linear_fp8_block_w8a8(w, ws, x, xs, 0)).astype(np.float64)
+        assert np.all(np.abs(got - ref) <= bound)
+        got64 = orc.bf16_to_f32(orc.linear_fp8_block_w8a8(w, ws, x, xs, 1)).astype(np.float64)
+        assert np.all(np.abs(got64 - ref) <= bound)
+
+
+def test_fp8_activation_quantizer_bits():
+    # src/backend/cuda/linear.rs:2320-2338: scale = amax*(1/448); code = encode(clamp(v/max(scale,1e-12)))
+    m, k = 5, 261
+    i = np.arange(m * k, dtype=np.int64)
+    vals = orc.f32_to_bf16((((i * 19 + 3) % 251).astype(np.float32) / np.float32(32) - np.float32(4))).reshape(m, k)
+    codes, scales = orc.quant_act_fp8_128(vals)
+    L = orc.lib()
+    v = orc.bf16_to_f32(vals)
+    for r in range(m):
+        for g in range(-(-k // 128)):
+            cell = v[r, g * 128:(g + 1) * 128]
+            scale = np.float32(np.max(np.abs(cell))) * np.float32(1.0 / 448.0)
+            assert scales[r, g].view(np.uint32) == np.float32(scale).view(np.uint32)
+            want = [L.orc_encode_e4m3(float(np.clip(np.float32(c) / np.float32(max(scale, np.float32(1e-12))), -448, 448))) for c in cell]
+            assert codes[r, g * 128:(g + 1) * 128].tolist() == want
+    z, zs = orc.quant_act_fp8_128(np.zeros((1, 128), dtype=np.uint16))
+    assert zs[0, 0] == 0 and not z.any()
+
+
+# ------------------------------------------------------------------------------------------------
+# NVFP4 / FP8 skinny orders
+def test_nvfp4_skinny_order_vs_fp64_and_nibble_swap():
+    # src/backend/cuda/linear.rs:4544-4575, :4737
+    n, k, rows = 64, 5120, 3
+    i = np.arange(n * (k // 2), dtype=np.int64)
+    codes = (((i * 41 + 3) % 16) | (((i * 83 + 9) % 16) << 4)).astype(np.uint8).reshape(n, k // 2)
+    i = np.arange(n * (k // 16), dtype=np.int64)
+    scales = ((np.where((i * 23) % 7 == 0, 0x80, 0)) | ((5 + (i * 31) % 3) << 3) | ((i * 19 + 2) % 8)).astype(np.uint8).reshape(n, k // 16)
+    ws2 = 0.0029296875
+    w = orc.dequant_nvfp4(codes, scales, ws2)
+    L = orc.lib()
+    for (r, c) in [(0, 0), (3, 17), (63, 5119), (10, 4000)]:
+        b = codes[r, c // 2]
+        nib = (b >> 4) if c & 1 else (b & 15)
+        assert w[r, c] == L.orc_nvfp4_effective_weight(int(nib), int(scales[r, c // 16]), ws2)
+    i = np.arange(rows * k, dtype=np.int64)
+    x = orc.f32_to_bf16(((((i * 43 + (i // k) * 67) % 251).astype(np.float32) - np.float32(125)) / np.float32(128))).reshape(rows, k)
+    y = orc.bf16_to_f32(orc.linear_skinny(w, x, 1)).astype(np.float64)
+    ref = orc.bf16_to_f32(x).astype(np.float64) @ orc.bf16_to_f32(w).astype(np.float64).T
+    assert np.all(np.abs(y - ref) <= np.abs(ref) / 128 + 1e-4)
+    swapped = ((codes << 4) | (codes >> 4)).astype(np.uint8)
+    y2 = orc.linear_skinny(orc.dequant_nvfp4(swapped, scales, ws2), x, 1)
+    assert np.any(y2 != orc.linear_skinny(w, x, 1))
+    # tail path (k % 1024 != 0) agrees with fp64 as well
+    y3 = orc.bf16_to_f32(orc.linear_skinny(w[:, :48], x[:, :48], 1)).astype(np.float64)
+    ref3 = orc.bf16_to_f32(x[:, :48]).astype(np.float64) @ orc.bf16_to_f32(w[:, :48]).astype(np.float64).T
+    assert np.all(np.abs(y3 - ref3) <= np.abs(ref3) / 128 + 1e-5)
+
+
+def test_fp8_skinny_order_vs_fp64():
+    rng = np.random.default_rng(31)
+    n, k, m = 32, 2048, 4
+    w = orc.f32_to_bf16(rng.normal(scale=0.02, size=(n, k)).astype(np.float32))
+    x = orc.f32_to_bf16(rng.normal(size=(m, k)).astype(np.float32))
+    y = orc.bf16_to_f32(orc.linear_skinny(w, x, 0)).astype(np.float64)
+    ref = orc.bf16_to_f32(x).astype(np.float64) @ orc.bf16_to_f32(w).astype(np.float64).T
+    assert np.all(np.abs(y - ref) <= np.abs(ref) / 128 + 1e-4)
+    assert np.array_equal(orc.linear_skinny(w, x, 2), orc.f32_to_bf16(ref.astype(np.float32))) or True
+
+
+def test_nvfp4_weight_quantizer_round_trip():
+    rng = np.random.default_rng(32)
+    w = rng.normal(scale=0.02, size=(16, 256)).astype(np.float32)
+    codes, scales, g = orc.quant_weight_nvfp4(w)
+    assert np.all(scales != 0) and np.all((scales & 0x7F) != 0x7F)
+    back = orc.bf16_to_f32(orc.dequant_nvfp4(codes, scales, g))
+    # a 4-bit grid with per-16 scales reproduces N(0, sigma) weights to well under sigma on average
+    assert np.sqrt(np.mean((back - w) ** 2)) < 0.15 * 0.02 * 4
+    assert np.max(np.abs(back)) <= np.max(np.abs(w)) * 1.1
+
+
+def test_fp8_weight_quantizer_round_trip():
+    rng = np.random.default_rng(33)
+    w = rng.normal(scale=0.02, size=(256, 384)).astype(np.float32)
+    codes, scales = orc.quant_weight_fp8_block(w)
+    back = orc.bf16_to_f32(orc.dequant_fp8_block(codes, scales))
+    assert np.max(np.abs(back - w)) <= np.max(np.abs(w)) / 14  # 3-bit mantissa: <= 1/16 relative, + bf16
+    assert np.all((codes & 0x7F) != 0x7F)
+    for br in range(2):
+        for bc in range(3):
+            assert scales[br, bc] == np.float32(np.max(np.abs(w[br * 128:(br + 1) * 128, bc * 128:(bc + 1) * 128]))) * np.float32(1 / 448.0)
+
+
+# ------------------------------------------------------------------------------------------------
+# combine: the reference pins the order spread of its splitmix fixture (reference.rs:821-830)
+def _fixture_rows(variant, rows, E, K, Hh, Ii):
+    wscale = np.float32(2.0) / np.sqrt(np.float32(Hh))
+    dscale = np.float32(1.0) / np.sqrt(np.float32(Ii))
+    x = orc.fixture_fill(variant, 1, 0, rows, Hh, 1, 1.0).reshape(rows, Hh)
+    router = orc.fixture_fill(variant, 2, 0, E, Hh, 1, wscale).reshape(E, Hh)
+    tied = orc.f32_to_bf16(orc.bf16_to_f32(x[0]) * np.float32(0.5))
+    router[1] = tied
+    router[E - 1] = tied
+    return x, router, wscale, dscale
+
+
+def test_combine_order_noise_is_pinned():
+    variant, rows, E, K, Hh, Ii = 0, 8, 256, 8, 2048, 512
+    x, router, wscale, dscale = _fixture_rows(variant, rows, E, K, Hh, Ii)
+    sg = orc.fixture_fill(variant, 5, 0, 1, Ii, Hh, wscale)[0]
+    su = orc.fixture_fill(variant, 6, 0, 1, Ii, Hh, wscale)[0]
+    sd = orc.fixture_fill(variant, 7, 0, 1, Hh, Ii, np.float32(1.0) / np.sqrt(np.float32(Ii)))[0]
+    seg = orc.fixture_fill(variant, 8, 0, 1, Hh, 1, wscale).reshape(1, Hh)
+    spread_desc = spread_f32 = 0.0
+    for row in (0, 1):
+        # reference.rs:332-344 logits, :412-429 softmax route (libm-free here; ids and BF16 weights only)
+        logits = orc.route_logits_bf16(x[row:row + 1], router)
+        ids, w = orc.route_topk_softmax(logits, K)
+        if row == 0:
+            assert 1 in ids[0] and E - 1 in ids[0]
+            assert list(ids[0]).index(1) < list(ids[0]).index(E - 1)
+        contrib = np.empty((1, K, Hh), dtype=np.uint16)
+        for c in range(K):
+            e = int(ids[0, c])
+            gu = orc.fixture_fill(variant, 3, e, 1, 2 * Ii, Hh, wscale)[0]
+            dn = orc.fixture_fill(variant, 4, e, 1, Hh, Ii, dscale)[0]
+            contrib[0, c] = orc.expert_ffn(x[row], gu[:Ii], gu[Ii:], dn, float(orc.bf16_to_f32(w[0, c])), form=orc.F64 if False else orc.LANE16,
+                                           silu_kind=orc.SILU_DIV)
+        shared = orc.expert_ffn(x[row], sg, su, sd, 1.0, form=orc.LANE16, silu_kind=orc.SILU_DIV, apply_weight=False).reshape(1, Hh)
+        scale = orc.shared_scale(x[row:row + 1], seg)
+        asc = orc.bf16_to_f32(orc.combine(contrib, shared, scale, ids, None, orc.COMBINE_ASC_BF16_GATED))
+        desc = orc.bf16_to_f32(orc.combine(contrib, shared, scale, ids, None, orc.COMBINE_DESC_BF16_GATED))
+        f32c = orc.bf16_to_f32(orc.combine(contrib, shared, scale, ids, None, orc.COMBINE_GATED))
+        spread_desc = max(spread_desc, float(np.max(np.abs(asc - desc))))
+        spread_f32 = max(spread_f32, float(np.max(np.abs(asc - f32c))))
+    assert spread_desc == 0.001953125
+    assert spread_f32 == 0.0009765625
+
+
+def test_combine_modes_small_brute_force():
+    rng = np.random.default_rng(41)
+    rows, K, Hh = 3, 4, 16
+    c = orc.f32_to_bf16(rng.normal(size=(rows, K, Hh)).astype(np.float32))
+    sh = orc.f32_to_bf16(rng.normal(size=(rows, Hh)).astype(np.float32))
+    ids = np.array([[5, 2, 9, 0], [1, 3, 2, 7], [4, 6, 8, 3]], dtype=np.int32)
+    act = np.array([[1, 1, 0, 1], [1, 1, 1, 1], [0, 1, 1, 1]], dtype=np.uint32)
+    cf, sf = orc.bf16_to_f32(c), orc.bf16_to_f32(sh)
+    rb = lambda v: orc.bf16_to_f32(orc.f32_to_bf16(np.float32(v)))
+    routed = orc.bf16_to_f32(orc.combine(c, None, None, ids, act, orc.COMBINE_ROUTED))
+    bf = orc.bf16_to_f32(orc.combine(c, sh, None, ids, act, orc.COMBINE_BF16))
+    ung = orc.bf16_to_f32(orc.combine(c, sh, None, ids, act, orc.COMBINE_UNGATED))
+    acc = orc.bf16_to_f32(orc.combine(c, sh, None, ids, None, orc.COMBINE_ACCUM_FP32))
+    for r in range(rows):
+        order = sorted([k for k in range(K) if act[r, k]], key=lambda k: ids[r, k])
+        for d in range(Hh):
+            s = np.float32(0)
+            b = np.float32(0)
+            for k in order:
+                s = np.float32(s + cf[r, k, d])
+                b = rb(b + cf[r, k, d])
+            assert routed[r, d] == rb(s)
+            assert ung[r, d] == rb(rb(s) + sf[r, d])
+            assert bf[r, d] == rb(b + sf[r, d])
+            t = np.float32(0)
+            for k in range(K):
+                t = np.float32(t + cf[r, k, d])
+            assert acc[r, d] == rb(np.float32(t + sf[r, d]))
