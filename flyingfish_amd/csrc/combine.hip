@@ -1,0 +1,147 @@
+// Ordered weighted combine of per-(row, choice) BF16 contributions with the shared expert.
+// Orders and rounding boundaries follow kernels/moe_combine.cu of the reference.
+#include "common.cuh"
+#include "api.h"
+
+namespace ffmoe {
+
+// scale[r] = bf16(sigmoid(bf16(dot))): thread-strided partial products (mul then add, not fused),
+// 32-lane shuffle-down trees, then the tree over the 8 group partials (kernels/moe_combine.cu:21-49).
+__global__ __launch_bounds__(256) void k_shared_scale(const uint16_t* __restrict__ x, const uint16_t* __restrict__ seg,
+                                                      uint16_t* __restrict__ scale, int hidden) {
+  __shared__ float red[32];
+  const int tid = threadIdx.x, row = blockIdx.x;
+  const uint16_t* xr = x + size_t(row) * hidden;
+  float part = 0.0f;
+  for (int c = tid; c < hidden; c += 256) part = __fadd_rn(part, __fmul_rn(bf16_to_f32(xr[c]), bf16_to_f32(seg[c])));
+#pragma unroll
+  for (int off = 16; off > 0; off >>= 1) {
+    const float o = __shfl_down(part, off, 32);
+    part = __fadd_rn(part, ((tid & 31) + off < 32) ? o : 0.0f);
+  }
+  if (tid < 32) red[tid] = 0.0f;
+  __syncthreads();
+  if ((tid & 31) == 0) red[tid >> 5] = part;
+  __syncthreads();
+  if (tid < 32) {
+    float v = red[tid];
+#pragma unroll
+    for (int off = 16; off > 0; off >>= 1) {
+      const float o = __shfl_down(v, off, 32);
+      v = __fadd_rn(v, (tid + off < 32) ? o : 0.0f);
+    }
+    if (tid == 0) scale[row] = f32_to_bf16(sigmoid1(bround(v)));
+  }
+}
+
+// One block per row; 8 BF16 per thread and step.
+__global__ __launch_bounds__(256) void k_combine(const uint16_t* __restrict__ contributions, const uint16_t* __restrict__ shared_out,
+                                                 const uint16_t* __restrict__ scale, const int* __restrict__ ids,
+                                                 const uint32_t* __restrict__ done, const uint32_t* __restrict__ final_active,
+                                                 uint16_t* __restrict__ y, uint32_t* __restrict__ status, int top_k, int hidden,
+                                                 int mode) {
+  const int tid = threadIdx.x, row = blockIdx.x;
+  const int a0 = row * top_k;
+  int order[FFMOE_MAX_TOP_K];
+  int live = 0;
+  if (mode == FFMOE_COMBINE_ACCUM_FP32 || mode == FFMOE_COMBINE_ACCUM_BF16) {
+    live = top_k;
+#pragma unroll 1
+    for (int c = 0; c < top_k; ++c) order[c] = c;
+  } else {
+    // stable insertion sort of the active choices by ascending expert id (kernels/moe_combine.cu:51-69)
+    bool bad = false;
+#pragma unroll 1
+    for (int c = 0; c < top_k; ++c) {
+      const uint32_t want = final_active ? final_active[a0 + c] : 1u;
+      if (done && done[a0 + c] != want) bad = true;
+      if (want == 0u) continue;
+      int p = live;
+      while (p > 0 && ids[a0 + order[p - 1]] > ids[a0 + c]) { order[p] = order[p - 1]; --p; }
+      order[p] = c;
+      ++live;
+    }
+    if (bad && status && tid == 0) atomicOr(status, 1u);
+  }
+  const float sc = (mode == FFMOE_COMBINE_GATED) ? bf16_to_f32(scale[row]) : 0.0f;
+  for (int d0 = tid * 8; d0 < hidden; d0 += 256 * 8) {
+    float acc[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j] = 0.0f;
+    for (int k = 0; k < live; ++k) {
+      const u32x4 c = load16(contributions + (size_t(a0) + order[k]) * hidden + d0);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        if (mode == FFMOE_COMBINE_BF16) {
+          acc[2 * q] = bround(__fadd_rn(acc[2 * q], bf16lo(c[q])));
+          acc[2 * q + 1] = bround(__fadd_rn(acc[2 * q + 1], bf16hi(c[q])));
+        } else {
+          acc[2 * q] = __fadd_rn(acc[2 * q], bf16lo(c[q]));
+          acc[2 * q + 1] = __fadd_rn(acc[2 * q + 1], bf16hi(c[q]));
+        }
+      }
+    }
+    u32x4 sh = {0, 0, 0, 0};
+    if (mode != FFMOE_COMBINE_ROUTED) sh = load16(shared_out + size_t(row) * hidden + d0);
+    u32x4 out;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      float r[2];
+#pragma unroll
+      for (int hsel = 0; hsel < 2; ++hsel) {
+        const float s = hsel ? bf16hi(sh[q]) : bf16lo(sh[q]);
+        const float a = acc[2 * q + hsel];
+        float v;
+        switch (mode) {
+          case FFMOE_COMBINE_GATED: v = __fadd_rn(bround(a), bround(__fmul_rn(sc, s))); break;
+          case FFMOE_COMBINE_UNGATED:
+          case FFMOE_COMBINE_ACCUM_BF16: v = __fadd_rn(bround(a), s); break;
+          case FFMOE_COMBINE_BF16:
+          case FFMOE_COMBINE_ACCUM_FP32: v = __fadd_rn(a, s); break;
+          default: v = a; break;
+        }
+        r[hsel] = v;
+      }
+      out[q] = pack_bf16x2(r[0], r[1]);
+    }
+    *reinterpret_cast<u32x4*>(y + size_t(row) * hidden + d0) = out;
+  }
+}
+
+}  // namespace ffmoe
+
+using namespace ffmoe;
+
+extern "C" __attribute__((visibility("default"))) int ffmoe_shared_scale(const void* x, const void* seg, void* scale, int rows, int hidden, void* stream) {
+  FF_REQUIRE(rows >= 1 && hidden >= 1, FFMOE_ERR_SHAPE, "shared_scale rows=%d hidden=%d", rows, hidden);
+  FF_PTR16(x); FF_PTR16(seg); FF_PTR2(scale);
+  FF_NO_OVERLAP(scale, size_t(rows) * 2, x, size_t(rows) * hidden * 2);
+  FF_NO_OVERLAP(scale, size_t(rows) * 2, seg, size_t(hidden) * 2);
+  hipLaunchKernelGGL(k_shared_scale, dim3(rows), dim3(256), 0, (hipStream_t)stream, (const uint16_t*)x, (const uint16_t*)seg,
+                     (uint16_t*)scale, hidden);
+  return ff_launch_status();
+}
+
+extern "C" __attribute__((visibility("default"))) int ffmoe_combine(const void* contributions, const void* shared_out, const void* scale, const int* ids,
+                             const uint32_t* done, const uint32_t* final_active, void* y, uint32_t* status, int rows,
+                             int top_k, int hidden, int mode, void* stream) {
+  FF_REQUIRE(rows >= 1 && top_k >= 1 && top_k <= FFMOE_MAX_TOP_K, FFMOE_ERR_SHAPE, "combine rows=%d top_k=%d out of range", rows, top_k);
+  FF_REQUIRE(hidden >= 8 && hidden % 8 == 0, FFMOE_ERR_SHAPE, "combine hidden=%d must be a positive multiple of 8", hidden);
+  FF_REQUIRE(mode >= 0 && mode <= FFMOE_COMBINE_ROUTED, FFMOE_ERR_UNSUPPORTED, "unknown combine mode %d", mode);
+  FF_PTR16(contributions); FF_PTR16(y);
+  const bool ordered = !(mode == FFMOE_COMBINE_ACCUM_FP32 || mode == FFMOE_COMBINE_ACCUM_BF16);
+  if (ordered) FF_PTR4(ids);
+  if (mode != FFMOE_COMBINE_ROUTED) FF_PTR16(shared_out);
+  if (mode == FFMOE_COMBINE_GATED) FF_PTR2(scale);
+  if (done) FF_PTR4(done);
+  if (final_active) FF_PTR4(final_active);
+  if (status) FF_PTR4(status);
+  const size_t yb = size_t(rows) * hidden * 2, cb = size_t(rows) * top_k * hidden * 2;
+  FF_NO_OVERLAP(y, yb, contributions, cb);
+  if (mode != FFMOE_COMBINE_ROUTED) FF_NO_OVERLAP(y, yb, shared_out, yb);
+  if (ordered) FF_NO_OVERLAP(y, yb, ids, size_t(rows) * top_k * 4);
+  hipLaunchKernelGGL(k_combine, dim3(rows), dim3(256), 0, (hipStream_t)stream, (const uint16_t*)contributions,
+                     (const uint16_t*)shared_out, (const uint16_t*)scale, ids, done, final_active, (uint16_t*)y, status, top_k,
+                     hidden, mode);
+  return ff_launch_status();
+}

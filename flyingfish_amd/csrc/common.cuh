@@ -1,0 +1,160 @@
+// Device-side helpers shared by every kernel of libffmoe (gfx950, wave64).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace ffmoe {
+
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int WAVE = 64;
+
+__device__ __forceinline__ float bf16_to_f32(uint16_t h) { return __uint_as_float(uint32_t(h) << 16); }
+__device__ __forceinline__ float bf16lo(uint32_t pair) { return __uint_as_float(pair << 16); }
+__device__ __forceinline__ float bf16hi(uint32_t pair) { return __uint_as_float(pair & 0xffff0000u); }
+
+// FP32 -> BF16 round-to-nearest-even (v_cvt_pk_bf16_f32 on gfx950).
+__device__ __forceinline__ uint16_t f32_to_bf16(float f) {
+  const __bf16 b = static_cast<__bf16>(f);
+  return __builtin_bit_cast(uint16_t, b);
+}
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  f32x2 v = {lo, hi};
+  const bf16x2 b = __builtin_convertvector(v, bf16x2);
+  return __builtin_bit_cast(uint32_t, b);
+}
+__device__ __forceinline__ float bround(float f) { return bf16_to_f32(f32_to_bf16(f)); }
+
+// acc + a.lo*b.lo + a.hi*b.hi over packed BF16 pairs (v_dot2c_f32_bf16).
+__device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float acc) {
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a), __builtin_bit_cast(bf16x2, b), acc, false);
+}
+
+// Two OCP E4M3 codes -> two f32 (v_cvt_pk_f32_fp8); hi selects the upper 16 bits of the dword.
+template <bool HI>
+__device__ __forceinline__ f32x2 e4m3x2_to_f32(uint32_t packed) {
+  return __builtin_amdgcn_cvt_pk_f32_fp8(packed, HI);
+}
+// Four codes of one dword scaled and rounded to BF16: two packed pairs (elements 0,1 and 2,3).
+__device__ __forceinline__ void dequant4_e4m3(uint32_t codes, float scale, uint32_t& w01, uint32_t& w23) {
+  const f32x2 lo = e4m3x2_to_f32<false>(codes);
+  const f32x2 hi = e4m3x2_to_f32<true>(codes);
+  w01 = pack_bf16x2(lo.x * scale, lo.y * scale);
+  w23 = pack_bf16x2(hi.x * scale, hi.y * scale);
+}
+__device__ __forceinline__ float e4m3_to_f32(uint8_t code) { return e4m3x2_to_f32<false>(uint32_t(code)).x; }
+
+// E4M3 code of a finite value already clamped to [-448, 448], round-to-nearest-even
+// (same function as src/fp8.rs:85-121 of the reference).
+__device__ __forceinline__ uint8_t e4m3_encode(float value) {
+  const uint32_t bits = __float_as_uint(value);
+  const uint32_t sign = (bits >> 24) & 0x80u;
+  const uint32_t mag = bits & 0x7fffffffu;
+  if (mag < 0x3c800000u) {  // |v| < 2^-6: subnormal grid m/512, ties to even
+    const float scaled = __uint_as_float(mag) * 512.0f;
+    const uint32_t m = uint32_t(__builtin_rintf(scaled));
+    return uint8_t(sign | m);  // m == 8 is code 0x08 = 2^-6, the first normal
+  }
+  uint32_t rounded = mag >> 20;
+  const uint32_t rest = mag & 0xfffffu;
+  rounded += (rest > 0x80000u || (rest == 0x80000u && (rounded & 1u))) ? 1u : 0u;
+  rounded -= 960u;  // (exponent 120) << 3
+  return uint8_t(sign | (rounded > 126u ? 126u : rounded));
+}
+
+// E2M1 magnitude table; both zero codes give +0 (kernels/nvfp4_linear.cu:12-14 of the reference).
+__device__ __forceinline__ float e2m1_to_f32(uint32_t nib) {
+  const uint32_t m = nib & 7u;
+  // {0, .5, 1, 1.5, 2, 3, 4, 6}: bits of the f32 value
+  const uint32_t expo = m < 2u ? (m == 0u ? 0u : 0x3f000000u) : (0x3f800000u + (((m >> 1) - 1u) << 23));
+  const uint32_t frac = (m >= 2u && (m & 1u)) ? 0x00400000u : 0u;
+  const uint32_t bits = expo | frac;
+  return __uint_as_float(m == 0u ? 0u : (bits | ((nib & 8u) << 28)));
+}
+
+// Deterministic expf: IEEE +,-,*,fma only, so the host restatement gives the same bits.
+// x = n ln2 + r, Cephes polynomial for (e^r - 1 - r)/r^2, two-step scaling by 2^n.
+__device__ __forceinline__ float det_expf(float x) {
+  if (x != x) return x;
+  if (!(x > -104.0f)) return 0.0f;
+  if (x > 88.72283935546875f) return __uint_as_float(0x7f800000u);
+  const float magic = 12582912.0f;
+  const float t = __fmaf_rn(x, 1.44269502162933349609375f, magic);
+  const float n = __fsub_rn(t, magic);
+  float r = __fmaf_rn(n, -0.693145751953125f, x);
+  r = __fmaf_rn(n, -1.428606765330187045037746429443359375e-06f, r);
+  float p = 1.9875691500e-4f;
+  p = __fmaf_rn(p, r, 1.3981999507e-3f);
+  p = __fmaf_rn(p, r, 8.3334519073e-3f);
+  p = __fmaf_rn(p, r, 4.1665795894e-2f);
+  p = __fmaf_rn(p, r, 1.6666665459e-1f);
+  p = __fmaf_rn(p, r, 5.0000001201e-1f);
+  const float r2 = __fmul_rn(r, r);
+  float y = __fmaf_rn(p, r2, r);
+  y = __fadd_rn(y, 1.0f);
+  const int ni = int(n);
+  const int a = ni >> 1, b = ni - a;
+  y = __fmul_rn(y, __uint_as_float(uint32_t(a + 127) << 23));
+  y = __fmul_rn(y, __uint_as_float(uint32_t(b + 127) << 23));
+  return y;
+}
+
+// log(1+u), 0 <= u <= 1.
+__device__ __forceinline__ float det_log1pf_unit(float u) {
+  const float w = __fadd_rn(1.0f, u);
+  if (w == 1.0f) return u;
+  float m = w;
+  float e = 0.0f;
+  if (m > 1.41421353816986083984375f) { m = __fmul_rn(m, 0.5f); e = 1.0f; }
+  const float f = __fsub_rn(m, 1.0f);
+  const float z = __fmul_rn(f, f);
+  float p = 7.0376836292e-2f;
+  p = __fmaf_rn(p, f, -1.1514610310e-1f);
+  p = __fmaf_rn(p, f, 1.1676998740e-1f);
+  p = __fmaf_rn(p, f, -1.2420140846e-1f);
+  p = __fmaf_rn(p, f, 1.4249322787e-1f);
+  p = __fmaf_rn(p, f, -1.6668057665e-1f);
+  p = __fmaf_rn(p, f, 2.0000714765e-1f);
+  p = __fmaf_rn(p, f, -2.4999993993e-1f);
+  p = __fmaf_rn(p, f, 3.3333331174e-1f);
+  float y = __fmul_rn(__fmul_rn(f, z), p);
+  y = __fmaf_rn(-0.5f, z, y);
+  float lg = __fadd_rn(f, y);
+  lg = __fmaf_rn(e, 0.693147182464599609375f, lg);
+  const float c = __fdiv_rn(__fsub_rn(u, __fsub_rn(w, 1.0f)), w);
+  return __fadd_rn(lg, c);
+}
+
+__device__ __forceinline__ float sigmoid1(float l) { return __fdiv_rn(1.0f, __fadd_rn(1.0f, det_expf(-l))); }
+
+// SwiGLU with the BF16 rounding boundary selected by `mode` (FFMOE_SWIGLU_*): returns BF16 bits.
+// SiLU = g / (1 + exp(-g)) as in the production decode kernels of the reference.
+__device__ __forceinline__ uint16_t swiglu_bf16(float g, float u, int mode, float limit) {
+  if (mode >= 2) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+  }
+  const float act = __fdiv_rn(g, __fadd_rn(1.0f, det_expf(-g)));
+  const float prod = (mode == 0 || mode == 2) ? __fmul_rn(bround(act), u) : __fmul_rn(act, u);
+  return f32_to_bf16(prod);
+}
+
+// Sum over the 64 lanes of a wave; every lane receives the total.
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, WAVE);
+  return v;
+}
+
+// 16-byte global load that bypasses nothing special: plain vector load, kept as one instruction.
+__device__ __forceinline__ u32x4 load16(const void* p) { return *reinterpret_cast<const u32x4*>(p); }
+// Streaming 16-byte load for data read exactly once (weights): non-temporal hint keeps it from
+// displacing reusable lines.
+__device__ __forceinline__ u32x4 load16_stream(const void* p) {
+  return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+}
+
+}  // namespace ffmoe

@@ -1,0 +1,40 @@
+// Internal structures of the decode path (not part of the C ABI).
+#pragma once
+#include <stdint.h>
+
+#define FFMOE_DECODE_RG 8              /* rows of one expert served by one pass over its weights */
+#define FFMOE_DECODE_MAX_ASSIGN 4096   /* rows * top_k handled by the single-block grouping kernel */
+
+namespace ffmoe {
+
+struct GroupDesc {
+  int expert;                 // expert id, -1 = shared expert
+  int n;                      // rows in this group (0 = nothing to do)
+  int row[FFMOE_DECODE_RG];   // token row of each member
+  int slot[FFMOE_DECODE_RG];  // activation / contribution slot: assignment index, or rows*top_k + row for the shared expert
+  int pad[2];
+};
+
+struct DecodeParams {
+  int rows, top_k, experts, hidden, inter, shared_inter, has_shared;
+  int swiglu, routed_weight, weights_f32;
+  float swiglu_limit;
+  const uint16_t* x;
+  const int* ids;
+  const uint32_t* active;
+  const void* weights;
+  const uint64_t* slots;
+  const uint32_t* valid;
+  const float* global_scales;
+  uint64_t shared_slot[6];
+  float shared_global[3];
+  uint16_t* contributions;
+  uint16_t* shared_out;
+  uint32_t* done;
+  uint16_t* h;       // [rows*top_k + rows, h_stride] BF16 activations between the two stages
+  int h_stride;
+  GroupDesc* groups;        // NULL = one group per assignment, built on the fly
+  int* counters;            // {routed groups, shared groups} when groups != NULL
+};
+
+}  // namespace ffmoe

@@ -1,0 +1,121 @@
+// Weight-streaming GEMV building blocks shared by the decode and the standalone linear kernels:
+// the three weight formats (16-byte lane chunks, in-register dequantization to packed BF16 pairs)
+// and the slab inner loop (weights in registers x activations in LDS, v_dot2 accumulation).
+#pragma once
+#include "common.cuh"
+
+namespace ffmoe {
+
+// ---------------------------------------------------------------------------------------------
+// weight formats
+struct FmtFp8 {
+  static constexpr int EPL = 16;  // elements per 16-byte lane chunk
+  struct Chunk { u32x4 codes; float scale; };
+  struct Row { const uint8_t* codes; const float* scales; };
+  // slot entries: codes [N,K] u8, scales [ceil(N/128), ceil(K/128)] f32
+  static __device__ __forceinline__ Row row(uint64_t codes, uint64_t scales, float, int j, int K) {
+    Row r;
+    r.codes = reinterpret_cast<const uint8_t*>(codes) + size_t(j) * K;
+    r.scales = reinterpret_cast<const float*>(scales) + size_t(j >> 7) * ((K + 127) >> 7);
+    return r;
+  }
+  static __device__ __forceinline__ void load(Chunk& c, const Row& r, int chunk, bool valid) {
+    const u32x4 z = {0, 0, 0, 0};
+    c.codes = valid ? load16_stream(r.codes + size_t(chunk) * 16) : z;
+    c.scale = valid ? r.scales[chunk >> 3] : 0.0f;
+  }
+  static __device__ __forceinline__ void dequant(const Chunk& c, uint32_t* w) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) dequant4_e4m3(c.codes[q], c.scale, w[2 * q], w[2 * q + 1]);
+  }
+};
+
+struct FmtNvfp4 {
+  static constexpr int EPL = 32;
+  struct Chunk { u32x4 codes; uint32_t scales; float global; };
+  struct Row { const uint8_t* codes; const uint8_t* scales; float global; };
+  // slot entries: codes [N,K/2] u8 (low nibble = even k), scales [N,K/16] e4m3; global f32
+  static __device__ __forceinline__ Row row(uint64_t codes, uint64_t scales, float global, int j, int K) {
+    Row r;
+    r.codes = reinterpret_cast<const uint8_t*>(codes) + size_t(j) * (K >> 1);
+    r.scales = reinterpret_cast<const uint8_t*>(scales) + size_t(j) * (K >> 4);
+    r.global = global;
+    return r;
+  }
+  static __device__ __forceinline__ void load(Chunk& c, const Row& r, int chunk, bool valid) {
+    const u32x4 z = {0, 0, 0, 0};
+    c.codes = valid ? load16_stream(r.codes + size_t(chunk) * 16) : z;
+    c.scales = valid ? uint32_t(*reinterpret_cast<const uint16_t*>(r.scales + size_t(chunk) * 2)) : 0u;
+    c.global = r.global;
+  }
+  static __device__ __forceinline__ void dequant(const Chunk& c, uint32_t* w) {
+    // s = e4m3(scale) * global first, then e2m1 * s (kernels/nvfp4_linear.cu:83-98 of the reference)
+    const f32x2 sc = e4m3x2_to_f32<false>(c.scales);
+    const float s0 = __fmul_rn(sc.x, c.global), s1 = __fmul_rn(sc.y, c.global);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const float s = q < 2 ? s0 : s1;
+      const uint32_t d = c.codes[q];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t byte = (d >> (8 * i)) & 0xffu;
+        w[4 * q + i] = pack_bf16x2(__fmul_rn(e2m1_to_f32(byte & 15u), s), __fmul_rn(e2m1_to_f32(byte >> 4), s));
+      }
+    }
+  }
+};
+
+struct FmtBf16 {
+  static constexpr int EPL = 8;
+  struct Chunk { u32x4 codes; };
+  struct Row { const uint8_t* codes; };
+  static __device__ __forceinline__ Row row(uint64_t codes, uint64_t, float, int j, int K) {
+    Row r;
+    r.codes = reinterpret_cast<const uint8_t*>(codes) + size_t(j) * K * 2;
+    return r;
+  }
+  static __device__ __forceinline__ void load(Chunk& c, const Row& r, int chunk, bool valid) {
+    const u32x4 z = {0, 0, 0, 0};
+    c.codes = valid ? load16_stream(r.codes + size_t(chunk) * 16) : z;
+  }
+  static __device__ __forceinline__ void dequant(const Chunk& c, uint32_t* w) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) w[q] = c.codes[q];
+  }
+};
+
+template <class F, int S, int NMAT>
+struct UnitBuf { typename F::Chunk c[NMAT][S]; };
+
+// One slab (S steps of 64 lane-chunks) of NMAT weight rows against the n activation rows in LDS;
+// partial sums stay in acc until the row's last slab.
+template <class F, int S, int NMAT, int RG>
+__device__ __forceinline__ void slab_compute(const UnitBuf<F, S, NMAT>& b, const uint8_t* xs, int K, int nchunks, int chunk0,
+                                             int n, int lane, float (&acc)[NMAT][RG]) {
+#pragma unroll
+  for (int s = 0; s < S; ++s) {
+    if (chunk0 + s * 64 < nchunks) {  // wave-uniform: steps wholly past the row do nothing
+      const int chunk = chunk0 + s * 64 + lane;
+      const int cl = chunk < nchunks ? chunk : 0;  // masked lanes carry zero weights; keep the LDS read in range
+      uint32_t w[NMAT][F::EPL / 2];
+#pragma unroll
+      for (int m = 0; m < NMAT; ++m) F::dequant(b.c[m][s], w[m]);
+#pragma unroll
+      for (int r = 0; r < RG; ++r) {
+        if (r < n) {
+          const u32x4* xp = reinterpret_cast<const u32x4*>(xs + size_t(r) * K * 2 + size_t(cl) * (F::EPL * 2));
+#pragma unroll
+          for (int v = 0; v < F::EPL / 8; ++v) {
+            const u32x4 xv = xp[v];
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+#pragma unroll
+              for (int m = 0; m < NMAT; ++m) acc[m][r] = dot2_bf16(w[m][4 * v + q], xv[q], acc[m][r]);
+          }
+        }
+      }
+    }
+  }
+}
+
+}  // namespace ffmoe

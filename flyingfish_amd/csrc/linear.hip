@@ -1,0 +1,238 @@
+// Standalone linears y[M,N] = x[M,K] W[N,K]^T for block-scaled FP8, NVFP4 and BF16 weights
+// (W8A16 / W4A16 arithmetic: BF16-rounded effective weights, FP32 accumulation, BF16 output),
+// the per-128 E4M3 activation quantizer and the elementwise SwiGLU.
+#include "gemv.cuh"
+#include "api.h"
+
+namespace ffmoe {
+
+struct LinearParams {
+  const uint16_t* x;   // [m, k] BF16
+  uint16_t* y;         // [m, n] BF16
+  uint64_t codes, scales;
+  const float* global; // device pointer (NVFP4) or NULL
+  int m, n, k;
+};
+
+// Each block walks a contiguous range of output columns; a wave streams one weight row at a time
+// against up to RG activation rows held in LDS; rows beyond RG are served by further passes.
+template <class F, int S, int RG>
+__global__ __launch_bounds__(256) void k_linear(const LinearParams p) {
+  constexpr int NW = 4;
+  extern __shared__ __align__(16) uint8_t xs[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int K = p.k;
+  const long long lo = (long long)p.n * blockIdx.x / gridDim.x, hi = (long long)p.n * (blockIdx.x + 1) / gridDim.x;
+  const int j0 = int(lo), count = int(hi - lo);
+  const float global = p.global ? *p.global : 1.0f;
+  const int nchunks = K / F::EPL;
+  const int nslabs = (nchunks + S * 64 - 1) / (S * 64);
+  const int my_units = count > wave ? (count - wave + NW - 1) / NW : 0;
+  const int items = my_units * nslabs;
+  for (int r0 = 0; r0 < p.m; r0 += RG) {
+    const int n = p.m - r0 < RG ? p.m - r0 : RG;
+    __syncthreads();
+    {
+      const u32x4* s4 = reinterpret_cast<const u32x4*>(p.x + size_t(r0) * K);
+      u32x4* d4 = reinterpret_cast<u32x4*>(xs);
+      const int words = n * (K >> 3);
+      for (int v = tid; v < words; v += 256) d4[v] = s4[v];
+    }
+    __syncthreads();
+    UnitBuf<F, S, 1> bufA, bufB;
+    float acc[1][RG];
+#pragma unroll
+    for (int r = 0; r < RG; ++r) acc[0][r] = 0.0f;
+    auto issue = [&](UnitBuf<F, S, 1>& b, int t) {
+      const int j = j0 + wave + (t / nslabs) * NW;
+      const int chunk0 = (t % nslabs) * (S * 64);
+      const typename F::Row rw = F::row(p.codes, p.scales, global, j, K);
+#pragma unroll
+      for (int s = 0; s < S; ++s) {
+        const int chunk = chunk0 + s * 64 + lane;
+        F::load(b.c[0][s], rw, chunk, chunk < nchunks);
+      }
+    };
+    auto finish = [&](const UnitBuf<F, S, 1>& b, int t) {
+      const int j = j0 + wave + (t / nslabs) * NW;
+      const int slab = t % nslabs;
+      slab_compute<F, S, 1, RG>(b, xs, K, nchunks, slab * (S * 64), n, lane, acc);
+      if (slab != nslabs - 1) return;
+#pragma unroll
+      for (int r = 0; r < RG; ++r)
+        if (r < n) acc[0][r] = wave_sum(acc[0][r]);
+#pragma unroll
+      for (int r = 0; r < RG; ++r) {
+        if (r < n && lane == r) p.y[size_t(r0 + r) * p.n + j] = f32_to_bf16(acc[0][r]);
+        acc[0][r] = 0.0f;
+      }
+    };
+    int t = 0;
+    if (t < items) issue(bufA, t);
+    while (t < items) {
+      if (t + 1 < items) issue(bufB, t + 1);
+      finish(bufA, t);
+      if (++t >= items) break;
+      if (t + 1 < items) issue(bufA, t + 1);
+      finish(bufB, t);
+      ++t;
+    }
+  }
+}
+
+// Per (row, 128-group): scale = amax * (1/448), code = e4m3(clamp(x / max(scale, 1e-12), +-448))
+// (kernels/fp8_linear.cu:12-48 of the reference). One wave per 4 cells, 16 lanes x 8 elements per cell.
+__global__ __launch_bounds__(256) void k_quant_fp8_128(const uint16_t* __restrict__ x, uint8_t* __restrict__ codes,
+                                                       float* __restrict__ scales, int m, int k) {
+  const int groups = (k + 127) >> 7;
+  const long long cell = (long long)blockIdx.x * 16 + (threadIdx.x >> 4);
+  if (cell >= (long long)m * groups) return;  // whole 16-lane groups leave together
+  const int sub = threadIdx.x & 15;
+  const long long row = cell / groups;
+  const int first = int(cell % groups) * 128 + sub * 8;
+  float v[8];
+  float amax = 0.0f;
+  const uint16_t* src = x + row * k + first;
+  if (first + 8 <= k) {
+    const u32x4 w = load16(src);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) { v[2 * q] = bf16lo(w[q]); v[2 * q + 1] = bf16hi(w[q]); }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = first + i < k ? bf16_to_f32(src[i]) : 0.0f;
+  }
+#pragma unroll
+  for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[i]));
+#pragma unroll
+  for (int off = 8; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 16));
+  const float scale = __fmul_rn(amax, 1.0f / 448.0f);
+  if (sub == 0) scales[cell] = scale;
+  const float divisor = fmaxf(scale, 1.0e-12f);
+  uint32_t out[2] = {0, 0};
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const float q = fminf(448.0f, fmaxf(-448.0f, __fdiv_rn(v[i], divisor)));
+    out[i >> 2] |= uint32_t(e4m3_encode(q)) << (8 * (i & 3));
+  }
+  uint8_t* dst = codes + row * k + first;
+  if (first + 8 <= k) {
+    u32x2 o = {out[0], out[1]};
+    *reinterpret_cast<u32x2*>(dst) = o;
+  } else {
+    for (int i = 0; i < 8; ++i)
+      if (first + i < k) dst[i] = uint8_t(out[i >> 2] >> (8 * (i & 3)));
+  }
+}
+
+// y = swiglu(gate, up), 8 elements per thread (kernels/act.cu:65-99, :125-159 of the reference).
+__global__ __launch_bounds__(256) void k_swiglu(const uint16_t* __restrict__ gate, const uint16_t* __restrict__ up,
+                                                uint16_t* __restrict__ y, long long vectors, int mode, float limit) {
+  const long long v = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (v >= vectors) return;
+  const u32x4 g = load16(gate + v * 8), u = load16(up + v * 8);
+  u32x4 o;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const uint32_t lo = swiglu_bf16(bf16lo(g[q]), bf16lo(u[q]), mode, limit);
+    const uint32_t hi = swiglu_bf16(bf16hi(g[q]), bf16hi(u[q]), mode, limit);
+    o[q] = lo | (hi << 16);
+  }
+  *reinterpret_cast<u32x4*>(y + v * 8) = o;
+}
+
+}  // namespace ffmoe
+
+using namespace ffmoe;
+
+namespace {
+int g_cus_l = 0;
+int num_cus_l() {
+  if (g_cus_l == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+      g_cus_l = n;
+    else
+      g_cus_l = 256;
+  }
+  return g_cus_l;
+}
+
+template <class F>
+int launch_linear(const LinearParams& p, hipStream_t st) {
+  // rows per pass bounded by 64 KiB of LDS
+  int blocks = num_cus_l() * 2;
+  if (blocks > (p.n + 3) / 4) blocks = (p.n + 3) / 4;
+  const size_t row = size_t(p.k) * 2;
+  if (p.m > 1 && 8 * row <= 64 * 1024) hipLaunchKernelGGL((k_linear<F, 4, 8>), dim3(blocks), dim3(256), 8 * row, st, p);
+  else if (p.m > 1 && 4 * row <= 64 * 1024) hipLaunchKernelGGL((k_linear<F, 4, 4>), dim3(blocks), dim3(256), 4 * row, st, p);
+  else hipLaunchKernelGGL((k_linear<F, 4, 1>), dim3(blocks), dim3(256), row, st, p);
+  return ff_launch_status();
+}
+
+int check_linear(const void* w, const void* x, const void* y, int m, int n, int k, int kgran) {
+  FF_REQUIRE(m >= 1 && n >= 1 && k >= kgran && k % kgran == 0, FFMOE_ERR_SHAPE, "linear m=%d n=%d k=%d (k must be a positive multiple of %d)", m, n, k, kgran);
+  FF_REQUIRE(size_t(k) * 2 <= 64 * 1024, FFMOE_ERR_SHAPE, "linear k=%d exceeds the LDS row staging (32768)", k);
+  FF_PTR16(w); FF_PTR16(x); FF_PTR16(y);
+  FF_NO_OVERLAP(y, size_t(m) * n * 2, x, size_t(m) * k * 2);
+  return 0;
+}
+}  // namespace
+
+extern "C" __attribute__((visibility("default"))) int ffmoe_quant_fp8_f32_128(const void* x, void* codes, float* scales, int m, int k, void* stream) {
+  FF_REQUIRE(m >= 1 && k >= 1, FFMOE_ERR_SHAPE, "quant m=%d k=%d", m, k);
+  FF_REQUIRE(k % 8 == 0, FFMOE_ERR_SHAPE, "quant k=%d must be a multiple of 8", k);
+  FF_PTR16(x); FF_PTR16(codes); FF_PTR4(scales);
+  const long long cells = (long long)m * ((k + 127) / 128);
+  FF_NO_OVERLAP(codes, size_t(m) * k, x, size_t(m) * k * 2);
+  FF_NO_OVERLAP(scales, size_t(cells) * 4, x, size_t(m) * k * 2);
+  FF_NO_OVERLAP(scales, size_t(cells) * 4, codes, size_t(m) * k);
+  hipLaunchKernelGGL(k_quant_fp8_128, dim3((unsigned)((cells + 15) / 16)), dim3(256), 0, (hipStream_t)stream,
+                     (const uint16_t*)x, (uint8_t*)codes, scales, m, k);
+  return ff_launch_status();
+}
+
+extern "C" __attribute__((visibility("default"))) int ffmoe_linear_fp8_block(const void* w_codes, const float* w_scales, const void* x, void* y, int m, int n, int k,
+                                      int act_mode, void* scratch, uint64_t scratch_bytes, void* stream) {
+  FF_TRY(check_linear(w_codes, x, y, m, n, k, 16));
+  FF_PTR4(w_scales);
+  if (act_mode == FFMOE_ACT_FP8_BLOCK128) {
+    const uint64_t groups = uint64_t(k + 127) / 128;
+    const uint64_t cb = (uint64_t(m) * k + 255) & ~uint64_t(255);
+    FF_PTR_ALIGNED(scratch, 256);
+    FF_REQUIRE(scratch_bytes >= cb + uint64_t(m) * groups * 4, FFMOE_ERR_SCRATCH, "linear scratch holds %llu bytes, %llu needed",
+               (unsigned long long)scratch_bytes, (unsigned long long)(cb + uint64_t(m) * groups * 4));
+    FF_TRY(ffmoe_quant_fp8_f32_128(x, scratch, (float*)((uint8_t*)scratch + cb), m, k, stream));
+    return ffmoe_linear_fp8_block_w8a8(w_codes, w_scales, scratch, (const float*)((uint8_t*)scratch + cb), y, m, n, k, stream);
+  }
+  FF_REQUIRE(act_mode == FFMOE_ACT_BF16, FFMOE_ERR_UNSUPPORTED, "unknown act_mode %d", act_mode);
+  LinearParams p{(const uint16_t*)x, (uint16_t*)y, (uint64_t)(uintptr_t)w_codes, (uint64_t)(uintptr_t)w_scales, nullptr, m, n, k};
+  return launch_linear<FmtFp8>(p, (hipStream_t)stream);
+}
+
+extern "C" __attribute__((visibility("default"))) int ffmoe_linear_nvfp4(const void* w_codes, const void* w_scales, const float* global_scale, const void* x, void* y,
+                                  int m, int n, int k, void* stream) {
+  FF_TRY(check_linear(w_codes, x, y, m, n, k, 32));
+  FF_PTR2(w_scales); FF_PTR4(global_scale);
+  LinearParams p{(const uint16_t*)x, (uint16_t*)y, (uint64_t)(uintptr_t)w_codes, (uint64_t)(uintptr_t)w_scales, global_scale, m, n, k};
+  return launch_linear<FmtNvfp4>(p, (hipStream_t)stream);
+}
+
+extern "C" __attribute__((visibility("default"))) int ffmoe_gemm_skinny_bf16(const void* w, const void* x, void* y, int m, int n, int k, void* stream) {
+  FF_TRY(check_linear(w, x, y, m, n, k, 8));
+  LinearParams p{(const uint16_t*)x, (uint16_t*)y, (uint64_t)(uintptr_t)w, 0, nullptr, m, n, k};
+  return launch_linear<FmtBf16>(p, (hipStream_t)stream);
+}
+
+extern "C" __attribute__((visibility("default"))) int ffmoe_swiglu(const void* gate, const void* up, void* y, int rows, int width, int mode, float limit, void* stream) {
+  FF_REQUIRE(rows >= 1 && width >= 8 && width % 8 == 0, FFMOE_ERR_SHAPE, "swiglu rows=%d width=%d (width must be a positive multiple of 8)", rows, width);
+  FF_REQUIRE(mode >= 0 && mode <= 3, FFMOE_ERR_UNSUPPORTED, "unknown SwiGLU mode %d", mode);
+  if (mode >= 2) FF_REQUIRE(limit > 0.0f && limit < INFINITY, FFMOE_ERR_SHAPE, "invalid SwiGLU limit %g", (double)limit);
+  FF_PTR16(gate); FF_PTR16(up); FF_PTR16(y);
+  const size_t bytes = size_t(rows) * width * 2;
+  FF_NO_OVERLAP(y, bytes, gate, bytes);
+  FF_NO_OVERLAP(y, bytes, up, bytes);
+  const long long vectors = (long long)rows * width / 8;
+  hipLaunchKernelGGL(k_swiglu, dim3((unsigned)((vectors + 255) / 256)), dim3(256), 0, (hipStream_t)stream, (const uint16_t*)gate,
+                     (const uint16_t*)up, (uint16_t*)y, vectors, mode, limit);
+  return ff_launch_status();
+}

@@ -1,0 +1,349 @@
+// Router kernels: logits (BF16 chain contract / FP32 wave-reduced) and deterministic top-k.
+// Behaviour follows kernels/moe_route.cu of the reference; the mapping to wave64 is new.
+#include "common.cuh"
+#include "api.h"
+
+namespace ffmoe {
+
+// ---------------------------------------------------------------------------------------------
+// logits[r,e] = bf16(fma chain over k ascending). One lane owns one (row, expert) chain
+// (kernels/moe_route.cu:392-403, :536-544). The chain is latency-bound by definition; the lane
+// keeps 8 x 16-byte router words in flight so the dependent fma sequence never waits on memory.
+__global__ __launch_bounds__(64) void k_route_logits_bf16(const uint16_t* __restrict__ x, const uint16_t* __restrict__ router,
+                                                          uint16_t* __restrict__ logits, int rows, int experts, int hidden) {
+  const int e = blockIdx.x * 64 + threadIdx.x;
+  const int row = blockIdx.y;
+  const bool live = e < experts;
+  const int words = hidden >> 3;
+  const u32x4* wr = reinterpret_cast<const u32x4*>(router + size_t(live ? e : 0) * hidden);
+  const u32x4* xr = reinterpret_cast<const u32x4*>(x + size_t(row) * hidden);
+  float acc = 0.0f;
+  constexpr int PF = 8;
+  int c = 0;
+  for (; c + PF <= words; c += PF) {
+    u32x4 wv[PF];
+#pragma unroll
+    for (int p = 0; p < PF; ++p) wv[p] = wr[c + p];
+#pragma unroll
+    for (int p = 0; p < PF; ++p) {
+      const u32x4 xv = xr[c + p];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        acc = __fmaf_rn(bf16lo(xv[q]), bf16lo(wv[p][q]), acc);
+        acc = __fmaf_rn(bf16hi(xv[q]), bf16hi(wv[p][q]), acc);
+      }
+    }
+  }
+  for (; c < words; ++c) {
+    const u32x4 wv = wr[c];
+    const u32x4 xv = xr[c];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      acc = __fmaf_rn(bf16lo(xv[q]), bf16lo(wv[q]), acc);
+      acc = __fmaf_rn(bf16hi(xv[q]), bf16hi(wv[q]), acc);
+    }
+  }
+  if (live) logits[size_t(row) * experts + e] = f32_to_bf16(acc);
+}
+
+// FP32 logits: one wave per expert, RB rows at a time; lane L chains the 8-element vectors
+// L, L+64, ...; lane partials are summed with a shuffle-down tree 32..1 (lane 0 holds the sum).
+template <int RB>
+__global__ __launch_bounds__(256) void k_route_logits_f32(const uint16_t* __restrict__ x, const uint16_t* __restrict__ router,
+                                                          float* __restrict__ logits, int rows, int experts, int hidden) {
+  const int lane = threadIdx.x & 63;
+  const int e = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int r0 = blockIdx.y * RB;
+  if (e >= experts) return;
+  const int words = hidden >> 3;
+  const u32x4* wr = reinterpret_cast<const u32x4*>(router + size_t(e) * hidden);
+  float acc[RB];
+#pragma unroll
+  for (int r = 0; r < RB; ++r) acc[r] = 0.0f;
+  for (int v = lane; v < words; v += 64) {
+    const u32x4 wv = wr[v];
+#pragma unroll
+    for (int r = 0; r < RB; ++r) {
+      if (r0 + r < rows) {
+        const u32x4 xv = reinterpret_cast<const u32x4*>(x + size_t(r0 + r) * hidden)[v];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          acc[r] = __fmaf_rn(bf16lo(xv[q]), bf16lo(wv[q]), acc[r]);
+          acc[r] = __fmaf_rn(bf16hi(xv[q]), bf16hi(wv[q]), acc[r]);
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < RB; ++r) {
+    float v = acc[r];
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      const float o = __shfl_down(v, off, 64);
+      v = __fadd_rn(v, (lane + off < 64) ? o : 0.0f);  // lanes past the end contribute nothing to lane 0
+    }
+    if (lane == 0 && r0 + r < rows) logits[size_t(r0 + r) * experts + e] = v;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Block-wide arg-max under (value desc, id asc); every thread receives the winner.
+struct Best { float v; int id; };
+__device__ __forceinline__ Best better(Best a, Best b) {
+  return (b.v > a.v || (b.v == a.v && b.id < a.id)) ? b : a;
+}
+__device__ __forceinline__ Best block_argmax(Best mine, float* s_v, int* s_id, int nwaves) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    Best o;
+    o.v = __shfl_xor(mine.v, off, 64);
+    o.id = __shfl_xor(mine.id, off, 64);
+    mine = better(mine, o);
+  }
+  if (nwaves == 1) return mine;
+  __syncthreads();  // previous round's readers are done with s_v/s_id
+  if (lane == 0) { s_v[wave] = mine.v; s_id[wave] = mine.id; }
+  __syncthreads();
+  Best r; r.v = s_v[0]; r.id = s_id[0];
+  for (int w = 1; w < nwaves; ++w) { Best o; o.v = s_v[w]; o.id = s_id[w]; r = better(r, o); }
+  return r;
+}
+
+// Softmax / sigmoid top-k over BF16 logits (kernels/moe_route.cu:154-301). One block per row, thread e
+// owns expert e. The softmax denominator is summed exactly as the reference's 32-lane warp trees.
+__global__ void k_route_topk(const uint16_t* __restrict__ logits, int* __restrict__ ids, uint16_t* __restrict__ weights,
+                             int experts, int top_k, int score_mode) {
+  __shared__ float s_red[32];
+  __shared__ float s_v[16];
+  __shared__ int s_id[16];
+  __shared__ float s_sel[FFMOE_MAX_TOP_K];
+  __shared__ int s_selid[FFMOE_MAX_TOP_K];
+  const int tid = threadIdx.x, row = blockIdx.x;
+  const int e = tid;
+  const bool live = e < experts;
+  const int nwaves = blockDim.x >> 6;
+  const int nw32 = blockDim.x >> 5;  // 32-lane groups, the reference's warps
+  const float logit = live ? bf16_to_f32(logits[size_t(row) * experts + e]) : -INFINITY;
+  float score;
+  if (score_mode == FFMOE_SCORE_SOFTMAX) {
+    float m = logit;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
+    if ((tid & 63) == 0) s_v[tid >> 6] = m;
+    __syncthreads();
+    for (int w = 0; w < nwaves; ++w) m = fmaxf(m, s_v[w]);
+    __syncthreads();
+    const float ev = live ? det_expf(__fsub_rn(logit, m)) : 0.0f;
+    float v = ev;
+#pragma unroll
+    for (int off = 16; off > 0; off >>= 1) {
+      const float o = __shfl_down(v, off, 32);
+      v = __fadd_rn(v, ((tid & 31) + off < 32) ? o : 0.0f);
+    }
+    if (tid < 32) s_red[tid] = 0.0f;
+    __syncthreads();
+    if ((tid & 31) == 0) s_red[tid >> 5] = v;
+    __syncthreads();
+    if (tid < 32) {
+      v = tid < nw32 ? s_red[tid] : 0.0f;
+#pragma unroll
+      for (int off = 16; off > 0; off >>= 1) {
+        const float o = __shfl_down(v, off, 32);
+        v = __fadd_rn(v, (tid + off < 32) ? o : 0.0f);
+      }
+      if (tid == 0) s_red[0] = v;
+    }
+    __syncthreads();
+    score = live ? __fdiv_rn(ev, s_red[0]) : -1.0f;
+  } else {
+    score = live ? sigmoid1(logit) : -1.0f;
+  }
+  bool taken = false;
+  for (int r = 0; r < top_k; ++r) {
+    Best mine;
+    mine.v = (!taken && live) ? score : -1.0f;
+    mine.id = live ? e : 0x7fffffff;
+    const Best win = block_argmax(mine, s_v, s_id, nwaves);
+    if (live && !taken && e == win.id) {
+      s_sel[r] = score;
+      s_selid[r] = e;
+      taken = true;
+    }
+  }
+  __syncthreads();
+  if (tid < top_k) {
+    float tsum = 0.0f;
+    for (int r = 0; r < top_k; ++r) tsum = __fadd_rn(tsum, s_sel[r]);
+    const float den = score_mode == FFMOE_SCORE_SOFTMAX ? tsum : __fadd_rn(tsum, 1.0e-20f);
+    ids[size_t(row) * top_k + tid] = s_selid[tid];
+    weights[size_t(row) * top_k + tid] = f32_to_bf16(__fdiv_rn(s_sel[tid], den));
+  }
+}
+
+// noaux_tc selection over FP32 logits (kernels/moe_route.cu:315-390), with the optional group filter.
+__global__ void k_route_topk_noaux(const float* __restrict__ logits, const float* __restrict__ bias, int bias_row_stride,
+                                   int* __restrict__ ids, void* __restrict__ weights, int weights_f32, int experts,
+                                   int top_k, int score_mode, float routed_scaling, int n_group, int topk_group) {
+  __shared__ float s_v[16];
+  __shared__ int s_id[16];
+  __shared__ float s_sel[FFMOE_MAX_TOP_K];
+  __shared__ int s_selid[FFMOE_MAX_TOP_K];
+  __shared__ float s_score[FFMOE_MAX_EXPERTS];
+  __shared__ float s_group[FFMOE_MAX_EXPERTS];
+  __shared__ unsigned char s_keep[FFMOE_MAX_EXPERTS];
+  const int tid = threadIdx.x, row = blockIdx.x;
+  const int e = tid;
+  const bool live = e < experts;
+  const int nwaves = blockDim.x >> 6;
+  float score = -1.0f, select = -INFINITY;
+  if (live) {
+    const float l = logits[size_t(row) * experts + e];
+    if (score_mode == FFMOE_NOAUX_SIGMOID) {
+      score = sigmoid1(l);
+    } else {
+      const float softplus = __fadd_rn(fmaxf(l, 0.0f), det_log1pf_unit(det_expf(-fabsf(l))));
+      score = __builtin_sqrtf(softplus);  // correctly rounded (hipcc default); __fsqrt_rn is the approximate native sqrt
+    }
+    select = __fadd_rn(score, bias ? bias[size_t(row) * bias_row_stride + e] : 0.0f);
+  }
+  bool allowed = live;
+  if (n_group > 1) {
+    s_score[tid] = select;
+    __syncthreads();
+    const int per = experts / n_group;
+    if (tid < n_group) {
+      float a = -INFINITY, b = -INFINITY;
+      for (int i = tid * per; i < (tid + 1) * per; ++i) {
+        const float v = s_score[i];
+        if (v > a) { b = a; a = v; } else if (v > b) { b = v; }
+      }
+      s_group[tid] = __fadd_rn(a, b);
+      s_keep[tid] = 0;
+    }
+    __syncthreads();
+    if (tid == 0) {
+      for (int r = 0; r < topk_group; ++r) {
+        int best = -1;
+        for (int g = 0; g < n_group; ++g)
+          if (!s_keep[g] && (best < 0 || s_group[g] > s_group[best])) best = g;
+        s_keep[best] = 1;
+      }
+    }
+    __syncthreads();
+    allowed = live && s_keep[e / per] != 0;
+    __syncthreads();
+  }
+  bool taken = false;
+  for (int r = 0; r < top_k; ++r) {
+    Best mine;
+    mine.v = (!taken && allowed) ? select : -INFINITY;
+    mine.id = (!taken && allowed) ? e : 0x7fffffff;
+    const Best win = block_argmax(mine, s_v, s_id, nwaves);
+    if (allowed && !taken && e == win.id) {
+      s_sel[r] = score;
+      s_selid[r] = e;
+      taken = true;
+    }
+  }
+  __syncthreads();
+  if (tid < top_k) {
+    float tsum = 0.0f;
+    for (int r = 0; r < top_k; ++r) tsum = __fadd_rn(tsum, s_sel[r]);
+    const float w = __fmul_rn(__fdiv_rn(s_sel[tid], __fadd_rn(tsum, 1.0e-20f)), routed_scaling);
+    ids[size_t(row) * top_k + tid] = s_selid[tid];
+    if (weights_f32) reinterpret_cast<float*>(weights)[size_t(row) * top_k + tid] = w;
+    else reinterpret_cast<uint16_t*>(weights)[size_t(row) * top_k + tid] = f32_to_bf16(w);
+  }
+}
+
+}  // namespace ffmoe
+
+using namespace ffmoe;
+
+static int check_route_dims(int rows, int experts, int hidden) {
+  FF_REQUIRE(rows >= 1 && experts >= 1 && experts <= FFMOE_MAX_EXPERTS, FFMOE_ERR_SHAPE,
+             "router rows=%d experts=%d outside [1, %d]", rows, experts, FFMOE_MAX_EXPERTS);
+  FF_REQUIRE(hidden >= 8 && (hidden & 7) == 0, FFMOE_ERR_SHAPE, "router hidden=%d must be a positive multiple of 8", hidden);
+  return 0;
+}
+
+extern "C" __attribute__((visibility("default"))) int ffmoe_route_logits_bf16(const void* x, const void* router, void* logits, int rows, int experts, int hidden,
+                                       void* stream) {
+  FF_TRY(check_route_dims(rows, experts, hidden));
+  FF_PTR16(x); FF_PTR16(router); FF_PTR16(logits);
+  FF_NO_OVERLAP(logits, size_t(rows) * experts * 2, x, size_t(rows) * hidden * 2);
+  FF_NO_OVERLAP(logits, size_t(rows) * experts * 2, router, size_t(experts) * hidden * 2);
+  hipLaunchKernelGGL(k_route_logits_bf16, dim3((experts + 63) / 64, rows), dim3(64), 0, (hipStream_t)stream,
+                     (const uint16_t*)x, (const uint16_t*)router, (uint16_t*)logits, rows, experts, hidden);
+  return ff_launch_status();
+}
+
+extern "C" __attribute__((visibility("default"))) int ffmoe_route_logits_f32(const void* x, const void* router, float* logits, int rows, int experts, int hidden,
+                                      void* stream) {
+  FF_TRY(check_route_dims(rows, experts, hidden));
+  FF_PTR16(x); FF_PTR16(router); FF_PTR4(logits);
+  FF_NO_OVERLAP(logits, size_t(rows) * experts * 4, x, size_t(rows) * hidden * 2);
+  FF_NO_OVERLAP(logits, size_t(rows) * experts * 4, router, size_t(experts) * hidden * 2);
+  if (rows == 1)
+    hipLaunchKernelGGL(k_route_logits_f32<1>, dim3((experts + 3) / 4, 1), dim3(256), 0, (hipStream_t)stream,
+                       (const uint16_t*)x, (const uint16_t*)router, logits, rows, experts, hidden);
+  else
+    hipLaunchKernelGGL(k_route_logits_f32<8>, dim3((experts + 3) / 4, (rows + 7) / 8), dim3(256), 0, (hipStream_t)stream,
+                       (const uint16_t*)x, (const uint16_t*)router, logits, rows, experts, hidden);
+  return ff_launch_status();
+}
+
+static int check_topk_dims(int rows, int experts, int top_k, bool allow_all) {
+  FF_REQUIRE(rows >= 1 && experts >= 1 && experts <= FFMOE_MAX_EXPERTS, FFMOE_ERR_SHAPE,
+             "router rows=%d experts=%d outside [1, %d]", rows, experts, FFMOE_MAX_EXPERTS);
+  FF_REQUIRE(top_k >= 1 && top_k <= FFMOE_MAX_TOP_K && (allow_all ? top_k <= experts : top_k < experts), FFMOE_ERR_SHAPE,
+             "top_k=%d outside [1, %d] or not below experts=%d", top_k, FFMOE_MAX_TOP_K, experts);
+  return 0;
+}
+
+extern "C" __attribute__((visibility("default"))) int ffmoe_route_topk(const void* logits, int* ids, void* weights, int rows, int experts, int top_k, int score,
+                                void* stream) {
+  FF_TRY(check_topk_dims(rows, experts, top_k, false));
+  FF_REQUIRE(score == FFMOE_SCORE_SOFTMAX || score == FFMOE_SCORE_SIGMOID, FFMOE_ERR_UNSUPPORTED, "unknown router score %d", score);
+  FF_PTR16(logits); FF_PTR4(ids); FF_PTR2(weights);
+  FF_NO_OVERLAP(ids, size_t(rows) * top_k * 4, logits, size_t(rows) * experts * 2);
+  FF_NO_OVERLAP(weights, size_t(rows) * top_k * 2, logits, size_t(rows) * experts * 2);
+  FF_NO_OVERLAP(ids, size_t(rows) * top_k * 4, weights, size_t(rows) * top_k * 2);
+  const int threads = (experts + 63) & ~63;
+  hipLaunchKernelGGL(k_route_topk, dim3(rows), dim3(threads), 0, (hipStream_t)stream, (const uint16_t*)logits, ids,
+                     (uint16_t*)weights, experts, top_k, score);
+  return ff_launch_status();
+}
+
+extern "C" __attribute__((visibility("default"))) int ffmoe_route_topk_noaux(const float* logits, const float* bias, int bias_row_stride, int* ids, void* weights,
+                                      int weights_f32, int rows, int experts, int top_k, int score_mode,
+                                      float routed_scaling, int n_group, int topk_group, void* stream) {
+  FF_TRY(check_topk_dims(rows, experts, top_k, true));
+  FF_REQUIRE(score_mode == 0 || score_mode == 1, FFMOE_ERR_UNSUPPORTED, "unknown noaux score mode %d", score_mode);
+  FF_REQUIRE(routed_scaling > 0.0f && routed_scaling < INFINITY, FFMOE_ERR_SHAPE, "invalid routed scaling %g", (double)routed_scaling);
+  FF_REQUIRE(bias_row_stride == 0 || bias_row_stride == experts, FFMOE_ERR_SHAPE, "bias row stride %d must be 0 or experts", bias_row_stride);
+  FF_REQUIRE(n_group >= 1 && topk_group >= 1 && topk_group <= n_group && experts % n_group == 0, FFMOE_ERR_SHAPE,
+             "invalid grouping n_group=%d topk_group=%d experts=%d", n_group, topk_group, experts);
+  FF_REQUIRE(n_group == 1 || (experts / n_group >= 2 && top_k <= topk_group * (experts / n_group)), FFMOE_ERR_SHAPE,
+             "groups of %d experts cannot supply top_k=%d from %d groups", experts / n_group, top_k, topk_group);
+  FF_PTR4(logits); FF_PTR4(ids);
+  if (bias) FF_PTR4(bias);
+  if (weights_f32) { FF_PTR4(weights); } else { FF_PTR2(weights); }
+  const size_t wbytes = size_t(rows) * top_k * (weights_f32 ? 4 : 2);
+  FF_NO_OVERLAP(ids, size_t(rows) * top_k * 4, logits, size_t(rows) * experts * 4);
+  FF_NO_OVERLAP(weights, wbytes, logits, size_t(rows) * experts * 4);
+  FF_NO_OVERLAP(ids, size_t(rows) * top_k * 4, weights, wbytes);
+  const int threads = (experts + 63) & ~63;
+  hipLaunchKernelGGL(k_route_topk_noaux, dim3(rows), dim3(threads), 0, (hipStream_t)stream, logits, bias, bias_row_stride,
+                     ids, weights, weights_f32, experts, top_k, score_mode, routed_scaling, n_group, topk_group);
+  return ff_launch_status();
+}
+
+extern "C" __attribute__((visibility("default"))) int ffmoe_route_decode(const void* x, const void* router, void* logits, int* ids, void* weights, int rows,
+                                  int experts, int hidden, int top_k, int score, void* stream) {
+  FF_TRY(check_topk_dims(rows, experts, top_k, false));
+  int rc = ffmoe_route_logits_bf16(x, router, logits, rows, experts, hidden, stream);
+  if (rc) return rc;
+  return ffmoe_route_topk(logits, ids, weights, rows, experts, top_k, score, stream);
+}

@@ -1,0 +1,314 @@
+"""Host-side operator objects over libffmoe, mirroring the reference's operator structs.
+
+  RouteOps      <- src/backend/cuda/moe/route.rs   (RouteOps::route / logits_f32 / topk_noaux)
+  ExpertTable   <- NativeMoe's slots[E,6] table    (src/backend/cuda/moe/decode.rs:683-698)
+  DecodeOps     <- src/backend/cuda/moe/decode.rs  (DecodeOps::contribute*, decode_scratch_bytes_mixed)
+  CombineOps    <- src/backend/cuda/moe/combine.rs (shared_scale, combine, combine_bf16, combine_accum, combine_routed)
+  Fp8Ops / NvFp4Ops / skinny <- src/backend/cuda/linear.rs
+  NativeMoe     <- decode.rs:771-777, :1187-1297   (route -> contribute -> combine for one layer)
+
+Tensors are torch CUDA tensors used as plain device buffers; the ops own nothing except scratch.
+Errors from the library are raised as capi.FfmoeError with the library's message.
+"""
+import ctypes
+
+import torch
+
+from . import capi
+
+_BF16 = torch.bfloat16
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else None
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _dense(t, name):
+    if not t.is_contiguous():
+        raise ValueError("%s must be dense row-major" % name)
+    return t
+
+
+class ExpertTable:
+    """All experts of one layer, resident in device memory.
+
+    FP8 block slot layout (src/experts/catalogue.rs:180-222): gate codes [I,H], up codes [I,H],
+    down codes [H,I], then gate/up scales [ceil(I/128), ceil(H/128)] f32 and down scales
+    [ceil(H/128), ceil(I/128)] f32. NVFP4 slot: packed codes then E4M3 group-16 scales, same order.
+    """
+
+    def __init__(self, fmt, experts, hidden, inter, storage, slots, global_scales=None, valid=None):
+        self.format, self.experts, self.hidden, self.inter = fmt, experts, hidden, inter
+        self.storage, self.slots, self.global_scales, self.valid = storage, slots, global_scales, valid
+
+    @staticmethod
+    def slot_layout(fmt, hidden, inter):
+        """byte offsets of {gate codes, gate scales, up codes, up scales, down codes, down scales} and slot size."""
+        if fmt == capi.FMT_FP8_BLOCK128:
+            w = hidden * inter
+            sgu = -(-inter // 128) * -(-hidden // 128) * 4
+            sd = -(-hidden // 128) * -(-inter // 128) * 4
+            offs = [0, 3 * w, w, 3 * w + sgu, 2 * w, 3 * w + 2 * sgu]
+            size = 3 * w + 2 * sgu + sd
+        elif fmt == capi.FMT_NVFP4:
+            w = hidden * inter // 2
+            s = hidden * inter // 16
+            offs = [0, 3 * w, w, 3 * w + s, 2 * w, 3 * w + 2 * s]
+            size = 3 * w + 3 * s
+        elif fmt == capi.FMT_BF16:
+            w = hidden * inter * 2
+            offs = [0, 0, w, 0, 2 * w, 0]
+            size = 3 * w
+        else:
+            raise ValueError("unknown format")
+        size = (size + 255) // 256 * 256
+        return offs, size
+
+    @classmethod
+    def allocate(cls, fmt, experts, hidden, inter, device="cuda"):
+        offs, size = cls.slot_layout(fmt, hidden, inter)
+        storage = torch.empty((experts, size), dtype=torch.uint8, device=device)
+        base = storage.data_ptr()
+        table = torch.tensor([[base + e * size + o for o in offs] for e in range(experts)], dtype=torch.int64)
+        slots = table.to(device)
+        gs = torch.ones((experts, 3), dtype=torch.float32, device=device) if fmt == capi.FMT_NVFP4 else None
+        t = cls(fmt, experts, hidden, inter, storage, slots, gs)
+        t.offsets, t.slot_bytes = offs, size
+        return t
+
+    def expert_views(self, e):
+        """(gate codes, gate scales, up codes, up scales, down codes, down scales) views of expert e."""
+        H, I = self.hidden, self.inter
+        row = self.storage[e]
+        o = self.offsets
+        if self.format == capi.FMT_FP8_BLOCK128:
+            sgu = (-(-I // 128), -(-H // 128))
+            sd = (-(-H // 128), -(-I // 128))
+            f32 = lambda off, shape: row[off:off + shape[0] * shape[1] * 4].view(torch.float32).view(shape)
+            return (row[o[0]:o[0] + I * H].view(I, H), f32(o[1], sgu), row[o[2]:o[2] + I * H].view(I, H), f32(o[3], sgu),
+                    row[o[4]:o[4] + H * I].view(H, I), f32(o[5], sd))
+        if self.format == capi.FMT_NVFP4:
+            return (row[o[0]:o[0] + I * H // 2].view(I, H // 2), row[o[1]:o[1] + I * H // 16].view(I, H // 16),
+                    row[o[2]:o[2] + I * H // 2].view(I, H // 2), row[o[3]:o[3] + I * H // 16].view(I, H // 16),
+                    row[o[4]:o[4] + H * I // 2].view(H, I // 2), row[o[5]:o[5] + H * I // 16].view(H, I // 16))
+        bf = lambda off, shape: row[off:off + shape[0] * shape[1] * 2].view(_BF16).view(shape)
+        return (bf(o[0], (I, H)), None, bf(o[2], (I, H)), None, bf(o[4], (H, I)), None)
+
+    def weight_bytes_per_expert(self):
+        H, I = self.hidden, self.inter
+        if self.format == capi.FMT_FP8_BLOCK128:
+            return 3 * H * I + 4 * (2 * -(-I // 128) * -(-H // 128) + -(-H // 128) * -(-I // 128))
+        if self.format == capi.FMT_NVFP4:
+            return 3 * H * I // 2 + 3 * H * I // 16 + 12
+        return 3 * H * I * 2
+
+    def c_struct(self):
+        return capi.ExpertTable(self.format, self.experts, self.hidden, self.inter, self.slots.data_ptr(),
+                                self.valid.data_ptr() if self.valid is not None else None,
+                                self.global_scales.data_ptr() if self.global_scales is not None else None)
+
+    def shared_struct(self, e=0):
+        """Describe expert e of this table as an always-on shared expert."""
+        s = capi.SharedExpert()
+        s.format, s.inter = self.format, self.inter
+        row = self.slots[e].tolist()
+        for i in range(6):
+            s.slot[i] = row[i]
+        gl = self.global_scales[e].tolist() if self.global_scales is not None else [1.0, 1.0, 1.0]
+        for i in range(3):
+            s.global_scales[i] = gl[i]
+        return s
+
+
+class RouteOps:
+    @staticmethod
+    def logits_bf16(x, router):
+        rows, hidden = x.shape
+        experts = router.shape[0]
+        out = torch.empty((rows, experts), dtype=_BF16, device=x.device)
+        capi.check(capi.lib().ffmoe_route_logits_bf16(_ptr(_dense(x, "x")), _ptr(_dense(router, "router")), _ptr(out), rows, experts, hidden, _stream()))
+        return out
+
+    @staticmethod
+    def logits_f32(x, router, out=None):
+        rows, hidden = x.shape
+        experts = router.shape[0]
+        if out is None:
+            out = torch.empty((rows, experts), dtype=torch.float32, device=x.device)
+        capi.check(capi.lib().ffmoe_route_logits_f32(_ptr(_dense(x, "x")), _ptr(_dense(router, "router")), _ptr(out), rows, experts, hidden, _stream()))
+        return out
+
+    @staticmethod
+    def topk(logits, top_k, score=capi.SCORE_SOFTMAX):
+        rows, experts = logits.shape
+        ids = torch.empty((rows, top_k), dtype=torch.int32, device=logits.device)
+        w = torch.empty((rows, top_k), dtype=_BF16, device=logits.device)
+        capi.check(capi.lib().ffmoe_route_topk(_ptr(_dense(logits, "logits")), _ptr(ids), _ptr(w), rows, experts, top_k, score, _stream()))
+        return ids, w
+
+    @staticmethod
+    def topk_noaux(logits, bias, top_k, score_mode=capi.NOAUX_SIGMOID, routed_scaling=1.0, n_group=1, topk_group=1,
+                   weights_f32=True, out=None):
+        rows, experts = logits.shape
+        if out is None:
+            ids = torch.empty((rows, top_k), dtype=torch.int32, device=logits.device)
+            w = torch.empty((rows, top_k), dtype=torch.float32 if weights_f32 else _BF16, device=logits.device)
+        else:
+            ids, w = out
+        stride = 0 if bias is None or bias.dim() == 1 else experts
+        capi.check(capi.lib().ffmoe_route_topk_noaux(_ptr(_dense(logits, "logits")), _ptr(bias), stride, _ptr(ids), _ptr(w),
+                                                     int(weights_f32), rows, experts, top_k, score_mode, routed_scaling,
+                                                     n_group, topk_group, _stream()))
+        return ids, w
+
+    @staticmethod
+    def route(x, router, top_k, score=capi.SCORE_SOFTMAX):
+        rows, hidden = x.shape
+        experts = router.shape[0]
+        logits = torch.empty((rows, experts), dtype=_BF16, device=x.device)
+        ids = torch.empty((rows, top_k), dtype=torch.int32, device=x.device)
+        w = torch.empty((rows, top_k), dtype=_BF16, device=x.device)
+        capi.check(capi.lib().ffmoe_route_decode(_ptr(_dense(x, "x")), _ptr(_dense(router, "router")), _ptr(logits), _ptr(ids), _ptr(w),
+                                                 rows, experts, hidden, top_k, score, _stream()))
+        return ids, w, logits
+
+
+class DecodeOps:
+    """Expert contributions for a decode batch; owns its scratch arena and output buffers."""
+
+    def __init__(self, table, shared=None, rows=1, top_k=8, act_mode=capi.ACT_BF16, swiglu=capi.SWIGLU_TWICE, swiglu_limit=0.0,
+                 routed_weight=capi.WEIGHT_AFTER_DOWN_BF16, weights_f32=False):
+        self.table, self.shared = table, shared
+        self.rows, self.top_k = rows, top_k
+        self.cfg = (act_mode, swiglu, swiglu_limit, routed_weight, int(weights_f32))
+        dev = table.slots.device
+        si = shared.inter if shared is not None else 0
+        nbytes = capi.lib().ffmoe_decode_scratch_bytes(rows, top_k, table.experts, table.hidden, table.inter, si)
+        self.scratch = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+        self.contributions = torch.empty((rows, top_k, table.hidden), dtype=_BF16, device=dev)
+        self.shared_out = torch.empty((rows, table.hidden), dtype=_BF16, device=dev) if shared is not None else None
+        self.done = torch.zeros((rows, top_k), dtype=torch.int32, device=dev)
+        self._table_c = table.c_struct()
+        self._shared_c = shared
+
+    def contribute(self, x, ids, weights, active=None):
+        act_mode, swiglu, limit, rw, wf32 = self.cfg
+        d = capi.Decode(self.rows, self.top_k, act_mode, swiglu, limit, rw, wf32,
+                        x.data_ptr(), ids.data_ptr(), active.data_ptr() if active is not None else None, weights.data_ptr(),
+                        self.contributions.data_ptr(), self.shared_out.data_ptr() if self.shared_out is not None else None,
+                        self.done.data_ptr(), self.scratch.data_ptr(), self.scratch.numel())
+        capi.check(capi.lib().ffmoe_decode_contribute(ctypes.byref(self._table_c),
+                                                      ctypes.byref(self._shared_c) if self._shared_c is not None else None,
+                                                      ctypes.byref(d), _stream()))
+        return self.contributions, self.shared_out
+
+
+class CombineOps:
+    @staticmethod
+    def shared_scale(x, seg):
+        rows, hidden = x.shape
+        out = torch.empty((rows,), dtype=_BF16, device=x.device)
+        capi.check(capi.lib().ffmoe_shared_scale(_ptr(x), _ptr(seg), _ptr(out), rows, hidden, _stream()))
+        return out
+
+    @staticmethod
+    def combine(contributions, shared_out, ids, mode, scale=None, done=None, final_active=None, status=None, out=None):
+        rows, top_k, hidden = contributions.shape
+        y = out if out is not None else torch.empty((rows, hidden), dtype=_BF16, device=contributions.device)
+        capi.check(capi.lib().ffmoe_combine(_ptr(contributions), _ptr(shared_out), _ptr(scale), _ptr(ids), _ptr(done),
+                                            _ptr(final_active), _ptr(y), _ptr(status), rows, top_k, hidden, mode, _stream()))
+        return y
+
+
+class Fp8Ops:
+    @staticmethod
+    def quantize(x):
+        m, k = x.shape
+        codes = torch.empty((m, k), dtype=torch.uint8, device=x.device)
+        scales = torch.empty((m, -(-k // 128)), dtype=torch.float32, device=x.device)
+        capi.check(capi.lib().ffmoe_quant_fp8_f32_128(_ptr(x), _ptr(codes), _ptr(scales), m, k, _stream()))
+        return codes, scales
+
+    @staticmethod
+    def linear(w_codes, w_scales, x, act_mode=capi.ACT_BF16, out=None):
+        n, k = w_codes.shape
+        m = x.shape[0]
+        y = out if out is not None else torch.empty((m, n), dtype=_BF16, device=x.device)
+        scratch = None
+        nbytes = 0
+        if act_mode == capi.ACT_FP8_BLOCK128:
+            nbytes = (m * k + 255) // 256 * 256 + m * -(-k // 128) * 4
+            scratch = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
+        capi.check(capi.lib().ffmoe_linear_fp8_block(_ptr(w_codes), _ptr(w_scales), _ptr(x), _ptr(y), m, n, k, act_mode,
+                                                     _ptr(scratch), nbytes, _stream()))
+        return y
+
+    @staticmethod
+    def linear_w8a8(w_codes, w_scales, x_codes, x_scales, out=None):
+        n, k = w_codes.shape
+        m = x_codes.shape[0]
+        y = out if out is not None else torch.empty((m, n), dtype=_BF16, device=x_codes.device)
+        capi.check(capi.lib().ffmoe_linear_fp8_block_w8a8(_ptr(w_codes), _ptr(w_scales), _ptr(x_codes), _ptr(x_scales), _ptr(y), m, n, k, _stream()))
+        return y
+
+
+class NvFp4Ops:
+    @staticmethod
+    def gemm(codes, scales, global_scale, x, out=None):
+        n, kh = codes.shape
+        k = kh * 2
+        m = x.shape[0]
+        y = out if out is not None else torch.empty((m, n), dtype=_BF16, device=x.device)
+        capi.check(capi.lib().ffmoe_linear_nvfp4(_ptr(codes), _ptr(scales), _ptr(global_scale), _ptr(x), _ptr(y), m, n, k, _stream()))
+        return y
+
+
+def gemm_skinny_bf16(w, x, out=None):
+    n, k = w.shape
+    m = x.shape[0]
+    y = out if out is not None else torch.empty((m, n), dtype=_BF16, device=x.device)
+    capi.check(capi.lib().ffmoe_gemm_skinny_bf16(_ptr(w), _ptr(x), _ptr(y), m, n, k, _stream()))
+    return y
+
+
+def swiglu(gate, up, mode=capi.SWIGLU_TWICE, limit=0.0):
+    rows, width = gate.shape
+    y = torch.empty_like(gate)
+    capi.check(capi.lib().ffmoe_swiglu(_ptr(gate), _ptr(up), _ptr(y), rows, width, mode, limit, _stream()))
+    return y
+
+
+class NativeMoe:
+    """One MoE layer, decode: FP32 router logits -> noaux top-k -> expert contributions -> combine.
+
+    Mirrors NativeMoe::new / run (decode.rs:683-698, :771-777, :1187-1297): geometry {hidden, intermediate, experts,
+    top_k, scaling, limit}, weights {router, bias, slots, shared}, fixed row count, run(x) -> y.
+    """
+
+    def __init__(self, table, shared, router, bias, rows, top_k, routed_scaling=1.0, n_group=1, topk_group=1,
+                 swiglu=capi.SWIGLU_TWICE, swiglu_limit=0.0, routed_weight=capi.WEIGHT_BEFORE_CONTRIBUTION_BF16,
+                 combine_mode=capi.COMBINE_BF16):
+        self.table, self.router, self.bias = table, router, bias
+        self.rows, self.top_k = rows, top_k
+        self.routing = (routed_scaling, n_group, topk_group)
+        self.combine_mode = combine_mode
+        dev = router.device
+        self.decode = DecodeOps(table, shared, rows, top_k, capi.ACT_BF16, swiglu, swiglu_limit, routed_weight, weights_f32=True)
+        self.logits = torch.empty((rows, table.experts), dtype=torch.float32, device=dev)
+        self.ids = torch.empty((rows, top_k), dtype=torch.int32, device=dev)
+        self.weights = torch.empty((rows, top_k), dtype=torch.float32, device=dev)
+        self.y = torch.empty((rows, table.hidden), dtype=_BF16, device=dev)
+        self.status = torch.zeros(1, dtype=torch.int32, device=dev)
+
+    def run(self, x):
+        scaling, ng, kg = self.routing
+        RouteOps.logits_f32(x, self.router, out=self.logits)
+        RouteOps.topk_noaux(self.logits, self.bias, self.top_k, capi.NOAUX_SIGMOID, scaling, ng, kg, True, out=(self.ids, self.weights))
+        self.decode.done.zero_()
+        contrib, shared_out = self.decode.contribute(x, self.ids, self.weights)
+        mode = self.combine_mode if shared_out is not None else capi.COMBINE_ROUTED
+        return CombineOps.combine(contrib, shared_out, self.ids, mode, done=self.decode.done, status=self.status, out=self.y)

@@ -1,0 +1,84 @@
+"""Seeded synthetic inputs and weight quantizers (torch, CPU or GPU).
+
+Recipes: weights ~ N(0, 0.02) quantized with absmax scales (FP8: one f32 scale per 128x128 block,
+s = amax * (1/448); NVFP4: E4M3 scale per 16 k-elements = amax/6 relative to an f32 global scale),
+activations ~ N(0, 1) in BF16, router gate ~ N(0, 0.02) in BF16. The encoders are the reference's:
+E4M3 round-to-nearest-even saturating at 448 (src/fp8.rs:85-121), E2M1 with its tie thresholds
+(kernels/q38_contract.cuh:180-187), stored NVFP4 scale code never 0 (q38_contract.cuh:207-209).
+"""
+import torch
+
+E4M3_MAX = 448.0
+
+
+def generator(seed, device="cpu"):
+    g = torch.Generator(device=device)
+    g.manual_seed(int(seed))
+    return g
+
+
+def normal(shape, std, seed, device="cpu", dtype=torch.float32):
+    return (torch.randn(shape, generator=generator(seed, device), device=device, dtype=torch.float32) * std).to(dtype)
+
+
+def e4m3_encode(x):
+    """float32 tensor already clamped to [-448, 448] -> uint8 E4M3 codes (RNE)."""
+    return x.to(torch.float8_e4m3fn).view(torch.uint8)
+
+
+def e4m3_decode(codes):
+    return codes.view(torch.float8_e4m3fn).to(torch.float32)
+
+
+def quant_fp8_block(w, block=128):
+    """w [N,K] f32 -> (codes uint8 [N,K], scales f32 [ceil(N/b), ceil(K/b)])."""
+    n, k = w.shape
+    gn, gk = -(-n // block), -(-k // block)
+    pad = torch.zeros((gn * block, gk * block), dtype=torch.float32, device=w.device)
+    pad[:n, :k] = w
+    blocks = pad.view(gn, block, gk, block)
+    amax = blocks.abs().amax(dim=(1, 3))
+    scales = amax * torch.tensor(1.0 / 448.0, dtype=torch.float32, device=w.device)
+    div = scales.clamp_min(1e-12)[:, None, :, None]
+    q = (blocks / div).clamp(-E4M3_MAX, E4M3_MAX)
+    codes = e4m3_encode(q).view(gn * block, gk * block)[:n, :k].contiguous()
+    return codes, scales.contiguous()
+
+
+def e2m1_encode(x):
+    """float32 -> 4-bit E2M1 codes (uint8), thresholds with ties toward the even code."""
+    m = x.abs()
+    code = torch.full_like(m, 7, dtype=torch.uint8)
+    code = torch.where(m <= 5.0, torch.tensor(6, dtype=torch.uint8, device=x.device), code)
+    code = torch.where(m < 3.5, torch.tensor(5, dtype=torch.uint8, device=x.device), code)
+    code = torch.where(m <= 2.5, torch.tensor(4, dtype=torch.uint8, device=x.device), code)
+    code = torch.where(m < 1.75, torch.tensor(3, dtype=torch.uint8, device=x.device), code)
+    code = torch.where(m <= 1.25, torch.tensor(2, dtype=torch.uint8, device=x.device), code)
+    code = torch.where(m < 0.75, torch.tensor(1, dtype=torch.uint8, device=x.device), code)
+    code = torch.where(m <= 0.25, torch.tensor(0, dtype=torch.uint8, device=x.device), code)
+    sign = (torch.signbit(x).to(torch.uint8) << 3)
+    return code | sign
+
+
+def quant_nvfp4(w):
+    """w [N,K] f32 (K % 16 == 0) -> (codes uint8 [N,K/2], scales uint8 [N,K/16], global f32 python float)."""
+    n, k = w.shape
+    g = w.view(n, k // 16, 16)
+    s16 = g.abs().amax(dim=2) / 6.0
+    glob = s16.max() / 448.0
+    if not bool(glob > 0):
+        glob = torch.tensor(1.0, dtype=torch.float32, device=w.device)
+    sc = e4m3_encode((s16 / glob).clamp(max=E4M3_MAX))
+    sc = torch.where(sc == 0, torch.tensor(1, dtype=torch.uint8, device=w.device), sc)
+    s = e4m3_decode(sc) * glob
+    q = e2m1_encode(g / s[:, :, None]).view(n, k)
+    codes = (q[:, 0::2] | (q[:, 1::2] << 4)).contiguous()
+    return codes, sc.contiguous(), float(glob)
+
+
+def zipf_popularity(experts, s, seed):
+    """log-popularity offsets: popularity proportional to rank^-s under a seeded expert permutation."""
+    perm = torch.randperm(experts, generator=generator(seed))
+    rank = torch.empty(experts, dtype=torch.float32)
+    rank[perm] = torch.arange(1, experts + 1, dtype=torch.float32)
+    return (-s) * torch.log(rank)

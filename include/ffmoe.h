@@ -1,0 +1,248 @@
+/*
+ * libffmoe — MI355X (gfx950) kernels for the quantized MoE expert-FFN path of GreatV/flyingfish:
+ * router top-k, block-scaled FP8 E4M3 / NVFP4 expert SwiGLU FFN for decode, token-sorted grouped
+ * GEMM prefill, and the ordered weighted combine.
+ *
+ * Conventions (they restate the reference's operator contract,
+ * src/backend/cuda/contracts.rs:80-137 and the per-op validators cited below):
+ *   - every tensor argument is a raw DEVICE pointer to a dense row-major array; the caller owns
+ *     all of them, including scratch, `contributions` and `done`;
+ *   - base pointers of BF16/FP8/FP4 tensors are 16-byte aligned, f32/i32/u32 tensors 4-byte;
+ *   - BF16 values are passed as uint16 bit patterns (`void*` in the signatures);
+ *   - `stream` is a hipStream_t (NULL = the default stream); calls only enqueue work;
+ *   - return value: 0 = ok, > 0 = hipError_t of a failed runtime call, < 0 = contract violation
+ *     detected on the host before anything was launched (`ffmoe_last_error()` has the text);
+ *   - nothing here allocates device memory.
+ */
+#ifndef FFMOE_H
+#define FFMOE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FFMOE_VERSION 1
+
+/* contract-violation codes (negative) */
+#define FFMOE_ERR_NULL        (-1)  /* required pointer is NULL */
+#define FFMOE_ERR_ALIGN       (-2)  /* base pointer misaligned */
+#define FFMOE_ERR_SHAPE       (-3)  /* extent out of range or inconsistent */
+#define FFMOE_ERR_OVERLAP     (-4)  /* an output aliases an input, scratch or another output */
+#define FFMOE_ERR_UNSUPPORTED (-5)  /* format / mode combination not implemented */
+#define FFMOE_ERR_SCRATCH     (-6)  /* scratch arena too small */
+
+/* limits of the routing contract (kernels/moe_route.cu:23-30, :462-466) */
+#define FFMOE_MAX_EXPERTS 1024
+#define FFMOE_MAX_TOP_K   32
+
+/* expert weight formats (src/model_spec.rs ExpertFormat / LinearFormat) */
+#define FFMOE_FMT_FP8_BLOCK128 0  /* E4M3 codes [N,K] + f32 scales [ceil(N/128), ceil(K/128)] (src/fp8.rs:31-36) */
+#define FFMOE_FMT_NVFP4        1  /* E2M1 pairs [N,K/2] (low nibble = even k) + E4M3 scales [N,K/16] + f32 global */
+#define FFMOE_FMT_BF16         2  /* BF16 [N,K] */
+
+/* activation arithmetic of the FP8 linears */
+#define FFMOE_ACT_BF16         0  /* W8A16: w = bf16(e4m3(code) * scale), FP32 accumulate against BF16 activations
+                                     (src/fp8.rs:138-140, src/cpu/expert_ffn.rs:592-679) */
+#define FFMOE_ACT_FP8_BLOCK128 1  /* W8A8: activations quantized per 128 to E4M3 with an f32 scale, per-128 dot then
+                                     one scale product (kernels/fp8_linear.cu:12-48, kernels/q38_contract.cuh:239-279) */
+
+/* SwiGLU rounding (src/model_spec.rs:61-69; src/cpu/expert_ffn.rs:58-100) */
+#define FFMOE_SWIGLU_TWICE          0  /* a = bf16(bf16(silu(g)) * u) */
+#define FFMOE_SWIGLU_ONCE           1  /* a = bf16(silu(g) * u) */
+#define FFMOE_SWIGLU_CLAMPED_TWICE  2  /* g = min(g,L), u = clamp(u,+-L), then TWICE */
+#define FFMOE_SWIGLU_CLAMPED_ONCE   3
+
+/* routed-weight boundary (src/model_spec.rs:70-75) */
+#define FFMOE_WEIGHT_AFTER_DOWN_BF16          0  /* c = bf16(bf16(d) * w) */
+#define FFMOE_WEIGHT_BEFORE_CONTRIBUTION_BF16 1  /* c = bf16(d * w) */
+
+/* router score */
+#define FFMOE_SCORE_SOFTMAX      0
+#define FFMOE_SCORE_SIGMOID      1
+#define FFMOE_NOAUX_SIGMOID      0  /* score_mode of the noaux kernels (kernels/moe_route.cu:329-336) */
+#define FFMOE_NOAUX_SQRTSOFTPLUS 1
+
+/* combine variants (kernels/moe_combine.cu) */
+#define FFMOE_COMBINE_GATED      0  /* moe_combine         :71-93   */
+#define FFMOE_COMBINE_UNGATED    1  /* moe_combine_ungated :95-116  */
+#define FFMOE_COMBINE_BF16       2  /* moe_combine_bf16    :592-613 */
+#define FFMOE_COMBINE_ACCUM_FP32 3  /* moe_combine_accum, fp32_accum = 1 :541-591 */
+#define FFMOE_COMBINE_ACCUM_BF16 4  /* moe_combine_accum, fp32_accum = 0 */
+#define FFMOE_COMBINE_ROUTED     5  /* moe_combine_routed  :176-196 */
+
+const char* ffmoe_last_error(void);
+int ffmoe_version(void);
+
+/* ------------------------------------------------------------------------------------------------
+ * Router. Replaces RouteOps (src/backend/cuda/moe/route.rs:450-499, :505-562, :721-769, :808-905)
+ * and the kernels of kernels/moe_route.cu.
+ */
+
+/* logits[r,e] = bf16(ascending FP32 fma chain over x[r,:] * router[e,:]).
+ * Replaces moe_route_logits_bf16 (kernels/moe_route.cu:408-457). hidden % 8 == 0. */
+int ffmoe_route_logits_bf16(const void* x, const void* router, void* logits,
+                            int rows, int experts, int hidden, void* stream);
+
+/* FP32 logits (replaces RouteOps::logits_f32, route.rs:505-562, a BLAS GEMM of undefined order).
+ * Order used here: 64 lanes, lane L chains fma over the 8-element vectors L, L+64, ... in ascending
+ * order, lane partials summed by a shuffle-down tree 32,16,8,4,2,1. hidden % 8 == 0. */
+int ffmoe_route_logits_f32(const void* x, const void* router, float* logits,
+                           int rows, int experts, int hidden, void* stream);
+
+/* Softmax or sigmoid top-k over BF16 logits; ids [rows,top_k] i32, weights [rows,top_k] BF16.
+ * Replaces moe_route_topk / moe_route_topk_sigmoid (kernels/moe_route.cu:459-491).
+ * 1 <= top_k <= 32, top_k < experts <= 1024. */
+int ffmoe_route_topk(const void* logits, int* ids, void* weights,
+                     int rows, int experts, int top_k, int score, void* stream);
+
+/* noaux_tc selection over FP32 logits: select on score+bias, weight = score/(sum+1e-20)*routed_scaling.
+ * Replaces moe_route_topk_noaux(_f32) (kernels/moe_route.cu:579-628; route.rs:721-769).
+ * bias may be NULL; bias_row_stride is `experts` for a [rows,experts] bias or 0 to broadcast one [experts] row.
+ * weights_f32 != 0 stores f32 weights, else BF16. n_group > 1 adds a group filter that the reference does not
+ * have (group score = sum of the two largest score+bias in the group; keep topk_group groups; ties to the
+ * lower group id); n_group == 1 is the reference kernel. experts % n_group == 0. */
+int ffmoe_route_topk_noaux(const float* logits, const float* bias, int bias_row_stride,
+                           int* ids, void* weights, int weights_f32,
+                           int rows, int experts, int top_k, int score_mode, float routed_scaling,
+                           int n_group, int topk_group, void* stream);
+
+/* Fused decode route: BF16 logits (stored) then softmax/sigmoid top-k.
+ * Replaces RouteOps::route / moe_route_decode_bf16 (route.rs:450-499; kernels/moe_route.cu:496-568). */
+int ffmoe_route_decode(const void* x, const void* router, void* logits, int* ids, void* weights,
+                       int rows, int experts, int hidden, int top_k, int score, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * Expert tables. All experts stay resident in HBM. A slot is six device addresses per expert, as
+ * NativeMoe's `slots[E,6]` (kernels/moe_ffn.cu:869-885; src/backend/cuda/moe/decode.rs:683-698):
+ *   {gate codes, gate scales, up codes, up scales, down codes, down scales}
+ * gate/up are [inter, hidden], down is [hidden, inter]. For FFMOE_FMT_BF16 the scale entries are ignored.
+ * For NVFP4 `global_scales` holds weight_scale_2 of gate, up, down per expert.
+ */
+typedef struct ffmoe_expert_table {
+  int format;                 /* FFMOE_FMT_* */
+  int experts, hidden, inter;
+  const uint64_t* slots;      /* device [experts, 6] */
+  const uint32_t* valid;      /* device [experts], 0 = not resident; NULL = all valid */
+  const float* global_scales; /* device [experts, 3] (NVFP4) or NULL */
+} ffmoe_expert_table;
+
+/* One always-on shared expert (MoeDecode::shared_gate/up/down, decode.rs:26-44). Addresses by value. */
+typedef struct ffmoe_shared_expert {
+  int format;                 /* FFMOE_FMT_* */
+  int inter;
+  uint64_t slot[6];           /* device addresses, same order as a table slot */
+  float global_scales[3];     /* NVFP4 only */
+} ffmoe_shared_expert;
+
+/* ------------------------------------------------------------------------------------------------
+ * Decode contribution: for every active (row, choice) the expert SwiGLU FFN output times the routing
+ * weight, plus the shared expert per row. Replaces DecodeOps::contribute(_routed,_shared,_w8a16)
+ * (src/backend/cuda/moe/decode.rs:421-589) and NativeMoe's dispatch (decode.rs:1187-1262), i.e. kernels
+ * moe_ffn_gate_up/_down(+_w8a16) and moe_ffn_dispatch_e4m3_f32_128 + moe_ffn_weight_f32 (kernels/moe_ffn.cu).
+ * Unlike the reference (rows <= 8/16) any row count is accepted; rows routed to the same expert share one
+ * pass over that expert's weights.
+ */
+typedef struct ffmoe_decode {
+  int rows, top_k;
+  int act_mode;        /* FFMOE_ACT_* (FP8 formats) */
+  int swiglu;          /* FFMOE_SWIGLU_* */
+  float swiglu_limit;  /* clamped modes: finite, > 0 */
+  int routed_weight;   /* FFMOE_WEIGHT_* */
+  int weights_f32;     /* routing weights are f32 (else BF16) */
+  const void* x;       /* [rows, hidden] BF16 */
+  const int* ids;      /* [rows, top_k] */
+  const uint32_t* active; /* [rows, top_k] or NULL = all active */
+  const void* weights; /* [rows, top_k] BF16 or f32 */
+  void* contributions; /* [rows, top_k, hidden] BF16 */
+  void* shared_out;    /* [rows, hidden] BF16 (NULL when there is no shared expert) */
+  uint32_t* done;      /* [rows, top_k]; set to 1 for every contributed slot (NULL = not tracked) */
+  void* scratch;       /* ffmoe_decode_scratch_bytes() bytes, 256-byte aligned */
+  uint64_t scratch_bytes;
+} ffmoe_decode;
+
+/* Scratch needed by ffmoe_decode_contribute (mirrors decode_scratch_bytes_mixed, decode.rs:52-59,
+ * plus the assignment-grouping tables and the quantized activations of FFMOE_ACT_FP8_BLOCK128). */
+uint64_t ffmoe_decode_scratch_bytes(int rows, int top_k, int experts, int hidden, int inter, int shared_inter);
+
+int ffmoe_decode_contribute(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared,
+                            const ffmoe_decode* args, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * Standalone linears, M <= 16 "skinny" and beyond. y[M,N] = x[M,K] * W[N,K]^T, BF16 in / BF16 out.
+ */
+
+/* Replaces fp8_quant_f32_128 (kernels/fp8_linear.cu:12-48): per (row, 128-group) scale = amax*(1/448),
+ * codes = e4m3_rne(clamp(x / max(scale,1e-12), +-448)). scales [m, ceil(k/128)] f32. */
+int ffmoe_quant_fp8_f32_128(const void* x, void* codes, float* scales, int m, int k, void* stream);
+
+/* Replaces Fp8Ops::bind_block + Fp8BlockPlan::run (src/backend/cuda/linear.rs:571-660) on pre-quantized
+ * activations: kernels fp8_block_f32_128_decode/_mma (kernels/fp8_linear.cu:194-206). */
+int ffmoe_linear_fp8_block_w8a8(const void* w_codes, const float* w_scales, const void* x_codes,
+                                const float* x_scales, void* y, int m, int n, int k, void* stream);
+
+/* BF16 activations against a 128x128-f32 block-scaled FP8 weight.
+ * act_mode FFMOE_ACT_BF16: w = bf16(e4m3*scale) in registers (the W8A16 contract of fp8_gemv_bf16 /
+ * fp8_skinny_bf16_mM, kernels/fp8_linear.cu:353-511, with f32 instead of BF16 scales).
+ * act_mode FFMOE_ACT_FP8_BLOCK128: NativeProjection::run (linear.rs:1352-1405): quantize then W8A8;
+ * needs scratch of m*k + 4*m*ceil(k/128) bytes (256-byte aligned), otherwise scratch may be NULL. */
+int ffmoe_linear_fp8_block(const void* w_codes, const float* w_scales, const void* x, void* y,
+                           int m, int n, int k, int act_mode, void* scratch, uint64_t scratch_bytes, void* stream);
+
+/* Replaces NvFp4Ops::gemm (linear.rs:488-551; kernels/nvfp4_linear.cu:50-252): W4A16,
+ * w = bf16(e2m1 * (e4m3(scale) * global)). global_scale is a device pointer to one f32. k % 16 == 0. */
+int ffmoe_linear_nvfp4(const void* w_codes, const void* w_scales, const float* global_scale,
+                       const void* x, void* y, int m, int n, int k, void* stream);
+
+/* Replaces gemm_skinny_bf16 (kernels/gemm_skinny.cu:509-675): BF16 weights [n,k]. */
+int ffmoe_gemm_skinny_bf16(const void* w, const void* x, void* y, int m, int n, int k, void* stream);
+
+/* Replaces silu_mul_split / silu_mul_split_clamped (kernels/act.cu:65-99, :125-159):
+ * y = swiglu(gate, up) over dense [rows, width] BF16 regions, width % 8 == 0. */
+int ffmoe_swiglu(const void* gate, const void* up, void* y, int rows, int width, int mode, float limit, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * Combine. Replaces CombineOps (src/backend/cuda/moe/combine.rs:440-760; kernels/moe_combine.cu).
+ */
+
+/* scale[r] = bf16(sigmoid(bf16(x[r,:] . seg))). Replaces moe_shared_scale (kernels/moe_combine.cu:21-49). */
+int ffmoe_shared_scale(const void* x, const void* seg, void* scale, int rows, int hidden, void* stream);
+
+/* y[r,:] from contributions [rows,top_k,hidden] and shared_out [rows,hidden] in the order of `mode`.
+ * ids/done/final_active are [rows,top_k]; a slot with done != final_active is a protocol violation: the
+ * reference traps (kernels/moe_combine.cu:56-58); here the row is still combined over final_active and bit 0
+ * of *status (device u32, may be NULL) is set. final_active NULL = all active; done NULL = not checked.
+ * ACCUM modes ignore ids/done/final_active. */
+int ffmoe_combine(const void* contributions, const void* shared_out, const void* scale, const int* ids,
+                  const uint32_t* done, const uint32_t* final_active, void* y, uint32_t* status,
+                  int rows, int top_k, int hidden, int mode, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * Prefill: many tokens, grouped by expert on the device (no host synchronisation), grouped FP8 GEMMs on
+ * MFMA in FFMOE_ACT_FP8_BLOCK128 arithmetic. Replaces PrefillOps::prefill_contribute
+ * (src/backend/cuda/moe/prefill.rs:1033-1408) and kernels moe_count_scan / moe_permute / moe_gemm_w8a16 /
+ * silu_mul / moe_scatter (kernels/moe_prefill.cu). Only FFMOE_FMT_FP8_BLOCK128 tables.
+ */
+typedef struct ffmoe_prefill {
+  int rows, top_k;
+  int swiglu; float swiglu_limit;
+  int routed_weight;
+  int weights_f32;
+  const void* x;           /* [rows, hidden] BF16 */
+  const int* ids;          /* [rows, top_k] */
+  const uint32_t* active;  /* [rows, top_k] or NULL */
+  const void* weights;     /* [rows, top_k] */
+  void* contributions;     /* [rows, top_k, hidden] BF16 */
+  uint32_t* done;          /* [rows, top_k] or NULL */
+  void* scratch; uint64_t scratch_bytes;
+} ffmoe_prefill;
+
+uint64_t ffmoe_prefill_scratch_bytes(int rows, int top_k, int experts, int hidden, int inter);
+int ffmoe_prefill_contribute(const ffmoe_expert_table* table, const ffmoe_prefill* args, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FFMOE_H */

@@ -1,0 +1,344 @@
+"""GPU parity: the HIP path (through the C ABI) against the CPU oracle on the same seeded inputs."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle as orc
+from flyingfish_amd import capi, synth
+from flyingfish_amd.ops import CombineOps, DecodeOps, ExpertTable, Fp8Ops, NativeMoe, NvFp4Ops, RouteOps, gemm_skinny_bf16, swiglu
+from helpers import assert_close_bf16, bf16_tensor, bits, make_table, oracle_contributions, oracle_shared
+
+pytestmark = pytest.mark.gpu
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden", "shared-ops.json")
+DEV = "cuda"
+
+
+def rand_bf16(shape, std, seed):
+    return synth.normal(shape, std, seed).to(torch.bfloat16)
+
+
+# ------------------------------------------------------------------------------------------------
+# codecs through the product path
+def test_device_e4m3_decode_all_codes():
+    # W[n, 0] = code n with unit scale, x = e_0  =>  y[n] = bf16(decode(n)); E4M3 values are exact in BF16
+    n, k = 256, 128
+    codes = torch.zeros((n, k), dtype=torch.uint8)
+    codes[:, 0] = torch.arange(256, dtype=torch.int32).to(torch.uint8)
+    codes[0x7F, 0] = 0
+    codes[0xFF, 0] = 0
+    scales = torch.ones((2, 1), dtype=torch.float32)
+    x = torch.zeros((1, k), dtype=torch.bfloat16)
+    x[0, 0] = 1.0
+    y = Fp8Ops.linear(codes.to(DEV), scales.to(DEV), x.to(DEV))
+    L = orc.lib()
+    want = np.array([0.0 if c in (0x7F, 0xFF) else L.orc_decode_e4m3(c) for c in range(256)], dtype=np.float32)
+    assert np.array_equal(y.float().cpu().numpy()[0], want)
+
+
+def test_device_effective_weight_rounding_matches_oracle():
+    # every code against awkward f32 scales: y[n] = bf16(decode(code) * scale) must equal the oracle bit for bit
+    n, k = 256, 128
+    codes = torch.zeros((n, k), dtype=torch.uint8)
+    col = torch.arange(256, dtype=torch.int32).to(torch.uint8)
+    col[0x7F] = 0
+    col[0xFF] = 0
+    codes[:, 0] = col
+    x = torch.zeros((1, k), dtype=torch.bfloat16)
+    x[0, 0] = 1.0
+    L = orc.lib()
+    for s0, s1 in [(1.0078125, 0.0123456), (3.3e-5, 7.77e-3), (1.9999999, 0.33333334)]:
+        scales = torch.tensor([[s0], [s1]], dtype=torch.float32)
+        y = bits(Fp8Ops.linear(codes.to(DEV), scales.to(DEV), x.to(DEV)))[0]
+        want = np.array([L.orc_effective_weight(int(col[c]), float(np.float32(s0 if c < 128 else s1))) for c in range(256)], dtype=np.uint16)
+        assert np.array_equal(y & 0x7FFF, want & 0x7FFF) and np.array_equal(y[want & 0x7FFF != 0], want[want & 0x7FFF != 0])
+
+
+def test_device_activation_quantizer_bits():
+    m, k = 7, 7168
+    x = rand_bf16((m, k), 1.0, 101)
+    x[3] = 0
+    x[4, :128] *= 1e-20
+    codes, scales = Fp8Ops.quantize(x.to(DEV))
+    wc, ws = orc.quant_act_fp8_128(bits(x))
+    assert np.array_equal(scales.cpu().numpy().view(np.uint32), ws.view(np.uint32))
+    assert np.array_equal(codes.cpu().numpy(), wc)
+    # reference fixture (src/backend/cuda/linear.rs:2320-2338), k with a ragged last group
+    m, k = 5, 264
+    i = np.arange(m * k, dtype=np.int64)
+    vals = orc.f32_to_bf16((((i * 19 + 3) % 251).astype(np.float32) / np.float32(32) - np.float32(4))).reshape(m, k)
+    codes, scales = Fp8Ops.quantize(bf16_tensor(vals))
+    wc, ws = orc.quant_act_fp8_128(vals)
+    assert np.array_equal(codes.cpu().numpy(), wc) and np.array_equal(scales.cpu().numpy().view(np.uint32), ws.view(np.uint32))
+
+
+def test_device_swiglu_golden_bits():
+    with open(GOLDEN) as f:
+        fx = json.load(f)["swiglu"]
+    n = len(fx["gate"])
+    g = np.zeros(16, np.float32); g[:n] = fx["gate"]
+    u = np.zeros(16, np.float32); u[:n] = fx["up"]
+    gt, ut = torch.from_numpy(g).to(torch.bfloat16).view(1, 16).to(DEV), torch.from_numpy(u).to(torch.bfloat16).view(1, 16).to(DEV)
+    assert bits(swiglu(gt, ut, capi.SWIGLU_CLAMPED_TWICE, fx["limit"]))[0, :n].tolist() == fx["twice"]
+    assert bits(swiglu(gt, ut, capi.SWIGLU_CLAMPED_ONCE, fx["limit"]))[0, :n].tolist() == fx["once"]
+    # dense random sweep against the oracle for all four modes
+    gg, uu = rand_bf16((8, 4096), 3.0, 5), rand_bf16((8, 4096), 3.0, 6)
+    for mode in range(4):
+        got = bits(swiglu(gg.to(DEV), uu.to(DEV), mode, 2.5))
+        want = orc.silu_mul(bits(gg), bits(uu), mode, 2.5, orc.SILU_DIV)
+        assert np.array_equal(got, want), mode
+
+
+# ------------------------------------------------------------------------------------------------
+# router
+@pytest.mark.parametrize("rows,experts,hidden", [(1, 64, 2048), (3, 256, 512), (2, 100, 264)])
+def test_route_logits_bf16_bit_exact(rows, experts, hidden):
+    x, w = rand_bf16((rows, hidden), 1.0, 11), rand_bf16((experts, hidden), 0.02, 12)
+    got = bits(RouteOps.logits_bf16(x.to(DEV), w.to(DEV)))
+    assert np.array_equal(got, orc.route_logits_bf16(bits(x), bits(w)))
+
+
+@pytest.mark.parametrize("rows,experts,hidden", [(1, 256, 7168), (9, 64, 2048), (5, 33, 520)])
+def test_route_logits_f32_bit_exact_and_close_to_f64(rows, experts, hidden):
+    x, w = rand_bf16((rows, hidden), 1.0, 13), rand_bf16((experts, hidden), 0.02, 14)
+    got = RouteOps.logits_f32(x.to(DEV), w.to(DEV)).cpu().numpy()
+    want = orc.route_logits_f32(bits(x), bits(w))
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    f64 = x.double().numpy() @ w.double().numpy().T
+    assert np.max(np.abs(got - f64)) <= 16 * 2.0 ** -24 * np.max(np.abs(x.double().numpy()) @ np.abs(w.double().numpy()).T)
+
+
+@pytest.mark.parametrize("score", [capi.SCORE_SOFTMAX, capi.SCORE_SIGMOID])
+@pytest.mark.parametrize("rows,experts,top_k", [(4, 64, 4), (3, 256, 8), (2, 1000, 32), (5, 48, 6)])
+def test_route_topk_bit_exact(score, rows, experts, top_k):
+    lg = rand_bf16((rows, experts), 1.5, 15 + experts)
+    lg[0, 1] = lg[0, experts - 1] = 6.0          # planted exact tie inside the top-k
+    lg[1, 7] = lg[1, 3]                           # planted tie somewhere
+    ids, w = RouteOps.topk(lg.to(DEV), top_k, score)
+    fn = orc.route_topk_softmax if score == capi.SCORE_SOFTMAX else orc.route_topk_sigmoid
+    wi, ww = fn(bits(lg), top_k)
+    assert np.array_equal(ids.cpu().numpy(), wi)
+    assert np.array_equal(bits(w), ww)
+    assert ids[0, 0] == 1 and ids[0, 1] == experts - 1
+
+
+def test_route_noaux_golden_and_random():
+    with open(GOLDEN) as f:
+        routers = json.load(f)["routers"]
+    for fx in routers:
+        mode = {"sigmoid": 0, "sqrtsoftplus": 1}[fx["mode"]]
+        lg = torch.tensor([fx["logits"]], dtype=torch.float32, device=DEV)
+        b = torch.tensor([fx["bias"]], dtype=torch.float32, device=DEV)
+        ids, w = RouteOps.topk_noaux(lg, b, fx["top_k"], mode, fx["scale"])
+        assert ids[0].tolist() == fx["ids"]
+        want = np.array(fx["weights"], dtype=np.float32)
+        assert np.all(np.abs(w[0].cpu().numpy() - want) <= 2e-6 * np.maximum(1, np.abs(want)))
+        oi, ow = orc.route_topk_noaux(lg.cpu().numpy(), b.cpu().numpy(), fx["top_k"], mode, fx["scale"])
+        assert np.array_equal(w.cpu().numpy().view(np.uint32), ow.view(np.uint32))
+    rng = np.random.default_rng(3)
+    for rows, experts, top_k, ng, kg in [(16, 256, 8, 1, 1), (16, 256, 8, 8, 4), (7, 64, 6, 4, 2), (3, 384, 6, 1, 1)]:
+        lg = rng.normal(size=(rows, experts)).astype(np.float32)
+        b = rng.normal(scale=0.2, size=(experts,)).astype(np.float32)
+        lg[0, 5] = lg[0, 9]
+        for mode in (0, 1):
+            for wf32 in (True, False):
+                ids, w = RouteOps.topk_noaux(torch.from_numpy(lg).to(DEV), torch.from_numpy(b).to(DEV), top_k, mode, 2.5, ng, kg, wf32)
+                oi, ow = orc.route_topk_noaux(lg, b[None, :], top_k, mode, 2.5, ng, kg)
+                assert np.array_equal(ids.cpu().numpy(), oi), (rows, experts, mode)
+                if wf32:
+                    assert np.array_equal(w.cpu().numpy().view(np.uint32), ow.view(np.uint32))
+                else:
+                    assert np.array_equal(bits(w), orc.f32_to_bf16(ow))
+
+
+def test_route_decode_fused_c1_shape():
+    x, w = rand_bf16((1, 2048), 1.0, 21), rand_bf16((64, 2048), 0.02, 22)
+    ids, wt, logits = RouteOps.route(x.to(DEV), w.to(DEV), 4, capi.SCORE_SOFTMAX)
+    ol = orc.route_logits_bf16(bits(x), bits(w))
+    oi, ow = orc.route_topk_softmax(ol, 4)
+    assert np.array_equal(bits(logits), ol) and np.array_equal(ids.cpu().numpy(), oi) and np.array_equal(bits(wt), ow)
+
+
+# ------------------------------------------------------------------------------------------------
+# decode contributions
+def _run_decode(fmt, experts, hidden, inter, rows, top_k, seed, shared, swiglu_mode=capi.SWIGLU_TWICE, limit=0.0,
+                boundary=capi.WEIGHT_AFTER_DOWN_BF16, weights_f32=False, with_active=False):
+    table, ref = make_table(fmt, experts + (1 if shared else 0), hidden, inter, seed)
+    sh = table.shared_struct(experts) if shared else None
+    table.experts = experts
+    x = rand_bf16((rows, hidden), 1.0, seed + 7)
+    g = synth.generator(seed + 8)
+    ids = torch.stack([torch.randperm(experts, generator=g)[:top_k] for _ in range(rows)]).to(torch.int32)
+    wt = torch.rand((rows, top_k), generator=g) * 0.5 + 0.05
+    wdev = wt.to(DEV) if weights_f32 else wt.to(torch.bfloat16).to(DEV)
+    wref = wt.numpy() if weights_f32 else wt.to(torch.bfloat16).float().numpy()
+    active = None
+    if with_active:
+        active = (torch.rand((rows, top_k), generator=g) > 0.3).to(torch.int32)
+    op = DecodeOps(table, sh, rows, top_k, capi.ACT_BF16, swiglu_mode, limit, boundary, weights_f32)
+    op.contributions.zero_()
+    contrib, shared_out = op.contribute(x.to(DEV), ids.to(DEV), wdev, active.to(DEV) if active is not None else None)
+    torch.cuda.synchronize()
+    want = oracle_contributions(ref, bits(x), ids.numpy(), wref, swiglu_mode, limit, boundary, active.numpy() if active is not None else None)
+    got = bits(contrib)
+    stats = assert_close_bf16(got, want, "contributions")
+    done = op.done.cpu().numpy()
+    assert np.array_equal(done != 0, np.ones_like(done, bool) if active is None else active.numpy() != 0)
+    if shared:
+        assert_close_bf16(bits(shared_out), oracle_shared(ref[experts], bits(x), swiglu_mode, limit), "shared_out")
+    return stats
+
+
+def test_decode_fp8_c1_shape_single_token():
+    # BASELINE config 1: hidden 2048, 64 experts, top-4, inter 1408, FP8 128x128 (weights for 8 experts are enough
+    # for one token; ids are drawn from them)
+    r, worst = _run_decode(capi.FMT_FP8_BLOCK128, 8, 2048, 1408, 1, 4, 31, shared=False)
+    print("C1 rel_l2=%.2e worst_ulp=%.2f" % (r, worst))
+
+
+@pytest.mark.parametrize("rows,top_k,shared", [(1, 8, True), (2, 4, True), (5, 3, False), (8, 4, True), (19, 2, True)])
+def test_decode_fp8_batched_rows_group_by_expert(rows, top_k, shared):
+    _run_decode(capi.FMT_FP8_BLOCK128, 8, 1024, 512, rows, top_k, 40 + rows, shared)
+
+
+def test_decode_fp8_modes_and_active_mask():
+    _run_decode(capi.FMT_FP8_BLOCK128, 6, 512, 384, 4, 3, 51, True, capi.SWIGLU_CLAMPED_TWICE, 0.05, capi.WEIGHT_BEFORE_CONTRIBUTION_BF16, True, True)
+    _run_decode(capi.FMT_FP8_BLOCK128, 6, 512, 384, 1, 3, 52, False, capi.SWIGLU_ONCE, 0.0, capi.WEIGHT_AFTER_DOWN_BF16, False, True)
+    _run_decode(capi.FMT_FP8_BLOCK128, 6, 512, 384, 3, 2, 53, True, capi.SWIGLU_CLAMPED_ONCE, 0.1, capi.WEIGHT_AFTER_DOWN_BF16, True, False)
+
+
+@pytest.mark.parametrize("rows", [1, 6])
+def test_decode_nvfp4(rows):
+    _run_decode(capi.FMT_NVFP4, 6, 1024, 512, rows, 3, 61, True)
+
+
+@pytest.mark.parametrize("rows", [1, 6])
+def test_decode_bf16_experts(rows):
+    _run_decode(capi.FMT_BF16, 5, 1024, 256, rows, 2, 71, True)
+
+
+def test_decode_dsv3_width_single_token():
+    # hidden 7168 / inter 2048 at DeepSeek-V3 width, 3 routed experts + shared, one token
+    _run_decode(capi.FMT_FP8_BLOCK128, 3, 7168, 2048, 1, 3, 81, True)
+
+
+def test_decode_row_count_invariance_bitwise():
+    # rows batched == each row run alone, bit for bit (src/backend/cuda/moe/decode_tests.rs:347-399)
+    experts, hidden, inter, rows, top_k = 8, 1024, 512, 6, 4
+    table, _ = make_table(capi.FMT_FP8_BLOCK128, experts, hidden, inter, 91)
+    x = rand_bf16((rows, hidden), 1.0, 92).to(DEV)
+    g = synth.generator(93)
+    ids = torch.stack([torch.randperm(experts, generator=g)[:top_k] for _ in range(rows)]).to(torch.int32).to(DEV)
+    wt = (torch.rand((rows, top_k), generator=g) + 0.1).to(torch.bfloat16).to(DEV)
+    batched = DecodeOps(table, None, rows, top_k)
+    full = batched.contribute(x, ids, wt)[0].clone()
+    single = DecodeOps(table, None, 1, top_k)
+    for r in range(rows):
+        one = single.contribute(x[r:r + 1].contiguous(), ids[r:r + 1].contiguous(), wt[r:r + 1].contiguous())[0]
+        assert torch.equal(one[0].view(torch.int16), full[r].view(torch.int16)), r
+
+
+def test_decode_mutation_controls():
+    # swapping two experts' codes or changing one scale must change the output (prefill_tests.rs:485-535)
+    experts, hidden, inter = 4, 512, 256
+    table, _ = make_table(capi.FMT_FP8_BLOCK128, experts, hidden, inter, 95)
+    x = rand_bf16((1, hidden), 1.0, 96).to(DEV)
+    ids = torch.tensor([[0, 1]], dtype=torch.int32, device=DEV)
+    wt = torch.tensor([[0.5, 0.25]], dtype=torch.bfloat16, device=DEV)
+    op = DecodeOps(table, None, 1, 2)
+    base = op.contribute(x, ids, wt)[0].clone()
+    v0, v1 = table.expert_views(0), table.expert_views(1)
+    tmp = v0[0].clone(); v0[0].copy_(v1[0]); v1[0].copy_(tmp)
+    swapped = op.contribute(x, ids, wt)[0].clone()
+    assert not torch.equal(base.view(torch.int16), swapped.view(torch.int16))
+    v1[0].copy_(v0[0]); v0[0].copy_(tmp)
+    assert torch.equal(op.contribute(x, ids, wt)[0].view(torch.int16), base.view(torch.int16))
+    v0[5][0, 0] *= 1.5
+    assert not torch.equal(op.contribute(x, ids, wt)[0].view(torch.int16), base.view(torch.int16))
+
+
+# ------------------------------------------------------------------------------------------------
+# standalone linears (BASELINE config 2 at reduced N so the oracle stays fast)
+@pytest.mark.parametrize("m", [1, 4, 16])
+@pytest.mark.parametrize("k,n", [(7168, 256), (2048, 384)])
+def test_linear_fp8_block_w8a16(m, k, n):
+    w = synth.normal((n, k), 0.02, 200 + m)
+    codes, scales = synth.quant_fp8_block(w)
+    x = rand_bf16((m, k), 1.0, 300 + m)
+    y = bits(Fp8Ops.linear(codes.to(DEV), scales.to(DEV), x.to(DEV)))
+    eff = orc.dequant_fp8_block(codes.numpy(), scales.numpy())
+    want = np.stack([[orc.f32_to_bf16(np.float32(orc.dot(orc.bf16_to_f32(bits(x)[r]), eff[c], orc.LANE8))) for c in range(n)] for r in range(m)]).astype(np.uint16).reshape(m, n)
+    assert_close_bf16(y, want, "fp8 linear")
+    f64 = orc.linear_skinny(eff, bits(x), 2)
+    assert_close_bf16(y, f64, "fp8 linear vs f64")
+
+
+@pytest.mark.parametrize("m", [1, 3, 16])
+def test_linear_nvfp4_and_bf16(m):
+    n, k = 192, 2048
+    w = synth.normal((n, k), 0.02, 400)
+    codes, scales, g = synth.quant_nvfp4(w)
+    x = rand_bf16((m, k), 1.0, 401 + m)
+    gs = torch.tensor([g], dtype=torch.float32, device=DEV)
+    y = bits(NvFp4Ops.gemm(codes.to(DEV), scales.to(DEV), gs, x.to(DEV)))
+    eff = orc.dequant_nvfp4(codes.numpy(), scales.numpy(), g)
+    assert_close_bf16(y, orc.linear_skinny(eff, bits(x), 1), "nvfp4 linear (reference skinny order)")
+    wb = w.to(torch.bfloat16)
+    yb = bits(gemm_skinny_bf16(wb.to(DEV), x.to(DEV)))
+    assert_close_bf16(yb, orc.linear_skinny(bits(wb), bits(x), 2), "bf16 skinny")
+    # nibble-swap control (src/backend/cuda/linear.rs:4737)
+    sw = ((codes << 4) | (codes >> 4)).to(torch.uint8)
+    y2 = bits(NvFp4Ops.gemm(sw.to(DEV), scales.to(DEV), gs, x.to(DEV)))
+    assert not np.array_equal(y, y2)
+
+
+# ------------------------------------------------------------------------------------------------
+# combine
+def test_combine_modes_bit_exact():
+    rows, top_k, hidden = 5, 8, 1024
+    c = rand_bf16((rows, top_k, hidden), 1.0, 500)
+    sh = rand_bf16((rows, hidden), 1.0, 501)
+    g = synth.generator(502)
+    ids = torch.stack([torch.randperm(64, generator=g)[:top_k] for _ in range(rows)]).to(torch.int32)
+    act = (torch.rand((rows, top_k), generator=g) > 0.25).to(torch.int32)
+    x = rand_bf16((rows, hidden), 1.0, 503)
+    seg = rand_bf16((hidden,), 0.05, 504)
+    scale = CombineOps.shared_scale(x.to(DEV), seg.to(DEV))
+    assert np.array_equal(bits(scale), orc.shared_scale(bits(x), bits(seg)))
+    status = torch.zeros(1, dtype=torch.int32, device=DEV)
+    for mode in range(6):
+        y = CombineOps.combine(c.to(DEV), sh.to(DEV), ids.to(DEV), mode, scale=scale, done=act.to(DEV), final_active=act.to(DEV), status=status)
+        want = orc.combine(bits(c), bits(sh), bits(scale), ids.numpy(), act.numpy().astype(np.uint32), mode)
+        assert np.array_equal(bits(y), want), mode
+    assert int(status.item()) == 0
+    # a slot whose done flag disagrees with final_active raises the status bit (the reference traps here)
+    bad = act.clone(); bad[2, 1] ^= 1
+    CombineOps.combine(c.to(DEV), sh.to(DEV), ids.to(DEV), capi.COMBINE_BF16, done=bad.to(DEV), final_active=act.to(DEV), status=status)
+    assert int(status.item()) == 1
+
+
+# ------------------------------------------------------------------------------------------------
+# whole layer
+def test_native_moe_layer_matches_oracle_pipeline():
+    experts, hidden, inter, rows, top_k = 16, 1024, 512, 4, 4
+    table, ref = make_table(capi.FMT_FP8_BLOCK128, experts + 1, hidden, inter, 600)
+    shared = table.shared_struct(experts)
+    table.experts = experts
+    router = rand_bf16((experts, hidden), 0.02, 601)
+    bias = synth.normal((experts,), 0.01, 602)
+    x = rand_bf16((rows, hidden), 1.0, 603)
+    layer = NativeMoe(table, shared, router.to(DEV), bias.to(DEV), rows, top_k, 2.5, 4, 2)
+    y = layer.run(x.to(DEV))
+    torch.cuda.synchronize()
+    assert int(layer.status.item()) == 0
+    lg = orc.route_logits_f32(bits(x), bits(router))
+    oi, ow = orc.route_topk_noaux(lg, bias.numpy()[None, :], top_k, 0, 2.5, 4, 2)
+    assert np.array_equal(layer.ids.cpu().numpy(), oi)
+    assert np.array_equal(layer.weights.cpu().numpy().view(np.uint32), ow.view(np.uint32))
+    contrib = oracle_contributions(ref, bits(x), oi, ow, orc.TWICE, 0.0, orc.BEFORE_CONTRIBUTION_BF16)
+    sh = oracle_shared(ref[experts], bits(x), orc.TWICE, 0.0)
+    want = orc.combine(contrib, sh, None, oi, None, orc.COMBINE_BF16)
+    # the BF16 running sum compounds one rounding per choice: allow top_k + 1 steps at the row scale
+    assert_close_bf16(bits(y), want, "layer output", max_ulp=top_k + 1, rel=4e-3)
