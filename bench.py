@@ -1,0 +1,219 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized MoE expert-FFN hot path on one MI355X.
+
+Workload (BASELINE config 3, the one the metric is quoted on): DeepSeek-V3-shape FP8 MoE decode layer,
+hidden 7168, 256 routed experts + 1 shared, expert intermediate 2048, sigmoid grouped top-8 (8 groups, keep 4),
+renormalised weights x 2.5, E4M3 weights with 128x128 f32 block scales, batch 1 by default.
+A step = one layer call (router logits -> top-k -> expert contributions -> combine) on one token batch
+already resident in HBM. Successive steps use different seeded tokens from a ring, so the selected experts
+change every step and their weights come from HBM, not from the 256 MB Infinity Cache.
+
+Prints ONE JSON line (see README / DESIGN.md for the fields).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--batch", type=int, default=1, help="decode tokens per step (1, 8, 64)")
+    ap.add_argument("--experts", type=int, default=256)
+    ap.add_argument("--ring", type=int, default=64, help="distinct token batches cycled through")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph per ring slot")
+    ap.add_argument("--seed", type=int, default=20251)
+    return ap.parse_args()
+
+
+def build_layer(args, torch, capi, ops, synth):
+    H, I, E, K = 7168, 2048, args.experts, 8
+    dev = "cuda"
+    table = ops.ExpertTable.allocate(capi.FMT_FP8_BLOCK128, E + 1, H, I, dev)
+    for e in range(E + 1):
+        v = table.expert_views(e)
+        for i, shape in enumerate([(I, H), (I, H), (H, I)]):
+            w = synth.normal(shape, 0.02, args.seed * 100003 + e * 3 + i, device=dev)
+            codes, scales = synth.quant_fp8_block(w)
+            v[2 * i].copy_(codes)
+            v[2 * i + 1].copy_(scales)
+    shared = table.shared_struct(E)
+    table.experts = E
+    router = synth.normal((E, H), 0.02, args.seed + 1, device=dev, dtype=torch.bfloat16)
+    bias = torch.zeros(E, dtype=torch.float32, device=dev)
+    layer = ops.NativeMoe(table, shared, router, bias, args.batch, K, routed_scaling=2.5, n_group=8, topk_group=4,
+                          swiglu=capi.SWIGLU_TWICE, routed_weight=capi.WEIGHT_AFTER_DOWN_BF16, combine_mode=capi.COMBINE_UNGATED)
+    xs = [synth.normal((args.batch, H), 1.0, args.seed + 1000 + i, device=dev, dtype=torch.bfloat16) for i in range(args.ring)]
+    return table, layer, xs, (H, I, E, K)
+
+
+def layer_bytes(table, distinct, rows, dims):
+    H, I, E, K = dims
+    per = table.weight_bytes_per_expert()
+    return (distinct + 1) * per + E * H * 2 + rows * H * 2 * (2 + K)
+
+
+def gate_up_bytes(distinct, rows, dims):
+    """Algorithmic bytes of one gate/up launch: gate+up codes and scales of every expert touched (routed distinct
+    + shared), the token rows read and the activations written."""
+    H, I, E, K = dims
+    per = 2 * I * H + 2 * 4 * (-(-I // 128)) * (-(-H // 128))
+    return (distinct + 1) * per + rows * H * 2 + rows * (K + 1) * I * 2
+
+
+def cpu_baseline(args, torch, table, layer, xs, dims):
+    """The reference's CPU expert path (multithreaded port in oracle/cpu_baseline.cpp) on a bounded sample of the
+    same workload: the routed + shared experts of a few ring slots, weights copied to host, cold between trials."""
+    import numpy as np
+    import oracle as orc
+    H, I, E, K = dims
+    threads = min(orc.cpubase().cpubase_max_threads(), len(os.sched_getaffinity(0)))
+    slots = list(range(min(6, len(xs))))  # 1 warm-up + 5 timed trials (src/cpu/expert_ffn.rs:3000-3034)
+    jobs = []
+    for s in slots:
+        layer.run(xs[s])
+        torch.cuda.synchronize()
+        ids = layer.ids.cpu().numpy()
+        wts = layer.weights.cpu().numpy()
+        rows = min(args.batch, 4)  # bounded sample: at most 4 token rows of the batch
+        experts, rws, w, ap = [], [], [], []
+        cache = {}
+
+        def host(e):
+            if e not in cache:
+                cache[e] = tuple(v.cpu().numpy() for v in table.expert_views(e))
+            return cache[e]
+        for r in range(rows):
+            for c in range(K):
+                experts.append(host(int(ids[r, c]))); rws.append(r); w.append(float(wts[r, c])); ap.append(1)
+            experts.append(host(E)); rws.append(r); w.append(1.0); ap.append(0)
+        x_bits = xs[s].view(torch.int16).cpu().numpy().view(np.uint16)
+        jobs.append((orc.CpuDecodeJob(x_bits, rws, experts, w, ap), rows))
+    times = []
+    for i, (job, rows) in enumerate(jobs):
+        t0 = time.perf_counter()
+        job.run(threads)
+        dt = time.perf_counter() - t0
+        if i > 0:
+            times.append(dt / rows)
+    times.sort()
+    med = times[len(times) // 2]
+    rows = jobs[0][1]
+    return {"value": med * 1e6, "unit": "us/layer per token row", "cores": threads, "kind": "port",
+            "isa": orc.cpubase().cpubase_isa().decode(),
+            "sample": "%d ring slots x %d token row(s), %d expert FFNs per row (top-%d + shared), weights cold per trial, "
+                      "1 warm-up + %d timed, median" % (len(jobs), rows, K + 1, K, len(times)),
+            "tokens_per_s": 1.0 / med}
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (expert-parallel sharding is described in DESIGN.md); "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from flyingfish_amd import capi, ops, synth
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(1)
+    capi.lib()  # fail loudly when the HIP library is missing
+    table, layer, xs, dims = build_layer(args, torch, capi, ops, synth)
+    H, I, E, K = dims
+    torch.cuda.synchronize()
+
+    # distinct experts per ring slot (measured from the ids)
+    distinct = []
+    for x in xs:
+        layer.run(x)
+        torch.cuda.synchronize()
+        distinct.append(int(torch.unique(layer.ids).numel()))
+    assert int(layer.status.item()) == 0, "combine saw a (row, choice) slot that was not contributed exactly once"
+
+    graphs = None
+    if not args.no_graph:
+        graphs = []
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for x in xs:
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g, stream=side):
+                    layer.run(x)
+                graphs.append(g)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+
+    def step(i):
+        if graphs is not None:
+            graphs[i % len(graphs)].replay()
+        else:
+            layer.run(xs[i % len(xs)])
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(args.warmup + i)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    us_per_layer = elapsed / args.steps * 1e6
+    used = [distinct[(args.warmup + i) % len(xs)] for i in range(args.steps)]
+    mean_distinct = sum(used) / len(used)
+    bytes_layer = layer_bytes(table, mean_distinct, args.batch, dims)
+
+    # dominant kernel: the gate/up + SwiGLU launch, timed alone with events on the launch stream
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    dec = layer.decode
+    for i in range(args.steps):
+        x = xs[(args.warmup + i) % len(xs)]
+        ops.RouteOps.logits_f32(x, layer.router, out=layer.logits)
+        ops.RouteOps.topk_noaux(layer.logits, layer.bias, K, capi.NOAUX_SIGMOID, 2.5, 8, 4, True, out=(layer.ids, layer.weights))
+        ev[i][0].record()
+        dec.contribute(x, layer.ids, layer.weights, stage=0)
+        ev[i][1].record()
+        dec.contribute(x, layer.ids, layer.weights, stage=1)
+    torch.cuda.synchronize()
+    kt = sorted(a.elapsed_time(b) * 1e3 for a, b in ev)  # us
+    k_avg = sum(kt) / len(kt)
+    k_bytes = gate_up_bytes(mean_distinct, args.batch, dims)
+    achieved = k_bytes / (k_avg * 1e-6) / 1e9
+
+    out = {
+        "metric": "moe_layer_decode_us", "value": us_per_layer, "unit": "us/layer", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": us_per_layer / 1e3,
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "fp8_e4m3 weights, bf16 activations, f32 accumulate",
+        "data": "synthetic",
+        "config": {"workload": "DeepSeek-V3-shape FP8 MoE decode layer (BASELINE config 3), batch %d" % args.batch,
+                   "hidden": H, "intermediate": I, "experts": E, "shared_experts": 1, "top_k": K,
+                   "routing": "sigmoid grouped top-8 (8 groups, keep 4), renormalised x2.5",
+                   "weights": "E4M3 + f32 128x128 block scales", "act_mode": "FFMOE_ACT_BF16 (W8A16)",
+                   "batch": args.batch, "ring": len(xs), "launch": "eager" if graphs is None else "hip graph per ring slot"},
+        "tokens_per_s": args.batch / (us_per_layer * 1e-6),
+        "distinct_routed_experts": mean_distinct,
+        "layer_bytes": bytes_layer,
+        "layer_hbm_gbps": bytes_layer / (us_per_layer * 1e-6) / 1e9,
+        "layer_hbm_frac": bytes_layer / (us_per_layer * 1e-6) / 1e9 / HBM_PEAK_GBPS,
+        "roofline": {"kernel": "k_decode_stage<FmtFp8, 4, 0, %d> (gate/up + SwiGLU)" % (1 if args.batch == 1 else 8),
+                     "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
+                     "bytes_per_launch": k_bytes, "avg_us": k_avg, "min_us": kt[0], "median_us": kt[len(kt) // 2]},
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(args, torch, table, layer, xs, dims)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -268,8 +268,8 @@ extern "C" __attribute__((visibility("default"))) uint64_t ffmoe_decode_scratch_
   return h + groups + 256;
 }
 
-extern "C" __attribute__((visibility("default"))) int ffmoe_decode_contribute(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared,
-                                       const ffmoe_decode* args, void* stream) {
+static int decode_impl(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared, const ffmoe_decode* args,
+                       int stage_mask, void* stream) {
   FF_REQUIRE(table && args, FFMOE_ERR_NULL, "table/args is NULL");
   const int R = args->rows, K = args->top_k, E = table->experts, H = table->hidden, I = table->inter;
   FF_REQUIRE(R >= 1 && K >= 1 && K <= FFMOE_MAX_TOP_K && E >= 1 && E <= FFMOE_MAX_EXPERTS, FFMOE_ERR_SHAPE,
@@ -355,7 +355,7 @@ extern "C" __attribute__((visibility("default"))) int ffmoe_decode_contribute(co
     p.groups = (GroupDesc*)(sc + hbytes);
     const uint64_t max_groups = uint64_t(A) + R + 2;
     p.counters = (int*)(sc + hbytes + ((max_groups * sizeof(GroupDesc) + 255) & ~uint64_t(255)));
-    hipLaunchKernelGGL(k_group_assignments, dim3(1), dim3(1024), A * sizeof(int), st, args->ids, args->active, table->valid, p.groups,
+    if (stage_mask & 1) hipLaunchKernelGGL(k_group_assignments, dim3(1), dim3(1024), A * sizeof(int), st, args->ids, args->active, table->valid, p.groups,
                        p.counters, R, K, E, p.has_shared, rg);
     FF_TRY(ff_launch_status());
   } else {
@@ -364,13 +364,28 @@ extern "C" __attribute__((visibility("default"))) int ffmoe_decode_contribute(co
   }
   switch (fmt) {
     case FFMOE_FMT_FP8_BLOCK128:
-      FF_TRY((launch_stage<FmtFp8, 0>(p, rg, st)));
-      return launch_stage<FmtFp8, 1>(p, rg, st);
+      if (stage_mask & 1) FF_TRY((launch_stage<FmtFp8, 0>(p, rg, st)));
+      if (stage_mask & 2) FF_TRY((launch_stage<FmtFp8, 1>(p, rg, st)));
+      break;
     case FFMOE_FMT_NVFP4:
-      FF_TRY((launch_stage<FmtNvfp4, 0>(p, rg, st)));
-      return launch_stage<FmtNvfp4, 1>(p, rg, st);
+      if (stage_mask & 1) FF_TRY((launch_stage<FmtNvfp4, 0>(p, rg, st)));
+      if (stage_mask & 2) FF_TRY((launch_stage<FmtNvfp4, 1>(p, rg, st)));
+      break;
     default:
-      FF_TRY((launch_stage<FmtBf16, 0>(p, rg, st)));
-      return launch_stage<FmtBf16, 1>(p, rg, st);
+      if (stage_mask & 1) FF_TRY((launch_stage<FmtBf16, 0>(p, rg, st)));
+      if (stage_mask & 2) FF_TRY((launch_stage<FmtBf16, 1>(p, rg, st)));
+      break;
   }
+  return 0;
+}
+
+extern "C" __attribute__((visibility("default"))) int ffmoe_decode_contribute(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared,
+                                       const ffmoe_decode* args, void* stream) {
+  return decode_impl(table, shared, args, 3, stream);
+}
+
+extern "C" __attribute__((visibility("default"))) int ffmoe_decode_contribute_stage(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared,
+                                             const ffmoe_decode* args, int stage, void* stream) {
+  FF_REQUIRE(stage == 0 || stage == 1, FFMOE_ERR_SHAPE, "decode stage %d is neither 0 (gate/up) nor 1 (down)", stage);
+  return decode_impl(table, shared, args, 1 << stage, stream);
 }

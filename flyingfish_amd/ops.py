@@ -195,15 +195,18 @@ class DecodeOps:
         self._table_c = table.c_struct()
         self._shared_c = shared
 
-    def contribute(self, x, ids, weights, active=None):
+    def contribute(self, x, ids, weights, active=None, stage=None):
+        """stage None = both launches; 0 / 1 = only the gate-up / only the down launch."""
         act_mode, swiglu, limit, rw, wf32 = self.cfg
         d = capi.Decode(self.rows, self.top_k, act_mode, swiglu, limit, rw, wf32,
                         x.data_ptr(), ids.data_ptr(), active.data_ptr() if active is not None else None, weights.data_ptr(),
                         self.contributions.data_ptr(), self.shared_out.data_ptr() if self.shared_out is not None else None,
                         self.done.data_ptr(), self.scratch.data_ptr(), self.scratch.numel())
-        capi.check(capi.lib().ffmoe_decode_contribute(ctypes.byref(self._table_c),
-                                                      ctypes.byref(self._shared_c) if self._shared_c is not None else None,
-                                                      ctypes.byref(d), _stream()))
+        sh = ctypes.byref(self._shared_c) if self._shared_c is not None else None
+        if stage is None:
+            capi.check(capi.lib().ffmoe_decode_contribute(ctypes.byref(self._table_c), sh, ctypes.byref(d), _stream()))
+        else:
+            capi.check(capi.lib().ffmoe_decode_contribute_stage(ctypes.byref(self._table_c), sh, ctypes.byref(d), stage, _stream()))
         return self.contributions, self.shared_out
 
 

@@ -170,6 +170,13 @@ uint64_t ffmoe_decode_scratch_bytes(int rows, int top_k, int experts, int hidden
 int ffmoe_decode_contribute(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared,
                             const ffmoe_decode* args, void* stream);
 
+/* The two launches of the contribution as separate calls, like the reference's gate_up and down launches
+ * (src/backend/cuda/moe/decode.rs:486-490 and :513-517): stage 0 = gate/up + SwiGLU into scratch (and the
+ * grouping of assignments by expert), stage 1 = down + routing weight from scratch. Stage 0 then stage 1 with the
+ * same arguments equals ffmoe_decode_contribute. */
+int ffmoe_decode_contribute_stage(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared,
+                                  const ffmoe_decode* args, int stage, void* stream);
+
 /* ------------------------------------------------------------------------------------------------
  * Standalone linears, M <= 16 "skinny" and beyond. y[M,N] = x[M,K] * W[N,K]^T, BF16 in / BF16 out.
  */

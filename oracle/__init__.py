@@ -334,3 +334,43 @@ def bf16_order_key(bits):
 
 def bf16_ulp_max(actual_bf16, ref_bf16):
     return int(np.max(np.abs(bf16_order_key(actual_bf16) - bf16_order_key(ref_bf16)))) if np.size(actual_bf16) else 0
+
+
+# ------------------------------------------------------------------------------------------------
+# multithreaded CPU baseline (cpu_baseline.cpp): port of the reference's two-phase CPU expert pool
+def cpubase():
+    global _base
+    if _base is None:
+        _base = _load(_BASE_PATH)
+        _base.cpubase_max_threads.restype = ctypes.c_int
+        _base.cpubase_isa.restype = ctypes.c_char_p
+    return _base
+
+
+class CpuDecodeJob:
+    """Host copies of the experts a decode batch touches, laid out for cpubase_moe_decode.
+
+    experts: list of (gate_codes, gate_scales, up_codes, up_scales, down_codes, down_scales) numpy arrays,
+    one entry per assignment (repeat the entry when two assignments share an expert).
+    """
+
+    def __init__(self, x_bf16, rows, experts, weights, apply_w, boundary=AFTER_DOWN_BF16):
+        self.x = _c(x_bf16, np.uint16)
+        self.rows = _c(rows, np.int32)
+        self.keep = [tuple(_c(a, a.dtype) for a in ex) for ex in experts]
+        self.ptrs = np.array([[a.ctypes.data for a in ex] for ex in self.keep], dtype=np.uint64)
+        self.w = _c(weights, np.float32)
+        self.apply = _c(apply_w, np.int32)
+        self.n = len(experts)
+        self.I, self.H = self.keep[0][0].shape
+        self.boundary = boundary
+        self.xf = np.empty((self.n, self.H), dtype=np.float32)
+        self.act = np.empty((self.n, self.I), dtype=np.uint16)
+        self.out = np.empty((self.n, self.H), dtype=np.uint16)
+
+    def run(self, threads):
+        rc = cpubase().cpubase_moe_decode(_p(self.x), _p(self.rows), _p(self.ptrs), _p(self.w), _p(self.apply), self.n, self.H,
+                                          self.I, self.boundary, int(threads), _p(self.xf), _p(self.act), _p(self.out))
+        if rc != 0:
+            raise RuntimeError("cpubase_moe_decode rejected the shapes")
+        return self.out

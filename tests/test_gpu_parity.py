@@ -340,5 +340,12 @@ def test_native_moe_layer_matches_oracle_pipeline():
     contrib = oracle_contributions(ref, bits(x), oi, ow, orc.TWICE, 0.0, orc.BEFORE_CONTRIBUTION_BF16)
     sh = oracle_shared(ref[experts], bits(x), orc.TWICE, 0.0)
     want = orc.combine(contrib, sh, None, oi, None, orc.COMBINE_BF16)
-    # the BF16 running sum compounds one rounding per choice: allow top_k + 1 steps at the row scale
-    assert_close_bf16(bits(y), want, "layer output", max_ulp=top_k + 1, rel=4e-3)
+    # Every contribution may sit 2 BF16 steps from the oracle's and the BF16 running sum rounds once per term, so the
+    # bound per element is 3 steps per term at the largest term's magnitude (the reference bounds its own GPU layer
+    # by measured combine-order spread + 1 ulp at the largest output, src/backend/cuda/moe/reference.rs:613-678).
+    terms = np.concatenate([orc.bf16_to_f32(contrib), orc.bf16_to_f32(sh)[:, None, :], orc.bf16_to_f32(want)[:, None, :]], axis=1)
+    mag = np.max(np.abs(terms), axis=1).astype(np.float64)
+    ulp = 2.0 ** (np.floor(np.log2(np.maximum(mag, 1e-30))) - 7)
+    err = np.abs(orc.bf16_to_f32(bits(y)).astype(np.float64) - orc.bf16_to_f32(want).astype(np.float64))
+    assert np.all(err <= 3 * (top_k + 1) * ulp), float(np.max(err / ulp))
+    assert orc.rel_l2(bits(y), want) <= 4e-3

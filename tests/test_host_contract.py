@@ -1,0 +1,136 @@
+"""Host-side checks that need no GPU: the C-ABI library loads, exports every declared symbol, and rejects
+contract violations before touching the device; the synthetic quantizers equal the oracle's; the CPU baseline
+equals the scalar oracle bit for bit."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+import oracle as orc
+from flyingfish_amd import capi, synth
+from flyingfish_amd.ops import ExpertTable
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "ffmoe.h")).read()
+    declared = set(re.findall(r"\b(ffmoe_[a-z0-9_]+)\s*\(", header))
+    lib = capi.lib()
+    for name in sorted(declared):
+        assert hasattr(lib, name), name
+    assert declared == set(capi.EXPORTS)
+    assert lib.ffmoe_version() == 1
+
+
+def test_route_contract_violations_are_reported_before_launch():
+    L = capi.lib()
+    assert L.ffmoe_route_topk(None, 16, 16, 1, 64, 4, 0, None) == capi.ERR_NULL and "NULL" in capi.last_error()
+    assert L.ffmoe_route_topk(24, 16, 32, 1, 64, 4, 0, None) == capi.ERR_ALIGN
+    assert L.ffmoe_route_topk(4096, 8192, 12288, 1, 64, 64, 0, None) == capi.ERR_SHAPE      # top_k > 32
+    assert L.ffmoe_route_topk(4096, 8192, 12288, 1, 2048, 4, 0, None) == capi.ERR_SHAPE     # experts > 1024
+    assert L.ffmoe_route_topk(4096, 8192, 12288, 1, 4, 4, 0, None) == capi.ERR_SHAPE        # top_k == experts
+    assert L.ffmoe_route_topk(4096, 4096, 12288, 1, 64, 4, 0, None) == capi.ERR_OVERLAP
+    assert L.ffmoe_route_logits_bf16(4096, 1 << 20, 1 << 21, 1, 64, 100, None) == capi.ERR_SHAPE  # hidden % 8
+    assert L.ffmoe_route_topk_noaux(4096, None, 0, 8192, 12288, 1, 1, 256, 8, 0, ctypes.c_float(-1.0), 1, 1, None) == capi.ERR_SHAPE
+    assert L.ffmoe_route_topk_noaux(4096, None, 0, 8192, 12288, 1, 1, 256, 8, 0, ctypes.c_float(2.5), 7, 4, None) == capi.ERR_SHAPE
+    assert L.ffmoe_route_topk_noaux(4096, None, 0, 8192, 12288, 1, 1, 256, 8, 3, ctypes.c_float(2.5), 1, 1, None) == capi.ERR_UNSUPPORTED
+
+
+def _decode_args(**kw):
+    d = dict(rows=1, top_k=4, act_mode=0, swiglu=0, swiglu_limit=0.0, routed_weight=0, weights_f32=0, x=1 << 20, ids=2 << 20,
+             active=None, weights=3 << 20, contributions=4 << 20, shared_out=None, done=None, scratch=8 << 20, scratch_bytes=1 << 20)
+    d.update(kw)
+    return capi.Decode(d["rows"], d["top_k"], d["act_mode"], d["swiglu"], d["swiglu_limit"], d["routed_weight"], d["weights_f32"],
+                       d["x"], d["ids"], d["active"], d["weights"], d["contributions"], d["shared_out"], d["done"], d["scratch"],
+                       d["scratch_bytes"])
+
+
+def test_decode_contract_violations_are_reported_before_launch():
+    L = capi.lib()
+    table = capi.ExpertTable(capi.FMT_FP8_BLOCK128, 64, 2048, 1408, 16 << 20, None, None)
+
+    def call(t=table, **kw):
+        a = _decode_args(**kw)
+        return L.ffmoe_decode_contribute(ctypes.byref(t), None, ctypes.byref(a), None)
+    assert call(x=None) == capi.ERR_NULL
+    assert call(x=(1 << 20) + 8) == capi.ERR_ALIGN
+    assert call(top_k=40) == capi.ERR_SHAPE
+    assert call(rows=4096) == capi.ERR_SHAPE and "prefill" in capi.last_error()
+    assert call(scratch_bytes=16) == capi.ERR_SCRATCH
+    assert call(contributions=1 << 20) == capi.ERR_OVERLAP
+    assert call(act_mode=1) == capi.ERR_UNSUPPORTED
+    assert call(swiglu=2, swiglu_limit=0.0) == capi.ERR_SHAPE
+    assert call(swiglu=7) == capi.ERR_UNSUPPORTED
+    bad = capi.ExpertTable(capi.FMT_FP8_BLOCK128, 64, 2000, 1408, 16 << 20, None, None)
+    assert call(t=bad) == capi.ERR_SHAPE
+    assert L.ffmoe_decode_contribute_stage(ctypes.byref(table), None, ctypes.byref(_decode_args()), 2, None) == capi.ERR_SHAPE
+    assert L.ffmoe_decode_scratch_bytes(1, 8, 256, 7168, 2048, 2048) >= 9 * 2048 * 2
+
+
+def test_linear_and_combine_contract_violations():
+    L = capi.lib()
+    assert L.ffmoe_linear_fp8_block(1 << 20, 2 << 20, 3 << 20, 4 << 20, 1, 256, 100, 0, None, 0, None) == capi.ERR_SHAPE
+    assert L.ffmoe_linear_fp8_block(1 << 20, 2 << 20, 3 << 20, 3 << 20, 1, 256, 128, 0, None, 0, None) == capi.ERR_OVERLAP
+    assert L.ffmoe_linear_fp8_block(1 << 20, 2 << 20, 3 << 20, 4 << 20, 1, 256, 128, 1, None, 0, None) == capi.ERR_NULL  # scratch
+    assert L.ffmoe_linear_nvfp4(1 << 20, 2 << 20, None, 3 << 20, 4 << 20, 1, 256, 128, None) == capi.ERR_NULL
+    assert L.ffmoe_combine(1 << 20, 2 << 20, None, 3 << 20, None, None, 4 << 20, None, 1, 8, 100, 2, None) == capi.ERR_SHAPE
+    assert L.ffmoe_combine(1 << 20, 2 << 20, None, 3 << 20, None, None, 4 << 20, None, 1, 8, 128, 0, None) == capi.ERR_NULL  # gated needs scale
+    assert L.ffmoe_combine(1 << 20, 2 << 20, None, 3 << 20, None, None, 4 << 20, None, 1, 8, 128, 9, None) == capi.ERR_UNSUPPORTED
+    assert L.ffmoe_swiglu(1 << 20, 2 << 20, 3 << 20, 1, 12, 0, ctypes.c_float(0), None) == capi.ERR_SHAPE
+    assert L.ffmoe_quant_fp8_f32_128(1 << 20, 1 << 20, 2 << 20, 1, 128, None) == capi.ERR_OVERLAP
+
+
+def test_slot_layout_matches_the_reference_catalogue():
+    # src/experts/catalogue.rs:180-222: codes gate|up|down, then gate, up, down scales; BASELINE byte counts
+    offs, size = ExpertTable.slot_layout(capi.FMT_FP8_BLOCK128, 7168, 2048)
+    w = 7168 * 2048
+    assert offs == [0, 3 * w, w, 3 * w + 16 * 56 * 4, 2 * w, 3 * w + 2 * 16 * 56 * 4]
+    assert 3 * w + 3 * 16 * 56 * 4 == 44050944 and size >= 44050944 and size % 256 == 0
+    offs, size = ExpertTable.slot_layout(capi.FMT_FP8_BLOCK128, 2048, 1408)
+    assert 3 * 2048 * 1408 == 8650752 and offs[1] == 8650752 and (size - 8650752) // 1 >= 2112
+    offs, size = ExpertTable.slot_layout(capi.FMT_NVFP4, 7168, 2048)
+    assert 3 * w // 2 == 22020096 and 3 * w // 16 == 2752512 and offs[1] == 22020096
+
+
+def test_synthetic_quantizers_equal_the_oracle():
+    w = synth.normal((256, 384), 0.02, 1)
+    c, s = synth.quant_fp8_block(w)
+    oc, os_ = orc.quant_weight_fp8_block(w.numpy())
+    assert np.array_equal(c.numpy(), oc) and np.array_equal(s.numpy().view(np.uint32), os_.view(np.uint32))
+    c4, s4, g = synth.quant_nvfp4(w)
+    o4, os4, og = orc.quant_weight_nvfp4(w.numpy())
+    assert np.array_equal(c4.numpy(), o4) and np.array_equal(s4.numpy(), os4) and g == og
+    x = torch.linspace(-448, 448, 200001)
+    tc = synth.e4m3_encode(x).numpy()
+    L = orc.lib()
+    for i in range(0, x.numel(), 389):
+        assert L.orc_encode_e4m3(float(x[i])) == tc[i]
+    ragged = synth.normal((130, 200), 0.02, 2)
+    c, s = synth.quant_fp8_block(ragged)
+    oc, os_ = orc.quant_weight_fp8_block(ragged.numpy())
+    assert np.array_equal(c.numpy(), oc) and np.array_equal(s.numpy().view(np.uint32), os_.view(np.uint32))
+
+
+@pytest.mark.parametrize("threads", [1, 3, 8])
+def test_cpu_baseline_equals_the_scalar_oracle(threads):
+    rng = np.random.default_rng(0)
+    H, I, n = 1024, 512, 3
+    x = orc.f32_to_bf16(rng.normal(size=(2, H)).astype(np.float32))
+    exs = []
+    for a in range(n):
+        mats = []
+        for shape in [(I, H), (I, H), (H, I)]:
+            c, s = orc.quant_weight_fp8_block(rng.normal(scale=0.02, size=shape).astype(np.float32))
+            mats += [c, s]
+        exs.append(tuple(mats))
+    rows, w, ap = [0, 1, 1], [0.5, 0.25, 1.0], [1, 1, 0]
+    for boundary in (orc.AFTER_DOWN_BF16, orc.BEFORE_CONTRIBUTION_BF16):
+        out = orc.CpuDecodeJob(x, rows, exs, w, ap, boundary).run(threads)
+        for a in range(n):
+            g, u, d = (orc.dequant_fp8_block(exs[a][i], exs[a][i + 1]) for i in (0, 2, 4))
+            ref = orc.expert_ffn(x[rows[a]], g, u, d, w[a], orc.TWICE, 0.0, boundary, orc.LANE16, orc.SILU_RCP, apply_weight=bool(ap[a]))
+            assert np.array_equal(ref, out[a])
