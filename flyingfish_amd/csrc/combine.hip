@@ -34,78 +34,90 @@ __global__ __launch_bounds__(256) void k_shared_scale(const uint16_t* __restrict
   }
 }
 
-// One block per row; 8 BF16 per thread and step.
+// grid (ceil(hidden / 2048), rows): one 16-byte vector of 8 BF16 per thread. The first top_k threads rank the
+// active choices by ascending expert id (stable), which is the order of the reference's insertion sort
+// (kernels/moe_combine.cu:51-69); the ranks go through LDS so the accumulation loop indexes no private array.
 __global__ __launch_bounds__(256) void k_combine(const uint16_t* __restrict__ contributions, const uint16_t* __restrict__ shared_out,
                                                  const uint16_t* __restrict__ scale, const int* __restrict__ ids,
                                                  const uint32_t* __restrict__ done, const uint32_t* __restrict__ final_active,
                                                  uint16_t* __restrict__ y, uint32_t* __restrict__ status, int top_k, int hidden,
                                                  int mode) {
-  const int tid = threadIdx.x, row = blockIdx.x;
+  __shared__ int s_order[FFMOE_MAX_TOP_K];
+  __shared__ int s_live;
+  const int tid = threadIdx.x, row = blockIdx.y;
   const int a0 = row * top_k;
-  int order[FFMOE_MAX_TOP_K];
-  int live = 0;
-  if (mode == FFMOE_COMBINE_ACCUM_FP32 || mode == FFMOE_COMBINE_ACCUM_BF16) {
-    live = top_k;
-#pragma unroll 1
-    for (int c = 0; c < top_k; ++c) order[c] = c;
-  } else {
-    // stable insertion sort of the active choices by ascending expert id (kernels/moe_combine.cu:51-69)
-    bool bad = false;
-#pragma unroll 1
-    for (int c = 0; c < top_k; ++c) {
-      const uint32_t want = final_active ? final_active[a0 + c] : 1u;
-      if (done && done[a0 + c] != want) bad = true;
-      if (want == 0u) continue;
-      int p = live;
-      while (p > 0 && ids[a0 + order[p - 1]] > ids[a0 + c]) { order[p] = order[p - 1]; --p; }
-      order[p] = c;
-      ++live;
-    }
-    if (bad && status && tid == 0) atomicOr(status, 1u);
-  }
-  const float sc = (mode == FFMOE_COMBINE_GATED) ? bf16_to_f32(scale[row]) : 0.0f;
-  for (int d0 = tid * 8; d0 < hidden; d0 += 256 * 8) {
-    float acc[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) acc[j] = 0.0f;
-    for (int k = 0; k < live; ++k) {
-      const u32x4 c = load16(contributions + (size_t(a0) + order[k]) * hidden + d0);
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        if (mode == FFMOE_COMBINE_BF16) {
-          acc[2 * q] = bround(__fadd_rn(acc[2 * q], bf16lo(c[q])));
-          acc[2 * q + 1] = bround(__fadd_rn(acc[2 * q + 1], bf16hi(c[q])));
-        } else {
-          acc[2 * q] = __fadd_rn(acc[2 * q], bf16lo(c[q]));
-          acc[2 * q + 1] = __fadd_rn(acc[2 * q + 1], bf16hi(c[q]));
+  const bool ordered = !(mode == FFMOE_COMBINE_ACCUM_FP32 || mode == FFMOE_COMBINE_ACCUM_BF16);
+  if (tid < top_k) {
+    if (!ordered) {
+      s_order[tid] = tid;
+    } else {
+      const uint32_t want = final_active ? final_active[a0 + tid] : 1u;
+      if (done && done[a0 + tid] != want && status && blockIdx.x == 0) atomicOr(status, 1u);
+      if (want != 0u) {
+        const int mine = ids[a0 + tid];
+        int rank = 0;
+        for (int c = 0; c < top_k; ++c) {
+          const bool act = final_active ? final_active[a0 + c] != 0u : true;
+          const int other = ids[a0 + c];
+          rank += (act && (other < mine || (other == mine && c < tid))) ? 1 : 0;
         }
+        s_order[rank] = tid;
       }
     }
-    u32x4 sh = {0, 0, 0, 0};
-    if (mode != FFMOE_COMBINE_ROUTED) sh = load16(shared_out + size_t(row) * hidden + d0);
-    u32x4 out;
+  }
+  if (tid == 0) {
+    int live = top_k;
+    if (ordered && final_active) {
+      live = 0;
+      for (int c = 0; c < top_k; ++c) live += final_active[a0 + c] != 0u ? 1 : 0;
+    }
+    s_live = live;
+  }
+  __syncthreads();
+  const int live = s_live;
+  const int d0 = (blockIdx.x * 256 + tid) * 8;
+  if (d0 >= hidden) return;
+  const float sc = (mode == FFMOE_COMBINE_GATED) ? bf16_to_f32(scale[row]) : 0.0f;
+  float acc[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) acc[j] = 0.0f;
+  for (int k = 0; k < live; ++k) {
+    const u32x4 c = load16(contributions + (size_t(a0) + s_order[k]) * hidden + d0);
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-      float r[2];
-#pragma unroll
-      for (int hsel = 0; hsel < 2; ++hsel) {
-        const float s = hsel ? bf16hi(sh[q]) : bf16lo(sh[q]);
-        const float a = acc[2 * q + hsel];
-        float v;
-        switch (mode) {
-          case FFMOE_COMBINE_GATED: v = __fadd_rn(bround(a), bround(__fmul_rn(sc, s))); break;
-          case FFMOE_COMBINE_UNGATED:
-          case FFMOE_COMBINE_ACCUM_BF16: v = __fadd_rn(bround(a), s); break;
-          case FFMOE_COMBINE_BF16:
-          case FFMOE_COMBINE_ACCUM_FP32: v = __fadd_rn(a, s); break;
-          default: v = a; break;
-        }
-        r[hsel] = v;
+      if (mode == FFMOE_COMBINE_BF16) {
+        acc[2 * q] = bround(__fadd_rn(acc[2 * q], bf16lo(c[q])));
+        acc[2 * q + 1] = bround(__fadd_rn(acc[2 * q + 1], bf16hi(c[q])));
+      } else {
+        acc[2 * q] = __fadd_rn(acc[2 * q], bf16lo(c[q]));
+        acc[2 * q + 1] = __fadd_rn(acc[2 * q + 1], bf16hi(c[q]));
       }
-      out[q] = pack_bf16x2(r[0], r[1]);
     }
-    *reinterpret_cast<u32x4*>(y + size_t(row) * hidden + d0) = out;
   }
+  u32x4 sh = {0, 0, 0, 0};
+  if (mode != FFMOE_COMBINE_ROUTED) sh = load16(shared_out + size_t(row) * hidden + d0);
+  u32x4 out;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    float r[2];
+#pragma unroll
+    for (int hsel = 0; hsel < 2; ++hsel) {
+      const float s = hsel ? bf16hi(sh[q]) : bf16lo(sh[q]);
+      const float a = acc[2 * q + hsel];
+      float v;
+      switch (mode) {
+        case FFMOE_COMBINE_GATED: v = __fadd_rn(bround(a), bround(__fmul_rn(sc, s))); break;
+        case FFMOE_COMBINE_UNGATED:
+        case FFMOE_COMBINE_ACCUM_BF16: v = __fadd_rn(bround(a), s); break;
+        case FFMOE_COMBINE_BF16:
+        case FFMOE_COMBINE_ACCUM_FP32: v = __fadd_rn(a, s); break;
+        default: v = a; break;
+      }
+      r[hsel] = v;
+    }
+    out[q] = pack_bf16x2(r[0], r[1]);
+  }
+  *reinterpret_cast<u32x4*>(y + size_t(row) * hidden + d0) = out;
 }
 
 }  // namespace ffmoe
@@ -140,7 +152,7 @@ extern "C" __attribute__((visibility("default"))) int ffmoe_combine(const void* 
   FF_NO_OVERLAP(y, yb, contributions, cb);
   if (mode != FFMOE_COMBINE_ROUTED) FF_NO_OVERLAP(y, yb, shared_out, yb);
   if (ordered) FF_NO_OVERLAP(y, yb, ids, size_t(rows) * top_k * 4);
-  hipLaunchKernelGGL(k_combine, dim3(rows), dim3(256), 0, (hipStream_t)stream, (const uint16_t*)contributions,
+  hipLaunchKernelGGL(k_combine, dim3((hidden / 8 + 255) / 256, rows), dim3(256), 0, (hipStream_t)stream, (const uint16_t*)contributions,
                      (const uint16_t*)shared_out, (const uint16_t*)scale, ids, done, final_active, (uint16_t*)y, status, top_k,
                      hidden, mode);
   return ff_launch_status();

@@ -142,19 +142,80 @@ __device__ __forceinline__ uint16_t swiglu_bf16(float g, float u, int mode, floa
   return f32_to_bf16(prod);
 }
 
+// ---------------------------------------------------------------------------------------------
+// Wave-wide reductions on the DPP data path (no LDS round trips). The sequence is the usual gfx9 one:
+// quad swaps, half-row and row mirrors leave every lane of a 16-lane row with the row total; two
+// row broadcasts then carry the totals up, so lane 63 ends with the wave total, which is read back
+// as a wave-uniform value. The summation order is fixed, so results do not depend on scheduling.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_or(float old, float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, old), __builtin_bit_cast(int, v), CTRL,
+                                                                ROW_MASK, 0xf, false));
+}
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ int dpp_or(int old, int v) {
+  return __builtin_amdgcn_update_dpp(old, v, CTRL, ROW_MASK, 0xf, false);
+}
+constexpr int DPP_QUAD_SWAP1 = 0xB1;    // quad_perm:[1,0,3,2]
+constexpr int DPP_QUAD_SWAP2 = 0x4E;    // quad_perm:[2,3,0,1]
+constexpr int DPP_ROW_HALF_MIRROR = 0x141;
+constexpr int DPP_ROW_MIRROR = 0x140;
+constexpr int DPP_ROW_BCAST15 = 0x142;
+constexpr int DPP_ROW_BCAST31 = 0x143;
+
 // Sum over the 64 lanes of a wave; every lane receives the total.
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, WAVE);
-  return v;
+  v += dpp_or<DPP_QUAD_SWAP1, 0xf>(0.0f, v);
+  v += dpp_or<DPP_QUAD_SWAP2, 0xf>(0.0f, v);
+  v += dpp_or<DPP_ROW_HALF_MIRROR, 0xf>(0.0f, v);
+  v += dpp_or<DPP_ROW_MIRROR, 0xf>(0.0f, v);
+  v += dpp_or<DPP_ROW_BCAST15, 0xa>(0.0f, v);
+  v += dpp_or<DPP_ROW_BCAST31, 0xc>(0.0f, v);
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+__device__ __forceinline__ float wave_max(float v) {
+  v = fmaxf(v, dpp_or<DPP_QUAD_SWAP1, 0xf>(v, v));
+  v = fmaxf(v, dpp_or<DPP_QUAD_SWAP2, 0xf>(v, v));
+  v = fmaxf(v, dpp_or<DPP_ROW_HALF_MIRROR, 0xf>(v, v));
+  v = fmaxf(v, dpp_or<DPP_ROW_MIRROR, 0xf>(v, v));
+  v = fmaxf(v, dpp_or<DPP_ROW_BCAST15, 0xa>(v, v));
+  v = fmaxf(v, dpp_or<DPP_ROW_BCAST31, 0xc>(v, v));
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+// Arg-max under (value desc, id asc); the winner is returned wave-uniform.
+__device__ __forceinline__ void wave_argmax(float& v, int& id) {
+#define FF_ARGMAX_STEP(CTRL, MASK)                                  \
+  {                                                                 \
+    const float ov = dpp_or<CTRL, MASK>(v, v);                      \
+    const int oi = dpp_or<CTRL, MASK>(id, id);                      \
+    const bool take = ov > v || (ov == v && oi < id);               \
+    v = take ? ov : v;                                              \
+    id = take ? oi : id;                                            \
+  }
+  FF_ARGMAX_STEP(DPP_QUAD_SWAP1, 0xf)
+  FF_ARGMAX_STEP(DPP_QUAD_SWAP2, 0xf)
+  FF_ARGMAX_STEP(DPP_ROW_HALF_MIRROR, 0xf)
+  FF_ARGMAX_STEP(DPP_ROW_MIRROR, 0xf)
+  FF_ARGMAX_STEP(DPP_ROW_BCAST15, 0xa)
+  FF_ARGMAX_STEP(DPP_ROW_BCAST31, 0xc)
+#undef FF_ARGMAX_STEP
+  v = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+  id = __builtin_amdgcn_readlane(id, 63);
 }
 
-// 16-byte global load that bypasses nothing special: plain vector load, kept as one instruction.
-__device__ __forceinline__ u32x4 load16(const void* p) { return *reinterpret_cast<const u32x4*>(p); }
-// Streaming 16-byte load for data read exactly once (weights): non-temporal hint keeps it from
+// Loads through pointers known to be global memory. Weight and scale addresses arrive as integers in slot
+// tables, so without the explicit address space the compiler would emit flat loads, which also count against
+// the LDS counter and serialize with the activation reads.
+#define FF_GLOBAL __attribute__((address_space(1)))
+template <class T>
+__device__ __forceinline__ T load_global(const void* p) {
+  return *(const FF_GLOBAL T*)(p);
+}
+__device__ __forceinline__ u32x4 load16(const void* p) { return load_global<u32x4>(p); }
+// Streaming 16-byte load for data read exactly once (weights): the non-temporal hint keeps it from
 // displacing reusable lines.
 __device__ __forceinline__ u32x4 load16_stream(const void* p) {
-  return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+  return __builtin_nontemporal_load((const FF_GLOBAL u32x4*)(p));
 }
 
 }  // namespace ffmoe

@@ -39,20 +39,30 @@ __device__ __forceinline__ void make_group(GroupDesc& gd, const DecodeParams& p,
   }
 }
 
+__device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
+
 // STAGE 0: gate/up + SwiGLU -> h[slot, j].   STAGE 1: down (+ routing weight) -> contributions / shared_out.
-template <class F, int S, int STAGE, int RG>
+// A unit is NR consecutive output rows of one group: stage 0 streams NR gate rows and the NR matching up rows
+// (2*NR weight rows sharing every activation read), stage 1 streams NR down rows.
+//
+// Every quantity that decides an address (group, expert, row index, slab) is held wave-uniform in scalar
+// registers, so weight loads take a scalar base plus one per-lane offset. A wave owns a contiguous run of
+// units of the segment; reduced sums of up to 64 units are parked one per lane and the epilogue (SwiGLU or
+// weighting, BF16 rounding, store) runs once per 64 units with coalesced stores.
+template <class F, int S, int STAGE, int RG, int NR>
 __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
-  constexpr int NMAT = STAGE == 0 ? 2 : 1;
+  constexpr int NROWS = STAGE == 0 ? 2 * NR : NR;
   constexpr int NW = 4;
   extern __shared__ __align__(16) uint8_t xs[];
   __shared__ GroupDesc s_gd;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = uni(tid >> 6);
   const int A = p.rows * p.top_k;
   const int n_routed = p.counters ? p.counters[0] : A;
   const int n_shared = p.counters ? p.counters[1] : (p.has_shared ? p.rows : 0);
-  // output rows per group
-  const int out_r = STAGE == 0 ? p.inter : p.hidden;
-  const int out_s = STAGE == 0 ? p.shared_inter : p.hidden;
+  // units per group
+  const int out_r = (STAGE == 0 ? p.inter : p.hidden) / NR;
+  const int out_s = (STAGE == 0 ? p.shared_inter : p.hidden) / NR;
   const long long routed_units = (long long)n_routed * out_r;
   const long long total = routed_units + (long long)n_shared * out_s;
   const long long lo = total * blockIdx.x / gridDim.x, hi = total * (blockIdx.x + 1) / gridDim.x;
@@ -67,88 +77,149 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
     __syncthreads();  // previous segment's readers are done with xs and s_gd
     if (tid == 0) make_group(s_gd, p, g);
     __syncthreads();
-    const GroupDesc gd = s_gd;
-    const bool shared = gd.expert < 0;
+    const int expert = uni(s_gd.expert);
+    const int gn = uni(s_gd.n);
+    int grow[RG], gslot[RG];
+#pragma unroll
+    for (int r = 0; r < RG; ++r) { grow[r] = uni(s_gd.row[r]); gslot[r] = uni(s_gd.slot[r]); }
+    const bool shared = expert < 0;
     const int Kg = STAGE == 0 ? p.hidden : (shared ? p.shared_inter : p.inter);
-    if (gd.n > 0) {
+    if (gn > 0) {
       // activations of the group -> LDS (row r at r*Kg*2)
       const uint16_t* src = STAGE == 0 ? p.x : p.h;
       const int row_words = Kg >> 3;  // 16-byte words per row
-      for (int r = 0; r < gd.n; ++r) {
-        const size_t base = STAGE == 0 ? size_t(gd.row[r]) * p.hidden : size_t(gd.slot[r]) * p.h_stride;
-        const u32x4* s4 = reinterpret_cast<const u32x4*>(src + base);
-        u32x4* d4 = reinterpret_cast<u32x4*>(xs + size_t(r) * Kg * 2);
-        for (int v = tid; v < row_words; v += 256) d4[v] = s4[v];
+#pragma unroll
+      for (int r = 0; r < RG; ++r) {
+        if (r < gn) {
+          const size_t base = STAGE == 0 ? size_t(grow[r]) * p.hidden : size_t(gslot[r]) * p.h_stride;
+          u32x4* d4 = reinterpret_cast<u32x4*>(xs + size_t(r) * Kg * 2);
+          for (int v = tid; v < row_words; v += 256) d4[v] = load16(src + base + size_t(v) * 8);
+        }
       }
     }
     __syncthreads();
-    if (gd.n > 0) {
-      const uint64_t* slot = shared ? p.shared_slot : p.slots + size_t(gd.expert) * 6;
-      const float* gl = shared ? p.shared_global : (p.global_scales ? p.global_scales + size_t(gd.expert) * 3 : nullptr);
-      uint64_t codes[NMAT], scales[NMAT];
-      float global[NMAT];
-      if (STAGE == 0) {
-        codes[0] = slot[0]; scales[0] = slot[1]; global[0] = gl ? gl[0] : 1.0f;
-        codes[NMAT - 1] = slot[2]; scales[NMAT - 1] = slot[3]; global[NMAT - 1] = gl ? gl[1] : 1.0f;
+    if (gn > 0) {
+      // weight row m of a unit comes from matrix m / NR (stage 0: gate, up; stage 1: down). The six addresses are
+      // fetched through scalar-friendly paths (kernel argument or global table), never through a generic pointer.
+      uint64_t sl[6];
+      float gl3[3];
+      if (shared) {
+#pragma unroll
+        for (int i = 0; i < 6; ++i) sl[i] = p.shared_slot[i];
+#pragma unroll
+        for (int i = 0; i < 3; ++i) gl3[i] = p.shared_global[i];
       } else {
-        codes[0] = slot[4]; scales[0] = slot[5]; global[0] = gl ? gl[2] : 1.0f;
+#pragma unroll
+        for (int i = 0; i < 6; ++i) sl[i] = load_global<uint64_t>(p.slots + size_t(expert) * 6 + i);
+#pragma unroll
+        for (int i = 0; i < 3; ++i) gl3[i] = p.global_scales ? load_global<float>(p.global_scales + size_t(expert) * 3 + i) : 1.0f;
+      }
+      uint64_t codes[2], scales[2];
+      float global[2];
+      if (STAGE == 0) {
+        codes[0] = sl[0]; scales[0] = sl[1]; global[0] = gl3[0];
+        codes[1] = sl[2]; scales[1] = sl[3]; global[1] = gl3[1];
+      } else {
+        codes[0] = codes[1] = sl[4]; scales[0] = scales[1] = sl[5]; global[0] = global[1] = gl3[2];
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        codes[i] = (uint64_t(uint32_t(uni(int(codes[i] >> 32)))) << 32) | uint32_t(uni(int(codes[i])));
+        scales[i] = (uint64_t(uint32_t(uni(int(scales[i] >> 32)))) << 32) | uint32_t(uni(int(scales[i])));
+        global[i] = __builtin_bit_cast(float, uni(__builtin_bit_cast(int, global[i])));
       }
       const int nchunks = Kg / F::EPL;
       const int nslabs = (nchunks + S * 64 - 1) / (S * 64);
-      // this wave's units: j0 + wave, j0 + wave + NW, ...; item t = (unit t / nslabs, slab t % nslabs)
-      const int my_units = count > wave ? (count - wave + NW - 1) / NW : 0;
+      // this wave's contiguous run of units inside the segment
+      const int w_lo = count * wave / NW, w_hi = count * (wave + 1) / NW;
+      const int my_units = w_hi - w_lo;
       const int items = my_units * nslabs;
-      UnitBuf<F, S, NMAT> bufA, bufB;
-      float acc[NMAT][RG];
+      const int jw = j0 + w_lo;  // first unit of the run
+      UnitBuf<F, S, NROWS> bufA, bufB;
+      float acc[NROWS][RG];
+      float park[NROWS][RG];  // lane L keeps the sums of unit (batch base + L)
 #pragma unroll
-      for (int m = 0; m < NMAT; ++m)
+      for (int m = 0; m < NROWS; ++m)
 #pragma unroll
-        for (int r = 0; r < RG; ++r) acc[m][r] = 0.0f;
-      auto issue = [&](UnitBuf<F, S, NMAT>& b, int t) {
-        const int j = j0 + wave + (t / nslabs) * NW;
+        for (int r = 0; r < RG; ++r) { acc[m][r] = 0.0f; park[m][r] = 0.0f; }
+      auto issue = [&](UnitBuf<F, S, NROWS>& b, int t) {
+        const int j = (jw + t / nslabs) * NR;  // first output row of the unit
         const int chunk0 = (t % nslabs) * (S * 64);
 #pragma unroll
-        for (int m = 0; m < NMAT; ++m) {
-          const typename F::Row rw = F::row(codes[m], scales[m], global[m], j, Kg);
+        for (int m = 0; m < NROWS; ++m) {
+          const int mat = m / NR;
+          const typename F::Row rw = F::row(codes[mat], scales[mat], global[mat], j + (m % NR), Kg);
 #pragma unroll
           for (int s = 0; s < S; ++s) {
             const int chunk = chunk0 + s * 64 + lane;
-            F::load(b.c[m][s], rw, chunk, chunk < nchunks);
+            F::load(b.c[m][s], rw, chunk < nchunks ? chunk : nchunks - 1);
           }
         }
       };
-      auto finish = [&](const UnitBuf<F, S, NMAT>& b, int t) {
-        const int j = j0 + wave + (t / nslabs) * NW;
-        const int slab = t % nslabs;
-        slab_compute<F, S, NMAT, RG>(b, xs, Kg, nchunks, slab * (S * 64), gd.n, lane, acc);
-        if (slab != nslabs - 1) return;
+      // epilogue for the units [ub, ub + nu) of the run, one unit per lane
+      auto flush = [&](int ub, int nu) {
+        if (lane < nu) {
+          const int j = (jw + ub + lane) * NR;
 #pragma unroll
-        for (int m = 0; m < NMAT; ++m)
+          for (int r = 0; r < RG; ++r) {
+            if (RG == 1 || r < gn) {
+              if (STAGE == 0) {
+                uint16_t outv[NR];
 #pragma unroll
-          for (int r = 0; r < RG; ++r)
-            if (r < gd.n) acc[m][r] = wave_sum(acc[m][r]);
+                for (int m = 0; m < NR; ++m)
+                  outv[m] = swiglu_bf16(bround(park[m][r]), bround(park[NR + m][r]), p.swiglu, p.swiglu_limit);
+                uint16_t* dst = p.h + size_t(gslot[r]) * p.h_stride + j;
 #pragma unroll
-        for (int r = 0; r < RG; ++r) {
-          if (r < gd.n && lane == r) {
-            if (STAGE == 0) {
-              const float gv = bround(acc[0][r]), uv = bround(acc[NMAT - 1][r]);
-              p.h[size_t(gd.slot[r]) * p.h_stride + j] = swiglu_bf16(gv, uv, p.swiglu, p.swiglu_limit);
-            } else if (shared) {
-              p.shared_out[size_t(gd.row[r]) * p.hidden + j] = f32_to_bf16(acc[0][r]);
-            } else {
-              const int a = gd.slot[r];
-              const float wk = p.weights_f32 ? reinterpret_cast<const float*>(p.weights)[a]
-                                             : bf16_to_f32(reinterpret_cast<const uint16_t*>(p.weights)[a]);
-              const float d = p.routed_weight == FFMOE_WEIGHT_AFTER_DOWN_BF16 ? bround(acc[0][r]) : acc[0][r];
-              p.contributions[size_t(a) * p.hidden + j] = f32_to_bf16(__fmul_rn(d, wk));
-              if (j == 0 && p.done) p.done[a] = 1u;
+                for (int m = 0; m < NR; ++m) dst[m] = outv[m];
+              } else if (shared) {
+                uint16_t* dst = p.shared_out + size_t(grow[r]) * p.hidden + j;
+                if (NR == 4) {
+                  u32x2 o = {pack_bf16x2(park[0][r], park[1][r]), pack_bf16x2(park[2 % NR][r], park[3 % NR][r])};
+                  *reinterpret_cast<u32x2*>(dst) = o;
+                } else {
+#pragma unroll
+                  for (int m = 0; m < NR; ++m) dst[m] = f32_to_bf16(park[m][r]);
+                }
+              } else {
+                const int a = gslot[r];
+                const float wk = p.weights_f32 ? reinterpret_cast<const float*>(p.weights)[a]
+                                               : bf16_to_f32(reinterpret_cast<const uint16_t*>(p.weights)[a]);
+                float v[NR];
+#pragma unroll
+                for (int m = 0; m < NR; ++m) {
+                  const float d = p.routed_weight == FFMOE_WEIGHT_AFTER_DOWN_BF16 ? bround(park[m][r]) : park[m][r];
+                  v[m] = __fmul_rn(d, wk);
+                }
+                uint16_t* dst = p.contributions + size_t(a) * p.hidden + j;
+                if (NR == 4) {
+                  u32x2 o = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2 % NR], v[3 % NR])};
+                  *reinterpret_cast<u32x2*>(dst) = o;
+                } else {
+#pragma unroll
+                  for (int m = 0; m < NR; ++m) dst[m] = f32_to_bf16(v[m]);
+                }
+                if (j == 0 && p.done) p.done[a] = 1u;
+              }
             }
           }
         }
+      };
+      auto finish = [&](const UnitBuf<F, S, NROWS>& b, int t) {
+        const int unit = t / nslabs, slab = t % nslabs;
+        slab_compute<F, S, NROWS, RG>(b, xs, Kg, nchunks, slab * (S * 64), gn, lane, acc);
+        if (slab != nslabs - 1) return;
+        const int slot_lane = unit & 63;
 #pragma unroll
-        for (int m = 0; m < NMAT; ++m)
+        for (int m = 0; m < NROWS; ++m)
 #pragma unroll
-          for (int r = 0; r < RG; ++r) acc[m][r] = 0.0f;
+          for (int r = 0; r < RG; ++r) {
+            if (RG == 1 || r < gn) {
+              const float total = wave_sum(acc[m][r]);
+              park[m][r] = lane == slot_lane ? total : park[m][r];
+            }
+            acc[m][r] = 0.0f;
+          }
+        if (slot_lane == 63) flush(unit - 63, 64);
       };
       int t = 0;
       if (t < items) issue(bufA, t);
@@ -160,6 +231,7 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
         finish(bufB, t);
         ++t;
       }
+      if (my_units & 63) flush(my_units & ~63, my_units & 63);
     }
     u0 = seg_end;
   }
@@ -238,8 +310,14 @@ int num_cus() {
   return g_cus;
 }
 
-// Steps (16-byte loads per lane and matrix) in flight per buffer; two buffers per wave.
-template <class F> struct Steps { static constexpr int value = 4; };
+// Launch shapes. S = 16-byte loads per lane and weight row in flight per buffer (two buffers per wave): a row
+// needs ceil(K / (64 * EPL)) steps; with one row of the group per pass (RG == 1) up to 8 steps go in one slab so
+// a whole row is prefetched at once, with several rows per pass the slab is capped at 4 steps to bound registers.
+// NR = output rows per unit: stage 0 streams 2*NR rows of `hidden` elements, stage 1 NR rows of `inter`.
+template <class F, int STAGE, int RG, int NR, int S>
+void launch_one(const DecodeParams& p, int blocks, size_t lds, hipStream_t st) {
+  hipLaunchKernelGGL((k_decode_stage<F, S, STAGE, RG, NR>), dim3(blocks), dim3(256), lds, st, p);
+}
 
 template <class F, int STAGE>
 int launch_stage(const DecodeParams& p, int rg, hipStream_t st) {
@@ -248,9 +326,26 @@ int launch_stage(const DecodeParams& p, int rg, hipStream_t st) {
   const int kmax = kr > ks ? kr : ks;
   const size_t lds = size_t(rg) * kmax * 2;
   const int blocks = num_cus() * 2;
-  constexpr int S = Steps<F>::value;
-  if (rg == 1) hipLaunchKernelGGL((k_decode_stage<F, S, STAGE, 1>), dim3(blocks), dim3(256), lds, st, p);
-  else hipLaunchKernelGGL((k_decode_stage<F, S, STAGE, FFMOE_DECODE_RG>), dim3(blocks), dim3(256), lds, st, p);
+  constexpr int NR = STAGE == 0 ? 1 : 4;
+  const int steps = (kmax / F::EPL + 63) / 64;
+  if (rg == 1) {
+    const int nslabs = (steps + 7) / 8;
+    const int S = (steps + nslabs - 1) / nslabs;
+    switch (S) {
+      case 1: launch_one<F, STAGE, 1, NR, 1>(p, blocks, lds, st); break;
+      case 2: launch_one<F, STAGE, 1, NR, 2>(p, blocks, lds, st); break;
+      case 3: launch_one<F, STAGE, 1, NR, 3>(p, blocks, lds, st); break;
+      case 4: launch_one<F, STAGE, 1, NR, 4>(p, blocks, lds, st); break;
+      case 5: launch_one<F, STAGE, 1, NR, 5>(p, blocks, lds, st); break;
+      case 6: launch_one<F, STAGE, 1, NR, 6>(p, blocks, lds, st); break;
+      case 7: launch_one<F, STAGE, 1, NR, 7>(p, blocks, lds, st); break;
+      default: launch_one<F, STAGE, 1, NR, 8>(p, blocks, lds, st); break;
+    }
+  } else {
+    if (steps == 1) launch_one<F, STAGE, FFMOE_DECODE_RG, NR, 1>(p, blocks, lds, st);
+    else if (steps == 2) launch_one<F, STAGE, FFMOE_DECODE_RG, NR, 2>(p, blocks, lds, st);
+    else launch_one<F, STAGE, FFMOE_DECODE_RG, NR, 4>(p, blocks, lds, st);
+  }
   return ff_launch_status();
 }
 
@@ -280,6 +375,7 @@ static int decode_impl(const ffmoe_expert_table* table, const ffmoe_shared_exper
   const int fmt = table->format;
   FF_REQUIRE(fmt == FFMOE_FMT_FP8_BLOCK128 || fmt == FFMOE_FMT_NVFP4 || fmt == FFMOE_FMT_BF16, FFMOE_ERR_UNSUPPORTED,
              "unknown expert format %d", fmt);
+  // every format's granule is a multiple of 4, the largest number of output rows a wave handles per unit
   const int gran = fmt == FFMOE_FMT_FP8_BLOCK128 ? 128 : (fmt == FFMOE_FMT_NVFP4 ? 32 : 8);
   FF_REQUIRE(H >= gran && I >= gran && H % gran == 0 && I % gran == 0, FFMOE_ERR_SHAPE,
              "hidden=%d inter=%d must be positive multiples of %d for this format", H, I, gran);

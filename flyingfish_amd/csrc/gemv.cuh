@@ -19,14 +19,17 @@ struct FmtFp8 {
     r.scales = reinterpret_cast<const float*>(scales) + size_t(j >> 7) * ((K + 127) >> 7);
     return r;
   }
-  static __device__ __forceinline__ void load(Chunk& c, const Row& r, int chunk, bool valid) {
-    const u32x4 z = {0, 0, 0, 0};
-    c.codes = valid ? load16_stream(r.codes + size_t(chunk) * 16) : z;
-    c.scale = valid ? r.scales[chunk >> 3] : 0.0f;
+  // Loads are unconditional and nothing consumes them here (the caller clamps `chunk` into the row), so no
+  // branch or wait sits between the prefetch and its use; masking happens at dequantization time.
+  // Offsets are unsigned 32-bit so the loads can take the row base from scalar registers.
+  static __device__ __forceinline__ void load(Chunk& c, const Row& r, int chunk) {
+    c.codes = load16_stream(r.codes + uint32_t(chunk) * 16u);
+    c.scale = load_global<float>(r.scales + (uint32_t(chunk) >> 3));
   }
-  static __device__ __forceinline__ void dequant(const Chunk& c, uint32_t* w) {
+  static __device__ __forceinline__ void dequant(const Chunk& c, uint32_t* w, bool valid) {
+    const float s = valid ? c.scale : 0.0f;  // masked lane: zero scale, zero weights
 #pragma unroll
-    for (int q = 0; q < 4; ++q) dequant4_e4m3(c.codes[q], c.scale, w[2 * q], w[2 * q + 1]);
+    for (int q = 0; q < 4; ++q) dequant4_e4m3(c.codes[q], s, w[2 * q], w[2 * q + 1]);
   }
 };
 
@@ -42,16 +45,16 @@ struct FmtNvfp4 {
     r.global = global;
     return r;
   }
-  static __device__ __forceinline__ void load(Chunk& c, const Row& r, int chunk, bool valid) {
-    const u32x4 z = {0, 0, 0, 0};
-    c.codes = valid ? load16_stream(r.codes + size_t(chunk) * 16) : z;
-    c.scales = valid ? uint32_t(*reinterpret_cast<const uint16_t*>(r.scales + size_t(chunk) * 2)) : 0u;
+  static __device__ __forceinline__ void load(Chunk& c, const Row& r, int chunk) {
+    c.codes = load16_stream(r.codes + uint32_t(chunk) * 16u);
+    c.scales = uint32_t(load_global<uint16_t>(r.scales + uint32_t(chunk) * 2u));
     c.global = r.global;
   }
-  static __device__ __forceinline__ void dequant(const Chunk& c, uint32_t* w) {
+  static __device__ __forceinline__ void dequant(const Chunk& c, uint32_t* w, bool valid) {
     // s = e4m3(scale) * global first, then e2m1 * s (kernels/nvfp4_linear.cu:83-98 of the reference)
     const f32x2 sc = e4m3x2_to_f32<false>(c.scales);
-    const float s0 = __fmul_rn(sc.x, c.global), s1 = __fmul_rn(sc.y, c.global);
+    const float gl = valid ? c.global : 0.0f;  // masked lane: zero scale, zero weights
+    const float s0 = __fmul_rn(sc.x, gl), s1 = __fmul_rn(sc.y, gl);
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       const float s = q < 2 ? s0 : s1;
@@ -74,44 +77,45 @@ struct FmtBf16 {
     r.codes = reinterpret_cast<const uint8_t*>(codes) + size_t(j) * K * 2;
     return r;
   }
-  static __device__ __forceinline__ void load(Chunk& c, const Row& r, int chunk, bool valid) {
-    const u32x4 z = {0, 0, 0, 0};
-    c.codes = valid ? load16_stream(r.codes + size_t(chunk) * 16) : z;
+  static __device__ __forceinline__ void load(Chunk& c, const Row& r, int chunk) {
+    c.codes = load16_stream(r.codes + uint32_t(chunk) * 16u);
   }
-  static __device__ __forceinline__ void dequant(const Chunk& c, uint32_t* w) {
+  static __device__ __forceinline__ void dequant(const Chunk& c, uint32_t* w, bool valid) {
+    const uint32_t keep = valid ? 0xffffffffu : 0u;
 #pragma unroll
-    for (int q = 0; q < 4; ++q) w[q] = c.codes[q];
+    for (int q = 0; q < 4; ++q) w[q] = c.codes[q] & keep;
   }
 };
 
-template <class F, int S, int NMAT>
-struct UnitBuf { typename F::Chunk c[NMAT][S]; };
+template <class F, int S, int NROWS>
+struct UnitBuf { typename F::Chunk c[NROWS][S]; };
 
-// One slab (S steps of 64 lane-chunks) of NMAT weight rows against the n activation rows in LDS;
-// partial sums stay in acc until the row's last slab.
-template <class F, int S, int NMAT, int RG>
-__device__ __forceinline__ void slab_compute(const UnitBuf<F, S, NMAT>& b, const uint8_t* xs, int K, int nchunks, int chunk0,
-                                             int n, int lane, float (&acc)[NMAT][RG]) {
+// One slab (S steps of 64 lane-chunks) of NROWS weight rows against the n activation rows in LDS;
+// the activation chunk is read once and used for every weight row. Partial sums stay in acc until
+// the rows' last slab. Straight-line code: chunks past the end of the row are masked per lane (zero
+// weights), never branched around, so the waits on the prefetched registers stay precise.
+template <class F, int S, int NROWS, int RG>
+__device__ __forceinline__ void slab_compute(const UnitBuf<F, S, NROWS>& b, const uint8_t* xs, int K, int nchunks, int chunk0,
+                                             int n, int lane, float (&acc)[NROWS][RG]) {
 #pragma unroll
   for (int s = 0; s < S; ++s) {
-    if (chunk0 + s * 64 < nchunks) {  // wave-uniform: steps wholly past the row do nothing
-      const int chunk = chunk0 + s * 64 + lane;
-      const int cl = chunk < nchunks ? chunk : 0;  // masked lanes carry zero weights; keep the LDS read in range
-      uint32_t w[NMAT][F::EPL / 2];
+    const int chunk = chunk0 + s * 64 + lane;
+    const bool valid = chunk < nchunks;
+    const int cl = valid ? chunk : 0;  // keep the LDS read in range
+    uint32_t w[NROWS][F::EPL / 2];
 #pragma unroll
-      for (int m = 0; m < NMAT; ++m) F::dequant(b.c[m][s], w[m]);
+    for (int m = 0; m < NROWS; ++m) F::dequant(b.c[m][s], w[m], valid);
 #pragma unroll
-      for (int r = 0; r < RG; ++r) {
-        if (r < n) {
-          const u32x4* xp = reinterpret_cast<const u32x4*>(xs + size_t(r) * K * 2 + size_t(cl) * (F::EPL * 2));
+    for (int r = 0; r < RG; ++r) {
+      if (RG == 1 || r < n) {
+        const u32x4* xp = reinterpret_cast<const u32x4*>(xs + size_t(r) * K * 2 + size_t(cl) * (F::EPL * 2));
 #pragma unroll
-          for (int v = 0; v < F::EPL / 8; ++v) {
-            const u32x4 xv = xp[v];
+        for (int v = 0; v < F::EPL / 8; ++v) {
+          const u32x4 xv = xp[v];
 #pragma unroll
-            for (int q = 0; q < 4; ++q)
+          for (int q = 0; q < 4; ++q)
 #pragma unroll
-              for (int m = 0; m < NMAT; ++m) acc[m][r] = dot2_bf16(w[m][4 * v + q], xv[q], acc[m][r]);
-          }
+            for (int m = 0; m < NROWS; ++m) acc[m][r] = dot2_bf16(w[m][4 * v + q], xv[q], acc[m][r]);
         }
       }
     }

@@ -50,7 +50,7 @@ __global__ __launch_bounds__(256) void k_linear(const LinearParams p) {
 #pragma unroll
       for (int s = 0; s < S; ++s) {
         const int chunk = chunk0 + s * 64 + lane;
-        F::load(b.c[0][s], rw, chunk, chunk < nchunks);
+        F::load(b.c[0][s], rw, chunk < nchunks ? chunk : nchunks - 1);
       }
     };
     auto finish = [&](const UnitBuf<F, S, 1>& b, int t) {

@@ -94,13 +94,7 @@ __device__ __forceinline__ Best better(Best a, Best b) {
 }
 __device__ __forceinline__ Best block_argmax(Best mine, float* s_v, int* s_id, int nwaves) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) {
-    Best o;
-    o.v = __shfl_xor(mine.v, off, 64);
-    o.id = __shfl_xor(mine.id, off, 64);
-    mine = better(mine, o);
-  }
+  wave_argmax(mine.v, mine.id);
   if (nwaves == 1) return mine;
   __syncthreads();  // previous round's readers are done with s_v/s_id
   if (lane == 0) { s_v[wave] = mine.v; s_id[wave] = mine.id; }
@@ -127,9 +121,7 @@ __global__ void k_route_topk(const uint16_t* __restrict__ logits, int* __restric
   const float logit = live ? bf16_to_f32(logits[size_t(row) * experts + e]) : -INFINITY;
   float score;
   if (score_mode == FFMOE_SCORE_SOFTMAX) {
-    float m = logit;
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
+    float m = wave_max(logit);
     if ((tid & 63) == 0) s_v[tid >> 6] = m;
     __syncthreads();
     for (int w = 0; w < nwaves; ++w) m = fmaxf(m, s_v[w]);
