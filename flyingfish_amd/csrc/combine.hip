@@ -81,21 +81,31 @@ __global__ __launch_bounds__(256) void k_combine(const uint16_t* __restrict__ co
   float acc[8];
 #pragma unroll
   for (int j = 0; j < 8; ++j) acc[j] = 0.0f;
-  for (int k = 0; k < live; ++k) {
-    const u32x4 c = load16(contributions + (size_t(a0) + s_order[k]) * hidden + d0);
+  u32x4 sh = {0, 0, 0, 0};
+  if (mode != FFMOE_COMBINE_ROUTED) sh = load16(shared_out + size_t(row) * hidden + d0);
+  for (int k0 = 0; k0 < live; k0 += 8) {
+    u32x4 c[8];
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      if (mode == FFMOE_COMBINE_BF16) {
-        acc[2 * q] = bround(__fadd_rn(acc[2 * q], bf16lo(c[q])));
-        acc[2 * q + 1] = bround(__fadd_rn(acc[2 * q + 1], bf16hi(c[q])));
-      } else {
-        acc[2 * q] = __fadd_rn(acc[2 * q], bf16lo(c[q]));
-        acc[2 * q + 1] = __fadd_rn(acc[2 * q + 1], bf16hi(c[q]));
+    for (int i = 0; i < 8; ++i) {
+      const int k = k0 + i < live ? k0 + i : live - 1;  // all eight loads go out before the first add
+      c[i] = load16(contributions + (size_t(a0) + s_order[k]) * hidden + d0);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      if (k0 + i < live) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          if (mode == FFMOE_COMBINE_BF16) {
+            acc[2 * q] = bround(__fadd_rn(acc[2 * q], bf16lo(c[i][q])));
+            acc[2 * q + 1] = bround(__fadd_rn(acc[2 * q + 1], bf16hi(c[i][q])));
+          } else {
+            acc[2 * q] = __fadd_rn(acc[2 * q], bf16lo(c[i][q]));
+            acc[2 * q + 1] = __fadd_rn(acc[2 * q + 1], bf16hi(c[i][q]));
+          }
+        }
       }
     }
   }
-  u32x4 sh = {0, 0, 0, 0};
-  if (mode != FFMOE_COMBINE_ROUTED) sh = load16(shared_out + size_t(row) * hidden + d0);
   u32x4 out;
 #pragma unroll
   for (int q = 0; q < 4; ++q) {

@@ -1,241 +1,16 @@
-// Decode expert FFN: weight-streaming grouped GEMV kernels for FP8-block, NVFP4 and BF16 experts.
-//
-// Work model. Assignments (row, choice) that hit the same expert are gathered into groups of at most
-// RG rows, so one pass over an expert's weights serves all of them. A "unit" is one output row of
-// one group (one gate row + one up row, or one down row). The unit space is split evenly over a
-// fixed grid; every block walks a contiguous unit range, so each wave streams whole weight rows
-// with 16-byte loads per lane (a wave covers 1 KiB of a row per load instruction), dequantizes in
-// registers and keeps one FP32 accumulator per (row-of-group, matrix), reduced across the wave at
-// the end of the unit. Activations of the group live in LDS. The loads of the next unit are issued
-// before the arithmetic of the current one, so every wave always has a full weight row in flight.
-//
-// Arithmetic (FFMOE_ACT_BF16): effective weight = bf16(decode(code) * scale) as in the reference's
-// CPU path (src/fp8.rs:138-145), FP32 accumulation, BF16 boundaries at gate, up, SiLU, product,
-// down and weighted contribution (src/cpu/expert_ffn.rs:592-679; kernels/moe_ffn.cu:198-209,293-301).
-#include "gemv.cuh"
+// Decode expert contribution: entry points, argument checks and the kernel that groups assignments by expert.
+// The streaming kernels live in decode_kernel.cuh and are instantiated per weight format.
+#include "common.cuh"
 #include "api.h"
 #include "decode.h"
 
 namespace ffmoe {
+int decode_launch_fp8(const DecodeParams& p, int rg, int stage_mask, hipStream_t st);
+int decode_launch_nvfp4(const DecodeParams& p, int rg, int stage_mask, hipStream_t st);
+int decode_launch_bf16(const DecodeParams& p, int rg, int stage_mask, hipStream_t st);
+}  // namespace ffmoe
 
-// ---------------------------------------------------------------------------------------------
-// group descriptors
-__device__ __forceinline__ void make_group(GroupDesc& gd, const DecodeParams& p, int g) {
-  if (p.groups) { gd = p.groups[g]; return; }
-  // ungrouped: one group per assignment, then one per shared row
-  const int A = p.rows * p.top_k;
-  gd.n = 1;
-  if (g < A) {
-    gd.expert = p.ids[g];
-    gd.row[0] = g / p.top_k;
-    gd.slot[0] = g;
-    if (p.active && p.active[g] == 0u) gd.n = 0;
-    if (p.valid && (unsigned)gd.expert < (unsigned)p.experts && p.valid[gd.expert] == 0u) gd.n = 0;
-    if ((unsigned)gd.expert >= (unsigned)p.experts) gd.n = 0;  // out-of-range id: contribute nothing, done stays 0
-  } else {
-    gd.expert = -1;
-    gd.row[0] = g - A;
-    gd.slot[0] = g;
-  }
-}
-
-__device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
-
-// STAGE 0: gate/up + SwiGLU -> h[slot, j].   STAGE 1: down (+ routing weight) -> contributions / shared_out.
-// A unit is NR consecutive output rows of one group: stage 0 streams NR gate rows and the NR matching up rows
-// (2*NR weight rows sharing every activation read), stage 1 streams NR down rows.
-//
-// Every quantity that decides an address (group, expert, row index, slab) is held wave-uniform in scalar
-// registers, so weight loads take a scalar base plus one per-lane offset. A wave owns a contiguous run of
-// units of the segment; reduced sums of up to 64 units are parked one per lane and the epilogue (SwiGLU or
-// weighting, BF16 rounding, store) runs once per 64 units with coalesced stores.
-template <class F, int S, int STAGE, int RG, int NR>
-__global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
-  constexpr int NROWS = STAGE == 0 ? 2 * NR : NR;
-  constexpr int NW = 4;
-  extern __shared__ __align__(16) uint8_t xs[];
-  __shared__ GroupDesc s_gd;
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = uni(tid >> 6);
-  const int A = p.rows * p.top_k;
-  const int n_routed = p.counters ? p.counters[0] : A;
-  const int n_shared = p.counters ? p.counters[1] : (p.has_shared ? p.rows : 0);
-  // units per group
-  const int out_r = (STAGE == 0 ? p.inter : p.hidden) / NR;
-  const int out_s = (STAGE == 0 ? p.shared_inter : p.hidden) / NR;
-  const long long routed_units = (long long)n_routed * out_r;
-  const long long total = routed_units + (long long)n_shared * out_s;
-  const long long lo = total * blockIdx.x / gridDim.x, hi = total * (blockIdx.x + 1) / gridDim.x;
-  long long u0 = lo;
-  while (u0 < hi) {
-    // group segment containing u0
-    int g, j0, width;
-    if (u0 < routed_units) { g = int(u0 / out_r); j0 = int(u0 % out_r); width = out_r; }
-    else { const long long v = u0 - routed_units; g = n_routed + int(v / out_s); j0 = int(v % out_s); width = out_s; }
-    const long long seg_end = u0 + (width - j0) < hi ? u0 + (width - j0) : hi;
-    const int count = int(seg_end - u0);
-    __syncthreads();  // previous segment's readers are done with xs and s_gd
-    if (tid == 0) make_group(s_gd, p, g);
-    __syncthreads();
-    const int expert = uni(s_gd.expert);
-    const int gn = uni(s_gd.n);
-    int grow[RG], gslot[RG];
-#pragma unroll
-    for (int r = 0; r < RG; ++r) { grow[r] = uni(s_gd.row[r]); gslot[r] = uni(s_gd.slot[r]); }
-    const bool shared = expert < 0;
-    const int Kg = STAGE == 0 ? p.hidden : (shared ? p.shared_inter : p.inter);
-    if (gn > 0) {
-      // activations of the group -> LDS (row r at r*Kg*2)
-      const uint16_t* src = STAGE == 0 ? p.x : p.h;
-      const int row_words = Kg >> 3;  // 16-byte words per row
-#pragma unroll
-      for (int r = 0; r < RG; ++r) {
-        if (r < gn) {
-          const size_t base = STAGE == 0 ? size_t(grow[r]) * p.hidden : size_t(gslot[r]) * p.h_stride;
-          u32x4* d4 = reinterpret_cast<u32x4*>(xs + size_t(r) * Kg * 2);
-          for (int v = tid; v < row_words; v += 256) d4[v] = load16(src + base + size_t(v) * 8);
-        }
-      }
-    }
-    __syncthreads();
-    if (gn > 0) {
-      // weight row m of a unit comes from matrix m / NR (stage 0: gate, up; stage 1: down). The six addresses are
-      // fetched through scalar-friendly paths (kernel argument or global table), never through a generic pointer.
-      uint64_t sl[6];
-      float gl3[3];
-      if (shared) {
-#pragma unroll
-        for (int i = 0; i < 6; ++i) sl[i] = p.shared_slot[i];
-#pragma unroll
-        for (int i = 0; i < 3; ++i) gl3[i] = p.shared_global[i];
-      } else {
-#pragma unroll
-        for (int i = 0; i < 6; ++i) sl[i] = load_global<uint64_t>(p.slots + size_t(expert) * 6 + i);
-#pragma unroll
-        for (int i = 0; i < 3; ++i) gl3[i] = p.global_scales ? load_global<float>(p.global_scales + size_t(expert) * 3 + i) : 1.0f;
-      }
-      uint64_t codes[2], scales[2];
-      float global[2];
-      if (STAGE == 0) {
-        codes[0] = sl[0]; scales[0] = sl[1]; global[0] = gl3[0];
-        codes[1] = sl[2]; scales[1] = sl[3]; global[1] = gl3[1];
-      } else {
-        codes[0] = codes[1] = sl[4]; scales[0] = scales[1] = sl[5]; global[0] = global[1] = gl3[2];
-      }
-#pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        codes[i] = (uint64_t(uint32_t(uni(int(codes[i] >> 32)))) << 32) | uint32_t(uni(int(codes[i])));
-        scales[i] = (uint64_t(uint32_t(uni(int(scales[i] >> 32)))) << 32) | uint32_t(uni(int(scales[i])));
-        global[i] = __builtin_bit_cast(float, uni(__builtin_bit_cast(int, global[i])));
-      }
-      const int nchunks = Kg / F::EPL;
-      const int nslabs = (nchunks + S * 64 - 1) / (S * 64);
-      // this wave's contiguous run of units inside the segment
-      const int w_lo = count * wave / NW, w_hi = count * (wave + 1) / NW;
-      const int my_units = w_hi - w_lo;
-      const int items = my_units * nslabs;
-      const int jw = j0 + w_lo;  // first unit of the run
-      UnitBuf<F, S, NROWS> bufA, bufB;
-      float acc[NROWS][RG];
-      float park[NROWS][RG];  // lane L keeps the sums of unit (batch base + L)
-#pragma unroll
-      for (int m = 0; m < NROWS; ++m)
-#pragma unroll
-        for (int r = 0; r < RG; ++r) { acc[m][r] = 0.0f; park[m][r] = 0.0f; }
-      auto issue = [&](UnitBuf<F, S, NROWS>& b, int t) {
-        const int j = (jw + t / nslabs) * NR;  // first output row of the unit
-        const int chunk0 = (t % nslabs) * (S * 64);
-#pragma unroll
-        for (int m = 0; m < NROWS; ++m) {
-          const int mat = m / NR;
-          const typename F::Row rw = F::row(codes[mat], scales[mat], global[mat], j + (m % NR), Kg);
-#pragma unroll
-          for (int s = 0; s < S; ++s) {
-            const int chunk = chunk0 + s * 64 + lane;
-            F::load(b.c[m][s], rw, chunk < nchunks ? chunk : nchunks - 1);
-          }
-        }
-      };
-      // epilogue for the units [ub, ub + nu) of the run, one unit per lane
-      auto flush = [&](int ub, int nu) {
-        if (lane < nu) {
-          const int j = (jw + ub + lane) * NR;
-#pragma unroll
-          for (int r = 0; r < RG; ++r) {
-            if (RG == 1 || r < gn) {
-              if (STAGE == 0) {
-                uint16_t outv[NR];
-#pragma unroll
-                for (int m = 0; m < NR; ++m)
-                  outv[m] = swiglu_bf16(bround(park[m][r]), bround(park[NR + m][r]), p.swiglu, p.swiglu_limit);
-                uint16_t* dst = p.h + size_t(gslot[r]) * p.h_stride + j;
-#pragma unroll
-                for (int m = 0; m < NR; ++m) dst[m] = outv[m];
-              } else if (shared) {
-                uint16_t* dst = p.shared_out + size_t(grow[r]) * p.hidden + j;
-                if (NR == 4) {
-                  u32x2 o = {pack_bf16x2(park[0][r], park[1][r]), pack_bf16x2(park[2 % NR][r], park[3 % NR][r])};
-                  *reinterpret_cast<u32x2*>(dst) = o;
-                } else {
-#pragma unroll
-                  for (int m = 0; m < NR; ++m) dst[m] = f32_to_bf16(park[m][r]);
-                }
-              } else {
-                const int a = gslot[r];
-                const float wk = p.weights_f32 ? reinterpret_cast<const float*>(p.weights)[a]
-                                               : bf16_to_f32(reinterpret_cast<const uint16_t*>(p.weights)[a]);
-                float v[NR];
-#pragma unroll
-                for (int m = 0; m < NR; ++m) {
-                  const float d = p.routed_weight == FFMOE_WEIGHT_AFTER_DOWN_BF16 ? bround(park[m][r]) : park[m][r];
-                  v[m] = __fmul_rn(d, wk);
-                }
-                uint16_t* dst = p.contributions + size_t(a) * p.hidden + j;
-                if (NR == 4) {
-                  u32x2 o = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2 % NR], v[3 % NR])};
-                  *reinterpret_cast<u32x2*>(dst) = o;
-                } else {
-#pragma unroll
-                  for (int m = 0; m < NR; ++m) dst[m] = f32_to_bf16(v[m]);
-                }
-                if (j == 0 && p.done) p.done[a] = 1u;
-              }
-            }
-          }
-        }
-      };
-      auto finish = [&](const UnitBuf<F, S, NROWS>& b, int t) {
-        const int unit = t / nslabs, slab = t % nslabs;
-        slab_compute<F, S, NROWS, RG>(b, xs, Kg, nchunks, slab * (S * 64), gn, lane, acc);
-        if (slab != nslabs - 1) return;
-        const int slot_lane = unit & 63;
-#pragma unroll
-        for (int m = 0; m < NROWS; ++m)
-#pragma unroll
-          for (int r = 0; r < RG; ++r) {
-            if (RG == 1 || r < gn) {
-              const float total = wave_sum(acc[m][r]);
-              park[m][r] = lane == slot_lane ? total : park[m][r];
-            }
-            acc[m][r] = 0.0f;
-          }
-        if (slot_lane == 63) flush(unit - 63, 64);
-      };
-      int t = 0;
-      if (t < items) issue(bufA, t);
-      while (t < items) {
-        if (t + 1 < items) issue(bufB, t + 1);
-        finish(bufA, t);
-        if (++t >= items) break;
-        if (t + 1 < items) issue(bufA, t + 1);
-        finish(bufB, t);
-        ++t;
-      }
-      if (my_units & 63) flush(my_units & ~63, my_units & 63);
-    }
-    u0 = seg_end;
-  }
-}
+namespace ffmoe {
 
 // ---------------------------------------------------------------------------------------------
 // Gather assignments by expert into groups of at most RGMAX rows (single block; A <= FFMOE_DECODE_MAX_ASSIGN).
@@ -296,60 +71,6 @@ __global__ __launch_bounds__(1024) void k_group_assignments(const int* __restric
 
 using namespace ffmoe;
 
-namespace {
-
-int g_cus = 0;
-int num_cus() {
-  if (g_cus == 0) {
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
-      g_cus = n;
-    else
-      g_cus = 256;
-  }
-  return g_cus;
-}
-
-// Launch shapes. S = 16-byte loads per lane and weight row in flight per buffer (two buffers per wave): a row
-// needs ceil(K / (64 * EPL)) steps; with one row of the group per pass (RG == 1) up to 8 steps go in one slab so
-// a whole row is prefetched at once, with several rows per pass the slab is capped at 4 steps to bound registers.
-// NR = output rows per unit: stage 0 streams 2*NR rows of `hidden` elements, stage 1 NR rows of `inter`.
-template <class F, int STAGE, int RG, int NR, int S>
-void launch_one(const DecodeParams& p, int blocks, size_t lds, hipStream_t st) {
-  hipLaunchKernelGGL((k_decode_stage<F, S, STAGE, RG, NR>), dim3(blocks), dim3(256), lds, st, p);
-}
-
-template <class F, int STAGE>
-int launch_stage(const DecodeParams& p, int rg, hipStream_t st) {
-  const int kr = STAGE == 0 ? p.hidden : p.inter;
-  const int ks = STAGE == 0 ? p.hidden : (p.has_shared ? p.shared_inter : p.inter);
-  const int kmax = kr > ks ? kr : ks;
-  const size_t lds = size_t(rg) * kmax * 2;
-  const int blocks = num_cus() * 2;
-  constexpr int NR = STAGE == 0 ? 1 : 4;
-  const int steps = (kmax / F::EPL + 63) / 64;
-  if (rg == 1) {
-    const int nslabs = (steps + 7) / 8;
-    const int S = (steps + nslabs - 1) / nslabs;
-    switch (S) {
-      case 1: launch_one<F, STAGE, 1, NR, 1>(p, blocks, lds, st); break;
-      case 2: launch_one<F, STAGE, 1, NR, 2>(p, blocks, lds, st); break;
-      case 3: launch_one<F, STAGE, 1, NR, 3>(p, blocks, lds, st); break;
-      case 4: launch_one<F, STAGE, 1, NR, 4>(p, blocks, lds, st); break;
-      case 5: launch_one<F, STAGE, 1, NR, 5>(p, blocks, lds, st); break;
-      case 6: launch_one<F, STAGE, 1, NR, 6>(p, blocks, lds, st); break;
-      case 7: launch_one<F, STAGE, 1, NR, 7>(p, blocks, lds, st); break;
-      default: launch_one<F, STAGE, 1, NR, 8>(p, blocks, lds, st); break;
-    }
-  } else {
-    if (steps == 1) launch_one<F, STAGE, FFMOE_DECODE_RG, NR, 1>(p, blocks, lds, st);
-    else if (steps == 2) launch_one<F, STAGE, FFMOE_DECODE_RG, NR, 2>(p, blocks, lds, st);
-    else launch_one<F, STAGE, FFMOE_DECODE_RG, NR, 4>(p, blocks, lds, st);
-  }
-  return ff_launch_status();
-}
-
-}  // namespace
 
 extern "C" __attribute__((visibility("default"))) uint64_t ffmoe_decode_scratch_bytes(int rows, int top_k, int experts, int hidden, int inter, int shared_inter) {
   (void)hidden;
@@ -459,20 +180,10 @@ static int decode_impl(const ffmoe_expert_table* table, const ffmoe_shared_exper
     p.counters = nullptr;
   }
   switch (fmt) {
-    case FFMOE_FMT_FP8_BLOCK128:
-      if (stage_mask & 1) FF_TRY((launch_stage<FmtFp8, 0>(p, rg, st)));
-      if (stage_mask & 2) FF_TRY((launch_stage<FmtFp8, 1>(p, rg, st)));
-      break;
-    case FFMOE_FMT_NVFP4:
-      if (stage_mask & 1) FF_TRY((launch_stage<FmtNvfp4, 0>(p, rg, st)));
-      if (stage_mask & 2) FF_TRY((launch_stage<FmtNvfp4, 1>(p, rg, st)));
-      break;
-    default:
-      if (stage_mask & 1) FF_TRY((launch_stage<FmtBf16, 0>(p, rg, st)));
-      if (stage_mask & 2) FF_TRY((launch_stage<FmtBf16, 1>(p, rg, st)));
-      break;
+    case FFMOE_FMT_FP8_BLOCK128: return decode_launch_fp8(p, rg, stage_mask, st);
+    case FFMOE_FMT_NVFP4: return decode_launch_nvfp4(p, rg, stage_mask, st);
+    default: return decode_launch_bf16(p, rg, stage_mask, st);
   }
-  return 0;
 }
 
 extern "C" __attribute__((visibility("default"))) int ffmoe_decode_contribute(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared,

@@ -1,0 +1,306 @@
+// Decode expert FFN kernel (both stages) and its launch policy, instantiated once per weight format in
+// decode_fp8.hip / decode_nvfp4.hip / decode_bf16.hip.
+//
+// Work model. Assignments (row, choice) that hit the same expert are gathered into groups of at most RG rows, so
+// one pass over an expert's weights serves all of them. A "unit" is NR consecutive output rows of one group. The
+// unit space is split evenly over a fixed grid; every block walks a contiguous unit range, so each wave streams
+// whole weight rows with 16-byte loads per lane (a wave covers 1 KiB of a row per load instruction), dequantizes
+// in registers and keeps one FP32 accumulator per (row-of-group, weight row), reduced across the wave at the end
+// of the unit. Activations of the group live in LDS.
+//
+// Arithmetic (FFMOE_ACT_BF16): effective weight = bf16(decode(code) * scale) as in the reference's CPU path
+// (src/fp8.rs:138-145), FP32 accumulation, BF16 boundaries at gate, up, SiLU, product, down and weighted
+// contribution (src/cpu/expert_ffn.rs:592-679; kernels/moe_ffn.cu:198-209,293-301).
+#pragma once
+#include "gemv.cuh"
+#include "api.h"
+#include "decode.h"
+
+namespace ffmoe {
+
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
+__device__ __forceinline__ float unif(float v) { return __builtin_bit_cast(float, uni(__builtin_bit_cast(int, v))); }
+__device__ __forceinline__ uint64_t uni64(uint64_t v) {
+  return (uint64_t(uint32_t(uni(int(v >> 32)))) << 32) | uint32_t(uni(int(uint32_t(v))));
+}
+
+// Group g as wave-uniform scalars. Without a descriptor table (one row per call) every assignment is its own
+// group and the shared expert follows the routed ones.
+template <int RG>
+__device__ __forceinline__ void load_group(const DecodeParams& p, int g, int& expert, int& n, int (&row)[RG], int (&slot)[RG]) {
+  if (p.groups) {
+    const int* gd = reinterpret_cast<const int*>(p.groups + g);
+    expert = uni(load_global<int>(gd));
+    n = uni(load_global<int>(gd + 1));
+#pragma unroll
+    for (int r = 0; r < RG; ++r) {
+      row[r] = uni(load_global<int>(gd + 2 + r));
+      slot[r] = uni(load_global<int>(gd + 2 + FFMOE_DECODE_RG + r));
+    }
+    return;
+  }
+  const int A = p.rows * p.top_k;
+#pragma unroll
+  for (int r = 0; r < RG; ++r) { row[r] = 0; slot[r] = 0; }
+  n = 1;
+  if (g < A) {
+    expert = uni(load_global<int>(p.ids + g));
+    row[0] = g / p.top_k;
+    slot[0] = g;
+    if (p.active && uni(int(load_global<uint32_t>(p.active + g))) == 0) n = 0;
+    if ((unsigned)expert >= (unsigned)p.experts) n = 0;  // out-of-range id: contribute nothing, done stays 0
+    else if (p.valid && uni(int(load_global<uint32_t>(p.valid + expert))) == 0) n = 0;
+  } else {
+    expert = -1;
+    row[0] = g - A;
+    slot[0] = g;
+  }
+}
+
+// STAGE 0: gate/up + SwiGLU -> h[slot, j].   STAGE 1: down (+ routing weight) -> contributions / shared_out.
+// A unit is NR consecutive output rows of one group: stage 0 streams NR gate rows and the NR matching up rows
+// (2*NR weight rows sharing every activation read), stage 1 streams NR down rows.
+//
+// Every quantity that decides an address (group, expert, row index, slab) is wave-uniform and lives in scalar
+// registers, so a weight load is a scalar base plus one per-lane offset. A wave owns a contiguous run of units
+// of the segment and keeps ONE register buffer of S steps per weight row: as soon as step s of the current item
+// has been consumed, step s of the next item is requested into the same registers, so a full row per weight
+// matrix is in flight at all times and the first requests of a segment go out before the activations are even
+// staged. Reduced sums of up to 64 units are parked one per lane; the epilogue (SwiGLU or weighting, BF16
+// rounding, store) runs once per 64 units with coalesced stores.
+template <class F, int S, int STAGE, int RG, int NR>
+__global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
+  constexpr int NROWS = STAGE == 0 ? 2 * NR : NR;
+  constexpr int NW = 4;
+  extern __shared__ __align__(16) uint8_t xs[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = uni(tid >> 6);
+  const int A = p.rows * p.top_k;
+  const int n_routed = p.counters ? uni(load_global<int>(p.counters)) : A;
+  const int n_shared = p.counters ? uni(load_global<int>(p.counters + 1)) : (p.has_shared ? p.rows : 0);
+  // units per group
+  const int out_r = (STAGE == 0 ? p.inter : p.hidden) / NR;
+  const int out_s = (STAGE == 0 ? p.shared_inter : p.hidden) / NR;
+  const long long routed_units = (long long)n_routed * out_r;
+  const long long total = routed_units + (long long)n_shared * out_s;
+  const long long lo = total * blockIdx.x / gridDim.x, hi = total * (blockIdx.x + 1) / gridDim.x;
+  long long u0 = lo;
+  while (u0 < hi) {
+    // group segment containing u0
+    int g, j0, width;
+    if (u0 < routed_units) { g = int(u0 / out_r); j0 = int(u0 % out_r); width = out_r; }
+    else { const long long v = u0 - routed_units; g = n_routed + int(v / out_s); j0 = int(v % out_s); width = out_s; }
+    const long long seg_end = u0 + (width - j0) < hi ? u0 + (width - j0) : hi;
+    const int count = int(seg_end - u0);
+    int expert, gn, grow[RG], gslot[RG];
+    load_group<RG>(p, g, expert, gn, grow, gslot);
+    const bool shared = expert < 0;
+    const int Kg = STAGE == 0 ? p.hidden : (shared ? p.shared_inter : p.inter);
+    // the six slot addresses through scalar-friendly paths (kernel argument or global table), never a generic pointer
+    uint64_t sl[6] = {0, 0, 0, 0, 0, 0};
+    float gl3[3] = {1.0f, 1.0f, 1.0f};
+    if (gn > 0) {
+      if (shared) {
+#pragma unroll
+        for (int i = 0; i < 6; ++i) sl[i] = p.shared_slot[i];
+#pragma unroll
+        for (int i = 0; i < 3; ++i) gl3[i] = p.shared_global[i];
+      } else {
+#pragma unroll
+        for (int i = 0; i < 6; ++i) sl[i] = uni64(load_global<uint64_t>(p.slots + size_t(expert) * 6 + i));
+        if (p.global_scales) {
+#pragma unroll
+          for (int i = 0; i < 3; ++i) gl3[i] = unif(load_global<float>(p.global_scales + size_t(expert) * 3 + i));
+        }
+      }
+    }
+    // weight row m of a unit comes from matrix m / NR (stage 0: gate, up; stage 1: down)
+    uint64_t codes[2], scales[2];
+    float global[2];
+    if (STAGE == 0) {
+      codes[0] = sl[0]; scales[0] = sl[1]; global[0] = gl3[0];
+      codes[1] = sl[2]; scales[1] = sl[3]; global[1] = gl3[1];
+    } else {
+      codes[0] = codes[1] = sl[4]; scales[0] = scales[1] = sl[5]; global[0] = global[1] = gl3[2];
+    }
+    // routing weights of the group's rows (stage 1), fetched up front so the epilogue never waits on them
+    float wk[RG];
+#pragma unroll
+    for (int r = 0; r < RG; ++r) {
+      wk[r] = 1.0f;
+      if (STAGE == 1 && !shared && r < gn) {
+        wk[r] = p.weights_f32 ? unif(load_global<float>(reinterpret_cast<const float*>(p.weights) + gslot[r]))
+                              : bf16_to_f32(uint16_t(uni(int(load_global<uint16_t>(reinterpret_cast<const uint16_t*>(p.weights) + gslot[r])))));
+      }
+    }
+    const int nchunks = Kg / F::EPL;
+    const int nslabs = (nchunks + S * 64 - 1) / (S * 64);
+    // this wave's contiguous run of units inside the segment
+    const int w_lo = count * wave / NW, w_hi = count * (wave + 1) / NW;
+    const int my_units = gn > 0 ? w_hi - w_lo : 0;
+    const int items = my_units * nslabs;
+    const int jw = j0 + w_lo;  // first unit of the run
+    typename F::Chunk buf[NROWS][S];
+    auto issue_step = [&](int t, int s) {
+      const int j = (jw + t / nslabs) * NR;  // first output row of the unit
+      const int chunk = (t % nslabs) * (S * 64) + s * 64 + lane;
+      const int cc = chunk < nchunks ? chunk : nchunks - 1;
+#pragma unroll
+      for (int m = 0; m < NROWS; ++m) {
+        const int mat = m / NR;
+        F::load(buf[m][s], F::row(codes[mat], scales[mat], global[mat], j + (m % NR), Kg), cc);
+      }
+    };
+    if (items > 0) {
+#pragma unroll
+      for (int s = 0; s < S; ++s) issue_step(0, s);
+    }
+    // activations of the group -> LDS (row r at r*Kg*2), behind the first weight requests
+    __syncthreads();  // the previous segment's readers are done with xs
+    if (gn > 0) {
+      const uint16_t* src = STAGE == 0 ? p.x : p.h;
+      const int row_words = Kg >> 3;  // 16-byte words per row
+#pragma unroll
+      for (int r = 0; r < RG; ++r) {
+        if (r < gn) {
+          const size_t base = STAGE == 0 ? size_t(grow[r]) * p.hidden : size_t(gslot[r]) * p.h_stride;
+          u32x4* d4 = reinterpret_cast<u32x4*>(xs + size_t(r) * Kg * 2);
+          for (int v = tid; v < row_words; v += 256) d4[v] = load16(src + base + size_t(v) * 8);
+        }
+      }
+    }
+    __syncthreads();
+    if (items > 0) {
+      float acc[NROWS][RG];
+      float park[NROWS][RG];  // lane L keeps the sums of unit (batch base + L)
+#pragma unroll
+      for (int m = 0; m < NROWS; ++m)
+#pragma unroll
+        for (int r = 0; r < RG; ++r) { acc[m][r] = 0.0f; park[m][r] = 0.0f; }
+      // epilogue for the units [ub, ub + nu) of the run, one unit per lane
+      auto flush = [&](int ub, int nu) {
+        if (lane < nu) {
+          const int j = (jw + ub + lane) * NR;
+#pragma unroll
+          for (int r = 0; r < RG; ++r) {
+            if (RG == 1 || r < gn) {
+              if (STAGE == 0) {
+                uint16_t* dst = p.h + size_t(gslot[r]) * p.h_stride + j;
+#pragma unroll
+                for (int m = 0; m < NR; ++m)
+                  dst[m] = swiglu_bf16(bround(park[m][r]), bround(park[NR + m][r]), p.swiglu, p.swiglu_limit);
+              } else {
+                float v[NR];
+#pragma unroll
+                for (int m = 0; m < NR; ++m) {
+                  if (shared) v[m] = park[m][r];
+                  else v[m] = __fmul_rn(p.routed_weight == FFMOE_WEIGHT_AFTER_DOWN_BF16 ? bround(park[m][r]) : park[m][r], wk[r]);
+                }
+                uint16_t* dst = shared ? p.shared_out + size_t(grow[r]) * p.hidden + j : p.contributions + size_t(gslot[r]) * p.hidden + j;
+                if (NR == 4) {
+                  u32x2 o = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2 % NR], v[3 % NR])};
+                  *reinterpret_cast<u32x2*>(dst) = o;
+                } else {
+#pragma unroll
+                  for (int m = 0; m < NR; ++m) dst[m] = f32_to_bf16(v[m]);
+                }
+                if (!shared && j == 0 && p.done) p.done[gslot[r]] = 1u;
+              }
+            }
+          }
+        }
+      };
+      auto compute_step = [&](int t, int s) {
+        const int chunk = (t % nslabs) * (S * 64) + s * 64 + lane;
+        step_compute<F, NROWS, RG, S>(buf, s, xs, Kg, nchunks, chunk, gn, acc);
+      };
+      auto item_end = [&](int t) {
+        const int unit = t / nslabs;
+        if (t % nslabs != nslabs - 1) return;
+        const int slot_lane = unit & 63;
+#pragma unroll
+        for (int m = 0; m < NROWS; ++m)
+#pragma unroll
+          for (int r = 0; r < RG; ++r) {
+            if (RG == 1 || r < gn) {
+              const float total = wave_sum(acc[m][r]);
+              park[m][r] = lane == slot_lane ? total : park[m][r];
+            }
+            acc[m][r] = 0.0f;
+          }
+        if (slot_lane == 63) flush(unit - 63, 64);
+      };
+      for (int t = 0; t + 1 < items; ++t) {
+#pragma unroll
+        for (int s = 0; s < S; ++s) {
+          compute_step(t, s);
+          issue_step(t + 1, s);
+        }
+        item_end(t);
+      }
+#pragma unroll
+      for (int s = 0; s < S; ++s) compute_step(items - 1, s);
+      item_end(items - 1);
+      if (my_units & 63) flush(my_units & ~63, my_units & 63);
+    }
+    u0 = seg_end;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Launch policy. A weight row needs steps = ceil(K / (64 * EPL)) 16-byte loads per lane. S of them are kept in
+// flight per weight row (one slab); rows longer than the format's cap take several slabs. The caps keep every
+// instantiation inside the register file without spills: stage 0 holds 2 weight rows per unit, stage 1 holds
+// Policy::NR1 rows; with several rows of a group per pass (RG > 1) the cap is halved.
+template <class F> struct Policy { static constexpr int S0 = 8, S0G = 4, NR1 = 4, S1 = 2, S1G = 2; };
+template <> struct Policy<FmtNvfp4> { static constexpr int S0 = 2, S0G = 2, NR1 = 2, S1 = 2, S1G = 1; };
+
+inline int decode_num_cus() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+      cus = n;
+    else
+      cus = 256;
+  }
+  return cus;
+}
+
+template <class F, int STAGE, int RG, int NR, int SMAX, int S = 1>
+void launch_steps(int want, const DecodeParams& p, int blocks, size_t lds, hipStream_t st) {
+  if constexpr (S <= SMAX) {
+    if (want == S) hipLaunchKernelGGL((k_decode_stage<F, S, STAGE, RG, NR>), dim3(blocks), dim3(256), lds, st, p);
+    else launch_steps<F, STAGE, RG, NR, SMAX, S + 1>(want, p, blocks, lds, st);
+  }
+}
+
+template <class F, int STAGE>
+int launch_stage(const DecodeParams& p, int rg, hipStream_t st) {
+  const int kr = STAGE == 0 ? p.hidden : p.inter;
+  const int ks = STAGE == 0 ? p.hidden : (p.has_shared ? p.shared_inter : p.inter);
+  const int kmax = kr > ks ? kr : ks;
+  const size_t lds = size_t(rg) * kmax * 2;
+  // blocks per CU: two for the long rows of the gate/up stage, three for the shorter down rows
+  const int blocks = decode_num_cus() * (STAGE == 0 ? 2 : 3);
+  constexpr int NR = STAGE == 0 ? 1 : Policy<F>::NR1;
+  constexpr int SMAX1 = STAGE == 0 ? Policy<F>::S0 : Policy<F>::S1;
+  constexpr int SMAXG = STAGE == 0 ? Policy<F>::S0G : Policy<F>::S1G;
+  const int steps = (kmax / F::EPL + 63) / 64;
+  const int smax = rg == 1 ? SMAX1 : SMAXG;
+  const int nslabs = (steps + smax - 1) / smax;
+  const int S = (steps + nslabs - 1) / nslabs;
+  if (rg == 1) launch_steps<F, STAGE, 1, NR, SMAX1>(S, p, blocks, lds, st);
+  else launch_steps<F, STAGE, FFMOE_DECODE_RG, NR, SMAXG>(S, p, blocks, lds, st);
+  return ff_launch_status();
+}
+
+template <class F>
+int launch_format(const DecodeParams& p, int rg, int stage_mask, hipStream_t st) {
+  if (stage_mask & 1) FF_TRY((launch_stage<F, 0>(p, rg, st)));
+  if (stage_mask & 2) FF_TRY((launch_stage<F, 1>(p, rg, st)));
+  return 0;
+}
+
+}  // namespace ffmoe

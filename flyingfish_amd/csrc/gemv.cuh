@@ -87,36 +87,28 @@ struct FmtBf16 {
   }
 };
 
-template <class F, int S, int NROWS>
-struct UnitBuf { typename F::Chunk c[NROWS][S]; };
-
-// One slab (S steps of 64 lane-chunks) of NROWS weight rows against the n activation rows in LDS;
-// the activation chunk is read once and used for every weight row. Partial sums stay in acc until
-// the rows' last slab. Straight-line code: chunks past the end of the row are masked per lane (zero
-// weights), never branched around, so the waits on the prefetched registers stay precise.
-template <class F, int S, int NROWS, int RG>
-__device__ __forceinline__ void slab_compute(const UnitBuf<F, S, NROWS>& b, const uint8_t* xs, int K, int nchunks, int chunk0,
-                                             int n, int lane, float (&acc)[NROWS][RG]) {
+// One step: this lane's 16-byte chunk of NROWS weight rows against the n activation rows in LDS. The activation
+// chunk is read once and used for every weight row. Straight-line code: a chunk past the end of the row is
+// masked (zero weights), never branched around, so the waits on the prefetched registers stay precise.
+template <class F, int NROWS, int RG, int S>
+__device__ __forceinline__ void step_compute(const typename F::Chunk (&c)[NROWS][S], int s, const uint8_t* xs, int K, int nchunks,
+                                             int chunk, int n, float (&acc)[NROWS][RG]) {
+  const bool valid = chunk < nchunks;
+  const int cl = valid ? chunk : 0;  // keep the LDS read in range
+  uint32_t w[NROWS][F::EPL / 2];
 #pragma unroll
-  for (int s = 0; s < S; ++s) {
-    const int chunk = chunk0 + s * 64 + lane;
-    const bool valid = chunk < nchunks;
-    const int cl = valid ? chunk : 0;  // keep the LDS read in range
-    uint32_t w[NROWS][F::EPL / 2];
+  for (int m = 0; m < NROWS; ++m) F::dequant(c[m][s], w[m], valid);
 #pragma unroll
-    for (int m = 0; m < NROWS; ++m) F::dequant(b.c[m][s], w[m], valid);
+  for (int r = 0; r < RG; ++r) {
+    if (RG == 1 || r < n) {
+      const u32x4* xp = reinterpret_cast<const u32x4*>(xs + size_t(r) * K * 2 + size_t(cl) * (F::EPL * 2));
 #pragma unroll
-    for (int r = 0; r < RG; ++r) {
-      if (RG == 1 || r < n) {
-        const u32x4* xp = reinterpret_cast<const u32x4*>(xs + size_t(r) * K * 2 + size_t(cl) * (F::EPL * 2));
+      for (int v = 0; v < F::EPL / 8; ++v) {
+        const u32x4 xv = xp[v];
 #pragma unroll
-        for (int v = 0; v < F::EPL / 8; ++v) {
-          const u32x4 xv = xp[v];
+        for (int q = 0; q < 4; ++q)
 #pragma unroll
-          for (int q = 0; q < 4; ++q)
-#pragma unroll
-            for (int m = 0; m < NROWS; ++m) acc[m][r] = dot2_bf16(w[m][4 * v + q], xv[q], acc[m][r]);
-        }
+          for (int m = 0; m < NROWS; ++m) acc[m][r] = dot2_bf16(w[m][4 * v + q], xv[q], acc[m][r]);
       }
     }
   }

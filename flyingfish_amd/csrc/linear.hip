@@ -14,68 +14,76 @@ struct LinearParams {
   int m, n, k;
 };
 
-// Each block walks a contiguous range of output columns; a wave streams one weight row at a time
-// against up to RG activation rows held in LDS; rows beyond RG are served by further passes.
+// Each block walks a contiguous range of output columns and each wave a contiguous run of it, streaming one
+// weight row at a time against up to RG activation rows held in LDS; rows beyond RG are served by further
+// passes. One register buffer of S steps per wave: step s of the next item is requested as soon as step s of
+// the current one has been consumed.
 template <class F, int S, int RG>
 __global__ __launch_bounds__(256) void k_linear(const LinearParams p) {
   constexpr int NW = 4;
   extern __shared__ __align__(16) uint8_t xs[];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int K = p.k;
   const long long lo = (long long)p.n * blockIdx.x / gridDim.x, hi = (long long)p.n * (blockIdx.x + 1) / gridDim.x;
-  const int j0 = int(lo), count = int(hi - lo);
-  const float global = p.global ? *p.global : 1.0f;
+  const int count = int(hi - lo);
+  const float global = p.global ? load_global<float>(p.global) : 1.0f;
   const int nchunks = K / F::EPL;
   const int nslabs = (nchunks + S * 64 - 1) / (S * 64);
-  const int my_units = count > wave ? (count - wave + NW - 1) / NW : 0;
+  const int w_lo = count * wave / NW, w_hi = count * (wave + 1) / NW;
+  const int my_units = w_hi - w_lo;
   const int items = my_units * nslabs;
+  const int jw = int(lo) + w_lo;
   for (int r0 = 0; r0 < p.m; r0 += RG) {
     const int n = p.m - r0 < RG ? p.m - r0 : RG;
-    __syncthreads();
-    {
-      const u32x4* s4 = reinterpret_cast<const u32x4*>(p.x + size_t(r0) * K);
-      u32x4* d4 = reinterpret_cast<u32x4*>(xs);
-      const int words = n * (K >> 3);
-      for (int v = tid; v < words; v += 256) d4[v] = s4[v];
+    typename F::Chunk buf[1][S];
+    auto issue_step = [&](int t, int s) {
+      const int j = jw + t / nslabs;
+      const int chunk = (t % nslabs) * (S * 64) + s * 64 + lane;
+      F::load(buf[0][s], F::row(p.codes, p.scales, global, j, K), chunk < nchunks ? chunk : nchunks - 1);
+    };
+    if (items > 0) {
+#pragma unroll
+      for (int s = 0; s < S; ++s) issue_step(0, s);
     }
     __syncthreads();
-    UnitBuf<F, S, 1> bufA, bufB;
-    float acc[1][RG];
+    {
+      u32x4* d4 = reinterpret_cast<u32x4*>(xs);
+      const int words = n * (K >> 3);
+      for (int v = tid; v < words; v += 256) d4[v] = load16(p.x + size_t(r0) * K + size_t(v) * 8);
+    }
+    __syncthreads();
+    if (items > 0) {
+      float acc[1][RG];
 #pragma unroll
-    for (int r = 0; r < RG; ++r) acc[0][r] = 0.0f;
-    auto issue = [&](UnitBuf<F, S, 1>& b, int t) {
-      const int j = j0 + wave + (t / nslabs) * NW;
-      const int chunk0 = (t % nslabs) * (S * 64);
-      const typename F::Row rw = F::row(p.codes, p.scales, global, j, K);
+      for (int r = 0; r < RG; ++r) acc[0][r] = 0.0f;
+      auto compute_step = [&](int t, int s) {
+        const int chunk = (t % nslabs) * (S * 64) + s * 64 + lane;
+        step_compute<F, 1, RG, S>(buf, s, xs, K, nchunks, chunk, n, acc);
+      };
+      auto item_end = [&](int t) {
+        if (t % nslabs != nslabs - 1) return;
+        const int j = jw + t / nslabs;
 #pragma unroll
-      for (int s = 0; s < S; ++s) {
-        const int chunk = chunk0 + s * 64 + lane;
-        F::load(b.c[0][s], rw, chunk < nchunks ? chunk : nchunks - 1);
+        for (int r = 0; r < RG; ++r) {
+          if (RG == 1 || r < n) {
+            const float total = wave_sum(acc[0][r]);
+            if (lane == r) p.y[size_t(r0 + r) * p.n + j] = f32_to_bf16(total);
+          }
+          acc[0][r] = 0.0f;
+        }
+      };
+      for (int t = 0; t + 1 < items; ++t) {
+#pragma unroll
+        for (int s = 0; s < S; ++s) {
+          compute_step(t, s);
+          issue_step(t + 1, s);
+        }
+        item_end(t);
       }
-    };
-    auto finish = [&](const UnitBuf<F, S, 1>& b, int t) {
-      const int j = j0 + wave + (t / nslabs) * NW;
-      const int slab = t % nslabs;
-      slab_compute<F, S, 1, RG>(b, xs, K, nchunks, slab * (S * 64), n, lane, acc);
-      if (slab != nslabs - 1) return;
 #pragma unroll
-      for (int r = 0; r < RG; ++r)
-        if (r < n) acc[0][r] = wave_sum(acc[0][r]);
-#pragma unroll
-      for (int r = 0; r < RG; ++r) {
-        if (r < n && lane == r) p.y[size_t(r0 + r) * p.n + j] = f32_to_bf16(acc[0][r]);
-        acc[0][r] = 0.0f;
-      }
-    };
-    int t = 0;
-    if (t < items) issue(bufA, t);
-    while (t < items) {
-      if (t + 1 < items) issue(bufB, t + 1);
-      finish(bufA, t);
-      if (++t >= items) break;
-      if (t + 1 < items) issue(bufA, t + 1);
-      finish(bufB, t);
-      ++t;
+      for (int s = 0; s < S; ++s) compute_step(items - 1, s);
+      item_end(items - 1);
     }
   }
 }

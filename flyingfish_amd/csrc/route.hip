@@ -47,29 +47,46 @@ __global__ __launch_bounds__(64) void k_route_logits_bf16(const uint16_t* __rest
 }
 
 // FP32 logits: one wave per expert, RB rows at a time; lane L chains the 8-element vectors
-// L, L+64, ...; lane partials are summed with a shuffle-down tree 32..1 (lane 0 holds the sum).
+// L, L+64, ... in ascending order; lane partials are summed with a shuffle-down tree 32..1 (lane 0 holds
+// the sum). Router words are fetched PF at a time so the chain waits on memory once per batch.
 template <int RB>
 __global__ __launch_bounds__(256) void k_route_logits_f32(const uint16_t* __restrict__ x, const uint16_t* __restrict__ router,
                                                           float* __restrict__ logits, int rows, int experts, int hidden) {
+  constexpr int PF = RB == 1 ? 8 : 4;
   const int lane = threadIdx.x & 63;
   const int e = blockIdx.x * 4 + (threadIdx.x >> 6);
   const int r0 = blockIdx.y * RB;
   if (e >= experts) return;
   const int words = hidden >> 3;
-  const u32x4* wr = reinterpret_cast<const u32x4*>(router + size_t(e) * hidden);
+  const uint16_t* wr = router + size_t(e) * hidden;
   float acc[RB];
 #pragma unroll
   for (int r = 0; r < RB; ++r) acc[r] = 0.0f;
-  for (int v = lane; v < words; v += 64) {
-    const u32x4 wv = wr[v];
+  for (int v0 = lane; v0 < words; v0 += 64 * PF) {
+    u32x4 wv[PF];
+#pragma unroll
+    for (int i = 0; i < PF; ++i) {
+      const int v = v0 + 64 * i;
+      wv[i] = load16(wr + size_t(v < words ? v : lane) * 8);
+    }
 #pragma unroll
     for (int r = 0; r < RB; ++r) {
       if (r0 + r < rows) {
-        const u32x4 xv = reinterpret_cast<const u32x4*>(x + size_t(r0 + r) * hidden)[v];
+        u32x4 xv[PF];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          acc[r] = __fmaf_rn(bf16lo(xv[q]), bf16lo(wv[q]), acc[r]);
-          acc[r] = __fmaf_rn(bf16hi(xv[q]), bf16hi(wv[q]), acc[r]);
+        for (int i = 0; i < PF; ++i) {
+          const int v = v0 + 64 * i;
+          xv[i] = load16(x + size_t(r0 + r) * hidden + size_t(v < words ? v : lane) * 8);
+        }
+#pragma unroll
+        for (int i = 0; i < PF; ++i) {
+          if (v0 + 64 * i < words) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              acc[r] = __fmaf_rn(bf16lo(xv[i][q]), bf16lo(wv[i][q]), acc[r]);
+              acc[r] = __fmaf_rn(bf16hi(xv[i][q]), bf16hi(wv[i][q]), acc[r]);
+            }
+          }
         }
       }
     }
@@ -87,21 +104,20 @@ __global__ __launch_bounds__(256) void k_route_logits_f32(const uint16_t* __rest
 }
 
 // ---------------------------------------------------------------------------------------------
-// Block-wide arg-max under (value desc, id asc); every thread receives the winner.
-struct Best { float v; int id; };
-__device__ __forceinline__ Best better(Best a, Best b) {
-  return (b.v > a.v || (b.v == a.v && b.id < a.id)) ? b : a;
-}
-__device__ __forceinline__ Best block_argmax(Best mine, float* s_v, int* s_id, int nwaves) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  wave_argmax(mine.v, mine.id);
-  if (nwaves == 1) return mine;
-  __syncthreads();  // previous round's readers are done with s_v/s_id
-  if (lane == 0) { s_v[wave] = mine.v; s_id[wave] = mine.id; }
-  __syncthreads();
-  Best r; r.v = s_v[0]; r.id = s_id[0];
-  for (int w = 1; w < nwaves; ++w) { Best o; o.v = s_v[w]; o.id = s_id[w]; r = better(r, o); }
-  return r;
+// Selection by rank. The reference runs top_k rounds of a block-wide arg-max under (score desc, id asc)
+// (kernels/moe_route.cu:205-235); that order is total, so the r-th pick is the candidate with exactly r
+// candidates ahead of it. Every thread counts the candidates ahead of its own in one pass over LDS.
+// s_key[e] = selection score of expert e, -inf for experts that cannot be picked; padded to a multiple of 4.
+__device__ __forceinline__ int rank_of(const float* s_key, int padded, float mine, int e) {
+  int rank = 0;
+  for (int i = 0; i < padded; i += 4) {
+    const float4 v = *reinterpret_cast<const float4*>(s_key + i);
+    rank += (v.x > mine || (v.x == mine && i + 0 < e)) ? 1 : 0;
+    rank += (v.y > mine || (v.y == mine && i + 1 < e)) ? 1 : 0;
+    rank += (v.z > mine || (v.z == mine && i + 2 < e)) ? 1 : 0;
+    rank += (v.w > mine || (v.w == mine && i + 3 < e)) ? 1 : 0;
+  }
+  return rank;
 }
 
 // Softmax / sigmoid top-k over BF16 logits (kernels/moe_route.cu:154-301). One block per row, thread e
@@ -110,9 +126,9 @@ __global__ void k_route_topk(const uint16_t* __restrict__ logits, int* __restric
                              int experts, int top_k, int score_mode) {
   __shared__ float s_red[32];
   __shared__ float s_v[16];
-  __shared__ int s_id[16];
   __shared__ float s_sel[FFMOE_MAX_TOP_K];
   __shared__ int s_selid[FFMOE_MAX_TOP_K];
+  __shared__ __align__(16) float s_key[FFMOE_MAX_EXPERTS];
   const int tid = threadIdx.x, row = blockIdx.x;
   const int e = tid;
   const bool live = e < experts;
@@ -147,21 +163,15 @@ __global__ void k_route_topk(const uint16_t* __restrict__ logits, int* __restric
       if (tid == 0) s_red[0] = v;
     }
     __syncthreads();
-    score = live ? __fdiv_rn(ev, s_red[0]) : -1.0f;
+    score = live ? __fdiv_rn(ev, s_red[0]) : -INFINITY;
   } else {
-    score = live ? sigmoid1(logit) : -1.0f;
+    score = live ? sigmoid1(logit) : -INFINITY;
   }
-  bool taken = false;
-  for (int r = 0; r < top_k; ++r) {
-    Best mine;
-    mine.v = (!taken && live) ? score : -1.0f;
-    mine.id = live ? e : 0x7fffffff;
-    const Best win = block_argmax(mine, s_v, s_id, nwaves);
-    if (live && !taken && e == win.id) {
-      s_sel[r] = score;
-      s_selid[r] = e;
-      taken = true;
-    }
+  s_key[tid] = score;  // blockDim is a multiple of 64 covering every expert
+  __syncthreads();
+  if (live) {
+    const int rank = rank_of(s_key, blockDim.x, score, e);
+    if (rank < top_k) { s_sel[rank] = score; s_selid[rank] = e; }
   }
   __syncthreads();
   if (tid < top_k) {
@@ -177,17 +187,14 @@ __global__ void k_route_topk(const uint16_t* __restrict__ logits, int* __restric
 __global__ void k_route_topk_noaux(const float* __restrict__ logits, const float* __restrict__ bias, int bias_row_stride,
                                    int* __restrict__ ids, void* __restrict__ weights, int weights_f32, int experts,
                                    int top_k, int score_mode, float routed_scaling, int n_group, int topk_group) {
-  __shared__ float s_v[16];
-  __shared__ int s_id[16];
   __shared__ float s_sel[FFMOE_MAX_TOP_K];
   __shared__ int s_selid[FFMOE_MAX_TOP_K];
-  __shared__ float s_score[FFMOE_MAX_EXPERTS];
-  __shared__ float s_group[FFMOE_MAX_EXPERTS];
-  __shared__ unsigned char s_keep[FFMOE_MAX_EXPERTS];
+  __shared__ __align__(16) float s_key[FFMOE_MAX_EXPERTS];
+  __shared__ float s_top[2 * FFMOE_MAX_EXPERTS / 2];
+  __shared__ __align__(16) float s_group[FFMOE_MAX_EXPERTS / 2 + 4];
   const int tid = threadIdx.x, row = blockIdx.x;
   const int e = tid;
   const bool live = e < experts;
-  const int nwaves = blockDim.x >> 6;
   float score = -1.0f, select = -INFINITY;
   if (live) {
     const float l = logits[size_t(row) * experts + e];
@@ -199,44 +206,33 @@ __global__ void k_route_topk_noaux(const float* __restrict__ logits, const float
     }
     select = __fadd_rn(score, bias ? bias[size_t(row) * bias_row_stride + e] : 0.0f);
   }
+  s_key[tid] = select;
+  __syncthreads();
   bool allowed = live;
   if (n_group > 1) {
-    s_score[tid] = select;
-    __syncthreads();
+    // the two largest selection scores of every group, by rank inside the group
     const int per = experts / n_group;
-    if (tid < n_group) {
-      float a = -INFINITY, b = -INFINITY;
-      for (int i = tid * per; i < (tid + 1) * per; ++i) {
-        const float v = s_score[i];
-        if (v > a) { b = a; a = v; } else if (v > b) { b = v; }
+    const int g = live ? e / per : 0;
+    if (live) {
+      int rank = 0;
+      for (int i = g * per; i < (g + 1) * per; ++i) {
+        const float v = s_key[i];
+        rank += (v > select || (v == select && i < e)) ? 1 : 0;
       }
-      s_group[tid] = __fadd_rn(a, b);
-      s_keep[tid] = 0;
+      if (rank < 2) s_top[2 * g + rank] = select;
     }
     __syncthreads();
-    if (tid == 0) {
-      for (int r = 0; r < topk_group; ++r) {
-        int best = -1;
-        for (int g = 0; g < n_group; ++g)
-          if (!s_keep[g] && (best < 0 || s_group[g] > s_group[best])) best = g;
-        s_keep[best] = 1;
-      }
-    }
+    const int gpad = (n_group + 3) & ~3;
+    if (tid < gpad) s_group[tid] = tid < n_group ? __fadd_rn(s_top[2 * tid], s_top[2 * tid + 1]) : -INFINITY;
     __syncthreads();
-    allowed = live && s_keep[e / per] != 0;
+    if (live) allowed = rank_of(s_group, gpad, s_group[g], g) < topk_group;
+    __syncthreads();
+    s_key[tid] = allowed ? select : -INFINITY;
     __syncthreads();
   }
-  bool taken = false;
-  for (int r = 0; r < top_k; ++r) {
-    Best mine;
-    mine.v = (!taken && allowed) ? select : -INFINITY;
-    mine.id = (!taken && allowed) ? e : 0x7fffffff;
-    const Best win = block_argmax(mine, s_v, s_id, nwaves);
-    if (allowed && !taken && e == win.id) {
-      s_sel[r] = score;
-      s_selid[r] = e;
-      taken = true;
-    }
+  if (allowed) {
+    const int rank = rank_of(s_key, blockDim.x, select, e);
+    if (rank < top_k) { s_sel[rank] = score; s_selid[rank] = e; }
   }
   __syncthreads();
   if (tid < top_k) {
