@@ -20,7 +20,7 @@ ERR_NULL, ERR_ALIGN, ERR_SHAPE, ERR_OVERLAP, ERR_UNSUPPORTED, ERR_SCRATCH = -1, 
 
 EXPORTS = [
     "ffmoe_last_error", "ffmoe_version",
-    "ffmoe_route_logits_bf16", "ffmoe_route_logits_f32", "ffmoe_route_topk", "ffmoe_route_topk_noaux", "ffmoe_route_decode",
+    "ffmoe_route_logits_bf16", "ffmoe_route_logits_f32", "ffmoe_route_topk", "ffmoe_route_topk_noaux", "ffmoe_route_noaux_decode", "ffmoe_route_decode",
     "ffmoe_decode_scratch_bytes", "ffmoe_decode_contribute", "ffmoe_decode_contribute_stage",
     "ffmoe_quant_fp8_f32_128", "ffmoe_linear_fp8_block_w8a8", "ffmoe_linear_fp8_block", "ffmoe_linear_nvfp4",
     "ffmoe_gemm_skinny_bf16", "ffmoe_swiglu",
@@ -78,6 +78,7 @@ def lib():
         L.ffmoe_route_logits_f32.argtypes = [P, P, P, I, I, I, P]
         L.ffmoe_route_topk.argtypes = [P, P, P, I, I, I, I, P]
         L.ffmoe_route_topk_noaux.argtypes = [P, P, I, P, P, I, I, I, I, I, F, I, I, P]
+        L.ffmoe_route_noaux_decode.argtypes = [P, P, P, I, P, P, P, I, P, I, I, I, I, I, F, I, I, P]
         L.ffmoe_route_decode.argtypes = [P, P, P, P, P, I, I, I, I, I, P]
         L.ffmoe_decode_scratch_bytes.restype = U64
         L.ffmoe_decode_scratch_bytes.argtypes = [I, I, I, I, I, I]

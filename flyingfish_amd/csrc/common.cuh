@@ -128,7 +128,9 @@ __device__ __forceinline__ float det_log1pf_unit(float u) {
   return __fadd_rn(lg, c);
 }
 
-__device__ __forceinline__ float sigmoid1(float l) { return __fdiv_rn(1.0f, __fadd_rn(1.0f, det_expf(-l))); }
+__device__ __forceinline__ float sigmoid1(float l) {
+  return __fdiv_rn(1.0f, __fadd_rn(1.0f, det_expf(-l)));
+}
 
 // SwiGLU with the BF16 rounding boundary selected by `mode` (FFMOE_SWIGLU_*): returns BF16 bits.
 // SiLU = g / (1 + exp(-g)) as in the production decode kernels of the reference.

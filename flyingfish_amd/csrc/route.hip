@@ -46,61 +46,78 @@ __global__ __launch_bounds__(64) void k_route_logits_bf16(const uint16_t* __rest
   if (live) logits[size_t(row) * experts + e] = f32_to_bf16(acc);
 }
 
-// FP32 logits: one wave per expert, RB rows at a time; lane L chains the 8-element vectors
-// L, L+64, ... in ascending order; lane partials are summed with a shuffle-down tree 32..1 (lane 0 holds
-// the sum). Router words are fetched PF at a time so the chain waits on memory once per batch.
-template <int RB>
-__global__ __launch_bounds__(256) void k_route_logits_f32(const uint16_t* __restrict__ x, const uint16_t* __restrict__ router,
-                                                          float* __restrict__ logits, int rows, int experts, int hidden) {
-  constexpr int PF = RB == 1 ? 8 : 4;
-  const int lane = threadIdx.x & 63;
-  const int e = blockIdx.x * 4 + (threadIdx.x >> 6);
-  const int r0 = blockIdx.y * RB;
-  if (e >= experts) return;
+// FP32 logits. One block of 256 threads per expert: thread p chains the 8-element vectors p, p+256, ... in ascending
+// order; the 256 partials are summed by a balanced pairwise tree in natural order (adjacent pairs, then pairs of
+// pairs, ...), which is what the DPP wave sum followed by ((w0+w1)+(w2+w3)) computes. The router row stays in
+// registers while the block walks over the token rows.
+__device__ __forceinline__ float logit_block_sum(float acc, float* s_part) {
+  const float w = wave_sum(acc);
+  const int wave = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) s_part[wave] = w;
+  __syncthreads();
+  const float total = __fadd_rn(__fadd_rn(s_part[0], s_part[1]), __fadd_rn(s_part[2], s_part[3]));
+  __syncthreads();
+  return total;
+}
+
+constexpr int LOGIT_PF = 4;  // vectors per thread held in registers: covers hidden <= 8192 in one batch
+
+__device__ __forceinline__ void logits_f32_rows(const uint16_t* __restrict__ x, const uint16_t* __restrict__ router,
+                                                float* __restrict__ logits, int e, int r0, int r1, int experts, int hidden,
+                                                float* s_part) {
+  const int tid = threadIdx.x;
   const int words = hidden >> 3;
   const uint16_t* wr = router + size_t(e) * hidden;
-  float acc[RB];
+  const bool one_batch = words <= 256 * LOGIT_PF;
+  u32x4 wv[LOGIT_PF];
+  if (one_batch) {
 #pragma unroll
-  for (int r = 0; r < RB; ++r) acc[r] = 0.0f;
-  for (int v0 = lane; v0 < words; v0 += 64 * PF) {
-    u32x4 wv[PF];
-#pragma unroll
-    for (int i = 0; i < PF; ++i) {
-      const int v = v0 + 64 * i;
-      wv[i] = load16(wr + size_t(v < words ? v : lane) * 8);
+    for (int i = 0; i < LOGIT_PF; ++i) {
+      const int v = tid + 256 * i;
+      wv[i] = load16(wr + size_t(v < words ? v : tid) * 8);
     }
+  }
+  for (int r = r0; r < r1; ++r) {
+    const uint16_t* xr = x + size_t(r) * hidden;
+    float acc = 0.0f;
+    for (int v0 = tid; v0 < words; v0 += 256 * LOGIT_PF) {
+      u32x4 xv[LOGIT_PF];
+      if (!one_batch) {
 #pragma unroll
-    for (int r = 0; r < RB; ++r) {
-      if (r0 + r < rows) {
-        u32x4 xv[PF];
-#pragma unroll
-        for (int i = 0; i < PF; ++i) {
-          const int v = v0 + 64 * i;
-          xv[i] = load16(x + size_t(r0 + r) * hidden + size_t(v < words ? v : lane) * 8);
+        for (int i = 0; i < LOGIT_PF; ++i) {
+          const int v = v0 + 256 * i;
+          wv[i] = load16(wr + size_t(v < words ? v : tid) * 8);
         }
+      }
 #pragma unroll
-        for (int i = 0; i < PF; ++i) {
-          if (v0 + 64 * i < words) {
+      for (int i = 0; i < LOGIT_PF; ++i) {
+        const int v = v0 + 256 * i;
+        xv[i] = load16(xr + size_t(v < words ? v : tid) * 8);
+      }
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-              acc[r] = __fmaf_rn(bf16lo(xv[i][q]), bf16lo(wv[i][q]), acc[r]);
-              acc[r] = __fmaf_rn(bf16hi(xv[i][q]), bf16hi(wv[i][q]), acc[r]);
-            }
+      for (int i = 0; i < LOGIT_PF; ++i) {
+        if (v0 + 256 * i < words) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            acc = __fmaf_rn(bf16lo(xv[i][q]), bf16lo(wv[i][q]), acc);
+            acc = __fmaf_rn(bf16hi(xv[i][q]), bf16hi(wv[i][q]), acc);
           }
         }
       }
     }
+    const float total = logit_block_sum(acc, s_part);
+    if (tid == 0) logits[size_t(r) * experts + e] = total;
   }
-#pragma unroll
-  for (int r = 0; r < RB; ++r) {
-    float v = acc[r];
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-      const float o = __shfl_down(v, off, 64);
-      v = __fadd_rn(v, (lane + off < 64) ? o : 0.0f);  // lanes past the end contribute nothing to lane 0
-    }
-    if (lane == 0 && r0 + r < rows) logits[size_t(r0 + r) * experts + e] = v;
-  }
+}
+
+constexpr int LOGIT_ROWS = 8;  // token rows per block
+
+__global__ __launch_bounds__(256) void k_route_logits_f32(const uint16_t* __restrict__ x, const uint16_t* __restrict__ router,
+                                                          float* __restrict__ logits, int rows, int experts, int hidden) {
+  __shared__ float s_part[4];
+  const int r0 = blockIdx.y * LOGIT_ROWS;
+  const int r1 = r0 + LOGIT_ROWS < rows ? r0 + LOGIT_ROWS : rows;
+  logits_f32_rows(x, router, logits, blockIdx.x, r0, r1, experts, hidden, s_part);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -110,7 +127,8 @@ __global__ __launch_bounds__(256) void k_route_logits_f32(const uint16_t* __rest
 // s_key[e] = selection score of expert e, -inf for experts that cannot be picked; padded to a multiple of 4.
 __device__ __forceinline__ int rank_of(const float* s_key, int padded, float mine, int e) {
   int rank = 0;
-  for (int i = 0; i < padded; i += 4) {
+#pragma unroll 8
+  for (int i = 0; i < padded; i += 4) {  // unrolled so that several LDS reads are in flight; one per trip is latency-bound
     const float4 v = *reinterpret_cast<const float4*>(s_key + i);
     rank += (v.x > mine || (v.x == mine && i + 0 < e)) ? 1 : 0;
     rank += (v.y > mine || (v.y == mine && i + 1 < e)) ? 1 : 0;
@@ -215,6 +233,7 @@ __global__ void k_route_topk_noaux(const float* __restrict__ logits, const float
     const int g = live ? e / per : 0;
     if (live) {
       int rank = 0;
+#pragma unroll 8
       for (int i = g * per; i < (g + 1) * per; ++i) {
         const float v = s_key[i];
         rank += (v > select || (v == select && i < e)) ? 1 : 0;
@@ -245,6 +264,161 @@ __global__ void k_route_topk_noaux(const float* __restrict__ logits, const float
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Single-wave selection, everything in registers: lane L holds the C = experts / 64 candidates L*C .. L*C+C-1 as
+// 64-bit keys (orderable score bits, ~id), so "higher score, then lower id" is one unsigned compare and keys are
+// unique. top_k rounds of (lane-local max, DPP wave max, retire the winner) reproduce the reference's block-wide
+// arg-max rounds (kernels/moe_route.cu:349-377) without LDS or barriers.
+__device__ __forceinline__ uint32_t orderable(float f) {
+  const uint32_t b = __float_as_uint(f);
+  return b ^ ((b >> 31) ? 0xffffffffu : 0x80000000u);
+}
+__device__ __forceinline__ uint64_t max_u64(uint64_t a, uint64_t b) { return a > b ? a : b; }
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ uint64_t dpp_u64(uint64_t v) {
+  const int lo = dpp_or<CTRL, ROW_MASK>(int(uint32_t(v)), int(uint32_t(v)));
+  const int hi = dpp_or<CTRL, ROW_MASK>(int(uint32_t(v >> 32)), int(uint32_t(v >> 32)));
+  return (uint64_t(uint32_t(hi)) << 32) | uint32_t(lo);
+}
+__device__ __forceinline__ uint64_t wave_max_u64(uint64_t v) {
+  v = max_u64(v, dpp_u64<DPP_QUAD_SWAP1, 0xf>(v));
+  v = max_u64(v, dpp_u64<DPP_QUAD_SWAP2, 0xf>(v));
+  v = max_u64(v, dpp_u64<DPP_ROW_HALF_MIRROR, 0xf>(v));
+  v = max_u64(v, dpp_u64<DPP_ROW_MIRROR, 0xf>(v));
+  v = max_u64(v, dpp_u64<DPP_ROW_BCAST15, 0xa>(v));
+  v = max_u64(v, dpp_u64<DPP_ROW_BCAST31, 0xc>(v));
+  const uint32_t lo = uint32_t(__builtin_amdgcn_readlane(int(uint32_t(v)), 63));
+  const uint32_t hi = uint32_t(__builtin_amdgcn_readlane(int(uint32_t(v >> 32)), 63));
+  return (uint64_t(hi) << 32) | lo;
+}
+
+// One wave selects for one row. Requires experts == 64 * C and, with groups, experts / n_group a multiple of C whose
+// lane span is a power of two. score[] = unbiased scores, select[] = score + bias of the lane's C candidates.
+template <int C>
+__device__ __forceinline__ void wave_select_noaux(const float (&score)[C], const float (&select)[C], int lane, int experts,
+                                                  int top_k, float routed_scaling, int n_group, int topk_group,
+                                                  int* __restrict__ ids_row, void* __restrict__ weights_row, int weights_f32) {
+  bool allowed = true;
+  if (n_group > 1) {
+    // the two largest selection scores of the lane, then of the lanes of its group (values only: the group score
+    // is their sum, so ties between members do not matter)
+    float a = -INFINITY, b = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < C; ++j) {
+      const float v = select[j];
+      b = fmaxf(b, fminf(a, v));
+      a = fmaxf(a, v);
+    }
+    const int span = (experts / n_group) / C;  // lanes per group
+    for (int off = 1; off < span; off <<= 1) {
+      const float oa = __shfl_xor(a, off, 64), ob = __shfl_xor(b, off, 64);
+      const float na = fmaxf(a, oa);
+      b = fmaxf(fminf(a, oa), fmaxf(b, ob));
+      a = na;
+    }
+    const float gscore = __fadd_rn(a, b);
+    const int g = lane / span;
+    // rank of the lane's group among the groups under (score desc, id asc)
+    int rank = 0;
+    for (int og = 0; og < n_group; ++og) {
+      const float os = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, gscore), og * span));
+      rank += (os > gscore || (os == gscore && og < g)) ? 1 : 0;
+    }
+    allowed = rank < topk_group;
+  }
+  uint64_t key[C];
+#pragma unroll
+  for (int j = 0; j < C; ++j)
+    key[j] = allowed ? (uint64_t(orderable(select[j])) << 32) | uint32_t(~uint32_t(lane * C + j)) : 0ull;
+  float tsum = 0.0f;
+  float my_w = 0.0f;  // lane r keeps the score of the r-th pick
+  int my_id = 0;
+  for (int r = 0; r < top_k; ++r) {
+    uint64_t best = key[0];
+#pragma unroll
+    for (int j = 1; j < C; ++j) best = max_u64(best, key[j]);
+    const uint64_t win = wave_max_u64(best);
+    const int id = int(~uint32_t(win));
+    float sc = 0.0f;
+#pragma unroll
+    for (int j = 0; j < C; ++j) {
+      const bool hit = key[j] == win;
+      sc = hit ? score[j] : sc;
+      key[j] = hit ? 0ull : key[j];
+    }
+    const float wsc = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, sc), id / C));
+    tsum = __fadd_rn(tsum, wsc);
+    if (lane == r) { my_w = wsc; my_id = id; }
+  }
+  if (lane < top_k) {
+    const float w = __fmul_rn(__fdiv_rn(my_w, __fadd_rn(tsum, 1.0e-20f)), routed_scaling);
+    ids_row[lane] = my_id;
+    if (weights_f32) reinterpret_cast<float*>(weights_row)[lane] = w;
+    else reinterpret_cast<uint16_t*>(weights_row)[lane] = f32_to_bf16(w);
+  }
+}
+
+__device__ __forceinline__ float noaux_score(float l, int score_mode) {
+  if (score_mode == FFMOE_NOAUX_SIGMOID) return sigmoid1(l);
+  const float softplus = __fadd_rn(fmaxf(l, 0.0f), det_log1pf_unit(det_expf(-fabsf(l))));
+  return __builtin_sqrtf(softplus);  // correctly rounded (hipcc default); __fsqrt_rn is the approximate native sqrt
+}
+
+template <int C>
+__device__ __forceinline__ void wave_route_row(const float* __restrict__ logits_row, const float* __restrict__ bias_row,
+                                               int lane, int experts, int top_k, int score_mode, float routed_scaling,
+                                               int n_group, int topk_group, int* ids_row, void* weights_row, int weights_f32) {
+  float score[C], select[C];
+#pragma unroll
+  for (int j = 0; j < C; ++j) {
+    const int e = lane * C + j;
+    const float l = logits_row[e];
+    score[j] = noaux_score(l, score_mode);
+    select[j] = __fadd_rn(score[j], bias_row ? bias_row[e] : 0.0f);
+  }
+  wave_select_noaux<C>(score, select, lane, experts, top_k, routed_scaling, n_group, topk_group, ids_row, weights_row, weights_f32);
+}
+
+__device__ __forceinline__ void wave_route_dispatch(const float* logits_row, const float* bias_row, int lane, int experts,
+                                                    int top_k, int score_mode, float routed_scaling, int n_group,
+                                                    int topk_group, int* ids_row, void* weights_row, int weights_f32) {
+  switch (experts >> 6) {
+    case 1: wave_route_row<1>(logits_row, bias_row, lane, experts, top_k, score_mode, routed_scaling, n_group, topk_group, ids_row, weights_row, weights_f32); break;
+    case 2: wave_route_row<2>(logits_row, bias_row, lane, experts, top_k, score_mode, routed_scaling, n_group, topk_group, ids_row, weights_row, weights_f32); break;
+    case 4: wave_route_row<4>(logits_row, bias_row, lane, experts, top_k, score_mode, routed_scaling, n_group, topk_group, ids_row, weights_row, weights_f32); break;
+    case 8: wave_route_row<8>(logits_row, bias_row, lane, experts, top_k, score_mode, routed_scaling, n_group, topk_group, ids_row, weights_row, weights_f32); break;
+    default: wave_route_row<16>(logits_row, bias_row, lane, experts, top_k, score_mode, routed_scaling, n_group, topk_group, ids_row, weights_row, weights_f32); break;
+  }
+}
+
+__global__ void k_fill_u32(uint32_t* p, uint32_t v, long long n) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = v;
+}
+
+// Host-side test for the register path: experts in {64,128,256,512,1024}; groups must tile the lanes.
+static bool wave_select_ok(int experts, int n_group) {
+  if (experts != 64 && experts != 128 && experts != 256 && experts != 512 && experts != 1024) return false;
+  if (n_group == 1) return true;
+  const int c = experts / 64, per = experts / n_group;
+  if (per % c) return false;
+  const int span = per / c;
+  return span >= 1 && span <= 64 && (span & (span - 1)) == 0;
+}
+
+// noaux selection, one wave per row (register path).
+__global__ __launch_bounds__(64) void k_route_topk_noaux_wave(const float* __restrict__ logits, const float* __restrict__ bias,
+                                                              int bias_row_stride, int* __restrict__ ids, void* __restrict__ weights,
+                                                              int weights_f32, uint32_t* __restrict__ done, int experts, int top_k,
+                                                              int score_mode, float routed_scaling, int n_group, int topk_group) {
+  const int row = blockIdx.x, lane = threadIdx.x;
+  if (done && lane < top_k) done[size_t(row) * top_k + lane] = 0u;  // the contribution of this row starts from a clean slate
+  void* wrow = weights_f32 ? (void*)(reinterpret_cast<float*>(weights) + size_t(row) * top_k)
+                           : (void*)(reinterpret_cast<uint16_t*>(weights) + size_t(row) * top_k);
+  wave_route_dispatch(logits + size_t(row) * experts, bias ? bias + size_t(row) * bias_row_stride : nullptr, lane, experts, top_k,
+                      score_mode, routed_scaling, n_group, topk_group, ids + size_t(row) * top_k, wrow, weights_f32);
+}
+
 }  // namespace ffmoe
 
 using namespace ffmoe;
@@ -273,12 +447,9 @@ extern "C" __attribute__((visibility("default"))) int ffmoe_route_logits_f32(con
   FF_PTR16(x); FF_PTR16(router); FF_PTR4(logits);
   FF_NO_OVERLAP(logits, size_t(rows) * experts * 4, x, size_t(rows) * hidden * 2);
   FF_NO_OVERLAP(logits, size_t(rows) * experts * 4, router, size_t(experts) * hidden * 2);
-  if (rows == 1)
-    hipLaunchKernelGGL(k_route_logits_f32<1>, dim3((experts + 3) / 4, 1), dim3(256), 0, (hipStream_t)stream,
-                       (const uint16_t*)x, (const uint16_t*)router, logits, rows, experts, hidden);
-  else
-    hipLaunchKernelGGL(k_route_logits_f32<8>, dim3((experts + 3) / 4, (rows + 7) / 8), dim3(256), 0, (hipStream_t)stream,
-                       (const uint16_t*)x, (const uint16_t*)router, logits, rows, experts, hidden);
+  FF_REQUIRE((rows + LOGIT_ROWS - 1) / LOGIT_ROWS <= 65535, FFMOE_ERR_SHAPE, "too many rows (%d) for one logits launch", rows);
+  hipLaunchKernelGGL(k_route_logits_f32, dim3(experts, (rows + LOGIT_ROWS - 1) / LOGIT_ROWS), dim3(256), 0, (hipStream_t)stream,
+                     (const uint16_t*)x, (const uint16_t*)router, logits, rows, experts, hidden);
   return ff_launch_status();
 }
 
@@ -322,6 +493,11 @@ extern "C" __attribute__((visibility("default"))) int ffmoe_route_topk_noaux(con
   FF_NO_OVERLAP(ids, size_t(rows) * top_k * 4, logits, size_t(rows) * experts * 4);
   FF_NO_OVERLAP(weights, wbytes, logits, size_t(rows) * experts * 4);
   FF_NO_OVERLAP(ids, size_t(rows) * top_k * 4, weights, wbytes);
+  if (wave_select_ok(experts, n_group)) {
+    hipLaunchKernelGGL(k_route_topk_noaux_wave, dim3(rows), dim3(64), 0, (hipStream_t)stream, logits, bias, bias_row_stride, ids,
+                       weights, weights_f32, (uint32_t*)nullptr, experts, top_k, score_mode, routed_scaling, n_group, topk_group);
+    return ff_launch_status();
+  }
   const int threads = (experts + 63) & ~63;
   hipLaunchKernelGGL(k_route_topk_noaux, dim3(rows), dim3(threads), 0, (hipStream_t)stream, logits, bias, bias_row_stride,
                      ids, weights, weights_f32, experts, top_k, score_mode, routed_scaling, n_group, topk_group);
@@ -334,4 +510,38 @@ extern "C" __attribute__((visibility("default"))) int ffmoe_route_decode(const v
   int rc = ffmoe_route_logits_bf16(x, router, logits, rows, experts, hidden, stream);
   if (rc) return rc;
   return ffmoe_route_topk(logits, ids, weights, rows, experts, top_k, score, stream);
+}
+
+extern "C" __attribute__((visibility("default"))) int ffmoe_route_noaux_decode(const void* x, const void* router, const float* bias, int bias_row_stride, float* logits, int* ids,
+                                        void* weights, int weights_f32, uint32_t* done, int rows, int experts, int hidden,
+                                        int top_k, int score_mode, float routed_scaling, int n_group, int topk_group,
+                                        void* stream) {
+  FF_TRY(ffmoe_route_logits_f32(x, router, logits, rows, experts, hidden, stream));
+  if (done) FF_PTR4(done);
+  if (wave_select_ok(experts, n_group)) {
+    // same checks as ffmoe_route_topk_noaux, then the register-path kernel, which also clears `done`
+    FF_TRY(check_topk_dims(rows, experts, top_k, true));
+    FF_REQUIRE(score_mode == 0 || score_mode == 1, FFMOE_ERR_UNSUPPORTED, "unknown noaux score mode %d", score_mode);
+    FF_REQUIRE(routed_scaling > 0.0f && routed_scaling < INFINITY, FFMOE_ERR_SHAPE, "invalid routed scaling %g", (double)routed_scaling);
+    FF_REQUIRE(bias_row_stride == 0 || bias_row_stride == experts, FFMOE_ERR_SHAPE, "bias row stride %d must be 0 or experts", bias_row_stride);
+    FF_REQUIRE(topk_group >= 1 && topk_group <= n_group && top_k <= topk_group * (experts / n_group), FFMOE_ERR_SHAPE,
+               "invalid grouping n_group=%d topk_group=%d top_k=%d", n_group, topk_group, top_k);
+    FF_PTR4(ids);
+    if (bias) FF_PTR4(bias);
+    if (weights_f32) { FF_PTR4(weights); } else { FF_PTR2(weights); }
+    const size_t wbytes = size_t(rows) * top_k * (weights_f32 ? 4 : 2), lbytes = size_t(rows) * experts * 4;
+    FF_NO_OVERLAP(ids, size_t(rows) * top_k * 4, logits, lbytes);
+    FF_NO_OVERLAP(weights, wbytes, logits, lbytes);
+    FF_NO_OVERLAP(ids, size_t(rows) * top_k * 4, weights, wbytes);
+    hipLaunchKernelGGL(k_route_topk_noaux_wave, dim3(rows), dim3(64), 0, (hipStream_t)stream, logits, bias, bias_row_stride, ids,
+                       weights, weights_f32, done, experts, top_k, score_mode, routed_scaling, n_group, topk_group);
+    return ff_launch_status();
+  }
+  if (done) {  // a fill kernel, not a memset node: callers may capture this call into a HIP graph
+    const long long n = (long long)rows * top_k;
+    hipLaunchKernelGGL(k_fill_u32, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, done, 0u, n);
+    FF_TRY(ff_launch_status());
+  }
+  return ffmoe_route_topk_noaux(logits, bias, bias_row_stride, ids, weights, weights_f32, rows, experts, top_k, score_mode,
+                                routed_scaling, n_group, topk_group, stream);
 }

@@ -166,6 +166,18 @@ class RouteOps:
         return ids, w
 
     @staticmethod
+    def route_noaux(x, router, bias, top_k, logits, ids, weights, done=None, score_mode=capi.NOAUX_SIGMOID,
+                    routed_scaling=1.0, n_group=1, topk_group=1):
+        """FP32 logits + noaux selection; clears `done` for the routed rows."""
+        rows, hidden = x.shape
+        experts = router.shape[0]
+        stride = 0 if bias is None or bias.dim() == 1 else experts
+        capi.check(capi.lib().ffmoe_route_noaux_decode(_ptr(x), _ptr(router), _ptr(bias), stride, _ptr(logits), _ptr(ids), _ptr(weights),
+                                                       int(weights.dtype == torch.float32), _ptr(done), rows, experts,
+                                                       hidden, top_k, score_mode, routed_scaling, n_group, topk_group, _stream()))
+        return ids, weights
+
+    @staticmethod
     def route(x, router, top_k, score=capi.SCORE_SOFTMAX):
         rows, hidden = x.shape
         experts = router.shape[0]
@@ -309,9 +321,8 @@ class NativeMoe:
 
     def run(self, x):
         scaling, ng, kg = self.routing
-        RouteOps.logits_f32(x, self.router, out=self.logits)
-        RouteOps.topk_noaux(self.logits, self.bias, self.top_k, capi.NOAUX_SIGMOID, scaling, ng, kg, True, out=(self.ids, self.weights))
-        self.decode.done.zero_()
+        RouteOps.route_noaux(x, self.router, self.bias, self.top_k, self.logits, self.ids, self.weights,
+                             done=self.decode.done, routed_scaling=scaling, n_group=ng, topk_group=kg)
         contrib, shared_out = self.decode.contribute(x, self.ids, self.weights)
         mode = self.combine_mode if shared_out is not None else capi.COMBINE_ROUTED
         return CombineOps.combine(contrib, shared_out, self.ids, mode, done=self.decode.done, status=self.status, out=self.y)

@@ -87,8 +87,8 @@ int ffmoe_route_logits_bf16(const void* x, const void* router, void* logits,
                             int rows, int experts, int hidden, void* stream);
 
 /* FP32 logits (replaces RouteOps::logits_f32, route.rs:505-562, a BLAS GEMM of undefined order).
- * Order used here: 64 lanes, lane L chains fma over the 8-element vectors L, L+64, ... in ascending
- * order, lane partials summed by a shuffle-down tree 32,16,8,4,2,1. hidden % 8 == 0. */
+ * Order used here: 256 partial chains, partial p chaining fma over the 8-element vectors p, p+256, ... in
+ * ascending order, summed by a balanced pairwise tree in natural order. hidden % 8 == 0. */
 int ffmoe_route_logits_f32(const void* x, const void* router, float* logits,
                            int rows, int experts, int hidden, void* stream);
 
@@ -108,6 +108,16 @@ int ffmoe_route_topk_noaux(const float* logits, const float* bias, int bias_row_
                            int* ids, void* weights, int weights_f32,
                            int rows, int experts, int top_k, int score_mode, float routed_scaling,
                            int n_group, int topk_group, void* stream);
+
+/* Decode route of the noaux_tc models: FP32 logits (ffmoe_route_logits_f32) then the noaux selection, which also
+ * clears `done` (optional, [rows, top_k]) for the rows routed, so the contribution that follows starts from a clean
+ * slate. Replaces NativeMoe::enqueue_route (src/backend/cuda/moe/decode.rs:1145-1168: logits GEMM +
+ * moe_route_topk_noaux_f32). Two launches: on this multi-die GPU a cross-block hand-over inside one kernel costs more
+ * than a kernel boundary. Results are bit-identical to ffmoe_route_logits_f32 followed by ffmoe_route_topk_noaux. */
+int ffmoe_route_noaux_decode(const void* x, const void* router, const float* bias, int bias_row_stride,
+                             float* logits, int* ids, void* weights, int weights_f32, uint32_t* done,
+                             int rows, int experts, int hidden, int top_k, int score_mode, float routed_scaling,
+                             int n_group, int topk_group, void* stream);
 
 /* Fused decode route: BF16 logits (stored) then softmax/sigmoid top-k.
  * Replaces RouteOps::route / moe_route_decode_bf16 (route.rs:450-499; kernels/moe_route.cu:496-568). */

@@ -365,25 +365,26 @@ ORC_API void orc_route_logits_bf16(const uint16_t* x, const uint16_t* w, uint16_
 
 // FP32 logits. The reference takes these from a BLAS GEMM whose summation order is undefined
 // (src/backend/cuda/moe/route.rs:505-562), so any order is within its contract; the order fixed
-// here is the one the HIP kernel uses, so ids can be compared bit for bit: 64 lanes, lane L owns
-// the 8-element vectors v = L, L+64, ... and chains fma over them in ascending order; the lane
-// partials are summed by a shuffle-down tree with offsets 32,16,8,4,2,1. PARITY UNPINNED at bit
-// level (tolerance-checked against float64 in the tests, as the reference's own tests do).
+// here is the one the HIP kernel uses, so ids can be compared bit for bit: 256 partial chains,
+// partial p owning the 8-element vectors v = p, p+256, ... with fma in ascending order; the 256
+// partials are summed by a balanced pairwise tree in natural order (adjacent pairs, then pairs of
+// pairs, ...). PARITY UNPINNED at bit level (tolerance-checked against float64 in the tests, as
+// the reference's own tests do).
 ORC_API void orc_route_logits_f32(const uint16_t* x, const uint16_t* w, float* logits, int rows, int experts, int hidden) {
   const int vectors = hidden / 8;
   for (int r = 0; r < rows; ++r)
     for (int e = 0; e < experts; ++e) {
-      float lanes[64];
-      for (int l = 0; l < 64; ++l) {
+      float part[256];
+      for (int p = 0; p < 256; ++p) {
         float acc = 0.0f;
-        for (int v = l; v < vectors; v += 64)
+        for (int v = p; v < vectors; v += 256)
           for (int s = 0; s < 8; ++s)
             acc = std::fmaf(bf16_f32(x[size_t(r) * hidden + v * 8 + s]), bf16_f32(w[size_t(e) * hidden + v * 8 + s]), acc);
-        lanes[l] = acc;
+        part[p] = acc;
       }
-      for (int off = 32; off > 0; off >>= 1)
-        for (int l = 0; l + off < 64; ++l) lanes[l] = lanes[l] + lanes[l + off];
-      logits[size_t(r) * experts + e] = lanes[0];
+      for (int width = 1; width < 256; width <<= 1)
+        for (int p = 0; p < 256; p += 2 * width) part[p] = part[p] + part[p + width];
+      logits[size_t(r) * experts + e] = part[0];
     }
 }
 

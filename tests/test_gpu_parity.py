@@ -153,6 +153,31 @@ def test_route_noaux_golden_and_random():
                     assert np.array_equal(bits(w), orc.f32_to_bf16(ow))
 
 
+@pytest.mark.parametrize("rows,experts,hidden,top_k,ng,kg", [(1, 256, 7168, 8, 8, 4), (5, 64, 1024, 6, 1, 1), (3, 100, 520, 4, 4, 2), (2, 1000, 256, 32, 1, 1)])
+def test_route_noaux_decode_equals_two_step_and_oracle(rows, experts, hidden, top_k, ng, kg):
+    x, w = rand_bf16((rows, hidden), 1.0, 31), rand_bf16((experts, hidden), 0.02, 32)
+    w[3] = w[7]                                   # two experts with identical logits: the tie goes to the lower id
+    bias = synth.normal((experts,), 0.05, 33)
+    bias[3] = bias[7]
+    logits = torch.empty((rows, experts), dtype=torch.float32, device=DEV)
+    ids = torch.empty((rows, top_k), dtype=torch.int32, device=DEV)
+    wts = torch.empty((rows, top_k), dtype=torch.float32, device=DEV)
+    done = torch.ones((rows, top_k), dtype=torch.int32, device=DEV)
+    for _ in range(2):
+        RouteOps.route_noaux(x.to(DEV), w.to(DEV), bias.to(DEV), top_k, logits, ids, wts, done=done,
+                             routed_scaling=2.5, n_group=ng, topk_group=kg)
+        torch.cuda.synchronize()
+        assert int(done.abs().sum().item()) == 0
+        ol = orc.route_logits_f32(bits(x), bits(w))
+        oi, ow = orc.route_topk_noaux(ol, bias.numpy()[None, :], top_k, 0, 2.5, ng, kg)
+        assert np.array_equal(logits.cpu().numpy().view(np.uint32), ol.view(np.uint32))
+        assert np.array_equal(ids.cpu().numpy(), oi)
+        assert np.array_equal(wts.cpu().numpy().view(np.uint32), ow.view(np.uint32))
+        done.fill_(1)
+    i2, w2 = RouteOps.topk_noaux(RouteOps.logits_f32(x.to(DEV), w.to(DEV)), bias.to(DEV), top_k, 0, 2.5, ng, kg, True)
+    assert torch.equal(i2, ids) and torch.equal(w2.view(torch.int32), wts.view(torch.int32))
+
+
 def test_route_decode_fused_c1_shape():
     x, w = rand_bf16((1, 2048), 1.0, 21), rand_bf16((64, 2048), 0.02, 22)
     ids, wt, logits = RouteOps.route(x.to(DEV), w.to(DEV), 4, capi.SCORE_SOFTMAX)
