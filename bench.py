@@ -21,6 +21,11 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
 
+# HBM bytes per gate/up launch from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of this script, each scaled by what
+# the same counter reads for a 256 MiB plain copy (--calibrate-copy); measured per workload, keyed by (batch, experts).
+# Summary and commands: profiles/decode_layer_fp8_c3_batch1.hbm_traffic.txt. Other workloads report null.
+GATE_UP_TRAFFIC_BYTES = {(1, 256): 265007737}
+
 
 def parse():
     ap = argparse.ArgumentParser()
@@ -33,6 +38,9 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--graph", action="store_true", help="replay one HIP graph per ring slot instead of launching eagerly "
                     "(eager is faster here: launches run ahead of the GPU, a graph replay adds a few microseconds per step)")
+    ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
+                    help="also run one plain device copy of this many MiB (a known-size kernel that scales the "
+                         "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     ap.add_argument("--seed", type=int, default=20251)
     return ap.parse_args()
 
@@ -133,6 +141,14 @@ def main():
     H, I, E, K = dims
     torch.cuda.synchronize()
 
+    if args.calibrate_copy:
+        src = torch.full((args.calibrate_copy << 20,), 3, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)  # reads and writes exactly calibrate_copy MiB
+        torch.cuda.synchronize()
+        del src, dst
+
     # distinct experts per ring slot (measured from the ids)
     distinct = []
     for x in xs:
@@ -217,7 +233,7 @@ def main():
         "layer_hbm_frac": bytes_layer / (us_per_layer * 1e-6) / 1e9 / HBM_PEAK_GBPS,
         "roofline": {"kernel": "ffmoe::k_decode_stage<FmtFp8, S, 0, RG, 1> (gate/up + SwiGLU stage of ffmoe_decode_contribute)",
                      "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
+                     "frac": achieved / HBM_PEAK_GBPS, "traffic": GATE_UP_TRAFFIC_BYTES.get((args.batch, args.experts)),
                      "bytes_per_launch": k_bytes, "avg_us": k_avg, "min_us": kt[0], "median_us": kt[len(kt) // 2],
                      "launches_timed": nb * batch},
     }
