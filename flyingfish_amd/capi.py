@@ -52,8 +52,8 @@ class Decode(ctypes.Structure):
 
 
 class Prefill(ctypes.Structure):
-    _fields_ = [("rows", I), ("top_k", I), ("swiglu", I), ("swiglu_limit", F), ("routed_weight", I), ("weights_f32", I),
-                ("x", P), ("ids", P), ("active", P), ("weights", P),
+    _fields_ = [("rows", I), ("top_k", I), ("act_mode", I), ("swiglu", I), ("swiglu_limit", F), ("routed_weight", I),
+                ("weights_f32", I), ("x", P), ("ids", P), ("active", P), ("weights", P),
                 ("contributions", P), ("done", P), ("scratch", P), ("scratch_bytes", U64)]
 
 

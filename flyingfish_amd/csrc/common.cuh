@@ -134,6 +134,24 @@ __device__ __forceinline__ float sigmoid1(float l) {
 
 // SwiGLU with the BF16 rounding boundary selected by `mode` (FFMOE_SWIGLU_*): returns BF16 bits.
 // SiLU = g / (1 + exp(-g)) as in the production decode kernels of the reference.
+// SiLU as x * sigmoid(x) with the two-branch sigmoid of the reference's dense activation kernels
+// (kernels/q38_contract.cuh:17-21, kernels/act.cu:152-156).
+__device__ __forceinline__ float silu_two_branch(float g) {
+  float s;
+  if (g >= 0.0f) s = __fdiv_rn(1.0f, __fadd_rn(1.0f, det_expf(-g)));
+  else { const float e = det_expf(g); s = __fdiv_rn(e, __fadd_rn(1.0f, e)); }
+  return __fmul_rn(g, s);
+}
+__device__ __forceinline__ uint16_t swiglu_bf16_two_branch(float g, float u, int mode, float limit) {
+  if (mode >= 2) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+  }
+  const float act = silu_two_branch(g);
+  const float prod = (mode == 0 || mode == 2) ? __fmul_rn(bround(act), u) : __fmul_rn(act, u);
+  return f32_to_bf16(prod);
+}
+
 __device__ __forceinline__ uint16_t swiglu_bf16(float g, float u, int mode, float limit) {
   if (mode >= 2) {
     g = fminf(g, limit);
@@ -203,6 +221,14 @@ __device__ __forceinline__ void wave_argmax(float& v, int& id) {
 #undef FF_ARGMAX_STEP
   v = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
   id = __builtin_amdgcn_readlane(id, 63);
+}
+
+// Wave-uniform copies of values every lane already agrees on: they move to scalar registers, so addresses built
+// from them use a scalar base.
+__device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
+__device__ __forceinline__ float unif(float v) { return __builtin_bit_cast(float, uni(__builtin_bit_cast(int, v))); }
+__device__ __forceinline__ uint64_t uni64(uint64_t v) {
+  return (uint64_t(uint32_t(uni(int(v >> 32)))) << 32) | uint32_t(uni(int(uint32_t(v))));
 }
 
 // Loads through pointers known to be global memory. Weight and scale addresses arrive as integers in slot

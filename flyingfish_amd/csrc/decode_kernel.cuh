@@ -19,11 +19,6 @@
 namespace ffmoe {
 
 // ---------------------------------------------------------------------------------------------
-__device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
-__device__ __forceinline__ float unif(float v) { return __builtin_bit_cast(float, uni(__builtin_bit_cast(int, v))); }
-__device__ __forceinline__ uint64_t uni64(uint64_t v) {
-  return (uint64_t(uint32_t(uni(int(v >> 32)))) << 32) | uint32_t(uni(int(uint32_t(v))));
-}
 
 // Group g as wave-uniform scalars. Without a descriptor table (one row per call) every assignment is its own
 // group and the shared expert follows the routed ones.

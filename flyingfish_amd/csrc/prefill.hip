@@ -1,11 +1,306 @@
-// Prefill path (token-sorted grouped FP8 GEMM on MFMA) and the W8A8 block linear.
-#include "common.cuh"
+// Prefill path: device-side grouping of (row, choice) assignments by expert, then the two grouped W8A8 GEMMs on the
+// FP8 matrix cores (gate/up + SwiGLU, down x routing weight scattered to contributions), and the standalone W8A8
+// block linear that shares the GEMM kernel.
+//
+// Reference shape of the pipeline: kernels/moe_prefill.cu:364-553 (count / scan / permute / grouped GEMM / scatter),
+// src/backend/cuda/moe/prefill.rs:1053-1408 (host orchestration). The reference reads the counts back to the host
+// between scan and GEMM (prefill.rs:1146-1147); here grids are sized from upper bounds and every kernel reads the
+// device-side totals, so the call enqueues without a host synchronisation.
+// Arithmetic: the reference's block-F32 W8A8 path (kernels/fp8_linear.cu:12-48, kernels/q38_contract.cuh:239-279,
+// kernels/act.cu:125-159, kernels/moe_ffn.cu:870-908) applied per assignment, so results do not depend on which
+// other rows share an expert.
+#include "w8a8_gemm.cuh"
 #include "api.h"
 
-extern "C" __attribute__((visibility("default"))) int ffmoe_linear_fp8_block_w8a8(const void*, const float*, const void*, const float*, void*, int, int, int, void*) {
-  return ffmoe::ff_fail(FFMOE_ERR_UNSUPPORTED, "ffmoe_linear_fp8_block_w8a8 is not built yet");
+namespace ffmoe {
+
+struct PrefillBook {
+  uint32_t* counts;   // [E]
+  uint32_t* offsets;  // [E + 1]
+  uint32_t* gbase;    // [E + 1] first group of each expert
+  uint32_t* totals;   // [0] units of the gate/up GEMM, [1] units of the down GEMM, [2] groups, [3] active assignments
+  int* perm;          // [A]
+  GemmGroup* groups;
+  u32x2* units0;
+  u32x2* units1;
+};
+
+__global__ void k_prefill_zero(uint32_t* counts, int experts, uint32_t* totals) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < experts) counts[i] = 0u;
+  if (i < 4) totals[i] = 0u;
 }
-extern "C" __attribute__((visibility("default"))) uint64_t ffmoe_prefill_scratch_bytes(int, int, int, int, int) { return 0; }
-extern "C" __attribute__((visibility("default"))) int ffmoe_prefill_contribute(const ffmoe_expert_table*, const ffmoe_prefill*, void*) {
-  return ffmoe::ff_fail(FFMOE_ERR_UNSUPPORTED, "ffmoe_prefill_contribute is not built yet");
+
+__device__ __forceinline__ bool assignment_live(const int* ids, const uint32_t* active, const uint32_t* valid, long long a, int experts, int& e) {
+  e = ids[a];
+  if ((unsigned)e >= (unsigned)experts) return false;
+  if (active && active[a] == 0u) return false;
+  if (valid && valid[e] == 0u) return false;
+  return true;
+}
+
+// histogram of live assignments per expert (kernels/moe_prefill.cu:364-420)
+__global__ __launch_bounds__(256) void k_prefill_count(const int* __restrict__ ids, const uint32_t* __restrict__ active,
+                                                       const uint32_t* __restrict__ valid, uint32_t* __restrict__ counts, long long A, int experts) {
+  const long long a = (long long)blockIdx.x * 256 + threadIdx.x;
+  int e;
+  if (a < A && assignment_live(ids, active, valid, a, experts, e)) atomicAdd(counts + e, 1u);
+}
+
+// exclusive scans over experts (row offsets and group offsets), group descriptors and the two unit lists
+// (kernels/moe_prefill.cu:421-472; unit order = expert, column tile, row group, so neighbours share weights)
+__global__ __launch_bounds__(1024) void k_prefill_plan(PrefillBook b, int experts, int tm, int tiles0, int tiles1) {
+  __shared__ uint32_t s_rows[1025], s_groups[1025], s_tmp[1024];
+  const int tid = threadIdx.x;
+  const uint32_t c = tid < experts ? b.counts[tid] : 0u;
+  const uint32_t g = (c + tm - 1) / tm;
+  // Hillis-Steele inclusive scans
+  uint32_t vr = c, vg = g;
+  s_tmp[tid] = vr; __syncthreads();
+  for (int off = 1; off < 1024; off <<= 1) {
+    const uint32_t add = tid >= off ? s_tmp[tid - off] : 0u;
+    __syncthreads();
+    vr += add; s_tmp[tid] = vr;
+    __syncthreads();
+  }
+  s_rows[tid + 1] = vr; if (tid == 0) s_rows[0] = 0u;
+  __syncthreads();
+  s_tmp[tid] = vg; __syncthreads();
+  for (int off = 1; off < 1024; off <<= 1) {
+    const uint32_t add = tid >= off ? s_tmp[tid - off] : 0u;
+    __syncthreads();
+    vg += add; s_tmp[tid] = vg;
+    __syncthreads();
+  }
+  s_groups[tid + 1] = vg; if (tid == 0) s_groups[0] = 0u;
+  __syncthreads();
+  if (tid < experts) { b.offsets[tid] = s_rows[tid]; b.gbase[tid] = s_groups[tid]; }
+  if (tid == 0) { b.offsets[experts] = s_rows[experts]; b.gbase[experts] = s_groups[experts]; }
+  const uint32_t G = s_groups[experts];
+  if (tid == 0) { b.totals[0] = G * tiles0; b.totals[1] = G * tiles1; b.totals[2] = G; b.totals[3] = s_rows[experts]; }
+  // group descriptors
+  for (uint32_t q = tid; q < G; q += 1024) {
+    int lo = 0, hi = experts;  // last e with s_groups[e] <= q
+    while (hi - lo > 1) { const int mid = (lo + hi) >> 1; if (s_groups[mid] <= q) lo = mid; else hi = mid; }
+    const uint32_t i = q - s_groups[lo];
+    const uint32_t cnt = s_rows[lo + 1] - s_rows[lo];
+    GemmGroup gd;
+    gd.expert = lo; gd.start = int(s_rows[lo] + i * tm); gd.n = int(min(uint32_t(tm), cnt - i * tm)); gd.pad = 0;
+    b.groups[q] = gd;
+  }
+  // unit lists
+  for (int pass = 0; pass < 2; ++pass) {
+    const uint32_t tiles = pass == 0 ? tiles0 : tiles1;
+    u32x2* units = pass == 0 ? b.units0 : b.units1;
+    for (uint32_t u = tid; u < G * tiles; u += 1024) {
+      const uint32_t key = u / tiles;
+      int lo = 0, hi = experts;
+      while (hi - lo > 1) { const int mid = (lo + hi) >> 1; if (s_groups[mid] <= key) lo = mid; else hi = mid; }
+      const uint32_t ge = s_groups[lo + 1] - s_groups[lo];
+      const uint32_t v = u - s_groups[lo] * tiles;
+      { const u32x2 e2 = {s_groups[lo] + v % ge, v / ge}; units[u] = e2; }
+    }
+  }
+}
+
+// stable fill: block e lists its assignments in ascending assignment order (the reference permutes with an atomic
+// cursor, kernels/moe_prefill.cu:475-510; per-row results make the order irrelevant, a fixed one keeps runs repeatable)
+__global__ __launch_bounds__(256) void k_prefill_fill(const int* __restrict__ ids, const uint32_t* __restrict__ active,
+                                                      const uint32_t* __restrict__ valid, PrefillBook b, long long A, int experts) {
+  __shared__ uint32_t s_wave[4];
+  const int e = blockIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const uint32_t cnt = b.counts[e];
+  if (cnt == 0u) return;
+  uint32_t run = b.offsets[e];
+  for (long long a0 = 0; a0 < A; a0 += 256) {
+    const long long a = a0 + tid;
+    int id;
+    const bool hit = a < A && assignment_live(ids, active, valid, a, experts, id) && id == e;
+    const uint64_t mask = __ballot(hit);
+    const uint32_t before = __popcll(mask & ((uint64_t(1) << lane) - 1));
+    if (lane == 0) s_wave[wave] = __popcll(mask);
+    __syncthreads();
+    uint32_t base = run;
+    for (int w = 0; w < wave; ++w) base += s_wave[w];
+    if (hit) b.perm[base + before] = int(a);
+    run += s_wave[0] + s_wave[1] + s_wave[2] + s_wave[3];
+    __syncthreads();
+  }
+}
+
+// rows beyond the live count keep whatever the scratch held: quantize only live rows
+__global__ __launch_bounds__(256) void k_quant_live(const uint16_t* __restrict__ x, uint8_t* __restrict__ codes, float* __restrict__ scales,
+                                                    const uint32_t* __restrict__ live_rows, int k) {
+  const int groups = k >> 7;
+  const long long cell = (long long)blockIdx.x * 16 + (threadIdx.x >> 4);
+  if (cell >= (long long)(*live_rows) * groups) return;
+  const int sub = threadIdx.x & 15;
+  const long long row = cell / groups;
+  const int first = int(cell % groups) * 128 + sub * 8;
+  float v[8];
+  const u32x4 w = load16(x + row * k + first);
+#pragma unroll
+  for (int q = 0; q < 4; ++q) { v[2 * q] = bf16lo(w[q]); v[2 * q + 1] = bf16hi(w[q]); }
+  float amax = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[i]));
+#pragma unroll
+  for (int off = 8; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 16));
+  const float scale = __fmul_rn(amax, 1.0f / 448.0f);
+  if (sub == 0) scales[cell] = scale;
+  const float divisor = fmaxf(scale, 1.0e-12f);
+  uint32_t out[2] = {0, 0};
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const float q = fminf(448.0f, fmaxf(-448.0f, __fdiv_rn(v[i], divisor)));
+    out[i >> 2] |= uint32_t(e4m3_encode(q)) << (8 * (i & 3));
+  }
+  const u32x2 o = {out[0], out[1]};
+  *reinterpret_cast<u32x2*>(codes + row * k + first) = o;
+}
+
+}  // namespace ffmoe
+
+using namespace ffmoe;
+
+namespace {
+int g_cus_p = 0;
+int num_cus_p() {
+  if (g_cus_p == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+      g_cus_p = n;
+    else
+      g_cus_p = 256;
+  }
+  return g_cus_p;
+}
+
+inline uint64_t up256(uint64_t v) { return (v + 255) & ~uint64_t(255); }
+
+// rows per group for an average of `avg` rows per expert
+int pick_mf(double avg) { return avg > 24.0 ? 4 : avg > 12.0 ? 2 : 1; }
+
+template <int MODE>
+int launch_gemm(const GemmParams& p, int mf, unsigned blocks, hipStream_t stream) {
+  switch (mf) {
+    case 1: hipLaunchKernelGGL((k_w8a8_grouped<1, MODE, 4>), dim3(blocks), dim3(256), 0, stream, p); break;
+    case 2: hipLaunchKernelGGL((k_w8a8_grouped<2, MODE, 4>), dim3(blocks), dim3(256), 0, stream, p); break;
+    default: hipLaunchKernelGGL((k_w8a8_grouped<4, MODE, 2>), dim3(blocks), dim3(256), 0, stream, p); break;
+  }
+  return ff_launch_status();
+}
+
+struct PrefillLayout {
+  uint64_t xq, sx, act, aq, sa, counts, offsets, gbase, totals, perm, groups, units0, units1, total;
+  uint64_t max_groups;
+};
+PrefillLayout prefill_layout(int rows, int top_k, int experts, int hidden, int inter) {
+  PrefillLayout l{};
+  const uint64_t A = uint64_t(rows) * top_k;
+  l.max_groups = uint64_t(experts) + (A + 15) / 16;
+  uint64_t off = 0;
+  auto take = [&](uint64_t bytes) { const uint64_t at = off; off += up256(bytes); return at; };
+  l.xq = take(uint64_t(rows) * hidden);
+  l.sx = take(uint64_t(rows) * (hidden / 128) * 4);
+  l.act = take(A * inter * 2);
+  l.aq = take(A * inter);
+  l.sa = take(A * (inter / 128) * 4);
+  l.counts = take(uint64_t(experts) * 4);
+  l.offsets = take(uint64_t(experts + 1) * 4);
+  l.gbase = take(uint64_t(experts + 1) * 4);
+  l.totals = take(16);
+  l.perm = take(A * 4);
+  l.groups = take(l.max_groups * sizeof(GemmGroup));
+  l.units0 = take(l.max_groups * uint64_t((inter + 127) / 128) * 8);
+  l.units1 = take(l.max_groups * uint64_t((hidden + 255) / 256) * 8);
+  l.total = off;
+  return l;
+}
+}  // namespace
+
+extern "C" __attribute__((visibility("default"))) int ffmoe_linear_fp8_block_w8a8(const void* w_codes, const float* w_scales, const void* x_codes,
+                                                                                 const float* x_scales, void* y, int m, int n, int k, void* stream) {
+  FF_REQUIRE(m >= 1 && n >= 16 && n % 16 == 0 && k >= 128 && k % 128 == 0, FFMOE_ERR_SHAPE,
+             "w8a8 linear m=%d n=%d k=%d (n must be a multiple of 16, k a multiple of 128)", m, n, k);
+  FF_PTR16(w_codes); FF_PTR4(w_scales); FF_PTR16(x_codes); FF_PTR4(x_scales); FF_PTR16(y);
+  FF_NO_OVERLAP(y, size_t(m) * n * 2, x_codes, size_t(m) * k);
+  FF_NO_OVERLAP(y, size_t(m) * n * 2, x_scales, size_t(m) * (k / 128) * 4);
+  const int mf = m > 32 ? 4 : m > 16 ? 2 : 1;
+  const int tm = 16 * mf;
+  GemmParams p{};
+  p.a_codes = (const uint8_t*)x_codes; p.a_scales = x_scales;
+  p.w0_codes = (uint64_t)(uintptr_t)w_codes; p.w0_scales = (uint64_t)(uintptr_t)w_scales;
+  p.total_units = uint32_t(((m + tm - 1) / tm) * ((n + 255) / 256));
+  p.out = (uint16_t*)y; p.rows_total = m; p.K = k; p.N = n; p.top_k = 1;
+  const unsigned blocks = (unsigned)std::min<uint32_t>(p.total_units, uint32_t(num_cus_p()) * 2u);
+  return launch_gemm<2>(p, mf, blocks, (hipStream_t)stream);
+}
+
+extern "C" __attribute__((visibility("default"))) uint64_t ffmoe_prefill_scratch_bytes(int rows, int top_k, int experts, int hidden, int inter) {
+  if (rows < 1 || top_k < 1 || experts < 1 || hidden < 128 || inter < 128) return 0;
+  return prefill_layout(rows, top_k, experts, hidden, inter).total;
+}
+
+extern "C" __attribute__((visibility("default"))) int ffmoe_prefill_contribute(const ffmoe_expert_table* table, const ffmoe_prefill* args, void* stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  FF_REQUIRE(table != nullptr && args != nullptr, FFMOE_ERR_NULL, "table or args is NULL");
+  FF_REQUIRE(table->format == FFMOE_FMT_FP8_BLOCK128, FFMOE_ERR_UNSUPPORTED, "prefill handles FFMOE_FMT_FP8_BLOCK128 experts only (format %d)", table->format);
+  FF_REQUIRE(args->act_mode == FFMOE_ACT_FP8_BLOCK128, FFMOE_ERR_UNSUPPORTED, "prefill runs on the FP8 matrix cores: act_mode must be FFMOE_ACT_FP8_BLOCK128");
+  const int E = table->experts, H = table->hidden, I = table->inter, R = args->rows, K = args->top_k;
+  FF_REQUIRE(E >= 1 && E <= FFMOE_MAX_EXPERTS, FFMOE_ERR_SHAPE, "experts=%d out of range", E);
+  FF_REQUIRE(R >= 1 && K >= 1 && K <= FFMOE_MAX_TOP_K && (long long)R * K <= 0x3fffffffLL, FFMOE_ERR_SHAPE, "rows=%d top_k=%d out of range", R, K);
+  FF_REQUIRE(H >= 128 && H % 128 == 0 && I >= 128 && I % 128 == 0, FFMOE_ERR_SHAPE, "hidden=%d and inter=%d must be multiples of 128", H, I);
+  FF_REQUIRE(args->swiglu >= 0 && args->swiglu <= 3, FFMOE_ERR_UNSUPPORTED, "unknown SwiGLU mode %d", args->swiglu);
+  if (args->swiglu >= 2) FF_REQUIRE(args->swiglu_limit > 0.0f && args->swiglu_limit < INFINITY, FFMOE_ERR_SHAPE, "invalid SwiGLU limit %g", (double)args->swiglu_limit);
+  FF_REQUIRE(args->routed_weight == FFMOE_WEIGHT_AFTER_DOWN_BF16 || args->routed_weight == FFMOE_WEIGHT_BEFORE_CONTRIBUTION_BF16,
+             FFMOE_ERR_UNSUPPORTED, "unknown routed_weight %d", args->routed_weight);
+  FF_PTR16(table->slots); FF_PTR16(args->x); FF_PTR4(args->ids); FF_PTR16(args->contributions);
+  if (args->weights_f32) FF_PTR4(args->weights); else FF_PTR2(args->weights);
+  const PrefillLayout l = prefill_layout(R, K, E, H, I);
+  FF_PTR_ALIGNED(args->scratch, 256);
+  FF_REQUIRE(args->scratch_bytes >= l.total, FFMOE_ERR_SCRATCH, "prefill scratch holds %llu bytes, %llu needed",
+             (unsigned long long)args->scratch_bytes, (unsigned long long)l.total);
+  const size_t A = size_t(R) * K;
+  FF_NO_OVERLAP(args->contributions, A * H * 2, args->x, size_t(R) * H * 2);
+  FF_NO_OVERLAP(args->contributions, A * H * 2, args->scratch, l.total);
+  FF_NO_OVERLAP(args->scratch, l.total, args->x, size_t(R) * H * 2);
+  FF_NO_OVERLAP(args->scratch, l.total, args->ids, A * 4);
+  if (args->done) { FF_PTR4(args->done); FF_NO_OVERLAP(args->done, A * 4, args->scratch, l.total); }
+
+  uint8_t* s = (uint8_t*)args->scratch;
+  PrefillBook b{(uint32_t*)(s + l.counts), (uint32_t*)(s + l.offsets), (uint32_t*)(s + l.gbase), (uint32_t*)(s + l.totals),
+                (int*)(s + l.perm), (GemmGroup*)(s + l.groups), (u32x2*)(s + l.units0), (u32x2*)(s + l.units1)};
+  const int mf = pick_mf(double(A) / E);
+  const int tm = 16 * mf;
+  const int tiles0 = (I + 127) / 128, tiles1 = (H + 255) / 256;
+
+  hipLaunchKernelGGL(k_prefill_zero, dim3((E + 255) / 256), dim3(256), 0, stream, b.counts, E, b.totals);
+  hipLaunchKernelGGL(k_prefill_count, dim3((unsigned)((A + 255) / 256)), dim3(256), 0, stream, args->ids, args->active, table->valid, b.counts, (long long)A, E);
+  hipLaunchKernelGGL(k_prefill_plan, dim3(1), dim3(1024), 0, stream, b, E, tm, tiles0, tiles1);
+  hipLaunchKernelGGL(k_prefill_fill, dim3(E), dim3(256), 0, stream, args->ids, args->active, table->valid, b, (long long)A, E);
+  FF_TRY(ff_launch_status());
+  // activations -> E4M3 + per-128 scales
+  FF_TRY(ffmoe_quant_fp8_f32_128(args->x, s + l.xq, (float*)(s + l.sx), R, H, stream_));
+
+  const unsigned blocks = (unsigned)num_cus_p() * 2u;
+  GemmParams p{};
+  p.slots = table->slots; p.groups = b.groups; p.perm = b.perm; p.top_k = K;
+  p.swiglu = args->swiglu; p.limit = args->swiglu_limit; p.routed_weight = args->routed_weight; p.weights_f32 = args->weights_f32;
+  // gate/up + SwiGLU
+  p.a_codes = s + l.xq; p.a_scales = (const float*)(s + l.sx); p.units = b.units0; p.unit_total = b.totals + 0;
+  p.out = (uint16_t*)(s + l.act); p.K = H; p.N = I;
+  FF_TRY(launch_gemm<0>(p, mf, blocks, stream));
+  // re-quantize the activations of the live rows
+  {
+    const long long cells = (long long)A * (I / 128);
+    hipLaunchKernelGGL(k_quant_live, dim3((unsigned)((cells + 15) / 16)), dim3(256), 0, stream, (const uint16_t*)(s + l.act), s + l.aq,
+                       (float*)(s + l.sa), (const uint32_t*)(b.totals + 3), I);
+    FF_TRY(ff_launch_status());
+  }
+  // down x routing weight, scattered to contributions[assignment]
+  p.a_codes = s + l.aq; p.a_scales = (const float*)(s + l.sa); p.units = b.units1; p.unit_total = b.totals + 1;
+  p.out = (uint16_t*)args->contributions; p.done = args->done; p.weights = args->weights; p.K = I; p.N = H;
+  return launch_gemm<1>(p, mf, blocks, stream);
 }

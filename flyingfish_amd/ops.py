@@ -222,6 +222,58 @@ class DecodeOps:
         return self.contributions, self.shared_out
 
 
+class PrefillOps:
+    """Expert contributions for a prefill cohort (many rows): device-side grouping by expert and two grouped W8A8
+    GEMMs. Host mirror of PrefillOps::prefill_contribute (src/backend/cuda/moe/prefill.rs:1033-1408); owns its scratch
+    arena and the contributions / done buffers."""
+
+    def __init__(self, table, rows, top_k, swiglu=capi.SWIGLU_TWICE, swiglu_limit=0.0,
+                 routed_weight=capi.WEIGHT_AFTER_DOWN_BF16, weights_f32=True):
+        self.table = table
+        self.rows, self.top_k = rows, top_k
+        self.cfg = (swiglu, swiglu_limit, routed_weight, int(weights_f32))
+        dev = table.slots.device
+        nbytes = capi.lib().ffmoe_prefill_scratch_bytes(rows, top_k, table.experts, table.hidden, table.inter)
+        self.scratch = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+        self.contributions = torch.empty((rows, top_k, table.hidden), dtype=_BF16, device=dev)
+        self.done = torch.zeros((rows, top_k), dtype=torch.int32, device=dev)
+        self._table_c = table.c_struct()
+
+    def scratch_views(self):
+        """The arena regions a caller may inspect after contribute(): same offsets as prefill_layout() in
+        csrc/prefill.hip (every region rounded up to 256 bytes). act[pos] is the BF16 SwiGLU output of the assignment
+        perm[pos]; offsets[e]..offsets[e+1] is expert e's segment; totals[3] is the number of live assignments."""
+        t = self.table
+        R, K, E, H, I = self.rows, self.top_k, t.experts, t.hidden, t.inter
+        A = R * K
+        off = 0
+        out = {}
+
+        def take(name, nbytes, dtype, shape):
+            nonlocal off
+            out[name] = self.scratch[off:off + nbytes].view(dtype).view(shape)
+            off += (nbytes + 255) // 256 * 256
+        take("xq", R * H, torch.uint8, (R, H))
+        take("sx", R * (H // 128) * 4, torch.float32, (R, H // 128))
+        take("act", A * I * 2, _BF16, (A, I))
+        take("aq", A * I, torch.uint8, (A, I))
+        take("sa", A * (I // 128) * 4, torch.float32, (A, I // 128))
+        take("counts", E * 4, torch.int32, (E,))
+        take("offsets", (E + 1) * 4, torch.int32, (E + 1,))
+        take("gbase", (E + 1) * 4, torch.int32, (E + 1,))
+        take("totals", 16, torch.int32, (4,))
+        take("perm", A * 4, torch.int32, (A,))
+        return out
+
+    def contribute(self, x, ids, weights, active=None):
+        swiglu, limit, rw, wf32 = self.cfg
+        a = capi.Prefill(self.rows, self.top_k, capi.ACT_FP8_BLOCK128, swiglu, limit, rw, wf32,
+                         x.data_ptr(), ids.data_ptr(), active.data_ptr() if active is not None else None, weights.data_ptr(),
+                         self.contributions.data_ptr(), self.done.data_ptr(), self.scratch.data_ptr(), self.scratch.numel())
+        capi.check(capi.lib().ffmoe_prefill_contribute(ctypes.byref(self._table_c), ctypes.byref(a), _stream()))
+        return self.contributions
+
+
 class CombineOps:
     @staticmethod
     def shared_scale(x, seg):

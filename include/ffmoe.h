@@ -237,13 +237,21 @@ int ffmoe_combine(const void* contributions, const void* shared_out, const void*
                   int rows, int top_k, int hidden, int mode, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
- * Prefill: many tokens, grouped by expert on the device (no host synchronisation), grouped FP8 GEMMs on
- * MFMA in FFMOE_ACT_FP8_BLOCK128 arithmetic. Replaces PrefillOps::prefill_contribute
- * (src/backend/cuda/moe/prefill.rs:1033-1408) and kernels moe_count_scan / moe_permute / moe_gemm_w8a16 /
- * silu_mul / moe_scatter (kernels/moe_prefill.cu). Only FFMOE_FMT_FP8_BLOCK128 tables.
+ * Prefill: many tokens, grouped by expert on the device (no host synchronisation: grids are sized from upper
+ * bounds and kernels read the device-side counts), then two grouped GEMMs on the FP8 matrix cores in
+ * FFMOE_ACT_FP8_BLOCK128 arithmetic: x is quantized per (row, 128) once, gate/up + SwiGLU (two-branch sigmoid,
+ * kernels/act.cu:125-159) writes BF16 activations in expert order, they are re-quantized, and down x routing
+ * weight is scattered to contributions[row, choice, :] with done[row, choice] = 1. Per assignment the arithmetic
+ * equals the reference's <=16-row block-FP8 pipeline (NativeMoe::run, src/backend/cuda/moe/decode.rs:1187-1297;
+ * kernels/moe_ffn.cu:870-908), which is how the reference runs block-FP8 prefill (in 16-row chunks).
+ * Replaces PrefillOps::prefill_contribute (src/backend/cuda/moe/prefill.rs:1033-1408) and kernels moe_count_scan /
+ * moe_permute / moe_gemm_* / silu_mul / moe_scatter_rows (kernels/moe_prefill.cu:364-553).
+ * Only FFMOE_FMT_FP8_BLOCK128 tables; hidden and inter multiples of 128. Assignments whose id is out of range,
+ * whose expert is not valid or whose active flag is 0 contribute nothing and keep done = 0.
  */
 typedef struct ffmoe_prefill {
   int rows, top_k;
+  int act_mode;            /* FFMOE_ACT_FP8_BLOCK128 */
   int swiglu; float swiglu_limit;
   int routed_weight;
   int weights_f32;

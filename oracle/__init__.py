@@ -261,6 +261,33 @@ def linear_fp8_block_w8a8(w_codes, w_scales, x_codes, x_scales, order=0, want_f3
     return (y, yf) if want_f32 else y
 
 
+def expert_ffn_w8a8(x, gate, sgate, up, sup, down, sdown, routing=1.0, rounding=TWICE, limit=0.0, boundary=AFTER_DOWN_BF16,
+                    order=0, silu_kind=SILU_SIGMOID2, apply_weight=True, return_act=False):
+    """One (row, choice) contribution on the block-F32 W8A8 path. x [H] bf16 bits; gate/up codes [I,H]; down [H,I]."""
+    x = _c(x, np.uint16)
+    gate, up, down = _c(gate, np.uint8), _c(up, np.uint8), _c(down, np.uint8)
+    sgate, sup, sdown = _c(sgate, np.float32), _c(sup, np.float32), _c(sdown, np.float32)
+    I, H = gate.shape
+    assert x.shape == (H,) and up.shape == (I, H) and down.shape == (H, I)
+    out = np.empty(H, dtype=np.uint16)
+    act = np.empty(I, dtype=np.uint16)
+    lib().orc_expert_ffn_w8a8(_p(x), _p(gate), _p(sgate), _p(up), _p(sup), _p(down), _p(sdown), H, I, ctypes.c_float(routing),
+                              rounding, ctypes.c_float(limit), boundary, order, silu_kind, int(bool(apply_weight)), _p(out), _p(act))
+    return (out, act) if return_act else out
+
+
+def expert_down_w8a8(act, down, sdown, routing=1.0, boundary=AFTER_DOWN_BF16, order=0, apply_weight=True):
+    """Second half of expert_ffn_w8a8 from a given BF16 activation [I]: re-quantize, down, routing weight."""
+    act = _c(act, np.uint16).reshape(1, -1)
+    aq, sa = quant_act_fp8_128(act)
+    d, lin = linear_fp8_block_w8a8(down, sdown, aq, sa, order=order, want_f32=True)
+    if not apply_weight:
+        return d[0]
+    w = np.float32(routing)
+    v = bf16_to_f32(d[0]) * w if boundary == AFTER_DOWN_BF16 else lin[0] * w
+    return f32_to_bf16(v.astype(np.float32))
+
+
 def linear_skinny(weight_bf16, x_bf16, kind=0):
     w = _c(weight_bf16, np.uint16)
     x = _c(x_bf16, np.uint16)

@@ -589,6 +589,34 @@ ORC_API void orc_linear_fp8_block_w8a8(const uint8_t* w, const float* sw, const 
     }
 }
 
+// One (row, choice) contribution on the block-F32 W8A8 path, the composition the reference runs for block-FP8 models
+// (NativeMoe::run, src/backend/cuda/moe/decode.rs:1187-1297): fp8_quant_f32_128 on x (kernels/fp8_linear.cu:12-48),
+// gate and up through fp8_block_decode to BF16 (kernels/moe_ffn.cu:870-891), SwiGLU on the BF16 pair
+// (kernels/act.cu:125-159), fp8_quant_f32_128 on the activation, down to BF16, then the routing weight
+// (kernels/moe_ffn.cu:894-908: bf16(float(bf16 down) * w); BeforeContributionBf16 multiplies the FP32 sum instead).
+// gate/up codes [I,H] + scales [ceil(I/128), H/128]; down codes [H,I] + scales [ceil(H/128), I/128].
+ORC_API void orc_expert_ffn_w8a8(const uint16_t* x, const uint8_t* gate, const float* sgate, const uint8_t* up, const float* sup,
+                                 const uint8_t* down, const float* sdown, int H, int I, float routing, int rounding, float limit,
+                                 int boundary, int order, int silu_k, int apply_weight, uint16_t* out, uint16_t* act_out) {
+  std::vector<uint8_t> xq(H), aq(I);
+  std::vector<float> sx((H + 127) / 128), sa((I + 127) / 128), lin(H);
+  std::vector<uint16_t> g(I), u(I), act(I), d(H);
+  orc_quant_act_fp8_128(x, 1, H, xq.data(), sx.data());
+  orc_linear_fp8_block_w8a8(gate, sgate, xq.data(), sx.data(), 1, I, H, order, g.data(), nullptr);
+  orc_linear_fp8_block_w8a8(up, sup, xq.data(), sx.data(), 1, I, H, order, u.data(), nullptr);
+  for (int j = 0; j < I; ++j) act[j] = silu_mul_bits(g[j], u[j], rounding, limit, silu_k);
+  if (act_out) std::memcpy(act_out, act.data(), size_t(I) * 2);
+  orc_quant_act_fp8_128(act.data(), 1, I, aq.data(), sa.data());
+  orc_linear_fp8_block_w8a8(down, sdown, aq.data(), sa.data(), 1, H, I, order, d.data(), lin.data());
+  for (int c = 0; c < H; ++c) {
+    float v;
+    if (!apply_weight) v = bf16_f32(d[c]);
+    else if (boundary == AFTER_DOWN_BF16) v = bf16_f32(d[c]) * routing;
+    else v = lin[c] * routing;
+    out[c] = bf16_rne(v);
+  }
+}
+
 // W8A16 skinny linear with the reduction of src/fp8.rs:245-287 (host mirror of
 // kernels/fp8_linear.cu:407-487) over BF16 effective weights [n,k]; the NVFP4 twin is
 // src/fp8.rs:290-340 (kernels/nvfp4_linear.cu:50-229). kind 0 = FP8 order, 1 = NVFP4 order,

@@ -1,0 +1,215 @@
+"""GPU parity of the FP8-matrix-core path: the W8A8 block linear and the grouped prefill, through the C ABI.
+
+Oracle: the block-F32 W8A8 arithmetic per assignment (oracle.expert_ffn_w8a8, oracle.linear_fp8_block_w8a8), both in
+the reference's 32-lane order and with FP64 accumulation. The matrix cores sum each 128-block in their own order, so
+BF16 outputs are compared within 2 BF16 steps / 1e-3 relative L2; grouping, permutation, scatter and done flags are
+exact properties.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle as orc
+from flyingfish_amd import capi, ops, synth
+from helpers import assert_close_bf16, bf16_tensor, bits
+
+pytestmark = pytest.mark.gpu
+
+
+def _fp8_matrix(n, k, seed, std=0.02):
+    w = synth.normal((n, k), std, seed)
+    codes, scales = synth.quant_fp8_block(w)
+    return codes, scales
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 256, 512), (5, 384, 256), (16, 256, 1024), (17, 272, 384), (33, 512, 256), (70, 256, 384), (130, 128, 256)])
+def test_linear_w8a8_matches_oracle(m, n, k):
+    wc, ws = _fp8_matrix(n, k, 7 + m)
+    x = synth.normal((m, k), 1.0, 99 + m, dtype=torch.bfloat16)
+    xq, sx = orc.quant_act_fp8_128(bits(x))
+    want, want_f32 = orc.linear_fp8_block_w8a8(wc.numpy(), ws.numpy(), xq, sx, order=0, want_f32=True)
+    want64 = orc.linear_fp8_block_w8a8(wc.numpy(), ws.numpy(), xq, sx, order=1)
+    y = ops.Fp8Ops.linear_w8a8(wc.cuda(), ws.cuda(), torch.from_numpy(xq).cuda(), torch.from_numpy(sx).cuda())
+    torch.cuda.synchronize()
+    assert_close_bf16(bits(y), want, "w8a8 linear vs 32-lane order", max_ulp=1)
+    assert_close_bf16(bits(y), want64, "w8a8 linear vs FP64", max_ulp=1)
+
+
+def test_linear_w8a8_device_quantizer_chain():
+    """ffmoe_linear_fp8_block(act_mode = FP8_BLOCK128) = device quantizer + W8A8 linear."""
+    m, n, k = 9, 256, 640
+    wc, ws = _fp8_matrix(n, k, 31)
+    x = synth.normal((m, k), 1.0, 32, dtype=torch.bfloat16)
+    xq, sx = orc.quant_act_fp8_128(bits(x))
+    want = orc.linear_fp8_block_w8a8(wc.numpy(), ws.numpy(), xq, sx, order=0)
+    y = ops.Fp8Ops.linear(wc.cuda(), ws.cuda(), x.cuda(), act_mode=capi.ACT_FP8_BLOCK128)
+    torch.cuda.synchronize()
+    assert_close_bf16(bits(y), want, "fp8 block linear, W8A8 mode", max_ulp=1)
+
+
+def test_linear_w8a8_wrong_scale_cell_is_detected():
+    """Mutation control (src/backend/cuda/linear.rs:2236-2250): a swapped scale cell must leave the tolerance."""
+    m, n, k = 4, 256, 512
+    wc, ws = _fp8_matrix(n, k, 41)
+    x = synth.normal((m, k), 1.0, 42, dtype=torch.bfloat16)
+    xq, sx = orc.quant_act_fp8_128(bits(x))
+    bad = ws.clone()
+    bad[0, 1] = bad[0, 1] * 2.0
+    want = orc.linear_fp8_block_w8a8(wc.numpy(), bad.numpy(), xq, sx, order=0)
+    y = ops.Fp8Ops.linear_w8a8(wc.cuda(), ws.cuda(), torch.from_numpy(xq).cuda(), torch.from_numpy(sx).cuda())
+    torch.cuda.synchronize()
+    assert orc.rel_l2(bits(y)[:, :128], want[:, :128]) > 1e-2
+
+
+def _make_fp8_table(experts, hidden, inter, seed):
+    table = ops.ExpertTable.allocate(capi.FMT_FP8_BLOCK128, experts, hidden, inter, "cuda")
+    host = []
+    for e in range(experts):
+        mats = []
+        views = table.expert_views(e)
+        for i, shape in enumerate([(inter, hidden), (inter, hidden), (hidden, inter)]):
+            codes, scales = _fp8_matrix(shape[0], shape[1], seed * 1000 + e * 3 + i)
+            views[2 * i].copy_(codes)
+            views[2 * i + 1].copy_(scales)
+            mats += [codes.numpy(), scales.numpy()]
+        host.append(mats)
+    return table, host
+
+
+def _routing(rows, top_k, experts, seed, skew=0.0):
+    rng = np.random.default_rng(seed)
+    p = np.arange(1, experts + 1, dtype=np.float64) ** -skew
+    p /= p.sum()
+    ids = np.stack([rng.choice(experts, size=top_k, replace=False, p=p) for _ in range(rows)]).astype(np.int32)
+    w = rng.uniform(0.05, 1.0, size=(rows, top_k)).astype(np.float32)
+    return ids, w
+
+
+def _check_prefill(op, host, x_bits, ids, w, swiglu, limit, boundary, live, got):
+    """Stage-wise parity. Dynamic activation quantization amplifies a 1-step difference in one activation (a new
+    group scale moves many codes), so the end-to-end output is only loosely comparable; each stage is compared
+    tightly on the inputs it actually saw:
+      1. bookkeeping: every live assignment appears once, inside its expert's segment, in ascending order;
+      2. act[pos] against the oracle's gate/up + SwiGLU of assignment perm[pos]: gate and up may each sit one BF16
+         step from the oracle's (the linear tests bound that), so their SwiGLU product within 3 steps, 1e-3 rel. L2;
+      3. contributions against the oracle's re-quantize + down + weighting of the GPU's own act: <= 2 BF16 steps;
+      4. end to end: assignments whose act equals the oracle's bit for bit (a minority: the matrix cores keep about
+         14 bits in a 128-term block sum, so a percent or two of the BF16 gate/up values round the other way) must
+         match the full oracle within 2 steps, the whole tensor within 5e-2 relative L2."""
+    rows, top_k = ids.shape
+    v = op.scratch_views()
+    n_live = int(live.sum())
+    assert int(v["totals"][3].item()) == n_live
+    perm = v["perm"].cpu().numpy()[:n_live]
+    offsets = v["offsets"].cpu().numpy()
+    flat_ids = ids.reshape(-1)
+    assert sorted(perm.tolist()) == np.flatnonzero(live.reshape(-1)).tolist()
+    for e in range(len(offsets) - 1):
+        seg = perm[offsets[e]:offsets[e + 1]]
+        assert np.all(flat_ids[seg] == e) and np.all(np.diff(seg) > 0)
+    act = bits(v["act"])[:n_live]
+    want_act = np.empty_like(act)
+    want_full = np.zeros((rows * top_k, x_bits.shape[1]), dtype=np.uint16)
+    want_down = np.zeros_like(want_full)
+    for pos, a in enumerate(perm):
+        r = a // top_k
+        g, sg, u, su, d, sd = host[int(flat_ids[a])]
+        wa = float(w.reshape(-1)[a])
+        want_full[a], want_act[pos] = orc.expert_ffn_w8a8(x_bits[r], g, sg, u, su, d, sd, wa, swiglu, limit, boundary, return_act=True)
+        want_down[a] = orc.expert_down_w8a8(act[pos], d, sd, wa, boundary)
+    assert_close_bf16(act, want_act, "prefill activations", max_ulp=3)
+    g2 = bits(got).reshape(rows * top_k, -1)
+    assert_close_bf16(g2[perm], want_down[perm], "prefill contributions from the device activations")
+    same = np.array([np.array_equal(act[pos], want_act[pos]) for pos in range(n_live)])
+    if same.any():
+        assert_close_bf16(g2[perm[same]], want_full[perm[same]], "prefill contributions, end to end")
+    assert orc.rel_l2(g2[perm], want_full[perm]) <= 5e-2
+    return g2
+
+
+@pytest.mark.parametrize("rows,top_k,experts,hidden,inter,skew", [
+    (48, 4, 8, 256, 128, 0.0),     # ~24 rows per expert -> 32-row groups
+    (40, 2, 16, 384, 384, 1.1),    # skewed, hidden not a multiple of the 256-column tile
+    (7, 3, 32, 256, 256, 0.0),     # fewer rows than experts -> 16-row groups, empty experts
+    (200, 4, 6, 256, 128, 1.1),    # > 64 rows on the popular experts -> several groups per expert
+])
+def test_prefill_matches_per_assignment_oracle(rows, top_k, experts, hidden, inter, skew):
+    table, host = _make_fp8_table(experts, hidden, inter, 5)
+    ids, w = _routing(rows, top_k, experts, 11, skew)
+    x = synth.normal((rows, hidden), 1.0, 12, dtype=torch.bfloat16)
+    op = ops.PrefillOps(table, rows, top_k, swiglu=capi.SWIGLU_CLAMPED_TWICE, swiglu_limit=10.0, weights_f32=True)
+    got = op.contribute(x.cuda(), torch.from_numpy(ids).cuda(), torch.from_numpy(w).cuda())
+    torch.cuda.synchronize()
+    assert int(op.done.sum().item()) == rows * top_k
+    _check_prefill(op, host, bits(x), ids, w, orc.CLAMPED_TWICE, 10.0, orc.AFTER_DOWN_BF16, np.ones_like(ids, dtype=bool), got)
+
+
+def test_prefill_skips_inactive_invalid_and_out_of_range():
+    rows, top_k, experts, hidden, inter = 24, 4, 8, 256, 128
+    table, host = _make_fp8_table(experts, hidden, inter, 6)
+    ids, w = _routing(rows, top_k, experts, 21)
+    ids[3, 1] = 99          # out of range
+    ids[5, 0] = -1
+    active = np.ones((rows, top_k), dtype=np.int32)
+    active[7, 2] = 0
+    active[8, :] = 0
+    valid = torch.ones(experts, dtype=torch.int32)
+    valid[2] = 0
+    table.valid = valid.cuda()
+    live = (active != 0) & (ids >= 0) & (ids < experts)
+    live &= np.where((ids >= 0) & (ids < experts), ids, 0) != 2
+    x = synth.normal((rows, hidden), 1.0, 22, dtype=torch.bfloat16)
+    op = ops.PrefillOps(table, rows, top_k, swiglu=capi.SWIGLU_TWICE, routed_weight=capi.WEIGHT_BEFORE_CONTRIBUTION_BF16, weights_f32=True)
+    sentinel = 0x7fc1
+    op.contributions.view(torch.int16).fill_(sentinel)
+    got = op.contribute(x.cuda(), torch.from_numpy(ids).cuda(), torch.from_numpy(w).cuda(), active=torch.from_numpy(active).cuda())
+    torch.cuda.synchronize()
+    done = op.done.cpu().numpy()
+    assert np.array_equal(done != 0, live)
+    g = _check_prefill(op, host, bits(x), ids, w, orc.TWICE, 0.0, orc.BEFORE_CONTRIBUTION_BF16, live, got)
+    assert np.all(g[~live.reshape(-1)] == sentinel), "a skipped assignment was written"
+
+
+def test_prefill_bf16_routing_weights():
+    rows, top_k, experts, hidden, inter = 20, 2, 4, 256, 128
+    table, host = _make_fp8_table(experts, hidden, inter, 8)
+    ids, w = _routing(rows, top_k, experts, 31)
+    wb = torch.from_numpy(w).to(torch.bfloat16)
+    x = synth.normal((rows, hidden), 1.0, 33, dtype=torch.bfloat16)
+    op = ops.PrefillOps(table, rows, top_k, weights_f32=False)
+    got = op.contribute(x.cuda(), torch.from_numpy(ids).cuda(), wb.cuda())
+    torch.cuda.synchronize()
+    _check_prefill(op, host, bits(x), ids, wb.float().numpy(), orc.TWICE, 0.0, orc.AFTER_DOWN_BF16, np.ones_like(ids, dtype=bool), got)
+
+
+def test_prefill_rows_do_not_depend_on_their_cohort():
+    """Per-row arithmetic: a row gives bit-identical contributions whether it is run with 300 other rows (64-row
+    groups), in a cohort of 9 (16-row groups) or alone."""
+    rows, top_k, experts, hidden, inter = 300, 4, 8, 512, 256
+    table, _ = _make_fp8_table(experts, hidden, inter, 9)
+    ids, w = _routing(rows, top_k, experts, 41, 1.1)
+    x = synth.normal((rows, hidden), 1.0, 42, dtype=torch.bfloat16).cuda()
+    ids_d, w_d = torch.from_numpy(ids).cuda(), torch.from_numpy(w).cuda()
+    full = ops.PrefillOps(table, rows, top_k)
+    ref = bits(full.contribute(x, ids_d, w_d)).copy()
+    for lo, n in [(0, 9), (123, 1), (290, 10)]:
+        part = ops.PrefillOps(table, n, top_k)
+        got = bits(part.contribute(x[lo:lo + n].contiguous(), ids_d[lo:lo + n].contiguous(), w_d[lo:lo + n].contiguous()))
+        assert np.array_equal(got, ref[lo:lo + n]), "rows %d..%d differ between cohorts" % (lo, lo + n)
+
+
+def test_prefill_then_combine_layer():
+    """contribute -> ordered combine equals the oracle's combine over the oracle's contributions within BF16 noise."""
+    rows, top_k, experts, hidden, inter = 32, 4, 8, 256, 128
+    table, host = _make_fp8_table(experts, hidden, inter, 10)
+    ids, w = _routing(rows, top_k, experts, 51)
+    x = synth.normal((rows, hidden), 1.0, 52, dtype=torch.bfloat16)
+    op = ops.PrefillOps(table, rows, top_k)
+    ids_d = torch.from_numpy(ids).cuda()
+    c = op.contribute(x.cuda(), ids_d, torch.from_numpy(w).cuda())
+    status = torch.zeros(1, dtype=torch.int32, device="cuda")
+    y = ops.CombineOps.combine(c, None, ids_d, capi.COMBINE_ROUTED, done=op.done, status=status)
+    torch.cuda.synchronize()
+    assert int(status.item()) == 0
+    want = orc.combine(bits(c), None, None, ids, None, capi.COMBINE_ROUTED)
+    assert np.array_equal(bits(y), want)
