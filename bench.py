@@ -32,7 +32,9 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--batch", type=int, default=1, help="decode tokens per step (1, 8, 64)")
+    ap.add_argument("--workload", choices=["decode", "prefill"], default="decode",
+                    help="decode = BASELINE config 3 (the headline line); prefill = config 5 (4096 tokens, Zipf s=1.1, FP8 matrix cores)")
+    ap.add_argument("--batch", type=int, default=None, help="tokens per step (decode: 1, 8, 64; prefill: 4096)")
     ap.add_argument("--experts", type=int, default=256)
     ap.add_argument("--ring", type=int, default=64, help="distinct token batches cycled through")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -45,7 +47,7 @@ def parse():
     return ap.parse_args()
 
 
-def build_layer(args, torch, capi, ops, synth):
+def build_layer(args, torch, capi, ops, synth, make_tokens=True):
     H, I, E, K = 7168, 2048, args.experts, 8
     dev = "cuda"
     table = ops.ExpertTable.allocate(capi.FMT_FP8_BLOCK128, E + 1, H, I, dev)
@@ -60,6 +62,8 @@ def build_layer(args, torch, capi, ops, synth):
     table.experts = E
     router = synth.normal((E, H), 0.02, args.seed + 1, device=dev, dtype=torch.bfloat16)
     bias = torch.zeros(E, dtype=torch.float32, device=dev)
+    if not make_tokens:
+        return table, None, None, (H, I, E, K)
     layer = ops.NativeMoe(table, shared, router, bias, args.batch, K, routed_scaling=2.5, n_group=8, topk_group=4,
                           swiglu=capi.SWIGLU_TWICE, routed_weight=capi.WEIGHT_AFTER_DOWN_BF16, combine_mode=capi.COMBINE_UNGATED)
     xs = [synth.normal((args.batch, H), 1.0, args.seed + 1000 + i, device=dev, dtype=torch.bfloat16) for i in range(args.ring)]
@@ -125,8 +129,94 @@ def cpu_baseline(args, torch, table, layer, xs, dims):
             "tokens_per_s": 1.0 / med}
 
 
+MFMA_FP8_PEAK_TFLOPS = 5000.0
+
+
+def prefill_main(args, torch, capi, ops, synth):
+    """BASELINE config 5: R tokens routed top-8 over 256 experts with Zipf(s=1.1) popularity (seeded router logits =
+    log popularity under a seeded expert permutation + Gumbel noise, so the top-8 is a draw without replacement),
+    grouped W8A8 GEMMs on the FP8 matrix cores, routed-only ordered combine. A step = top-k selection from the logits
+    + prefill contribute + combine on inputs resident in HBM."""
+    import math
+    R = args.batch
+    table, layer, _, dims = build_layer(args, torch, capi, ops, synth, make_tokens=False)
+    H, I, E, K = dims
+    dev = "cuda"
+    g = torch.Generator(device="cpu").manual_seed(args.seed + 77)
+    order = torch.randperm(E, generator=g)
+    pop = torch.empty(E, dtype=torch.float64)
+    pop[order] = torch.arange(1, E + 1, dtype=torch.float64) ** -1.1
+    u = torch.rand((R, E), generator=g, dtype=torch.float64).clamp_(1e-12, 1.0 - 1e-12)
+    logits = (pop.log()[None, :] - (-u.log()).log()).to(torch.float32).to(dev)
+    x = synth.normal((R, H), 1.0, args.seed + 5000, device=dev, dtype=torch.bfloat16)
+    bias = torch.zeros(E, dtype=torch.float32, device=dev)
+    pre = ops.PrefillOps(table, R, K, swiglu=capi.SWIGLU_TWICE, weights_f32=True)
+    ids = torch.empty((R, K), dtype=torch.int32, device=dev)
+    wts = torch.empty((R, K), dtype=torch.float32, device=dev)
+    y = torch.empty((R, H), dtype=torch.bfloat16, device=dev)
+    status = torch.zeros(1, dtype=torch.int32, device=dev)
+
+    def step():
+        ops.RouteOps.topk_noaux(logits, bias, K, score_mode=capi.NOAUX_SIGMOID, routed_scaling=2.5, weights_f32=True, out=(ids, wts))
+        pre.done.zero_()
+        c = pre.contribute(x, ids, wts)
+        ops.CombineOps.combine(c, None, ids, capi.COMBINE_ROUTED, done=pre.done, status=status, out=y)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    assert int(status.item()) == 0
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / args.steps * 1e3
+    counts = torch.bincount(ids.reshape(-1).long(), minlength=E).cpu()
+    touched = int((counts > 0).sum())
+    A = R * K
+    flop_total = A * 6.0 * H * I
+    # dominant kernel: the gate/up grouped GEMM, timed alone with events on the launch stream
+    nb = max(3, min(args.steps, 20))
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(nb)]
+    ev2 = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(nb)]
+    for a, b in ev:
+        a.record(); pre.contribute(x, ids, wts, stage=1); b.record()
+    for a, b in ev2:
+        a.record(); pre.contribute(x, ids, wts, stage=3); b.record()
+    torch.cuda.synchronize()
+    k0 = sorted(a.elapsed_time(b) for a, b in ev)
+    k1 = sorted(a.elapsed_time(b) for a, b in ev2)
+    k0_avg, k1_avg = sum(k0) / len(k0), sum(k1) / len(k1)
+    flop0 = A * 4.0 * H * I
+    per = table.weight_bytes_per_expert()
+    out = {
+        "metric": "moe_prefill_ms", "value": ms, "unit": "ms/cohort", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "fp8_e4m3 weights x fp8_e4m3 activations (per-128 f32 scales), f32 accumulate", "data": "synthetic",
+        "config": {"workload": "DeepSeek-V3-shape FP8 MoE prefill (BASELINE config 5), %d tokens, Zipf s=1.1" % R,
+                   "hidden": H, "intermediate": I, "experts": E, "top_k": K, "act_mode": "FFMOE_ACT_FP8_BLOCK128 (W8A8)",
+                   "tokens": R, "experts_touched": touched, "max_rows_per_expert": int(counts.max()), "min_rows_per_expert": int(counts.min())},
+        "tokens_per_s": R / (ms * 1e-3),
+        "routed_tflop": flop_total / 1e12,
+        "cohort_tflops": flop_total / (ms * 1e-3) / 1e12,
+        "cohort_mfma_frac": flop_total / (ms * 1e-3) / 1e12 / MFMA_FP8_PEAK_TFLOPS,
+        "weight_bytes_once": touched * per,
+        "cohort_weight_gbps": touched * per / (ms * 1e-3) / 1e9,
+        "roofline": {"kernel": "ffmoe::k_w8a8_grouped<MF, 0, P> (gate/up grouped GEMM + SwiGLU)", "bound": "mfma",
+                     "achieved": flop0 / (k0_avg * 1e-3) / 1e12, "peak": MFMA_FP8_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": flop0 / (k0_avg * 1e-3) / 1e12 / MFMA_FP8_PEAK_TFLOPS, "traffic": None,
+                     "flop_per_launch": flop0, "avg_ms": k0_avg, "min_ms": k0[0],
+                     "weight_bytes_once": touched * per * 2 // 3, "weight_gbps": touched * per * 2 / 3 / (k0_avg * 1e-3) / 1e9},
+        "down_kernel": {"kernel": "ffmoe::k_w8a8_grouped<MF, 1, P>", "avg_ms": k1_avg, "min_ms": k1[0],
+                        "tflops": A * 2.0 * H * I / (k1_avg * 1e-3) / 1e12},
+    }
+    print(json.dumps(out))
+
+
 def main():
     args = parse()
+    if args.batch is None:
+        args.batch = 1 if args.workload == "decode" else 4096
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (expert-parallel sharding is described in DESIGN.md); "
               "run with --gpus 1", file=sys.stderr)
@@ -137,6 +227,10 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(1)
     capi.lib()  # fail loudly when the HIP library is missing
+    if args.workload == "prefill":
+        if args.steps == 200 and args.warmup == 20:
+            args.steps, args.warmup = 10, 2
+        return prefill_main(args, torch, capi, ops, synth)
     table, layer, xs, dims = build_layer(args, torch, capi, ops, synth)
     H, I, E, K = dims
     torch.cuda.synchronize()

@@ -25,7 +25,7 @@ EXPORTS = [
     "ffmoe_quant_fp8_f32_128", "ffmoe_linear_fp8_block_w8a8", "ffmoe_linear_fp8_block", "ffmoe_linear_nvfp4",
     "ffmoe_gemm_skinny_bf16", "ffmoe_swiglu",
     "ffmoe_shared_scale", "ffmoe_combine",
-    "ffmoe_prefill_scratch_bytes", "ffmoe_prefill_contribute",
+    "ffmoe_prefill_scratch_bytes", "ffmoe_prefill_contribute", "ffmoe_prefill_contribute_stage",
 ]
 
 P = ctypes.c_void_p
@@ -95,6 +95,7 @@ def lib():
         L.ffmoe_prefill_scratch_bytes.restype = U64
         L.ffmoe_prefill_scratch_bytes.argtypes = [I, I, I, I, I]
         L.ffmoe_prefill_contribute.argtypes = [ctypes.POINTER(ExpertTable), ctypes.POINTER(Prefill), P]
+        L.ffmoe_prefill_contribute_stage.argtypes = [ctypes.POINTER(ExpertTable), ctypes.POINTER(Prefill), I, P]
         for name in EXPORTS:
             fn = getattr(L, name)
             if fn.restype is ctypes.c_int or name not in ("ffmoe_last_error", "ffmoe_decode_scratch_bytes", "ffmoe_prefill_scratch_bytes"):

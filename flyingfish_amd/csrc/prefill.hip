@@ -11,6 +11,8 @@
 // other rows share an expert.
 #include "w8a8_gemm.cuh"
 #include "api.h"
+#include <algorithm>
+#include <cstdlib>
 
 namespace ffmoe {
 
@@ -180,14 +182,18 @@ int num_cus_p() {
 inline uint64_t up256(uint64_t v) { return (v + 255) & ~uint64_t(255); }
 
 // rows per group for an average of `avg` rows per expert
-int pick_mf(double avg) { return avg > 24.0 ? 4 : avg > 12.0 ? 2 : 1; }
+int pick_mf(double avg) {
+  if (const char* f = getenv("FFMOE_PREFILL_MF")) return atoi(f);
+  return avg > 24.0 ? 4 : avg > 12.0 ? 2 : 1;
+}
 
 template <int MODE>
 int launch_gemm(const GemmParams& p, int mf, unsigned blocks, hipStream_t stream) {
   switch (mf) {
     case 1: hipLaunchKernelGGL((k_w8a8_grouped<1, MODE, 4>), dim3(blocks), dim3(256), 0, stream, p); break;
     case 2: hipLaunchKernelGGL((k_w8a8_grouped<2, MODE, 4>), dim3(blocks), dim3(256), 0, stream, p); break;
-    default: hipLaunchKernelGGL((k_w8a8_grouped<4, MODE, 2>), dim3(blocks), dim3(256), 0, stream, p); break;
+    case 4: hipLaunchKernelGGL((k_w8a8_grouped<4, MODE, 2>), dim3(blocks), dim3(256), 0, stream, p); break;
+    default: hipLaunchKernelGGL((k_w8a8_grouped<8, MODE, 2>), dim3(blocks), dim3(256), 0, stream, p); break;
   }
   return ff_launch_status();
 }
@@ -234,7 +240,7 @@ extern "C" __attribute__((visibility("default"))) int ffmoe_linear_fp8_block_w8a
   p.w0_codes = (uint64_t)(uintptr_t)w_codes; p.w0_scales = (uint64_t)(uintptr_t)w_scales;
   p.total_units = uint32_t(((m + tm - 1) / tm) * ((n + 255) / 256));
   p.out = (uint16_t*)y; p.rows_total = m; p.K = k; p.N = n; p.top_k = 1;
-  const unsigned blocks = (unsigned)std::min<uint32_t>(p.total_units, uint32_t(num_cus_p()) * 2u);
+  const unsigned blocks = (unsigned)std::min<uint32_t>((p.total_units + 7u) & ~7u, uint32_t(num_cus_p()) * 2u) & ~7u;
   return launch_gemm<2>(p, mf, blocks, (hipStream_t)stream);
 }
 
@@ -243,7 +249,18 @@ extern "C" __attribute__((visibility("default"))) uint64_t ffmoe_prefill_scratch
   return prefill_layout(rows, top_k, experts, hidden, inter).total;
 }
 
-extern "C" __attribute__((visibility("default"))) int ffmoe_prefill_contribute(const ffmoe_expert_table* table, const ffmoe_prefill* args, void* stream_) {
+namespace {
+int prefill_impl(const ffmoe_expert_table* table, const ffmoe_prefill* args, int stages, void* stream_);
+}
+extern "C" __attribute__((visibility("default"))) int ffmoe_prefill_contribute(const ffmoe_expert_table* table, const ffmoe_prefill* args, void* stream) {
+  return prefill_impl(table, args, 15, stream);
+}
+extern "C" __attribute__((visibility("default"))) int ffmoe_prefill_contribute_stage(const ffmoe_expert_table* table, const ffmoe_prefill* args, int stage, void* stream) {
+  FF_REQUIRE(stage >= 0 && stage <= 3, FFMOE_ERR_SHAPE, "prefill stage %d (0 plan, 1 gate/up, 2 re-quantize, 3 down)", stage);
+  return prefill_impl(table, args, 1 << stage, stream);
+}
+namespace {
+int prefill_impl(const ffmoe_expert_table* table, const ffmoe_prefill* args, int stages, void* stream_) {
   hipStream_t stream = (hipStream_t)stream_;
   FF_REQUIRE(table != nullptr && args != nullptr, FFMOE_ERR_NULL, "table or args is NULL");
   FF_REQUIRE(table->format == FFMOE_FMT_FP8_BLOCK128, FFMOE_ERR_UNSUPPORTED, "prefill handles FFMOE_FMT_FP8_BLOCK128 experts only (format %d)", table->format);
@@ -276,31 +293,35 @@ extern "C" __attribute__((visibility("default"))) int ffmoe_prefill_contribute(c
   const int tm = 16 * mf;
   const int tiles0 = (I + 127) / 128, tiles1 = (H + 255) / 256;
 
-  hipLaunchKernelGGL(k_prefill_zero, dim3((E + 255) / 256), dim3(256), 0, stream, b.counts, E, b.totals);
-  hipLaunchKernelGGL(k_prefill_count, dim3((unsigned)((A + 255) / 256)), dim3(256), 0, stream, args->ids, args->active, table->valid, b.counts, (long long)A, E);
-  hipLaunchKernelGGL(k_prefill_plan, dim3(1), dim3(1024), 0, stream, b, E, tm, tiles0, tiles1);
-  hipLaunchKernelGGL(k_prefill_fill, dim3(E), dim3(256), 0, stream, args->ids, args->active, table->valid, b, (long long)A, E);
-  FF_TRY(ff_launch_status());
-  // activations -> E4M3 + per-128 scales
-  FF_TRY(ffmoe_quant_fp8_f32_128(args->x, s + l.xq, (float*)(s + l.sx), R, H, stream_));
-
-  const unsigned blocks = (unsigned)num_cus_p() * 2u;
+  if (stages & 1) {
+    hipLaunchKernelGGL(k_prefill_zero, dim3((E + 255) / 256), dim3(256), 0, stream, b.counts, E, b.totals);
+    hipLaunchKernelGGL(k_prefill_count, dim3((unsigned)((A + 255) / 256)), dim3(256), 0, stream, args->ids, args->active, table->valid, b.counts, (long long)A, E);
+    hipLaunchKernelGGL(k_prefill_plan, dim3(1), dim3(1024), 0, stream, b, E, tm, tiles0, tiles1);
+    hipLaunchKernelGGL(k_prefill_fill, dim3(E), dim3(256), 0, stream, args->ids, args->active, table->valid, b, (long long)A, E);
+    FF_TRY(ff_launch_status());
+    // activations -> E4M3 + per-128 scales
+    FF_TRY(ffmoe_quant_fp8_f32_128(args->x, s + l.xq, (float*)(s + l.sx), R, H, stream_));
+  }
+  const unsigned blocks = ((unsigned)num_cus_p() * 2u) & ~7u;
   GemmParams p{};
   p.slots = table->slots; p.groups = b.groups; p.perm = b.perm; p.top_k = K;
   p.swiglu = args->swiglu; p.limit = args->swiglu_limit; p.routed_weight = args->routed_weight; p.weights_f32 = args->weights_f32;
-  // gate/up + SwiGLU
-  p.a_codes = s + l.xq; p.a_scales = (const float*)(s + l.sx); p.units = b.units0; p.unit_total = b.totals + 0;
-  p.out = (uint16_t*)(s + l.act); p.K = H; p.N = I;
-  FF_TRY(launch_gemm<0>(p, mf, blocks, stream));
-  // re-quantize the activations of the live rows
-  {
+  if (stages & 2) {  // gate/up + SwiGLU
+    p.a_codes = s + l.xq; p.a_scales = (const float*)(s + l.sx); p.units = b.units0; p.unit_total = b.totals + 0;
+    p.out = (uint16_t*)(s + l.act); p.K = H; p.N = I;
+    FF_TRY(launch_gemm<0>(p, mf, blocks, stream));
+  }
+  if (stages & 4) {  // re-quantize the activations of the live rows
     const long long cells = (long long)A * (I / 128);
     hipLaunchKernelGGL(k_quant_live, dim3((unsigned)((cells + 15) / 16)), dim3(256), 0, stream, (const uint16_t*)(s + l.act), s + l.aq,
                        (float*)(s + l.sa), (const uint32_t*)(b.totals + 3), I);
     FF_TRY(ff_launch_status());
   }
-  // down x routing weight, scattered to contributions[assignment]
-  p.a_codes = s + l.aq; p.a_scales = (const float*)(s + l.sa); p.units = b.units1; p.unit_total = b.totals + 1;
-  p.out = (uint16_t*)args->contributions; p.done = args->done; p.weights = args->weights; p.K = I; p.N = H;
-  return launch_gemm<1>(p, mf, blocks, stream);
+  if (stages & 8) {  // down x routing weight, scattered to contributions[assignment]
+    p.a_codes = s + l.aq; p.a_scales = (const float*)(s + l.sa); p.units = b.units1; p.unit_total = b.totals + 1;
+    p.out = (uint16_t*)args->contributions; p.done = args->done; p.weights = args->weights; p.K = I; p.N = H;
+    FF_TRY(launch_gemm<1>(p, mf, blocks, stream));
+  }
+  return 0;
 }
+}  // namespace

@@ -49,7 +49,7 @@ template <int MODE>
 __device__ __forceinline__ constexpr int gemm_tile_cols() { return MODE == 0 ? 128 : 256; }
 
 template <int MF, int MODE, int P>
-__global__ __launch_bounds__(256) void k_w8a8_grouped(const GemmParams p) {
+__global__ __launch_bounds__(256, MF <= 4 ? 2 : 1) void k_w8a8_grouped(const GemmParams p) {
   constexpr int TM = 16 * MF;
   constexpr int CHUNKS = TM * 8;                    // 16-byte token chunks per K block
   constexpr int CPT = (CHUNKS + 255) / 256;         // chunks a thread moves per K block
@@ -61,7 +61,13 @@ __global__ __launch_bounds__(256) void k_w8a8_grouped(const GemmParams p) {
   const uint32_t total = p.unit_total ? uint32_t(uni(int(load_global<uint32_t>(p.unit_total)))) : p.total_units;
   const int ntiles = (N + gemm_tile_cols<MODE>() - 1) / gemm_tile_cols<MODE>();
 
-  for (uint32_t u = blockIdx.x; u < total; u += gridDim.x) {
+  // Blocks are dealt to the 8 XCDs round-robin, and each XCD has its own L2. The unit list is cut into 8 contiguous
+  // spans, one per XCD, and the blocks of an XCD walk their span side by side, so the row groups of one (expert,
+  // column tile) meet in the same L2 and its weights leave HBM once.
+  const uint32_t xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3, per_xcd = gridDim.x >> 3;
+  const uint32_t span = (total + 7u) >> 3;
+  const uint32_t span_end = min(total, (xcd + 1u) * span);
+  for (uint32_t u = xcd * span + slot; u < span_end; u += per_xcd) {
 
     int expert, start, n, t;
     if (p.groups) {
@@ -137,7 +143,10 @@ __global__ __launch_bounds__(256) void k_w8a8_grouped(const GemmParams p) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) acc[m][f][r] = 0.0f;
 
-    // prologue: weight fragments of the first P K blocks, token tile 0
+    // prologue: weight fragments of the first P K blocks, token tile 0 into LDS, token tile 1 into registers.
+    // Loads retire in issue order, so anything consumed early must be requested before anything consumed late: in
+    // steady state an iteration first requests token tile kb+2 (written to LDS one iteration later) and then the
+    // weight fragments of K block kb+P, so waiting for the tokens never forces the younger weight loads to land.
     u32x4 w[P][4][2];
 #pragma unroll
     for (int s = 0; s < P; ++s) {
@@ -148,6 +157,8 @@ __global__ __launch_bounds__(256) void k_w8a8_grouped(const GemmParams p) {
         w[s][f][1] = load16(wrow[f] + kb * 128u + 16u);
       }
     }
+    u32x4 tv[CPT];
+    float tsv;
     {
 #pragma unroll
       for (int i = 0; i < CPT; ++i) {
@@ -155,8 +166,23 @@ __global__ __launch_bounds__(256) void k_w8a8_grouped(const GemmParams p) {
         if (stage_chunk) *reinterpret_cast<u32x4*>(&tile[0][tdst[i]]) = v;
       }
       if (tid < TM) *reinterpret_cast<float*>(&tile[0][TM * 128 + tid * 4]) = load_global<float>(ssrc);
+      const uint32_t k1 = uint32_t(min(1, KB - 1));
+#pragma unroll
+      for (int i = 0; i < CPT; ++i) tv[i] = load16(tsrc[i] + k1 * 128u);
+      tsv = load_global<float>(ssrc + k1);
     }
     __syncthreads();
+
+    // LDS addresses of this lane's token fragment pieces (buffer 0)
+    int tlo[MF], thi[MF], tsx[MF];
+#pragma unroll
+    for (int m = 0; m < MF; ++m) {
+      const int trow = 16 * m + (lane & 15);
+      const int q2 = (lane >> 4) * 2;
+      tlo[m] = trow * 128 + (((q2) ^ (trow & 7)) << 4);
+      thi[m] = trow * 128 + (((q2 + 1) ^ (trow & 7)) << 4);
+      tsx[m] = TM * 128 + trow * 4;
+    }
 
     for (int kb0 = 0; kb0 < KB; kb0 += 64) {
       // block scales of K blocks kb0 .. kb0+63, one per lane
@@ -169,40 +195,47 @@ __global__ __launch_bounds__(256) void k_w8a8_grouped(const GemmParams p) {
         for (int s = 0; s < P; ++s) {
           const int kb = kbo + s;
           if (kb < kend) {
-            const int buf = kb & 1;
-            // request the next token tile
-            u32x4 tv[CPT];
-            const uint32_t kn = uint32_t(min(kb + 1, KB - 1));
-#pragma unroll
-            for (int i = 0; i < CPT; ++i) tv[i] = load16(tsrc[i] + kn * 128u);
-            const float tsv = load_global<float>(ssrc + kn);
-
-            const float s0 = unif(__builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, swl0), kb - kb0)));
-            const float s1 = MODE == 0 ? unif(__builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, swl1), kb - kb0))) : s0;
+            const uint8_t* tb = tile[kb & 1];
+            const float s0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, swl0), kb - kb0));
+            const float s1 = MODE == 0 ? __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, swl1), kb - kb0)) : s0;
+            // every row fragment is computed, also the padding of a short group: straight-line code lets the matrix
+            // core overlap with the scale fmas, and short groups are bandwidth-bound anyway
+            v4f pr[MF][4];
+            float sc[MF][2];
 #pragma unroll
             for (int m = 0; m < MF; ++m) {
-              if (m == 0 || 16 * m < n) {
-                const int trow = 16 * m + (lane & 15);
-                const int q2 = (lane >> 4) * 2;
-                const u32x4 lo = *reinterpret_cast<const u32x4*>(&tile[buf][trow * 128 + (((q2) ^ (trow & 7)) << 4)]);
-                const u32x4 hi = *reinterpret_cast<const u32x4*>(&tile[buf][trow * 128 + (((q2 + 1) ^ (trow & 7)) << 4)]);
-                const float sx = *reinterpret_cast<const float*>(&tile[buf][TM * 128 + trow * 4]);
-                const v8i tok = {int(lo[0]), int(lo[1]), int(lo[2]), int(lo[3]), int(hi[0]), int(hi[1]), int(hi[2]), int(hi[3])};
-                const float sc0 = __fmul_rn(s0, sx), sc1 = __fmul_rn(s1, sx);
+              const u32x4 lo = *reinterpret_cast<const u32x4*>(tb + tlo[m]);
+              const u32x4 hi = *reinterpret_cast<const u32x4*>(tb + thi[m]);
+              const float sx = *reinterpret_cast<const float*>(tb + tsx[m]);
+              const v8i tok = {int(lo[0]), int(lo[1]), int(lo[2]), int(lo[3]), int(hi[0]), int(hi[1]), int(hi[2]), int(hi[3])};
+              sc[m][0] = __fmul_rn(s0, sx);
+              sc[m][1] = __fmul_rn(s1, sx);
 #pragma unroll
-                for (int f = 0; f < 4; ++f) {
-                  const v8i wf = {int(w[s][f][0][0]), int(w[s][f][0][1]), int(w[s][f][0][2]), int(w[s][f][0][3]),
-                                  int(w[s][f][1][0]), int(w[s][f][1][1]), int(w[s][f][1][2]), int(w[s][f][1][3])};
-                  const v4f z = {0.0f, 0.0f, 0.0f, 0.0f};
-                  const v4f pr = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, tok, z, 0, 0, 0, 0, 0, 0);
-                  const float sc = (MODE == 0 && f >= 2) ? sc1 : sc0;
-#pragma unroll
-                  for (int r = 0; r < 4; ++r) acc[m][f][r] = __fmaf_rn(pr[r], sc, acc[m][f][r]);
-                }
+              for (int f = 0; f < 4; ++f) {
+                const v8i wf = {int(w[s][f][0][0]), int(w[s][f][0][1]), int(w[s][f][0][2]), int(w[s][f][0][3]),
+                                int(w[s][f][1][0]), int(w[s][f][1][1]), int(w[s][f][1][2]), int(w[s][f][1][3])};
+                const v4f z = {0.0f, 0.0f, 0.0f, 0.0f};
+                pr[m][f] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, tok, z, 0, 0, 0, 0, 0, 0);
               }
             }
-            // this slot's fragments are consumed: request K block kb + P into the same registers
+#pragma unroll
+            for (int m = 0; m < MF; ++m)
+#pragma unroll
+              for (int f = 0; f < 4; ++f)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[m][f][r] = __fmaf_rn(pr[m][f][r], sc[m][(MODE == 0 && f >= 2) ? 1 : 0], acc[m][f][r]);
+            // publish token tile kb+1 (requested one iteration ago)
+#pragma unroll
+            for (int i = 0; i < CPT; ++i)
+              if (stage_chunk) *reinterpret_cast<u32x4*>(&tile[(kb & 1) ^ 1][tdst[i]]) = tv[i];
+            if (tid < TM) *reinterpret_cast<float*>(&tile[(kb & 1) ^ 1][TM * 128 + tid * 4]) = tsv;
+            __syncthreads();
+            // request token tile kb+2, then K block kb+P of the weights into the slot just consumed
             {
+              const uint32_t kn = uint32_t(min(kb + 2, KB - 1));
+#pragma unroll
+              for (int i = 0; i < CPT; ++i) tv[i] = load16(tsrc[i] + kn * 128u);
+              tsv = load_global<float>(ssrc + kn);
               const uint32_t kw = uint32_t(min(kb + P, KB - 1));
 #pragma unroll
               for (int f = 0; f < 4; ++f) {
@@ -210,12 +243,6 @@ __global__ __launch_bounds__(256) void k_w8a8_grouped(const GemmParams p) {
                 w[s][f][1] = load16(wrow[f] + kw * 128u + 16u);
               }
             }
-            // publish the next token tile
-#pragma unroll
-            for (int i = 0; i < CPT; ++i)
-              if (stage_chunk) *reinterpret_cast<u32x4*>(&tile[buf ^ 1][tdst[i]]) = tv[i];
-            if (tid < TM) *reinterpret_cast<float*>(&tile[buf ^ 1][TM * 128 + tid * 4]) = tsv;
-            __syncthreads();
           }
         }
       }

@@ -265,12 +265,16 @@ class PrefillOps:
         take("perm", A * 4, torch.int32, (A,))
         return out
 
-    def contribute(self, x, ids, weights, active=None):
+    def contribute(self, x, ids, weights, active=None, stage=None):
+        """stage None = the whole call; 0..3 = one step (plan, gate/up, re-quantize, down)."""
         swiglu, limit, rw, wf32 = self.cfg
         a = capi.Prefill(self.rows, self.top_k, capi.ACT_FP8_BLOCK128, swiglu, limit, rw, wf32,
                          x.data_ptr(), ids.data_ptr(), active.data_ptr() if active is not None else None, weights.data_ptr(),
                          self.contributions.data_ptr(), self.done.data_ptr(), self.scratch.data_ptr(), self.scratch.numel())
-        capi.check(capi.lib().ffmoe_prefill_contribute(ctypes.byref(self._table_c), ctypes.byref(a), _stream()))
+        if stage is None:
+            capi.check(capi.lib().ffmoe_prefill_contribute(ctypes.byref(self._table_c), ctypes.byref(a), _stream()))
+        else:
+            capi.check(capi.lib().ffmoe_prefill_contribute_stage(ctypes.byref(self._table_c), ctypes.byref(a), stage, _stream()))
         return self.contributions
 
 

@@ -266,6 +266,10 @@ typedef struct ffmoe_prefill {
 
 uint64_t ffmoe_prefill_scratch_bytes(int rows, int top_k, int experts, int hidden, int inter);
 int ffmoe_prefill_contribute(const ffmoe_expert_table* table, const ffmoe_prefill* args, void* stream);
+/* One step of the same call, for timing a kernel alone (the steps of one cohort must run in order once before any of
+ * them is repeated): 0 = count / scan / fill + quantize x, 1 = gate/up GEMM + SwiGLU, 2 = re-quantize activations,
+ * 3 = down GEMM + routing weight + scatter. No counterpart in the reference. */
+int ffmoe_prefill_contribute_stage(const ffmoe_expert_table* table, const ffmoe_prefill* args, int stage, void* stream);
 
 #ifdef __cplusplus
 }
