@@ -35,6 +35,9 @@ def parse():
     ap.add_argument("--workload", choices=["decode", "prefill"], default="decode",
                     help="decode = BASELINE config 3 (the headline line); prefill = config 5 (4096 tokens, Zipf s=1.1, FP8 matrix cores)")
     ap.add_argument("--batch", type=int, default=None, help="tokens per step (decode: 1, 8, 64; prefill: 4096)")
+    ap.add_argument("--format", choices=["fp8", "nvfp4"], default="fp8",
+                    help="routed-expert format: fp8 = config 3 (shared expert FP8 too); nvfp4 = config 4 (NVFP4 routed experts, "
+                         "BF16 shared expert, quoted at --batch 32)")
     ap.add_argument("--experts", type=int, default=256)
     ap.add_argument("--ring", type=int, default=64, help="distinct token batches cycled through")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -50,20 +53,44 @@ def parse():
 def build_layer(args, torch, capi, ops, synth, make_tokens=True):
     H, I, E, K = 7168, 2048, args.experts, 8
     dev = "cuda"
-    table = ops.ExpertTable.allocate(capi.FMT_FP8_BLOCK128, E + 1, H, I, dev)
+    nvfp4 = args.format == "nvfp4"
+    if nvfp4:
+        table = ops.ExpertTable.allocate(capi.FMT_NVFP4, E, H, I, dev)
+        shared_table = ops.ExpertTable.allocate(capi.FMT_BF16, 1, H, I, dev)
+    else:
+        table = ops.ExpertTable.allocate(capi.FMT_FP8_BLOCK128, E + 1, H, I, dev)
+        shared_table = None
     for e in range(E + 1):
-        v = table.expert_views(e)
+        routed = e < E
+        v = table.expert_views(e) if (routed or not nvfp4) else shared_table.expert_views(0)
+        gl = []
         for i, shape in enumerate([(I, H), (I, H), (H, I)]):
             w = synth.normal(shape, 0.02, args.seed * 100003 + e * 3 + i, device=dev)
-            codes, scales = synth.quant_fp8_block(w)
-            v[2 * i].copy_(codes)
-            v[2 * i + 1].copy_(scales)
-    shared = table.shared_struct(E)
-    table.experts = E
-    router = synth.normal((E, H), 0.02, args.seed + 1, device=dev, dtype=torch.bfloat16)
-    bias = torch.zeros(E, dtype=torch.float32, device=dev)
+            if nvfp4 and routed:
+                codes, scales, g = synth.quant_nvfp4(w)
+                v[2 * i].copy_(codes)
+                v[2 * i + 1].copy_(scales)
+                gl.append(g)
+            elif nvfp4:
+                v[2 * i].copy_(w.to(torch.bfloat16))
+            else:
+                codes, scales = synth.quant_fp8_block(w)
+                v[2 * i].copy_(codes)
+                v[2 * i + 1].copy_(scales)
+        if nvfp4 and routed:
+            table.global_scales[e] = torch.tensor(gl, dtype=torch.float32)
+    if nvfp4:
+        shared = shared_table.shared_struct(0)
+        table.shared_table = shared_table  # keep the storage alive
+        table.shared_bytes = shared_table.weight_bytes_per_expert()
+    else:
+        shared = table.shared_struct(E)
+        table.experts = E
+        table.shared_bytes = table.weight_bytes_per_expert()
     if not make_tokens:
         return table, None, None, (H, I, E, K)
+    router = synth.normal((E, H), 0.02, args.seed + 1, device=dev, dtype=torch.bfloat16)
+    bias = torch.zeros(E, dtype=torch.float32, device=dev)
     layer = ops.NativeMoe(table, shared, router, bias, args.batch, K, routed_scaling=2.5, n_group=8, topk_group=4,
                           swiglu=capi.SWIGLU_TWICE, routed_weight=capi.WEIGHT_AFTER_DOWN_BF16, combine_mode=capi.COMBINE_UNGATED)
     xs = [synth.normal((args.batch, H), 1.0, args.seed + 1000 + i, device=dev, dtype=torch.bfloat16) for i in range(args.ring)]
@@ -73,15 +100,15 @@ def build_layer(args, torch, capi, ops, synth, make_tokens=True):
 def layer_bytes(table, distinct, rows, dims):
     H, I, E, K = dims
     per = table.weight_bytes_per_expert()
-    return (distinct + 1) * per + E * H * 2 + rows * H * 2 * (2 + K)
+    return distinct * per + table.shared_bytes + E * H * 2 + rows * H * 2 * (2 + K)
 
 
-def gate_up_bytes(distinct, rows, dims):
+def gate_up_bytes(table, distinct, rows, dims):
     """Algorithmic bytes of one gate/up launch: gate+up codes and scales of every expert touched (routed distinct
-    + shared), the token rows read and the activations written."""
+    + shared), the token rows read and the activations written. Gate and up are two thirds of an expert's bytes in
+    every format."""
     H, I, E, K = dims
-    per = 2 * I * H + 2 * 4 * (-(-I // 128)) * (-(-H // 128))
-    return (distinct + 1) * per + rows * H * 2 + rows * (K + 1) * I * 2
+    return (distinct * table.weight_bytes_per_expert() + table.shared_bytes) * 2 // 3 + rows * H * 2 + rows * (K + 1) * I * 2
 
 
 def cpu_baseline(args, torch, table, layer, xs, dims):
@@ -307,31 +334,34 @@ def main():
     kt = sorted(a.elapsed_time(b) * 1e3 / batch for a, b in ev)  # us per launch
     k_avg = sum(kt) / len(kt)
     mean_distinct_k = sum(distinct) / len(distinct)
-    k_bytes = gate_up_bytes(mean_distinct_k, args.batch, dims)
+    k_bytes = gate_up_bytes(table, mean_distinct_k, args.batch, dims)
     achieved = k_bytes / (k_avg * 1e-6) / 1e9
 
     out = {
         "metric": "moe_layer_decode_us", "value": us_per_layer, "unit": "us/layer", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": us_per_layer / 1e3,
-        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "fp8_e4m3 weights, bf16 activations, f32 accumulate",
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": ("fp8_e4m3" if args.format == "fp8" else "nvfp4 (e2m1 + e4m3 group scales)") + " weights, bf16 activations, f32 accumulate",
         "data": "synthetic",
-        "config": {"workload": "DeepSeek-V3-shape FP8 MoE decode layer (BASELINE config 3), batch %d" % args.batch,
+        "config": {"workload": ("DeepSeek-V3-shape FP8 MoE decode layer (BASELINE config 3), batch %d" % args.batch) if args.format == "fp8" else
+                               ("DeepSeek-V3-shape MoE decode layer, NVFP4 routed experts + BF16 shared expert (BASELINE config 4), batch %d" % args.batch),
                    "hidden": H, "intermediate": I, "experts": E, "shared_experts": 1, "top_k": K,
                    "routing": "sigmoid grouped top-8 (8 groups, keep 4), renormalised x2.5",
-                   "weights": "E4M3 + f32 128x128 block scales", "act_mode": "FFMOE_ACT_BF16 (W8A16)",
+                   "weights": "E4M3 + f32 128x128 block scales" if args.format == "fp8" else "E2M1 pairs + E4M3 scale per 16 + f32 global",
+                   "act_mode": "FFMOE_ACT_BF16 (W8A16)" if args.format == "fp8" else "BF16 activations (W4A16)",
                    "batch": args.batch, "ring": len(xs), "launch": "eager" if graphs is None else "hip graph per ring slot"},
         "tokens_per_s": args.batch / (us_per_layer * 1e-6),
         "distinct_routed_experts": mean_distinct,
         "layer_bytes": bytes_layer,
         "layer_hbm_gbps": bytes_layer / (us_per_layer * 1e-6) / 1e9,
         "layer_hbm_frac": bytes_layer / (us_per_layer * 1e-6) / 1e9 / HBM_PEAK_GBPS,
-        "roofline": {"kernel": "ffmoe::k_decode_stage<FmtFp8, S, 0, RG, 1> (gate/up + SwiGLU stage of ffmoe_decode_contribute)",
+        "roofline": {"kernel": "ffmoe::k_decode_stage<%s, S, 0, RG, NR> (gate/up + SwiGLU stage of ffmoe_decode_contribute)" % ("FmtFp8" if args.format == "fp8" else "FmtNvfp4"),
                      "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBPS, "traffic": GATE_UP_TRAFFIC_BYTES.get((args.batch, args.experts)),
+                     "frac": achieved / HBM_PEAK_GBPS, "traffic": GATE_UP_TRAFFIC_BYTES.get((args.batch, args.experts)) if args.format == "fp8" else None,
                      "bytes_per_launch": k_bytes, "avg_us": k_avg, "min_us": kt[0], "median_us": kt[len(kt) // 2],
                      "launches_timed": nb * batch},
     }
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and args.format == "fp8":
         out["cpu_baseline"] = cpu_baseline(args, torch, table, layer, xs, dims)
     print(json.dumps(out))
 

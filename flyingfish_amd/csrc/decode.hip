@@ -84,11 +84,16 @@ extern "C" __attribute__((visibility("default"))) uint64_t ffmoe_decode_scratch_
   return h + groups + 256;
 }
 
+// layout_k >= 0: the call processes args->top_k choices per row (0 = the shared expert only) but lays the scratch
+// arena out for layout_k choices, so a routed pass and a shared pass of another weight format can share one arena.
+// Pass 1 keeps its group descriptors and counters behind those of pass 0: the passes may be issued stage by stage
+// (both gate/up launches, then both down launches), so neither may overwrite the other's grouping.
 static int decode_impl(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared, const ffmoe_decode* args,
-                       int stage_mask, void* stream) {
+                       int stage_mask, void* stream, int layout_k = -1, int pass = 0) {
   FF_REQUIRE(table && args, FFMOE_ERR_NULL, "table/args is NULL");
   const int R = args->rows, K = args->top_k, E = table->experts, H = table->hidden, I = table->inter;
-  FF_REQUIRE(R >= 1 && K >= 1 && K <= FFMOE_MAX_TOP_K && E >= 1 && E <= FFMOE_MAX_EXPERTS, FFMOE_ERR_SHAPE,
+  const int LK = layout_k < 0 ? K : layout_k;
+  FF_REQUIRE(R >= 1 && K >= 0 && (K >= 1 || shared) && K <= FFMOE_MAX_TOP_K && LK >= K && E >= 1 && E <= FFMOE_MAX_EXPERTS, FFMOE_ERR_SHAPE,
              "decode rows=%d top_k=%d experts=%d out of range", R, K, E);
   FF_REQUIRE((long long)R * K <= FFMOE_DECODE_MAX_ASSIGN, FFMOE_ERR_SHAPE,
              "decode handles at most %d assignments per call (got %lld); use ffmoe_prefill_contribute", FFMOE_DECODE_MAX_ASSIGN,
@@ -110,7 +115,7 @@ static int decode_impl(const ffmoe_expert_table* table, const ffmoe_shared_exper
              args->routed_weight);
   FF_PTR16(args->x); FF_PTR4(args->ids); FF_PTR16(args->contributions); FF_PTR16(table->slots);
   if (args->weights_f32) { FF_PTR4(args->weights); } else { FF_PTR2(args->weights); }
-  if (fmt == FFMOE_FMT_NVFP4) FF_PTR4(table->global_scales);
+  if (fmt == FFMOE_FMT_NVFP4 && K > 0) FF_PTR4(table->global_scales);
   int SI = I;
   if (shared) {
     FF_REQUIRE(shared->format == fmt, FFMOE_ERR_UNSUPPORTED, "shared expert format %d differs from the table format %d",
@@ -121,7 +126,7 @@ static int decode_impl(const ffmoe_expert_table* table, const ffmoe_shared_exper
     for (int i = 0; i < 6; i += 2)
       FF_REQUIRE(shared->slot[i] != 0 && shared->slot[i] % 16 == 0, FFMOE_ERR_ALIGN, "shared expert slot[%d] is NULL or misaligned", i);
   }
-  const uint64_t need = ffmoe_decode_scratch_bytes(R, K, E, H, I, shared ? SI : 0);
+  const uint64_t need = ffmoe_decode_scratch_bytes(R, LK > 0 ? LK : 1, E, H, I, shared ? SI : 0);
   FF_PTR_ALIGNED(args->scratch, 256);
   FF_REQUIRE(args->scratch_bytes >= need, FFMOE_ERR_SCRATCH, "decode scratch holds %llu bytes, %llu needed",
              (unsigned long long)args->scratch_bytes, (unsigned long long)need);
@@ -158,9 +163,10 @@ static int decode_impl(const ffmoe_expert_table* table, const ffmoe_shared_exper
   for (int i = 0; i < 3; ++i) p.shared_global[i] = shared ? shared->global_scales[i] : 1.0f;
   p.contributions = (uint16_t*)args->contributions; p.shared_out = (uint16_t*)args->shared_out; p.done = args->done;
   uint8_t* sc = (uint8_t*)args->scratch;
-  p.h = (uint16_t*)sc;
+  const size_t LA = size_t(R) * LK;
+  p.h = (uint16_t*)sc + (LA - A) * imax;  // slot s of this call -> arena row (LA - A) + s
   p.h_stride = imax;
-  const uint64_t hbytes = ((uint64_t(A) + R) * imax * 2 + 255) & ~uint64_t(255);
+  const uint64_t hbytes = ((uint64_t(LA) + R) * imax * 2 + 255) & ~uint64_t(255);
   hipStream_t st = (hipStream_t)stream;
   int rg = 1;
   // LDS budget per block: rg rows of the widest contraction; two blocks per CU must fit in 160 KiB
@@ -169,9 +175,9 @@ static int decode_impl(const ffmoe_expert_table* table, const ffmoe_shared_exper
     while (rg > 1 && size_t(rg) * kmax_lds * 2 > 64 * 1024) rg >>= 1;
   }
   if (rg > 1) {
-    p.groups = (GroupDesc*)(sc + hbytes);
-    const uint64_t max_groups = uint64_t(A) + R + 2;
-    p.counters = (int*)(sc + hbytes + ((max_groups * sizeof(GroupDesc) + 255) & ~uint64_t(255)));
+    p.groups = (GroupDesc*)(sc + hbytes) + (pass ? LA + 1 : 0);
+    const uint64_t max_groups = uint64_t(LA) + R + 2;
+    p.counters = (int*)(sc + hbytes + ((max_groups * sizeof(GroupDesc) + 255) & ~uint64_t(255))) + 2 * pass;
     if (stage_mask & 1) hipLaunchKernelGGL(k_group_assignments, dim3(1), dim3(1024), A * sizeof(int), st, args->ids, args->active, table->valid, p.groups,
                        p.counters, R, K, E, p.has_shared, rg);
     FF_TRY(ff_launch_status());
@@ -186,13 +192,28 @@ static int decode_impl(const ffmoe_expert_table* table, const ffmoe_shared_exper
   }
 }
 
+// A shared expert stored in another weight format than the routed experts (NVFP4 experts next to a BF16 shared expert)
+// runs as two passes over one arena: the routed choices with the table's kernels, then the shared expert alone with the
+// kernels of its own format.
+static int decode_dispatch(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared, const ffmoe_decode* args,
+                           int stage_mask, void* stream) {
+  if (!table || !args || !shared || shared->format == table->format) return decode_impl(table, shared, args, stage_mask, stream);
+  FF_TRY(decode_impl(table, nullptr, args, stage_mask, stream, args->top_k));
+  ffmoe_expert_table as_shared = *table;
+  as_shared.format = shared->format;
+  ffmoe_decode only_shared = *args;
+  only_shared.top_k = 0;
+  only_shared.done = nullptr;
+  return decode_impl(&as_shared, shared, &only_shared, stage_mask, stream, args->top_k, 1);
+}
+
 extern "C" __attribute__((visibility("default"))) int ffmoe_decode_contribute(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared,
                                        const ffmoe_decode* args, void* stream) {
-  return decode_impl(table, shared, args, 3, stream);
+  return decode_dispatch(table, shared, args, 3, stream);
 }
 
 extern "C" __attribute__((visibility("default"))) int ffmoe_decode_contribute_stage(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared,
                                              const ffmoe_decode* args, int stage, void* stream) {
   FF_REQUIRE(stage == 0 || stage == 1, FFMOE_ERR_SHAPE, "decode stage %d is neither 0 (gate/up) nor 1 (down)", stage);
-  return decode_impl(table, shared, args, 1 << stage, stream);
+  return decode_dispatch(table, shared, args, 1 << stage, stream);
 }

@@ -3,6 +3,7 @@
 // and the slab inner loop (weights in registers x activations in LDS, v_dot2 accumulation).
 #pragma once
 #include "common.cuh"
+#include <type_traits>
 
 namespace ffmoe {
 
@@ -66,6 +67,40 @@ struct FmtNvfp4 {
       }
     }
   }
+  // Split form of the same weights. An E2M1 magnitude is 2^j or 1.5 * 2^j, and scaling by a power of two commutes
+  // with both roundings, so bf16(e2m1 * s) is exactly 2^j * b1 or 2^j * b15 with b1 = bf16(s), b15 = bf16(f32(1.5 s)).
+  // With m = the raw E2M1 value and u = m with its mantissa bit cleared (2^j for both classes),
+  //     sum x * w  =  c1 * sum x*u  +  c2 * sum x*m,     c1 = 3 b1 - 2 b15,   c2 = 2 (b15 - b1)
+  // (a 2^j element contributes x u (c1 + c2) = x u b1, a 1.5 * 2^j element x u (c1 + 1.5 c2) = x u b15). c1 and c2
+  // are exact in FP32, m and u are exact BF16 values straight from the hardware FP4 conversion, so per element
+  // this costs one conversion, one AND and two dot2 lanes instead of a multiply and a rounding per weight.
+  struct Split { uint32_t m[16], u[16]; float c1[2], c2[2]; };
+  static __device__ __forceinline__ void split(const Chunk& c, Split& o, bool valid) {
+    const f32x2 sc = e4m3x2_to_f32<false>(c.scales);
+    const float gl = valid ? c.global : 0.0f;
+#pragma unroll
+    for (int g = 0; g < 2; ++g) {
+      const float s = __fmul_rn(g == 0 ? sc.x : sc.y, gl);
+      const float b1 = bround(s), b15 = bround(__fmul_rn(1.5f, s));
+      o.c1[g] = __fsub_rn(__fmul_rn(3.0f, b1), __fmul_rn(2.0f, b15));
+      o.c2[g] = __fmul_rn(2.0f, __fsub_rn(b15, b1));
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const uint32_t d = c.codes[q];
+      // byte i of the dword: low nibble = even k -> low half of the pair
+      const bf16x2 p0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(d, 1.0f, 0);
+      const bf16x2 p1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(d, 1.0f, 1);
+      const bf16x2 p2 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(d, 1.0f, 2);
+      const bf16x2 p3 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(d, 1.0f, 3);
+      o.m[4 * q + 0] = __builtin_bit_cast(uint32_t, p0);
+      o.m[4 * q + 1] = __builtin_bit_cast(uint32_t, p1);
+      o.m[4 * q + 2] = __builtin_bit_cast(uint32_t, p2);
+      o.m[4 * q + 3] = __builtin_bit_cast(uint32_t, p3);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o.u[4 * q + i] = o.m[4 * q + i] & 0xffbfffbfu;
+    }
+  }
 };
 
 struct FmtBf16 {
@@ -95,6 +130,38 @@ __device__ __forceinline__ void step_compute(const typename F::Chunk (&c)[NROWS]
                                              int chunk, int n, float (&acc)[NROWS][RG]) {
   const bool valid = chunk < nchunks;
   const int cl = valid ? chunk : 0;  // keep the LDS read in range
+  if constexpr (std::is_same<F, FmtNvfp4>::value) {
+    // two groups of 16 per chunk, each with its own pair of constants (see FmtNvfp4::split)
+    FmtNvfp4::Split w[NROWS];
+#pragma unroll
+    for (int m = 0; m < NROWS; ++m) FmtNvfp4::split(c[m][s], w[m], valid);
+#pragma unroll
+    for (int r = 0; r < RG; ++r) {
+      if (RG == 1 || r < n) {
+        const u32x4* xp = reinterpret_cast<const u32x4*>(xs + size_t(r) * K * 2 + size_t(cl) * 64);
+#pragma unroll
+        for (int g = 0; g < 2; ++g) {
+          const u32x4 xa = xp[2 * g], xb = xp[2 * g + 1];
+#pragma unroll
+          for (int m = 0; m < NROWS; ++m) {
+            float sm = 0.0f, su = 0.0f;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              sm = dot2_bf16(w[m].m[8 * g + q], xa[q], sm);
+              su = dot2_bf16(w[m].u[8 * g + q], xa[q], su);
+            }
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              sm = dot2_bf16(w[m].m[8 * g + 4 + q], xb[q], sm);
+              su = dot2_bf16(w[m].u[8 * g + 4 + q], xb[q], su);
+            }
+            acc[m][r] = __fmaf_rn(su, w[m].c1[g], __fmaf_rn(sm, w[m].c2[g], acc[m][r]));
+          }
+        }
+      }
+    }
+    return;
+  }
   uint32_t w[NROWS][F::EPL / 2];
 #pragma unroll
   for (int m = 0; m < NROWS; ++m) F::dequant(c[m][s], w[m], valid);

@@ -244,6 +244,35 @@ def test_decode_bf16_experts(rows):
     _run_decode(capi.FMT_BF16, 5, 1024, 256, rows, 2, 71, True)
 
 
+@pytest.mark.parametrize("rows,routed_fmt,shared_fmt", [(1, capi.FMT_NVFP4, capi.FMT_BF16), (6, capi.FMT_NVFP4, capi.FMT_BF16),
+                                                        (3, capi.FMT_FP8_BLOCK128, capi.FMT_BF16)])
+def test_decode_shared_expert_in_another_format(rows, routed_fmt, shared_fmt):
+    """BASELINE config 4: NVFP4 routed experts next to a BF16 shared expert (two passes over one scratch arena)."""
+    experts, hidden, inter, top_k, seed = 6, 1024, 512, 3, 91
+    table, ref = make_table(routed_fmt, experts, hidden, inter, seed)
+    stable, sref = make_table(shared_fmt, 1, hidden, inter, seed + 1)
+    sh = stable.shared_struct(0)
+    x = rand_bf16((rows, hidden), 1.0, seed + 7)
+    g = synth.generator(seed + 8)
+    ids = torch.stack([torch.randperm(experts, generator=g)[:top_k] for _ in range(rows)]).to(torch.int32)
+    wt = (torch.rand((rows, top_k), generator=g) * 0.5 + 0.05).to(torch.bfloat16)
+    op = DecodeOps(table, sh, rows, top_k, capi.ACT_BF16, capi.SWIGLU_TWICE, 0.0, capi.WEIGHT_AFTER_DOWN_BF16, False)
+    contrib, shared_out = op.contribute(x.to(DEV), ids.to(DEV), wt.to(DEV))
+    torch.cuda.synchronize()
+    want = oracle_contributions(ref, bits(x), ids.numpy(), wt.float().numpy(), capi.SWIGLU_TWICE, 0.0, capi.WEIGHT_AFTER_DOWN_BF16)
+    assert_close_bf16(bits(contrib), want, "contributions")
+    assert_close_bf16(bits(shared_out), oracle_shared(sref[0], bits(x), capi.SWIGLU_TWICE, 0.0), "shared_out")
+    assert np.all(op.done.cpu().numpy() != 0)
+    # the two stages may also be issued one by one
+    c0 = bits(contrib).copy()
+    s0 = bits(shared_out).copy()
+    op.contributions.zero_(); op.shared_out.zero_()
+    op.contribute(x.to(DEV), ids.to(DEV), wt.to(DEV), stage=0)
+    op.contribute(x.to(DEV), ids.to(DEV), wt.to(DEV), stage=1)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(op.contributions), c0) and np.array_equal(bits(op.shared_out), s0)
+
+
 def test_decode_dsv3_width_single_token():
     # hidden 7168 / inter 2048 at DeepSeek-V3 width, 3 routed experts + shared, one token
     _run_decode(capi.FMT_FP8_BLOCK128, 3, 7168, 2048, 1, 3, 81, True)
