@@ -248,7 +248,7 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
 // flight per weight row (one slab); rows longer than the format's cap take several slabs. The caps keep every
 // instantiation inside the register file without spills: stage 0 holds 2 weight rows per unit, stage 1 holds
 // Policy::NR1 rows; with several rows of a group per pass (RG > 1) the cap is halved.
-template <class F> struct Policy { static constexpr int S0 = 8, S0G = 4, NR1 = 4, NR1G = 4, S1 = 2, S1G = 2; };
+template <class F> struct Policy { static constexpr int S0 = 8, S0G = 8, NR1 = 4, NR1G = 4, S1 = 2, S1G = 2; };
 template <> struct Policy<FmtNvfp4> { static constexpr int S0 = 4, S0G = 2, NR1 = 4, NR1G = 2, S1 = 2, S1G = 1; };
 
 inline int decode_num_cus() {

@@ -178,12 +178,12 @@ class RouteOps:
         return ids, weights
 
     @staticmethod
-    def route(x, router, top_k, score=capi.SCORE_SOFTMAX):
+    def route(x, router, top_k, score=capi.SCORE_SOFTMAX, logits=None, ids=None, weights=None):
         rows, hidden = x.shape
         experts = router.shape[0]
-        logits = torch.empty((rows, experts), dtype=_BF16, device=x.device)
-        ids = torch.empty((rows, top_k), dtype=torch.int32, device=x.device)
-        w = torch.empty((rows, top_k), dtype=_BF16, device=x.device)
+        logits = logits if logits is not None else torch.empty((rows, experts), dtype=_BF16, device=x.device)
+        ids = ids if ids is not None else torch.empty((rows, top_k), dtype=torch.int32, device=x.device)
+        w = weights if weights is not None else torch.empty((rows, top_k), dtype=_BF16, device=x.device)
         capi.check(capi.lib().ffmoe_route_decode(_ptr(_dense(x, "x")), _ptr(_dense(router, "router")), _ptr(logits), _ptr(ids), _ptr(w),
                                                  rows, experts, hidden, top_k, score, _stream()))
         return ids, w, logits
