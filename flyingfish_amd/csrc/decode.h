@@ -37,4 +37,13 @@ struct DecodeParams {
   int* counters;            // {routed groups, shared groups} when groups != NULL
 };
 
+// one-token finish (down + routing weight + combine in one launch)
+struct FinishParams {
+  DecodeParams d;
+  const uint16_t* scale;  // [1] BF16 shared-expert gate (FFMOE_COMBINE_GATED)
+  uint16_t* y;            // [hidden]
+  uint32_t* status;       // |= 1 when a live choice names an expert that is out of range or not valid
+  int mode;               // FFMOE_COMBINE_*
+};
+
 }  // namespace ffmoe

@@ -5,9 +5,13 @@
 #include "decode.h"
 
 namespace ffmoe {
+
 int decode_launch_fp8(const DecodeParams& p, int rg, int stage_mask, hipStream_t st);
 int decode_launch_nvfp4(const DecodeParams& p, int rg, int stage_mask, hipStream_t st);
 int decode_launch_bf16(const DecodeParams& p, int rg, int stage_mask, hipStream_t st);
+int decode_finish_fp8(const FinishParams& q, hipStream_t st);
+int decode_finish_nvfp4(const FinishParams& q, hipStream_t st);
+int decode_finish_bf16(const FinishParams& q, hipStream_t st);
 }  // namespace ffmoe
 
 namespace ffmoe {
@@ -89,7 +93,7 @@ extern "C" __attribute__((visibility("default"))) uint64_t ffmoe_decode_scratch_
 // Pass 1 keeps its group descriptors and counters behind those of pass 0: the passes may be issued stage by stage
 // (both gate/up launches, then both down launches), so neither may overwrite the other's grouping.
 static int decode_impl(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared, const ffmoe_decode* args,
-                       int stage_mask, void* stream, int layout_k = -1, int pass = 0) {
+                       int stage_mask, void* stream, int layout_k = -1, int pass = 0, const FinishParams* fin = nullptr) {
   FF_REQUIRE(table && args, FFMOE_ERR_NULL, "table/args is NULL");
   const int R = args->rows, K = args->top_k, E = table->experts, H = table->hidden, I = table->inter;
   const int LK = layout_k < 0 ? K : layout_k;
@@ -185,6 +189,15 @@ static int decode_impl(const ffmoe_expert_table* table, const ffmoe_shared_exper
     p.groups = nullptr;
     p.counters = nullptr;
   }
+  if (fin) {
+    FinishParams q = *fin;
+    q.d = p;
+    switch (fmt) {
+      case FFMOE_FMT_FP8_BLOCK128: return decode_finish_fp8(q, st);
+      case FFMOE_FMT_NVFP4: return decode_finish_nvfp4(q, st);
+      default: return decode_finish_bf16(q, st);
+    }
+  }
   switch (fmt) {
     case FFMOE_FMT_FP8_BLOCK128: return decode_launch_fp8(p, rg, stage_mask, st);
     case FFMOE_FMT_NVFP4: return decode_launch_nvfp4(p, rg, stage_mask, st);
@@ -216,4 +229,25 @@ extern "C" __attribute__((visibility("default"))) int ffmoe_decode_contribute_st
                                              const ffmoe_decode* args, int stage, void* stream) {
   FF_REQUIRE(stage == 0 || stage == 1, FFMOE_ERR_SHAPE, "decode stage %d is neither 0 (gate/up) nor 1 (down)", stage);
   return decode_dispatch(table, shared, args, 1 << stage, stream);
+}
+
+extern "C" __attribute__((visibility("default"))) int ffmoe_decode_finish(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared,
+                                                                         const ffmoe_decode* args, const void* scale, void* y, uint32_t* status,
+                                                                         int combine_mode, void* stream) {
+  FF_REQUIRE(table && args, FFMOE_ERR_NULL, "table/args is NULL");
+  FF_REQUIRE(args->rows == 1, FFMOE_ERR_UNSUPPORTED, "ffmoe_decode_finish handles one token row (rows=%d)", args->rows);
+  FF_REQUIRE(!shared || shared->format == table->format, FFMOE_ERR_UNSUPPORTED, "ffmoe_decode_finish needs the shared expert in the table's format");
+  FF_REQUIRE(!shared || shared->inter == table->inter, FFMOE_ERR_UNSUPPORTED, "ffmoe_decode_finish needs shared inter == inter");
+  FF_REQUIRE(combine_mode >= 0 && combine_mode <= FFMOE_COMBINE_ROUTED, FFMOE_ERR_UNSUPPORTED, "unknown combine mode %d", combine_mode);
+  FF_REQUIRE(shared || combine_mode == FFMOE_COMBINE_ROUTED, FFMOE_ERR_SHAPE, "combine mode %d needs a shared expert", combine_mode);
+  FF_PTR16(y);
+  if (combine_mode == FFMOE_COMBINE_GATED) FF_PTR2(scale);
+  if (status) FF_PTR4(status);
+  FF_NO_OVERLAP(y, size_t(table->hidden) * 2, args->scratch, args->scratch_bytes);
+  FF_NO_OVERLAP(y, size_t(table->hidden) * 2, args->x, size_t(table->hidden) * 2);
+  FinishParams fin{};
+  fin.scale = (const uint16_t*)scale; fin.y = (uint16_t*)y; fin.status = status; fin.mode = combine_mode;
+  // the shared expert takes part only in the modes that add it
+  const ffmoe_shared_expert* sh = combine_mode == FFMOE_COMBINE_ROUTED ? nullptr : shared;
+  return decode_impl(table, sh, args, 0, stream, -1, 0, &fin);
 }

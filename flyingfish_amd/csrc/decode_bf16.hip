@@ -1,6 +1,7 @@
 // Decode stages for FmtBf16 experts.
-#include "decode_kernel.cuh"
+#include "finish_kernel.cuh"
 
 namespace ffmoe {
 int decode_launch_bf16(const DecodeParams& p, int rg, int stage_mask, hipStream_t st) { return launch_format<FmtBf16>(p, rg, stage_mask, st); }
+int decode_finish_bf16(const FinishParams& q, hipStream_t st) { return launch_finish<FmtBf16>(q, st); }
 }  // namespace ffmoe

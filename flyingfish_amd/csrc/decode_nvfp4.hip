@@ -1,6 +1,7 @@
 // Decode stages for FmtNvfp4 experts.
-#include "decode_kernel.cuh"
+#include "finish_kernel.cuh"
 
 namespace ffmoe {
 int decode_launch_nvfp4(const DecodeParams& p, int rg, int stage_mask, hipStream_t st) { return launch_format<FmtNvfp4>(p, rg, stage_mask, st); }
+int decode_finish_nvfp4(const FinishParams& q, hipStream_t st) { return launch_finish<FmtNvfp4>(q, st); }
 }  // namespace ffmoe

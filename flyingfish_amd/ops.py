@@ -221,6 +221,21 @@ class DecodeOps:
             capi.check(capi.lib().ffmoe_decode_contribute_stage(ctypes.byref(self._table_c), sh, ctypes.byref(d), stage, _stream()))
         return self.contributions, self.shared_out
 
+    def finish(self, x, ids, weights, mode, y, status=None, scale=None, active=None):
+        """rows == 1: down + routing weight + ordered combine in one launch, after contribute(stage=0) on the same
+        arguments. Returns False (nothing launched) when the shape is outside the fast path."""
+        act_mode, swiglu, limit, rw, wf32 = self.cfg
+        d = capi.Decode(self.rows, self.top_k, act_mode, swiglu, limit, rw, wf32,
+                        x.data_ptr(), ids.data_ptr(), active.data_ptr() if active is not None else None, weights.data_ptr(),
+                        self.contributions.data_ptr(), self.shared_out.data_ptr() if self.shared_out is not None else None,
+                        self.done.data_ptr(), self.scratch.data_ptr(), self.scratch.numel())
+        sh = ctypes.byref(self._shared_c) if self._shared_c is not None else None
+        rc = capi.lib().ffmoe_decode_finish(ctypes.byref(self._table_c), sh, ctypes.byref(d), _ptr(scale), _ptr(y), _ptr(status), mode, _stream())
+        if rc == capi.ERR_UNSUPPORTED:
+            return False
+        capi.check(rc)
+        return True
+
 
 class PrefillOps:
     """Expert contributions for a prefill cohort (many rows): device-side grouping by expert and two grouped W8A8
@@ -374,11 +389,23 @@ class NativeMoe:
         self.weights = torch.empty((rows, top_k), dtype=torch.float32, device=dev)
         self.y = torch.empty((rows, table.hidden), dtype=_BF16, device=dev)
         self.status = torch.zeros(1, dtype=torch.int32, device=dev)
+        # one-token finish in a single launch (ffmoe_decode_finish). Off by default: on MI355X it measured 33 us
+        # against 26 + 4.6 us for the separate down and combine launches at the DeepSeek-V3 shape.
+        self.fused_finish = False
 
     def run(self, x):
         scaling, ng, kg = self.routing
         RouteOps.route_noaux(x, self.router, self.bias, self.top_k, self.logits, self.ids, self.weights,
                              done=self.decode.done, routed_scaling=scaling, n_group=ng, topk_group=kg)
-        contrib, shared_out = self.decode.contribute(x, self.ids, self.weights)
+        if self.rows == 1 and self.fused_finish:
+            # one token: gate/up launch, then down + weighting + combine in a single launch
+            self.decode.contribute(x, self.ids, self.weights, stage=0)
+            mode = self.combine_mode if self.decode.shared_out is not None else capi.COMBINE_ROUTED
+            if self.decode.finish(x, self.ids, self.weights, mode, self.y, status=self.status):
+                return self.y
+            self.fused_finish = False
+            contrib, shared_out = self.decode.contribute(x, self.ids, self.weights, stage=1)
+        else:
+            contrib, shared_out = self.decode.contribute(x, self.ids, self.weights)
         mode = self.combine_mode if shared_out is not None else capi.COMBINE_ROUTED
         return CombineOps.combine(contrib, shared_out, self.ids, mode, done=self.decode.done, status=self.status, out=self.y)

@@ -187,6 +187,20 @@ int ffmoe_decode_contribute(const ffmoe_expert_table* table, const ffmoe_shared_
 int ffmoe_decode_contribute_stage(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared,
                                   const ffmoe_decode* args, int stage, void* stream);
 
+/* One-token finish: the down projection of every live choice and of the shared expert, the routing weight and the
+ * ordered combine in ONE launch, for rows == 1. Call after ffmoe_decode_contribute_stage(table, shared, args, 0, stream)
+ * with the same table / shared / args (the gate/up activations are taken from args->scratch); writes y[hidden] and
+ * nothing else (contributions, shared_out and done stay untouched). y is bit-identical to
+ * ffmoe_decode_contribute_stage(.., 1, ..) followed by ffmoe_combine(mode): it replaces moe_down + moe_ffn_weight_f32 +
+ * moe_combine{,_ungated,_bf16,_accum,_routed} (kernels/moe_ffn.cu:211-302,894-908; kernels/moe_combine.cu:51-116,
+ * 541-613) of NativeMoe::run (src/backend/cuda/moe/decode.rs:1187-1297). args->active plays the role of final_active;
+ * *status |= 1 when a live choice names an expert that is out of range or not valid.
+ * Returns FFMOE_ERR_UNSUPPORTED (nothing launched) when the shape is outside the fast path (rows != 1, more than 9
+ * groups, shared expert of another format or width, rows of the down matrix longer than two 64-lane steps): run the
+ * two separate calls then. */
+int ffmoe_decode_finish(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared, const ffmoe_decode* args,
+                        const void* scale, void* y, uint32_t* status, int combine_mode, void* stream);
+
 /* ------------------------------------------------------------------------------------------------
  * Standalone linears, M <= 16 "skinny" and beyond. y[M,N] = x[M,K] * W[N,K]^T, BF16 in / BF16 out.
  */

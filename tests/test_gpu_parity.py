@@ -273,6 +273,78 @@ def test_decode_shared_expert_in_another_format(rows, routed_fmt, shared_fmt):
     assert np.array_equal(bits(op.contributions), c0) and np.array_equal(bits(op.shared_out), s0)
 
 
+@pytest.mark.parametrize("fmt,hidden,inter,top_k,shared", [
+    (capi.FMT_FP8_BLOCK128, 1024, 512, 8, True),     # 9 groups, one step per row
+    (capi.FMT_FP8_BLOCK128, 512, 2048, 3, True),     # 4 groups, two steps per row
+    (capi.FMT_FP8_BLOCK128, 1024, 384, 4, False),    # routed only
+    (capi.FMT_NVFP4, 1024, 512, 6, True),
+    (capi.FMT_BF16, 1024, 256, 2, True),
+])
+def test_decode_finish_equals_down_plus_combine(fmt, hidden, inter, top_k, shared):
+    """One-token finish (one launch) against the separate down and combine launches: bit-identical y in every
+    combine mode, with and without inactive choices; oracle parity of the separate path is covered above."""
+    experts, seed = 10, 97
+    table, ref = make_table(fmt, experts + (1 if shared else 0), hidden, inter, seed)
+    sh = table.shared_struct(experts) if shared else None
+    table.experts = experts
+    x = rand_bf16((1, hidden), 1.0, seed + 7).to(DEV)
+    g = synth.generator(seed + 8)
+    ids = torch.randperm(experts, generator=g)[:top_k].to(torch.int32).view(1, top_k).to(DEV)
+    wt = (torch.rand((1, top_k), generator=g) * 0.5 + 0.05).to(DEV)
+    scale = rand_bf16((1,), 0.5, seed + 9).to(DEV)
+    modes = [capi.COMBINE_ROUTED] if not shared else [capi.COMBINE_GATED, capi.COMBINE_UNGATED, capi.COMBINE_BF16,
+                                                      capi.COMBINE_ACCUM_FP32, capi.COMBINE_ACCUM_BF16]
+    for with_active in (False, True):
+        active = None
+        if with_active:
+            a = torch.ones((1, top_k), dtype=torch.int32)
+            a[0, 0] = 0
+            a[0, top_k - 1] = 0 if top_k > 2 else 1
+            active = a.to(DEV)
+        op = DecodeOps(table, sh, 1, top_k, capi.ACT_BF16, capi.SWIGLU_TWICE, 0.0, capi.WEIGHT_AFTER_DOWN_BF16, True)
+        op.done.zero_()
+        op.contributions.zero_()  # the accumulate modes add every slot, live or not: skipped slots must read as zero
+        contrib, shared_out = op.contribute(x, ids, wt, active)
+        for mode in modes:
+            want = CombineOps.combine(contrib, shared_out, ids, mode, scale=scale, done=op.done, final_active=active)
+            y = torch.full((1, hidden), 7.0, dtype=torch.bfloat16, device=DEV)
+            status = torch.zeros(1, dtype=torch.int32, device=DEV)
+            op.contribute(x, ids, wt, active, stage=0)
+            assert op.finish(x, ids, wt, mode, y, status=status, scale=scale, active=active)
+            torch.cuda.synchronize()
+            assert int(status.item()) == 0
+            assert np.array_equal(bits(y), bits(want)), "mode %d active %s" % (mode, with_active)
+
+
+def test_decode_finish_flags_bad_expert_and_declines_unsupported_shapes():
+    table, _ = make_table(capi.FMT_FP8_BLOCK128, 5, 512, 256, 5)
+    sh = table.shared_struct(4)
+    table.experts = 4
+    x = rand_bf16((1, 512), 1.0, 3).to(DEV)
+    ids = torch.tensor([[1, 9, 2]], dtype=torch.int32, device=DEV)  # 9 is out of range
+    wt = torch.full((1, 3), 0.25, device=DEV)
+    op = DecodeOps(table, sh, 1, 3, capi.ACT_BF16, capi.SWIGLU_TWICE, 0.0, capi.WEIGHT_AFTER_DOWN_BF16, True)
+    op.contribute(x, ids, wt, stage=0)
+    y = torch.zeros((1, 512), dtype=torch.bfloat16, device=DEV)
+    status = torch.zeros(1, dtype=torch.int32, device=DEV)
+    assert op.finish(x, ids, wt, capi.COMBINE_UNGATED, y, status=status)
+    torch.cuda.synchronize()
+    assert int(status.item()) == 1
+    # the two good choices and the shared expert still add up
+    good = torch.tensor([[1, 2]], dtype=torch.int32, device=DEV)
+    op2 = DecodeOps(table, sh, 1, 2, capi.ACT_BF16, capi.SWIGLU_TWICE, 0.0, capi.WEIGHT_AFTER_DOWN_BF16, True)
+    c2, s2 = op2.contribute(x, good, wt[:, :2].contiguous())
+    want = CombineOps.combine(c2, s2, good, capi.COMBINE_UNGATED)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(y), bits(want))
+    # two rows: outside the fast path, nothing launched
+    op3 = DecodeOps(table, sh, 2, 2, capi.ACT_BF16, capi.SWIGLU_TWICE, 0.0, capi.WEIGHT_AFTER_DOWN_BF16, True)
+    x2 = rand_bf16((2, 512), 1.0, 4).to(DEV)
+    ids2 = torch.tensor([[0, 1], [2, 3]], dtype=torch.int32, device=DEV)
+    y2 = torch.zeros((2, 512), dtype=torch.bfloat16, device=DEV)
+    assert not op3.finish(x2, ids2, torch.full((2, 2), 0.5, device=DEV), capi.COMBINE_UNGATED, y2)
+
+
 def test_decode_dsv3_width_single_token():
     # hidden 7168 / inter 2048 at DeepSeek-V3 width, 3 routed experts + shared, one token
     _run_decode(capi.FMT_FP8_BLOCK128, 3, 7168, 2048, 1, 3, 81, True)
