@@ -54,7 +54,8 @@ class Decode(ctypes.Structure):
 class Prefill(ctypes.Structure):
     _fields_ = [("rows", I), ("top_k", I), ("act_mode", I), ("swiglu", I), ("swiglu_limit", F), ("routed_weight", I),
                 ("weights_f32", I), ("x", P), ("ids", P), ("active", P), ("weights", P),
-                ("contributions", P), ("done", P), ("scratch", P), ("scratch_bytes", U64)]
+                ("contributions", P), ("done", P), ("scratch", P), ("scratch_bytes", U64),
+                ("shared", ctypes.POINTER(SharedExpert)), ("shared_out", P)]
 
 
 class FfmoeError(RuntimeError):
@@ -94,7 +95,7 @@ def lib():
         L.ffmoe_combine.argtypes = [P, P, P, P, P, P, P, P, I, I, I, I, P]
         L.ffmoe_decode_finish.argtypes = [ctypes.POINTER(ExpertTable), ctypes.POINTER(SharedExpert), ctypes.POINTER(Decode), P, P, P, I, P]
         L.ffmoe_prefill_scratch_bytes.restype = U64
-        L.ffmoe_prefill_scratch_bytes.argtypes = [I, I, I, I, I]
+        L.ffmoe_prefill_scratch_bytes.argtypes = [I, I, I, I, I, I]
         L.ffmoe_prefill_contribute.argtypes = [ctypes.POINTER(ExpertTable), ctypes.POINTER(Prefill), P]
         L.ffmoe_prefill_contribute_stage.argtypes = [ctypes.POINTER(ExpertTable), ctypes.POINTER(Prefill), I, P]
         for name in EXPORTS:

@@ -12,6 +12,7 @@ int decode_launch_bf16(const DecodeParams& p, int rg, int stage_mask, hipStream_
 int decode_finish_fp8(const FinishParams& q, hipStream_t st);
 int decode_finish_nvfp4(const FinishParams& q, hipStream_t st);
 int decode_finish_bf16(const FinishParams& q, hipStream_t st);
+int prefill_impl(const ffmoe_expert_table* table, const ffmoe_prefill* args, int stages, void* stream);
 }  // namespace ffmoe
 
 namespace ffmoe {
@@ -85,7 +86,10 @@ extern "C" __attribute__((visibility("default"))) uint64_t ffmoe_decode_scratch_
   (void)experts;
   const uint64_t max_groups = A + rows + 2;  // worst case: one row per group
   const uint64_t groups = (max_groups * sizeof(GroupDesc) + 255) & ~uint64_t(255);
-  return h + groups + 256;
+  // FFMOE_ACT_FP8_BLOCK128 runs on the grouped matrix-core path, which lays the arena out differently
+  const uint64_t w8a8 = ffmoe_prefill_scratch_bytes(rows, top_k, experts, hidden, inter, shared_inter);
+  const uint64_t own = h + groups + 256;
+  return own > w8a8 ? own : w8a8;
 }
 
 // layout_k >= 0: the call processes args->top_k choices per row (0 = the shared expert only) but lays the scratch
@@ -210,6 +214,18 @@ static int decode_impl(const ffmoe_expert_table* table, const ffmoe_shared_exper
 // kernels of its own format.
 static int decode_dispatch(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared, const ffmoe_decode* args,
                            int stage_mask, void* stream) {
+  if (table && args && args->act_mode == FFMOE_ACT_FP8_BLOCK128) {
+    // W8A8 (the reference's block-F32 model path, kernels/moe_ffn.cu:870-908): activations are quantized per 128 and
+    // the dot products run on the FP8 matrix cores through the grouped kernels of the prefill path, whatever the
+    // row count; the shared expert goes through the same kernels as one dense group.
+    ffmoe_prefill pf{};
+    pf.rows = args->rows; pf.top_k = args->top_k; pf.act_mode = args->act_mode;
+    pf.swiglu = args->swiglu; pf.swiglu_limit = args->swiglu_limit; pf.routed_weight = args->routed_weight; pf.weights_f32 = args->weights_f32;
+    pf.x = args->x; pf.ids = args->ids; pf.active = args->active; pf.weights = args->weights;
+    pf.contributions = args->contributions; pf.done = args->done; pf.scratch = args->scratch; pf.scratch_bytes = args->scratch_bytes;
+    pf.shared = shared; pf.shared_out = args->shared_out;
+    return prefill_impl(table, &pf, (stage_mask & 1 ? 3 : 0) | (stage_mask & 2 ? 12 : 0), stream);
+  }
   if (!table || !args || !shared || shared->format == table->format) return decode_impl(table, shared, args, stage_mask, stream);
   FF_TRY(decode_impl(table, nullptr, args, stage_mask, stream, args->top_k));
   ffmoe_expert_table as_shared = *table;

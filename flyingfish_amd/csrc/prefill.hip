@@ -199,10 +199,10 @@ int launch_gemm(const GemmParams& p, int mf, unsigned blocks, hipStream_t stream
 }
 
 struct PrefillLayout {
-  uint64_t xq, sx, act, aq, sa, counts, offsets, gbase, totals, perm, groups, units0, units1, total;
+  uint64_t xq, sx, act, aq, sa, counts, offsets, gbase, totals, perm, groups, units0, units1, sh_act, sh_aq, sh_sa, total;
   uint64_t max_groups;
 };
-PrefillLayout prefill_layout(int rows, int top_k, int experts, int hidden, int inter) {
+PrefillLayout prefill_layout(int rows, int top_k, int experts, int hidden, int inter, int shared_inter) {
   PrefillLayout l{};
   const uint64_t A = uint64_t(rows) * top_k;
   l.max_groups = uint64_t(experts) + (A + 15) / 16;
@@ -221,6 +221,11 @@ PrefillLayout prefill_layout(int rows, int top_k, int experts, int hidden, int i
   l.groups = take(l.max_groups * sizeof(GemmGroup));
   l.units0 = take(l.max_groups * uint64_t((inter + 127) / 128) * 8);
   l.units1 = take(l.max_groups * uint64_t((hidden + 255) / 256) * 8);
+  if (shared_inter > 0) {
+    l.sh_act = take(uint64_t(rows) * shared_inter * 2);
+    l.sh_aq = take(uint64_t(rows) * shared_inter);
+    l.sh_sa = take(uint64_t(rows) * (shared_inter / 128) * 4);
+  }
   l.total = off;
   return l;
 }
@@ -244,12 +249,12 @@ extern "C" __attribute__((visibility("default"))) int ffmoe_linear_fp8_block_w8a
   return launch_gemm<2>(p, mf, blocks, (hipStream_t)stream);
 }
 
-extern "C" __attribute__((visibility("default"))) uint64_t ffmoe_prefill_scratch_bytes(int rows, int top_k, int experts, int hidden, int inter) {
-  if (rows < 1 || top_k < 1 || experts < 1 || hidden < 128 || inter < 128) return 0;
-  return prefill_layout(rows, top_k, experts, hidden, inter).total;
+extern "C" __attribute__((visibility("default"))) uint64_t ffmoe_prefill_scratch_bytes(int rows, int top_k, int experts, int hidden, int inter, int shared_inter) {
+  if (rows < 1 || top_k < 1 || experts < 1 || hidden < 128 || inter < 128 || shared_inter < 0) return 0;
+  return prefill_layout(rows, top_k, experts, hidden, inter, shared_inter).total;
 }
 
-namespace {
+namespace ffmoe {
 int prefill_impl(const ffmoe_expert_table* table, const ffmoe_prefill* args, int stages, void* stream_);
 }
 extern "C" __attribute__((visibility("default"))) int ffmoe_prefill_contribute(const ffmoe_expert_table* table, const ffmoe_prefill* args, void* stream) {
@@ -259,7 +264,7 @@ extern "C" __attribute__((visibility("default"))) int ffmoe_prefill_contribute_s
   FF_REQUIRE(stage >= 0 && stage <= 3, FFMOE_ERR_SHAPE, "prefill stage %d (0 plan, 1 gate/up, 2 re-quantize, 3 down)", stage);
   return prefill_impl(table, args, 1 << stage, stream);
 }
-namespace {
+namespace ffmoe {
 int prefill_impl(const ffmoe_expert_table* table, const ffmoe_prefill* args, int stages, void* stream_) {
   hipStream_t stream = (hipStream_t)stream_;
   FF_REQUIRE(table != nullptr && args != nullptr, FFMOE_ERR_NULL, "table or args is NULL");
@@ -275,7 +280,17 @@ int prefill_impl(const ffmoe_expert_table* table, const ffmoe_prefill* args, int
              FFMOE_ERR_UNSUPPORTED, "unknown routed_weight %d", args->routed_weight);
   FF_PTR16(table->slots); FF_PTR16(args->x); FF_PTR4(args->ids); FF_PTR16(args->contributions);
   if (args->weights_f32) FF_PTR4(args->weights); else FF_PTR2(args->weights);
-  const PrefillLayout l = prefill_layout(R, K, E, H, I);
+  const ffmoe_shared_expert* shared = args->shared;
+  int SI = 0;
+  if (shared) {
+    SI = shared->inter;
+    FF_REQUIRE(shared->format == FFMOE_FMT_FP8_BLOCK128, FFMOE_ERR_UNSUPPORTED, "prefill needs an FFMOE_FMT_FP8_BLOCK128 shared expert (format %d)", shared->format);
+    FF_REQUIRE(SI >= 128 && SI % 128 == 0, FFMOE_ERR_SHAPE, "shared inter=%d must be a positive multiple of 128", SI);
+    FF_PTR16(args->shared_out);
+    for (int i = 0; i < 6; ++i)
+      FF_REQUIRE(shared->slot[i] != 0 && shared->slot[i] % (i % 2 ? 4 : 16) == 0, FFMOE_ERR_ALIGN, "shared expert slot[%d] is NULL or misaligned", i);
+  }
+  const PrefillLayout l = prefill_layout(R, K, E, H, I, SI);
   FF_PTR_ALIGNED(args->scratch, 256);
   FF_REQUIRE(args->scratch_bytes >= l.total, FFMOE_ERR_SCRATCH, "prefill scratch holds %llu bytes, %llu needed",
              (unsigned long long)args->scratch_bytes, (unsigned long long)l.total);
@@ -285,6 +300,11 @@ int prefill_impl(const ffmoe_expert_table* table, const ffmoe_prefill* args, int
   FF_NO_OVERLAP(args->scratch, l.total, args->x, size_t(R) * H * 2);
   FF_NO_OVERLAP(args->scratch, l.total, args->ids, A * 4);
   if (args->done) { FF_PTR4(args->done); FF_NO_OVERLAP(args->done, A * 4, args->scratch, l.total); }
+  if (shared) {
+    FF_NO_OVERLAP(args->shared_out, size_t(R) * H * 2, args->scratch, l.total);
+    FF_NO_OVERLAP(args->shared_out, size_t(R) * H * 2, args->x, size_t(R) * H * 2);
+    FF_NO_OVERLAP(args->shared_out, size_t(R) * H * 2, args->contributions, A * H * 2);
+  }
 
   uint8_t* s = (uint8_t*)args->scratch;
   PrefillBook b{(uint32_t*)(s + l.counts), (uint32_t*)(s + l.offsets), (uint32_t*)(s + l.gbase), (uint32_t*)(s + l.totals),
@@ -322,6 +342,32 @@ int prefill_impl(const ffmoe_expert_table* table, const ffmoe_prefill* args, int
     p.out = (uint16_t*)args->contributions; p.done = args->done; p.weights = args->weights; p.K = I; p.N = H;
     FF_TRY(launch_gemm<1>(p, mf, blocks, stream));
   }
+  if (shared) {
+    // the always-on expert: the same three steps over all rows in their own order (no grouping, no routing weight),
+    // as the reference runs it on the block-FP8 path (src/backend/cuda/moe/decode.rs:1187-1297)
+    const int smf = R > 32 ? 4 : R > 16 ? 2 : 1;
+    const int stm = 16 * smf;
+    const uint32_t sgroups = uint32_t((R + stm - 1) / stm);
+    GemmParams q{};
+    q.rows_total = R; q.top_k = 1;
+    q.swiglu = args->swiglu; q.limit = args->swiglu_limit;
+    if (stages & 2) {
+      q.a_codes = s + l.xq; q.a_scales = (const float*)(s + l.sx);
+      q.w0_codes = shared->slot[0]; q.w0_scales = shared->slot[1]; q.w1_codes = shared->slot[2]; q.w1_scales = shared->slot[3];
+      q.total_units = sgroups * uint32_t((SI + 127) / 128);
+      q.out = (uint16_t*)(s + l.sh_act); q.K = H; q.N = SI;
+      FF_TRY(launch_gemm<0>(q, smf, std::min<unsigned>(blocks, (q.total_units + 7u) & ~7u), stream));
+    }
+    if (stages & 4)
+      FF_TRY(ffmoe_quant_fp8_f32_128(s + l.sh_act, s + l.sh_aq, (float*)(s + l.sh_sa), R, SI, stream_));
+    if (stages & 8) {
+      q.a_codes = s + l.sh_aq; q.a_scales = (const float*)(s + l.sh_sa);
+      q.w0_codes = shared->slot[4]; q.w0_scales = shared->slot[5]; q.w1_codes = 0; q.w1_scales = 0;
+      q.total_units = sgroups * uint32_t((H + 255) / 256);
+      q.out = (uint16_t*)args->shared_out; q.K = SI; q.N = H;
+      FF_TRY(launch_gemm<2>(q, smf, std::min<unsigned>(blocks, (q.total_units + 7u) & ~7u), stream));
+    }
+  }
   return 0;
 }
-}  // namespace
+}  // namespace ffmoe

@@ -243,16 +243,19 @@ class PrefillOps:
     arena and the contributions / done buffers."""
 
     def __init__(self, table, rows, top_k, swiglu=capi.SWIGLU_TWICE, swiglu_limit=0.0,
-                 routed_weight=capi.WEIGHT_AFTER_DOWN_BF16, weights_f32=True):
+                 routed_weight=capi.WEIGHT_AFTER_DOWN_BF16, weights_f32=True, shared=None):
         self.table = table
         self.rows, self.top_k = rows, top_k
         self.cfg = (swiglu, swiglu_limit, routed_weight, int(weights_f32))
         dev = table.slots.device
-        nbytes = capi.lib().ffmoe_prefill_scratch_bytes(rows, top_k, table.experts, table.hidden, table.inter)
+        si = shared.inter if shared is not None else 0
+        nbytes = capi.lib().ffmoe_prefill_scratch_bytes(rows, top_k, table.experts, table.hidden, table.inter, si)
         self.scratch = torch.empty(nbytes, dtype=torch.uint8, device=dev)
         self.contributions = torch.empty((rows, top_k, table.hidden), dtype=_BF16, device=dev)
+        self.shared_out = torch.empty((rows, table.hidden), dtype=_BF16, device=dev) if shared is not None else None
         self.done = torch.zeros((rows, top_k), dtype=torch.int32, device=dev)
         self._table_c = table.c_struct()
+        self._shared_c = shared
 
     def scratch_views(self):
         """The arena regions a caller may inspect after contribute(): same offsets as prefill_layout() in
@@ -278,6 +281,15 @@ class PrefillOps:
         take("gbase", (E + 1) * 4, torch.int32, (E + 1,))
         take("totals", 16, torch.int32, (4,))
         take("perm", A * 4, torch.int32, (A,))
+        if self._shared_c is not None:
+            SI = self._shared_c.inter
+            max_groups = E + (A + 15) // 16
+            take("groups", max_groups * 16, torch.uint8, (max_groups * 16,))
+            take("units0", max_groups * (-(-I // 128)) * 8, torch.uint8, (-1,))
+            take("units1", max_groups * (-(-H // 256)) * 8, torch.uint8, (-1,))
+            take("sh_act", R * SI * 2, _BF16, (R, SI))
+            take("sh_aq", R * SI, torch.uint8, (R, SI))
+            take("sh_sa", R * (SI // 128) * 4, torch.float32, (R, SI // 128))
         return out
 
     def contribute(self, x, ids, weights, active=None, stage=None):
@@ -285,7 +297,9 @@ class PrefillOps:
         swiglu, limit, rw, wf32 = self.cfg
         a = capi.Prefill(self.rows, self.top_k, capi.ACT_FP8_BLOCK128, swiglu, limit, rw, wf32,
                          x.data_ptr(), ids.data_ptr(), active.data_ptr() if active is not None else None, weights.data_ptr(),
-                         self.contributions.data_ptr(), self.done.data_ptr(), self.scratch.data_ptr(), self.scratch.numel())
+                         self.contributions.data_ptr(), self.done.data_ptr(), self.scratch.data_ptr(), self.scratch.numel(),
+                         ctypes.pointer(self._shared_c) if self._shared_c is not None else None,
+                         self.shared_out.data_ptr() if self.shared_out is not None else None)
         if stage is None:
             capi.check(capi.lib().ffmoe_prefill_contribute(ctypes.byref(self._table_c), ctypes.byref(a), _stream()))
         else:

@@ -276,9 +276,11 @@ typedef struct ffmoe_prefill {
   void* contributions;     /* [rows, top_k, hidden] BF16 */
   uint32_t* done;          /* [rows, top_k] or NULL */
   void* scratch; uint64_t scratch_bytes;
+  const ffmoe_shared_expert* shared; /* always-on expert (FFMOE_FMT_FP8_BLOCK128), or NULL */
+  void* shared_out;        /* [rows, hidden] BF16 = bf16(down output), no routing weight (with shared) */
 } ffmoe_prefill;
 
-uint64_t ffmoe_prefill_scratch_bytes(int rows, int top_k, int experts, int hidden, int inter);
+uint64_t ffmoe_prefill_scratch_bytes(int rows, int top_k, int experts, int hidden, int inter, int shared_inter);
 int ffmoe_prefill_contribute(const ffmoe_expert_table* table, const ffmoe_prefill* args, void* stream);
 /* One step of the same call, for timing a kernel alone (the steps of one cohort must run in order once before any of
  * them is repeated): 0 = count / scan / fill + quantize x, 1 = gate/up GEMM + SwiGLU, 2 = re-quantize activations,

@@ -213,3 +213,54 @@ def test_prefill_then_combine_layer():
     assert int(status.item()) == 0
     want = orc.combine(bits(c), None, None, ids, None, capi.COMBINE_ROUTED)
     assert np.array_equal(bits(y), want)
+
+
+def _oracle_shared_w8a8(mats, x_bits, swiglu, limit):
+    """(shared_out, activation) of the always-on expert per row: the W8A8 FFN without a routing weight."""
+    g, sg, u, su, d, sd = mats
+    return [orc.expert_ffn_w8a8(x_bits[r], g, sg, u, su, d, sd, 1.0, swiglu, limit, orc.AFTER_DOWN_BF16, apply_weight=False, return_act=True)
+            for r in range(x_bits.shape[0])]
+
+
+@pytest.mark.parametrize("rows", [1, 5, 40])
+def test_prefill_shared_expert(rows):
+    """The always-on expert as one dense group through the same kernels: activations within 3 BF16 steps of the oracle,
+    shared_out within 2 steps of the oracle's down stage applied to the device activations."""
+    top_k, experts, hidden, inter = 2, 6, 256, 384
+    table, host = _make_fp8_table(experts + 1, hidden, inter, 12)
+    shared = table.shared_struct(experts)
+    table.experts = experts
+    ids, w = _routing(rows, top_k, experts, 61)
+    x = synth.normal((rows, hidden), 1.0, 62, dtype=torch.bfloat16)
+    op = ops.PrefillOps(table, rows, top_k, shared=shared)
+    got = op.contribute(x.cuda(), torch.from_numpy(ids).cuda(), torch.from_numpy(w).cuda())
+    torch.cuda.synchronize()
+    _check_prefill(op, host, bits(x), ids, w, orc.TWICE, 0.0, orc.AFTER_DOWN_BF16, np.ones_like(ids, dtype=bool), got)
+    # shared expert: scratch regions follow the routed ones (see PrefillOps.scratch_views)
+    sh_act = bits(op.scratch_views()["sh_act"])
+    g, sg, u, su, d, sd = host[experts]
+    want = _oracle_shared_w8a8(host[experts], bits(x), orc.TWICE, 0.0)
+    want_act = np.stack([a for _, a in want])
+    assert_close_bf16(sh_act, want_act, "shared activations", max_ulp=3)
+    want_out = np.stack([orc.expert_down_w8a8(sh_act[r], d, sd, apply_weight=False) for r in range(rows)])
+    assert_close_bf16(bits(op.shared_out), want_out, "shared_out from the device activations")
+
+
+@pytest.mark.parametrize("rows,top_k", [(1, 4), (3, 2)])
+def test_decode_w8a8_act_mode_runs_the_same_arithmetic(rows, top_k):
+    """ffmoe_decode_contribute with FFMOE_ACT_FP8_BLOCK128 = the grouped W8A8 path: bit-identical to PrefillOps."""
+    experts, hidden, inter = 6, 256, 256
+    table, _ = _make_fp8_table(experts + 1, hidden, inter, 13)
+    shared = table.shared_struct(experts)
+    table.experts = experts
+    ids, w = _routing(rows, top_k, experts, 71)
+    x = synth.normal((rows, hidden), 1.0, 72, dtype=torch.bfloat16).cuda()
+    ids_d, w_d = torch.from_numpy(ids).cuda(), torch.from_numpy(w).cuda()
+    pre = ops.PrefillOps(table, rows, top_k, shared=shared)
+    pre.contribute(x, ids_d, w_d)
+    dec = ops.DecodeOps(table, shared, rows, top_k, act_mode=capi.ACT_FP8_BLOCK128, weights_f32=True)
+    dec.done.zero_()
+    c, s = dec.contribute(x, ids_d, w_d)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(c), bits(pre.contributions)) and np.array_equal(bits(s), bits(pre.shared_out))
+    assert int(dec.done.sum().item()) == rows * top_k
