@@ -63,7 +63,8 @@ def test_decode_contract_violations_are_reported_before_launch():
     assert call(scratch_bytes=16) == capi.ERR_SCRATCH
     assert call(contributions=1 << 20) == capi.ERR_OVERLAP
     assert call(act_mode=2) == capi.ERR_UNSUPPORTED
-    assert call(act_mode=1) == capi.ERR_SHAPE and "128" in capi.last_error()  # the W8A8 path needs inter % 128 == 0 (1408 is not)
+    nv = capi.ExpertTable(capi.FMT_NVFP4, 64, 2048, 1408, 16 << 20, None, 32 << 20)
+    assert call(t=nv, act_mode=1) == capi.ERR_UNSUPPORTED  # the W8A8 path takes FP8 block experts only
     assert call(swiglu=2, swiglu_limit=0.0) == capi.ERR_SHAPE
     assert call(swiglu=7) == capi.ERR_UNSUPPORTED
     bad = capi.ExpertTable(capi.FMT_FP8_BLOCK128, 64, 2000, 1408, 16 << 20, None, None)
