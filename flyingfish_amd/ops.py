@@ -199,9 +199,9 @@ class DecodeOps:
         self.cfg = (act_mode, swiglu, swiglu_limit, routed_weight, int(weights_f32))
         dev = table.slots.device
         si = shared.inter if shared is not None else 0
-        nbytes = capi.lib().ffmoe_decode_scratch_bytes(rows, top_k, table.experts, table.hidden, table.inter, si)
+        nbytes = capi.lib().ffmoe_decode_scratch_bytes(rows, max(top_k, 1), table.experts, table.hidden, table.inter, si)
         self.scratch = torch.empty(nbytes, dtype=torch.uint8, device=dev)
-        self.contributions = torch.empty((rows, top_k, table.hidden), dtype=_BF16, device=dev)
+        self.contributions = torch.empty((rows, max(top_k, 1), table.hidden), dtype=_BF16, device=dev)
         self.shared_out = torch.empty((rows, table.hidden), dtype=_BF16, device=dev) if shared is not None else None
         self.done = torch.zeros((rows, top_k), dtype=torch.int32, device=dev)
         self._table_c = table.c_struct()
