@@ -475,3 +475,32 @@ def test_native_moe_layer_matches_oracle_pipeline():
     err = np.abs(orc.bf16_to_f32(bits(y)).astype(np.float64) - orc.bf16_to_f32(want).astype(np.float64))
     assert np.all(err <= 3 * (top_k + 1) * ulp), float(np.max(err / ulp))
     assert orc.rel_l2(bits(y), want) <= 4e-3
+
+
+def test_decode_layer_graph_replay_equals_eager():
+    """Eager-vs-graph bit equality of the whole decode layer (route, contribute, combine), several replays."""
+    table, _ = make_table(capi.FMT_FP8_BLOCK128, 9, 1024, 512, 23)
+    sh = table.shared_struct(8)
+    table.experts = 8
+    router = rand_bf16((8, 1024), 0.02, 24).to(DEV)
+    bias = torch.zeros(8, device=DEV)
+    for rows in (1, 4):
+        layer = NativeMoe(table, sh, router, bias, rows, 3, routed_scaling=2.5, combine_mode=capi.COMBINE_UNGATED,
+                          routed_weight=capi.WEIGHT_AFTER_DOWN_BF16)
+        x = rand_bf16((rows, 1024), 1.0, 25 + rows).to(DEV)
+        eager = bits(layer.run(x)).copy()
+        torch.cuda.synchronize()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(g, stream=side):
+                layer.run(x)
+        torch.cuda.current_stream().wait_stream(side)
+        for it in range(3):
+            layer.y.zero_()
+            torch.cuda.synchronize()
+            g.replay()
+            torch.cuda.synchronize()
+            assert np.array_equal(bits(layer.y), eager), "rows %d replay %d" % (rows, it)
+        assert int(layer.status.item()) == 0

@@ -264,3 +264,68 @@ def test_decode_w8a8_act_mode_runs_the_same_arithmetic(rows, top_k):
     torch.cuda.synchronize()
     assert np.array_equal(bits(c), bits(pre.contributions)) and np.array_equal(bits(s), bits(pre.shared_out))
     assert int(dec.done.sum().item()) == rows * top_k
+
+
+def test_prefill_token_order_reversal_reverses_outputs_bitwise():
+    """Row-permutation invariance (src/backend/cuda/moe/prefill_tests.rs:424-484): feeding the tokens in reverse order
+    gives the reversed contributions bit for bit."""
+    rows, top_k, experts, hidden, inter = 90, 4, 8, 256, 256
+    table, _ = _make_fp8_table(experts, hidden, inter, 14)
+    ids, w = _routing(rows, top_k, experts, 81, 1.1)
+    x = synth.normal((rows, hidden), 1.0, 82, dtype=torch.bfloat16).cuda()
+    ids_d, w_d = torch.from_numpy(ids).cuda(), torch.from_numpy(w).cuda()
+    op = ops.PrefillOps(table, rows, top_k)
+    fwd = bits(op.contribute(x, ids_d, w_d)).copy()
+    rev = bits(op.contribute(x.flip(0).contiguous(), ids_d.flip(0).contiguous(), w_d.flip(0).contiguous())).copy()
+    assert np.array_equal(rev[::-1], fwd)
+
+
+def test_prefill_mutation_controls_change_the_output():
+    """Swapping two experts' codes, or their scales, must change the contributions that used them
+    (src/backend/cuda/moe/prefill_tests.rs:485-535)."""
+    rows, top_k, experts, hidden, inter = 40, 2, 4, 256, 128
+    table, _ = _make_fp8_table(experts, hidden, inter, 15)
+    ids, w = _routing(rows, top_k, experts, 91)
+    x = synth.normal((rows, hidden), 1.0, 92, dtype=torch.bfloat16).cuda()
+    ids_d, w_d = torch.from_numpy(ids).cuda(), torch.from_numpy(w).cuda()
+    op = ops.PrefillOps(table, rows, top_k)
+    base = bits(op.contribute(x, ids_d, w_d)).copy()
+    uses = (ids == 0) | (ids == 1)
+    assert uses.any() and (~uses).any()
+    for which in (0, 1):  # 0: gate codes, 1: gate scales
+        a, b = table.expert_views(0)[which], table.expert_views(1)[which]
+        ta = a.clone(); a.copy_(b); b.copy_(ta)
+        got = bits(op.contribute(x, ids_d, w_d)).copy()
+        changed = np.any(got != base, axis=2)
+        assert np.all(changed[uses]) and not np.any(changed[~uses]), "mutation %d" % which
+        tb = a.clone(); a.copy_(b); b.copy_(tb)  # swap back
+    assert np.array_equal(bits(op.contribute(x, ids_d, w_d)), base)
+
+
+def test_prefill_graph_replay_equals_eager():
+    """Eager-vs-graph bit equality (src/backend/cuda/moe/testing.rs:8-31): the whole call is capturable (no host
+    read-back, no memset nodes); three replays with eager work in between all reproduce the eager result."""
+    rows, top_k, experts, hidden, inter = 70, 4, 8, 256, 256
+    table, _ = _make_fp8_table(experts + 1, hidden, inter, 16)
+    shared = table.shared_struct(experts)
+    table.experts = experts
+    ids, w = _routing(rows, top_k, experts, 95)
+    x = synth.normal((rows, hidden), 1.0, 96, dtype=torch.bfloat16).cuda()
+    ids_d, w_d = torch.from_numpy(ids).cuda(), torch.from_numpy(w).cuda()
+    op = ops.PrefillOps(table, rows, top_k, shared=shared)
+    eager_c = bits(op.contribute(x, ids_d, w_d)).copy()
+    eager_s = bits(op.shared_out).copy()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(g, stream=side):
+            op.contribute(x, ids_d, w_d)
+    torch.cuda.current_stream().wait_stream(side)
+    for it in range(3):
+        op.contributions.zero_(); op.shared_out.zero_()
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(bits(op.contributions), eager_c) and np.array_equal(bits(op.shared_out), eager_s), "replay %d" % it
