@@ -25,7 +25,7 @@ EXPORTS = [
     "ffmoe_quant_fp8_f32_128", "ffmoe_linear_fp8_block_w8a8", "ffmoe_linear_fp8_block", "ffmoe_linear_nvfp4",
     "ffmoe_gemm_skinny_bf16", "ffmoe_swiglu",
     "ffmoe_shared_scale", "ffmoe_combine",
-    "ffmoe_prefill_scratch_bytes", "ffmoe_prefill_contribute", "ffmoe_prefill_contribute_stage",
+    "ffmoe_combine_residual", "ffmoe_prefill_scratch_bytes", "ffmoe_prefill_contribute", "ffmoe_prefill_contribute_stage",
 ]
 
 P = ctypes.c_void_p
@@ -94,6 +94,7 @@ def lib():
         L.ffmoe_shared_scale.argtypes = [P, P, P, I, I, P]
         L.ffmoe_combine.argtypes = [P, P, P, P, P, P, P, P, I, I, I, I, P]
         L.ffmoe_decode_finish.argtypes = [ctypes.POINTER(ExpertTable), ctypes.POINTER(SharedExpert), ctypes.POINTER(Decode), P, P, P, I, P]
+        L.ffmoe_combine_residual.argtypes = [P, P, P, P, P, ctypes.c_longlong, P, P, P, P, P, P, I, I, I, P]
         L.ffmoe_prefill_scratch_bytes.restype = U64
         L.ffmoe_prefill_scratch_bytes.argtypes = [I, I, I, I, I, I]
         L.ffmoe_prefill_contribute.argtypes = [ctypes.POINTER(ExpertTable), ctypes.POINTER(Prefill), P]

@@ -324,6 +324,19 @@ class CombineOps:
         return y
 
 
+    @staticmethod
+    def combine_residual(shared_out, residual=None, y_out=None, contributions=None, routed_in=None, ids=None, seg=None, x=None,
+                         done=None, final_active=None, status=None):
+        """ff = bf16(bf16(routed) + gated); y_out = ff, or residual += ff in place (combine_residual / join_routed_residual)."""
+        rows, hidden = shared_out.shape
+        top_k = contributions.shape[1] if contributions is not None else 1
+        x_stride = x.stride(0) if x is not None else hidden
+        capi.check(capi.lib().ffmoe_combine_residual(_ptr(contributions), _ptr(routed_in), _ptr(shared_out), _ptr(seg), _ptr(x), x_stride,
+                                                     _ptr(ids), _ptr(done), _ptr(final_active), _ptr(residual), _ptr(y_out), _ptr(status),
+                                                     rows, top_k, hidden, _stream()))
+        return y_out if y_out is not None else residual
+
+
 class Fp8Ops:
     @staticmethod
     def quantize(x):

@@ -250,6 +250,20 @@ int ffmoe_combine(const void* contributions, const void* shared_out, const void*
                   const uint32_t* done, const uint32_t* final_active, void* y, uint32_t* status,
                   int rows, int top_k, int hidden, int mode, void* stream);
 
+/* Combine group with the residual add, and the peer-join form. Replaces moe_combine_residual{,_scalar} and
+ * moe_join_routed_residual{,_scalar} (kernels/moe_combine.cu:246-533; CombineOps::combine_residual / join_routed*,
+ * src/backend/cuda/moe/combine.rs:608-760):
+ *   ff = BF16(BF16(routed) + gated),  gated = BF16(scale_row * shared) if seg != NULL else shared,
+ *   scale_row = ffmoe_shared_scale(x_row, seg) computed in the same launch,
+ *   routed = ordered FP32 sum of the row's live contributions (contributions != NULL) or routed_in (the sum a peer
+ *   computed; exactly one of the two is given),
+ *   y_out != NULL: y_out = ff; else residual = BF16(residual + ff) in place.
+ * x row r starts at x + r * x_stride elements. */
+int ffmoe_combine_residual(const void* contributions, const void* routed_in, const void* shared_out, const void* seg,
+                           const void* x, long long x_stride, const int* ids, const uint32_t* done,
+                           const uint32_t* final_active, void* residual, void* y_out, uint32_t* status,
+                           int rows, int top_k, int hidden, void* stream);
+
 /* ------------------------------------------------------------------------------------------------
  * Prefill: many tokens, grouped by expert on the device (no host synchronisation: grids are sized from upper
  * bounds and kernels read the device-side counts), then two grouped GEMMs on the FP8 matrix cores in

@@ -445,6 +445,45 @@ def test_combine_modes_bit_exact():
     assert int(status.item()) == 1
 
 
+def test_combine_residual_and_peer_join_bit_exact():
+    """combine + residual add in one launch, gated and ungated, in place and to y_out, and the form that takes a routed
+    sum computed elsewhere (kernels/moe_combine.cu:246-533), against the oracle's combine + BF16 adds."""
+    rows, top_k, hidden = 3, 6, 2304   # 2304 = 9 x 256: the last block of a row is partly empty
+    c = rand_bf16((rows, top_k, hidden), 1.0, 510)
+    sh = rand_bf16((rows, hidden), 1.0, 511)
+    g = synth.generator(512)
+    ids = torch.stack([torch.randperm(32, generator=g)[:top_k] for _ in range(rows)]).to(torch.int32)
+    act = (torch.rand((rows, top_k), generator=g) > 0.25).to(torch.int32)
+    xw = rand_bf16((rows, hidden + 64), 1.0, 513)       # x rows live inside wider rows (x_stride > hidden)
+    x = xw[:, :hidden]
+    seg = rand_bf16((hidden,), 0.05, 514)
+    res0 = rand_bf16((rows, hidden), 1.0, 515)
+    scale = orc.shared_scale(bits(x.contiguous()), bits(seg))
+    actn = act.numpy().astype(np.uint32)
+
+    def bf16_add(a_bits, b_bits):
+        return orc.f32_to_bf16(orc.bf16_to_f32(a_bits) + orc.bf16_to_f32(b_bits))
+    xd = xw.to(DEV)[:, :hidden]
+    status = torch.zeros(1, dtype=torch.int32, device=DEV)
+    for gated in (True, False):
+        ff = orc.combine(bits(c), bits(sh), scale, ids.numpy(), actn, capi.COMBINE_GATED if gated else capi.COMBINE_UNGATED)
+        kw = dict(seg=seg.to(DEV), x=xd) if gated else {}
+        y = torch.empty((rows, hidden), dtype=torch.bfloat16, device=DEV)
+        CombineOps.combine_residual(sh.to(DEV), y_out=y, contributions=c.to(DEV), ids=ids.to(DEV), done=act.to(DEV),
+                                    final_active=act.to(DEV), status=status, **kw)
+        assert np.array_equal(bits(y), ff), "y_out gated=%s" % gated
+        res = res0.clone().to(DEV)
+        CombineOps.combine_residual(sh.to(DEV), residual=res, contributions=c.to(DEV), ids=ids.to(DEV), done=act.to(DEV),
+                                    final_active=act.to(DEV), status=status, **kw)
+        assert np.array_equal(bits(res), bf16_add(bits(res0), ff)), "residual gated=%s" % gated
+        # peer join: the routed sum arrives as BF16
+        routed = orc.combine(bits(c), None, None, ids.numpy(), actn, capi.COMBINE_ROUTED)
+        res = res0.clone().to(DEV)
+        CombineOps.combine_residual(sh.to(DEV), residual=res, routed_in=bf16_tensor(routed), **kw)
+        assert np.array_equal(bits(res), bf16_add(bits(res0), ff)), "join gated=%s" % gated
+    assert int(status.item()) == 0
+
+
 # ------------------------------------------------------------------------------------------------
 # whole layer
 def test_native_moe_layer_matches_oracle_pipeline():
