@@ -20,7 +20,7 @@ ERR_NULL, ERR_ALIGN, ERR_SHAPE, ERR_OVERLAP, ERR_UNSUPPORTED, ERR_SCRATCH = -1, 
 
 EXPORTS = [
     "ffmoe_last_error", "ffmoe_version",
-    "ffmoe_route_logits_bf16", "ffmoe_route_logits_f32", "ffmoe_route_topk", "ffmoe_route_topk_noaux", "ffmoe_route_noaux_decode", "ffmoe_route_decode",
+    "ffmoe_route_logits_bf16", "ffmoe_route_logits_f32", "ffmoe_route_topk", "ffmoe_route_topk_noaux", "ffmoe_route_noaux_decode", "ffmoe_route_decode", "ffmoe_slot_publish", "ffmoe_route_mask",
     "ffmoe_decode_scratch_bytes", "ffmoe_decode_contribute", "ffmoe_decode_contribute_stage", "ffmoe_decode_finish",
     "ffmoe_quant_fp8_f32_128", "ffmoe_linear_fp8_block_w8a8", "ffmoe_linear_fp8_block", "ffmoe_linear_nvfp4",
     "ffmoe_gemm_skinny_bf16", "ffmoe_swiglu",
@@ -36,7 +36,7 @@ U64 = ctypes.c_uint64
 
 class ExpertTable(ctypes.Structure):
     _fields_ = [("format", I), ("experts", I), ("hidden", I), ("inter", I),
-                ("slots", P), ("valid", P), ("global_scales", P)]
+                ("slots", P), ("valid", P), ("global_scales", P), ("generation", P)]
 
 
 class SharedExpert(ctypes.Structure):
@@ -48,14 +48,14 @@ class Decode(ctypes.Structure):
                 ("routed_weight", I), ("weights_f32", I),
                 ("x", P), ("ids", P), ("active", P), ("weights", P),
                 ("contributions", P), ("shared_out", P), ("done", P),
-                ("scratch", P), ("scratch_bytes", U64)]
+                ("scratch", P), ("scratch_bytes", U64), ("assignment_gen", P)]
 
 
 class Prefill(ctypes.Structure):
     _fields_ = [("rows", I), ("top_k", I), ("act_mode", I), ("swiglu", I), ("swiglu_limit", F), ("routed_weight", I),
                 ("weights_f32", I), ("x", P), ("ids", P), ("active", P), ("weights", P),
                 ("contributions", P), ("done", P), ("scratch", P), ("scratch_bytes", U64),
-                ("shared", ctypes.POINTER(SharedExpert)), ("shared_out", P)]
+                ("shared", ctypes.POINTER(SharedExpert)), ("shared_out", P), ("assignment_gen", P)]
 
 
 class FfmoeError(RuntimeError):
@@ -81,6 +81,8 @@ def lib():
         L.ffmoe_route_topk_noaux.argtypes = [P, P, I, P, P, I, I, I, I, I, F, I, I, P]
         L.ffmoe_route_noaux_decode.argtypes = [P, P, P, I, P, P, P, I, P, I, I, I, I, I, F, I, I, P]
         L.ffmoe_route_decode.argtypes = [P, P, P, P, P, I, I, I, I, I, P]
+        L.ffmoe_slot_publish.argtypes = [P, P, P, I, I, I, ctypes.POINTER(U64 * 6), U64, P, P]
+        L.ffmoe_route_mask.argtypes = [P, P, P, P, P, P, I, I, P]
         L.ffmoe_decode_scratch_bytes.restype = U64
         L.ffmoe_decode_scratch_bytes.argtypes = [I, I, I, I, I, I]
         L.ffmoe_decode_contribute.argtypes = [ctypes.POINTER(ExpertTable), ctypes.POINTER(SharedExpert), ctypes.POINTER(Decode), P]

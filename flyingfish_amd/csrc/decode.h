@@ -25,6 +25,8 @@ struct DecodeParams {
   const void* weights;
   const uint64_t* slots;
   const uint32_t* valid;
+  const uint64_t* generation;      // per expert, or NULL
+  const uint64_t* assignment_gen;  // per assignment, or NULL
   const float* global_scales;
   uint64_t shared_slot[6];
   float shared_global[3];

@@ -22,7 +22,8 @@ namespace ffmoe {
 // Groups are ordered by expert id, rows inside a group by assignment index, so the result does not
 // depend on scheduling. counters[0] = routed groups, counters[1] = shared groups.
 __global__ __launch_bounds__(1024) void k_group_assignments(const int* __restrict__ ids, const uint32_t* __restrict__ active,
-                                                            const uint32_t* __restrict__ valid,
+                                                            const uint32_t* __restrict__ valid, const uint64_t* __restrict__ generation,
+                                                            const uint64_t* __restrict__ assignment_gen,
                                                             GroupDesc* __restrict__ groups, int* __restrict__ counters,
                                                             int rows, int top_k, int experts, int has_shared, int rgmax) {
   extern __shared__ int s_ids[];  // [A] expert id or -1
@@ -32,6 +33,7 @@ __global__ __launch_bounds__(1024) void k_group_assignments(const int* __restric
   for (int a = tid; a < A; a += blockDim.x) {
     int e = (!active || active[a]) ? ids[a] : -1;
     if ((unsigned)e >= (unsigned)experts || (valid && valid[e] == 0u)) e = -1;
+    else if (generation && assignment_gen && generation[e] != assignment_gen[a]) e = -1;  // stale choice
     s_ids[a] = e;
   }
   __syncthreads();
@@ -167,6 +169,9 @@ static int decode_impl(const ffmoe_expert_table* table, const ffmoe_shared_exper
   p.weights_f32 = args->weights_f32;
   p.x = (const uint16_t*)args->x; p.ids = args->ids; p.active = args->active; p.weights = args->weights;
   p.slots = table->slots; p.valid = table->valid; p.global_scales = table->global_scales;
+  p.generation = table->generation; p.assignment_gen = args->assignment_gen;
+  if (p.generation) FF_PTR_ALIGNED(p.generation, 8);
+  if (p.assignment_gen) FF_PTR_ALIGNED(p.assignment_gen, 8);
   for (int i = 0; i < 6; ++i) p.shared_slot[i] = shared ? shared->slot[i] : 0;
   for (int i = 0; i < 3; ++i) p.shared_global[i] = shared ? shared->global_scales[i] : 1.0f;
   p.contributions = (uint16_t*)args->contributions; p.shared_out = (uint16_t*)args->shared_out; p.done = args->done;
@@ -186,7 +191,7 @@ static int decode_impl(const ffmoe_expert_table* table, const ffmoe_shared_exper
     p.groups = (GroupDesc*)(sc + hbytes) + (pass ? LA + 1 : 0);
     const uint64_t max_groups = uint64_t(LA) + R + 2;
     p.counters = (int*)(sc + hbytes + ((max_groups * sizeof(GroupDesc) + 255) & ~uint64_t(255))) + 2 * pass;
-    if (stage_mask & 1) hipLaunchKernelGGL(k_group_assignments, dim3(1), dim3(1024), A * sizeof(int), st, args->ids, args->active, table->valid, p.groups,
+    if (stage_mask & 1) hipLaunchKernelGGL(k_group_assignments, dim3(1), dim3(1024), A * sizeof(int), st, args->ids, args->active, table->valid, p.generation, p.assignment_gen, p.groups,
                        p.counters, R, K, E, p.has_shared, rg);
     FF_TRY(ff_launch_status());
   } else {
@@ -223,7 +228,7 @@ static int decode_dispatch(const ffmoe_expert_table* table, const ffmoe_shared_e
     pf.swiglu = args->swiglu; pf.swiglu_limit = args->swiglu_limit; pf.routed_weight = args->routed_weight; pf.weights_f32 = args->weights_f32;
     pf.x = args->x; pf.ids = args->ids; pf.active = args->active; pf.weights = args->weights;
     pf.contributions = args->contributions; pf.done = args->done; pf.scratch = args->scratch; pf.scratch_bytes = args->scratch_bytes;
-    pf.shared = shared; pf.shared_out = args->shared_out;
+    pf.shared = shared; pf.shared_out = args->shared_out; pf.assignment_gen = args->assignment_gen;
     return prefill_impl(table, &pf, (stage_mask & 1 ? 3 : 0) | (stage_mask & 2 ? 12 : 0), stream);
   }
   if (!table || !args || !shared || shared->format == table->format) return decode_impl(table, shared, args, stage_mask, stream);

@@ -46,6 +46,8 @@ __device__ __forceinline__ void load_group(const DecodeParams& p, int g, int& ex
     if (p.active && uni(int(load_global<uint32_t>(p.active + g))) == 0) n = 0;
     if ((unsigned)expert >= (unsigned)p.experts) n = 0;  // out-of-range id: contribute nothing, done stays 0
     else if (p.valid && uni(int(load_global<uint32_t>(p.valid + expert))) == 0) n = 0;
+    else if (p.generation && p.assignment_gen &&
+             uni64(load_global<uint64_t>(p.generation + expert)) != uni64(load_global<uint64_t>(p.assignment_gen + g))) n = 0;  // stale choice
   } else {
     expert = -1;
     row[0] = g - A;

@@ -30,7 +30,8 @@ __global__ __launch_bounds__(256) void k_decode_finish(const FinishParams q) {
   auto is_live = [&](int c) {
     const int e = p.ids[c];
     if (p.active && p.active[c] == 0u) return false;
-    return (unsigned)e < (unsigned)p.experts && !(p.valid && p.valid[e] == 0u);
+    if ((unsigned)e >= (unsigned)p.experts || (p.valid && p.valid[e] == 0u)) return false;
+    return !(p.generation && p.assignment_gen && p.generation[e] != p.assignment_gen[c]);
   };
   if (tid < K) {
     const int mine = p.ids[tid];

@@ -33,20 +33,21 @@ __global__ void k_prefill_zero(uint32_t* counts, int experts, uint32_t* totals) 
   if (i < 4) totals[i] = 0u;
 }
 
-__device__ __forceinline__ bool assignment_live(const int* ids, const uint32_t* active, const uint32_t* valid, long long a, int experts, int& e) {
-  e = ids[a];
-  if ((unsigned)e >= (unsigned)experts) return false;
-  if (active && active[a] == 0u) return false;
-  if (valid && valid[e] == 0u) return false;
+struct LiveTest { const int* ids; const uint32_t* active; const uint32_t* valid; const uint64_t* generation; const uint64_t* assignment_gen; int experts; };
+__device__ __forceinline__ bool assignment_live(const LiveTest& t, long long a, int& e) {
+  e = t.ids[a];
+  if ((unsigned)e >= (unsigned)t.experts) return false;
+  if (t.active && t.active[a] == 0u) return false;
+  if (t.valid && t.valid[e] == 0u) return false;
+  if (t.generation && t.assignment_gen && t.generation[e] != t.assignment_gen[a]) return false;  // stale choice
   return true;
 }
 
 // histogram of live assignments per expert (kernels/moe_prefill.cu:364-420)
-__global__ __launch_bounds__(256) void k_prefill_count(const int* __restrict__ ids, const uint32_t* __restrict__ active,
-                                                       const uint32_t* __restrict__ valid, uint32_t* __restrict__ counts, long long A, int experts) {
+__global__ __launch_bounds__(256) void k_prefill_count(const LiveTest t, uint32_t* __restrict__ counts, long long A) {
   const long long a = (long long)blockIdx.x * 256 + threadIdx.x;
   int e;
-  if (a < A && assignment_live(ids, active, valid, a, experts, e)) atomicAdd(counts + e, 1u);
+  if (a < A && assignment_live(t, a, e)) atomicAdd(counts + e, 1u);
 }
 
 // exclusive scans over experts (row offsets and group offsets), group descriptors and the two unit lists
@@ -107,8 +108,7 @@ __global__ __launch_bounds__(1024) void k_prefill_plan(PrefillBook b, int expert
 
 // stable fill: block e lists its assignments in ascending assignment order (the reference permutes with an atomic
 // cursor, kernels/moe_prefill.cu:475-510; per-row results make the order irrelevant, a fixed one keeps runs repeatable)
-__global__ __launch_bounds__(256) void k_prefill_fill(const int* __restrict__ ids, const uint32_t* __restrict__ active,
-                                                      const uint32_t* __restrict__ valid, PrefillBook b, long long A, int experts) {
+__global__ __launch_bounds__(256) void k_prefill_fill(const LiveTest lt, PrefillBook b, long long A) {
   __shared__ uint32_t s_wave[4];
   const int e = blockIdx.x;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -118,7 +118,7 @@ __global__ __launch_bounds__(256) void k_prefill_fill(const int* __restrict__ id
   for (long long a0 = 0; a0 < A; a0 += 256) {
     const long long a = a0 + tid;
     int id;
-    const bool hit = a < A && assignment_live(ids, active, valid, a, experts, id) && id == e;
+    const bool hit = a < A && assignment_live(lt, a, id) && id == e;
     const uint64_t mask = __ballot(hit);
     const uint32_t before = __popcll(mask & ((uint64_t(1) << lane) - 1));
     if (lane == 0) s_wave[wave] = __popcll(mask);
@@ -315,9 +315,10 @@ int prefill_impl(const ffmoe_expert_table* table, const ffmoe_prefill* args, int
 
   if (stages & 1) {
     hipLaunchKernelGGL(k_prefill_zero, dim3((E + 255) / 256), dim3(256), 0, stream, b.counts, E, b.totals);
-    hipLaunchKernelGGL(k_prefill_count, dim3((unsigned)((A + 255) / 256)), dim3(256), 0, stream, args->ids, args->active, table->valid, b.counts, (long long)A, E);
+    const LiveTest lt{args->ids, args->active, table->valid, table->generation, args->assignment_gen, E};
+    hipLaunchKernelGGL(k_prefill_count, dim3((unsigned)((A + 255) / 256)), dim3(256), 0, stream, lt, b.counts, (long long)A);
     hipLaunchKernelGGL(k_prefill_plan, dim3(1), dim3(1024), 0, stream, b, E, tm, tiles0, tiles1);
-    hipLaunchKernelGGL(k_prefill_fill, dim3(E), dim3(256), 0, stream, args->ids, args->active, table->valid, b, (long long)A, E);
+    hipLaunchKernelGGL(k_prefill_fill, dim3(E), dim3(256), 0, stream, lt, b, (long long)A);
     FF_TRY(ff_launch_status());
     // activations -> E4M3 + per-128 scales
     FF_TRY(ffmoe_quant_fp8_f32_128(args->x, s + l.xq, (float*)(s + l.sx), R, H, stream_));

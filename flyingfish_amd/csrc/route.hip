@@ -545,3 +545,68 @@ extern "C" __attribute__((visibility("default"))) int ffmoe_route_noaux_decode(c
   return ffmoe_route_topk_noaux(logits, bias, bias_row_stride, ids, weights, weights_f32, rows, experts, top_k, score_mode,
                                 routed_scaling, n_group, topk_group, stream);
 }
+
+// ---------------------------------------------------------------------------------------------
+// expert residency protocol
+namespace ffmoe {
+__global__ void k_slot_publish(uint64_t* slots, uint32_t* valid, uint64_t* generation, int incoming, int victim,
+                               uint64_t s0, uint64_t s1, uint64_t s2, uint64_t s3, uint64_t s4, uint64_t s5, uint64_t epoch, uint32_t* status) {
+  if (blockIdx.x != 0 || threadIdx.x != 0) return;
+  if (valid[incoming] == 1u && generation[incoming] >= epoch) {  // an epoch must move forward
+    if (status) atomicOr(status, 1u);
+    return;
+  }
+  if (victim >= 0) {
+    valid[victim] = 0u;
+    generation[victim] = 0;
+    for (int i = 0; i < 6; ++i) slots[size_t(victim) * 6 + i] = 0;
+  }
+  const uint64_t in[6] = {s0, s1, s2, s3, s4, s5};
+  for (int i = 0; i < 6; ++i) slots[size_t(incoming) * 6 + i] = in[i];
+  generation[incoming] = epoch;
+  valid[incoming] = 1u;
+}
+
+__global__ __launch_bounds__(256) void k_route_mask(const int* __restrict__ ids, const uint32_t* __restrict__ valid,
+                                                    const uint64_t* __restrict__ generation, uint32_t* __restrict__ active,
+                                                    uint64_t* __restrict__ assignment_gen, uint32_t* __restrict__ status, int assignments, int experts) {
+  const int a = blockIdx.x * 256 + threadIdx.x;
+  if (a >= assignments) return;
+  const int e = ids[a];
+  if ((unsigned)e >= (unsigned)experts || valid[e] > 1u || (valid[e] == 1u && generation[e] == 0)) {
+    if (status) atomicOr(status, 1u);
+    active[a] = 0u;
+    assignment_gen[a] = 0;
+    return;
+  }
+  active[a] = valid[e];
+  assignment_gen[a] = valid[e] ? generation[e] : 0;
+}
+}  // namespace ffmoe
+
+extern "C" __attribute__((visibility("default"))) int ffmoe_slot_publish(uint64_t* slots, uint32_t* valid, uint64_t* generation, int experts, int incoming,
+                                                                        int victim, const uint64_t incoming_slot[6], uint64_t epoch, uint32_t* status,
+                                                                        void* stream) {
+  FF_PTR16(slots); FF_PTR4(valid); FF_PTR_ALIGNED(generation, 8);
+  FF_REQUIRE(incoming_slot != nullptr, FFMOE_ERR_NULL, "incoming_slot is NULL");
+  FF_REQUIRE(experts >= 1 && experts <= FFMOE_MAX_EXPERTS && incoming >= 0 && incoming < experts && victim >= -1 && victim < experts && victim != incoming,
+             FFMOE_ERR_SHAPE, "slot_publish experts=%d incoming=%d victim=%d", experts, incoming, victim);
+  FF_REQUIRE(epoch != 0, FFMOE_ERR_SHAPE, "slot_publish epoch must not be 0");
+  for (int i = 0; i < 6; i += 2)
+    FF_REQUIRE(incoming_slot[i] != 0 && incoming_slot[i] % 16 == 0, FFMOE_ERR_ALIGN, "incoming_slot[%d] is NULL or misaligned", i);
+  if (status) FF_PTR4(status);
+  hipLaunchKernelGGL(ffmoe::k_slot_publish, dim3(1), dim3(1), 0, (hipStream_t)stream, slots, valid, generation, incoming, victim, incoming_slot[0],
+                     incoming_slot[1], incoming_slot[2], incoming_slot[3], incoming_slot[4], incoming_slot[5], epoch, status);
+  return ffmoe::ff_launch_status();
+}
+
+extern "C" __attribute__((visibility("default"))) int ffmoe_route_mask(const int* ids, const uint32_t* valid, const uint64_t* generation, uint32_t* active,
+                                                                      uint64_t* assignment_gen, uint32_t* status, int assignments, int experts, void* stream) {
+  FF_PTR4(ids); FF_PTR4(valid); FF_PTR_ALIGNED(generation, 8); FF_PTR4(active); FF_PTR_ALIGNED(assignment_gen, 8);
+  FF_REQUIRE(assignments >= 1 && experts >= 1 && experts <= FFMOE_MAX_EXPERTS, FFMOE_ERR_SHAPE, "route_mask assignments=%d experts=%d", assignments, experts);
+  if (status) FF_PTR4(status);
+  FF_NO_OVERLAP(active, size_t(assignments) * 4, ids, size_t(assignments) * 4);
+  hipLaunchKernelGGL(ffmoe::k_route_mask, dim3((assignments + 255) / 256), dim3(256), 0, (hipStream_t)stream, ids, valid, generation, active,
+                     assignment_gen, status, assignments, experts);
+  return ffmoe::ff_launch_status();
+}

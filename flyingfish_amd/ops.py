@@ -107,9 +107,11 @@ class ExpertTable:
         return 3 * H * I * 2
 
     def c_struct(self):
+        gen = getattr(self, "generation", None)
         return capi.ExpertTable(self.format, self.experts, self.hidden, self.inter, self.slots.data_ptr(),
                                 self.valid.data_ptr() if self.valid is not None else None,
-                                self.global_scales.data_ptr() if self.global_scales is not None else None)
+                                self.global_scales.data_ptr() if self.global_scales is not None else None,
+                                gen.data_ptr() if gen is not None else None)
 
     def shared_struct(self, e=0):
         """Describe expert e of this table as an always-on shared expert."""
@@ -189,6 +191,25 @@ class RouteOps:
         return ids, w, logits
 
 
+class Residency:
+    """Expert residency protocol over an ExpertTable (src/experts/arena.rs:220-483): publish / retire slots on the
+    stream, mask a routing result against the table."""
+
+    @staticmethod
+    def publish(table, incoming, slot_addresses, epoch, victim=-1, status=None):
+        arr = (capi.U64 * 6)(*[int(a) for a in slot_addresses])
+        capi.check(capi.lib().ffmoe_slot_publish(table.slots.data_ptr(), table.valid.data_ptr(), table.generation.data_ptr(), table.experts,
+                                                 incoming, victim, ctypes.byref(arr), epoch, _ptr(status), _stream()))
+
+    @staticmethod
+    def mask(table, ids, status=None):
+        active = torch.empty(ids.shape, dtype=torch.int32, device=ids.device)
+        gen = torch.empty(ids.shape, dtype=torch.int64, device=ids.device)
+        capi.check(capi.lib().ffmoe_route_mask(_ptr(ids), table.valid.data_ptr(), table.generation.data_ptr(), _ptr(active), _ptr(gen),
+                                               _ptr(status), ids.numel(), table.experts, _stream()))
+        return active, gen
+
+
 class DecodeOps:
     """Expert contributions for a decode batch; owns its scratch arena and output buffers."""
 
@@ -207,13 +228,13 @@ class DecodeOps:
         self._table_c = table.c_struct()
         self._shared_c = shared
 
-    def contribute(self, x, ids, weights, active=None, stage=None):
+    def contribute(self, x, ids, weights, active=None, stage=None, assignment_gen=None):
         """stage None = both launches; 0 / 1 = only the gate-up / only the down launch."""
         act_mode, swiglu, limit, rw, wf32 = self.cfg
         d = capi.Decode(self.rows, self.top_k, act_mode, swiglu, limit, rw, wf32,
                         x.data_ptr(), ids.data_ptr(), active.data_ptr() if active is not None else None, weights.data_ptr(),
                         self.contributions.data_ptr(), self.shared_out.data_ptr() if self.shared_out is not None else None,
-                        self.done.data_ptr(), self.scratch.data_ptr(), self.scratch.numel())
+                        self.done.data_ptr(), self.scratch.data_ptr(), self.scratch.numel(), _ptr(assignment_gen))
         sh = ctypes.byref(self._shared_c) if self._shared_c is not None else None
         if stage is None:
             capi.check(capi.lib().ffmoe_decode_contribute(ctypes.byref(self._table_c), sh, ctypes.byref(d), _stream()))
@@ -228,7 +249,7 @@ class DecodeOps:
         d = capi.Decode(self.rows, self.top_k, act_mode, swiglu, limit, rw, wf32,
                         x.data_ptr(), ids.data_ptr(), active.data_ptr() if active is not None else None, weights.data_ptr(),
                         self.contributions.data_ptr(), self.shared_out.data_ptr() if self.shared_out is not None else None,
-                        self.done.data_ptr(), self.scratch.data_ptr(), self.scratch.numel())
+                        self.done.data_ptr(), self.scratch.data_ptr(), self.scratch.numel(), None)
         sh = ctypes.byref(self._shared_c) if self._shared_c is not None else None
         rc = capi.lib().ffmoe_decode_finish(ctypes.byref(self._table_c), sh, ctypes.byref(d), _ptr(scale), _ptr(y), _ptr(status), mode, _stream())
         if rc == capi.ERR_UNSUPPORTED:
@@ -292,14 +313,14 @@ class PrefillOps:
             take("sh_sa", R * (SI // 128) * 4, torch.float32, (R, SI // 128))
         return out
 
-    def contribute(self, x, ids, weights, active=None, stage=None):
+    def contribute(self, x, ids, weights, active=None, stage=None, assignment_gen=None):
         """stage None = the whole call; 0..3 = one step (plan, gate/up, re-quantize, down)."""
         swiglu, limit, rw, wf32 = self.cfg
         a = capi.Prefill(self.rows, self.top_k, capi.ACT_FP8_BLOCK128, swiglu, limit, rw, wf32,
                          x.data_ptr(), ids.data_ptr(), active.data_ptr() if active is not None else None, weights.data_ptr(),
                          self.contributions.data_ptr(), self.done.data_ptr(), self.scratch.data_ptr(), self.scratch.numel(),
                          ctypes.pointer(self._shared_c) if self._shared_c is not None else None,
-                         self.shared_out.data_ptr() if self.shared_out is not None else None)
+                         self.shared_out.data_ptr() if self.shared_out is not None else None, _ptr(assignment_gen))
         if stage is None:
             capi.check(capi.lib().ffmoe_prefill_contribute(ctypes.byref(self._table_c), ctypes.byref(a), _stream()))
         else:

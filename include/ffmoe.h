@@ -137,6 +137,7 @@ typedef struct ffmoe_expert_table {
   const uint64_t* slots;      /* device [experts, 6] */
   const uint32_t* valid;      /* device [experts], 0 = not resident; NULL = all valid */
   const float* global_scales; /* device [experts, 3] (NVFP4) or NULL */
+  const uint64_t* generation; /* device [experts] residency epoch of each slot (ffmoe_slot_publish), or NULL */
 } ffmoe_expert_table;
 
 /* One always-on shared expert (MoeDecode::shared_gate/up/down, decode.rs:26-44). Addresses by value. */
@@ -171,6 +172,10 @@ typedef struct ffmoe_decode {
   uint32_t* done;      /* [rows, top_k]; set to 1 for every contributed slot (NULL = not tracked) */
   void* scratch;       /* ffmoe_decode_scratch_bytes() bytes, 256-byte aligned */
   uint64_t scratch_bytes;
+  const uint64_t* assignment_gen; /* [rows, top_k] epoch each choice was routed against (ffmoe_route_mask), or NULL.
+                                     With table->generation: a choice whose expert has been replaced since (epochs
+                                     differ) contributes nothing and keeps done = 0, where the reference traps
+                                     (kernels/moe_ffn.cu:140-154) */
 } ffmoe_decode;
 
 /* Scratch needed by ffmoe_decode_contribute (mirrors decode_scratch_bytes_mixed, decode.rs:52-59,
@@ -200,6 +205,25 @@ int ffmoe_decode_contribute_stage(const ffmoe_expert_table* table, const ffmoe_s
  * two separate calls then. */
 int ffmoe_decode_finish(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared, const ffmoe_decode* args,
                         const void* scale, void* y, uint32_t* status, int combine_mode, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * Expert residency protocol (src/experts/arena.rs:220-483). With every expert resident the table is constant and
+ * none of this is needed; an engine that swaps experts in and out publishes each change on the stream and masks
+ * the routing against the table before the expert launches.
+ */
+
+/* Replaces moe_slot_publish (kernels/moe_route.cu:650-670): stream-ordered publication of expert `incoming` (its six
+ * slot addresses and a strictly increasing epoch) and retirement of `victim` (-1 = none): valid[victim] = 0,
+ * generation[victim] = 0, its slot row cleared. Contract violations (bad ids, NULL or misaligned addresses, epoch 0,
+ * epoch not above the one of a slot that is already valid) are reported on the host where the arguments show them and
+ * through *status |= 1 where only the device table does. */
+int ffmoe_slot_publish(uint64_t* slots, uint32_t* valid, uint64_t* generation, int experts, int incoming, int victim,
+                       const uint64_t incoming_slot[6], uint64_t epoch, uint32_t* status, void* stream);
+
+/* Replaces moe_route_mask (kernels/moe_route.cu:672-681): active[a] = valid[ids[a]], assignment_gen[a] = its epoch
+ * (0 when not resident). *status |= 1 for an id out of range or a table entry that is valid without an epoch. */
+int ffmoe_route_mask(const int* ids, const uint32_t* valid, const uint64_t* generation, uint32_t* active,
+                     uint64_t* assignment_gen, uint32_t* status, int assignments, int experts, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
  * Standalone linears, M <= 16 "skinny" and beyond. y[M,N] = x[M,K] * W[N,K]^T, BF16 in / BF16 out.
@@ -292,6 +316,7 @@ typedef struct ffmoe_prefill {
   void* scratch; uint64_t scratch_bytes;
   const ffmoe_shared_expert* shared; /* always-on expert (FFMOE_FMT_FP8_BLOCK128), or NULL */
   void* shared_out;        /* [rows, hidden] BF16 = bf16(down output), no routing weight (with shared) */
+  const uint64_t* assignment_gen; /* as in ffmoe_decode, or NULL */
 } ffmoe_prefill;
 
 uint64_t ffmoe_prefill_scratch_bytes(int rows, int top_k, int experts, int hidden, int inter, int shared_inter);

@@ -484,6 +484,61 @@ def test_combine_residual_and_peer_join_bit_exact():
     assert int(status.item()) == 0
 
 
+def test_residency_protocol_publish_mask_and_stale_choices():
+    """Slot publication, routing mask and the epoch check (kernels/moe_route.cu:650-681, kernels/moe_ffn.cu:140-154):
+    a choice routed against an epoch that has since been replaced contributes nothing and leaves done = 0, which the
+    combine reports through its status word (the reference traps)."""
+    from flyingfish_amd.ops import Residency
+    experts, hidden, inter, rows, top_k = 6, 512, 256, 2, 3
+    table, ref = make_table(capi.FMT_FP8_BLOCK128, experts, hidden, inter, 700)
+    addresses = table.slots.cpu().clone()
+    # start with an empty table and publish experts 0..4 at epochs 1..5; expert 5 stays out
+    table.slots.zero_()
+    table.valid = torch.zeros(experts, dtype=torch.int32, device=DEV)
+    table.generation = torch.zeros(experts, dtype=torch.int64, device=DEV)
+    status = torch.zeros(1, dtype=torch.int32, device=DEV)
+    for e in range(5):
+        Residency.publish(table, e, addresses[e].tolist(), epoch=e + 1, status=status)
+    torch.cuda.synchronize()
+    assert table.valid.cpu().tolist() == [1, 1, 1, 1, 1, 0] and table.generation.cpu().tolist() == [1, 2, 3, 4, 5, 0]
+    assert torch.equal(table.slots.cpu()[:5], addresses[:5]) and int(status.item()) == 0
+    ids = torch.tensor([[0, 5, 2], [4, 1, 3]], dtype=torch.int32, device=DEV)
+    active, gen = Residency.mask(table, ids, status=status)
+    torch.cuda.synchronize()
+    assert active.cpu().tolist() == [[1, 0, 1], [1, 1, 1]] and gen.cpu().tolist() == [[1, 0, 3], [5, 2, 4]] and int(status.item()) == 0
+    x = rand_bf16((rows, hidden), 1.0, 701).to(DEV)
+    wt = torch.full((rows, top_k), 0.5, device=DEV)
+    op = DecodeOps(table, None, rows, top_k, capi.ACT_BF16, capi.SWIGLU_TWICE, 0.0, capi.WEIGHT_AFTER_DOWN_BF16, True)
+    op.done.zero_()
+    op.contribute(x, ids, wt, active, assignment_gen=gen)
+    torch.cuda.synchronize()
+    assert op.done.cpu().tolist() == [[1, 0, 1], [1, 1, 1]]
+    first = bits(op.contributions).copy()
+    # expert 2 is replaced (same weights, new epoch 9; expert 5 comes in over victim 1): choices routed earlier against
+    # epochs 3 and 2 are now stale
+    Residency.publish(table, 2, addresses[2].tolist(), epoch=9, status=status)
+    Residency.publish(table, 5, addresses[5].tolist(), epoch=10, victim=1, status=status)
+    op.done.zero_()
+    op.contributions.zero_()
+    op.contribute(x, ids, wt, active, assignment_gen=gen)
+    torch.cuda.synchronize()
+    assert op.done.cpu().tolist() == [[1, 0, 0], [1, 0, 1]]
+    second = bits(op.contributions)
+    assert np.array_equal(second[0, 0], first[0, 0]) and np.array_equal(second[1, 2], first[1, 2]) and not second[0, 2].any() and not second[1, 1].any()
+    CombineOps.combine(op.contributions, None, ids, capi.COMBINE_ROUTED, done=op.done, final_active=active, status=status)
+    torch.cuda.synchronize()
+    assert int(status.item()) == 1
+    # an epoch may only move forward; out-of-range ids are flagged by the mask
+    status.zero_()
+    Residency.publish(table, 0, addresses[0].tolist(), epoch=1, status=status)
+    torch.cuda.synchronize()
+    assert int(status.item()) == 1
+    status.zero_()
+    Residency.mask(table, torch.tensor([[0, 77, 2]], dtype=torch.int32, device=DEV), status=status)
+    torch.cuda.synchronize()
+    assert int(status.item()) == 1
+
+
 # ------------------------------------------------------------------------------------------------
 # whole layer
 def test_native_moe_layer_matches_oracle_pipeline():
