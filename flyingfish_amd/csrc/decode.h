@@ -15,7 +15,17 @@ struct GroupDesc {
   int pad[2];
 };
 
+// Top-k selection inside the gate/up kernel (one token row): every block selects from the FP32 logits in its prologue,
+// block 0 publishes ids and weights for the later launches. logits == NULL: ids and weights are inputs.
+struct RouteInline {
+  const float* logits;  // [experts]
+  const float* bias;    // [experts] or NULL
+  int score_mode, n_group, topk_group;
+  float routed_scaling;
+};
+
 struct DecodeParams {
+  RouteInline route;
   int rows, top_k, experts, hidden, inter, shared_inter, has_shared;
   int swiglu, routed_weight, weights_f32;
   float swiglu_limit;

@@ -99,7 +99,8 @@ extern "C" __attribute__((visibility("default"))) uint64_t ffmoe_decode_scratch_
 // Pass 1 keeps its group descriptors and counters behind those of pass 0: the passes may be issued stage by stage
 // (both gate/up launches, then both down launches), so neither may overwrite the other's grouping.
 static int decode_impl(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared, const ffmoe_decode* args,
-                       int stage_mask, void* stream, int layout_k = -1, int pass = 0, const FinishParams* fin = nullptr) {
+                       int stage_mask, void* stream, int layout_k = -1, int pass = 0, const FinishParams* fin = nullptr,
+                       const RouteInline* route = nullptr) {
   FF_REQUIRE(table && args, FFMOE_ERR_NULL, "table/args is NULL");
   const int R = args->rows, K = args->top_k, E = table->experts, H = table->hidden, I = table->inter;
   const int LK = layout_k < 0 ? K : layout_k;
@@ -163,6 +164,7 @@ static int decode_impl(const ffmoe_expert_table* table, const ffmoe_shared_exper
   FF_REQUIRE(size_t(kmax_lds) * 2 <= 160 * 1024 / 2, FFMOE_ERR_SHAPE, "row of %d BF16 does not fit the LDS staging", kmax_lds);
 
   DecodeParams p;
+  p.route = route ? *route : RouteInline{nullptr, nullptr, 0, 1, 1, 1.0f};
   p.rows = R; p.top_k = K; p.experts = E; p.hidden = H; p.inter = I; p.shared_inter = SI;
   p.has_shared = shared ? 1 : 0;
   p.swiglu = args->swiglu; p.swiglu_limit = args->swiglu_limit; p.routed_weight = args->routed_weight;
@@ -271,4 +273,31 @@ extern "C" __attribute__((visibility("default"))) int ffmoe_decode_finish(const 
   // the shared expert takes part only in the modes that add it
   const ffmoe_shared_expert* sh = combine_mode == FFMOE_COMBINE_ROUTED ? nullptr : shared;
   return decode_impl(table, sh, args, 0, stream, -1, 0, &fin);
+}
+
+extern "C" __attribute__((visibility("default"))) int ffmoe_decode_contribute_from_logits(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared,
+                                                                                         const ffmoe_decode* args, const float* logits, const float* bias,
+                                                                                         int score_mode, float routed_scaling, int n_group, int topk_group,
+                                                                                         void* stream) {
+  FF_REQUIRE(table && args, FFMOE_ERR_NULL, "table/args is NULL");
+  FF_REQUIRE(args->rows == 1, FFMOE_ERR_UNSUPPORTED, "selection inside the gate/up launch handles one token row (rows=%d)", args->rows);
+  FF_REQUIRE(args->act_mode == FFMOE_ACT_BF16, FFMOE_ERR_UNSUPPORTED, "selection inside the gate/up launch needs FFMOE_ACT_BF16");
+  FF_REQUIRE(!shared || shared->format == table->format, FFMOE_ERR_UNSUPPORTED, "selection inside the gate/up launch needs the shared expert in the table's format");
+  FF_REQUIRE(args->weights_f32 == 1 && args->active == nullptr && args->assignment_gen == nullptr, FFMOE_ERR_UNSUPPORTED,
+             "selection inside the gate/up launch writes f32 weights and takes no active mask or epochs");
+  const int E = table->experts, K = args->top_k;
+  FF_REQUIRE(E == 64 || E == 128 || E == 256 || E == 512 || E == 1024, FFMOE_ERR_UNSUPPORTED, "experts=%d is not 64 * 2^n", E);
+  FF_REQUIRE(K >= 1 && K <= FFMOE_MAX_TOP_K && K < E, FFMOE_ERR_SHAPE, "top_k=%d out of range", K);
+  FF_REQUIRE(score_mode == FFMOE_NOAUX_SIGMOID || score_mode == FFMOE_NOAUX_SQRTSOFTPLUS, FFMOE_ERR_UNSUPPORTED, "unknown score mode %d", score_mode);
+  FF_REQUIRE(routed_scaling > 0.0f && routed_scaling < INFINITY, FFMOE_ERR_SHAPE, "routed_scaling=%g", (double)routed_scaling);
+  FF_REQUIRE(n_group >= 1 && topk_group >= 1 && topk_group <= n_group && E % n_group == 0, FFMOE_ERR_SHAPE, "n_group=%d topk_group=%d", n_group, topk_group);
+  if (n_group > 1) {
+    const int c = E / 64, per = E / n_group;
+    FF_REQUIRE(per % c == 0 && ((per / c) & (per / c - 1)) == 0 && topk_group * per >= K, FFMOE_ERR_UNSUPPORTED,
+               "groups of %d experts do not tile the wave, or the kept groups hold fewer than top_k experts", per);
+  }
+  FF_PTR4(logits);
+  if (bias) FF_PTR4(bias);
+  const RouteInline route{logits, bias, score_mode, n_group, topk_group, routed_scaling};
+  return decode_impl(table, shared, args, 3, stream, -1, 0, nullptr, &route);
 }

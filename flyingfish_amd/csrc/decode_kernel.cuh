@@ -13,6 +13,7 @@
 // contribution (src/cpu/expert_ffn.rs:592-679; kernels/moe_ffn.cu:198-209,293-301).
 #pragma once
 #include "gemv.cuh"
+#include "route_select.cuh"
 #include "api.h"
 #include "decode.h"
 
@@ -23,7 +24,8 @@ namespace ffmoe {
 // Group g as wave-uniform scalars. Without a descriptor table (one row per call) every assignment is its own
 // group and the shared expert follows the routed ones.
 template <int RG>
-__device__ __forceinline__ void load_group(const DecodeParams& p, int g, int& expert, int& n, int (&row)[RG], int (&slot)[RG]) {
+__device__ __forceinline__ void load_group(const DecodeParams& p, int g, int& expert, int& n, int (&row)[RG], int (&slot)[RG],
+                                           const int* inline_ids = nullptr) {
   if (p.groups) {
     const int* gd = reinterpret_cast<const int*>(p.groups + g);
     expert = uni(load_global<int>(gd));
@@ -40,7 +42,7 @@ __device__ __forceinline__ void load_group(const DecodeParams& p, int g, int& ex
   for (int r = 0; r < RG; ++r) { row[r] = 0; slot[r] = 0; }
   n = 1;
   if (g < A) {
-    expert = uni(load_global<int>(p.ids + g));
+    expert = inline_ids ? uni(inline_ids[g]) : uni(load_global<int>(p.ids + g));
     row[0] = g / p.top_k;
     slot[0] = g;
     if (p.active && uni(int(load_global<uint32_t>(p.active + g))) == 0) n = 0;
@@ -74,6 +76,23 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = uni(tid >> 6);
   const int A = p.rows * p.top_k;
+  // one token, selection in the prologue: wave 0 selects into LDS, block 0 publishes ids, weights and clean done flags
+  __shared__ int s_route_ids[FFMOE_MAX_TOP_K];
+  __shared__ float s_route_w[FFMOE_MAX_TOP_K];
+  const bool inline_route = STAGE == 0 && RG == 1 && p.route.logits != nullptr;
+  if (STAGE == 0 && RG == 1) {
+    if (inline_route) {
+      if (wave == 0)
+        wave_route_dispatch(p.route.logits, p.route.bias, lane, p.experts, p.top_k, p.route.score_mode, p.route.routed_scaling,
+                            p.route.n_group, p.route.topk_group, s_route_ids, s_route_w, 1);
+      __syncthreads();
+      if (blockIdx.x == 0 && tid < p.top_k) {
+        const_cast<int*>(p.ids)[tid] = s_route_ids[tid];
+        reinterpret_cast<float*>(const_cast<void*>(p.weights))[tid] = s_route_w[tid];
+        if (p.done) p.done[tid] = 0u;
+      }
+    }
+  }
   const int n_routed = p.counters ? uni(load_global<int>(p.counters)) : A;
   const int n_shared = p.counters ? uni(load_global<int>(p.counters + 1)) : (p.has_shared ? p.rows : 0);
   // units per group
@@ -91,7 +110,7 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
     const long long seg_end = u0 + (width - j0) < hi ? u0 + (width - j0) : hi;
     const int count = int(seg_end - u0);
     int expert, gn, grow[RG], gslot[RG];
-    load_group<RG>(p, g, expert, gn, grow, gslot);
+    load_group<RG>(p, g, expert, gn, grow, gslot, inline_route ? s_route_ids : nullptr);
     const bool shared = expert < 0;
     const int Kg = STAGE == 0 ? p.hidden : (shared ? p.shared_inter : p.inter);
     // the six slot addresses through scalar-friendly paths (kernel argument or global table), never a generic pointer

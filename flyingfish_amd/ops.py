@@ -242,6 +242,22 @@ class DecodeOps:
             capi.check(capi.lib().ffmoe_decode_contribute_stage(ctypes.byref(self._table_c), sh, ctypes.byref(d), stage, _stream()))
         return self.contributions, self.shared_out
 
+    def contribute_from_logits(self, x, logits, bias, ids, weights, score_mode=capi.NOAUX_SIGMOID, routed_scaling=1.0, n_group=1, topk_group=1):
+        """One token: top-k selection inside the gate/up launch; ids / weights (f32) are written. Returns None when the
+        shape is outside the fast path (nothing launched)."""
+        act_mode, swiglu, limit, rw, wf32 = self.cfg
+        d = capi.Decode(self.rows, self.top_k, act_mode, swiglu, limit, rw, wf32,
+                        x.data_ptr(), ids.data_ptr(), None, weights.data_ptr(),
+                        self.contributions.data_ptr(), self.shared_out.data_ptr() if self.shared_out is not None else None,
+                        self.done.data_ptr(), self.scratch.data_ptr(), self.scratch.numel(), None)
+        sh = ctypes.byref(self._shared_c) if self._shared_c is not None else None
+        rc = capi.lib().ffmoe_decode_contribute_from_logits(ctypes.byref(self._table_c), sh, ctypes.byref(d), _ptr(logits), _ptr(bias),
+                                                            score_mode, routed_scaling, n_group, topk_group, _stream())
+        if rc == capi.ERR_UNSUPPORTED:
+            return None
+        capi.check(rc)
+        return self.contributions, self.shared_out
+
     def finish(self, x, ids, weights, mode, y, status=None, scale=None, active=None):
         """rows == 1: down + routing weight + ordered combine in one launch, after contribute(stage=0) on the same
         arguments. Returns False (nothing launched) when the shape is outside the fast path."""
@@ -440,9 +456,21 @@ class NativeMoe:
         # one-token finish in a single launch (ffmoe_decode_finish). Off by default: on MI355X it measured 33 us
         # against 26 + 4.6 us for the separate down and combine launches at the DeepSeek-V3 shape.
         self.fused_finish = False
+        # one token: run the top-k selection in the prologue of the gate/up launch (one launch less)
+        self.inline_select = True
 
     def run(self, x):
         scaling, ng, kg = self.routing
+        if self.rows == 1 and self.inline_select:
+            # one token: logits launch, then gate/up with the selection in its prologue, down, combine (4 launches)
+            RouteOps.logits_f32(x, self.router, out=self.logits)
+            got = self.decode.contribute_from_logits(x, self.logits, self.bias if self.bias.dim() == 1 else self.bias[0], self.ids, self.weights,
+                                                     routed_scaling=scaling, n_group=ng, topk_group=kg)
+            if got is not None:
+                contrib, shared_out = got
+                mode = self.combine_mode if shared_out is not None else capi.COMBINE_ROUTED
+                return CombineOps.combine(contrib, shared_out, self.ids, mode, done=self.decode.done, status=self.status, out=self.y)
+            self.inline_select = False
         RouteOps.route_noaux(x, self.router, self.bias, self.top_k, self.logits, self.ids, self.weights,
                              done=self.decode.done, routed_scaling=scaling, n_group=ng, topk_group=kg)
         if self.rows == 1 and self.fused_finish:

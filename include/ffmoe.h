@@ -192,6 +192,16 @@ int ffmoe_decode_contribute(const ffmoe_expert_table* table, const ffmoe_shared_
 int ffmoe_decode_contribute_stage(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared,
                                   const ffmoe_decode* args, int stage, void* stream);
 
+/* One token, selection inside the gate/up launch: logits [experts] FP32 (from ffmoe_route_logits_f32) go in, and the
+ * top-k selection of ffmoe_route_topk_noaux (same arithmetic, bit for bit) runs in the prologue of every block of the
+ * gate/up launch instead of a launch of its own; args->ids and args->weights (f32) are OUTPUTS here, written for the
+ * down launch and the combine, and args->done is cleared. Replaces moe_route_select_noaux + moe_gate_up + moe_down for
+ * rows == 1 (kernels/moe_route.cu:315-390, kernels/moe_ffn.cu:98-302) with one launch less. Needs experts = 64 * 2^n,
+ * FFMOE_ACT_BF16, f32 weights, no active mask; FFMOE_ERR_UNSUPPORTED otherwise (use the separate calls). */
+int ffmoe_decode_contribute_from_logits(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared,
+                                        const ffmoe_decode* args, const float* logits, const float* bias,
+                                        int score_mode, float routed_scaling, int n_group, int topk_group, void* stream);
+
 /* One-token finish: the down projection of every live choice and of the shared expert, the routing weight and the
  * ordered combine in ONE launch, for rows == 1. Call after ffmoe_decode_contribute_stage(table, shared, args, 0, stream)
  * with the same table / shared / args (the gate/up activations are taken from args->scratch); writes y[hidden] and

@@ -598,3 +598,42 @@ def test_decode_layer_graph_replay_equals_eager():
             torch.cuda.synchronize()
             assert np.array_equal(bits(layer.y), eager), "rows %d replay %d" % (rows, it)
         assert int(layer.status.item()) == 0
+
+
+@pytest.mark.parametrize("fmt", [capi.FMT_FP8_BLOCK128, capi.FMT_NVFP4])
+@pytest.mark.parametrize("experts,n_group,topk_group", [(64, 1, 1), (256, 8, 4)])
+def test_one_token_selection_inside_gate_up_launch(fmt, experts, n_group, topk_group):
+    """ffmoe_decode_contribute_from_logits: ids, weights, contributions and y equal the separate top-k launch bit for bit."""
+    hidden, inter, top_k = 512, 256, 6
+    table, _ = make_table(fmt, experts + 1, hidden, inter, 61)
+    sh = table.shared_struct(experts)
+    table.experts = experts
+    router = rand_bf16((experts, hidden), 0.05, 62).to(DEV)
+    bias = (torch.randn(experts, generator=torch.Generator().manual_seed(63)) * 0.1).to(DEV)
+    x = rand_bf16((1, hidden), 1.0, 64).to(DEV)
+    got = {}
+    for inline in (False, True):
+        layer = NativeMoe(table, sh, router, bias, 1, top_k, routed_scaling=2.5, n_group=n_group, topk_group=topk_group)
+        layer.inline_select = inline
+        layer.decode.done.fill_(7)  # stale flags: both paths must clear them
+        y = bits(layer.run(x)).copy()
+        assert layer.inline_select == inline
+        got[inline] = (layer.ids.cpu().numpy().copy(), layer.weights.cpu().numpy().copy(), bits(layer.decode.contributions).copy(), y,
+                       layer.decode.done.cpu().numpy().copy())
+        assert int(layer.status.item()) == 0
+    for name, a, b in zip(("ids", "weights", "contributions", "y", "done"), got[False], got[True]):
+        assert np.array_equal(a, b), name
+    assert got[True][4].ravel().tolist() == [1] * top_k
+    # and against the oracle's selection
+    ids, w = orc.route_topk_noaux(orc.route_logits_f32(bits(x), bits(router)), bias.cpu().numpy()[None, :], top_k, 0, 2.5, n_group, topk_group)
+    assert np.array_equal(ids, got[True][0]) and np.array_equal(w.view(np.uint32), got[True][1].view(np.uint32))
+
+
+def test_selection_inside_gate_up_launch_rejects_batches():
+    table, _ = make_table(capi.FMT_FP8_BLOCK128, 64, 256, 128, 71)
+    ops = DecodeOps(table, None, 2, 2, capi.ACT_BF16, weights_f32=True)
+    x = rand_bf16((2, 256), 1.0, 72).to(DEV)
+    logits = torch.zeros((2, 64), device=DEV)
+    ids = torch.zeros((2, 2), dtype=torch.int32, device=DEV)
+    w = torch.zeros((2, 2), device=DEV)
+    assert ops.contribute_from_logits(x, logits, None, ids, w) is None
