@@ -41,6 +41,8 @@ def parse():
     ap.add_argument("--experts", type=int, default=256)
     ap.add_argument("--ring", type=int, default=64, help="distinct token batches cycled through")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--one-launch", action="store_true", help="one token: selection, gate/up, down and combine in the one resident "
+                    "launch (ffmoe_decode_token_layer) instead of launches of their own")
     ap.add_argument("--separate-topk", action="store_true", help="one token: run the top-k selection as a launch of its own "
                     "instead of in the prologue of the gate/up launch")
     ap.add_argument("--graph", action="store_true", help="replay one HIP graph per ring slot instead of launching eagerly "
@@ -96,6 +98,7 @@ def build_layer(args, torch, capi, ops, synth, make_tokens=True):
     layer = ops.NativeMoe(table, shared, router, bias, args.batch, K, routed_scaling=2.5, n_group=8, topk_group=4,
                           swiglu=capi.SWIGLU_TWICE, routed_weight=capi.WEIGHT_AFTER_DOWN_BF16, combine_mode=capi.COMBINE_UNGATED)
     layer.inline_select = not args.separate_topk
+    layer.one_launch = args.one_launch
     xs = [synth.normal((args.batch, H), 1.0, args.seed + 1000 + i, device=dev, dtype=torch.bfloat16) for i in range(args.ring)]
     return table, layer, xs, (H, I, E, K)
 

@@ -21,7 +21,7 @@ ERR_NULL, ERR_ALIGN, ERR_SHAPE, ERR_OVERLAP, ERR_UNSUPPORTED, ERR_SCRATCH = -1, 
 EXPORTS = [
     "ffmoe_last_error", "ffmoe_version",
     "ffmoe_route_logits_bf16", "ffmoe_route_logits_f32", "ffmoe_route_topk", "ffmoe_route_topk_noaux", "ffmoe_route_noaux_decode", "ffmoe_route_decode", "ffmoe_slot_publish", "ffmoe_route_mask",
-    "ffmoe_decode_scratch_bytes", "ffmoe_decode_contribute", "ffmoe_decode_contribute_stage", "ffmoe_decode_finish", "ffmoe_decode_contribute_from_logits",
+    "ffmoe_decode_scratch_bytes", "ffmoe_decode_contribute", "ffmoe_decode_contribute_stage", "ffmoe_decode_finish", "ffmoe_decode_contribute_from_logits", "ffmoe_decode_token_layer",
     "ffmoe_quant_fp8_f32_128", "ffmoe_linear_fp8_block_w8a8", "ffmoe_linear_fp8_block", "ffmoe_linear_nvfp4",
     "ffmoe_gemm_skinny_bf16", "ffmoe_swiglu",
     "ffmoe_shared_scale", "ffmoe_combine",
@@ -97,6 +97,8 @@ def lib():
         L.ffmoe_combine.argtypes = [P, P, P, P, P, P, P, P, I, I, I, I, P]
         L.ffmoe_decode_contribute_from_logits.argtypes = [ctypes.POINTER(ExpertTable), ctypes.POINTER(SharedExpert), ctypes.POINTER(Decode),
                                                           P, P, I, F, I, I, P]
+        L.ffmoe_decode_token_layer.argtypes = [ctypes.POINTER(ExpertTable), ctypes.POINTER(SharedExpert), ctypes.POINTER(Decode),
+                                               P, P, I, F, I, I, P, P, P, I, P]
         L.ffmoe_decode_finish.argtypes = [ctypes.POINTER(ExpertTable), ctypes.POINTER(SharedExpert), ctypes.POINTER(Decode), P, P, P, I, P]
         L.ffmoe_combine_residual.argtypes = [P, P, P, P, P, ctypes.c_longlong, P, P, P, P, P, P, I, I, I, P]
         L.ffmoe_prefill_scratch_bytes.restype = U64

@@ -2,6 +2,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <type_traits>
 
 namespace ffmoe {
 
@@ -240,6 +241,33 @@ __device__ __forceinline__ T load_global(const void* p) {
   return *(const FF_GLOBAL T*)(p);
 }
 __device__ __forceinline__ u32x4 load16(const void* p) { return load_global<u32x4>(p); }
+// f(std::integral_constant<int, 0>{}) ... f(std::integral_constant<int, N - 1>{}): a loop whose index is a constant
+// expression in the body (register arrays indexed by it stay in registers)
+template <int N, int I = 0, class Fn>
+__device__ __forceinline__ void static_for(Fn&& f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    static_for<N, I + 1>(f);
+  }
+}
+// LDS hand-over between the lanes of ONE wave: earlier LDS writes of the wave are complete and later reads are not
+// moved above this point (LDS operations of a wave execute in order; the fence also stops the compiler).
+__device__ __forceinline__ void wave_lds_fence() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+}
+// Device-coherent accesses (relaxed, agent scope): the store is written through to memory and the load is served from
+// there, so blocks on different XCDs (each with its own L2) can hand data to each other inside one kernel without
+// cache-wide write-back / invalidate operations. Ordering comes from a counter the consumer polls the same way.
+__device__ __forceinline__ void store_agent(uint16_t* p, uint16_t v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ void store_agent(uint32_t* p, uint32_t v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ u32x4 load16_agent(const void* p) {
+  const uint64_t* q = reinterpret_cast<const uint64_t*>(p);
+  const uint64_t a = __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  const uint64_t b = __hip_atomic_load(q + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return u32x4{uint32_t(a), uint32_t(a >> 32), uint32_t(b), uint32_t(b >> 32)};
+}
 // Streaming 16-byte load for data read exactly once (weights): the non-temporal hint keeps it from
 // displacing reusable lines.
 __device__ __forceinline__ u32x4 load16_stream(const void* p) {

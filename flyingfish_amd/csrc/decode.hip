@@ -3,6 +3,8 @@
 #include "common.cuh"
 #include "api.h"
 #include "decode.h"
+#include <atomic>
+#include <stdlib.h>
 
 namespace ffmoe {
 
@@ -12,10 +14,46 @@ int decode_launch_bf16(const DecodeParams& p, int rg, int stage_mask, hipStream_
 int decode_finish_fp8(const FinishParams& q, hipStream_t st);
 int decode_finish_nvfp4(const FinishParams& q, hipStream_t st);
 int decode_finish_bf16(const FinishParams& q, hipStream_t st);
+int decode_token_layer_fp8(const FinishParams& q, hipStream_t st);
+int decode_token_layer_nvfp4(const FinishParams& q, hipStream_t st);
+int decode_token_layer_bf16(const FinishParams& q, hipStream_t st);
 int prefill_impl(const ffmoe_expert_table* table, const ffmoe_prefill* args, int stages, void* stream);
 }  // namespace ffmoe
 
 namespace ffmoe {
+
+// Device-side state of the one-launch token layer, zero when the module is loaded: the launch counter whose low 16
+// bits tag the activations of a launch, and 16 slots of {exit counter, 128 claim counters}, every counter on its own
+// 128-byte line. Calls take slots round-robin, so launches in flight on different streams do not share counters.
+// Every launch leaves its slot at zero.
+#define FFMOE_TOKEN_SLOTS 16
+#define FFMOE_TOKEN_SLOT_WORDS (129 * 32)
+static __device__ __align__(256) unsigned int g_token_state[32 + FFMOE_TOKEN_SLOTS * FFMOE_TOKEN_SLOT_WORDS];
+
+static bool token_layer_sync(FinishParams* q) {
+  static std::atomic<unsigned int*> base[16];
+  static std::atomic<unsigned int> next{0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return false;
+  unsigned int* b = base[dev].load(std::memory_order_acquire);
+  if (!b) {
+    if (hipGetSymbolAddress((void**)&b, HIP_SYMBOL(g_token_state)) != hipSuccess || !b) {
+      (void)hipGetLastError();
+      return false;
+    }
+    base[dev].store(b, std::memory_order_release);
+  }
+  static const unsigned int limit = [] {
+    const char* e = getenv("FFMOE_TOKEN_SPIN_LIMIT");
+    return e ? (unsigned int)strtoul(e, nullptr, 10) : 100000u;
+  }();
+  const unsigned int slot = next.fetch_add(1, std::memory_order_relaxed) % FFMOE_TOKEN_SLOTS;
+  q->gen = b;
+  q->exited = b + 32 + slot * FFMOE_TOKEN_SLOT_WORDS;
+  q->claims = q->exited + 32;
+  q->spin_limit = limit;
+  return true;
+}
 
 // ---------------------------------------------------------------------------------------------
 // Gather assignments by expert into groups of at most RGMAX rows (single block; A <= FFMOE_DECODE_MAX_ASSIGN).
@@ -84,7 +122,8 @@ extern "C" __attribute__((visibility("default"))) uint64_t ffmoe_decode_scratch_
   if (rows < 1 || top_k < 1 || experts < 1 || inter < 1) return 0;
   const uint64_t A = uint64_t(rows) * top_k;
   const uint64_t imax = uint64_t(inter > shared_inter ? inter : shared_inter);
-  const uint64_t h = ((A + rows) * imax * 2 + 255) & ~uint64_t(255);
+  // one token: the one-launch layer keeps its activations as 32-bit tagged words
+  const uint64_t h = ((A + rows) * imax * (rows == 1 ? 4 : 2) + 255) & ~uint64_t(255);
   (void)experts;
   const uint64_t max_groups = A + rows + 2;  // worst case: one row per group
   const uint64_t groups = (max_groups * sizeof(GroupDesc) + 255) & ~uint64_t(255);
@@ -203,6 +242,16 @@ static int decode_impl(const ffmoe_expert_table* table, const ffmoe_shared_exper
   if (fin) {
     FinishParams q = *fin;
     q.d = p;
+    if (q.whole) {
+      if (!token_layer_sync(&q)) return ff_fail(FFMOE_ERR_UNSUPPORTED, "one-launch token layer: no device counters on this device");
+      q.h32 = (uint32_t*)sc;
+      q.d.h_stride = imax;
+      switch (fmt) {
+        case FFMOE_FMT_FP8_BLOCK128: return decode_token_layer_fp8(q, st);
+        case FFMOE_FMT_NVFP4: return decode_token_layer_nvfp4(q, st);
+        default: return decode_token_layer_bf16(q, st);
+      }
+    }
     switch (fmt) {
       case FFMOE_FMT_FP8_BLOCK128: return decode_finish_fp8(q, st);
       case FFMOE_FMT_NVFP4: return decode_finish_nvfp4(q, st);
@@ -300,4 +349,46 @@ extern "C" __attribute__((visibility("default"))) int ffmoe_decode_contribute_fr
   if (bias) FF_PTR4(bias);
   const RouteInline route{logits, bias, score_mode, n_group, topk_group, routed_scaling};
   return decode_impl(table, shared, args, 3, stream, -1, 0, nullptr, &route);
+}
+
+extern "C" __attribute__((visibility("default"))) int ffmoe_decode_token_layer(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared,
+                                                                              const ffmoe_decode* args, const float* logits, const float* bias,
+                                                                              int score_mode, float routed_scaling, int n_group, int topk_group,
+                                                                              const void* scale, void* y, uint32_t* status, int combine_mode,
+                                                                              void* stream) {
+  FF_REQUIRE(table && args, FFMOE_ERR_NULL, "table/args is NULL");
+  FF_REQUIRE(args->rows == 1, FFMOE_ERR_UNSUPPORTED, "ffmoe_decode_token_layer handles one token row (rows=%d)", args->rows);
+  FF_REQUIRE(args->act_mode == FFMOE_ACT_BF16, FFMOE_ERR_UNSUPPORTED, "ffmoe_decode_token_layer needs FFMOE_ACT_BF16");
+  FF_REQUIRE(!shared || shared->format == table->format, FFMOE_ERR_UNSUPPORTED, "ffmoe_decode_token_layer needs the shared expert in the table's format");
+  FF_REQUIRE(combine_mode >= 0 && combine_mode <= FFMOE_COMBINE_ROUTED, FFMOE_ERR_UNSUPPORTED, "unknown combine mode %d", combine_mode);
+  FF_REQUIRE(shared || combine_mode == FFMOE_COMBINE_ROUTED, FFMOE_ERR_SHAPE, "combine mode %d needs a shared expert", combine_mode);
+  FF_PTR16(y);
+  if (combine_mode == FFMOE_COMBINE_GATED) FF_PTR2(scale);
+  if (status) FF_PTR4(status);
+  FF_NO_OVERLAP(y, size_t(table->hidden) * 2, args->scratch, args->scratch_bytes);
+  FF_NO_OVERLAP(y, size_t(table->hidden) * 2, args->x, size_t(table->hidden) * 2);
+  RouteInline route{nullptr, nullptr, 0, 1, 1, 1.0f};
+  if (logits) {
+    FF_REQUIRE(args->weights_f32 == 1 && args->active == nullptr && args->assignment_gen == nullptr, FFMOE_ERR_UNSUPPORTED,
+               "selection inside the launch writes f32 weights and takes no active mask or epochs");
+    const int E = table->experts, K = args->top_k;
+    FF_REQUIRE(E == 64 || E == 128 || E == 256 || E == 512 || E == 1024, FFMOE_ERR_UNSUPPORTED, "experts=%d is not 64 * 2^n", E);
+    FF_REQUIRE(K >= 1 && K <= FFMOE_MAX_TOP_K && K < E, FFMOE_ERR_SHAPE, "top_k=%d out of range", K);
+    FF_REQUIRE(score_mode == FFMOE_NOAUX_SIGMOID || score_mode == FFMOE_NOAUX_SQRTSOFTPLUS, FFMOE_ERR_UNSUPPORTED, "unknown score mode %d", score_mode);
+    FF_REQUIRE(routed_scaling > 0.0f && routed_scaling < INFINITY, FFMOE_ERR_SHAPE, "routed_scaling=%g", (double)routed_scaling);
+    FF_REQUIRE(n_group >= 1 && topk_group >= 1 && topk_group <= n_group && E % n_group == 0, FFMOE_ERR_SHAPE, "n_group=%d topk_group=%d", n_group, topk_group);
+    if (n_group > 1) {
+      const int c = E / 64, per = E / n_group;
+      FF_REQUIRE(per % c == 0 && ((per / c) & (per / c - 1)) == 0 && topk_group * per >= K, FFMOE_ERR_UNSUPPORTED,
+                 "groups of %d experts do not tile the wave, or the kept groups hold fewer than top_k experts", per);
+    }
+    FF_PTR4(logits);
+    if (bias) FF_PTR4(bias);
+    route = RouteInline{logits, bias, score_mode, n_group, topk_group, routed_scaling};
+  }
+  FinishParams fin{};
+  fin.scale = (const uint16_t*)scale; fin.y = (uint16_t*)y; fin.status = status; fin.mode = combine_mode; fin.whole = 1;
+  // the shared expert takes part only in the modes that add it
+  const ffmoe_shared_expert* sh = combine_mode == FFMOE_COMBINE_ROUTED ? nullptr : shared;
+  return decode_impl(table, sh, args, 0, stream, -1, 0, &fin, logits ? &route : nullptr);
 }

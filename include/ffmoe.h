@@ -202,6 +202,24 @@ int ffmoe_decode_contribute_from_logits(const ffmoe_expert_table* table, const f
                                         const ffmoe_decode* args, const float* logits, const float* bias,
                                         int score_mode, float routed_scaling, int n_group, int topk_group, void* stream);
 
+/* One token, everything after the router logits in ONE launch: top-k selection (when logits != NULL; same arithmetic as
+ * ffmoe_route_topk_noaux, args->ids and args->weights (f32) are then OUTPUTS), gate/up + SwiGLU, down, routing weight
+ * and the ordered combine into y [hidden] BF16. Replaces the launches moe_route_select_noaux, moe_gate_up, moe_down /
+ * moe_ffn_weight_f32 and moe_combine* of NativeMoe::run for one token (src/backend/cuda/moe/decode.rs:1187-1297); ids,
+ * weights and y are bit-identical to those launches. logits == NULL: args->ids / weights / active are inputs as in
+ * ffmoe_decode_contribute. The grid stays resident and hands activations between its blocks through args->scratch
+ * (ffmoe_decode_scratch_bytes bytes, which must have been zero-filled ONCE before the first call that uses it: a word
+ * of the arena counts as an activation of this launch only if it carries the launch's non-zero tag);
+ * contributions, shared_out and done are not written. Bit 0 of *status is set for
+ * a live choice naming an expert that is out of range or not valid (its contribution is skipped), bit 1 if a block
+ * gave up waiting for another (y is then not valid; happens only when the grid cannot be resident at once, e.g. two
+ * such launches running concurrently on one GPU, each holding part of the CUs). FFMOE_ERR_UNSUPPORTED (nothing
+ * launched): rows != 1, a shape outside the kernel's register buffers, or a shared expert of another format; use
+ * the separate calls then. */
+int ffmoe_decode_token_layer(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared, const ffmoe_decode* args,
+                             const float* logits, const float* bias, int score_mode, float routed_scaling, int n_group,
+                             int topk_group, const void* scale, void* y, uint32_t* status, int combine_mode, void* stream);
+
 /* One-token finish: the down projection of every live choice and of the shared expert, the routing weight and the
  * ordered combine in ONE launch, for rows == 1. Call after ffmoe_decode_contribute_stage(table, shared, args, 0, stream)
  * with the same table / shared / args (the gate/up activations are taken from args->scratch); writes y[hidden] and
