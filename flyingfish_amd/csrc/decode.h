@@ -63,6 +63,7 @@ struct FinishParams {
   unsigned int* exited;   // blocks that left the kernel; the last one clears it and advances gen
   unsigned int* claims;   // 128 claim counters, 32 words apart: gate/up and down phase of up to 64 grid partitions
   unsigned int spin_limit;
+  int dynamic;            // 1: work items claimed from the counters, 0: fixed round-robin shares
 };
 
 }  // namespace ffmoe

@@ -52,6 +52,8 @@ static bool token_layer_sync(FinishParams* q) {
   q->exited = b + 32 + slot * FFMOE_TOKEN_SLOT_WORDS;
   q->claims = q->exited + 32;
   q->spin_limit = limit;
+  static const int dynamic = [] { const char* e = getenv("FFMOE_TOKEN_STATIC"); return (e && e[0] == '1') ? 0 : 1; }();
+  q->dynamic = dynamic;
   return true;
 }
 

@@ -69,7 +69,7 @@ __global__ __launch_bounds__(256) void k_token_layer(const FinishParams q) {
   // to the older wave of its SIMD for the whole kernel), and with fixed shares the slow half of the grid finishes long
   // after the fast half has gone idle. The grid is split into NP partitions (block index mod NP), each with its own
   // claim counters: a device-wide atomic on one address takes tens of nanoseconds, so the claims are spread over NP
-  // addresses; partition k owns the work items c * NP + k. A wave's first
+  // addresses; item_of() below says which items a partition owns. A wave's first
   // two items per phase are fixed (claims 0 .. 2 * waves - 1 of its partition), the rest come from the counter, always
   // two items ahead of the one being computed, so the atomic's round trip is never waited for.
   const int NP = (gridDim.x & 63) == 0 ? 64 : ((gridDim.x & 7) == 0 ? 8 : 1);
@@ -81,6 +81,10 @@ __global__ __launch_bounds__(256) void k_token_layer(const FinishParams q) {
   unsigned int* cnt_dn = q.claims + (64 + part) * 32;
   // The claim is an atomic INCREMENT (wrap bound 2^32 - 1), not an add: the compiler rewrites a wave's atomic adds
   // into one aggregated add whose result it needs at once, and that wait would drain the wave's weight requests.
+  // Work item of claim c of this partition: the item space is cut into runs of `pwaves` consecutive items dealt
+  // round-robin to the partitions, so the waves of a block (and the blocks of a partition, which share an XCD) work on
+  // neighbouring weight rows at the same time.
+  auto item_of = [&](int c) { return ((c / pwaves) * NP + part) * pwaves + (c % pwaves); };
   auto claim_request = [&](unsigned int* cnt, int& pend) {
     if (lane == 0) pend = int(__builtin_amdgcn_atomic_inc32(cnt, 0xffffffffu, __ATOMIC_RELAXED, "agent"));
   };
@@ -112,8 +116,9 @@ __global__ __launch_bounds__(256) void k_token_layer(const FinishParams q) {
     F::load(gbuf[0][s], r[0], cc);
     F::load(gbuf[1][s], r[1], cc);
   };
-  int f_cur = pw * NP + part;             // fixed claims 0 and 1
-  int f_nxt = (pwaves + pw) * NP + part;
+  int f_cur = item_of(pw);            // fixed claims 0 and 1
+  int f_nxt = item_of(pwaves + pw);
+  int f_claim = pwaves + pw;          // claim index of f_nxt (fixed shares only)
   int cpos = 0, cj = 0;
   // the token is requested ahead of the weights (loads return in order) and written to LDS behind them
   constexpr int XV = 4;
@@ -191,7 +196,7 @@ __global__ __launch_bounds__(256) void k_token_layer(const FinishParams q) {
   const int ng = nr + has_shared;
   const int Utot = SIu + nr * I;
 
-  int pend = 0;  // lane 0: claim in flight (the item after f_nxt)
+  int pend = 0;  // lane 0: the claim of the current pass
   bool have = f_cur < Utot;
   if (have && !early) {
     gu_decode(f_cur, cpos, cj);
@@ -199,18 +204,18 @@ __global__ __launch_bounds__(256) void k_token_layer(const FinishParams q) {
 #pragma unroll
     for (int s = 0; s < S0; ++s) gu_issue(crow, s);
   }
-  if (have && f_nxt < Utot) claim_request(cnt_gu, pend);
   auto gu_finish_item = [&](float (&acc)[2][1]) {
     const float g = wave_sum(acc[0][0]), u = wave_sum(acc[1][0]);
     const uint32_t hv = swiglu_bf16(bround(g), bround(u), p.swiglu, p.swiglu_limit);
     const int row = (has_shared && cpos == 0) ? K : cpos - has_shared;
     if (lane == 0) store_agent(q.h32 + size_t(row) * p.h_stride + cj, (tag << 16) | hv);
   };
+  // Every pass computes item f_cur while requesting the weights of f_nxt, and claims the item after that: the claim
+  // goes out first (ahead of the pass's weight requests, so it returns before them) and is read at the end of the
+  // same pass, so no memory operation other than the weight requests is in flight across the loop edge.
   while (have) {
     if (f_nxt >= Utot) break;
-    // the item after next: its claim was requested one item ago, ahead of the loads now in flight
-    const int f_nn = (2 * pwaves + uni(pend)) * NP + part;
-    claim_request(cnt_gu, pend);  // unconditional (a claim past the end is harmless): the loop body stays straight-line
+    if (q.dynamic) claim_request(cnt_gu, pend);
     int npos, nj;
     gu_decode(f_nxt, npos, nj);
     gu_rows(npos, nj, nrow);
@@ -222,7 +227,13 @@ __global__ __launch_bounds__(256) void k_token_layer(const FinishParams q) {
     }
     gu_finish_item(acc);
     cpos = npos; cj = nj;
-    f_cur = f_nxt; f_nxt = f_nn;
+    f_cur = f_nxt;
+    if (q.dynamic) {
+      f_nxt = item_of(2 * pwaves + uni(pend));
+    } else {
+      f_claim += pwaves;
+      f_nxt = item_of(f_claim);
+    }
     crow[0] = nrow[0]; crow[1] = nrow[1];
   }
   // ---- down phase: first rows requested before the activations are looked at ---------------------------------
@@ -232,8 +243,9 @@ __global__ __launch_bounds__(256) void k_token_layer(const FinishParams q) {
   // current item's are consumed (about ng * 2 * inter bytes in flight per wave).
   constexpr int G = FFMOE_TOKEN_GROUPS;
   typename F::Chunk dbuf[G][1][S1];
-  int d_cur = pw * NP + part;             // fixed claims 0 and 1
-  int d_nxt = (pwaves + pw) * NP + part;
+  int d_cur = item_of(pw);            // fixed claims 0 and 1
+  int d_nxt = item_of(pwaves + pw);
+  int d_claim = pwaves + pw;
   // Straight-line requests: a position past the last group reads one 16-byte word of the token instead (the same
   // word for every lane), so the number of loads in flight never depends on a branch and the waits stay exact.
   auto d_issue = [&](auto slot_c, int d) {
@@ -260,10 +272,7 @@ __global__ __launch_bounds__(256) void k_token_layer(const FinishParams q) {
     for (int s = 0; s < S0; ++s) step_compute<F, 2, 1, S0>(gbuf, s, xs, H, nchunks0, s * 64 + lane, 1, acc);
     gu_finish_item(acc);
   }
-  if (d_cur < H) {
-    static_for<G>([&](auto pc) { d_issue(pc, d_cur); });
-    claim_request(cnt_dn, pend);
-  }
+  if (d_cur < H) static_for<G>([&](auto pc) { d_issue(pc, d_cur); });
   // rows of choices that are not live are rewritten too (tagged zeros): every word of the arena carries the tag of the
   // latest launch that used it, so a stale word can never be older than one launch
   {
@@ -346,10 +355,15 @@ __global__ __launch_bounds__(256) void k_token_layer(const FinishParams q) {
     if (lane == 0) q.y[d_cur] = f32_to_bf16(v);
   };
   while (d_nxt < H) {  // d_cur < d_nxt: both valid
-    const int d_nn = (2 * pwaves + uni(pend)) * NP + part;
-    claim_request(cnt_dn, pend);
+    if (q.dynamic) claim_request(cnt_dn, pend);  // the item after d_nxt; read at the end of this pass
     down_row(std::false_type{});
-    d_cur = d_nxt; d_nxt = d_nn;
+    d_cur = d_nxt;
+    if (q.dynamic) {
+      d_nxt = item_of(2 * pwaves + uni(pend));
+    } else {
+      d_claim += pwaves;
+      d_nxt = item_of(d_claim);
+    }
   }
   if (d_cur < H) down_row(std::true_type{});
   __syncthreads();
