@@ -7,7 +7,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libffmoe.so")
-SOURCES = ["api.cpp", "route.hip", "decode.hip", "decode_fp8.hip", "decode_nvfp4.hip", "decode_bf16.hip", "linear.hip", "combine.hip", "prefill.hip"]
+SOURCES = ["api.cpp", "route.hip", "decode.hip", "decode_fp8.hip", "decode_nvfp4.hip", "decode_bf16.hip", "decode_fp8c.hip", "decode_form.hip", "linear.hip", "combine.hip", "prefill.hip"]
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-fvisibility=hidden",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
 
@@ -23,7 +23,7 @@ def _compile(src):
 
 
 def build(verbose=False):
-    with ThreadPoolExecutor(max_workers=min(6, len(SOURCES))) as pool:
+    with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as pool:
         objs = list(pool.map(_compile, SOURCES))
     cmd = ["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs]
     res = subprocess.run(cmd, capture_output=True, text=True)

@@ -11,12 +11,16 @@ namespace ffmoe {
 int decode_launch_fp8(const DecodeParams& p, int rg, int stage_mask, hipStream_t st);
 int decode_launch_nvfp4(const DecodeParams& p, int rg, int stage_mask, hipStream_t st);
 int decode_launch_bf16(const DecodeParams& p, int rg, int stage_mask, hipStream_t st);
+int decode_launch_fp8c(const DecodeParams& p, int rg, int stage_mask, hipStream_t st);
 int decode_finish_fp8(const FinishParams& q, hipStream_t st);
 int decode_finish_nvfp4(const FinishParams& q, hipStream_t st);
 int decode_finish_bf16(const FinishParams& q, hipStream_t st);
+int decode_finish_fp8c(const FinishParams& q, hipStream_t st);
 int decode_token_layer_fp8(const FinishParams& q, hipStream_t st);
 int decode_token_layer_nvfp4(const FinishParams& q, hipStream_t st);
 int decode_token_layer_bf16(const FinishParams& q, hipStream_t st);
+int decode_token_layer_fp8c(const FinishParams& q, hipStream_t st);
+int decode_form_launch(int fmt, int form, const DecodeParams& p, int stage_mask, hipStream_t st);
 int prefill_impl(const ffmoe_expert_table* table, const ffmoe_prefill* args, int stages, void* stream);
 }  // namespace ffmoe
 
@@ -141,7 +145,7 @@ extern "C" __attribute__((visibility("default"))) uint64_t ffmoe_decode_scratch_
 // (both gate/up launches, then both down launches), so neither may overwrite the other's grouping.
 static int decode_impl(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared, const ffmoe_decode* args,
                        int stage_mask, void* stream, int layout_k = -1, int pass = 0, const FinishParams* fin = nullptr,
-                       const RouteInline* route = nullptr) {
+                       const RouteInline* route = nullptr, int form = -1) {
   FF_REQUIRE(table && args, FFMOE_ERR_NULL, "table/args is NULL");
   const int R = args->rows, K = args->top_k, E = table->experts, H = table->hidden, I = table->inter;
   const int LK = layout_k < 0 ? K : layout_k;
@@ -151,10 +155,10 @@ static int decode_impl(const ffmoe_expert_table* table, const ffmoe_shared_exper
              "decode handles at most %d assignments per call (got %lld); use ffmoe_prefill_contribute", FFMOE_DECODE_MAX_ASSIGN,
              (long long)R * K);
   const int fmt = table->format;
-  FF_REQUIRE(fmt == FFMOE_FMT_FP8_BLOCK128 || fmt == FFMOE_FMT_NVFP4 || fmt == FFMOE_FMT_BF16, FFMOE_ERR_UNSUPPORTED,
+  FF_REQUIRE(fmt == FFMOE_FMT_FP8_BLOCK128 || fmt == FFMOE_FMT_NVFP4 || fmt == FFMOE_FMT_BF16 || fmt == FFMOE_FMT_FP8_CHANNEL, FFMOE_ERR_UNSUPPORTED,
              "unknown expert format %d", fmt);
   // every format's granule is a multiple of 4, the largest number of output rows a wave handles per unit
-  const int gran = fmt == FFMOE_FMT_FP8_BLOCK128 ? 128 : (fmt == FFMOE_FMT_NVFP4 ? 32 : 8);
+  const int gran = fmt == FFMOE_FMT_FP8_BLOCK128 ? 128 : (fmt == FFMOE_FMT_NVFP4 ? 32 : (fmt == FFMOE_FMT_FP8_CHANNEL ? 16 : 8));
   FF_REQUIRE(H >= gran && I >= gran && H % gran == 0 && I % gran == 0, FFMOE_ERR_SHAPE,
              "hidden=%d inter=%d must be positive multiples of %d for this format", H, I, gran);
   FF_REQUIRE(args->act_mode == FFMOE_ACT_BF16, FFMOE_ERR_UNSUPPORTED,
@@ -224,6 +228,11 @@ static int decode_impl(const ffmoe_expert_table* table, const ffmoe_shared_exper
   p.h_stride = imax;
   const uint64_t hbytes = ((uint64_t(LA) + R) * imax * 2 + 255) & ~uint64_t(255);
   hipStream_t st = (hipStream_t)stream;
+  if (form >= 0) {  // the reference's reduction orders: one launch block per (rows of a choice), no grouping
+    p.groups = nullptr;
+    p.counters = nullptr;
+    return decode_form_launch(fmt, form, p, stage_mask, st);
+  }
   int rg = 1;
   // LDS budget per block: rg rows of the widest contraction; two blocks per CU must fit in 160 KiB
   if (R > 1) {
@@ -251,18 +260,21 @@ static int decode_impl(const ffmoe_expert_table* table, const ffmoe_shared_exper
       switch (fmt) {
         case FFMOE_FMT_FP8_BLOCK128: return decode_token_layer_fp8(q, st);
         case FFMOE_FMT_NVFP4: return decode_token_layer_nvfp4(q, st);
+        case FFMOE_FMT_FP8_CHANNEL: return decode_token_layer_fp8c(q, st);
         default: return decode_token_layer_bf16(q, st);
       }
     }
     switch (fmt) {
       case FFMOE_FMT_FP8_BLOCK128: return decode_finish_fp8(q, st);
       case FFMOE_FMT_NVFP4: return decode_finish_nvfp4(q, st);
+      case FFMOE_FMT_FP8_CHANNEL: return decode_finish_fp8c(q, st);
       default: return decode_finish_bf16(q, st);
     }
   }
   switch (fmt) {
     case FFMOE_FMT_FP8_BLOCK128: return decode_launch_fp8(p, rg, stage_mask, st);
     case FFMOE_FMT_NVFP4: return decode_launch_nvfp4(p, rg, stage_mask, st);
+    case FFMOE_FMT_FP8_CHANNEL: return decode_launch_fp8c(p, rg, stage_mask, st);
     default: return decode_launch_bf16(p, rg, stage_mask, st);
   }
 }
@@ -393,4 +405,17 @@ extern "C" __attribute__((visibility("default"))) int ffmoe_decode_token_layer(c
   // the shared expert takes part only in the modes that add it
   const ffmoe_shared_expert* sh = combine_mode == FFMOE_COMBINE_ROUTED ? nullptr : shared;
   return decode_impl(table, sh, args, 0, stream, -1, 0, &fin, logits ? &route : nullptr);
+}
+
+extern "C" __attribute__((visibility("default"))) int ffmoe_decode_contribute_form(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared,
+                                                                                  const ffmoe_decode* args, int form, void* stream) {
+  FF_REQUIRE(table && args, FFMOE_ERR_NULL, "table/args is NULL");
+  FF_REQUIRE(form == FFMOE_FORM_LANE16 || form == FFMOE_FORM_LANE8, FFMOE_ERR_UNSUPPORTED, "unknown reduction form %d", form);
+  FF_REQUIRE(table->format == FFMOE_FMT_BF16 || table->format == FFMOE_FMT_FP8_CHANNEL, FFMOE_ERR_UNSUPPORTED,
+             "the reference's reduction orders are built for BF16 and per-channel FP8 experts (format %d)", table->format);
+  FF_REQUIRE(!shared || shared->format == table->format, FFMOE_ERR_UNSUPPORTED, "shared expert format %d differs from the table format %d",
+             shared ? shared->format : -1, table->format);
+  FF_REQUIRE(args->act_mode == FFMOE_ACT_BF16, FFMOE_ERR_UNSUPPORTED, "the reference's reduction orders need FFMOE_ACT_BF16");
+  FF_REQUIRE(args->rows <= 65535 && args->top_k + 1 <= 65535, FFMOE_ERR_SHAPE, "rows=%d top_k=%d exceed the launch grid", args->rows, args->top_k);
+  return decode_impl(table, shared, args, 3, stream, -1, 0, nullptr, nullptr, form);
 }

@@ -34,6 +34,32 @@ struct FmtFp8 {
   }
 };
 
+// E4M3 codes [N,K] with one BF16 scale per output row (the reference's per-channel W8A16 experts,
+// src/experts/catalogue.rs:31-39; effective weight bf16(e4m3(code) * f32(scale)), src/fp8.rs:138-140)
+struct FmtFp8Channel {
+  static constexpr int EPL = 16;
+  struct Chunk { u32x4 codes; uint32_t scale; };  // scale: BF16 bits of the row's scale
+  struct Row { const uint8_t* codes; const uint16_t* scale; };
+  // slot entries: codes [N,K] u8, scales [N] bf16
+  static __device__ __forceinline__ Row row(uint64_t codes, uint64_t scales, float, int j, int K) {
+    Row r;
+    r.codes = reinterpret_cast<const uint8_t*>(codes) + size_t(j) * K;
+    r.scale = reinterpret_cast<const uint16_t*>(scales) + j;
+    return r;
+  }
+  // the scale travels with every chunk (one 2-byte word, the same for all lanes) so that nothing waits for it before
+  // the weights themselves are used
+  static __device__ __forceinline__ void load(Chunk& c, const Row& r, int chunk) {
+    c.codes = load16_stream(r.codes + uint32_t(chunk) * 16u);
+    c.scale = uint32_t(load_global<uint16_t>(r.scale));
+  }
+  static __device__ __forceinline__ void dequant(const Chunk& c, uint32_t* w, bool valid) {
+    const float s = valid ? bf16_to_f32(uint16_t(c.scale)) : 0.0f;  // masked lane: zero scale, zero weights
+#pragma unroll
+    for (int q = 0; q < 4; ++q) dequant4_e4m3(c.codes[q], s, w[2 * q], w[2 * q + 1]);
+  }
+};
+
 struct FmtNvfp4 {
   static constexpr int EPL = 32;
   struct Chunk { u32x4 codes; uint32_t scales; float global; };

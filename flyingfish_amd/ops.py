@@ -39,6 +39,7 @@ class ExpertTable:
     FP8 block slot layout (src/experts/catalogue.rs:180-222): gate codes [I,H], up codes [I,H],
     down codes [H,I], then gate/up scales [ceil(I/128), ceil(H/128)] f32 and down scales
     [ceil(H/128), ceil(I/128)] f32. NVFP4 slot: packed codes then E4M3 group-16 scales, same order.
+    FP8 per-channel slot (catalogue.rs:31-39, :54-61): the three code matrices, then BF16 scales [I], [I], [H].
     """
 
     def __init__(self, fmt, experts, hidden, inter, storage, slots, global_scales=None, valid=None):
@@ -59,6 +60,10 @@ class ExpertTable:
             s = hidden * inter // 16
             offs = [0, 3 * w, w, 3 * w + s, 2 * w, 3 * w + 2 * s]
             size = 3 * w + 3 * s
+        elif fmt == capi.FMT_FP8_CHANNEL:
+            w = hidden * inter
+            offs = [0, 3 * w, w, 3 * w + 2 * inter, 2 * w, 3 * w + 4 * inter]
+            size = 3 * w + 4 * inter + 2 * hidden
         elif fmt == capi.FMT_BF16:
             w = hidden * inter * 2
             offs = [0, 0, w, 0, 2 * w, 0]
@@ -95,6 +100,10 @@ class ExpertTable:
             return (row[o[0]:o[0] + I * H // 2].view(I, H // 2), row[o[1]:o[1] + I * H // 16].view(I, H // 16),
                     row[o[2]:o[2] + I * H // 2].view(I, H // 2), row[o[3]:o[3] + I * H // 16].view(I, H // 16),
                     row[o[4]:o[4] + H * I // 2].view(H, I // 2), row[o[5]:o[5] + H * I // 16].view(H, I // 16))
+        if self.format == capi.FMT_FP8_CHANNEL:
+            sc = lambda off, n: row[off:off + n * 2].view(_BF16)
+            return (row[o[0]:o[0] + I * H].view(I, H), sc(o[1], I), row[o[2]:o[2] + I * H].view(I, H), sc(o[3], I),
+                    row[o[4]:o[4] + H * I].view(H, I), sc(o[5], H))
         bf = lambda off, shape: row[off:off + shape[0] * shape[1] * 2].view(_BF16).view(shape)
         return (bf(o[0], (I, H)), None, bf(o[2], (I, H)), None, bf(o[4], (H, I)), None)
 
@@ -104,6 +113,8 @@ class ExpertTable:
             return 3 * H * I + 4 * (2 * -(-I // 128) * -(-H // 128) + -(-H // 128) * -(-I // 128))
         if self.format == capi.FMT_NVFP4:
             return 3 * H * I // 2 + 3 * H * I // 16 + 12
+        if self.format == capi.FMT_FP8_CHANNEL:
+            return 3 * H * I + 2 * (2 * I + H)
         return 3 * H * I * 2
 
     def c_struct(self):
@@ -230,15 +241,18 @@ class DecodeOps:
         self._table_c = table.c_struct()
         self._shared_c = shared
 
-    def contribute(self, x, ids, weights, active=None, stage=None, assignment_gen=None):
-        """stage None = both launches; 0 / 1 = only the gate-up / only the down launch."""
+    def contribute(self, x, ids, weights, active=None, stage=None, assignment_gen=None, form=None):
+        """stage None = both launches; 0 / 1 = only the gate-up / only the down launch. form = capi.FORM_LANE16 /
+        FORM_LANE8: the reference's own summation orders, bit-equal to its CPU path (DecodeOps::new_invariant_*)."""
         act_mode, swiglu, limit, rw, wf32 = self.cfg
         d = capi.Decode(self.rows, self.top_k, act_mode, swiglu, limit, rw, wf32,
                         x.data_ptr(), ids.data_ptr(), active.data_ptr() if active is not None else None, weights.data_ptr(),
                         self.contributions.data_ptr(), self.shared_out.data_ptr() if self.shared_out is not None else None,
                         self.done.data_ptr(), self.scratch.data_ptr(), self.scratch.numel(), _ptr(assignment_gen))
         sh = ctypes.byref(self._shared_c) if self._shared_c is not None else None
-        if stage is None:
+        if form is not None:
+            capi.check(capi.lib().ffmoe_decode_contribute_form(ctypes.byref(self._table_c), sh, ctypes.byref(d), form, _stream()))
+        elif stage is None:
             capi.check(capi.lib().ffmoe_decode_contribute(ctypes.byref(self._table_c), sh, ctypes.byref(d), _stream()))
         else:
             capi.check(capi.lib().ffmoe_decode_contribute_stage(ctypes.byref(self._table_c), sh, ctypes.byref(d), stage, _stream()))

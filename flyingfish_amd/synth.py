@@ -45,6 +45,15 @@ def quant_fp8_block(w, block=128):
     return codes, scales.contiguous()
 
 
+def quant_fp8_channel(w):
+    """w [N,K] f32 -> (codes uint8 [N,K], scales bf16 [N]): one scale per output row, amax/448 rounded to BF16."""
+    amax = w.abs().amax(dim=1)
+    scales = (amax * torch.tensor(1.0 / 448.0, dtype=torch.float32, device=w.device)).to(torch.bfloat16)
+    div = scales.to(torch.float32).clamp_min(1e-12)[:, None]
+    q = (w / div).clamp(-E4M3_MAX, E4M3_MAX)
+    return e4m3_encode(q).contiguous(), scales.contiguous()
+
+
 def e2m1_encode(x):
     """float32 -> 4-bit E2M1 codes (uint8), thresholds with ties toward the even code."""
     m = x.abs()

@@ -42,6 +42,7 @@ extern "C" {
 #define FFMOE_FMT_FP8_BLOCK128 0  /* E4M3 codes [N,K] + f32 scales [ceil(N/128), ceil(K/128)] (src/fp8.rs:31-36) */
 #define FFMOE_FMT_NVFP4        1  /* E2M1 pairs [N,K/2] (low nibble = even k) + E4M3 scales [N,K/16] + f32 global */
 #define FFMOE_FMT_BF16         2  /* BF16 [N,K] */
+#define FFMOE_FMT_FP8_CHANNEL  3  /* E4M3 codes [N,K] + one BF16 scale per output row [N] (src/experts/catalogue.rs:31-39) */
 
 /* activation arithmetic of the FP8 linears */
 #define FFMOE_ACT_BF16         0  /* W8A16: w = bf16(e4m3(code) * scale), FP32 accumulate against BF16 activations
@@ -191,6 +192,19 @@ int ffmoe_decode_contribute(const ffmoe_expert_table* table, const ffmoe_shared_
  * same arguments equals ffmoe_decode_contribute. */
 int ffmoe_decode_contribute_stage(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared,
                                   const ffmoe_decode* args, int stage, void* stream);
+
+/* Expert contributions in the reference's own summation orders, bit for bit: the same call as ffmoe_decode_contribute,
+ * but every dot product follows Form::Lane16 or Form::Lane8 of the reference's CPU path
+ * (src/cpu/expert_ffn.rs:689-776; GPU: the invariant kernels moe_ffn_*_lane16, kernels/moe_ffn.cu:364-393, and the
+ * production kernels moe_gate_up / moe_down, kernels/moe_ffn.cu:98-302), with the SiLU form that goes with it, so
+ * contributions and shared_out equal the CPU path's to the last bit (mixed CPU / GPU expert tiering stays
+ * reproducible). Replaces DecodeOps::new_invariant_with_boundaries + contribute (src/backend/cuda/moe/decode.rs:342-520).
+ * FFMOE_FMT_BF16 and FFMOE_FMT_FP8_CHANNEL tables only (the formats the CPU path executes); slower than
+ * ffmoe_decode_contribute, whose 64-lane sums match these orders to 2 BF16 ulp. */
+#define FFMOE_FORM_LANE16 0
+#define FFMOE_FORM_LANE8  1
+int ffmoe_decode_contribute_form(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared, const ffmoe_decode* args,
+                                 int form, void* stream);
 
 /* One token, selection inside the gate/up launch: logits [experts] FP32 (from ffmoe_route_logits_f32) go in, and the
  * top-k selection of ffmoe_route_topk_noaux (same arithmetic, bit for bit) runs in the prologue of every block of the

@@ -42,6 +42,11 @@ def make_table(fmt, experts, hidden, inter, seed, device="cuda", std=0.02):
                 views[2 * i + 1].copy_(scales)
                 gl.append(g)
                 eff.append(orc.dequant_nvfp4(codes.numpy(), scales.numpy(), g))
+            elif fmt == capi.FMT_FP8_CHANNEL:
+                codes, scales = synth.quant_fp8_channel(w)
+                views[2 * i].copy_(codes)
+                views[2 * i + 1].copy_(scales)
+                eff.append(orc.dequant_fp8_channel(codes.numpy(), bits(scales)))
             else:
                 wb = w.to(torch.bfloat16)
                 views[2 * i].copy_(wb)
