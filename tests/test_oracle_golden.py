@@ -602,3 +602,35 @@ def test_combine_modes_small_brute_force():
             for k in range(K):
                 t = np.float32(t + cf[r, k, d])
             assert acc[r, d] == rb(np.float32(t + sf[r, d]))
+
+
+def test_dot_form_order_witnesses():
+    """Inputs on which the two summation orders of src/cpu/expert_ffn.rs:689-776 (and a plain chain) give different,
+    hand-computable results, so a wrong lane index, a chain instead of a tree or a wrong pairing fails."""
+    def w_of(values, n):
+        w = np.zeros(n, dtype=np.float32)
+        for k, v in values.items():
+            w[k] = v
+        return orc.f32_to_bf16(w)
+
+    big = float(2 ** 27)
+    # element k goes to Lane16 accumulator k % 16: 0 and 16 cancel exactly, the 1.0 at element 1 survives. Lane8 sums
+    # elements 0..7 in one chain first: 2^27 + 1 loses the 1.
+    w = w_of({0: big, 16: -big, 1: 1.0}, 32)
+    x = np.ones(32, dtype=np.float32)
+    assert orc.dot(x, w, orc.LANE16) == 1.0
+    assert orc.dot(x, w, orc.LANE8) == 0.0
+    # Lane16 ends in a pairwise tree ((l0+l1)+(l2+l3))...: (2^24+1) -> 2^24, (1-2^24) exact, sum 1. A chain gives 0.
+    t = float(2 ** 24)
+    w = w_of({0: t, 1: 1.0, 2: 1.0, 3: -t}, 16)
+    assert orc.dot(np.ones(16, dtype=np.float32), w, orc.LANE16) == 1.0
+    # Lane8 pairs accumulator 0 with 4 first: vectors 0 and 4 cancel, vector 1 survives; pairing 0 with 1 would lose it.
+    w = w_of({0: t, 32: -t, 8: 1.0}, 64)
+    assert orc.dot(np.ones(64, dtype=np.float32), w, orc.LANE8) == 1.0
+    # and inside a Lane8 vector the eight products are a chain from zero: 2^24, +1 (lost), -2^24 -> 0, not 1
+    w = w_of({0: t, 1: 1.0, 2: -t}, 8)
+    assert orc.dot(np.ones(8, dtype=np.float32), w, orc.LANE8) == 0.0
+    # while Lane16 keeps them in three different accumulators: (2^24 + 1) + (-2^24 + 0) = 2^24 - 2^24 = 0 as well, but
+    # with the 1 moved next to its partner in the tree (element 3) it survives: (2^24 + 0) + (-2^24 + 1)
+    w = w_of({0: t, 2: -t, 3: 1.0}, 16)
+    assert orc.dot(np.ones(16, dtype=np.float32), w, orc.LANE16) == 1.0
