@@ -32,8 +32,10 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", choices=["decode", "prefill"], default="decode",
-                    help="decode = BASELINE config 3 (the headline line); prefill = config 5 (4096 tokens, Zipf s=1.1, FP8 matrix cores)")
+    ap.add_argument("--workload", choices=["decode", "prefill", "widening"], default="decode",
+                    help="decode = BASELINE config 3 (the headline line); prefill = config 5 (4096 tokens, Zipf s=1.1, FP8 matrix cores); "
+                         "widening = the formats and fused steps next to the path (per-channel FP8 / BF16 experts, Lane16 / Lane8 orders, "
+                         "combine + residual)")
     ap.add_argument("--batch", type=int, default=None, help="tokens per step (decode: 1, 8, 64; prefill: 4096)")
     ap.add_argument("--format", choices=["fp8", "nvfp4"], default="fp8",
                     help="routed-expert format: fp8 = config 3 (shared expert FP8 too); nvfp4 = config 4 (NVFP4 routed experts, "
@@ -246,6 +248,74 @@ def prefill_main(args, torch, capi, ops, synth):
     print(json.dumps(out))
 
 
+def widening_main(args, torch, capi, ops, synth):
+    """The rows next to the headline path, timed at the DeepSeek-V3 layer shape with one token (8 of 16 experts +
+    shared expert, weights = random codes, resident): per-channel FP8 and BF16 experts on the streaming decode path,
+    the same experts in the reference's Lane16 / Lane8 summation orders (ffmoe_decode_contribute_form), and the fused
+    combine + shared gate + residual add. One JSON line; value = the per-channel FP8 streaming contribution."""
+    H, I, E, K = 7168, 2048, 16, 8
+    dev = "cuda"
+    g = torch.Generator(device="cpu").manual_seed(args.seed)
+    xs = [synth.normal((1, H), 1.0, args.seed + 1000 + i, device=dev, dtype=torch.bfloat16) for i in range(8)]
+    idl = [torch.randperm(E, generator=g)[:K].reshape(1, K).to(torch.int32).to(dev) for _ in range(8)]
+    w = (torch.rand((1, K), generator=g) * 0.5 + 0.05).to(dev)
+
+    def timed(fn, n):
+        for i in range(5):
+            fn(i)
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for i in range(n):
+            fn(i)
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) * 1e3 / n
+
+    rows = {}
+    for name, fmt in (("fp8_per_channel", capi.FMT_FP8_CHANNEL), ("bf16", capi.FMT_BF16)):
+        table = ops.ExpertTable.allocate(fmt, E + 1, H, I, dev)
+        for e in range(E + 1):
+            v = table.expert_views(e)
+            for i in range(3):
+                if fmt == capi.FMT_FP8_CHANNEL:
+                    v[2 * i].random_(0, 120)
+                    v[2 * i + 1].fill_(0.001)
+                else:
+                    v[2 * i].normal_(0.0, 0.02)
+        shared = table.shared_struct(E)
+        table.experts = E
+        dec = ops.DecodeOps(table, shared, 1, K, weights_f32=True)
+        nbytes = (K + 1) * table.weight_bytes_per_expert()
+        us = timed(lambda i: dec.contribute(xs[i % 8], idl[i % 8], w), args.steps)
+        rows[name] = {"streaming_us": us, "weight_bytes": nbytes, "streaming_gbps": nbytes / (us * 1e-6) / 1e9,
+                      "streaming_hbm_frac": nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS}
+        for fname, form in (("lane16", capi.FORM_LANE16), ("lane8", capi.FORM_LANE8)):
+            us_f = timed(lambda i: dec.contribute(xs[i % 8], idl[i % 8], w, form=form), max(4, args.steps // 8))
+            rows[name][fname + "_us"] = us_f
+            rows[name][fname + "_gbps"] = nbytes / (us_f * 1e-6) / 1e9
+        del dec, table
+    # fused combine + shared gate + residual (one token and 64 tokens)
+    for R in (1, 64):
+        contrib = synth.normal((R, K, H), 0.05, 3, device=dev, dtype=torch.bfloat16)
+        shared_out = synth.normal((R, H), 0.05, 4, device=dev, dtype=torch.bfloat16)
+        x = synth.normal((R, H), 1.0, 5, device=dev, dtype=torch.bfloat16)
+        resid = synth.normal((R, H), 1.0, 6, device=dev, dtype=torch.bfloat16)
+        seg = synth.normal((H,), 0.02, 7, device=dev, dtype=torch.bfloat16)
+        ids = torch.stack([torch.randperm(E, generator=g)[:K] for _ in range(R)]).to(torch.int32).to(dev)
+        us = timed(lambda i: ops.CombineOps.combine_residual(shared_out, residual=resid, contributions=contrib, ids=ids, seg=seg, x=x), args.steps)
+        rows["combine_residual_rows_%d" % R] = {"us": us, "bytes": R * H * 2 * (K + 4), "gbps": R * H * 2 * (K + 4) / (us * 1e-6) / 1e9}
+    out = {"metric": "moe_decode_contribution_us", "value": rows["fp8_per_channel"]["streaming_us"], "unit": "us/call", "n_gpus": 1,
+           "steps": args.steps, "warmup": 5, "ms_per_step": rows["fp8_per_channel"]["streaming_us"] / 1e3, "higher_is_better": False,
+           "scaling": "weak", "vs_baseline": None, "dtype": "fp8_e4m3 (per-channel bf16 scales) / bf16 weights, bf16 activations, f32 accumulate",
+           "data": "synthetic",
+           "config": {"workload": "rows next to the headline path at the DeepSeek-V3 layer shape, one token: per-channel FP8 and BF16 "
+                                  "experts (streaming and Lane16 / Lane8 orders), fused combine + residual",
+                      "hidden": H, "intermediate": I, "experts_resident": E + 1, "top_k": K, "shared_experts": 1},
+           "rows": rows}
+    print(json.dumps(out))
+
+
 def main():
     args = parse()
     if args.batch is None:
@@ -264,6 +334,8 @@ def main():
         if args.steps == 200 and args.warmup == 20:
             args.steps, args.warmup = 10, 2
         return prefill_main(args, torch, capi, ops, synth)
+    if args.workload == "widening":
+        return widening_main(args, torch, capi, ops, synth)
     table, layer, xs, dims = build_layer(args, torch, capi, ops, synth)
     H, I, E, K = dims
     torch.cuda.synchronize()
