@@ -7,7 +7,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libffmoe.so")
-SOURCES = ["api.cpp", "route.hip", "decode.hip", "decode_fp8.hip", "decode_nvfp4.hip", "decode_bf16.hip", "decode_fp8c.hip", "decode_form.hip", "linear.hip", "combine.hip", "prefill.hip"]
+SOURCES = ["api.cpp", "route.hip", "decode.hip", "decode_fp8.hip", "decode_nvfp4.hip", "decode_bf16.hip", "decode_fp8c.hip", "decode_form.hip", "e8m0.hip", "linear.hip", "combine.hip", "prefill.hip"]
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-fvisibility=hidden",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
 

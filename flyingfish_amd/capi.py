@@ -9,11 +9,11 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libffmoe.so")
 
 # enums of include/ffmoe.h
-FMT_FP8_BLOCK128, FMT_NVFP4, FMT_BF16, FMT_FP8_CHANNEL = 0, 1, 2, 3
+FMT_FP8_BLOCK128, FMT_NVFP4, FMT_BF16, FMT_FP8_CHANNEL, FMT_E2M1_E8M0, FMT_E4M3_E8M0_32 = 0, 1, 2, 3, 4, 5
 FORM_LANE16, FORM_LANE8 = 0, 1
-ACT_BF16, ACT_FP8_BLOCK128 = 0, 1
+ACT_BF16, ACT_FP8_BLOCK128, ACT_E4M3_E8M0_32 = 0, 1, 2
 SWIGLU_TWICE, SWIGLU_ONCE, SWIGLU_CLAMPED_TWICE, SWIGLU_CLAMPED_ONCE = 0, 1, 2, 3
-WEIGHT_AFTER_DOWN_BF16, WEIGHT_BEFORE_CONTRIBUTION_BF16 = 0, 1
+WEIGHT_AFTER_DOWN_BF16, WEIGHT_BEFORE_CONTRIBUTION_BF16, WEIGHT_BEFORE_DOWN_F32 = 0, 1, 2
 SCORE_SOFTMAX, SCORE_SIGMOID = 0, 1
 NOAUX_SIGMOID, NOAUX_SQRTSOFTPLUS = 0, 1
 COMBINE_GATED, COMBINE_UNGATED, COMBINE_BF16, COMBINE_ACCUM_FP32, COMBINE_ACCUM_BF16, COMBINE_ROUTED = range(6)
@@ -22,7 +22,7 @@ ERR_NULL, ERR_ALIGN, ERR_SHAPE, ERR_OVERLAP, ERR_UNSUPPORTED, ERR_SCRATCH = -1, 
 EXPORTS = [
     "ffmoe_last_error", "ffmoe_version",
     "ffmoe_route_logits_bf16", "ffmoe_route_logits_f32", "ffmoe_route_topk", "ffmoe_route_topk_noaux", "ffmoe_route_noaux_decode", "ffmoe_route_decode", "ffmoe_slot_publish", "ffmoe_route_mask",
-    "ffmoe_decode_scratch_bytes", "ffmoe_decode_contribute", "ffmoe_decode_contribute_stage", "ffmoe_decode_finish", "ffmoe_decode_contribute_from_logits", "ffmoe_decode_token_layer", "ffmoe_decode_contribute_form",
+    "ffmoe_decode_scratch_bytes", "ffmoe_decode_contribute", "ffmoe_decode_contribute_stage", "ffmoe_decode_finish", "ffmoe_decode_contribute_from_logits", "ffmoe_decode_token_layer", "ffmoe_decode_contribute_form", "ffmoe_e8m0_scratch_bytes", "ffmoe_decode_contribute_e8m0", "ffmoe_act_quant_e8m0",
     "ffmoe_quant_fp8_f32_128", "ffmoe_linear_fp8_block_w8a8", "ffmoe_linear_fp8_block", "ffmoe_linear_nvfp4",
     "ffmoe_gemm_skinny_bf16", "ffmoe_swiglu",
     "ffmoe_shared_scale", "ffmoe_combine",
@@ -101,6 +101,10 @@ def lib():
         L.ffmoe_decode_token_layer.argtypes = [ctypes.POINTER(ExpertTable), ctypes.POINTER(SharedExpert), ctypes.POINTER(Decode),
                                                P, P, I, F, I, I, P, P, P, I, P]
         L.ffmoe_decode_contribute_form.argtypes = [ctypes.POINTER(ExpertTable), ctypes.POINTER(SharedExpert), ctypes.POINTER(Decode), I, P]
+        L.ffmoe_e8m0_scratch_bytes.restype = ctypes.c_uint64
+        L.ffmoe_e8m0_scratch_bytes.argtypes = [I, I, I, I, I]
+        L.ffmoe_decode_contribute_e8m0.argtypes = [ctypes.POINTER(ExpertTable), ctypes.POINTER(SharedExpert), ctypes.POINTER(Decode), P]
+        L.ffmoe_act_quant_e8m0.argtypes = [P, P, P, I, I, P]
         L.ffmoe_decode_finish.argtypes = [ctypes.POINTER(ExpertTable), ctypes.POINTER(SharedExpert), ctypes.POINTER(Decode), P, P, P, I, P]
         L.ffmoe_combine_residual.argtypes = [P, P, P, P, P, ctypes.c_longlong, P, P, P, P, P, P, I, I, I, P]
         L.ffmoe_prefill_scratch_bytes.restype = U64

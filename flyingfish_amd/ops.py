@@ -64,6 +64,17 @@ class ExpertTable:
             w = hidden * inter
             offs = [0, 3 * w, w, 3 * w + 2 * inter, 2 * w, 3 * w + 4 * inter]
             size = 3 * w + 4 * inter + 2 * hidden
+        elif fmt == capi.FMT_E2M1_E8M0:
+            w = hidden * inter // 2
+            s = hidden * inter // 32
+            offs = [0, 3 * w, w, 3 * w + s, 2 * w, 3 * w + 2 * s]
+            size = 3 * w + 3 * s
+        elif fmt == capi.FMT_E4M3_E8M0_32:
+            w = hidden * inter
+            sgu = -(-inter // 32) * (hidden // 32)
+            sd = -(-hidden // 32) * (inter // 32)
+            offs = [0, 3 * w, w, 3 * w + sgu, 2 * w, 3 * w + 2 * sgu]
+            size = 3 * w + 2 * sgu + sd
         elif fmt == capi.FMT_BF16:
             w = hidden * inter * 2
             offs = [0, 0, w, 0, 2 * w, 0]
@@ -100,6 +111,15 @@ class ExpertTable:
             return (row[o[0]:o[0] + I * H // 2].view(I, H // 2), row[o[1]:o[1] + I * H // 16].view(I, H // 16),
                     row[o[2]:o[2] + I * H // 2].view(I, H // 2), row[o[3]:o[3] + I * H // 16].view(I, H // 16),
                     row[o[4]:o[4] + H * I // 2].view(H, I // 2), row[o[5]:o[5] + H * I // 16].view(H, I // 16))
+        if self.format == capi.FMT_E2M1_E8M0:
+            return (row[o[0]:o[0] + I * H // 2].view(I, H // 2), row[o[1]:o[1] + I * H // 32].view(I, H // 32),
+                    row[o[2]:o[2] + I * H // 2].view(I, H // 2), row[o[3]:o[3] + I * H // 32].view(I, H // 32),
+                    row[o[4]:o[4] + H * I // 2].view(H, I // 2), row[o[5]:o[5] + H * I // 32].view(H, I // 32))
+        if self.format == capi.FMT_E4M3_E8M0_32:
+            gi, gh = -(-I // 32), -(-H // 32)
+            return (row[o[0]:o[0] + I * H].view(I, H), row[o[1]:o[1] + gi * (H // 32)].view(gi, H // 32),
+                    row[o[2]:o[2] + I * H].view(I, H), row[o[3]:o[3] + gi * (H // 32)].view(gi, H // 32),
+                    row[o[4]:o[4] + H * I].view(H, I), row[o[5]:o[5] + gh * (I // 32)].view(gh, I // 32))
         if self.format == capi.FMT_FP8_CHANNEL:
             sc = lambda off, n: row[off:off + n * 2].view(_BF16)
             return (row[o[0]:o[0] + I * H].view(I, H), sc(o[1], I), row[o[2]:o[2] + I * H].view(I, H), sc(o[3], I),
@@ -115,6 +135,10 @@ class ExpertTable:
             return 3 * H * I // 2 + 3 * H * I // 16 + 12
         if self.format == capi.FMT_FP8_CHANNEL:
             return 3 * H * I + 2 * (2 * I + H)
+        if self.format == capi.FMT_E2M1_E8M0:
+            return 3 * H * I // 2 + 3 * H * I // 32
+        if self.format == capi.FMT_E4M3_E8M0_32:
+            return 3 * H * I + 2 * -(-I // 32) * (H // 32) + -(-H // 32) * (I // 32)
         return 3 * H * I * 2
 
     def c_struct(self):
@@ -305,6 +329,41 @@ class DecodeOps:
             return False
         capi.check(rc)
         return True
+
+
+class E8m0DecodeOps:
+    """Expert contributions in the E8M0 block-32 contract (W4A8 routed experts, W8A8 32x32-block shared expert, exact
+    integer dots). Host mirror of MoeExpertW4A8 / the W8A8 shared expert ops (src/backend/cuda/moe/w4a8.rs:248-420),
+    for rows x top_k choices per call; owns its scratch arena and output buffers."""
+
+    def __init__(self, table, shared=None, rows=1, top_k=8, swiglu_limit=10.0):
+        self.table, self.shared, self.rows, self.top_k, self.limit = table, shared, rows, top_k, swiglu_limit
+        dev = table.slots.device
+        si = shared.inter if shared is not None else 0
+        nbytes = capi.lib().ffmoe_e8m0_scratch_bytes(rows, top_k, table.hidden, table.inter, si)
+        self.scratch = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+        self.contributions = torch.empty((rows, max(top_k, 1), table.hidden), dtype=_BF16, device=dev)
+        self.shared_out = torch.empty((rows, table.hidden), dtype=_BF16, device=dev) if shared is not None else None
+        self.done = torch.zeros((rows, max(top_k, 1)), dtype=torch.int32, device=dev)
+        self._table_c = table.c_struct()
+        self._shared_c = shared
+
+    def contribute(self, x, ids, weights, active=None):
+        d = capi.Decode(self.rows, self.top_k, capi.ACT_E4M3_E8M0_32, capi.SWIGLU_CLAMPED_ONCE, self.limit, capi.WEIGHT_BEFORE_DOWN_F32, 1,
+                        x.data_ptr(), ids.data_ptr(), active.data_ptr() if active is not None else None, weights.data_ptr(),
+                        self.contributions.data_ptr(), self.shared_out.data_ptr() if self.shared_out is not None else None,
+                        self.done.data_ptr(), self.scratch.data_ptr(), self.scratch.numel(), None)
+        sh = ctypes.byref(self._shared_c) if self._shared_c is not None else None
+        capi.check(capi.lib().ffmoe_decode_contribute_e8m0(ctypes.byref(self._table_c), sh, ctypes.byref(d), _stream()))
+        return self.contributions, self.shared_out
+
+    @staticmethod
+    def act_quant(x):
+        rows, k = x.shape
+        codes = torch.empty((rows, k), dtype=torch.uint8, device=x.device)
+        scales = torch.empty((rows, k // 32), dtype=torch.uint8, device=x.device)
+        capi.check(capi.lib().ffmoe_act_quant_e8m0(_ptr(_dense(x, "x")), _ptr(codes), _ptr(scales), rows, k, _stream()))
+        return codes, scales
 
 
 class PrefillOps:

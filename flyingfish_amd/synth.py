@@ -54,6 +54,42 @@ def quant_fp8_channel(w):
     return e4m3_encode(q).contiguous(), scales.contiguous()
 
 
+def _pow2_ceil_exponent(v):
+    """ceil(log2(v)) of positive float32 values, from the bit pattern (exact)."""
+    bits = v.to(torch.float32).view(torch.int32)
+    return ((bits >> 23) & 0xff) - 127 + ((bits & 0x7fffff) != 0).to(torch.int32)
+
+
+def quant_e2m1_e8m0(w):
+    """w [N,K] f32 -> (packed E2M1 codes uint8 [N,K/2], low nibble = even k; E8M0 scale codes uint8 [N,K/32]): one
+    power-of-two scale per 32 elements of a row, 2^ceil(log2(amax/6))."""
+    n, k = w.shape
+    blocks = w.view(n, k // 32, 32)
+    amax = blocks.abs().amax(dim=2).clamp_min(2.0 ** -100)
+    exp = _pow2_ceil_exponent(amax / 6.0).clamp(-127, 127)
+    scale = torch.pow(torch.tensor(2.0, dtype=torch.float64, device=w.device), exp.to(torch.float64)).to(torch.float32)
+    q = (blocks / scale[:, :, None]).clamp(-6.0, 6.0).reshape(n, k)
+    codes = e2m1_encode(q)
+    packed = (codes[:, 0::2] | (codes[:, 1::2] << 4)).contiguous()
+    return packed, (exp + 127).to(torch.uint8).contiguous()
+
+
+def quant_e4m3_e8m0_block32(w):
+    """w [N,K] f32 -> (E4M3 codes uint8 [N,K], E8M0 scale codes uint8 [ceil(N/32), K/32]): one power-of-two scale per
+    32x32 block, 2^ceil(log2(amax/448))."""
+    n, k = w.shape
+    gn = -(-n // 32)
+    pad = torch.zeros((gn * 32, k), dtype=torch.float32, device=w.device)
+    pad[:n] = w
+    blocks = pad.view(gn, 32, k // 32, 32)
+    amax = blocks.abs().amax(dim=(1, 3)).clamp_min(2.0 ** -100)
+    exp = _pow2_ceil_exponent(amax / 448.0).clamp(-127, 127)
+    scale = torch.pow(torch.tensor(2.0, dtype=torch.float64, device=w.device), exp.to(torch.float64)).to(torch.float32)
+    q = (blocks / scale[:, None, :, None]).clamp(-E4M3_MAX, E4M3_MAX)
+    codes = e4m3_encode(q).view(gn * 32, k)[:n].contiguous()
+    return codes, (exp + 127).to(torch.uint8).contiguous()
+
+
 def e2m1_encode(x):
     """float32 -> 4-bit E2M1 codes (uint8), thresholds with ties toward the even code."""
     m = x.abs()

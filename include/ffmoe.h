@@ -43,12 +43,16 @@ extern "C" {
 #define FFMOE_FMT_NVFP4        1  /* E2M1 pairs [N,K/2] (low nibble = even k) + E4M3 scales [N,K/16] + f32 global */
 #define FFMOE_FMT_BF16         2  /* BF16 [N,K] */
 #define FFMOE_FMT_FP8_CHANNEL  3  /* E4M3 codes [N,K] + one BF16 scale per output row [N] (src/experts/catalogue.rs:31-39) */
+#define FFMOE_FMT_E2M1_E8M0     4  /* E2M1 pairs [N,K/2] (low nibble = even k) + E8M0 scales [N,K/32] (kernels/moe_ffn.cu:398-403) */
+#define FFMOE_FMT_E4M3_E8M0_32  5  /* E4M3 codes [N,K] + E8M0 scales [ceil(N/32), K/32], one per 32x32 block (kernels/moe_ffn.cu:743-747) */
 
 /* activation arithmetic of the FP8 linears */
 #define FFMOE_ACT_BF16         0  /* W8A16: w = bf16(e4m3(code) * scale), FP32 accumulate against BF16 activations
                                      (src/fp8.rs:138-140, src/cpu/expert_ffn.rs:592-679) */
 #define FFMOE_ACT_FP8_BLOCK128 1  /* W8A8: activations quantized per 128 to E4M3 with an f32 scale, per-128 dot then
                                      one scale product (kernels/fp8_linear.cu:12-48, kernels/q38_contract.cuh:239-279) */
+#define FFMOE_ACT_E4M3_E8M0_32  2  /* activations quantized per 32 to E4M3 with a power-of-two (E8M0) scale, exact integer dots
+                                     (ffmoe_decode_contribute_e8m0 only) */
 
 /* SwiGLU rounding (src/model_spec.rs:61-69; src/cpu/expert_ffn.rs:58-100) */
 #define FFMOE_SWIGLU_TWICE          0  /* a = bf16(bf16(silu(g)) * u) */
@@ -59,6 +63,8 @@ extern "C" {
 /* routed-weight boundary (src/model_spec.rs:70-75) */
 #define FFMOE_WEIGHT_AFTER_DOWN_BF16          0  /* c = bf16(bf16(d) * w) */
 #define FFMOE_WEIGHT_BEFORE_CONTRIBUTION_BF16 1  /* c = bf16(d * w) */
+#define FFMOE_WEIGHT_BEFORE_DOWN_F32          2  /* the f32 weight multiplies the SwiGLU product before its BF16 cast, i.e. before
+                                                  the down projection (E8M0 contract, kernels/moe_ffn.cu:411-414) */
 
 /* router score */
 #define FFMOE_SCORE_SOFTMAX      0
@@ -205,6 +211,25 @@ int ffmoe_decode_contribute_stage(const ffmoe_expert_table* table, const ffmoe_s
 #define FFMOE_FORM_LANE8  1
 int ffmoe_decode_contribute_form(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared, const ffmoe_decode* args,
                                  int form, void* stream);
+
+/* Experts of the E8M0 block-32 contract (DeepSeek-V4.1 formats) in exact arithmetic. Routed experts are W4A8
+ * (FFMOE_FMT_E2M1_E8M0), the shared expert W8A8 with 32x32 block scales (FFMOE_FMT_E4M3_E8M0_32); every activation row
+ * is quantized to E4M3 with one E8M0 scale per 32 elements (amax floored at 1e-4, scale 2^ceil(log2(amax / 448))); a
+ * 32-element group dot is an exact integer, the groups are accumulated in ascending order by an FP64 fma and the total
+ * takes one BF16 rounding with the double-rounding tie repaired; gate is clamped from above and up on both sides by
+ * swiglu_limit, the FP32 SiLU * up * routed weight takes one BF16 cast and that row is quantized again for the down
+ * projection. Replaces moe_act_quant_e4m0, moe_ffn_dispatch_{gate_up,down}_e2m1_e8m0_exact and
+ * moe_ffn_{gate_up,down}_e4m3_block32_exact (kernels/moe_ffn.cu:463-467,601-700; kernels/q38_contract.cuh:53-101,
+ * 153-170; host: MoeExpertW4A8 / w8a8, src/backend/cuda/moe/w4a8.rs:248-420), for rows x top_k choices in one call.
+ * args: act_mode = FFMOE_ACT_E4M3_E8M0_32, routed_weight = FFMOE_WEIGHT_BEFORE_DOWN_F32, weights_f32 = 1,
+ * swiglu_limit > 0; swiglu is ignored (the contract fixes it). contributions[row, choice, :] already carry the routed
+ * weight. A choice that is inactive, out of range, not valid or stale writes nothing and keeps done = 0 (the reference
+ * traps). scratch: ffmoe_e8m0_scratch_bytes. */
+uint64_t ffmoe_e8m0_scratch_bytes(int rows, int top_k, int hidden, int inter, int shared_inter);
+int ffmoe_decode_contribute_e8m0(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared, const ffmoe_decode* args,
+                                 void* stream);
+/* x [rows, k] BF16 -> codes [rows, k] E4M3, scales [rows, k / 32] E8M0 (moe_act_quant_e4m0, kernels/moe_ffn.cu:444-467). */
+int ffmoe_act_quant_e8m0(const void* x, void* codes, void* scales, int rows, int k, void* stream);
 
 /* One token, selection inside the gate/up launch: logits [experts] FP32 (from ffmoe_route_logits_f32) go in, and the
  * top-k selection of ffmoe_route_topk_noaux (same arithmetic, bit for bit) runs in the prologue of every block of the

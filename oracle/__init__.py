@@ -288,6 +288,43 @@ def expert_down_w8a8(act, down, sdown, routing=1.0, boundary=AFTER_DOWN_BF16, or
     return f32_to_bf16(v.astype(np.float32))
 
 
+def act_quant_e8m0(x_bf16):
+    """rows of BF16 bits [rows, k] -> (E4M3 codes [rows, k], E8M0 scale codes [rows, k / 32])."""
+    x = _c(x_bf16, np.uint16)
+    rows, k = x.shape
+    codes = np.empty((rows, k), dtype=np.uint8)
+    scales = np.empty((rows, k // 32), dtype=np.uint8)
+    if lib().orc_act_quant_e8m0(_p(x), rows, k, _p(codes), _p(scales)) != 0:
+        raise ValueError("activation scale exponent out of range")
+    return codes, scales
+
+
+def scaled_dot_exact(packed, w, sw, x_codes, x_scales):
+    """One exact dot of the E8M0 contract -> (FP64 total, BF16 bits)."""
+    w, sw, xc, xs = _c(w, np.uint8), _c(sw, np.uint8), _c(x_codes, np.uint8), _c(x_scales, np.uint8)
+    total = ctypes.c_double()
+    rounded = ctypes.c_uint16()
+    if lib().orc_scaled_dot_exact(int(packed), _p(w), _p(sw), _p(xc), _p(xs), xc.size, ctypes.byref(total), ctypes.byref(rounded)) != 0:
+        raise ValueError("NaN code or 0xff scale")
+    return total.value, rounded.value
+
+
+def expert_ffn_e8m0(packed, x, gate, sgate, up, sup, down, sdown, limit, route_weight=1.0, return_act=False):
+    """One expert on one token in the exact E8M0 contract; see orc_expert_ffn_e8m0."""
+    x = _c(x, np.uint16)
+    H = x.size
+    down = _c(down, np.uint8)
+    I = down.shape[1] * (2 if packed else 1)
+    out = np.empty(H, dtype=np.uint16)
+    act = np.empty(I, dtype=np.uint16)
+    rc = lib().orc_expert_ffn_e8m0(int(packed), _p(x), _p(_c(gate, np.uint8)), _p(_c(sgate, np.uint8)), _p(_c(up, np.uint8)),
+                                   _p(_c(sup, np.uint8)), _p(down), _p(_c(sdown, np.uint8)), H, I, ctypes.c_float(limit),
+                                   ctypes.c_float(route_weight), _p(out), _p(act))
+    if rc != 0:
+        raise ValueError("orc_expert_ffn_e8m0 failed (%d)" % rc)
+    return (out, act) if return_act else out
+
+
 def linear_skinny(weight_bf16, x_bf16, kind=0):
     w = _c(weight_bf16, np.uint16)
     x = _c(x_bf16, np.uint16)

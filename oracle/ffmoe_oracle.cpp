@@ -779,3 +779,127 @@ ORC_API void orc_fixture_fill(uint64_t salt, uint64_t a0, int n0, int n1, int n2
 ORC_API void orc_pattern_fill(uint64_t seed0, double phase, long n, uint16_t* out) {
   for (long i = 0; i < n; ++i) out[i] = bf16_rne(float(std::sin(double(seed0 + uint64_t(i)) * 0.6180339887498949 + phase) * 0.75));
 }
+
+// =============================================================================================
+// E8M0 block-32 experts of the DeepSeek-V4.1 contract: W4A8 routed experts (E2M1 weights, one E8M0 scale per 32
+// elements of a row) and the W8A8 shared expert (E4M3 weights, one E8M0 scale per 32x32 block), activations quantized
+// to E4M3 with one E8M0 scale per 32 elements, dots as exact integers (kernels/q38_contract.cuh:53-101,140-170;
+// kernels/moe_ffn.cu:601-700).
+namespace {
+// q38_contract.cuh:132-137
+inline int act_quant_log2_ceil(float v) {
+  uint32_t bits;
+  std::memcpy(&bits, &v, 4);
+  const int exponent = int((bits >> 23) & 0xffu) - 127;
+  return exponent + ((bits & 0x7fffffu) != 0u ? 1 : 0);
+}
+// q38_contract.cuh:53-90: per 32 elements the integer sum of av * bv (E4M3 activation as an integer multiple of 2^-9,
+// E2M1 weight as a multiple of 2^-1 or E4M3 weight as a multiple of 2^-9), then total = fma(sum, 2^(sa + sb - bias),
+// total) in FP64, groups in ascending order. Returns false on a NaN code or a 0xff scale (the reference traps).
+bool scaled_dot_exact(bool packed, const uint8_t* w, const uint8_t* sw, const uint8_t* x, const uint8_t* sx, int k, double* out) {
+  static const uint32_t e2m1_int[8] = {0, 1, 2, 3, 4, 6, 8, 12};
+  double total = 0.0;
+  for (int group = 0; group < k / 32; ++group) {
+    long long sum = 0;
+    for (int lane = 0; lane < 32; ++lane) {
+      const int inner = group * 32 + lane;
+      const uint8_t a = x[inner];
+      if ((a & 127) == 127) return false;
+      const uint32_t ae = (a >> 3) & 15;
+      const uint32_t av = ae ? (8u + (a & 7u)) << (ae - 1) : (a & 7u);
+      uint32_t bv, sign;
+      if (packed) {
+        const uint8_t b = (w[inner / 2] >> (4 * (inner & 1))) & 15;
+        bv = e2m1_int[b & 7];
+        sign = (a >> 7) ^ (b >> 3);
+      } else {
+        const uint8_t b = w[inner];
+        if ((b & 127) == 127) return false;
+        const uint32_t be = (b >> 3) & 15;
+        bv = be ? (8u + (b & 7u)) << (be - 1) : (b & 7u);
+        sign = uint32_t(a ^ b) >> 7;
+      }
+      const long long prod = (long long)(uint64_t(av) * bv);
+      sum += sign ? -prod : prod;
+    }
+    const uint8_t sa = sx[group], sb = sw[group];
+    if (sa == 255 || sb == 255) return false;
+    const int exponent = int(sa) + int(sb) - (packed ? 264 : 272);
+    total = std::fma(double(sum), std::ldexp(1.0, exponent), total);
+  }
+  *out = total;
+  return true;
+}
+// q38_contract.cuh:92-98: FP64 -> BF16 through FP32 with the double-rounding tie repaired
+inline uint16_t bf16_round_f64(double value) {
+  float rounded = float(value);
+  uint32_t bits;
+  std::memcpy(&bits, &rounded, 4);
+  if ((bits & 65535u) == 32768u && double(rounded) != value)
+    rounded = std::nextafterf(rounded, value < double(rounded) ? -INFINITY : INFINITY);
+  return bf16_rne(rounded);
+}
+}  // namespace
+
+// q38_contract.cuh:153-170 (act_quant32) over rows of k BF16 values, k a multiple of 32: amax floored at 1e-4, scale
+// 2^ceil(log2(amax / 448)) as an E8M0 code, codes = E4M3 RNE of value / scale clamped to +-448. Returns 0, or -1 when
+// an exponent leaves [-127, 127] (the reference traps).
+ORC_API int orc_act_quant_e8m0(const uint16_t* x, int rows, int k, uint8_t* codes, uint8_t* scales) {
+  for (int r = 0; r < rows; ++r)
+    for (int g = 0; g < k / 32; ++g) {
+      const uint16_t* src = x + size_t(r) * k + size_t(g) * 32;
+      float amax = 0.0f;
+      for (int i = 0; i < 32; ++i) amax = std::fmax(amax, std::fabs(bf16_f32(src[i])));
+      amax = std::fmax(amax, 1e-4f);
+      const int exponent = act_quant_log2_ceil(amax * (1.0f / 448.0f));
+      if (exponent < -127 || exponent > 127) return -1;
+      const float scale = std::ldexp(1.0f, exponent);
+      for (int i = 0; i < 32; ++i)
+        codes[size_t(r) * k + size_t(g) * 32 + i] = encode_e4m3(std::fmin(448.0f, std::fmax(-448.0f, bf16_f32(src[i]) / scale)));
+      scales[size_t(r) * (k / 32) + g] = uint8_t(exponent + 127);
+    }
+  return 0;
+}
+
+// One exact dot, exposed for the tests: packed = 1 E2M1 weights (two per byte, low nibble first), 0 E4M3 weights.
+ORC_API int orc_scaled_dot_exact(int packed, const uint8_t* w, const uint8_t* sw, const uint8_t* x, const uint8_t* sx, int k,
+                                 double* total, uint16_t* rounded) {
+  double t;
+  if (!scaled_dot_exact(packed != 0, w, sw, x, sx, k, &t)) return -1;
+  *total = t;
+  *rounded = bf16_round_f64(t);
+  return 0;
+}
+
+// One expert on one token in the exact contract (kernels/moe_ffn.cu:601-657; host sequence
+// src/backend/cuda/moe/w4a8.rs:268-360): quantize x, gate/up exact dots -> BF16 each, gate clamped from above, up on
+// both sides, FP32 SiLU times up times the routed weight, one BF16 cast; quantize that row; down exact dots -> BF16.
+// packed = 1: E2M1 codes [N, K/2] with scales [N, K/32]; packed = 0: E4M3 codes [N, K] with scales [ceil(N/32), K/32].
+// act_out (optional) receives the BF16 down-input row [I].
+ORC_API int orc_expert_ffn_e8m0(int packed, const uint16_t* x, const uint8_t* gate, const uint8_t* sgate, const uint8_t* up,
+                                const uint8_t* sup, const uint8_t* down, const uint8_t* sdown, int H, int I, float limit,
+                                float route_weight, uint16_t* out, uint16_t* act_out) {
+  if (H % 32 || I % 32 || !(limit > 0.0f)) return -2;
+  std::vector<uint8_t> xc(H), xs(H / 32), hc(I), hs(I / 32);
+  std::vector<uint16_t> h(I);
+  if (orc_act_quant_e8m0(x, 1, H, xc.data(), xs.data())) return -1;
+  const int stride_gu = packed ? H / 2 : H, stride_d = packed ? I / 2 : I;
+  for (int j = 0; j < I; ++j) {
+    const int sr = packed ? j : j / 32;
+    double g64, u64;
+    if (!scaled_dot_exact(packed, gate + size_t(j) * stride_gu, sgate + size_t(sr) * (H / 32), xc.data(), xs.data(), H, &g64)) return -1;
+    if (!scaled_dot_exact(packed, up + size_t(j) * stride_gu, sup + size_t(sr) * (H / 32), xc.data(), xs.data(), H, &u64)) return -1;
+    const float g = std::fmin(bf16_f32(bf16_round_f64(g64)), limit);
+    const float u = std::fmax(std::fmin(bf16_f32(bf16_round_f64(u64)), limit), -limit);
+    h[j] = bf16_rne(((g / (1.0f + det_expf(-g))) * u) * route_weight);
+  }
+  if (act_out) std::memcpy(act_out, h.data(), size_t(I) * 2);
+  if (orc_act_quant_e8m0(h.data(), 1, I, hc.data(), hs.data())) return -1;
+  for (int d = 0; d < H; ++d) {
+    const int sr = packed ? d : d / 32;
+    double t;
+    if (!scaled_dot_exact(packed, down + size_t(d) * stride_d, sdown + size_t(sr) * (I / 32), hc.data(), hs.data(), I, &t)) return -1;
+    out[d] = bf16_round_f64(t);
+  }
+  return 0;
+}

@@ -1,0 +1,86 @@
+"""F4: experts of the E8M0 block-32 contract (W4A8 routed, W8A8 32x32-block shared expert) in exact arithmetic, through
+the C ABI, bit-equal to the oracle's restatement of kernels/q38_contract.cuh:53-101,153-170 and
+kernels/moe_ffn.cu:601-700 (pinned on the CPU against rational arithmetic and closed forms)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle as orc
+from flyingfish_amd import capi, synth
+from flyingfish_amd.ops import E8m0DecodeOps, ExpertTable
+from helpers import bits
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def rand_bf16(shape, std, seed):
+    return synth.normal(shape, std, seed).to(torch.bfloat16)
+
+
+def _tables(experts, hidden, inter, shared_inter, seed):
+    routed = ExpertTable.allocate(capi.FMT_E2M1_E8M0, experts, hidden, inter, DEV)
+    ref = []
+    for e in range(experts):
+        v = routed.expert_views(e)
+        mats = []
+        for i, shape in enumerate([(inter, hidden), (inter, hidden), (hidden, inter)]):
+            codes, scales = synth.quant_e2m1_e8m0(synth.normal(shape, 0.05, seed * 1000 + e * 3 + i))
+            v[2 * i].copy_(codes); v[2 * i + 1].copy_(scales)
+            mats += [codes.numpy(), scales.numpy()]
+        ref.append(mats)
+    sh_table = ExpertTable.allocate(capi.FMT_E4M3_E8M0_32, 1, hidden, shared_inter, DEV)
+    v = sh_table.expert_views(0)
+    sh_ref = []
+    for i, shape in enumerate([(shared_inter, hidden), (shared_inter, hidden), (hidden, shared_inter)]):
+        codes, scales = synth.quant_e4m3_e8m0_block32(synth.normal(shape, 0.05, seed * 1000 + 900 + i))
+        v[2 * i].copy_(codes); v[2 * i + 1].copy_(scales)
+        sh_ref += [codes.numpy(), scales.numpy()]
+    return routed, ref, sh_table, sh_ref
+
+
+def test_act_quant_e8m0_bit_exact():
+    x = (synth.normal((5, 256), 1.0, 3) * torch.exp(synth.normal((5, 1), 3.0, 4))).to(torch.bfloat16)
+    x[2, 32:64] = 0  # an all-zero group takes the amax floor
+    codes, scales = E8m0DecodeOps.act_quant(x.to(DEV))
+    torch.cuda.synchronize()
+    oc, os_ = orc.act_quant_e8m0(bits(x))
+    assert np.array_equal(codes.cpu().numpy(), oc) and np.array_equal(scales.cpu().numpy(), os_)
+
+
+@pytest.mark.parametrize("hidden,inter,shared_inter,rows,top_k", [(256, 128, 128, 1, 2), (512, 256, 384, 3, 3), (1024, 512, 512, 2, 4)])
+def test_e8m0_experts_bit_exact(hidden, inter, shared_inter, rows, top_k):
+    experts, limit = 6, 7.0
+    routed, ref, sh_table, sh_ref = _tables(experts, hidden, inter, shared_inter, 41 + rows)
+    sh = sh_table.shared_struct(0)
+    x = rand_bf16((rows, hidden), 1.0, 5 + rows)
+    g = synth.generator(6 + rows)
+    ids = torch.stack([torch.randperm(experts, generator=g)[:top_k] for _ in range(rows)]).to(torch.int32)
+    wt = torch.rand((rows, top_k), generator=g) * 0.5 + 0.05
+    active = torch.ones((rows, top_k), dtype=torch.int32)
+    if rows > 1:
+        active[1, 0] = 0
+    op = E8m0DecodeOps(routed, sh, rows, top_k, limit)
+    op.contributions.zero_()
+    contrib, shared_out = op.contribute(x.to(DEV), ids.to(DEV), wt.to(DEV), active.to(DEV))
+    torch.cuda.synchronize()
+    got, got_sh, xb = bits(contrib), bits(shared_out), bits(x)
+    for r in range(rows):
+        for c in range(top_k):
+            if not active[r, c]:
+                assert not got[r, c].any()
+                continue
+            want = orc.expert_ffn_e8m0(1, xb[r], *ref[int(ids[r, c])], limit, float(wt[r, c]))
+            assert np.array_equal(got[r, c], want), (r, c)
+        assert np.array_equal(got_sh[r], orc.expert_ffn_e8m0(0, xb[r], *sh_ref, limit, 1.0)), r
+    assert np.array_equal(op.done.cpu().numpy(), active.numpy())
+
+
+def test_e8m0_entry_checks_its_contract():
+    routed, _, sh_table, _ = _tables(2, 64, 32, 32, 9)
+    op = E8m0DecodeOps(routed, sh_table.shared_struct(0), 1, 1, 7.0)
+    op.limit = 0.0  # the contract clamps: a limit is required
+    x = rand_bf16((1, 64), 1.0, 1).to(DEV)
+    ids = torch.zeros((1, 1), dtype=torch.int32, device=DEV)
+    with pytest.raises(capi.FfmoeError):
+        op.contribute(x, ids, torch.ones((1, 1), device=DEV))

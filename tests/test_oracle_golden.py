@@ -634,3 +634,95 @@ def test_dot_form_order_witnesses():
     # with the 1 moved next to its partner in the tree (element 3) it survives: (2^24 + 0) + (-2^24 + 1)
     w = w_of({0: t, 2: -t, 3: 1.0}, 16)
     assert orc.dot(np.ones(16, dtype=np.float32), w, orc.LANE16) == 1.0
+
+
+# ------------------------------------------------------------------------------------------------
+# E8M0 block-32 contract (kernels/q38_contract.cuh:53-101, 140-170)
+def _e4m3_value(code):
+    from fractions import Fraction
+    sign = -1 if code & 0x80 else 1
+    e, m = (code >> 3) & 15, code & 7
+    mag = Fraction(m, 512) if e == 0 else Fraction(8 + m, 8) * Fraction(2) ** (e - 7)
+    return sign * mag
+
+
+def test_act_quant_e8m0_closed_forms():
+    """Scale = 2^ceil(log2(amax/448)) with amax floored at 1e-4; codes = E4M3 RNE of value / scale."""
+    # amax exactly 448 * 2^3: the quotient is a power of two, ceil keeps it; the extreme element becomes 448 (0x7e)
+    x = np.zeros((1, 32), dtype=np.float32)
+    x[0, 0], x[0, 1], x[0, 5] = 3584.0, -1792.0, 8.0
+    codes, scales = orc.act_quant_e8m0(orc.f32_to_bf16(x))
+    assert scales[0, 0] == 127 + 3
+    assert codes[0, 0] == 0x7e and codes[0, 1] == 0xf6 and codes[0, 5] == 0x38  # 448, -224, 1.0
+    # just above a power of two: the exponent moves up by one and the extreme element lands near 224
+    x[0, 0] = 3600.0
+    codes, scales = orc.act_quant_e8m0(orc.f32_to_bf16(x))
+    assert scales[0, 0] == 127 + 4 and codes[0, 0] == 0x76  # bf16(3600) = 3600 -> 225 -> RNE to 224
+    # an all-zero group takes the floor: amax = 1e-4 -> 2^ceil(log2(1e-4/448)) = 2^-22
+    codes, scales = orc.act_quant_e8m0(np.zeros((1, 32), dtype=np.uint16))
+    assert scales[0, 0] == 127 - 22 and not codes.any()
+    # every code decodes back to within half an E4M3 step of value / scale (brute force, seeded)
+    rng = np.random.default_rng(3)
+    xb = orc.f32_to_bf16((rng.standard_normal((4, 64)) * np.exp(rng.uniform(-6, 6, (4, 1)))).astype(np.float32))
+    codes, scales = orc.act_quant_e8m0(xb)
+    xv = orc.bf16_to_f32(xb).astype(np.float64)
+    for r in range(4):
+        for g in range(2):
+            s = 2.0 ** (int(scales[r, g]) - 127)
+            blk = xv[r, g * 32:(g + 1) * 32]
+            amax = max(np.abs(blk).max(), 1e-4)
+            assert s / 2 < amax / 448.0 * (1 + 1e-6) and amax / 448.0 <= s * (1 + 1e-6)
+            for i in range(32):
+                q = float(_e4m3_value(int(codes[r, g * 32 + i])))
+                assert abs(q - blk[i] / s) <= max(abs(blk[i] / s) * 2.0 ** -4, 2.0 ** -10)
+
+
+@pytest.mark.parametrize("packed", [1, 0])
+def test_scaled_dot_exact_against_rational_arithmetic(packed):
+    """The exact dot is an integer sum per 32 elements times a power of two, accumulated by FMA in FP64: with block
+    scales close together every partial sum is exact, so the total must equal the rational dot product of the decoded
+    operands, and its BF16 rounding the correctly rounded one."""
+    from fractions import Fraction
+    e2m1 = [Fraction(v) for v in (0, 0.5, 1, 1.5, 2, 3, 4, 6)]
+    rng = np.random.default_rng(11 + packed)
+    k = 128
+    xc = rng.integers(0, 256, k).astype(np.uint8)
+    xc[(xc & 127) == 127] = 0x31
+    xs = rng.integers(120, 132, k // 32).astype(np.uint8)
+    sw = rng.integers(118, 130, k // 32).astype(np.uint8)
+    if packed:
+        w = rng.integers(0, 256, k // 2).astype(np.uint8)
+        wv = [(-1 if (n >> 3) & 1 else 1) * e2m1[n & 7] for b in w for n in (b & 15, b >> 4)]
+    else:
+        w = rng.integers(0, 256, k).astype(np.uint8)
+        w[(w & 127) == 127] = 0x22
+        wv = [_e4m3_value(int(c)) for c in w]
+    exact = sum(_e4m3_value(int(xc[i])) * wv[i] * Fraction(2) ** (int(xs[i // 32]) - 127) * Fraction(2) ** (int(sw[i // 32]) - 127)
+                for i in range(k))
+    total, rounded = orc.scaled_dot_exact(packed, w, sw, xc, xs)
+    assert Fraction(total) == exact
+    # correctly rounded BF16 of the exact value: nearest, ties to even
+    f = float(exact)
+    lo = orc.f32_to_bf16(np.array([f], dtype=np.float32))[0]
+    cands = [int(lo) + d for d in (-1, 0, 1)]
+    best = min(cands, key=lambda b: (abs(Fraction(float(orc.bf16_to_f32(np.array([b], dtype=np.uint16))[0])) - exact), b & 1))
+    assert rounded == best
+
+
+def test_bf16_round_f64_repairs_the_double_rounding_tie():
+    """A value just above a BF16 tie that FP32 rounding would land exactly on the tie: the plain f64 -> f32 -> bf16 chain
+    rounds to even (down), the repaired one up. Built from one E4M3 x E4M3 product pair in two groups."""
+    # total = 2^0 * (1 + 2^-8) + 2^-40: f32 sees 1.00390625 exactly (the tie between bf16 1.0 and 1.0078125), bf16 RNE of
+    # that gives 1.0; the true value is above the tie, so the repaired rounding gives 0x3f81.
+    k = 64
+    xc = np.zeros(k, dtype=np.uint8); w = np.zeros(k, dtype=np.uint8)
+    xs = np.array([127, 127], dtype=np.uint8)
+    # group 0: x = 1.0 (0x38), weights: 1.0 (0x38) -> 1; plus x = 2^-8 (code for 2^-8: e=0 subnormal m=2 -> 2/512) * 1.0
+    xc[0], w[0] = 0x38, 0x38
+    xc[1], w[1] = 0x02, 0x38
+    # group 1: 1.0 * 1.0 with block scale 2^-40
+    xc[32], w[32] = 0x38, 0x38
+    sw = np.array([127, 127 - 40], dtype=np.uint8)
+    total, rounded = orc.scaled_dot_exact(0, w, sw, xc, xs)
+    assert total == 1.0 + 2.0 ** -8 + 2.0 ** -40
+    assert rounded == 0x3f81
