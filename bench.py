@@ -295,6 +295,23 @@ def widening_main(args, torch, capi, ops, synth):
             rows[name][fname + "_us"] = us_f
             rows[name][fname + "_gbps"] = nbytes / (us_f * 1e-6) / 1e9
         del dec, table
+    # E8M0 block-32 contract: W4A8 routed experts + W8A8 32x32-block shared expert, exact integer dots
+    table = ops.ExpertTable.allocate(capi.FMT_E2M1_E8M0, E, H, I, dev)
+    sh_table = ops.ExpertTable.allocate(capi.FMT_E4M3_E8M0_32, 1, H, I, dev)
+    for t, n in ((table, E), (sh_table, 1)):
+        for e in range(n):
+            v = t.expert_views(e)
+            for i in range(3):
+                v[2 * i].random_(0, 256)
+                if t is sh_table:
+                    v[2 * i].bitwise_and_(0x77)  # no E4M3 NaN codes
+                v[2 * i + 1].random_(118, 124)
+    e8 = ops.E8m0DecodeOps(table, sh_table.shared_struct(0), 1, K, 10.0)
+    nbytes = K * table.weight_bytes_per_expert() + sh_table.weight_bytes_per_expert()
+    us = timed(lambda i: e8.contribute(xs[i % 8], idl[i % 8], w), max(4, args.steps // 4))
+    rows["e8m0_w4a8_routed_w8a8_shared_exact"] = {"us": us, "weight_bytes": nbytes, "gbps": nbytes / (us * 1e-6) / 1e9,
+                                                  "hbm_frac": nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS}
+    del e8, table, sh_table
     # fused combine + shared gate + residual (one token and 64 tokens)
     for R in (1, 64):
         contrib = synth.normal((R, K, H), 0.05, 3, device=dev, dtype=torch.bfloat16)

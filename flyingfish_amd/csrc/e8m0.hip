@@ -69,7 +69,7 @@ extern "C" __attribute__((visibility("default"))) int ffmoe_decode_contribute_e8
   FF_REQUIRE(args->scratch_bytes >= l.total, FFMOE_ERR_SCRATCH, "scratch holds %llu bytes, %llu needed (ffmoe_e8m0_scratch_bytes)",
              (unsigned long long)args->scratch_bytes, (unsigned long long)l.total);
   const int imax = I > (shared ? SI : 0) ? I : SI;
-  FF_REQUIRE(size_t(H > imax ? H : imax) * 4 + 512 <= 64 * 1024, FFMOE_ERR_SHAPE, "a row of %d activations does not fit the LDS staging", H > imax ? H : imax);
+  FF_REQUIRE(size_t((H > imax ? H : imax) / 32) * 33 * 4 <= 64 * 1024, FFMOE_ERR_SHAPE, "a row of %d activations does not fit the LDS staging", H > imax ? H : imax);
   uint8_t* sc = (uint8_t*)args->scratch;
   E8m0Params q;
   DecodeParams& p = q.d;
@@ -89,7 +89,7 @@ extern "C" __attribute__((visibility("default"))) int ffmoe_decode_contribute_e8
   const int S = R * K + R;
   hipLaunchKernelGGL(k_act_quant_e8m0, dim3((H / 32 + 7) / 8, R), dim3(256), 0, st, p.x, H, sc + l.xq, H, sc + l.xs, H / 32, H, (const uint32_t*)nullptr);
   hipLaunchKernelGGL(k_e8m0_live, dim3((S + 255) / 256), dim3(256), 0, st, p, live);
-  hipLaunchKernelGGL((k_e8m0_stage<0>), dim3((imax + 255) / 256, R, K + 1), dim3(256), size_t(H) * 4 + H / 32, st, q);
+  hipLaunchKernelGGL((k_e8m0_stage<0>), dim3((imax + 7) / 8, R, K + 1), dim3(256), size_t(H / 32) * 33 * 4, st, q);
   FF_TRY(ff_launch_status());
   // every live down-input row is quantized over imax elements (a shorter row leaves its tail unused)
   if (K > 0)
@@ -98,6 +98,6 @@ extern "C" __attribute__((visibility("default"))) int ffmoe_decode_contribute_e8
   if (shared)
     hipLaunchKernelGGL(k_act_quant_e8m0, dim3((SI / 32 + 7) / 8, R), dim3(256), 0, st, p.h + size_t(R) * K * imax, imax,
                        sc + l.hq + size_t(R) * K * imax, imax, sc + l.hs + size_t(R) * K * (imax / 32), imax / 32, SI, (const uint32_t*)(live + R * K));
-  hipLaunchKernelGGL((k_e8m0_stage<1>), dim3((H + 255) / 256, R, K + 1), dim3(256), size_t(imax) * 4 + imax / 32, st, q);
+  hipLaunchKernelGGL((k_e8m0_stage<1>), dim3((H + 7) / 8, R, K + 1), dim3(256), size_t(imax / 32) * 33 * 4, st, q);
   return ff_launch_status();
 }

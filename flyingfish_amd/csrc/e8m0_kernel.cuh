@@ -10,10 +10,10 @@
 // tie repaired. Gate clamps from above, up on both sides, FP32 SiLU * up * routed weight, one BF16 cast; that row is
 // quantized again for the down projection.
 //
-// Mapping. The reference gives a 32-lane warp to an output row and a lane to an element of the group; here a LANE owns
-// an output ROW: all 64 lanes walk the groups in step, the 32 activations of the group are the same for every lane (LDS
-// broadcast reads of pre-decoded signed integers), the group sum and the FP64 chain live in the lane, and nothing is
-// reduced across lanes. The result is the same by construction: integer sums are order-free, the FP64 chain is per row.
+// Mapping. The reference gives a 32-lane warp to an output row and a lane to an element of the group; here eight lanes
+// share an output row, each owning a contiguous eighth of the groups: a lane computes whole group sums (exact integers,
+// order-free; for E2M1 weights as packed-byte dot products) and its own FP64 chain, and the eight totals are added at
+// the end (see k_e8m0_stage for why that is the reference's result).
 #pragma once
 #include "decode_kernel.cuh"
 
@@ -91,7 +91,58 @@ __global__ void k_e8m0_live(const DecodeParams p, uint32_t* __restrict__ live) {
   live[s] = gn > 0 ? 1u : 0u;
 }
 
-// grid (ceil(out / 256), rows, top_k + 1), block 256: thread = output row of (token row y, choice z | shared expert).
+// One group of a routed (E2M1) weight row against the pre-split activations of the group: the exact integer
+// sum of av * bv over 32 elements. act = 24 dwords: three planes of signed 7-bit pieces of av (av = p0 + (p1 << 7) +
+// (p2 << 14)), first the 16 even elements, then the 16 odd ones, four elements per dword, so that the low nibbles of
+// a weight dword (elements 8c, 8c+2, ...) and its high nibbles meet their activations as packed bytes in
+// v_dot4_i32_i8. Weight magnitudes come from a byte permute over the table {0,1,2,3,4,6,8,12}.
+__device__ __forceinline__ int e2m1_group_sum(const u32x4 w, const int* __restrict__ act) {
+  int acc0 = 0, acc1 = 0, acc2 = 0;
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    const uint32_t we = w[c], wo = w[c] >> 4;
+    uint32_t be, bo;
+    {
+      const uint32_t mag = __builtin_amdgcn_perm(0x0C080604u, 0x03020100u, we & 0x07070707u);
+      uint32_t sg = (we >> 3) & 0x01010101u;
+      sg &= ((mag + 0x7f7f7f7fu) >> 7) & 0x01010101u;  // a negative zero stays zero (no carry into the next byte)
+      be = (mag ^ ((sg << 8) - sg)) + sg;              // signed bytes
+    }
+    {
+      const uint32_t mag = __builtin_amdgcn_perm(0x0C080604u, 0x03020100u, wo & 0x07070707u);
+      uint32_t sg = (wo >> 3) & 0x01010101u;
+      sg &= ((mag + 0x7f7f7f7fu) >> 7) & 0x01010101u;
+      bo = (mag ^ ((sg << 8) - sg)) + sg;
+    }
+    acc0 = __builtin_amdgcn_sdot4(act[c], int(be), acc0, false);
+    acc0 = __builtin_amdgcn_sdot4(act[4 + c], int(bo), acc0, false);
+    acc1 = __builtin_amdgcn_sdot4(act[8 + c], int(be), acc1, false);
+    acc1 = __builtin_amdgcn_sdot4(act[12 + c], int(bo), acc1, false);
+    acc2 = __builtin_amdgcn_sdot4(act[16 + c], int(be), acc2, false);
+    acc2 = __builtin_amdgcn_sdot4(act[20 + c], int(bo), acc2, false);
+  }
+  return acc0 + (acc1 << 7) + (acc2 << 14);  // |sum| < 2^27
+}
+
+// The same sum element by element from the raw codes (any operand layout): the slow path of a row whose groups span
+// too many binades for an order-free FP64 sum, and the reference of the fast path in the tests.
+__device__ __forceinline__ long long e8m0_group_sum_plain(bool packed, const uint8_t* __restrict__ wrow, const uint8_t* __restrict__ xcodes, int g) {
+  long long sum = 0;
+  for (int i = 0; i < 32; ++i) {
+    const int inner = g * 32 + i;
+    const int av = e4m3_int(xcodes[inner]);
+    const int bv = packed ? e2m1_int((wrow[inner >> 1] >> (4 * (inner & 1))) & 15u) : e4m3_int(wrow[inner]);
+    sum += (long long)av * bv;
+  }
+  return sum;
+}
+
+// grid (ceil(out / 8), rows, top_k + 1), block 256 = RPB output rows x SEG segments of the contraction (32 x 8 for a
+// routed expert, whose blocks past ceil(out / 32) leave at once; 8 x 32 for the shared expert): lane (row, seg) sums the
+// groups [G * seg / SEG, G * (seg + 1) / SEG) of its row in ascending order, the partial totals are then added. That equals the reference's one chain over all groups whenever no addition rounds, which is certain when
+// sum |term| < 2^53 * (the smallest term's unit): every partial sum of the row, in any order, is then a multiple of
+// that unit below 2^53 of them, i.e. exactly representable. The lanes carry sum |term| and the smallest unit and check
+// it; a row that fails (block scales spanning ~26 binades or more) is recomputed by one lane in the reference's order.
 // STAGE 0: gate/up exact dots -> clamped SwiGLU * routed weight -> h (BF16). STAGE 1: down exact dots -> BF16.
 template <int STAGE>
 __global__ __launch_bounds__(256) void k_e8m0_stage(const E8m0Params q) {
@@ -109,19 +160,44 @@ __global__ __launch_bounds__(256) void k_e8m0_stage(const E8m0Params q) {
   const int Kg = STAGE == 0 ? p.hidden : (is_shared ? p.shared_inter : p.inter);
   const int out = STAGE == 0 ? (is_shared ? p.shared_inter : p.inter) : p.hidden;
   const int G = Kg >> 5;
-  if (int(blockIdx.x) * 256 >= out) return;
-  // activations of the row: signed integers (multiples of 2^-9) and scale codes, read by every lane alike
-  int* avs = reinterpret_cast<int*>(lds);
-  uint8_t* sxs = lds + size_t(Kg) * 4;
-  {
-    const uint8_t* codes = STAGE == 0 ? q.xq + size_t(r) * p.hidden : q.hq + size_t(gslot[0]) * p.h_stride;
-    const uint8_t* scales = STAGE == 0 ? q.xs + size_t(r) * (p.hidden >> 5) : q.hs + size_t(gslot[0]) * (p.h_stride >> 5);
-    for (int i = tid; i < Kg; i += 256) avs[i] = e4m3_int(codes[i]);
-    for (int i = tid; i < G; i += 256) sxs[i] = scales[i];
+  // lanes per output row: 8 for the packed-byte dot products of the routed experts, 32 for the shared expert, whose
+  // E4M3 x E4M3 products need 64-bit arithmetic per element (four times the work per group)
+  const int SEG = packed ? 8 : 32;
+  const int RPB = 256 / SEG;  // output rows per block
+  if (int(blockIdx.x) * RPB >= out) return;
+  const uint8_t* xcodes = STAGE == 0 ? q.xq + size_t(r) * p.hidden : q.hq + size_t(gslot[0]) * p.h_stride;
+  const uint8_t* xscales = STAGE == 0 ? q.xs + size_t(r) * (p.hidden >> 5) : q.hs + size_t(gslot[0]) * (p.h_stride >> 5);
+  // activations of the token, per group: packed path 24 dwords of signed 7-bit pieces (see e2m1_group_sum), plain path
+  // 32 signed integers; one more dword holds the group's scale code. The odd stride spreads the segments over banks.
+  const int gstride = packed ? 25 : 33;
+  int* act = reinterpret_cast<int*>(lds);
+  if (packed) {
+    for (int v = tid; v < G * 8; v += 256) {  // one dword of each plane per thread: four elements
+      const int g = v >> 3, c = v & 7;        // c < 4: even elements 8c, 8c+2, ..; c >= 4: odd elements
+      uint32_t w0 = 0, w1 = 0, w2 = 0;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int e = (c & 3) * 8 + 2 * i + (c >> 2);
+        const int av = e4m3_int(xcodes[g * 32 + e]);
+        const int mag = av < 0 ? -av : av;
+        const int sg = av < 0 ? -1 : 1;
+        w0 |= uint32_t((sg * (mag & 127)) & 0xff) << (8 * i);
+        w1 |= uint32_t((sg * ((mag >> 7) & 127)) & 0xff) << (8 * i);
+        w2 |= uint32_t((sg * (mag >> 14)) & 0xff) << (8 * i);
+      }
+      int* dst = act + size_t(g) * gstride;
+      dst[c] = int(w0); dst[8 + c] = int(w1); dst[16 + c] = int(w2);
+      if (c == 0) dst[24] = xscales[g];
+    }
+  } else {
+    for (int v = tid; v < Kg; v += 256) act[size_t(v >> 5) * gstride + (v & 31)] = e4m3_int(xcodes[v]);
+    for (int g = tid; g < G; g += 256) act[size_t(g) * gstride + 32] = xscales[g];
   }
   __syncthreads();
-  const int j = blockIdx.x * 256 + tid;
-  if (j >= out) return;
+  const int j = blockIdx.x * RPB + tid / SEG;
+  const int seg = tid % SEG;
+  const bool row_ok = j < out;
+  const int jr = row_ok ? j : out - 1;  // lanes past the end repeat the last row and store nothing
   uint64_t sl[6];
 #pragma unroll
   for (int i = 0; i < 6; ++i) sl[i] = is_shared ? p.shared_slot[i] : p.slots[size_t(expert) * 6 + i];
@@ -131,44 +207,76 @@ __global__ __launch_bounds__(256) void k_e8m0_stage(const E8m0Params q) {
 #pragma unroll
   for (int m = 0; m < NMAT; ++m) {
     const int base = STAGE == 0 ? 2 * m : 4;
-    wrow[m] = reinterpret_cast<const uint8_t*>(sl[base]) + size_t(j) * (packed ? Kg >> 1 : Kg);
-    srow[m] = reinterpret_cast<const uint8_t*>(sl[base + 1]) + size_t(packed ? j : j >> 5) * G;
+    wrow[m] = reinterpret_cast<const uint8_t*>(sl[base]) + size_t(jr) * (packed ? Kg >> 1 : Kg);
+    srow[m] = reinterpret_cast<const uint8_t*>(sl[base + 1]) + size_t(packed ? jr : jr >> 5) * G;
   }
   const int bias = packed ? 264 : 272;
-  double total[NMAT];
+  const int g_lo = G * seg / SEG, g_hi = G * (seg + 1) / SEG;
+  double total[NMAT], mass[NMAT];
+  int emin[NMAT];
 #pragma unroll
-  for (int m = 0; m < NMAT; ++m) total[m] = 0.0;
-  for (int g = 0; g < G; ++g) {
-    const int sa = sxs[g];
-    const int4* a4 = reinterpret_cast<const int4*>(avs + size_t(g) * 32);
+  for (int m = 0; m < NMAT; ++m) { total[m] = 0.0; mass[m] = 0.0; emin[m] = 4096; }
+  auto add_group = [&](int m, int g, long long sum, int sa) {
+    const int e = sa + int(srow[m][g]) - bias;
+    const double scale = pow2_f64(e);
+    total[m] = fma(double(sum), scale, total[m]);
+    mass[m] += fabs(double(sum) * scale);
+    if (sum != 0) emin[m] = e < emin[m] ? e : emin[m];
+  };
+  if (packed) {
+    for (int g0 = g_lo; g0 < g_hi; g0 += 4) {  // four groups of weights requested together
+      u32x4 w[NMAT][4];
 #pragma unroll
-    for (int m = 0; m < NMAT; ++m) {
-      long long sum = 0;
-      if (packed) {
-        const u32x4 w = load16(wrow[m] + size_t(g) * 16);
-        int isum = 0;  // |av * bv| < 2^22, 32 terms: fits 32 bits
+      for (int b = 0; b < 4; ++b) {
+        const int g = g0 + b < g_hi ? g0 + b : g_hi - 1;
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
-          const int4 lo = a4[2 * c], hi = a4[2 * c + 1];
-          const int av[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        for (int m = 0; m < NMAT; ++m) w[m][b] = load16(wrow[m] + size_t(g) * 16);
+      }
 #pragma unroll
-          for (int n = 0; n < 8; ++n) isum += av[n] * e2m1_int((w[c] >> (4 * n)) & 15u);
-        }
-        sum = isum;
-      } else {
-        const u32x4 w0 = load16(wrow[m] + size_t(g) * 32), w1 = load16(wrow[m] + size_t(g) * 32 + 16);
+      for (int b = 0; b < 4; ++b) {
+        const int g = g0 + b;
+        if (g < g_hi) {
+          const int* ag = act + size_t(g) * gstride;
 #pragma unroll
-        for (int c = 0; c < 8; ++c) {
-          const int4 a = a4[c];
-          const uint32_t w = c < 4 ? w0[c] : w1[c - 4];
-          sum += (long long)a.x * e4m3_int(w & 0xffu) + (long long)a.y * e4m3_int((w >> 8) & 0xffu) +
-                 (long long)a.z * e4m3_int((w >> 16) & 0xffu) + (long long)a.w * e4m3_int(w >> 24);
+          for (int m = 0; m < NMAT; ++m) add_group(m, g, e2m1_group_sum(w[m][b], ag), ag[24]);
         }
       }
-      const int sb = srow[m][g];
-      total[m] = fma(double(sum), pow2_f64(sa + sb - bias), total[m]);
+    }
+  } else {
+    for (int g = g_lo; g < g_hi; ++g) {
+      const int* ag = act + size_t(g) * gstride;
+#pragma unroll
+      for (int m = 0; m < NMAT; ++m) {
+        const u32x4 w0 = load16(wrow[m] + size_t(g) * 32), w1 = load16(wrow[m] + size_t(g) * 32 + 16);
+        long long sum = 0;
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+          const uint32_t w = c < 4 ? w0[c] : w1[c - 4];
+          sum += (long long)ag[4 * c] * e4m3_int(w & 0xffu) + (long long)ag[4 * c + 1] * e4m3_int((w >> 8) & 0xffu) +
+                 (long long)ag[4 * c + 2] * e4m3_int((w >> 16) & 0xffu) + (long long)ag[4 * c + 3] * e4m3_int(w >> 24);
+        }
+        add_group(m, g, sum, ag[32]);
+      }
     }
   }
+  // the eight segments of a row
+#pragma unroll
+  for (int m = 0; m < NMAT; ++m) {
+    for (int off = 1; off < SEG; off <<= 1) {
+      total[m] += __shfl_xor(total[m], off, SEG);
+      mass[m] += __shfl_xor(mass[m], off, SEG);
+      const int o = __shfl_xor(emin[m], off, SEG);
+      emin[m] = o < emin[m] ? o : emin[m];
+    }
+    const bool exact = emin[m] == 4096 || mass[m] < pow2_f64(53 + emin[m]);
+    if (!exact && seg == 0) {  // the reference's order, one group after the other
+      double t = 0.0;
+      for (int g = 0; g < G; ++g)
+        t = fma(double(e8m0_group_sum_plain(packed, wrow[m], xcodes, g)), pow2_f64(int(xscales[g]) + int(srow[m][g]) - bias), t);
+      total[m] = t;
+    }
+  }
+  if (!row_ok || seg != 0) return;
   if (STAGE == 0) {
     const float g = fminf(bf16_to_f32(bf16_round_f64(total[0])), p.swiglu_limit);
     const float u = fmaxf(fminf(bf16_to_f32(bf16_round_f64(total[NMAT - 1])), p.swiglu_limit), -p.swiglu_limit);

@@ -84,3 +84,32 @@ def test_e8m0_entry_checks_its_contract():
     ids = torch.zeros((1, 1), dtype=torch.int32, device=DEV)
     with pytest.raises(capi.FfmoeError):
         op.contribute(x, ids, torch.ones((1, 1), device=DEV))
+
+
+def test_e8m0_rows_whose_scales_span_many_binades_take_the_ordered_path():
+    """Block scales spread over ~100 binades: partial sums round, so only the reference's group order gives its bits."""
+    experts, hidden, inter, rows, top_k, limit = 3, 256, 128, 2, 2, 7.0
+    routed, ref, sh_table, sh_ref = _tables(experts, hidden, inter, inter, 77)
+    g = synth.generator(78)
+    for e in range(experts):
+        v = routed.expert_views(e)
+        for i in (1, 3, 5):
+            wild = torch.randint(70, 175, v[i].shape, generator=g, dtype=torch.uint8)
+            v[i].copy_(wild)
+            ref[e][i] = wild.numpy()
+    v = sh_table.expert_views(0)
+    for i in (1, 3, 5):
+        wild = torch.randint(90, 150, v[i].shape, generator=g, dtype=torch.uint8)
+        v[i].copy_(wild)
+        sh_ref[i] = wild.numpy()
+    x = rand_bf16((rows, hidden), 1.0, 79)
+    ids = torch.tensor([[0, 2], [1, 0]], dtype=torch.int32)
+    wt = torch.tensor([[0.3, 0.2], [0.4, 0.1]])
+    op = E8m0DecodeOps(routed, sh_table.shared_struct(0), rows, top_k, limit)
+    contrib, shared_out = op.contribute(x.to(DEV), ids.to(DEV), wt.to(DEV))
+    torch.cuda.synchronize()
+    got, got_sh, xb = bits(contrib), bits(shared_out), bits(x)
+    for r in range(rows):
+        for c in range(top_k):
+            assert np.array_equal(got[r, c], orc.expert_ffn_e8m0(1, xb[r], *ref[int(ids[r, c])], limit, float(wt[r, c]))), (r, c)
+        assert np.array_equal(got_sh[r], orc.expert_ffn_e8m0(0, xb[r], *sh_ref, limit, 1.0)), r
