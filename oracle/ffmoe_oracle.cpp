@@ -14,6 +14,9 @@
 //   * expert FFN on BF16 / per-channel FP8 weights .......... pinned (FP64 boundary oracle at 0 BF16 steps)
 //   * W8A8 quantizer + block dot ............................ pinned (FP64 gamma bound, wrong-cell mutant)
 //   * NVFP4 / BF16-scale skinny linear orders ............... pinned (closed-form dequant table, FP64 bound)
+//   * Lane16 / Lane8 summation orders ....................... pinned (hand-computed cancellation witnesses)
+//   * E8M0 block-32 contract: activation quantizer, exact
+//     integer dot, repaired BF16 rounding ................... pinned (closed forms, rational arithmetic, tie witness)
 //   * combine variants ...................................... pinned (order-spread constants of the fixture)
 //   * expert FFN composed over 128x128-f32 block scales or
 //     NVFP4 weights, grouped routing with n_group > 1,
