@@ -8,7 +8,7 @@ A step = one layer call (router logits -> top-k -> expert contributions -> combi
 already resident in HBM. Successive steps use different seeded tokens from a ring, so the selected experts
 change every step and their weights come from HBM, not from the 256 MB Infinity Cache.
 
-Prints ONE JSON line (see README / DESIGN.md for the fields).
+Prints ONE JSON line.
 """
 import argparse
 import json
@@ -338,7 +338,7 @@ def main():
     if args.batch is None:
         args.batch = 1 if args.workload == "decode" else 4096
     if args.gpus != 1:
-        print("bench.py measures one GPU: this build has no multi-GPU path (expert-parallel sharding is described in DESIGN.md); "
+        print("bench.py measures one GPU: this build has no multi-GPU path; "
               "run with --gpus 1", file=sys.stderr)
         sys.exit(2)
     import torch
