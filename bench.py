@@ -311,7 +311,11 @@ def widening_main(args, torch, capi, ops, synth):
     us = timed(lambda i: e8.contribute(xs[i % 8], idl[i % 8], w), max(4, args.steps // 4))
     rows["e8m0_w4a8_routed_w8a8_shared_exact"] = {"us": us, "weight_bytes": nbytes, "gbps": nbytes / (us * 1e-6) / 1e9,
                                                   "hbm_frac": nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS}
-    del e8, table, sh_table
+    e8f = ops.E8m0DecodeOps(table, sh_table.shared_struct(0), 1, K, 10.0, exact=False)
+    us = timed(lambda i: e8f.contribute(xs[i % 8], idl[i % 8], w), max(4, args.steps // 4))
+    rows["e8m0_w4a8_routed_w8a8_shared_fp32_chain"] = {"us": us, "weight_bytes": nbytes, "gbps": nbytes / (us * 1e-6) / 1e9,
+                                                       "hbm_frac": nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS}
+    del e8, e8f, table, sh_table
     # fused combine + shared gate + residual (one token and 64 tokens)
     for R in (1, 64):
         contrib = synth.normal((R, K, H), 0.05, 3, device=dev, dtype=torch.bfloat16)

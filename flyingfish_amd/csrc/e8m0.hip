@@ -51,8 +51,9 @@ extern "C" __attribute__((visibility("default"))) int ffmoe_decode_contribute_e8
   const int SI = shared ? shared->inter : I;
   FF_REQUIRE(H >= 32 && I >= 32 && SI >= 32 && H % 32 == 0 && I % 32 == 0 && SI % 32 == 0, FFMOE_ERR_SHAPE,
              "hidden=%d inter=%d shared inter=%d must be positive multiples of 32", H, I, SI);
-  FF_REQUIRE(args->act_mode == FFMOE_ACT_E4M3_E8M0_32, FFMOE_ERR_UNSUPPORTED, "act_mode %d: this path quantizes activations to E4M3 with E8M0 scales per 32",
-             args->act_mode);
+  FF_REQUIRE(args->act_mode == FFMOE_ACT_E4M3_E8M0_32 || args->act_mode == FFMOE_ACT_E4M3_E8M0_32_F32, FFMOE_ERR_UNSUPPORTED,
+             "act_mode %d: this path quantizes activations to E4M3 with E8M0 scales per 32", args->act_mode);
+  const bool exact = args->act_mode == FFMOE_ACT_E4M3_E8M0_32;
   FF_REQUIRE(args->swiglu_limit > 0.0f && args->swiglu_limit < INFINITY, FFMOE_ERR_SHAPE, "the contract clamps the SwiGLU inputs: limit %g",
              (double)args->swiglu_limit);
   FF_REQUIRE(args->routed_weight == FFMOE_WEIGHT_BEFORE_DOWN_F32 && args->weights_f32 == 1, FFMOE_ERR_UNSUPPORTED,
@@ -89,7 +90,8 @@ extern "C" __attribute__((visibility("default"))) int ffmoe_decode_contribute_e8
   const int S = R * K + R;
   hipLaunchKernelGGL(k_act_quant_e8m0, dim3((H / 32 + 7) / 8, R), dim3(256), 0, st, p.x, H, sc + l.xq, H, sc + l.xs, H / 32, H, (const uint32_t*)nullptr);
   hipLaunchKernelGGL(k_e8m0_live, dim3((S + 255) / 256), dim3(256), 0, st, p, live);
-  hipLaunchKernelGGL((k_e8m0_stage<0>), dim3((imax + 7) / 8, R, K + 1), dim3(256), size_t(H / 32) * 33 * 4, st, q);
+  if (exact) hipLaunchKernelGGL((k_e8m0_stage<0>), dim3((imax + 7) / 8, R, K + 1), dim3(256), size_t(H / 32) * 33 * 4, st, q);
+  else hipLaunchKernelGGL((k_e8m0_stage_f32<0>), dim3((imax + 7) / 8, R, K + 1), dim3(256), size_t(H) * 4 + size_t(H / 32) * 4, st, q);
   FF_TRY(ff_launch_status());
   // every live down-input row is quantized over imax elements (a shorter row leaves its tail unused)
   if (K > 0)
@@ -98,6 +100,7 @@ extern "C" __attribute__((visibility("default"))) int ffmoe_decode_contribute_e8
   if (shared)
     hipLaunchKernelGGL(k_act_quant_e8m0, dim3((SI / 32 + 7) / 8, R), dim3(256), 0, st, p.h + size_t(R) * K * imax, imax,
                        sc + l.hq + size_t(R) * K * imax, imax, sc + l.hs + size_t(R) * K * (imax / 32), imax / 32, SI, (const uint32_t*)(live + R * K));
-  hipLaunchKernelGGL((k_e8m0_stage<1>), dim3((H + 7) / 8, R, K + 1), dim3(256), size_t(imax / 32) * 33 * 4, st, q);
+  if (exact) hipLaunchKernelGGL((k_e8m0_stage<1>), dim3((H + 7) / 8, R, K + 1), dim3(256), size_t(imax / 32) * 33 * 4, st, q);
+  else hipLaunchKernelGGL((k_e8m0_stage_f32<1>), dim3((H + 7) / 8, R, K + 1), dim3(256), size_t(imax) * 4 + size_t(imax / 32) * 4, st, q);
   return ff_launch_status();
 }

@@ -293,4 +293,119 @@ __global__ __launch_bounds__(256) void k_e8m0_stage(const E8m0Params q) {
   }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// The FP32-chain variant (kernels/moe_ffn.cu:469-576 W4A8, :764-865 W8A8 shared expert): the reference gives a 32-lane
+// warp to an output row; here a half wave plays the warp, lane for lane, so chunk ownership, the fma chains and the
+// xor-butterfly sum are the reference's and the result is bit-equal to it (up to its expf).
+
+// E2M1 nibble -> FP32 (kernels/moe_ffn.cu:425-431)
+__device__ __forceinline__ float e2m1_f32(uint32_t nibble) {
+  const uint32_t u = nibble & 7u;
+  uint32_t bits = 0x3F000000u + u * 0x400000u;
+  bits = u == 0u ? 0u : (u == 1u ? 0x3F000000u : bits);
+  return __uint_as_float(bits | ((nibble & 8u) << 28));
+}
+__device__ __forceinline__ float half_wave_sum(float v) {
+#pragma unroll
+  for (int off = 16; off > 0; off >>= 1) v = __fadd_rn(v, __shfl_xor(v, off, 32));
+  return v;
+}
+
+// grid (ceil(out / 8), rows, top_k + 1), block 256 = 8 output rows x 32 lanes (the reference's launch shape).
+template <int STAGE>
+__global__ __launch_bounds__(256) void k_e8m0_stage_f32(const E8m0Params q) {
+  const DecodeParams& p = q.d;
+  extern __shared__ __align__(16) uint8_t lds[];
+  const int tid = threadIdx.x;
+  const int r = blockIdx.y, z = blockIdx.z;
+  const bool is_shared = z == p.top_k;
+  if (is_shared && !p.has_shared) return;
+  const int A = p.rows * p.top_k;
+  int expert, gn, grow[1], gslot[1];
+  load_group<1>(p, is_shared ? A + r : r * p.top_k + z, expert, gn, grow, gslot);
+  if (gn == 0) return;
+  const bool packed = !is_shared;
+  const int Kg = STAGE == 0 ? p.hidden : (is_shared ? p.shared_inter : p.inter);
+  const int out = STAGE == 0 ? (is_shared ? p.shared_inter : p.inter) : p.hidden;
+  const int G = Kg >> 5;
+  if (int(blockIdx.x) * 8 >= out) return;
+  // decoded activations and scales of the token
+  float* xf = reinterpret_cast<float*>(lds);
+  float* sxf = xf + Kg;
+  {
+    const uint8_t* codes = STAGE == 0 ? q.xq + size_t(r) * p.hidden : q.hq + size_t(gslot[0]) * p.h_stride;
+    const uint8_t* scales = STAGE == 0 ? q.xs + size_t(r) * (p.hidden >> 5) : q.hs + size_t(gslot[0]) * (p.h_stride >> 5);
+    for (int i = tid; i < Kg; i += 256) xf[i] = e4m3_to_f32(codes[i]);
+    for (int i = tid; i < G; i += 256) sxf[i] = __uint_as_float(uint32_t(scales[i]) << 23);  // 2^(code - 127); code 0 is the denormal 2^-127
+  }
+  __syncthreads();
+  const int j = blockIdx.x * 8 + (tid >> 5);
+  const int lane = tid & 31;
+  const bool row_ok = j < out;
+  const int jr = row_ok ? j : out - 1;
+  uint64_t sl[6];
+#pragma unroll
+  for (int i = 0; i < 6; ++i) sl[i] = is_shared ? p.shared_slot[i] : p.slots[size_t(expert) * 6 + i];
+  constexpr int NMAT = STAGE == 0 ? 2 : 1;
+  float acc[NMAT];
+#pragma unroll
+  for (int m = 0; m < NMAT; ++m) {
+    const int base = STAGE == 0 ? 2 * m : 4;
+    const uint8_t* wrow = reinterpret_cast<const uint8_t*>(sl[base]) + size_t(jr) * (packed ? Kg >> 1 : Kg);
+    const uint8_t* srow = reinterpret_cast<const uint8_t*>(sl[base + 1]) + size_t(packed ? jr : jr >> 5) * G;
+    float a = 0.0f;
+    if (packed) {
+      // lane L takes the 8-element chunks L, L + 32, ... (kernels/moe_ffn.cu:472-505)
+      const int chunks = Kg >> 3;
+      for (int chunk = lane; chunk < chunks; chunk += 32) {
+        const uint32_t word = load_global<uint32_t>(wrow + size_t(chunk) * 4);
+        const f32x4 x0 = *reinterpret_cast<const f32x4*>(xf + size_t(chunk) * 8), x1 = *reinterpret_cast<const f32x4*>(xf + size_t(chunk) * 8 + 4);
+        const float xv[8] = {x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+        float sum = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const uint32_t byte = (word >> (8 * i)) & 0xffu;
+          sum = __fmaf_rn(e2m1_f32(byte & 0xfu), xv[2 * i], sum);
+          sum = __fmaf_rn(e2m1_f32(byte >> 4), xv[2 * i + 1], sum);
+        }
+        const int group = chunk >> 2;
+        const float sw = __uint_as_float(uint32_t(srow[group]) << 23);
+        a = __fmaf_rn(sum, __fmul_rn(sxf[group], sw), a);
+      }
+    } else {
+      // eight K blocks per pass, a block split over four lanes of eight elements (kernels/moe_ffn.cu:768-797)
+      const int sub = lane & 3, stride = lane >> 2;
+      for (int base_g = 0; base_g < G; base_g += 8) {
+        const int block = base_g + stride;
+        float sum = 0.0f;
+        if (block < G) {
+          const u32x2 w = load_global<u32x2>(wrow + size_t(block) * 32 + sub * 8);
+          const float* xa = xf + size_t(block) * 32 + sub * 8;
+#pragma unroll
+          for (int i = 0; i < 8; ++i) sum = __fmaf_rn(e4m3_to_f32(uint8_t((w[i >> 2] >> (8 * (i & 3))) & 0xffu)), xa[i], sum);
+        }
+        sum = __fadd_rn(sum, __shfl_xor(sum, 1, 4));
+        sum = __fadd_rn(sum, __shfl_xor(sum, 2, 4));
+        if (sub == 0 && block < G) a = __fmaf_rn(sum, __fmul_rn(sxf[block], __uint_as_float(uint32_t(srow[block]) << 23)), a);
+      }
+    }
+    acc[m] = half_wave_sum(a);
+  }
+  if (!row_ok || lane != 0) return;
+  if (STAGE == 0) {
+    const float g = fminf(bround(acc[0]), p.swiglu_limit);
+    const float u = fmaxf(fminf(bround(acc[NMAT - 1]), p.swiglu_limit), -p.swiglu_limit);
+    const float silu = __fdiv_rn(g, __fadd_rn(1.0f, det_expf(-g)));
+    const float prod = __fmul_rn(silu, u);
+    p.h[size_t(gslot[0]) * p.h_stride + j] = f32_to_bf16(is_shared ? prod : __fmul_rn(prod, reinterpret_cast<const float*>(p.weights)[gslot[0]]));
+  } else {
+    const uint16_t o = f32_to_bf16(acc[0]);
+    if (is_shared) p.shared_out[size_t(r) * p.hidden + j] = o;
+    else {
+      p.contributions[size_t(gslot[0]) * p.hidden + j] = o;
+      if (j == 0 && p.done) p.done[gslot[0]] = 1u;
+    }
+  }
+}
+
 }  // namespace ffmoe

@@ -336,8 +336,9 @@ class E8m0DecodeOps:
     integer dots). Host mirror of MoeExpertW4A8 / the W8A8 shared expert ops (src/backend/cuda/moe/w4a8.rs:248-420),
     for rows x top_k choices per call; owns its scratch arena and output buffers."""
 
-    def __init__(self, table, shared=None, rows=1, top_k=8, swiglu_limit=10.0):
+    def __init__(self, table, shared=None, rows=1, top_k=8, swiglu_limit=10.0, exact=True):
         self.table, self.shared, self.rows, self.top_k, self.limit = table, shared, rows, top_k, swiglu_limit
+        self.act_mode = capi.ACT_E4M3_E8M0_32 if exact else capi.ACT_E4M3_E8M0_32_F32
         dev = table.slots.device
         si = shared.inter if shared is not None else 0
         nbytes = capi.lib().ffmoe_e8m0_scratch_bytes(rows, top_k, table.hidden, table.inter, si)
@@ -349,7 +350,7 @@ class E8m0DecodeOps:
         self._shared_c = shared
 
     def contribute(self, x, ids, weights, active=None):
-        d = capi.Decode(self.rows, self.top_k, capi.ACT_E4M3_E8M0_32, capi.SWIGLU_CLAMPED_ONCE, self.limit, capi.WEIGHT_BEFORE_DOWN_F32, 1,
+        d = capi.Decode(self.rows, self.top_k, self.act_mode, capi.SWIGLU_CLAMPED_ONCE, self.limit, capi.WEIGHT_BEFORE_DOWN_F32, 1,
                         x.data_ptr(), ids.data_ptr(), active.data_ptr() if active is not None else None, weights.data_ptr(),
                         self.contributions.data_ptr(), self.shared_out.data_ptr() if self.shared_out is not None else None,
                         self.done.data_ptr(), self.scratch.data_ptr(), self.scratch.numel(), None)

@@ -53,6 +53,8 @@ extern "C" {
                                      one scale product (kernels/fp8_linear.cu:12-48, kernels/q38_contract.cuh:239-279) */
 #define FFMOE_ACT_E4M3_E8M0_32  2  /* activations quantized per 32 to E4M3 with a power-of-two (E8M0) scale, exact integer dots
                                      (ffmoe_decode_contribute_e8m0 only) */
+#define FFMOE_ACT_E4M3_E8M0_32_F32 3  /* the same quantizer with the FP32 fma chains and 32-lane order of the reference's
+                                        moe_ffn_dispatch_*_e2m1_e8m0 / moe_ffn_*_e4m3_block32 (kernels/moe_ffn.cu:469-576,764-865) */
 
 /* SwiGLU rounding (src/model_spec.rs:61-69; src/cpu/expert_ffn.rs:58-100) */
 #define FFMOE_SWIGLU_TWICE          0  /* a = bf16(bf16(silu(g)) * u) */
@@ -221,7 +223,10 @@ int ffmoe_decode_contribute_form(const ffmoe_expert_table* table, const ffmoe_sh
  * projection. Replaces moe_act_quant_e4m0, moe_ffn_dispatch_{gate_up,down}_e2m1_e8m0_exact and
  * moe_ffn_{gate_up,down}_e4m3_block32_exact (kernels/moe_ffn.cu:463-467,601-700; kernels/q38_contract.cuh:53-101,
  * 153-170; host: MoeExpertW4A8 / w8a8, src/backend/cuda/moe/w4a8.rs:248-420), for rows x top_k choices in one call.
- * args: act_mode = FFMOE_ACT_E4M3_E8M0_32, routed_weight = FFMOE_WEIGHT_BEFORE_DOWN_F32, weights_f32 = 1,
+ * act_mode = FFMOE_ACT_E4M3_E8M0_32_F32 selects the reference's FP32-chain kernels instead (per 8-element chunk an fma
+ * chain, chunk sums scaled in FP32, 32-lane xor-butterfly sum; moe_ffn_dispatch_{gate_up,down}_e2m1_e8m0 and
+ * moe_ffn_{gate_up,down}_e4m3_block32), reproduced lane for lane.
+ * args: act_mode as above, routed_weight = FFMOE_WEIGHT_BEFORE_DOWN_F32, weights_f32 = 1,
  * swiglu_limit > 0; swiglu is ignored (the contract fixes it). contributions[row, choice, :] already carry the routed
  * weight. A choice that is inactive, out of range, not valid or stale writes nothing and keeps done = 0 (the reference
  * traps). scratch: ffmoe_e8m0_scratch_bytes. */

@@ -325,6 +325,28 @@ def expert_ffn_e8m0(packed, x, gate, sgate, up, sup, down, sdown, limit, route_w
     return (out, act) if return_act else out
 
 
+def e8m0_dot_f32(packed, w, sw, x_codes, x_scales):
+    """One dot of the FP32-chain variant of the E8M0 contract (32-lane order of the reference's kernels)."""
+    w, sw, xc, xs = _c(w, np.uint8), _c(sw, np.uint8), _c(x_codes, np.uint8), _c(x_scales, np.uint8)
+    lib().orc_e8m0_dot_f32.restype = ctypes.c_float
+    return float(lib().orc_e8m0_dot_f32(int(packed), _p(w), _p(sw), _p(xc), _p(xs), xc.size))
+
+
+def expert_ffn_e8m0_f32(packed, x, gate, sgate, up, sup, down, sdown, limit, route_weight=1.0):
+    """One expert on one token, FP32-chain variant; see orc_expert_ffn_e8m0_f32."""
+    x = _c(x, np.uint16)
+    H = x.size
+    down = _c(down, np.uint8)
+    I = down.shape[1] * (2 if packed else 1)
+    out = np.empty(H, dtype=np.uint16)
+    rc = lib().orc_expert_ffn_e8m0_f32(int(packed), _p(x), _p(_c(gate, np.uint8)), _p(_c(sgate, np.uint8)), _p(_c(up, np.uint8)),
+                                       _p(_c(sup, np.uint8)), _p(down), _p(_c(sdown, np.uint8)), H, I, ctypes.c_float(limit),
+                                       ctypes.c_float(route_weight), _p(out), None)
+    if rc != 0:
+        raise ValueError("orc_expert_ffn_e8m0_f32 failed (%d)" % rc)
+    return out
+
+
 def linear_skinny(weight_bf16, x_bf16, kind=0):
     w = _c(weight_bf16, np.uint16)
     x = _c(x_bf16, np.uint16)

@@ -906,3 +906,112 @@ ORC_API int orc_expert_ffn_e8m0(int packed, const uint16_t* x, const uint8_t* ga
   }
   return 0;
 }
+
+// ---------------------------------------------------------------------------------------------
+// The FP32-chain variant of the same formats (kernels/moe_ffn.cu:469-576 W4A8, :764-865 W8A8 shared expert): one
+// 32-lane warp per output row, FP32 fma chains, the block scales multiply chunk sums in FP32, xor-butterfly warp sum.
+namespace {
+// q38_contract.cuh:36-42
+inline float e8m0_decode_f32(uint8_t code) {
+  if (code == 0xffu) return NAN;
+  return std::ldexp(1.0f, int(code) - 127);
+}
+// kernels/moe_ffn.cu:425-431
+inline float e2m1_f32(unsigned nibble) {
+  const unsigned u = nibble & 7u;
+  uint32_t bits = 0x3F000000u + u * 0x400000u;
+  if (u == 0u) bits = 0u;
+  else if (u == 1u) bits = 0x3F000000u;
+  bits |= (nibble & 8u) << 28;
+  float f;
+  std::memcpy(&f, &bits, 4);
+  return f;
+}
+// kernels/moe_ffn.cu:437-442: every lane receives the total
+inline float warp_sum_xor32(float* v) {
+  for (int off = 16; off > 0; off >>= 1) {
+    float n[32];
+    for (int l = 0; l < 32; ++l) n[l] = v[l] + v[l ^ off];
+    std::memcpy(v, n, sizeof(n));
+  }
+  return v[0];
+}
+// kernels/moe_ffn.cu:472-505: lane L takes the 8-element chunks L, L+32, ...
+float w4a8_dot_f32(const uint8_t* w, const uint8_t* sw, const uint8_t* x, const uint8_t* sx, int k) {
+  float lanes[32];
+  const int chunks = k / 8;
+  for (int lane = 0; lane < 32; ++lane) {
+    float acc = 0.0f;
+    for (int chunk = lane; chunk < chunks; chunk += 32) {
+      float sum = 0.0f;
+      for (int i = 0; i < 4; ++i) {
+        const unsigned byte = w[size_t(chunk) * 4 + i];
+        sum = std::fmaf(e2m1_f32(byte & 0xfu), decode_e4m3(x[size_t(chunk) * 8 + 2 * i]), sum);
+        sum = std::fmaf(e2m1_f32(byte >> 4), decode_e4m3(x[size_t(chunk) * 8 + 2 * i + 1]), sum);
+      }
+      const int group = chunk / 4;
+      acc = std::fmaf(sum, e8m0_decode_f32(sx[group]) * e8m0_decode_f32(sw[group]), acc);
+    }
+    lanes[lane] = acc;
+  }
+  return warp_sum_xor32(lanes);
+}
+// kernels/moe_ffn.cu:768-797: lane = (block slot lane >> 2, quarter lane & 3); eight K blocks per pass
+float w8a8_dot_f32(const uint8_t* w, const uint8_t* sw, const uint8_t* x, const uint8_t* sx, int k) {
+  float lanes[32];
+  const int groups = k / 32;
+  for (int l = 0; l < 32; ++l) lanes[l] = 0.0f;
+  for (int base = 0; base < groups; base += 8) {
+    for (int stride = 0; stride < 8; ++stride) {
+      const int block = base + stride;
+      if (block >= groups) continue;
+      float part[4];
+      for (int sub = 0; sub < 4; ++sub) {
+        float sum = 0.0f;
+        for (int i = 0; i < 8; ++i) {
+          const size_t at = size_t(block) * 32 + sub * 8 + i;
+          sum = std::fmaf(decode_e4m3(w[at]), decode_e4m3(x[at]), sum);
+        }
+        part[sub] = sum;
+      }
+      // xor 1 then xor 2 inside the quad; quarter 0 keeps (p0 + p1) + (p2 + p3)
+      const float s = (part[0] + part[1]) + (part[2] + part[3]);
+      lanes[stride * 4] = std::fmaf(s, e8m0_decode_f32(sx[block]) * e8m0_decode_f32(sw[block]), lanes[stride * 4]);
+    }
+  }
+  return warp_sum_xor32(lanes);
+}
+}  // namespace
+
+// packed = 1: W4A8 dot of one row; 0: W8A8 dot of one row (sw = the scale row of its 32-row block).
+ORC_API float orc_e8m0_dot_f32(int packed, const uint8_t* w, const uint8_t* sw, const uint8_t* x, const uint8_t* sx, int k) {
+  return packed ? w4a8_dot_f32(w, sw, x, sx, k) : w8a8_dot_f32(w, sw, x, sx, k);
+}
+
+// One expert on one token, FP32-chain variant (kernels/moe_ffn.cu:507-576, :799-865); same layouts as
+// orc_expert_ffn_e8m0. The shared expert (packed = 0) carries no routed weight.
+ORC_API int orc_expert_ffn_e8m0_f32(int packed, const uint16_t* x, const uint8_t* gate, const uint8_t* sgate, const uint8_t* up,
+                                    const uint8_t* sup, const uint8_t* down, const uint8_t* sdown, int H, int I, float limit,
+                                    float route_weight, uint16_t* out, uint16_t* act_out) {
+  if (H % 32 || I % 32 || !(limit > 0.0f)) return -2;
+  std::vector<uint8_t> xc(H), xs(H / 32), hc(I), hs(I / 32);
+  std::vector<uint16_t> h(I);
+  if (orc_act_quant_e8m0(x, 1, H, xc.data(), xs.data())) return -1;
+  const int stride_gu = packed ? H / 2 : H, stride_d = packed ? I / 2 : I;
+  for (int j = 0; j < I; ++j) {
+    const int sr = packed ? j : j / 32;
+    const float gate_v = orc_e8m0_dot_f32(packed, gate + size_t(j) * stride_gu, sgate + size_t(sr) * (H / 32), xc.data(), xs.data(), H);
+    const float up_v = orc_e8m0_dot_f32(packed, up + size_t(j) * stride_gu, sup + size_t(sr) * (H / 32), xc.data(), xs.data(), H);
+    const float g = std::fmin(bround(gate_v), limit);
+    const float u = std::fmax(std::fmin(bround(up_v), limit), -limit);
+    const float silu = g / (1.0f + det_expf(-g));
+    h[j] = packed ? bf16_rne((silu * u) * route_weight) : bf16_rne(silu * u);
+  }
+  if (act_out) std::memcpy(act_out, h.data(), size_t(I) * 2);
+  if (orc_act_quant_e8m0(h.data(), 1, I, hc.data(), hs.data())) return -1;
+  for (int d = 0; d < H; ++d) {
+    const int sr = packed ? d : d / 32;
+    out[d] = bf16_rne(orc_e8m0_dot_f32(packed, down + size_t(d) * stride_d, sdown + size_t(sr) * (I / 32), hc.data(), hs.data(), I));
+  }
+  return 0;
+}

@@ -113,3 +113,24 @@ def test_e8m0_rows_whose_scales_span_many_binades_take_the_ordered_path():
         for c in range(top_k):
             assert np.array_equal(got[r, c], orc.expert_ffn_e8m0(1, xb[r], *ref[int(ids[r, c])], limit, float(wt[r, c]))), (r, c)
         assert np.array_equal(got_sh[r], orc.expert_ffn_e8m0(0, xb[r], *sh_ref, limit, 1.0)), r
+
+
+@pytest.mark.parametrize("hidden,inter,shared_inter,rows,top_k", [(256, 128, 128, 1, 2), (1024, 512, 384, 3, 3)])
+def test_e8m0_fp32_chain_variant_bit_exact(hidden, inter, shared_inter, rows, top_k):
+    """act_mode FFMOE_ACT_E4M3_E8M0_32_F32: the reference's 32-lane FP32 kernels, reproduced lane for lane."""
+    experts, limit = 5, 7.0
+    routed, ref, sh_table, sh_ref = _tables(experts, hidden, inter, shared_inter, 141 + rows)
+    x = rand_bf16((rows, hidden), 1.0, 15 + rows)
+    g = synth.generator(16 + rows)
+    ids = torch.stack([torch.randperm(experts, generator=g)[:top_k] for _ in range(rows)]).to(torch.int32)
+    wt = torch.rand((rows, top_k), generator=g) * 0.5 + 0.05
+    op = E8m0DecodeOps(routed, sh_table.shared_struct(0), rows, top_k, limit, exact=False)
+    contrib, shared_out = op.contribute(x.to(DEV), ids.to(DEV), wt.to(DEV))
+    torch.cuda.synchronize()
+    got, got_sh, xb = bits(contrib), bits(shared_out), bits(x)
+    for r in range(rows):
+        for c in range(top_k):
+            want = orc.expert_ffn_e8m0_f32(1, xb[r], *ref[int(ids[r, c])], limit, float(wt[r, c]))
+            assert np.array_equal(got[r, c], want), (r, c)
+        assert np.array_equal(got_sh[r], orc.expert_ffn_e8m0_f32(0, xb[r], *sh_ref, limit, 1.0)), r
+    assert np.all(op.done.cpu().numpy() == 1)

@@ -726,3 +726,46 @@ def test_bf16_round_f64_repairs_the_double_rounding_tie():
     total, rounded = orc.scaled_dot_exact(0, w, sw, xc, xs)
     assert total == 1.0 + 2.0 ** -8 + 2.0 ** -40
     assert rounded == 0x3f81
+
+
+@pytest.mark.parametrize("packed", [1, 0])
+def test_e8m0_fp32_chain_tracks_the_exact_dot(packed):
+    """The FP32-chain variant rounds every fma; against the exact dot it must stay within n * 2^-24 of sum |term|
+    (the reference tests its kernels against an FP64 oracle the same way), and a wrong scale group must break that."""
+    rng = np.random.default_rng(21 + packed)
+    k = 512
+    xc = rng.integers(0, 256, k).astype(np.uint8)
+    xc[(xc & 127) == 127] = 0x31
+    xs = rng.integers(122, 130, k // 32).astype(np.uint8)
+    sw = rng.integers(120, 128, k // 32).astype(np.uint8)
+    w = rng.integers(0, 256, k // 2 if packed else k).astype(np.uint8)
+    if not packed:
+        w[(w & 127) == 127] = 0x22
+    total, _ = orc.scaled_dot_exact(packed, w, sw, xc, xs)
+    got = orc.e8m0_dot_f32(packed, w, sw, xc, xs)
+    # sum of |term| from the decoded operands
+    e2m1 = [0, 0.5, 1, 1.5, 2, 3, 4, 6]
+    wv = [(-1 if (n >> 3) & 1 else 1) * e2m1[n & 7] for b in w for n in (b & 15, b >> 4)] if packed else [float(_e4m3_value(int(c))) for c in w]
+    mass = sum(abs(float(_e4m3_value(int(xc[i]))) * wv[i]) * 2.0 ** (int(xs[i // 32]) + int(sw[i // 32]) - 254) for i in range(k))
+    assert abs(got - total) <= k * 2.0 ** -24 * mass
+    sw2 = sw.copy(); sw2[3] += 4
+    assert abs(orc.e8m0_dot_f32(packed, w, sw2, xc, xs) - total) > k * 2.0 ** -24 * mass
+
+
+def test_e8m0_fp32_chain_order_witness():
+    """W4A8: lane L owns the 8-element chunks L, L+32, ...; inside a chunk the eight products are a chain from zero.
+    The witness checks lane ownership: chunk 0 and chunk 32 both belong to lane 0, carry +-2688 * 2^20 and cancel there;
+    spread over two lanes the warp sum would meet 2688 * 2^20 + 1 and lose the 1."""
+    k = 8 * 64
+    xc = np.full(k, 0x38, dtype=np.uint8)           # 1.0
+    w = np.zeros(k // 2, dtype=np.uint8)
+    xs = np.full(k // 32, 127, dtype=np.uint8)
+    sw = np.full(k // 32, 127, dtype=np.uint8)
+    xc[0] = 0x7e                                     # 448 in chunk 0
+    xc[32 * 8] = 0x7e                                # 448 in chunk 32 (same lane)
+    w[0] = 0x07                                      # +6 at element 0
+    w[32 * 4] = 0x0f                                 # -6 at element 256
+    sw[0] = 127 + 20; sw[8] = 127 + 20               # both chunks scaled by 2^20: +-2818572288
+    w[16] = 0x02                                     # +1 at element 32 (chunk 4, lane 4, group 1 with unit scale):
+                                                     # it survives only because lane 0 cancels to zero before the warp sum
+    assert orc.e8m0_dot_f32(1, w, sw, xc, xs) == 1.0
