@@ -157,10 +157,8 @@ __global__ __launch_bounds__(256) void k_decode_form(const DecodeParams p) {
   const int sub = tid % LPR;
   if (j >= out) return;
   uint64_t sl[6];
-  float gl3[3] = {1.0f, 1.0f, 1.0f};
 #pragma unroll
   for (int i = 0; i < 6; ++i) sl[i] = is_shared ? p.shared_slot[i] : p.slots[size_t(expert) * 6 + i];
-  (void)gl3;
   if (STAGE == 0) {
     const FormRow<F> gate(sl[0], sl[1], j, Kg), up(sl[2], sl[3], j, Kg);
     const float g = form_dot<F, FORM>(xs, gate, Kg, sub);
