@@ -86,6 +86,103 @@ def test_linear_and_combine_contract_violations():
     assert L.ffmoe_quant_fp8_f32_128(1 << 20, 1 << 20, 2 << 20, 1, 128, None) == capi.ERR_OVERLAP
 
 
+def _prefill_args(**kw):
+    d = dict(rows=64, top_k=4, act_mode=capi.ACT_FP8_BLOCK128, swiglu=0, swiglu_limit=0.0, routed_weight=0, weights_f32=1, x=1 << 20,
+             ids=2 << 20, active=None, weights=3 << 20, contributions=64 << 20, done=None, scratch=256 << 20, scratch_bytes=1 << 30,
+             shared=None, shared_out=None, assignment_gen=None)
+    d.update(kw)
+    return capi.Prefill(d["rows"], d["top_k"], d["act_mode"], d["swiglu"], d["swiglu_limit"], d["routed_weight"], d["weights_f32"],
+                        d["x"], d["ids"], d["active"], d["weights"], d["contributions"], d["done"], d["scratch"], d["scratch_bytes"],
+                        d["shared"], d["shared_out"], d["assignment_gen"])
+
+
+def test_prefill_contract_violations_are_reported_before_launch():
+    L = capi.lib()
+    table = capi.ExpertTable(capi.FMT_FP8_BLOCK128, 64, 2048, 1408 - 1408 % 128, 16 << 20, None, None)
+
+    def call(t=table, **kw):
+        a = _prefill_args(**kw)
+        return L.ffmoe_prefill_contribute(ctypes.byref(t), ctypes.byref(a), None)
+    assert L.ffmoe_prefill_contribute(None, None, None) == capi.ERR_NULL
+    assert call(act_mode=capi.ACT_BF16) == capi.ERR_UNSUPPORTED and "matrix cores" in capi.last_error()
+    nv = capi.ExpertTable(capi.FMT_NVFP4, 64, 2048, 1280, 16 << 20, None, 32 << 20)
+    assert call(t=nv) == capi.ERR_UNSUPPORTED
+    assert call(top_k=40) == capi.ERR_SHAPE
+    assert call(swiglu=2, swiglu_limit=0.0) == capi.ERR_SHAPE
+    assert call(routed_weight=capi.WEIGHT_BEFORE_DOWN_F32) == capi.ERR_UNSUPPORTED
+    assert call(scratch_bytes=4096) == capi.ERR_SCRATCH
+    assert call(scratch=(256 << 20) + 16) == capi.ERR_ALIGN
+    assert call(contributions=1 << 20) == capi.ERR_OVERLAP
+    odd = capi.ExpertTable(capi.FMT_FP8_BLOCK128, 64, 2048, 1408, 16 << 20, None, None)  # 1408 = 11 * 128 is fine, 1400 is not
+    assert call(t=odd, scratch_bytes=16) == capi.ERR_SCRATCH
+    bad = capi.ExpertTable(capi.FMT_FP8_BLOCK128, 64, 2048, 1400, 16 << 20, None, None)
+    assert call(t=bad) == capi.ERR_SHAPE
+    assert L.ffmoe_prefill_contribute_stage(ctypes.byref(table), ctypes.byref(_prefill_args()), 7, None) == capi.ERR_SHAPE
+    assert L.ffmoe_prefill_scratch_bytes(0, 8, 256, 7168, 2048, 0) == 0
+    need = L.ffmoe_prefill_scratch_bytes(4096, 8, 256, 7168, 2048, 0)
+    assert need >= 4096 * 8 * 2048 * 3 + 4096 * 7168  # BF16 + E4M3 activations of every assignment, quantized x
+
+
+def test_token_and_form_entry_contract_violations():
+    L = capi.lib()
+    fp8 = capi.ExpertTable(capi.FMT_FP8_BLOCK128, 256, 7168, 2048, 16 << 20, None, None)
+    f = ctypes.c_float
+    logits, y = 5 << 20, 6 << 20
+
+    def from_logits(t=fp8, score=capi.NOAUX_SIGMOID, scaling=2.5, n_group=8, topk_group=4, lg=logits, **kw):
+        a = _decode_args(**{**dict(top_k=8, weights_f32=1), **kw})
+        return L.ffmoe_decode_contribute_from_logits(ctypes.byref(t), None, ctypes.byref(a), lg, None, score, f(scaling), n_group, topk_group, None)
+    assert from_logits(rows=2) == capi.ERR_UNSUPPORTED and "one token row" in capi.last_error()
+    assert from_logits(act_mode=capi.ACT_FP8_BLOCK128) == capi.ERR_UNSUPPORTED
+    assert from_logits(weights_f32=0) == capi.ERR_UNSUPPORTED
+    assert from_logits(t=capi.ExpertTable(capi.FMT_FP8_BLOCK128, 96, 7168, 2048, 16 << 20, None, None)) == capi.ERR_UNSUPPORTED
+    assert from_logits(score=5) == capi.ERR_UNSUPPORTED
+    assert from_logits(scaling=-1.0) == capi.ERR_SHAPE
+    assert from_logits(n_group=8, topk_group=9) == capi.ERR_SHAPE
+    assert from_logits(lg=logits + 2) == capi.ERR_ALIGN
+
+    def token_layer(combine=capi.COMBINE_ROUTED, yy=y, **kw):
+        a = _decode_args(**{**dict(top_k=8, weights_f32=1), **kw})
+        return L.ffmoe_decode_token_layer(ctypes.byref(fp8), None, ctypes.byref(a), logits, None, capi.NOAUX_SIGMOID, f(2.5), 8, 4, None, yy, None,
+                                          combine, None)
+    assert token_layer(rows=4) == capi.ERR_UNSUPPORTED
+    assert token_layer(combine=17) == capi.ERR_UNSUPPORTED
+    assert token_layer(combine=capi.COMBINE_UNGATED) == capi.ERR_SHAPE and "shared expert" in capi.last_error()
+    assert token_layer(yy=y + 2) == capi.ERR_ALIGN
+
+    def form(t, form_id=capi.FORM_LANE16, **kw):
+        a = _decode_args(**kw)
+        return L.ffmoe_decode_contribute_form(ctypes.byref(t), None, ctypes.byref(a), form_id, None)
+    bf16 = capi.ExpertTable(capi.FMT_BF16, 64, 2048, 1408, 16 << 20, None, None)
+    assert form(fp8) == capi.ERR_UNSUPPORTED          # block-scaled experts have no Lane16 / Lane8 reference order
+    assert form(bf16, form_id=3) == capi.ERR_UNSUPPORTED
+    assert form(bf16, act_mode=capi.ACT_FP8_BLOCK128) == capi.ERR_UNSUPPORTED
+    assert form(bf16, x=None) == capi.ERR_NULL
+
+
+def test_e8m0_entry_contract_violations():
+    L = capi.lib()
+    t = capi.ExpertTable(capi.FMT_E2M1_E8M0, 16, 7168, 2048, 16 << 20, None, None)
+
+    def call(tt=t, **kw):
+        d = dict(top_k=8, act_mode=capi.ACT_E4M3_E8M0_32, swiglu=capi.SWIGLU_CLAMPED_ONCE, swiglu_limit=10.0,
+                 routed_weight=capi.WEIGHT_BEFORE_DOWN_F32, weights_f32=1, scratch_bytes=1 << 30)
+        d.update(kw)
+        a = _decode_args(**d)
+        return L.ffmoe_decode_contribute_e8m0(ctypes.byref(tt), None, ctypes.byref(a), None)
+    assert L.ffmoe_decode_contribute_e8m0(None, None, None, None) == capi.ERR_NULL
+    assert call(tt=capi.ExpertTable(capi.FMT_FP8_BLOCK128, 16, 7168, 2048, 16 << 20, None, None)) == capi.ERR_UNSUPPORTED
+    assert call(act_mode=capi.ACT_BF16) == capi.ERR_UNSUPPORTED
+    assert call(swiglu_limit=0.0) == capi.ERR_SHAPE
+    assert call(routed_weight=capi.WEIGHT_AFTER_DOWN_BF16) == capi.ERR_UNSUPPORTED
+    assert call(weights_f32=0) == capi.ERR_UNSUPPORTED
+    assert call(tt=capi.ExpertTable(capi.FMT_E2M1_E8M0, 16, 7168 + 16, 2048, 16 << 20, None, None)) == capi.ERR_SHAPE
+    assert call(scratch_bytes=64) == capi.ERR_SCRATCH and "ffmoe_e8m0_scratch_bytes" in capi.last_error()
+    assert L.ffmoe_act_quant_e8m0(None, 1 << 20, 2 << 20, 1, 64, None) == capi.ERR_NULL
+    assert L.ffmoe_act_quant_e8m0(1 << 20, 2 << 20, 3 << 20, 1, 48, None) == capi.ERR_SHAPE
+    assert L.ffmoe_e8m0_scratch_bytes(1, 8, 7168, 2048, 2048) > 0
+
+
 def test_slot_layout_matches_the_reference_catalogue():
     # src/experts/catalogue.rs:180-222: codes gate|up|down, then gate, up, down scales; BASELINE byte counts
     offs, size = ExpertTable.slot_layout(capi.FMT_FP8_BLOCK128, 7168, 2048)
