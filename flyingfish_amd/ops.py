@@ -318,10 +318,14 @@ class DecodeOps:
         """rows == 1: selection (when logits are given; ids / weights are then outputs), gate/up, down, routing weight and
         the ordered combine in ONE launch. Returns False (nothing launched) when the shape is outside the fast path."""
         act_mode, swiglu, limit, rw, wf32 = self.cfg
+        # an arena of its own: the launch recognises its activations by a 16-bit tag in the upper half of each word, and
+        # the untagged BF16 activations the other entry points leave in self.scratch could pass for a tagged word
+        if getattr(self, "token_scratch", None) is None:
+            self.token_scratch = torch.zeros_like(self.scratch)
         d = capi.Decode(self.rows, self.top_k, act_mode, swiglu, limit, rw, wf32,
                         x.data_ptr(), ids.data_ptr(), active.data_ptr() if active is not None else None, weights.data_ptr(),
                         self.contributions.data_ptr(), self.shared_out.data_ptr() if self.shared_out is not None else None,
-                        self.done.data_ptr(), self.scratch.data_ptr(), self.scratch.numel(), None)
+                        self.done.data_ptr(), self.token_scratch.data_ptr(), self.token_scratch.numel(), None)
         sh = ctypes.byref(self._shared_c) if self._shared_c is not None else None
         rc = capi.lib().ffmoe_decode_token_layer(ctypes.byref(self._table_c), sh, ctypes.byref(d), _ptr(logits), _ptr(bias), score_mode,
                                                  routed_scaling, n_group, topk_group, _ptr(scale), _ptr(y), _ptr(status), mode, _stream())
