@@ -248,6 +248,17 @@ def expert_ffn(x, gate, up, down, routing=1.0, rounding=TWICE, limit=0.0, bounda
     return (out, act) if return_act else out
 
 
+def expert_down(act, down, routing=1.0, boundary=AFTER_DOWN_BF16, form=LANE8, apply_weight=True):
+    """Second half of expert_ffn from a given BF16 activation [I]: down [H, I], routing weight at `boundary`."""
+    act = _c(act, np.uint16)
+    down = _c(down, np.uint16)
+    H, I = down.shape
+    assert act.shape == (I,)
+    out = np.empty(H, dtype=np.uint16)
+    lib().orc_expert_down(_p(act), _p(down), H, I, ctypes.c_float(routing), boundary, form, int(bool(apply_weight)), _p(out))
+    return out
+
+
 def linear_fp8_block_w8a8(w_codes, w_scales, x_codes, x_scales, order=0, want_f32=False):
     w = _c(w_codes, np.uint8)
     sw = _c(w_scales, np.float32)

@@ -552,6 +552,23 @@ ORC_API void orc_expert_ffn(const uint16_t* x, const uint16_t* gate, const uint1
   }
 }
 
+// The second half of orc_expert_ffn from a given BF16 activation [I] (src/cpu/expert_ffn.rs:470-497): lets a test
+// judge the down stage on the activations the device itself produced. Equal to orc_expert_ffn bit for bit when fed
+// its act_out (tests/test_oracle_golden.py).
+ORC_API void orc_expert_down(const uint16_t* act, const uint16_t* down, int H, int I, float routing, int boundary, int form,
+                             int apply_weight, uint16_t* out) {
+  std::vector<float> af(I);
+  for (int j = 0; j < I; ++j) af[j] = bf16_f32(act[j]);
+  for (int d = 0; d < H; ++d) {
+    const float lin = dot_form(af.data(), down + size_t(d) * I, I, form);
+    float v;
+    if (!apply_weight) v = bround(lin);
+    else if (boundary == AFTER_DOWN_BF16) v = bround(lin) * routing;
+    else v = lin * routing;
+    out[d] = bf16_rne(v);
+  }
+}
+
 // =============================================================================================
 // W8A8 block linear: kernels/q38_contract.cuh:239-279 (fp8_block_decode<float,128>): per output
 // and per 128-group, lane L of 32 chains fma over elements L, L+32, L+64, L+96, a shuffle-down

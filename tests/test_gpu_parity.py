@@ -244,6 +244,70 @@ def test_decode_bf16_experts(rows):
     _run_decode(capi.FMT_BF16, 5, 1024, 256, rows, 2, 71, True)
 
 
+@pytest.mark.parametrize("seed", range(32))
+def test_decode_seeded_shape_sweep(seed):
+    """Shapes the fixed cases do not visit: every format at odd multiples of its granule (row tails, partial slabs,
+    hidden < inter and the reverse), 1..17 rows, 1..8 choices, with and without a shared expert, an active mask, every
+    SwiGLU rounding and both routing-weight boundaries; the configuration is a function of the seed alone.
+
+    Each launch is held to the bar on its own inputs: the activations against the oracle's, the down stage against the
+    oracle's down stage on the activations the device produced. End to end the two stages compose: one flipped BF16
+    step of an activation can move a cancelled down output by more than two of its own steps at these small shapes, so
+    that comparison keeps the relative-L2 bar and allows four steps."""
+    rng = np.random.default_rng(1000 + seed)
+    fmt = [capi.FMT_FP8_BLOCK128, capi.FMT_NVFP4, capi.FMT_BF16, capi.FMT_FP8_CHANNEL][seed % 4]
+    gran = {capi.FMT_FP8_BLOCK128: 128, capi.FMT_NVFP4: 32, capi.FMT_BF16: 8, capi.FMT_FP8_CHANNEL: 16}[fmt]
+    hidden = gran * int(rng.integers(128 // gran, 1536 // gran + 1))
+    inter = gran * int(rng.integers(128 // gran, 1024 // gran + 1))
+    experts = int(rng.integers(2, 13))
+    top_k = int(rng.integers(1, min(8, experts) + 1))
+    rows = int(rng.choice([1, 1, 2, 3, 4, 7, 9, 17]))
+    mode = int(rng.integers(0, 4))
+    limit = float(rng.choice([0.03, 0.1, 1.0])) if mode >= 2 else 0.0
+    boundary = int(rng.integers(0, 2))
+    shared, weights_f32, with_active = bool(rng.integers(0, 2)), bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+    print("fmt=%d hidden=%d inter=%d experts=%d top_k=%d rows=%d mode=%d limit=%g boundary=%d shared=%d f32=%d mask=%d" %
+          (fmt, hidden, inter, experts, top_k, rows, mode, limit, boundary, shared, weights_f32, with_active), flush=True)
+    table, ref = make_table(fmt, experts + (1 if shared else 0), hidden, inter, 3000 + seed)
+    sh = table.shared_struct(experts) if shared else None
+    table.experts = experts
+    x = rand_bf16((rows, hidden), 1.0, 3007 + seed)
+    g = synth.generator(3008 + seed)
+    ids = torch.stack([torch.randperm(experts, generator=g)[:top_k] for _ in range(rows)]).to(torch.int32)
+    wt = torch.rand((rows, top_k), generator=g) * 0.5 + 0.05
+    wdev = wt.to(DEV) if weights_f32 else wt.to(torch.bfloat16).to(DEV)
+    wref = wt.numpy() if weights_f32 else wt.to(torch.bfloat16).float().numpy()
+    active = (torch.rand((rows, top_k), generator=g) > 0.3).to(torch.int32) if with_active else torch.ones((rows, top_k), dtype=torch.int32)
+    op = DecodeOps(table, sh, rows, top_k, capi.ACT_BF16, mode, limit, boundary, weights_f32)
+    op.contributions.zero_()
+    contrib, shared_out = op.contribute(x.to(DEV), ids.to(DEV), wdev, active.to(DEV) if with_active else None)
+    torch.cuda.synchronize()
+    got = bits(contrib)
+    A = rows * top_k
+    h = bits(op.scratch[: (A + rows) * inter * 2].view(torch.bfloat16).view(A + rows, inter))  # slot a, then A + row for the shared expert
+    done = op.done.cpu().numpy()
+    assert np.array_equal(done != 0, active.numpy() != 0)
+    xb = bits(x)
+    for r in range(rows):
+        for c in range(top_k):
+            if not active[r, c]:
+                assert not got[r, c].any()
+                continue
+            ge, ue, de = ref[int(ids[r, c])]
+            want, act = orc.expert_ffn(xb[r], ge, ue, de, float(wref[r, c]), mode, limit, boundary, orc.LANE8, orc.SILU_DIV, return_act=True)
+            assert_close_bf16(h[r * top_k + c][None, :], act[None, :], "activations row %d choice %d" % (r, c))
+            assert_close_bf16(got[r, c][None, :], orc.expert_down(h[r * top_k + c], de, float(wref[r, c]), boundary, orc.LANE8)[None, :],
+                              "down stage row %d choice %d" % (r, c))
+            assert_close_bf16(got[r, c][None, :], want[None, :], "contribution row %d choice %d" % (r, c), max_ulp=4)
+        if shared:
+            ge, ue, de = ref[experts]
+            want, act = orc.expert_ffn(xb[r], ge, ue, de, 1.0, mode, limit, 0, orc.LANE8, orc.SILU_DIV, apply_weight=False, return_act=True)
+            so = bits(shared_out)[r]
+            assert_close_bf16(h[A + r][None, :], act[None, :], "shared activations row %d" % r)
+            assert_close_bf16(so[None, :], orc.expert_down(h[A + r], de, 1.0, 0, orc.LANE8, False)[None, :], "shared down stage row %d" % r)
+            assert_close_bf16(so[None, :], want[None, :], "shared_out row %d" % r, max_ulp=4)
+
+
 @pytest.mark.parametrize("rows,routed_fmt,shared_fmt", [(1, capi.FMT_NVFP4, capi.FMT_BF16), (6, capi.FMT_NVFP4, capi.FMT_BF16),
                                                         (3, capi.FMT_FP8_BLOCK128, capi.FMT_BF16)])
 def test_decode_shared_expert_in_another_format(rows, routed_fmt, shared_fmt):

@@ -769,3 +769,20 @@ def test_e8m0_fp32_chain_order_witness():
     w[16] = 0x02                                     # +1 at element 32 (chunk 4, lane 4, group 1 with unit scale):
                                                      # it survives only because lane 0 cancels to zero before the warp sum
     assert orc.e8m0_dot_f32(1, w, sw, xc, xs) == 1.0
+
+
+def test_expert_down_is_the_second_half_of_expert_ffn():
+    """expert_down fed the activation expert_ffn reports gives expert_ffn's output bit for bit, in every form, at both
+    routing-weight boundaries and for the unweighted shared expert; a changed activation changes the result."""
+    rng = np.random.default_rng(5)
+    H, I = 96, 72
+    bf = lambda a: orc.f32_to_bf16(a.astype(np.float32))
+    x, g, u, d = bf(rng.normal(0, 1, H)), bf(rng.normal(0, 0.1, (I, H))), bf(rng.normal(0, 0.1, (I, H))), bf(rng.normal(0, 0.1, (H, I)))
+    for form in (orc.LANE16, orc.LANE8):
+        for boundary in (0, 1):
+            for apply_weight in (True, False):
+                out, act = orc.expert_ffn(x, g, u, d, 0.37, orc.TWICE, 0.0, boundary, form, orc.SILU_DIV, apply_weight=apply_weight, return_act=True)
+                assert np.array_equal(orc.expert_down(act, d, 0.37, boundary, form, apply_weight), out)
+    act2 = act.copy()
+    act2[3] ^= 0x0040
+    assert not np.array_equal(orc.expert_down(act2, d, 0.37, 1, orc.LANE8, False), out)
