@@ -153,6 +153,48 @@ def test_route_noaux_golden_and_random():
                     assert np.array_equal(bits(w), orc.f32_to_bf16(ow))
 
 
+@pytest.mark.parametrize("seed", range(24))
+def test_route_seeded_sweep_bit_exact(seed):
+    """Router shapes the fixed cases do not visit: expert counts that are not powers of two, top_k from 1 to 32, rows
+    1..40, grouped selection with every divisor pair, planted ties, both score functions, both weight types. Ids and
+    weights are compared bit for bit."""
+    rng = np.random.default_rng(2000 + seed)
+    experts = int(rng.choice([8, 33, 48, 64, 100, 160, 256, 384, 1000]))
+    top_k = int(rng.integers(1, min(32, experts - 1) + 1))
+    rows = int(rng.choice([1, 2, 5, 17, 40]))
+    lg = rng.normal(size=(rows, experts)).astype(np.float32) * float(rng.choice([0.5, 2.0, 6.0]))
+    for r in range(rows):  # planted exact ties: the lower id must win
+        a, b = rng.choice(experts, 2, replace=False)
+        lg[r, a] = lg[r, b]
+    b = rng.normal(scale=0.2, size=(experts,)).astype(np.float32)
+    # noaux with the group filter where the shape allows one
+    groupings = [(1, 1)]
+    for ng in (2, 4, 8):
+        if experts % ng == 0:
+            for kg in range(1, ng + 1):
+                if kg * (experts // ng) >= top_k:
+                    groupings.append((ng, kg))
+    ng, kg = groupings[int(rng.integers(0, len(groupings)))]
+    mode = int(rng.integers(0, 2))
+    scaling = float(rng.choice([1.0, 1.5, 2.5]))
+    print("experts=%d top_k=%d rows=%d groups=%d/%d mode=%d scaling=%g" % (experts, top_k, rows, ng, kg, mode, scaling), flush=True)
+    try:
+        ids, w = RouteOps.topk_noaux(torch.from_numpy(lg).to(DEV), torch.from_numpy(b).to(DEV), top_k, mode, scaling, ng, kg, True)
+    except capi.FfmoeError as e:
+        assert e.code == capi.ERR_UNSUPPORTED and ng > 1, e  # a group width the wave selection does not take
+        ng, kg = 1, 1
+        ids, w = RouteOps.topk_noaux(torch.from_numpy(lg).to(DEV), torch.from_numpy(b).to(DEV), top_k, mode, scaling, ng, kg, True)
+    oi, ow = orc.route_topk_noaux(lg, b[None, :], top_k, mode, scaling, ng, kg)
+    assert np.array_equal(ids.cpu().numpy(), oi)
+    assert np.array_equal(w.cpu().numpy().view(np.uint32), ow.view(np.uint32))
+    # softmax / sigmoid top-k on BF16 logits
+    lb = torch.from_numpy(lg).to(torch.bfloat16)
+    for score, fn in ((capi.SCORE_SOFTMAX, orc.route_topk_softmax), (capi.SCORE_SIGMOID, orc.route_topk_sigmoid)):
+        i2, w2 = RouteOps.topk(lb.to(DEV), top_k, score)
+        wi, ww = fn(bits(lb), top_k)
+        assert np.array_equal(i2.cpu().numpy(), wi) and np.array_equal(bits(w2), ww)
+
+
 @pytest.mark.parametrize("rows,experts,hidden,top_k,ng,kg", [(1, 256, 7168, 8, 8, 4), (5, 64, 1024, 6, 1, 1), (3, 100, 520, 4, 4, 2), (2, 1000, 256, 32, 1, 1)])
 def test_route_noaux_decode_equals_two_step_and_oracle(rows, experts, hidden, top_k, ng, kg):
     x, w = rand_bf16((rows, hidden), 1.0, 31), rand_bf16((experts, hidden), 0.02, 32)
@@ -507,6 +549,30 @@ def test_combine_modes_bit_exact():
     bad = act.clone(); bad[2, 1] ^= 1
     CombineOps.combine(c.to(DEV), sh.to(DEV), ids.to(DEV), capi.COMBINE_BF16, done=bad.to(DEV), final_active=act.to(DEV), status=status)
     assert int(status.item()) == 1
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_combine_seeded_sweep_bit_exact(seed):
+    """Combine shapes the fixed case does not visit (1..33 rows, 1..8 choices, hidden any multiple of 8 up to 2048,
+    rows with no active choice at all), every mode, bit for bit."""
+    rng = np.random.default_rng(4000 + seed)
+    rows, top_k = int(rng.choice([1, 2, 7, 33])), int(rng.integers(1, 9))
+    hidden = 8 * int(rng.integers(16, 257))
+    experts = int(rng.integers(top_k, 65)) + 1
+    c = rand_bf16((rows, top_k, hidden), 1.0, 4100 + seed)
+    sh = rand_bf16((rows, hidden), 1.0, 4200 + seed)
+    g = synth.generator(4300 + seed)
+    ids = torch.stack([torch.randperm(experts, generator=g)[:top_k] for _ in range(rows)]).to(torch.int32)
+    act = (torch.rand((rows, top_k), generator=g) > 0.3).to(torch.int32)
+    act[0] = 0  # a row whose choices are all inactive
+    scale = rand_bf16((rows,), 0.5, 4400 + seed).to(DEV)
+    status = torch.zeros(1, dtype=torch.int32, device=DEV)
+    print("rows=%d top_k=%d hidden=%d experts=%d" % (rows, top_k, hidden, experts), flush=True)
+    for mode in range(6):
+        y = CombineOps.combine(c.to(DEV), sh.to(DEV), ids.to(DEV), mode, scale=scale, done=act.to(DEV), final_active=act.to(DEV), status=status)
+        want = orc.combine(bits(c), bits(sh), bits(scale), ids.numpy(), act.numpy().astype(np.uint32), mode)
+        assert np.array_equal(bits(y), want), mode
+    assert int(status.item()) == 0
 
 
 def test_combine_residual_and_peer_join_bit_exact():
