@@ -144,6 +144,34 @@ def test_prefill_matches_per_assignment_oracle(rows, top_k, experts, hidden, int
     _check_prefill(op, host, bits(x), ids, w, orc.CLAMPED_TWICE, 10.0, orc.AFTER_DOWN_BF16, np.ones_like(ids, dtype=bool), got)
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_prefill_seeded_sweep(seed):
+    """Cohorts the fixed cases do not visit: 1..300 rows, 1..8 choices, 2..40 experts, hidden and inter any multiple of
+    128 from 256 to 640, uniform to heavily skewed routing (experts without rows, one expert with most of them), every
+    SwiGLU rounding and both routing-weight boundaries; the configuration is a function of the seed alone."""
+    rng = np.random.default_rng(6000 + seed)
+    experts = int(rng.choice([2, 5, 8, 17, 40]))
+    top_k = int(rng.integers(1, min(8, experts) + 1))
+    rows = int(rng.choice([1, 3, 16, 17, 65, 130, 300]))
+    # at least two 128-wide blocks per contraction: a single block sum leaves the matrix core with about 14 bits, which
+    # for a cancelled output is not always inside two BF16 steps of the row's scale
+    hidden, inter = 128 * int(rng.integers(2, 6)), 128 * int(rng.integers(2, 6))
+    skew = float(rng.choice([0.0, 1.1, 3.0]))
+    mode = int(rng.integers(0, 4))
+    limit = float(rng.choice([0.5, 10.0])) if mode >= 2 else 0.0
+    boundary = int(rng.integers(0, 2))
+    print("rows=%d top_k=%d experts=%d hidden=%d inter=%d skew=%g mode=%d limit=%g boundary=%d" %
+          (rows, top_k, experts, hidden, inter, skew, mode, limit, boundary), flush=True)
+    table, host = _make_fp8_table(experts, hidden, inter, 60 + seed)
+    ids, w = _routing(rows, top_k, experts, 6100 + seed, skew)
+    x = synth.normal((rows, hidden), 1.0, 6200 + seed, dtype=torch.bfloat16)
+    op = ops.PrefillOps(table, rows, top_k, swiglu=mode, swiglu_limit=limit, routed_weight=boundary, weights_f32=True)
+    got = op.contribute(x.cuda(), torch.from_numpy(ids).cuda(), torch.from_numpy(w).cuda())
+    torch.cuda.synchronize()
+    assert int(op.done.sum().item()) == rows * top_k
+    _check_prefill(op, host, bits(x), ids, w, mode, limit, boundary, np.ones_like(ids, dtype=bool), got)
+
+
 def test_prefill_skips_inactive_invalid_and_out_of_range():
     rows, top_k, experts, hidden, inter = 24, 4, 8, 256, 128
     table, host = _make_fp8_table(experts, hidden, inter, 6)
