@@ -76,6 +76,38 @@ def test_e8m0_experts_bit_exact(hidden, inter, shared_inter, rows, top_k):
     assert np.array_equal(op.done.cpu().numpy(), active.numpy())
 
 
+@pytest.mark.parametrize("seed", range(10))
+@pytest.mark.parametrize("exact", [True, False])
+def test_e8m0_experts_seeded_sweep(seed, exact):
+    """Bit equality at widths the fixed cases do not visit (any multiple of 32 from 64 to 1024, shared expert of another
+    width, 1..5 rows, 1..6 choices, activations scaled over several binades), in the exact arithmetic and in the
+    FP32-chain variant."""
+    rng = np.random.default_rng(8000 + seed)
+    hidden = 32 * int(rng.integers(2, 33))
+    inter = 32 * int(rng.integers(2, 17))
+    shared_inter = 32 * int(rng.integers(2, 17))
+    experts = int(rng.integers(2, 8))
+    top_k = int(rng.integers(1, min(6, experts) + 1))
+    rows = int(rng.choice([1, 2, 5]))
+    limit = float(rng.choice([0.5, 7.0]))
+    print("hidden=%d inter=%d shared_inter=%d experts=%d top_k=%d rows=%d limit=%g exact=%d" %
+          (hidden, inter, shared_inter, experts, top_k, rows, limit, exact), flush=True)
+    routed, ref, sh_table, sh_ref = _tables(experts, hidden, inter, shared_inter, 8100 + seed)
+    x = (synth.normal((rows, hidden), 1.0, 8200 + seed) * float(rng.choice([0.01, 1.0, 30.0]))).to(torch.bfloat16)
+    g = synth.generator(8300 + seed)
+    ids = torch.stack([torch.randperm(experts, generator=g)[:top_k] for _ in range(rows)]).to(torch.int32)
+    wt = torch.rand((rows, top_k), generator=g) * 0.5 + 0.05
+    op = E8m0DecodeOps(routed, sh_table.shared_struct(0), rows, top_k, limit, exact=exact)
+    contrib, shared_out = op.contribute(x.to(DEV), ids.to(DEV), wt.to(DEV))
+    torch.cuda.synchronize()
+    got, got_sh, xb = bits(contrib), bits(shared_out), bits(x)
+    ffn = orc.expert_ffn_e8m0 if exact else orc.expert_ffn_e8m0_f32
+    for r in range(rows):
+        for c in range(top_k):
+            assert np.array_equal(got[r, c], ffn(1, xb[r], *ref[int(ids[r, c])], limit, float(wt[r, c]))), (r, c)
+        assert np.array_equal(got_sh[r], ffn(0, xb[r], *sh_ref, limit, 1.0)), r
+
+
 def test_e8m0_entry_checks_its_contract():
     routed, _, sh_table, _ = _tables(2, 64, 32, 32, 9)
     op = E8m0DecodeOps(routed, sh_table.shared_struct(0), 1, 1, 7.0)

@@ -82,6 +82,42 @@ def test_reference_summation_orders_bit_exact(fmt, form, hidden, inter, rows, to
     assert np.array_equal(op.done.cpu().numpy(), active.numpy())
 
 
+@pytest.mark.parametrize("seed", range(16))
+def test_reference_summation_orders_seeded_sweep(seed):
+    """Bit equality with the reference's two reduction orders at widths the fixed cases do not visit (any multiple of
+    the format's granule from 64 to 1536, hence every residue of the 16- and 64-element strides), 1..9 rows, 1..6
+    choices, with and without a shared expert, every rounding, both boundaries."""
+    rng = np.random.default_rng(7000 + seed)
+    fmt = capi.FMT_BF16 if seed % 2 == 0 else capi.FMT_FP8_CHANNEL
+    form = capi.FORM_LANE16 if (seed // 2) % 2 == 0 else capi.FORM_LANE8
+    gran = 8 if fmt == capi.FMT_BF16 else 16
+    hidden = gran * int(rng.integers(64 // gran, 1536 // gran + 1))
+    inter = gran * int(rng.integers(64 // gran, 768 // gran + 1))
+    experts = int(rng.integers(2, 9))
+    top_k = int(rng.integers(1, min(6, experts) + 1))
+    rows = int(rng.choice([1, 2, 4, 9]))
+    rounding = int(rng.integers(0, 4))
+    limit = float(rng.choice([0.05, 1.0])) if rounding >= 2 else 0.0
+    boundary = int(rng.integers(0, 2))
+    shared = bool(rng.integers(0, 2))
+    print("fmt=%d form=%d hidden=%d inter=%d experts=%d top_k=%d rows=%d rounding=%d limit=%g boundary=%d shared=%d" %
+          (fmt, form, hidden, inter, experts, top_k, rows, rounding, limit, boundary, shared), flush=True)
+    table, ref, sh, x, ids, wt = _case(fmt, experts, hidden, inter, rows, top_k, 7100 + seed, shared)
+    op = DecodeOps(table, sh, rows, top_k, capi.ACT_BF16, rounding, limit, boundary, True)
+    contrib, shared_out = op.contribute(x.to(DEV), ids.to(DEV), wt.to(DEV), form=form)
+    torch.cuda.synchronize()
+    oform = orc.LANE16 if form == capi.FORM_LANE16 else orc.LANE8
+    kind = orc.SILU_RCP if (form == capi.FORM_LANE16 and rounding in (capi.SWIGLU_TWICE, capi.SWIGLU_CLAMPED_TWICE)) else orc.SILU_DIV
+    xb, got = bits(x), bits(contrib)
+    for r in range(rows):
+        for c in range(top_k):
+            want = orc.expert_ffn(xb[r], *ref[int(ids[r, c])], float(wt[r, c]), rounding, limit, boundary, oform, kind)
+            assert np.array_equal(got[r, c], want), (r, c)
+        if shared:
+            want_sh = orc.expert_ffn(xb[r], *ref[experts], 1.0, rounding, limit, 0, oform, kind, apply_weight=False)
+            assert np.array_equal(bits(shared_out)[r], want_sh), r
+
+
 def test_form_entry_rejects_other_formats():
     table, _ = make_table(capi.FMT_FP8_BLOCK128, 2, 256, 128, 5)
     op = DecodeOps(table, None, 1, 1, weights_f32=True)
