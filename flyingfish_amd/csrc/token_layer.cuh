@@ -14,7 +14,8 @@
 //     (launch tag << 16 | BF16 value) with a device-coherent store. A reader accepts a word only when its tag is this
 //     launch's, so data and "ready" flag are one atomic store: no waiting for stores to be acknowledged and no
 //     cache-wide operations (a release / acquire pair at device scope writes back and invalidates whole L2s; with
-//     2048 waves doing that the layer took 60 us longer).
+//     2048 waves doing that the layer took 60 us longer). The arena starts zero-filled (tag 0 is never used) and the
+//     last block to leave clears the words again, so a launch never meets words of an earlier one.
 //   * Down phase. A work item is one OUTPUT row of y with the rows of every group's down matrix that produce it, in
 //     combine order, so the per-expert results of a row meet in one wave: weighting and the ordered combine happen in
 //     registers, contributions are neither written nor read back. The first down rows are requested before the block
@@ -55,10 +56,10 @@ __global__ __launch_bounds__(256) void k_token_layer(const FinishParams q) {
   __shared__ uint64_t s_slot[FFMOE_MAX_TOP_K][6];
   __shared__ float s_glob[FFMOE_MAX_TOP_K][3];
   __shared__ float s_wk[FFMOE_MAX_TOP_K];
-  __shared__ int s_nr, s_gave_up;
+  __shared__ int s_nr, s_gave_up, s_last;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = uni(tid >> 6);
-  // launch tag, 1 .. 65535: never 0, so an arena that was zero-filled once holds no word that looks valid
+  // launch tag, 1 .. 65535: never 0, so a zero-filled arena holds no word that looks valid
   const uint32_t tag = 1u + uint32_t(uni(int(__hip_atomic_load(q.gen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)))) % 65535u;
   const bool ordered = !(q.mode == FFMOE_COMBINE_ACCUM_FP32 || q.mode == FFMOE_COMBINE_ACCUM_BF16);
   const bool select_here = p.route.logits != nullptr;
@@ -273,14 +274,6 @@ __global__ __launch_bounds__(256) void k_token_layer(const FinishParams q) {
     gu_finish_item(acc);
   }
   if (d_cur < H) static_for<G>([&](auto pc) { d_issue(pc, d_cur); });
-  // rows of choices that are not live are rewritten too (tagged zeros): every word of the arena carries the tag of the
-  // latest launch that used it, so a stale word can never be older than one launch
-  {
-    const long long NW = (long long)gridDim.x * 4, gw = (long long)blockIdx.x * 4 + wave;
-    const int lo = int((long long)I * gw / NW), hi = int((long long)I * (gw + 1) / NW);
-    for (int row = nr; row < K; ++row)
-      for (int j = lo + lane; j < hi; j += 64) store_agent(q.h32 + size_t(row) * p.h_stride + j, tag << 16);
-  }
   // Activations of every group: tagged words -> BF16 rows in LDS, by the whole block. A word is accepted only with
   // this launch's tag; the last words arrive when the slowest wave of the grid has finished its last gate/up item,
   // and until then the rows requested above keep the memory pipe busy.
@@ -370,11 +363,20 @@ __global__ __launch_bounds__(256) void k_token_layer(const FinishParams q) {
   if (tid == 0) {
     if (s_gave_up && q.status) atomicOr(q.status, 2u);
     const unsigned int left = __hip_atomic_fetch_add(q.exited, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (left + 1 == gridDim.x) {  // last block out: clear the claim counters, the next launch gets a new tag
+    s_last = left + 1 == gridDim.x;
+    if (s_last) {  // last block out: clear the claim counters, the next launch gets a new tag
       for (int i = 0; i < 128; ++i) __hip_atomic_store(q.claims + i * 32, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       __hip_atomic_store(q.exited, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       __hip_atomic_fetch_add(q.gen, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
+  }
+  __syncthreads();
+  // Every other block has left, so nobody reads the arena any more: the last block hands it back zero-filled, as it
+  // found it. A launch therefore never meets a word of an earlier one, whatever their shapes and however often the
+  // 16-bit tag has come round.
+  if (s_last) {
+    const int words = (K + 1) * p.h_stride;
+    for (int i = tid; i < words; i += 256) q.h32[i] = 0u;
   }
 }
 

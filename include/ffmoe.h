@@ -252,12 +252,11 @@ int ffmoe_decode_contribute_from_logits(const ffmoe_expert_table* table, const f
  * moe_ffn_weight_f32 and moe_combine* of NativeMoe::run for one token (src/backend/cuda/moe/decode.rs:1187-1297); ids,
  * weights and y are bit-identical to those launches. logits == NULL: args->ids / weights / active are inputs as in
  * ffmoe_decode_contribute. The grid stays resident and hands activations between its blocks through args->scratch
- * (ffmoe_decode_scratch_bytes bytes, which must have been zero-filled ONCE before the first call that uses it: a word
- * of the arena counts as an activation of this launch only if its upper half carries the launch's non-zero 16-bit
- * tag. The arena therefore belongs to this entry point and to ONE (top_k, shared expert) shape: the other entry
- * points store untagged BF16 pairs in their scratch, whose upper halves can equal a tag, and the tag repeats every
- * 65535 launches of a device, which is harmless only while every launch rewrites every word the next one waits for.
- * Zero-fill the arena again before changing either);
+ * (ffmoe_decode_scratch_bytes bytes, which must be zero-filled ONCE before the first call that uses it: a word of
+ * the arena counts as an activation of the launch only if its upper half carries the launch's non-zero 16-bit tag,
+ * and the last block of every launch hands the arena back zero-filled. The arena belongs to this entry point: the
+ * other entry points store untagged BF16 pairs in their scratch, whose upper halves can equal a tag, so zero-fill it
+ * again after lending it to one of them);
  * contributions, shared_out and done are not written. Bit 0 of *status is set for
  * a live choice naming an expert that is out of range or not valid (its contribution is skipped), bit 1 if a block
  * gave up waiting for another (y is then not valid; happens only when the grid cannot be resident at once, e.g. two

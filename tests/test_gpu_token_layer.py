@@ -122,6 +122,40 @@ def test_token_layer_at_dsv3_width_many_launches():
             assert np.array_equal(bits(y), want[i]), it
     torch.cuda.synchronize()
     assert np.array_equal(bits(y), want[39 % 4]) and int(status.item()) == 0
+    # every launch hands its arena back zero-filled, so no launch can meet a word of an earlier one
+    assert int(op.token_scratch.view(torch.int32).count_nonzero().item()) == 0
+
+
+def test_token_layer_shapes_may_alternate_on_one_arena():
+    """Two layers of different shape (top_k, widths, with and without a shared expert) take turns on ONE arena: each
+    launch must reproduce its separate launches, which holds only because the arena is clean between launches."""
+    cases = []
+    arena = None
+    for n, (hidden, inter, experts, top_k, shared) in enumerate([(1024, 512, 8, 6, True), (512, 1024, 6, 2, False)]):
+        table, _ = make_table(capi.FMT_FP8_BLOCK128, experts + (1 if shared else 0), hidden, inter, 300 + n)
+        sh = table.shared_struct(experts) if shared else None
+        table.experts = experts
+        op = DecodeOps(table, sh, 1, top_k, capi.ACT_BF16, capi.SWIGLU_TWICE, 0.0, capi.WEIGHT_AFTER_DOWN_BF16, True)
+        x = rand_bf16((1, hidden), 1.0, 310 + n).to(DEV)
+        gi = synth.generator(320 + n)
+        ids = torch.randperm(experts, generator=gi)[:top_k].to(torch.int32).view(1, top_k).to(DEV)
+        wt = (torch.rand((1, top_k), generator=gi) * 0.5 + 0.05).to(DEV)
+        mode = capi.COMBINE_UNGATED if shared else capi.COMBINE_ROUTED
+        op.done.zero_()
+        c, s = op.contribute(x, ids, wt)
+        want = bits(CombineOps.combine(c, s, ids, mode, done=op.done)).copy()
+        cases.append((op, x, ids, wt, mode, want, torch.zeros((1, hidden), dtype=torch.bfloat16, device=DEV)))
+    size = max(c[0].scratch.numel() for c in cases)
+    arena = torch.zeros(size, dtype=torch.uint8, device=DEV)
+    for op, *_ in cases:
+        op.token_scratch = arena[: op.scratch.numel()]
+    status = torch.zeros(1, dtype=torch.int32, device=DEV)
+    for it in range(12):
+        op, x, ids, wt, mode, want, y = cases[it % 2]
+        assert op.token_layer(x, ids, wt, mode, y, status=status)
+        torch.cuda.synchronize()
+        assert np.array_equal(bits(y), want), it
+    assert int(status.item()) == 0 and int(arena.view(torch.int32).count_nonzero().item()) == 0
 
 
 def test_token_layer_flags_bad_expert_and_declines_batches():
