@@ -3,6 +3,7 @@
 // the per-128 E4M3 activation quantizer and the elementwise SwiGLU.
 #include "gemv.cuh"
 #include "api.h"
+#include <cstdlib>
 
 namespace ffmoe {
 
@@ -85,6 +86,100 @@ __global__ __launch_bounds__(256) void k_linear(const LinearParams p) {
       for (int s = 0; s < S; ++s) compute_step(items - 1, s);
       item_end(items - 1);
     }
+  }
+}
+
+// Skinny linear for 5..16 activation rows per pass on the BF16 matrix cores (FP8 128x128-block weights). The
+// streaming kernel above pays one v_dot2 per weight pair and activation row and serves at most 4 (K > 4096) or 8 rows
+// per pass over the weights; here the weights are dequantized once (the same BF16 effective weights, bit for bit) and a
+// 16-row activation panel meets them in v_mfma_f32_16x16x32_bf16: products of BF16 values are exact in FP32, the sum
+// is the matrix core's FP32 accumulation, so the result differs from the FP32 fma chain only in summation order.
+//
+// Block = 8 waves on TR weight rows (8 rows when that is what it takes to have a block per CU, the upper half of the
+// 16-row operand then repeats them and is dropped); the waves split the contraction. x goes through LDS in panels of
+// at most 3584 columns x 16 rows (rows past m are zeros). Per 64 columns a lane loads 16 codes of one weight row
+// (columns 16c .. 16c+15 of the 64 for lane group c), which feed two instructions (first and second 8), and reads the
+// matching 2 x 8 activations of its token from LDS. The eight partial tiles are added in wave order through LDS.
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+
+template <int TR>
+__global__ __launch_bounds__(512) void k_linear_fp8_mfma(const LinearParams p, int m0) {
+  constexpr int NW = 8, UMAX = 7, PANEL = 3584;
+  extern __shared__ __align__(16) uint8_t lds[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = uni(tid >> 6);
+  const int K = p.k, N = p.n;
+  const int n0 = blockIdx.x * TR;
+  const int mcount = p.m - m0 < 16 ? p.m - m0 : 16;
+  const int i = lane & 15, c = lane >> 4;
+  const uint8_t* wrow = reinterpret_cast<const uint8_t*>(p.codes) + size_t(n0 + (i & (TR - 1))) * K + c * 16;
+  const float* srow = reinterpret_cast<const float*>(p.scales) + size_t(n0 >> 7) * ((K + 127) >> 7);  // TR divides 128
+  const int panel = K < PANEL ? K : PANEL;
+  const int stride = panel * 2 + 16;  // bytes per token row in LDS; the 16 spread the 16 tokens of a read over all banks
+  f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+  u32x4 wv[UMAX], wn[UMAX];
+  float sc[UMAX], sn[UMAX];
+  // unconditional requests (clamped index), masked at use
+  auto request = [&](int k_lo, u32x4 (&wd)[UMAX], float (&sd)[UMAX]) {
+    const int pk = K - k_lo < panel ? K - k_lo : panel;
+    const int units = pk >> 6;
+    const int u_lo = units * wave / NW, u_hi = units * (wave + 1) / NW;  // at most UMAX units of 64 columns
+#pragma unroll
+    for (int u = 0; u < UMAX; ++u) {
+      const int idx = u_lo + u < u_hi ? u_lo + u : (u_hi > u_lo ? u_hi - 1 : 0);
+      const int k0 = k_lo + 64 * idx;
+      wd[u] = load16_stream(wrow + k0);
+      sd[u] = load_global<float>(srow + (k0 >> 7));
+    }
+  };
+  request(0, wv, sc);
+  for (int k_lo = 0; k_lo < K; k_lo += panel) {
+    const int pk = K - k_lo < panel ? K - k_lo : panel;
+    const int units = pk >> 6;
+    const int u_lo = units * wave / NW, u_hi = units * (wave + 1) / NW;
+    __syncthreads();  // the previous panel has been read
+    {
+      const int per_row = pk >> 3;
+      for (int v = tid; v < 16 * per_row; v += 512) {
+        const int j = v / per_row, q = v - j * per_row;
+        u32x4 val = {0u, 0u, 0u, 0u};
+        if (j < mcount) val = load16(p.x + size_t(m0 + j) * K + k_lo + q * 8);
+        *reinterpret_cast<u32x4*>(lds + size_t(j) * stride + q * 16) = val;
+      }
+    }
+    __syncthreads();
+    const bool more = k_lo + panel < K;
+    if (more) request(k_lo + panel, wn, sn);  // the next panel's weights travel while this one is multiplied
+#pragma unroll
+    for (int u = 0; u < UMAX; ++u) {
+      if (u_lo + u < u_hi) {
+        uint32_t w[8];
+#pragma unroll
+        for (int d = 0; d < 4; ++d) dequant4_e4m3(wv[u][d], sc[u], w[2 * d], w[2 * d + 1]);
+        const uint8_t* xb = lds + size_t(i) * stride + size_t(64 * (u_lo + u) + 16 * c) * 2;
+        const u32x4 b0 = *reinterpret_cast<const u32x4*>(xb), b1 = *reinterpret_cast<const u32x4*>(xb + 16);
+        const u32x4 a0 = {w[0], w[1], w[2], w[3]}, a1 = {w[4], w[5], w[6], w[7]};
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a0), __builtin_bit_cast(bf16x8_t, b0), acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a1), __builtin_bit_cast(bf16x8_t, b1), acc, 0, 0, 0);
+      }
+    }
+    if (more) {
+#pragma unroll
+      for (int u = 0; u < UMAX; ++u) { wv[u] = wn[u]; sc[u] = sn[u]; }
+    }
+  }
+  // lane (token i, group c) holds weight rows 4c .. 4c+3 of the tile; the waves' tiles are added in wave order
+  __syncthreads();
+  float* red = reinterpret_cast<float*>(lds);  // [wave][row 0..15][token 0..15]
+#pragma unroll
+  for (int r = 0; r < 4; ++r) red[(wave * 16 + 4 * c + r) * 16 + i] = acc[r];
+  __syncthreads();
+  if (tid < 16 * TR) {
+    const int j = tid / TR, r = tid - j * TR;
+    float v = red[r * 16 + j];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) v = __fadd_rn(v, red[(w * 16 + r) * 16 + j]);
+    if (j < mcount) p.y[size_t(m0 + j) * N + n0 + r] = f32_to_bf16(v);
   }
 }
 
@@ -214,6 +309,20 @@ extern "C" __attribute__((visibility("default"))) int ffmoe_linear_fp8_block(con
   }
   FF_REQUIRE(act_mode == FFMOE_ACT_BF16, FFMOE_ERR_UNSUPPORTED, "unknown act_mode %d", act_mode);
   LinearParams p{(const uint16_t*)x, (uint16_t*)y, (uint64_t)(uintptr_t)w_codes, (uint64_t)(uintptr_t)w_scales, nullptr, m, n, k};
+  // more rows than the streaming kernel serves in one pass over the weights: the matrix-core kernel, 16 rows per pass
+  const int one_pass = size_t(k) * 2 * 8 <= 64 * 1024 ? 8 : 4;
+  (void)one_pass;
+  if (m > 4 && k % 64 == 0 && n % 16 == 0 && !getenv("FFMOE_LINEAR_NO_MFMA")) {
+    const int panel = k < 3584 ? k : 3584;
+    const size_t tile = size_t(16) * (panel * 2 + 16);
+    const size_t lds = tile > 8 * 16 * 16 * 4 ? tile : 8 * 16 * 16 * 4;  // the x panel, later the eight partial tiles
+    const bool wide = n / 16 >= num_cus_l();
+    for (int m0 = 0; m0 < m; m0 += 16) {
+      if (wide) hipLaunchKernelGGL((k_linear_fp8_mfma<16>), dim3(n / 16), dim3(512), lds, (hipStream_t)stream, p, m0);
+      else hipLaunchKernelGGL((k_linear_fp8_mfma<8>), dim3(n / 8), dim3(512), lds, (hipStream_t)stream, p, m0);
+    }
+    return ff_launch_status();
+  }
   return launch_linear<FmtFp8>(p, (hipStream_t)stream);
 }
 

@@ -315,7 +315,9 @@ int ffmoe_linear_fp8_block_w8a8(const void* w_codes, const float* w_scales, cons
 
 /* BF16 activations against a 128x128-f32 block-scaled FP8 weight.
  * act_mode FFMOE_ACT_BF16: w = bf16(e4m3*scale) in registers (the W8A16 contract of fp8_gemv_bf16 /
- * fp8_skinny_bf16_mM, kernels/fp8_linear.cu:353-511, with f32 instead of BF16 scales).
+ * fp8_skinny_bf16_mM, kernels/fp8_linear.cu:353-511, with f32 instead of BF16 scales). Up to 4 rows are FP32 fma
+ * chains per weight row; more rows (k % 64 == 0, n % 16 == 0) take the same effective weights through the BF16 matrix
+ * cores, 16 rows per pass over the weights: FP32 accumulation in the instruction's order, same tolerance.
  * act_mode FFMOE_ACT_FP8_BLOCK128: NativeProjection::run (linear.rs:1352-1405): quantize then W8A8;
  * needs scratch of m*k + 4*m*ceil(k/128) bytes (256-byte aligned), otherwise scratch may be NULL. */
 int ffmoe_linear_fp8_block(const void* w_codes, const float* w_scales, const void* x, void* y,

@@ -507,6 +507,33 @@ def test_linear_fp8_block_w8a16(m, k, n):
     assert_close_bf16(y, f64, "fp8 linear vs f64")
 
 
+@pytest.mark.parametrize("m,k,n", [
+    (5, 7168, 64),     # two x panels, 8-row tiles
+    (16, 3648, 48),    # 57 column units: a second panel of one unit, waves without work
+    (33, 256, 4096),   # a block per 16 weight rows, three passes of 16 / 16 / 1 rows
+    (9, 192, 32),      # three units for eight waves
+])
+def test_linear_fp8_block_matrix_core_path(m, k, n):
+    """More than 4 rows go through the BF16 matrix cores: the same effective weights, FP32 accumulation in the
+    instruction's order; against the reference's Lane8 order and the FP64 sum, and against the streaming kernel."""
+    import os
+    w = synth.normal((n, k), 0.02, 700 + m)
+    codes, scales = synth.quant_fp8_block(w)
+    x = rand_bf16((m, k), 1.0, 710 + m)
+    y = bits(Fp8Ops.linear(codes.to(DEV), scales.to(DEV), x.to(DEV)))
+    eff = orc.dequant_fp8_block(codes.numpy(), scales.numpy())
+    assert_close_bf16(y, orc.linear_skinny(eff, bits(x), 2), "fp8 linear (matrix cores) vs f64")
+    os.environ["FFMOE_LINEAR_NO_MFMA"] = "1"
+    try:
+        y2 = bits(Fp8Ops.linear(codes.to(DEV), scales.to(DEV), x.to(DEV)))
+    finally:
+        del os.environ["FFMOE_LINEAR_NO_MFMA"]
+    assert_close_bf16(y, y2, "fp8 linear: matrix cores vs streaming kernel")
+    # rows are independent: a row computed alone (streaming kernel) and inside the 16-row panel agree to the bar, and
+    # the panel's padding rows leave nothing behind
+    assert orc.rel_l2(y, y2) < 1e-3
+
+
 @pytest.mark.parametrize("m", [1, 3, 16])
 def test_linear_nvfp4_and_bf16(m):
     n, k = 192, 2048
