@@ -89,22 +89,22 @@ __global__ __launch_bounds__(256) void k_linear(const LinearParams p) {
   }
 }
 
-// Skinny linear for 5..16 activation rows per pass on the BF16 matrix cores (FP8 128x128-block weights). The
-// streaming kernel above pays one v_dot2 per weight pair and activation row and serves at most 4 (K > 4096) or 8 rows
-// per pass over the weights; here the weights are dequantized once (the same BF16 effective weights, bit for bit) and a
-// 16-row activation panel meets them in v_mfma_f32_16x16x32_bf16: products of BF16 values are exact in FP32, the sum
-// is the matrix core's FP32 accumulation, so the result differs from the FP32 fma chain only in summation order.
+// Skinny linear for up to 16 activation rows per pass on the BF16 matrix cores. The streaming kernel above pays one
+// v_dot2 per weight pair and activation row and serves at most 4 (K > 4096) or 8 rows per pass over the weights; here
+// the weights are dequantized once (the same BF16 effective weights, bit for bit) and a 16-row activation panel meets
+// them in v_mfma_f32_16x16x32_bf16: products of BF16 values are exact in FP32, the sum is the matrix core's FP32
+// accumulation, so the result differs from the FP32 fma chain only in summation order.
 //
-// Block = 8 waves on TR weight rows (8 rows when that is what it takes to have a block per CU, the upper half of the
+// Block = 8 waves on TR weight rows (8 rows when that is what it takes to have a block per CU; the upper half of the
 // 16-row operand then repeats them and is dropped); the waves split the contraction. x goes through LDS in panels of
-// at most 3584 columns x 16 rows (rows past m are zeros). Per 64 columns a lane loads 16 codes of one weight row
-// (columns 16c .. 16c+15 of the 64 for lane group c), which feed two instructions (first and second 8), and reads the
-// matching 2 x 8 activations of its token from LDS. The eight partial tiles are added in wave order through LDS.
+// at most 3584 columns x 16 rows (rows past m are zeros). A unit is 4 * EPL columns: lane (row i, group c) loads the
+// 16-byte chunk 4 * unit + c of its weight row (EPL elements), which feeds EPL / 8 instructions of 8 elements each,
+// and reads the matching activations of its token from LDS. The eight partial tiles are added in wave order.
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 
-template <int TR>
-__global__ __launch_bounds__(512) void k_linear_fp8_mfma(const LinearParams p, int m0) {
-  constexpr int NW = 8, UMAX = 7, PANEL = 3584;
+template <class F, int TR>
+__global__ __launch_bounds__(512) void k_linear_mfma(const LinearParams p, int m0) {
+  constexpr int NW = 8, PANEL = 3584, UC = 4 * F::EPL, UMAX = (PANEL / UC + NW - 1) / NW;
   extern __shared__ __align__(16) uint8_t lds[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = uni(tid >> 6);
@@ -112,30 +112,27 @@ __global__ __launch_bounds__(512) void k_linear_fp8_mfma(const LinearParams p, i
   const int n0 = blockIdx.x * TR;
   const int mcount = p.m - m0 < 16 ? p.m - m0 : 16;
   const int i = lane & 15, c = lane >> 4;
-  const uint8_t* wrow = reinterpret_cast<const uint8_t*>(p.codes) + size_t(n0 + (i & (TR - 1))) * K + c * 16;
-  const float* srow = reinterpret_cast<const float*>(p.scales) + size_t(n0 >> 7) * ((K + 127) >> 7);  // TR divides 128
+  const float global = p.global ? load_global<float>(p.global) : 1.0f;
+  const typename F::Row wrow = F::row(p.codes, p.scales, global, n0 + (i & (TR - 1)), K);
   const int panel = K < PANEL ? K : PANEL;
   const int stride = panel * 2 + 16;  // bytes per token row in LDS; the 16 spread the 16 tokens of a read over all banks
   f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
-  u32x4 wv[UMAX], wn[UMAX];
-  float sc[UMAX], sn[UMAX];
+  typename F::Chunk wv[UMAX], wn[UMAX];
   // unconditional requests (clamped index), masked at use
-  auto request = [&](int k_lo, u32x4 (&wd)[UMAX], float (&sd)[UMAX]) {
+  auto request = [&](int k_lo, typename F::Chunk (&wd)[UMAX]) {
     const int pk = K - k_lo < panel ? K - k_lo : panel;
-    const int units = pk >> 6;
-    const int u_lo = units * wave / NW, u_hi = units * (wave + 1) / NW;  // at most UMAX units of 64 columns
+    const int units = pk / UC;
+    const int u_lo = units * wave / NW, u_hi = units * (wave + 1) / NW;  // at most UMAX units
 #pragma unroll
     for (int u = 0; u < UMAX; ++u) {
       const int idx = u_lo + u < u_hi ? u_lo + u : (u_hi > u_lo ? u_hi - 1 : 0);
-      const int k0 = k_lo + 64 * idx;
-      wd[u] = load16_stream(wrow + k0);
-      sd[u] = load_global<float>(srow + (k0 >> 7));
+      F::load(wd[u], wrow, (k_lo + UC * idx) / F::EPL + c);
     }
   };
-  request(0, wv, sc);
+  request(0, wv);
   for (int k_lo = 0; k_lo < K; k_lo += panel) {
     const int pk = K - k_lo < panel ? K - k_lo : panel;
-    const int units = pk >> 6;
+    const int units = pk / UC;
     const int u_lo = units * wave / NW, u_hi = units * (wave + 1) / NW;
     __syncthreads();  // the previous panel has been read
     {
@@ -149,23 +146,24 @@ __global__ __launch_bounds__(512) void k_linear_fp8_mfma(const LinearParams p, i
     }
     __syncthreads();
     const bool more = k_lo + panel < K;
-    if (more) request(k_lo + panel, wn, sn);  // the next panel's weights travel while this one is multiplied
+    if (more) request(k_lo + panel, wn);  // the next panel's weights travel while this one is multiplied
 #pragma unroll
     for (int u = 0; u < UMAX; ++u) {
       if (u_lo + u < u_hi) {
-        uint32_t w[8];
+        uint32_t w[F::EPL / 2];
+        F::dequant(wv[u], w, true);
+        const uint8_t* xb = lds + size_t(i) * stride + size_t(UC * (u_lo + u) + F::EPL * c) * 2;
 #pragma unroll
-        for (int d = 0; d < 4; ++d) dequant4_e4m3(wv[u][d], sc[u], w[2 * d], w[2 * d + 1]);
-        const uint8_t* xb = lds + size_t(i) * stride + size_t(64 * (u_lo + u) + 16 * c) * 2;
-        const u32x4 b0 = *reinterpret_cast<const u32x4*>(xb), b1 = *reinterpret_cast<const u32x4*>(xb + 16);
-        const u32x4 a0 = {w[0], w[1], w[2], w[3]}, a1 = {w[4], w[5], w[6], w[7]};
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a0), __builtin_bit_cast(bf16x8_t, b0), acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a1), __builtin_bit_cast(bf16x8_t, b1), acc, 0, 0, 0);
+        for (int t = 0; t < F::EPL / 8; ++t) {
+          const u32x4 b = *reinterpret_cast<const u32x4*>(xb + 16 * t);
+          const u32x4 a = {w[4 * t], w[4 * t + 1], w[4 * t + 2], w[4 * t + 3]};
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), acc, 0, 0, 0);
+        }
       }
     }
     if (more) {
 #pragma unroll
-      for (int u = 0; u < UMAX; ++u) { wv[u] = wn[u]; sc[u] = sn[u]; }
+      for (int u = 0; u < UMAX; ++u) wv[u] = wn[u];
     }
   }
   // lane (token i, group c) holds weight rows 4c .. 4c+3 of the tile; the waves' tiles are added in wave order
@@ -272,6 +270,23 @@ int launch_linear(const LinearParams& p, hipStream_t st) {
   return ff_launch_status();
 }
 
+// the matrix-core kernel takes whole units of 4 * EPL columns
+template <class F>
+bool mfma_linear_fits(int k) { return k % (4 * F::EPL) == 0 && !getenv("FFMOE_LINEAR_NO_MFMA"); }
+
+template <class F>
+int launch_linear_mfma(const LinearParams& p, hipStream_t st) {
+  const int panel = p.k < 3584 ? p.k : 3584;
+  const size_t tile = size_t(16) * (panel * 2 + 16);
+  const size_t lds = tile > 8 * 16 * 16 * 4 ? tile : 8 * 16 * 16 * 4;  // the x panel, later the eight partial tiles
+  const bool wide = p.n / 16 >= num_cus_l();
+  for (int m0 = 0; m0 < p.m; m0 += 16) {
+    if (wide) hipLaunchKernelGGL((k_linear_mfma<F, 16>), dim3(p.n / 16), dim3(512), lds, st, p, m0);
+    else hipLaunchKernelGGL((k_linear_mfma<F, 8>), dim3(p.n / 8), dim3(512), lds, st, p, m0);
+  }
+  return ff_launch_status();
+}
+
 int check_linear(const void* w, const void* x, const void* y, int m, int n, int k, int kgran) {
   FF_REQUIRE(m >= 1 && n >= 1 && k >= kgran && k % kgran == 0, FFMOE_ERR_SHAPE, "linear m=%d n=%d k=%d (k must be a positive multiple of %d)", m, n, k, kgran);
   FF_REQUIRE(size_t(k) * 2 <= 64 * 1024, FFMOE_ERR_SHAPE, "linear k=%d exceeds the LDS row staging (32768)", k);
@@ -309,20 +324,7 @@ extern "C" __attribute__((visibility("default"))) int ffmoe_linear_fp8_block(con
   }
   FF_REQUIRE(act_mode == FFMOE_ACT_BF16, FFMOE_ERR_UNSUPPORTED, "unknown act_mode %d", act_mode);
   LinearParams p{(const uint16_t*)x, (uint16_t*)y, (uint64_t)(uintptr_t)w_codes, (uint64_t)(uintptr_t)w_scales, nullptr, m, n, k};
-  // more rows than the streaming kernel serves in one pass over the weights: the matrix-core kernel, 16 rows per pass
-  const int one_pass = size_t(k) * 2 * 8 <= 64 * 1024 ? 8 : 4;
-  (void)one_pass;
-  if (m > 4 && k % 64 == 0 && n % 16 == 0 && !getenv("FFMOE_LINEAR_NO_MFMA")) {
-    const int panel = k < 3584 ? k : 3584;
-    const size_t tile = size_t(16) * (panel * 2 + 16);
-    const size_t lds = tile > 8 * 16 * 16 * 4 ? tile : 8 * 16 * 16 * 4;  // the x panel, later the eight partial tiles
-    const bool wide = n / 16 >= num_cus_l();
-    for (int m0 = 0; m0 < m; m0 += 16) {
-      if (wide) hipLaunchKernelGGL((k_linear_fp8_mfma<16>), dim3(n / 16), dim3(512), lds, (hipStream_t)stream, p, m0);
-      else hipLaunchKernelGGL((k_linear_fp8_mfma<8>), dim3(n / 8), dim3(512), lds, (hipStream_t)stream, p, m0);
-    }
-    return ff_launch_status();
-  }
+  if (m > 4 && n % 16 == 0 && mfma_linear_fits<FmtFp8>(k)) return launch_linear_mfma<FmtFp8>(p, (hipStream_t)stream);
   return launch_linear<FmtFp8>(p, (hipStream_t)stream);
 }
 
@@ -331,12 +333,15 @@ extern "C" __attribute__((visibility("default"))) int ffmoe_linear_nvfp4(const v
   FF_TRY(check_linear(w_codes, x, y, m, n, k, 32));
   FF_PTR2(w_scales); FF_PTR4(global_scale);
   LinearParams p{(const uint16_t*)x, (uint16_t*)y, (uint64_t)(uintptr_t)w_codes, (uint64_t)(uintptr_t)w_scales, global_scale, m, n, k};
+  // up to 16 rows: the direct kernel, bit-equal to the reference's host mirror; beyond, its matrix-core path (nvfp4_linear.cu:262-573)
+  if (m > 16 && n % 16 == 0 && mfma_linear_fits<FmtNvfp4>(k)) return launch_linear_mfma<FmtNvfp4>(p, (hipStream_t)stream);
   return launch_linear<FmtNvfp4>(p, (hipStream_t)stream);
 }
 
 extern "C" __attribute__((visibility("default"))) int ffmoe_gemm_skinny_bf16(const void* w, const void* x, void* y, int m, int n, int k, void* stream) {
   FF_TRY(check_linear(w, x, y, m, n, k, 8));
   LinearParams p{(const uint16_t*)x, (uint16_t*)y, (uint64_t)(uintptr_t)w, 0, nullptr, m, n, k};
+  if (m > 4 && n % 16 == 0 && mfma_linear_fits<FmtBf16>(k)) return launch_linear_mfma<FmtBf16>(p, (hipStream_t)stream);
   return launch_linear<FmtBf16>(p, (hipStream_t)stream);
 }
 

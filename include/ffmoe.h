@@ -324,11 +324,14 @@ int ffmoe_linear_fp8_block(const void* w_codes, const float* w_scales, const voi
                            int m, int n, int k, int act_mode, void* scratch, uint64_t scratch_bytes, void* stream);
 
 /* Replaces NvFp4Ops::gemm (linear.rs:488-551; kernels/nvfp4_linear.cu:50-252): W4A16,
- * w = bf16(e2m1 * (e4m3(scale) * global)). global_scale is a device pointer to one f32. k % 16 == 0. */
+ * w = bf16(e2m1 * (e4m3(scale) * global)). global_scale is a device pointer to one f32. k % 16 == 0. Up to 16 rows
+ * run the direct kernel (the reference's host mirror order); more rows with k % 128 == 0 and n % 16 == 0 the BF16
+ * matrix cores, as the reference switches to its MMA kernel there (kernels/nvfp4_linear.cu:262-573). */
 int ffmoe_linear_nvfp4(const void* w_codes, const void* w_scales, const float* global_scale,
                        const void* x, void* y, int m, int n, int k, void* stream);
 
-/* Replaces gemm_skinny_bf16 (kernels/gemm_skinny.cu:509-675): BF16 weights [n,k]. */
+/* Replaces gemm_skinny_bf16 (kernels/gemm_skinny.cu:509-675): BF16 weights [n,k]. More than 4 rows with k % 32 == 0
+ * and n % 16 == 0 run on the BF16 matrix cores (FP32 accumulation in the instruction's order). */
 int ffmoe_gemm_skinny_bf16(const void* w, const void* x, void* y, int m, int n, int k, void* stream);
 
 /* Replaces silu_mul_split / silu_mul_split_clamped (kernels/act.cu:65-99, :125-159):

@@ -534,6 +534,25 @@ def test_linear_fp8_block_matrix_core_path(m, k, n):
     assert orc.rel_l2(y, y2) < 1e-3
 
 
+@pytest.mark.parametrize("m,k,n", [(40, 2048, 192), (17, 3712, 48), (21, 128, 4096)])
+def test_linear_nvfp4_and_bf16_matrix_core_path(m, k, n):
+    """NVFP4 beyond 16 rows (the reference switches to its MMA kernel there, nvfp4_linear.cu:262-573, bounded by
+    max_abs 0.03125 / rmse 0.004 in its tests; here the usual bar against the FP64 sum) and BF16 weights beyond 4."""
+    w = synth.normal((n, k), 0.02, 800 + m)
+    codes, scales, g = synth.quant_nvfp4(w)
+    x = rand_bf16((m, k), 1.0, 801 + m)
+    gs = torch.tensor([g], dtype=torch.float32, device=DEV)
+    y = bits(NvFp4Ops.gemm(codes.to(DEV), scales.to(DEV), gs, x.to(DEV)))
+    eff = orc.dequant_nvfp4(codes.numpy(), scales.numpy(), g)
+    want = orc.linear_skinny(eff, bits(x), 2)
+    assert_close_bf16(y, want, "nvfp4 linear (matrix cores) vs f64")
+    d = orc.bf16_to_f32(y).astype(np.float64) - orc.bf16_to_f32(want).astype(np.float64)
+    assert np.abs(d).max() <= 0.03125 and np.sqrt((d * d).mean()) <= 0.004
+    wb = w.to(torch.bfloat16)
+    yb = bits(gemm_skinny_bf16(wb.to(DEV), x.to(DEV)))
+    assert_close_bf16(yb, orc.linear_skinny(bits(wb), bits(x), 2), "bf16 skinny (matrix cores)")
+
+
 @pytest.mark.parametrize("m", [1, 3, 16])
 def test_linear_nvfp4_and_bf16(m):
     n, k = 192, 2048
