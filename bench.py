@@ -43,6 +43,8 @@ def parse():
     ap.add_argument("--experts", type=int, default=256)
     ap.add_argument("--ring", type=int, default=64, help="distinct token batches cycled through")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--prefill-act", choices=["fp8", "bf16"], default="fp8", help="prefill: W8A8 on the FP8 matrix cores (block-FP8 "
+                    "experts) or the decode path's W*A16 arithmetic on the BF16 matrix cores (any --format)")
     ap.add_argument("--one-launch", action="store_true", help="one token: selection, gate/up, down and combine in the one resident "
                     "launch (ffmoe_decode_token_layer) instead of launches of their own")
     ap.add_argument("--separate-topk", action="store_true", help="one token: run the top-k selection as a launch of its own "
@@ -165,6 +167,7 @@ def cpu_baseline(args, torch, table, layer, xs, dims):
 
 
 MFMA_FP8_PEAK_TFLOPS = 5000.0
+MFMA_BF16_PEAK_TFLOPS = 2500.0
 
 
 def prefill_main(args, torch, capi, ops, synth):
@@ -185,7 +188,9 @@ def prefill_main(args, torch, capi, ops, synth):
     logits = (pop.log()[None, :] - (-u.log()).log()).to(torch.float32).to(dev)
     x = synth.normal((R, H), 1.0, args.seed + 5000, device=dev, dtype=torch.bfloat16)
     bias = torch.zeros(E, dtype=torch.float32, device=dev)
-    pre = ops.PrefillOps(table, R, K, swiglu=capi.SWIGLU_TWICE, weights_f32=True)
+    a16 = args.prefill_act == "bf16" or args.format == "nvfp4"
+    pre = ops.PrefillOps(table, R, K, swiglu=capi.SWIGLU_TWICE, weights_f32=True, act_mode=capi.ACT_BF16 if a16 else capi.ACT_FP8_BLOCK128)
+    peak = MFMA_BF16_PEAK_TFLOPS if a16 else MFMA_FP8_PEAK_TFLOPS
     ids = torch.empty((R, K), dtype=torch.int32, device=dev)
     wts = torch.empty((R, K), dtype=torch.float32, device=dev)
     y = torch.empty((R, H), dtype=torch.bfloat16, device=dev)
@@ -227,22 +232,25 @@ def prefill_main(args, torch, capi, ops, synth):
     out = {
         "metric": "moe_prefill_ms", "value": ms, "unit": "ms/cohort", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
-        "dtype": "fp8_e4m3 weights x fp8_e4m3 activations (per-128 f32 scales), f32 accumulate", "data": "synthetic",
-        "config": {"workload": "DeepSeek-V3-shape FP8 MoE prefill (BASELINE config 5), %d tokens, Zipf s=1.1" % R,
-                   "hidden": H, "intermediate": I, "experts": E, "top_k": K, "act_mode": "FFMOE_ACT_FP8_BLOCK128 (W8A8)",
+        "dtype": ("%s weights dequantized to bf16 x bf16 activations, f32 accumulate" % args.format) if a16 else
+                 "fp8_e4m3 weights x fp8_e4m3 activations (per-128 f32 scales), f32 accumulate", "data": "synthetic",
+        "config": {"workload": ("DeepSeek-V3-shape %s MoE prefill, %d tokens, Zipf s=1.1" % (args.format.upper(), R)) if a16 else
+                               "DeepSeek-V3-shape FP8 MoE prefill (BASELINE config 5), %d tokens, Zipf s=1.1" % R,
+                   "hidden": H, "intermediate": I, "experts": E, "top_k": K,
+                   "act_mode": "FFMOE_ACT_BF16 (W*A16 on the BF16 matrix cores)" if a16 else "FFMOE_ACT_FP8_BLOCK128 (W8A8)",
                    "tokens": R, "experts_touched": touched, "max_rows_per_expert": int(counts.max()), "min_rows_per_expert": int(counts.min())},
         "tokens_per_s": R / (ms * 1e-3),
         "routed_tflop": flop_total / 1e12,
         "cohort_tflops": flop_total / (ms * 1e-3) / 1e12,
-        "cohort_mfma_frac": flop_total / (ms * 1e-3) / 1e12 / MFMA_FP8_PEAK_TFLOPS,
+        "cohort_mfma_frac": flop_total / (ms * 1e-3) / 1e12 / peak,
         "weight_bytes_once": touched * per,
         "cohort_weight_gbps": touched * per / (ms * 1e-3) / 1e9,
-        "roofline": {"kernel": "ffmoe::k_w8a8_grouped<MF, 0, P> (gate/up grouped GEMM + SwiGLU)", "bound": "mfma",
-                     "achieved": flop0 / (k0_avg * 1e-3) / 1e12, "peak": MFMA_FP8_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": flop0 / (k0_avg * 1e-3) / 1e12 / MFMA_FP8_PEAK_TFLOPS, "traffic": None,
+        "roofline": {"kernel": ("ffmoe::k_w16_grouped<F, MF, 0, P>" if a16 else "ffmoe::k_w8a8_grouped<MF, 0, P>") + " (gate/up grouped GEMM + SwiGLU)", "bound": "mfma",
+                     "achieved": flop0 / (k0_avg * 1e-3) / 1e12, "peak": peak, "unit": "TFLOP/s",
+                     "frac": flop0 / (k0_avg * 1e-3) / 1e12 / peak, "traffic": None,
                      "flop_per_launch": flop0, "avg_ms": k0_avg, "min_ms": k0[0],
                      "weight_bytes_once": touched * per * 2 // 3, "weight_gbps": touched * per * 2 / 3 / (k0_avg * 1e-3) / 1e9},
-        "down_kernel": {"kernel": "ffmoe::k_w8a8_grouped<MF, 1, P>", "avg_ms": k1_avg, "min_ms": k1[0],
+        "down_kernel": {"kernel": "ffmoe::k_w16_grouped<F, MF, 1, P>" if a16 else "ffmoe::k_w8a8_grouped<MF, 1, P>", "avg_ms": k1_avg, "min_ms": k1[0],
                         "tflops": A * 2.0 * H * I / (k1_avg * 1e-3) / 1e12},
     }
     print(json.dumps(out))

@@ -10,6 +10,7 @@
 // kernels/act.cu:125-159, kernels/moe_ffn.cu:870-908) applied per assignment, so results do not depend on which
 // other rows share an expert.
 #include "w8a8_gemm.cuh"
+#include "w16_gemm.cuh"
 #include "api.h"
 #include <algorithm>
 #include <cstdlib>
@@ -198,6 +199,25 @@ int launch_gemm(const GemmParams& p, int mf, unsigned blocks, hipStream_t stream
   return ff_launch_status();
 }
 
+template <class F, int MODE>
+int launch_w16(const W16Params& p, int mf, unsigned blocks, hipStream_t stream) {
+  switch (mf) {
+    case 1: hipLaunchKernelGGL((k_w16_grouped<F, 1, MODE, 2>), dim3(blocks), dim3(256), 0, stream, p); break;
+    case 2: hipLaunchKernelGGL((k_w16_grouped<F, 2, MODE, 2>), dim3(blocks), dim3(256), 0, stream, p); break;
+    default: hipLaunchKernelGGL((k_w16_grouped<F, 4, MODE, 2>), dim3(blocks), dim3(256), 0, stream, p); break;
+  }
+  return ff_launch_status();
+}
+template <int MODE>
+int launch_w16_fmt(int format, const W16Params& p, int mf, unsigned blocks, hipStream_t stream) {
+  switch (format) {
+    case FFMOE_FMT_FP8_BLOCK128: return launch_w16<FmtFp8, MODE>(p, mf, blocks, stream);
+    case FFMOE_FMT_NVFP4: return launch_w16<FmtNvfp4, MODE>(p, mf, blocks, stream);
+    case FFMOE_FMT_FP8_CHANNEL: return launch_w16<FmtFp8Channel, MODE>(p, mf, blocks, stream);
+    default: return launch_w16<FmtBf16, MODE>(p, mf, blocks, stream);
+  }
+}
+
 struct PrefillLayout {
   uint64_t xq, sx, act, aq, sa, counts, offsets, gbase, totals, perm, groups, units0, units1, sh_act, sh_aq, sh_sa, total;
   uint64_t max_groups;
@@ -268,12 +288,23 @@ namespace ffmoe {
 int prefill_impl(const ffmoe_expert_table* table, const ffmoe_prefill* args, int stages, void* stream_) {
   hipStream_t stream = (hipStream_t)stream_;
   FF_REQUIRE(table != nullptr && args != nullptr, FFMOE_ERR_NULL, "table or args is NULL");
-  FF_REQUIRE(table->format == FFMOE_FMT_FP8_BLOCK128, FFMOE_ERR_UNSUPPORTED, "prefill handles FFMOE_FMT_FP8_BLOCK128 experts only (format %d)", table->format);
-  FF_REQUIRE(args->act_mode == FFMOE_ACT_FP8_BLOCK128, FFMOE_ERR_UNSUPPORTED, "prefill runs on the FP8 matrix cores: act_mode must be FFMOE_ACT_FP8_BLOCK128");
+  // FFMOE_ACT_FP8_BLOCK128: W8A8 on the FP8 matrix cores (block-FP8 experts); FFMOE_ACT_BF16: the decode path's W*A16
+  // arithmetic on the BF16 matrix cores, any expert format
+  const bool a16 = args->act_mode == FFMOE_ACT_BF16;
+  FF_REQUIRE(a16 || args->act_mode == FFMOE_ACT_FP8_BLOCK128, FFMOE_ERR_UNSUPPORTED, "prefill act_mode %d (FFMOE_ACT_FP8_BLOCK128 or FFMOE_ACT_BF16)", args->act_mode);
+  if (a16)
+    FF_REQUIRE(table->format == FFMOE_FMT_FP8_BLOCK128 || table->format == FFMOE_FMT_NVFP4 || table->format == FFMOE_FMT_BF16 || table->format == FFMOE_FMT_FP8_CHANNEL,
+               FFMOE_ERR_UNSUPPORTED, "unknown expert format %d", table->format);
+  else
+    FF_REQUIRE(table->format == FFMOE_FMT_FP8_BLOCK128, FFMOE_ERR_UNSUPPORTED, "the W8A8 prefill runs on the FP8 matrix cores and takes FFMOE_FMT_FP8_BLOCK128 experts only (format %d)", table->format);
   const int E = table->experts, H = table->hidden, I = table->inter, R = args->rows, K = args->top_k;
   FF_REQUIRE(E >= 1 && E <= FFMOE_MAX_EXPERTS, FFMOE_ERR_SHAPE, "experts=%d out of range", E);
   FF_REQUIRE(R >= 1 && K >= 1 && K <= FFMOE_MAX_TOP_K && (long long)R * K <= 0x3fffffffLL, FFMOE_ERR_SHAPE, "rows=%d top_k=%d out of range", R, K);
-  FF_REQUIRE(H >= 128 && H % 128 == 0 && I >= 128 && I % 128 == 0, FFMOE_ERR_SHAPE, "hidden=%d and inter=%d must be multiples of 128", H, I);
+  if (a16 && table->format != FFMOE_FMT_FP8_BLOCK128)
+    FF_REQUIRE(H >= 64 && H % 64 == 0 && I >= 64 && I % 64 == 0, FFMOE_ERR_SHAPE, "hidden=%d and inter=%d must be multiples of 64", H, I);
+  else
+    FF_REQUIRE(H >= 128 && H % 128 == 0 && I >= 128 && I % 128 == 0, FFMOE_ERR_SHAPE, "hidden=%d and inter=%d must be multiples of 128", H, I);
+  if (a16 && table->format == FFMOE_FMT_NVFP4) FF_PTR4(table->global_scales);
   FF_REQUIRE(args->swiglu >= 0 && args->swiglu <= 3, FFMOE_ERR_UNSUPPORTED, "unknown SwiGLU mode %d", args->swiglu);
   if (args->swiglu >= 2) FF_REQUIRE(args->swiglu_limit > 0.0f && args->swiglu_limit < INFINITY, FFMOE_ERR_SHAPE, "invalid SwiGLU limit %g", (double)args->swiglu_limit);
   FF_REQUIRE(args->routed_weight == FFMOE_WEIGHT_AFTER_DOWN_BF16 || args->routed_weight == FFMOE_WEIGHT_BEFORE_CONTRIBUTION_BF16,
@@ -284,11 +315,22 @@ int prefill_impl(const ffmoe_expert_table* table, const ffmoe_prefill* args, int
   int SI = 0;
   if (shared) {
     SI = shared->inter;
-    FF_REQUIRE(shared->format == FFMOE_FMT_FP8_BLOCK128, FFMOE_ERR_UNSUPPORTED, "prefill needs an FFMOE_FMT_FP8_BLOCK128 shared expert (format %d)", shared->format);
-    FF_REQUIRE(SI >= 128 && SI % 128 == 0, FFMOE_ERR_SHAPE, "shared inter=%d must be a positive multiple of 128", SI);
+    if (a16) {
+      FF_REQUIRE(shared->format == FFMOE_FMT_FP8_BLOCK128 || shared->format == FFMOE_FMT_NVFP4 || shared->format == FFMOE_FMT_BF16 || shared->format == FFMOE_FMT_FP8_CHANNEL,
+                 FFMOE_ERR_UNSUPPORTED, "unknown shared expert format %d", shared->format);
+      const int gran = shared->format == FFMOE_FMT_FP8_BLOCK128 ? 128 : 64;
+      FF_REQUIRE(SI >= gran && SI % gran == 0 && H % gran == 0, FFMOE_ERR_SHAPE, "shared inter=%d and hidden=%d must be multiples of %d", SI, H, gran);
+    } else {
+      FF_REQUIRE(shared->format == FFMOE_FMT_FP8_BLOCK128, FFMOE_ERR_UNSUPPORTED, "the W8A8 prefill needs an FFMOE_FMT_FP8_BLOCK128 shared expert (format %d)", shared->format);
+      FF_REQUIRE(SI >= 128 && SI % 128 == 0, FFMOE_ERR_SHAPE, "shared inter=%d must be a positive multiple of 128", SI);
+    }
     FF_PTR16(args->shared_out);
-    for (int i = 0; i < 6; ++i)
-      FF_REQUIRE(shared->slot[i] != 0 && shared->slot[i] % (i % 2 ? 4 : 16) == 0, FFMOE_ERR_ALIGN, "shared expert slot[%d] is NULL or misaligned", i);
+    for (int i = 0; i < 6; ++i) {
+      const bool scale_entry = i % 2 == 1;
+      if (scale_entry && shared->format == FFMOE_FMT_BF16) continue;  // BF16 weights carry no scales
+      FF_REQUIRE(shared->slot[i] != 0 && shared->slot[i] % (scale_entry ? (shared->format == FFMOE_FMT_FP8_BLOCK128 ? 4 : 2) : 16) == 0, FFMOE_ERR_ALIGN,
+                 "shared expert slot[%d] is NULL or misaligned", i);
+    }
   }
   const PrefillLayout l = prefill_layout(R, K, E, H, I, SI);
   FF_PTR_ALIGNED(args->scratch, 256);
@@ -321,9 +363,51 @@ int prefill_impl(const ffmoe_expert_table* table, const ffmoe_prefill* args, int
     hipLaunchKernelGGL(k_prefill_fill, dim3(E), dim3(256), 0, stream, lt, b, (long long)A);
     FF_TRY(ff_launch_status());
     // activations -> E4M3 + per-128 scales
-    FF_TRY(ffmoe_quant_fp8_f32_128(args->x, s + l.xq, (float*)(s + l.sx), R, H, stream_));
+    if (!a16) FF_TRY(ffmoe_quant_fp8_f32_128(args->x, s + l.xq, (float*)(s + l.sx), R, H, stream_));
   }
   const unsigned blocks = ((unsigned)num_cus_p() * 2u) & ~7u;
+  if (a16) {
+    // BF16 activations end to end: x -> (gate/up + SwiGLU) -> act -> (down x routing weight) -> contributions
+    W16Params p{};
+    p.slots = table->slots; p.global_scales = table->format == FFMOE_FMT_NVFP4 ? table->global_scales : nullptr;
+    p.groups = b.groups; p.perm = b.perm; p.top_k = K;
+    p.swiglu = args->swiglu; p.limit = args->swiglu_limit; p.routed_weight = args->routed_weight; p.weights_f32 = args->weights_f32;
+    if (stages & 2) {
+      p.a = (const uint16_t*)args->x; p.units = b.units0; p.unit_total = b.totals + 0;
+      p.out = (uint16_t*)(s + l.act); p.K = H; p.N = I;
+      FF_TRY(launch_w16_fmt<0>(table->format, p, mf, blocks, stream));
+    }
+    if (stages & 8) {
+      p.a = (const uint16_t*)(s + l.act); p.units = b.units1; p.unit_total = b.totals + 1;
+      p.out = (uint16_t*)args->contributions; p.done = args->done; p.weights = args->weights; p.K = I; p.N = H;
+      FF_TRY(launch_w16_fmt<1>(table->format, p, mf, blocks, stream));
+    }
+    if (shared) {
+      const int smf = R > 32 ? 4 : R > 16 ? 2 : 1;
+      const int stm = 16 * smf;
+      const uint32_t sgroups = uint32_t((R + stm - 1) / stm);
+      W16Params q{};
+      q.rows_total = R; q.top_k = 1;
+      q.swiglu = args->swiglu; q.limit = args->swiglu_limit;
+      if (stages & 2) {
+        q.a = (const uint16_t*)args->x;
+        q.w0_codes = shared->slot[0]; q.w0_scales = shared->slot[1]; q.w1_codes = shared->slot[2]; q.w1_scales = shared->slot[3];
+        q.g0 = shared->global_scales[0]; q.g1 = shared->global_scales[1];
+        q.total_units = sgroups * uint32_t((SI + 127) / 128);
+        q.out = (uint16_t*)(s + l.sh_act); q.K = H; q.N = SI;
+        FF_TRY(launch_w16_fmt<0>(shared->format, q, smf, std::min<unsigned>(blocks, (q.total_units + 7u) & ~7u), stream));
+      }
+      if (stages & 8) {
+        q.a = (const uint16_t*)(s + l.sh_act);
+        q.w0_codes = shared->slot[4]; q.w0_scales = shared->slot[5]; q.w1_codes = 0; q.w1_scales = 0;
+        q.g0 = shared->global_scales[2]; q.g1 = q.g0;
+        q.total_units = sgroups * uint32_t((H + 255) / 256);
+        q.out = (uint16_t*)args->shared_out; q.K = SI; q.N = H;
+        FF_TRY(launch_w16_fmt<2>(shared->format, q, smf, std::min<unsigned>(blocks, (q.total_units + 7u) & ~7u), stream));
+      }
+    }
+    return 0;
+  }
   GemmParams p{};
   p.slots = table->slots; p.groups = b.groups; p.perm = b.perm; p.top_k = K;
   p.swiglu = args->swiglu; p.limit = args->swiglu_limit; p.routed_weight = args->routed_weight; p.weights_f32 = args->weights_f32;

@@ -1,0 +1,348 @@
+// Grouped W*A16 GEMM on the BF16 matrix cores: the prefill form of the decode path's arithmetic. Weights of any expert
+// format are dequantized in registers to the very BF16 effective weights the decode kernels use
+// (bf16(e4m3 * scale), bf16(e2m1 * (e4m3(scale) * global)), src/fp8.rs:138-145), activations stay BF16, and
+// v_mfma_f32_16x16x32_bf16 accumulates the exact products in FP32 over the whole contraction. This is what the reference's
+// prefill computes for its per-channel FP8 and BF16 experts (moe_gemm_w8a16 and the BF16 grouped GEMM,
+// kernels/moe_prefill.cu:157-350, src/backend/cuda/moe/prefill.rs:1053-1408), whose summation order its own tests bound
+// by tolerance only; NVFP4 and block-FP8 experts get the same treatment.
+//
+// Work model, unit list and token staging are those of k_w8a8_grouped (w8a8_gemm.cuh): a unit is one group of at most
+// 16 * MF token rows of an expert x one tile of output columns, a K block is 64 columns = 128 bytes of a BF16 token row
+// (staged through LDS, XOR-swizzled, shared by the four waves), each wave owns four 16-row weight fragments and streams
+// them global -> registers P K blocks ahead. Per K block a lane holds 16 columns of one weight row: after dequantization
+// two operands of 8 columns, i.e. two instructions per (weight fragment, token fragment).
+//
+// MODE 0: gate/up + SwiGLU with the decode path's roundings (kernels/moe_ffn.cu:98-302) -> act[pos, j]
+// MODE 1: down, then the routing weight at the configured boundary -> contributions[assignment, d], done = 1
+// MODE 2: plain product -> y[row, n] (the shared expert's down projection)
+#pragma once
+#include "gemv.cuh"
+#include "w8a8_gemm.cuh"
+
+namespace ffmoe {
+
+typedef __bf16 w16_bf16x8 __attribute__((ext_vector_type(8)));
+
+// 16 consecutive columns of one weight row -> 8 packed BF16 pairs of effective weights
+template <class F>
+struct W16;
+
+template <>
+struct W16<FmtFp8> {
+  struct Frag { u32x4 codes; float scale; };
+  struct Row { const uint8_t* codes; const float* scales; };
+  static __device__ __forceinline__ Row row(uint64_t codes, uint64_t scales, float, int j, int K) {
+    return Row{reinterpret_cast<const uint8_t*>(codes) + size_t(j) * K, reinterpret_cast<const float*>(scales) + size_t(j >> 7) * ((K + 127) >> 7)};
+  }
+  static __device__ __forceinline__ void load(Frag& f, const Row& r, uint32_t col) {
+    f.codes = load16(r.codes + col);
+    f.scale = load_global<float>(r.scales + (col >> 7));
+  }
+  static __device__ __forceinline__ void dequant(const Frag& f, uint32_t (&w)[8]) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) dequant4_e4m3(f.codes[q], f.scale, w[2 * q], w[2 * q + 1]);
+  }
+};
+
+template <>
+struct W16<FmtFp8Channel> {
+  struct Frag { u32x4 codes; };
+  struct Row { const uint8_t* codes; float scale; };
+  static __device__ __forceinline__ Row row(uint64_t codes, uint64_t scales, float, int j, int K) {
+    return Row{reinterpret_cast<const uint8_t*>(codes) + size_t(j) * K, bf16_to_f32(load_global<uint16_t>(reinterpret_cast<const uint16_t*>(scales) + j))};
+  }
+  static __device__ __forceinline__ void load(Frag& f, const Row& r, uint32_t col) { f.codes = load16(r.codes + col); }
+  static __device__ __forceinline__ void dequant(const Frag& f, const Row& r, uint32_t (&w)[8]) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) dequant4_e4m3(f.codes[q], r.scale, w[2 * q], w[2 * q + 1]);
+  }
+};
+
+template <>
+struct W16<FmtBf16> {
+  struct Frag { u32x4 lo, hi; };
+  struct Row { const uint8_t* codes; };
+  static __device__ __forceinline__ Row row(uint64_t codes, uint64_t, float, int j, int K) {
+    return Row{reinterpret_cast<const uint8_t*>(codes) + size_t(j) * K * 2};
+  }
+  static __device__ __forceinline__ void load(Frag& f, const Row& r, uint32_t col) {
+    f.lo = load16(r.codes + col * 2u);
+    f.hi = load16(r.codes + col * 2u + 16u);
+  }
+  static __device__ __forceinline__ void dequant(const Frag& f, uint32_t (&w)[8]) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) { w[q] = f.lo[q]; w[4 + q] = f.hi[q]; }
+  }
+};
+
+template <>
+struct W16<FmtNvfp4> {
+  struct Frag { u32x2 codes; uint32_t scale; };
+  struct Row { const uint8_t* codes; const uint8_t* scales; float global; };
+  static __device__ __forceinline__ Row row(uint64_t codes, uint64_t scales, float global, int j, int K) {
+    return Row{reinterpret_cast<const uint8_t*>(codes) + size_t(j) * (K >> 1), reinterpret_cast<const uint8_t*>(scales) + size_t(j) * (K >> 4), global};
+  }
+  static __device__ __forceinline__ void load(Frag& f, const Row& r, uint32_t col) {
+    f.codes = load_global<u32x2>(r.codes + (col >> 1));
+    f.scale = uint32_t(load_global<uint8_t>(r.scales + (col >> 4)));  // 16 columns are one scale group
+  }
+  // s = e4m3(scale) * global first, then bf16(e2m1 * s) (kernels/nvfp4_linear.cu:83-98); the E2M1 values come from the
+  // hardware conversion as exact BF16 pairs, low nibble = even column
+  static __device__ __forceinline__ void dequant(const Frag& f, const Row& r, uint32_t (&w)[8]) {
+    const float s = __fmul_rn(e4m3x2_to_f32<false>(f.scale).x, r.global);
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+      const uint32_t d = f.codes[q];
+      uint32_t pr[4];
+      pr[0] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(d, 1.0f, 0));
+      pr[1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(d, 1.0f, 1));
+      pr[2] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(d, 1.0f, 2));
+      pr[3] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(d, 1.0f, 3));
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        w[4 * q + i] = pack_bf16x2(__fmul_rn(__uint_as_float(pr[i] << 16), s), __fmul_rn(__uint_as_float(pr[i] & 0xffff0000u), s));
+    }
+  }
+};
+
+// formats whose dequantization needs the row (a per-row scale or the global scale)
+template <class F> struct W16NeedsRow { static constexpr bool value = false; };
+template <> struct W16NeedsRow<FmtFp8Channel> { static constexpr bool value = true; };
+template <> struct W16NeedsRow<FmtNvfp4> { static constexpr bool value = true; };
+
+struct W16Params {
+  const uint16_t* a;         // activations [*, K] BF16
+  const uint64_t* slots;     // [E, 6] expert table, or NULL: the four addresses below
+  uint64_t w0_codes, w0_scales, w1_codes, w1_scales;  // MODE 0: gate, up; MODE 1/2: w0 only
+  const float* global_scales;  // [E, 3] (NVFP4 table) or NULL
+  float g0, g1;              // global scales when slots == NULL
+  const GemmGroup* groups;   // NULL: rows split arithmetically into groups of TM
+  const u32x2* units;
+  const uint32_t* unit_total;
+  uint32_t total_units;
+  const int* perm;           // permuted position -> assignment index (NULL: identity)
+  const void* weights;       // routing weights per assignment (MODE 1)
+  uint16_t* out;
+  uint32_t* done;
+  int rows_total;
+  int K, N, top_k, weights_f32, swiglu, routed_weight;
+  float limit;
+};
+
+template <class F, int MF, int MODE, int P>
+__global__ __launch_bounds__(256, 2) void k_w16_grouped(const W16Params p) {
+  constexpr int TM = 16 * MF;
+  constexpr int CHUNKS = TM * 8;             // 16-byte token chunks per K block (64 BF16 columns = 128 bytes per row)
+  constexpr int CPT = (CHUNKS + 255) / 256;
+  constexpr int TILE = TM * 128;
+  __shared__ __attribute__((aligned(16))) uint8_t tile[2][TILE];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = uni(tid >> 6);
+  const int K = p.K, N = p.N, KB = K >> 6;
+  const uint32_t total = p.unit_total ? uint32_t(uni(int(load_global<uint32_t>(p.unit_total)))) : p.total_units;
+  const int ntiles = (N + gemm_tile_cols<MODE>() - 1) / gemm_tile_cols<MODE>();
+
+  // one contiguous span of the unit list per XCD (see k_w8a8_grouped)
+  const uint32_t xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3, per_xcd = gridDim.x >> 3;
+  const uint32_t span = (total + 7u) >> 3;
+  const uint32_t span_end = min(total, (xcd + 1u) * span);
+  for (uint32_t u = xcd * span + slot; u < span_end; u += per_xcd) {
+    int expert, start, n, t;
+    if (p.groups) {
+      const u32x2 un = load_global<u32x2>(p.units + u);
+      const int g = uni(int(un.x));
+      t = uni(int(un.y));
+      const int* gd = reinterpret_cast<const int*>(p.groups + g);
+      expert = uni(load_global<int>(gd));
+      start = uni(load_global<int>(gd + 1));
+      n = uni(load_global<int>(gd + 2));
+    } else {
+      const int g = int(u) / ntiles;
+      t = int(u) - g * ntiles;
+      expert = 0;
+      start = g * TM;
+      n = min(TM, p.rows_total - start);
+    }
+    uint64_t wc[2], ws[2];
+    float gl[2] = {p.g0, p.g1};
+    if (p.slots) {
+      const uint64_t* sl = p.slots + size_t(expert) * 6;
+      if (MODE == 0) {
+        wc[0] = uni64(load_global<uint64_t>(sl + 0)); ws[0] = uni64(load_global<uint64_t>(sl + 1));
+        wc[1] = uni64(load_global<uint64_t>(sl + 2)); ws[1] = uni64(load_global<uint64_t>(sl + 3));
+      } else {
+        wc[0] = wc[1] = uni64(load_global<uint64_t>(sl + 4)); ws[0] = ws[1] = uni64(load_global<uint64_t>(sl + 5));
+      }
+      if (p.global_scales) {
+        const float* g3 = p.global_scales + size_t(expert) * 3;
+        gl[0] = unif(load_global<float>(g3 + (MODE == 0 ? 0 : 2)));
+        gl[1] = MODE == 0 ? unif(load_global<float>(g3 + 1)) : gl[0];
+      }
+    } else {
+      wc[0] = p.w0_codes; ws[0] = p.w0_scales;
+      wc[1] = MODE == 0 ? p.w1_codes : p.w0_codes; ws[1] = MODE == 0 ? p.w1_scales : p.w0_scales;
+      if (MODE != 0) gl[1] = gl[0];
+    }
+    // weight rows of this lane's four fragments; fragments past N are clamped onto the last 16 rows and dropped at the store
+    int col0[4];
+    typename W16<F>::Row wrow[4];
+#pragma unroll
+    for (int f = 0; f < 4; ++f) {
+      col0[f] = MODE == 0 ? t * 128 + wave * 32 + (f & 1) * 16 : t * 256 + wave * 64 + f * 16;
+      const int base = min(col0[f], N - 16);
+      const int which = MODE == 0 ? f >> 1 : 0;
+      wrow[f] = W16<F>::row(wc[which], ws[which], gl[which], base + (lane & 15), K);
+    }
+    const uint32_t wcol = uint32_t(lane >> 4) * 16u;  // this lane's 16 columns inside a K block
+
+    // token rows this thread stages
+    const uint8_t* tsrc[CPT];
+    int tdst[CPT];
+#pragma unroll
+    for (int i = 0; i < CPT; ++i) {
+      const int q = min(tid + 256 * i, CHUNKS - 1);
+      const int m = q >> 3, c = q & 7;
+      const int pos = start + min(m, n - 1);
+      const int row = MODE == 0 && p.perm ? load_global<int>(p.perm + pos) / p.top_k : pos;
+      tsrc[i] = reinterpret_cast<const uint8_t*>(p.a) + size_t(row) * K * 2 + c * 16;
+      tdst[i] = m * 128 + ((c ^ (m & 7)) << 4);
+    }
+    const bool stage_chunk = CHUNKS >= 256 || tid < CHUNKS;
+
+    v4f acc[MF][4];
+#pragma unroll
+    for (int m = 0; m < MF; ++m)
+#pragma unroll
+      for (int f = 0; f < 4; ++f) acc[m][f] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+
+    // prologue: weights of the first P K blocks, token tile 0 into LDS, token tile 1 into registers (requests are
+    // issued in the order they are consumed: loads retire in order)
+    typename W16<F>::Frag w[P][4];
+#pragma unroll
+    for (int s = 0; s < P; ++s) {
+      const uint32_t kb = uint32_t(min(s, KB - 1));
+#pragma unroll
+      for (int f = 0; f < 4; ++f) W16<F>::load(w[s][f], wrow[f], kb * 64u + wcol);
+    }
+    u32x4 tv[CPT];
+    {
+#pragma unroll
+      for (int i = 0; i < CPT; ++i) {
+        const u32x4 v = load16(tsrc[i]);
+        if (stage_chunk) *reinterpret_cast<u32x4*>(&tile[0][tdst[i]]) = v;
+      }
+      const uint32_t k1 = uint32_t(min(1, KB - 1));
+#pragma unroll
+      for (int i = 0; i < CPT; ++i) tv[i] = load16(tsrc[i] + k1 * 128u);
+    }
+    __syncthreads();
+
+    // LDS addresses of this lane's token operands: row (16 m + lane % 16), columns 16 (lane / 16) .. + 15 = chunks 2q, 2q + 1
+    int tlo[MF], thi[MF];
+#pragma unroll
+    for (int m = 0; m < MF; ++m) {
+      const int trow = 16 * m + (lane & 15);
+      const int q2 = (lane >> 4) * 2;
+      tlo[m] = trow * 128 + (((q2) ^ (trow & 7)) << 4);
+      thi[m] = trow * 128 + (((q2 + 1) ^ (trow & 7)) << 4);
+    }
+
+    for (int kbo = 0; kbo < KB; kbo += P) {
+#pragma unroll
+      for (int s = 0; s < P; ++s) {
+        const int kb = kbo + s;
+        if (kb < KB) {
+          const uint8_t* tb = tile[kb & 1];
+          w16_bf16x8 a0[4], a1[4];
+#pragma unroll
+          for (int f = 0; f < 4; ++f) {
+            uint32_t wd[8];
+            if constexpr (W16NeedsRow<F>::value) W16<F>::dequant(w[s][f], wrow[f], wd);
+            else W16<F>::dequant(w[s][f], wd);
+            const u32x4 x0 = {wd[0], wd[1], wd[2], wd[3]}, x1 = {wd[4], wd[5], wd[6], wd[7]};
+            a0[f] = __builtin_bit_cast(w16_bf16x8, x0);
+            a1[f] = __builtin_bit_cast(w16_bf16x8, x1);
+          }
+#pragma unroll
+          for (int m = 0; m < MF; ++m) {
+            const u32x4 lo = *reinterpret_cast<const u32x4*>(tb + tlo[m]);
+            const u32x4 hi = *reinterpret_cast<const u32x4*>(tb + thi[m]);
+            const w16_bf16x8 b0 = __builtin_bit_cast(w16_bf16x8, lo), b1 = __builtin_bit_cast(w16_bf16x8, hi);
+#pragma unroll
+            for (int f = 0; f < 4; ++f) {
+              acc[m][f] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0[f], b0, acc[m][f], 0, 0, 0);
+              acc[m][f] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1[f], b1, acc[m][f], 0, 0, 0);
+            }
+          }
+          // publish token tile kb+1 (requested one iteration ago)
+#pragma unroll
+          for (int i = 0; i < CPT; ++i)
+            if (stage_chunk) *reinterpret_cast<u32x4*>(&tile[(kb & 1) ^ 1][tdst[i]]) = tv[i];
+          __syncthreads();
+          // request token tile kb+2, then K block kb+P of the weights into the slot just consumed
+          {
+            const uint32_t kn = uint32_t(min(kb + 2, KB - 1));
+#pragma unroll
+            for (int i = 0; i < CPT; ++i) tv[i] = load16(tsrc[i] + kn * 128u);
+            const uint32_t kw = uint32_t(min(kb + P, KB - 1));
+#pragma unroll
+            for (int f = 0; f < 4; ++f) W16<F>::load(w[s][f], wrow[f], kw * 64u + wcol);
+          }
+        }
+      }
+    }
+
+    // epilogue: a lane holds token (lane % 16) of each row fragment and output columns 4 (lane / 16) .. + 3 of each
+    // weight fragment
+    const int tk = lane & 15, sub = (lane >> 4) * 4;
+#pragma unroll
+    for (int m = 0; m < MF; ++m) {
+      const int token = 16 * m + tk;
+      if (token < n) {
+        const int pos = start + token;
+        if (MODE == 0) {
+#pragma unroll
+          for (int f = 0; f < 2; ++f) {
+            const int col = col0[f] + sub;
+            if (col0[f] + 16 <= N) {
+              uint32_t o[2];
+#pragma unroll
+              for (int h = 0; h < 2; ++h) {
+                const uint32_t lo = swiglu_bf16(bround(acc[m][f][2 * h]), bround(acc[m][f + 2][2 * h]), p.swiglu, p.limit);
+                const uint32_t hi = swiglu_bf16(bround(acc[m][f][2 * h + 1]), bround(acc[m][f + 2][2 * h + 1]), p.swiglu, p.limit);
+                o[h] = lo | (hi << 16);
+              }
+              const u32x2 v = {o[0], o[1]};
+              *reinterpret_cast<u32x2*>(p.out + size_t(pos) * N + col) = v;
+            }
+          }
+        } else {
+          const int a = (MODE == 1 && p.perm) ? load_global<int>(p.perm + pos) : pos;
+          float rw = 1.0f;
+          if (MODE == 1 && p.weights)
+            rw = p.weights_f32 ? load_global<float>(reinterpret_cast<const float*>(p.weights) + a)
+                               : bf16_to_f32(load_global<uint16_t>(reinterpret_cast<const uint16_t*>(p.weights) + a));
+#pragma unroll
+          for (int f = 0; f < 4; ++f) {
+            const int col = col0[f] + sub;
+            if (col0[f] + 16 <= N) {
+              float v[4];
+#pragma unroll
+              for (int r = 0; r < 4; ++r) {
+                if (MODE == 1 && p.weights)
+                  v[r] = p.routed_weight == FFMOE_WEIGHT_AFTER_DOWN_BF16 ? __fmul_rn(bround(acc[m][f][r]), rw) : __fmul_rn(acc[m][f][r], rw);
+                else
+                  v[r] = acc[m][f][r];
+              }
+              const u32x2 o = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+              *reinterpret_cast<u32x2*>(p.out + size_t(a) * N + col) = o;
+            }
+          }
+          if (MODE == 1 && p.done && t == 0 && wave == 0 && lane < 16) p.done[a] = 1u;
+        }
+      }
+    }
+  }
+}
+
+}  // namespace ffmoe

@@ -377,9 +377,12 @@ class PrefillOps:
     arena and the contributions / done buffers."""
 
     def __init__(self, table, rows, top_k, swiglu=capi.SWIGLU_TWICE, swiglu_limit=0.0,
-                 routed_weight=capi.WEIGHT_AFTER_DOWN_BF16, weights_f32=True, shared=None):
+                 routed_weight=capi.WEIGHT_AFTER_DOWN_BF16, weights_f32=True, shared=None, act_mode=capi.ACT_FP8_BLOCK128):
+        """act_mode ACT_FP8_BLOCK128: W8A8 on the FP8 matrix cores (block-FP8 experts); ACT_BF16: the decode path's
+        W*A16 arithmetic on the BF16 matrix cores, experts of any format."""
         self.table = table
         self.rows, self.top_k = rows, top_k
+        self.act_mode = act_mode
         self.cfg = (swiglu, swiglu_limit, routed_weight, int(weights_f32))
         dev = table.slots.device
         si = shared.inter if shared is not None else 0
@@ -429,7 +432,7 @@ class PrefillOps:
     def contribute(self, x, ids, weights, active=None, stage=None, assignment_gen=None):
         """stage None = the whole call; 0..3 = one step (plan, gate/up, re-quantize, down)."""
         swiglu, limit, rw, wf32 = self.cfg
-        a = capi.Prefill(self.rows, self.top_k, capi.ACT_FP8_BLOCK128, swiglu, limit, rw, wf32,
+        a = capi.Prefill(self.rows, self.top_k, self.act_mode, swiglu, limit, rw, wf32,
                          x.data_ptr(), ids.data_ptr(), active.data_ptr() if active is not None else None, weights.data_ptr(),
                          self.contributions.data_ptr(), self.done.data_ptr(), self.scratch.data_ptr(), self.scratch.numel(),
                          ctypes.pointer(self._shared_c) if self._shared_c is not None else None,

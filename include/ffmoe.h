@@ -378,12 +378,20 @@ int ffmoe_combine_residual(const void* contributions, const void* routed_in, con
  * kernels/moe_ffn.cu:870-908), which is how the reference runs block-FP8 prefill (in 16-row chunks).
  * Replaces PrefillOps::prefill_contribute (src/backend/cuda/moe/prefill.rs:1033-1408) and kernels moe_count_scan /
  * moe_permute / moe_gemm_* / silu_mul / moe_scatter_rows (kernels/moe_prefill.cu:364-553).
- * Only FFMOE_FMT_FP8_BLOCK128 tables; hidden and inter multiples of 128. Assignments whose id is out of range,
- * whose expert is not valid or whose active flag is 0 contribute nothing and keep done = 0.
+ * That is act_mode FFMOE_ACT_FP8_BLOCK128 (W8A8): FFMOE_FMT_FP8_BLOCK128 tables only, hidden and inter multiples of 128.
+ * act_mode FFMOE_ACT_BF16 runs the cohort in the decode path's W*A16 arithmetic instead: experts of any format
+ * (block FP8, NVFP4, per-channel FP8, BF16; the shared expert may have another format than the table) are
+ * dequantized in registers to the BF16 effective weights of ffmoe_decode_contribute, activations stay BF16 between
+ * the stages, and the grouped GEMMs run on the BF16 matrix cores with FP32 accumulation: what the reference's prefill
+ * computes for its per-channel FP8 and BF16 experts (moe_gemm_w8a16 and the BF16 grouped GEMM,
+ * kernels/moe_prefill.cu:157-350, whose summation order is bounded by tolerance only), with the decode path's SwiGLU
+ * roundings and routing-weight boundaries; hidden and inter multiples of 64 (128 for block FP8).
+ * Assignments whose id is out of range, whose expert is not valid or whose active flag is 0 contribute nothing and
+ * keep done = 0.
  */
 typedef struct ffmoe_prefill {
   int rows, top_k;
-  int act_mode;            /* FFMOE_ACT_FP8_BLOCK128 */
+  int act_mode;            /* FFMOE_ACT_FP8_BLOCK128 or FFMOE_ACT_BF16 */
   int swiglu; float swiglu_limit;
   int routed_weight;
   int weights_f32;
@@ -394,7 +402,7 @@ typedef struct ffmoe_prefill {
   void* contributions;     /* [rows, top_k, hidden] BF16 */
   uint32_t* done;          /* [rows, top_k] or NULL */
   void* scratch; uint64_t scratch_bytes;
-  const ffmoe_shared_expert* shared; /* always-on expert (FFMOE_FMT_FP8_BLOCK128), or NULL */
+  const ffmoe_shared_expert* shared; /* always-on expert (W8A8: FFMOE_FMT_FP8_BLOCK128), or NULL */
   void* shared_out;        /* [rows, hidden] BF16 = bf16(down output), no routing weight (with shared) */
   const uint64_t* assignment_gen; /* as in ffmoe_decode, or NULL */
 } ffmoe_prefill;

@@ -172,6 +172,68 @@ def test_prefill_seeded_sweep(seed):
     _check_prefill(op, host, bits(x), ids, w, mode, limit, boundary, np.ones_like(ids, dtype=bool), got)
 
 
+@pytest.mark.parametrize("fmt", [capi.FMT_FP8_BLOCK128, capi.FMT_NVFP4, capi.FMT_BF16, capi.FMT_FP8_CHANNEL])
+@pytest.mark.parametrize("rows,top_k,experts,hidden,inter,skew,shared", [
+    (40, 3, 6, 256, 128, 1.1, True),     # groups of 16..64 rows, shared expert of the same format
+    (150, 2, 5, 384, 320, 3.0, False),   # one expert with most of the rows, widths that are 64 mod 128
+    (3, 4, 12, 128, 192, 0.0, True),     # fewer rows than experts
+])
+def test_prefill_w16_matches_the_decode_oracle(fmt, rows, top_k, experts, hidden, inter, skew, shared):
+    """act_mode FFMOE_ACT_BF16: the decode path's W*A16 arithmetic for whole cohorts on the BF16 matrix cores, every
+    expert format. Stage-wise against the oracle of the decode path (the same effective weights; the matrix core's FP32
+    accumulation against the reference's FP32 chains): activations, then the down stage on the device's activations."""
+    from helpers import make_table
+    if fmt == capi.FMT_FP8_BLOCK128 and (hidden % 128 or inter % 128):
+        pytest.skip("128 x 128 block scales")
+    table, ref = make_table(fmt, experts + (1 if shared else 0), hidden, inter, 900 + rows)
+    sh = table.shared_struct(experts) if shared else None
+    table.experts = experts
+    ids, w = _routing(rows, top_k, experts, 910 + rows, skew)
+    active = np.ones_like(ids, dtype=np.uint32)
+    if rows > 2:
+        active[1, 0] = 0
+    x = synth.normal((rows, hidden), 1.0, 920 + rows, dtype=torch.bfloat16)
+    mode, limit, boundary = capi.SWIGLU_CLAMPED_TWICE, 1.0, capi.WEIGHT_BEFORE_CONTRIBUTION_BF16
+    op = ops.PrefillOps(table, rows, top_k, swiglu=mode, swiglu_limit=limit, routed_weight=boundary, weights_f32=True, shared=sh,
+                        act_mode=capi.ACT_BF16)
+    op.contributions.zero_()
+    got = op.contribute(x.cuda(), torch.from_numpy(ids).cuda(), torch.from_numpy(w).cuda(), active=torch.from_numpy(active).cuda())
+    torch.cuda.synchronize()
+    assert np.array_equal(op.done.cpu().numpy() != 0, active != 0)
+    v = op.scratch_views()
+    n_live = int(active.sum())
+    assert int(v["totals"][3].item()) == n_live
+    perm = v["perm"].cpu().numpy()[:n_live]
+    act = bits(v["act"])[:n_live]
+    g2 = bits(got).reshape(rows * top_k, -1)
+    xb = bits(x)
+    flat_ids, flat_w = ids.reshape(-1), w.reshape(-1)
+    assert sorted(perm.tolist()) == np.flatnonzero(active.reshape(-1)).tolist()
+    want_full = np.zeros_like(g2)
+    for pos, a in enumerate(perm):
+        ge, ue, de = ref[int(flat_ids[a])]
+        want, want_act = orc.expert_ffn(xb[a // top_k], ge, ue, de, float(flat_w[a]), mode, limit, boundary, orc.LANE8, orc.SILU_DIV, return_act=True)
+        assert_close_bf16(act[pos][None, :], want_act[None, :], "activations of assignment %d" % a)
+        assert_close_bf16(g2[a][None, :], orc.expert_down(act[pos], de, float(flat_w[a]), boundary, orc.LANE8)[None, :], "down stage of assignment %d" % a)
+        want_full[a] = want
+    # end to end the two stages compose (a flipped BF16 step of an activation moves a cancelled down output by several of
+    # its own steps at these widths): the relative-L2 bar on the whole tensor, element-wise a loose bound
+    assert_close_bf16(g2[perm], want_full[perm], "contributions, end to end", max_ulp=16)
+    dead = np.flatnonzero(active.reshape(-1) == 0)
+    assert not g2[dead].any()
+    if shared:
+        ge, ue, de = ref[experts]
+        so = bits(op.shared_out)
+        sh_act = bits(v["sh_act"])
+        want_sh = np.zeros_like(so)
+        for r in range(rows):
+            want, want_act = orc.expert_ffn(xb[r], ge, ue, de, 1.0, mode, limit, 0, orc.LANE8, orc.SILU_DIV, apply_weight=False, return_act=True)
+            assert_close_bf16(sh_act[r][None, :], want_act[None, :], "shared activations row %d" % r)
+            assert_close_bf16(so[r][None, :], orc.expert_down(sh_act[r], de, 1.0, 0, orc.LANE8, False)[None, :], "shared down row %d" % r)
+            want_sh[r] = want
+        assert_close_bf16(so, want_sh, "shared_out, end to end", max_ulp=16)
+
+
 def test_prefill_skips_inactive_invalid_and_out_of_range():
     rows, top_k, experts, hidden, inter = 24, 4, 8, 256, 128
     table, host = _make_fp8_table(experts, hidden, inter, 6)

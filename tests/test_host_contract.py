@@ -104,9 +104,13 @@ def test_prefill_contract_violations_are_reported_before_launch():
         a = _prefill_args(**kw)
         return L.ffmoe_prefill_contribute(ctypes.byref(t), ctypes.byref(a), None)
     assert L.ffmoe_prefill_contribute(None, None, None) == capi.ERR_NULL
-    assert call(act_mode=capi.ACT_BF16) == capi.ERR_UNSUPPORTED and "matrix cores" in capi.last_error()
+    assert call(act_mode=capi.ACT_E4M3_E8M0_32) == capi.ERR_UNSUPPORTED
     nv = capi.ExpertTable(capi.FMT_NVFP4, 64, 2048, 1280, 16 << 20, None, 32 << 20)
-    assert call(t=nv) == capi.ERR_UNSUPPORTED
+    assert call(t=nv) == capi.ERR_UNSUPPORTED and "matrix cores" in capi.last_error()  # W8A8 takes block-FP8 experts only
+    nv_bare = capi.ExpertTable(capi.FMT_NVFP4, 64, 2048, 1280, 16 << 20, None, None)
+    assert call(t=nv_bare, act_mode=capi.ACT_BF16) == capi.ERR_NULL   # W4A16 prefill: the table must bring its global scales
+    odd16 = capi.ExpertTable(capi.FMT_BF16, 64, 2048 + 32, 1280, 16 << 20, None, None)
+    assert call(t=odd16, act_mode=capi.ACT_BF16) == capi.ERR_SHAPE  # multiples of 64 on the BF16 matrix cores
     assert call(top_k=40) == capi.ERR_SHAPE
     assert call(swiglu=2, swiglu_limit=0.0) == capi.ERR_SHAPE
     assert call(routed_weight=capi.WEIGHT_BEFORE_DOWN_F32) == capi.ERR_UNSUPPORTED
