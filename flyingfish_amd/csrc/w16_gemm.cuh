@@ -110,6 +110,14 @@ template <class F> struct W16NeedsRow { static constexpr bool value = false; };
 template <> struct W16NeedsRow<FmtFp8Channel> { static constexpr bool value = true; };
 template <> struct W16NeedsRow<FmtNvfp4> { static constexpr bool value = true; };
 
+// Formats whose 16 columns are 16 bytes (64 bytes of a row per K block): their weights are requested row-contiguously
+// (4 lanes per row, 16 rows per instruction, whole 64-byte segments) and turned into the operand's lane order through
+// a wave-private LDS buffer. Requested directly in operand order, a lane owns 16 bytes of ONE row, the 16 consecutive
+// lanes of a quarter wave touch 16 different lines, and the vector L1 spends one look-up per 16 bytes.
+template <class F> struct W16Transpose { static constexpr bool value = false; };
+template <> struct W16Transpose<FmtFp8> { static constexpr bool value = true; };
+template <> struct W16Transpose<FmtFp8Channel> { static constexpr bool value = true; };
+
 struct W16Params {
   const uint16_t* a;         // activations [*, K] BF16
   const uint64_t* slots;     // [E, 6] expert table, or NULL: the four addresses below
@@ -135,10 +143,16 @@ __global__ __launch_bounds__(256, 2) void k_w16_grouped(const W16Params p) {
   constexpr int CHUNKS = TM * 8;             // 16-byte token chunks per K block (64 BF16 columns = 128 bytes per row)
   constexpr int CPT = (CHUNKS + 255) / 256;
   constexpr int TILE = TM * 128;
+  constexpr bool TR = W16Transpose<F>::value;
   __shared__ __attribute__((aligned(16))) uint8_t tile[2][TILE];
+  __shared__ __attribute__((aligned(16))) uint8_t wstage[TR ? 4 : 1][TR ? 4 : 1][TR ? 1024 : 16];  // [wave][fragment][16 rows x 64 B]
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = uni(tid >> 6);
   const int K = p.K, N = p.N, KB = K >> 6;
+  // wave-private transposition buffer: written as (row lane / 4, 16-byte piece lane % 4), read as (row lane % 16, piece
+  // lane / 16); pieces are XOR-swizzled by (row / 4) % 4 so that the 16 rows of a read fall into distinct banks
+  const int wr_off = (lane >> 2) * 64 + (((lane & 3) ^ ((lane >> 4) & 3)) << 4);
+  const int rd_off = (lane & 15) * 64 + (((lane >> 4) ^ ((lane >> 2) & 3)) << 4);
   const uint32_t total = p.unit_total ? uint32_t(uni(int(load_global<uint32_t>(p.unit_total)))) : p.total_units;
   const int ntiles = (N + gemm_tile_cols<MODE>() - 1) / gemm_tile_cols<MODE>();
 
@@ -193,7 +207,18 @@ __global__ __launch_bounds__(256, 2) void k_w16_grouped(const W16Params p) {
       const int which = MODE == 0 ? f >> 1 : 0;
       wrow[f] = W16<F>::row(wc[which], ws[which], gl[which], base + (lane & 15), K);
     }
-    const uint32_t wcol = uint32_t(lane >> 4) * 16u;  // this lane's 16 columns inside a K block
+    const uint32_t wcol = TR ? 0u : uint32_t(lane >> 4) * 16u;  // this lane's 16 columns inside a K block
+    typename W16<F>::Row lrow[4];  // what the loads address: the operand's row, or the row-contiguous pattern
+#pragma unroll
+    for (int f = 0; f < 4; ++f) {
+      if constexpr (TR) {
+        const int which = MODE == 0 ? f >> 1 : 0;
+        lrow[f] = W16<F>::row(wc[which], ws[which], gl[which], min(col0[f], N - 16) + (lane >> 2), K);
+        lrow[f].codes += (lane & 3) * 16;
+      } else {
+        lrow[f] = wrow[f];
+      }
+    }
 
     // token rows this thread stages
     const uint8_t* tsrc[CPT];
@@ -222,7 +247,7 @@ __global__ __launch_bounds__(256, 2) void k_w16_grouped(const W16Params p) {
     for (int s = 0; s < P; ++s) {
       const uint32_t kb = uint32_t(min(s, KB - 1));
 #pragma unroll
-      for (int f = 0; f < 4; ++f) W16<F>::load(w[s][f], wrow[f], kb * 64u + wcol);
+      for (int f = 0; f < 4; ++f) W16<F>::load(w[s][f], lrow[f], kb * 64u + wcol);
     }
     u32x4 tv[CPT];
     {
@@ -254,11 +279,23 @@ __global__ __launch_bounds__(256, 2) void k_w16_grouped(const W16Params p) {
         if (kb < KB) {
           const uint8_t* tb = tile[kb & 1];
           w16_bf16x8 a0[4], a1[4];
+          typename W16<F>::Frag wm[4];
+#pragma unroll
+          for (int f = 0; f < 4; ++f) wm[f] = w[s][f];
+          if constexpr (TR) {  // LDS operations of one wave execute in order: no wait between the writes and the reads
+            uint8_t* wl = &wstage[wave][0][0];
+#pragma unroll
+            for (int f = 0; f < 4; ++f) *reinterpret_cast<u32x4*>(wl + f * 1024 + wr_off) = w[s][f].codes;
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int f = 0; f < 4; ++f) wm[f].codes = *reinterpret_cast<const u32x4*>(wl + f * 1024 + rd_off);
+            __builtin_amdgcn_wave_barrier();
+          }
 #pragma unroll
           for (int f = 0; f < 4; ++f) {
             uint32_t wd[8];
-            if constexpr (W16NeedsRow<F>::value) W16<F>::dequant(w[s][f], wrow[f], wd);
-            else W16<F>::dequant(w[s][f], wd);
+            if constexpr (W16NeedsRow<F>::value) W16<F>::dequant(wm[f], wrow[f], wd);
+            else W16<F>::dequant(wm[f], wd);
             const u32x4 x0 = {wd[0], wd[1], wd[2], wd[3]}, x1 = {wd[4], wd[5], wd[6], wd[7]};
             a0[f] = __builtin_bit_cast(w16_bf16x8, x0);
             a1[f] = __builtin_bit_cast(w16_bf16x8, x1);
@@ -286,7 +323,7 @@ __global__ __launch_bounds__(256, 2) void k_w16_grouped(const W16Params p) {
             for (int i = 0; i < CPT; ++i) tv[i] = load16(tsrc[i] + kn * 128u);
             const uint32_t kw = uint32_t(min(kb + P, KB - 1));
 #pragma unroll
-            for (int f = 0; f < 4; ++f) W16<F>::load(w[s][f], wrow[f], kw * 64u + wcol);
+            for (int f = 0; f < 4; ++f) W16<F>::load(w[s][f], lrow[f], kw * 64u + wcol);
           }
         }
       }
