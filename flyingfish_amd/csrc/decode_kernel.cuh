@@ -272,7 +272,7 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
 template <class F> struct Policy { static constexpr int S0 = 8, S0G = 8, NR0 = 1, NR1 = 4, NR1G = 4, S1 = 2, S1G = 2; };
 // NVFP4: two gate and two up rows per unit (NR0 = 2, as many bytes in flight per wave as FP8) measured slower
 // (96 against 91 us per C4 layer): its gate/up stage is bound by the conversion work, not by requests in flight
-template <> struct Policy<FmtNvfp4> { static constexpr int S0 = 4, S0G = 2, NR0 = 1, NR1 = 4, NR1G = 2, S1 = 2, S1G = 1; };
+template <> struct Policy<FmtNvfp4> { static constexpr int S0 = 4, S0G = 4, NR0 = 1, NR1 = 4, NR1G = 2, S1 = 2, S1G = 2; };
 
 inline int decode_num_cus() {
   static int cus = 0;
