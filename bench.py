@@ -32,10 +32,10 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", choices=["decode", "prefill", "widening"], default="decode",
+    ap.add_argument("--workload", choices=["decode", "prefill", "widening", "linear"], default="decode",
                     help="decode = BASELINE config 3 (the headline line); prefill = config 5 (4096 tokens, Zipf s=1.1, FP8 matrix cores); "
                          "widening = the formats and fused steps next to the path (per-channel FP8 / BF16 experts, Lane16 / Lane8 orders, "
-                         "combine + residual)")
+                         "combine + residual); linear = config 2 (standalone FP8 block skinny linear, M = 1, 4, 16, 64)")
     ap.add_argument("--batch", type=int, default=None, help="tokens per step (decode: 1, 8, 64; prefill: 4096)")
     ap.add_argument("--format", choices=["fp8", "nvfp4"], default="fp8",
                     help="routed-expert format: fp8 = config 3 (shared expert FP8 too); nvfp4 = config 4 (NVFP4 routed experts, "
@@ -256,6 +256,46 @@ def prefill_main(args, torch, capi, ops, synth):
     print(json.dumps(out))
 
 
+def linear_main(args, torch, capi, ops, synth):
+    """BASELINE config 2: the standalone FP8 128x128-block skinny linear, bf16 in and out, M in {1, 4, 16} (and 64) at
+    (K, N) = (7168, 2048) and (2048, 7168), over a ring of 24 weight sets (353 MB, beyond the caches). One JSON line;
+    value = M = 16 at K 7168, the case the matrix-core path was built for."""
+    dev = "cuda"
+    rows = {}
+    for k, n in ((7168, 2048), (2048, 7168)):
+        ring = 24
+        ws = []
+        for i in range(ring):
+            w = synth.normal((n, k), 0.02, args.seed + 31 * i + k, device=dev)
+            ws.append(synth.quant_fp8_block(w))
+        for m in (1, 4, 16, 64):
+            x = synth.normal((m, k), 1.0, args.seed + m, device=dev, dtype=torch.bfloat16)
+            y = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
+            for c, sc in ws:
+                ops.Fp8Ops.linear(c, sc, x, out=y)
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            reps = max(1, args.steps // ring)
+            e0.record()
+            for _ in range(reps):
+                for c, sc in ws:
+                    ops.Fp8Ops.linear(c, sc, x, out=y)
+            e1.record()
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) * 1e3 / (reps * ring)
+            nbytes = n * k + 4 * ((n + 127) // 128) * ((k + 127) // 128) + 2 * m * (k + n)
+            rows["k%d_n%d_m%d" % (k, n, m)] = {"us": us, "gbps": nbytes / us / 1e3, "hbm_frac": nbytes / us / 1e3 / HBM_PEAK_GBPS}
+    head = rows["k7168_n2048_m16"]
+    out = {"metric": "fp8_block_linear_us", "value": head["us"], "unit": "us/call", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+           "ms_per_step": head["us"] * 1e-3, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+           "dtype": "fp8_e4m3 weights (f32 128x128 block scales), bf16 activations, f32 accumulate", "data": "synthetic",
+           "config": {"workload": "standalone FP8 block-scaled skinny linear (BASELINE config 2), M = 16, K = 7168, N = 2048"},
+           "roofline": {"kernel": "ffmoe::k_linear_mfma<FmtFp8, TR> (more than 4 rows) / ffmoe::k_linear<FmtFp8, S, RG>", "bound": "hbm",
+                        "achieved": head["gbps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": head["hbm_frac"], "traffic": None},
+           "cases": rows}
+    print(json.dumps(out))
+
+
 def widening_main(args, torch, capi, ops, synth):
     """The rows next to the headline path, timed at the DeepSeek-V3 layer shape with one token (8 of 16 experts +
     shared expert, weights = random codes, resident): per-channel FP8 and BF16 experts on the streaming decode path,
@@ -365,6 +405,8 @@ def main():
         return prefill_main(args, torch, capi, ops, synth)
     if args.workload == "widening":
         return widening_main(args, torch, capi, ops, synth)
+    if args.workload == "linear":
+        return linear_main(args, torch, capi, ops, synth)
     table, layer, xs, dims = build_layer(args, torch, capi, ops, synth)
     H, I, E, K = dims
     torch.cuda.synchronize()
