@@ -151,9 +151,11 @@ static int decode_impl(const ffmoe_expert_table* table, const ffmoe_shared_exper
   const int LK = layout_k < 0 ? K : layout_k;
   FF_REQUIRE(R >= 1 && K >= 0 && (K >= 1 || shared) && K <= FFMOE_MAX_TOP_K && LK >= K && E >= 1 && E <= FFMOE_MAX_EXPERTS, FFMOE_ERR_SHAPE,
              "decode rows=%d top_k=%d experts=%d out of range", R, K, E);
-  FF_REQUIRE((long long)R * K <= FFMOE_DECODE_MAX_ASSIGN, FFMOE_ERR_SHAPE,
-             "decode handles at most %d assignments per call (got %lld); use ffmoe_prefill_contribute", FFMOE_DECODE_MAX_ASSIGN,
-             (long long)R * K);
+  // the reduction-order kernels take one launch block per (row, choice) and no grouping pass: any cohort the grid holds
+  if (form < 0)
+    FF_REQUIRE((long long)R * K <= FFMOE_DECODE_MAX_ASSIGN, FFMOE_ERR_SHAPE,
+               "decode handles at most %d assignments per call (got %lld); use ffmoe_prefill_contribute", FFMOE_DECODE_MAX_ASSIGN,
+               (long long)R * K);
   const int fmt = table->format;
   FF_REQUIRE(fmt == FFMOE_FMT_FP8_BLOCK128 || fmt == FFMOE_FMT_NVFP4 || fmt == FFMOE_FMT_BF16 || fmt == FFMOE_FMT_FP8_CHANNEL, FFMOE_ERR_UNSUPPORTED,
              "unknown expert format %d", fmt);

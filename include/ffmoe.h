@@ -208,7 +208,9 @@ int ffmoe_decode_contribute_stage(const ffmoe_expert_table* table, const ffmoe_s
  * contributions and shared_out equal the CPU path's to the last bit (mixed CPU / GPU expert tiering stays
  * reproducible). Replaces DecodeOps::new_invariant_with_boundaries + contribute (src/backend/cuda/moe/decode.rs:342-520).
  * FFMOE_FMT_BF16 and FFMOE_FMT_FP8_CHANNEL tables only (the formats the CPU path executes); slower than
- * ffmoe_decode_contribute, whose 64-lane sums match these orders to 2 BF16 ulp. */
+ * ffmoe_decode_contribute, whose 64-lane sums match these orders to 2 BF16 ulp. No limit on rows * top_k beyond the
+ * launch grid (rows <= 65535): a prefill cohort in these orders, the arithmetic of moe_gemm_lane16*
+ * (kernels/moe_prefill.cu:13-71), is this call with the cohort's rows. */
 #define FFMOE_FORM_LANE16 0
 #define FFMOE_FORM_LANE8  1
 int ffmoe_decode_contribute_form(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared, const ffmoe_decode* args,

@@ -118,6 +118,28 @@ def test_reference_summation_orders_seeded_sweep(seed):
             assert np.array_equal(bits(shared_out)[r], want_sh), r
 
 
+@pytest.mark.parametrize("form", [capi.FORM_LANE16, capi.FORM_LANE8])
+def test_reference_summation_orders_take_whole_cohorts(form):
+    """More assignments than the streaming decode path groups in one call (600 rows x 8 choices): the reduction-order
+    kernels have no grouping pass, so a prefill cohort runs through the same entry, bit-equal row by row - the
+    arithmetic of the reference's moe_gemm_lane16 pipeline (kernels/moe_prefill.cu:13-71: one 16-lane chain per (row,
+    column), no weight reuse across rows)."""
+    experts, hidden, inter, rows, top_k = 12, 128, 64, 600, 8
+    table, ref, sh, x, ids, wt = _case(capi.FMT_BF16, experts, hidden, inter, rows, top_k, 7600 + form, True)
+    op = DecodeOps(table, sh, rows, top_k, capi.ACT_BF16, capi.SWIGLU_TWICE, 0.0, capi.WEIGHT_AFTER_DOWN_BF16, True)
+    contrib, shared_out = op.contribute(x.to(DEV), ids.to(DEV), wt.to(DEV), form=form)
+    torch.cuda.synchronize()
+    oform = orc.LANE16 if form == capi.FORM_LANE16 else orc.LANE8
+    kind = orc.SILU_RCP if form == capi.FORM_LANE16 else orc.SILU_DIV
+    xb, got, got_sh = bits(x), bits(contrib), bits(shared_out)
+    for r in list(range(0, rows, 37)) + [rows - 1]:
+        for c in range(top_k):
+            want = orc.expert_ffn(xb[r], *ref[int(ids[r, c])], float(wt[r, c]), orc.TWICE, 0.0, 0, oform, kind)
+            assert np.array_equal(got[r, c], want), (r, c)
+        assert np.array_equal(got_sh[r], orc.expert_ffn(xb[r], *ref[experts], 1.0, orc.TWICE, 0.0, 0, oform, kind, apply_weight=False)), r
+    assert int(op.done.sum().item()) == rows * top_k
+
+
 def test_form_entry_rejects_other_formats():
     table, _ = make_table(capi.FMT_FP8_BLOCK128, 2, 256, 128, 5)
     op = DecodeOps(table, None, 1, 1, weights_f32=True)
