@@ -197,6 +197,10 @@ def test_slot_layout_matches_the_reference_catalogue():
     assert 3 * 2048 * 1408 == 8650752 and offs[1] == 8650752 and (size - 8650752) // 1 >= 2112
     offs, size = ExpertTable.slot_layout(capi.FMT_NVFP4, 7168, 2048)
     assert 3 * w // 2 == 22020096 and 3 * w // 16 == 2752512 and offs[1] == 22020096
+    # the published DeepSeek-V4.1 grid (tests/deepseek_contract.rs:587-644): hidden 5120, intermediate 2304, E2M1 codes with
+    # [rows, cols / 32] E8M0 scales: 3 x 5,898,240 code bytes + 3 x 368,640 scale bytes, codes first, then the scales
+    offs, size = ExpertTable.slot_layout(capi.FMT_E2M1_E8M0, 5120, 2304)
+    assert offs == [0, 17_694_720, 5_898_240, 18_063_360, 11_796_480, 18_432_000] and size == 18_800_640
 
 
 def test_synthetic_quantizers_equal_the_oracle():
