@@ -11,6 +11,7 @@
 // other rows share an expert.
 #include "w8a8_gemm.cuh"
 #include "w16_gemm.cuh"
+#include "mx_gemm.cuh"
 #include "api.h"
 #include <algorithm>
 #include <cstdlib>
@@ -218,6 +219,16 @@ int launch_w16_fmt(int format, const W16Params& p, int mf, unsigned blocks, hipS
   }
 }
 
+template <int MODE, int PACKED>
+int launch_mx(const MxParams& p, int mf, unsigned blocks, hipStream_t stream) {
+  switch (mf) {
+    case 1: hipLaunchKernelGGL((k_mx_grouped<1, MODE, PACKED, 2>), dim3(blocks), dim3(256), 0, stream, p); break;
+    case 2: hipLaunchKernelGGL((k_mx_grouped<2, MODE, PACKED, 2>), dim3(blocks), dim3(256), 0, stream, p); break;
+    default: hipLaunchKernelGGL((k_mx_grouped<4, MODE, PACKED, 2>), dim3(blocks), dim3(256), 0, stream, p); break;
+  }
+  return ff_launch_status();
+}
+
 struct PrefillLayout {
   uint64_t xq, sx, act, aq, sa, counts, offsets, gbase, totals, perm, groups, units0, units1, sh_act, sh_aq, sh_sa, total;
   uint64_t max_groups;
@@ -291,12 +302,24 @@ int prefill_impl(const ffmoe_expert_table* table, const ffmoe_prefill* args, int
   // FFMOE_ACT_FP8_BLOCK128: W8A8 on the FP8 matrix cores (block-FP8 experts); FFMOE_ACT_BF16: the decode path's W*A16
   // arithmetic on the BF16 matrix cores, any expert format
   const bool a16 = args->act_mode == FFMOE_ACT_BF16;
+  // FFMOE_FMT_E2M1_E8M0 experts with FFMOE_ACT_E4M3_E8M0_32: the W4A8 contract on the MX matrix cores
+  const bool mx = table->format == FFMOE_FMT_E2M1_E8M0;
+  if (mx) {
+    FF_REQUIRE(args->act_mode == FFMOE_ACT_E4M3_E8M0_32, FFMOE_ERR_UNSUPPORTED, "E2M1/E8M0 experts take FFMOE_ACT_E4M3_E8M0_32 activations (act_mode %d)", args->act_mode);
+    FF_REQUIRE(args->routed_weight == FFMOE_WEIGHT_BEFORE_DOWN_F32 && args->weights_f32 == 1, FFMOE_ERR_UNSUPPORTED,
+               "the routed weight is an f32 applied before the down projection (FFMOE_WEIGHT_BEFORE_DOWN_F32)");
+    FF_REQUIRE(args->swiglu_limit > 0.0f && args->swiglu_limit < INFINITY, FFMOE_ERR_SHAPE, "the contract clamps the SwiGLU inputs: limit %g", (double)args->swiglu_limit);
+    FF_REQUIRE(!args->shared || args->shared->format == FFMOE_FMT_E4M3_E8M0_32, FFMOE_ERR_UNSUPPORTED, "the shared expert must be FFMOE_FMT_E4M3_E8M0_32 (format %d)",
+               args->shared ? args->shared->format : -1);
+    FF_REQUIRE((long long)args->rows * args->top_k <= 65535, FFMOE_ERR_SHAPE, "the activation quantizer takes at most 65535 assignments per call (rows=%d top_k=%d)", args->rows, args->top_k);
+  } else {
   FF_REQUIRE(a16 || args->act_mode == FFMOE_ACT_FP8_BLOCK128, FFMOE_ERR_UNSUPPORTED, "prefill act_mode %d (FFMOE_ACT_FP8_BLOCK128 or FFMOE_ACT_BF16)", args->act_mode);
   if (a16)
     FF_REQUIRE(table->format == FFMOE_FMT_FP8_BLOCK128 || table->format == FFMOE_FMT_NVFP4 || table->format == FFMOE_FMT_BF16 || table->format == FFMOE_FMT_FP8_CHANNEL,
                FFMOE_ERR_UNSUPPORTED, "unknown expert format %d", table->format);
   else
     FF_REQUIRE(table->format == FFMOE_FMT_FP8_BLOCK128, FFMOE_ERR_UNSUPPORTED, "the W8A8 prefill runs on the FP8 matrix cores and takes FFMOE_FMT_FP8_BLOCK128 experts only (format %d)", table->format);
+  }
   const int E = table->experts, H = table->hidden, I = table->inter, R = args->rows, K = args->top_k;
   FF_REQUIRE(E >= 1 && E <= FFMOE_MAX_EXPERTS, FFMOE_ERR_SHAPE, "experts=%d out of range", E);
   FF_REQUIRE(R >= 1 && K >= 1 && K <= FFMOE_MAX_TOP_K && (long long)R * K <= 0x3fffffffLL, FFMOE_ERR_SHAPE, "rows=%d top_k=%d out of range", R, K);
@@ -307,15 +330,18 @@ int prefill_impl(const ffmoe_expert_table* table, const ffmoe_prefill* args, int
   if (a16 && table->format == FFMOE_FMT_NVFP4) FF_PTR4(table->global_scales);
   FF_REQUIRE(args->swiglu >= 0 && args->swiglu <= 3, FFMOE_ERR_UNSUPPORTED, "unknown SwiGLU mode %d", args->swiglu);
   if (args->swiglu >= 2) FF_REQUIRE(args->swiglu_limit > 0.0f && args->swiglu_limit < INFINITY, FFMOE_ERR_SHAPE, "invalid SwiGLU limit %g", (double)args->swiglu_limit);
-  FF_REQUIRE(args->routed_weight == FFMOE_WEIGHT_AFTER_DOWN_BF16 || args->routed_weight == FFMOE_WEIGHT_BEFORE_CONTRIBUTION_BF16,
-             FFMOE_ERR_UNSUPPORTED, "unknown routed_weight %d", args->routed_weight);
+  if (!mx)
+    FF_REQUIRE(args->routed_weight == FFMOE_WEIGHT_AFTER_DOWN_BF16 || args->routed_weight == FFMOE_WEIGHT_BEFORE_CONTRIBUTION_BF16,
+               FFMOE_ERR_UNSUPPORTED, "unknown routed_weight %d", args->routed_weight);
   FF_PTR16(table->slots); FF_PTR16(args->x); FF_PTR4(args->ids); FF_PTR16(args->contributions);
   if (args->weights_f32) FF_PTR4(args->weights); else FF_PTR2(args->weights);
   const ffmoe_shared_expert* shared = args->shared;
   int SI = 0;
   if (shared) {
     SI = shared->inter;
-    if (a16) {
+    if (mx) {
+      FF_REQUIRE(SI >= 128 && SI % 128 == 0, FFMOE_ERR_SHAPE, "shared inter=%d must be a positive multiple of 128", SI);
+    } else if (a16) {
       FF_REQUIRE(shared->format == FFMOE_FMT_FP8_BLOCK128 || shared->format == FFMOE_FMT_NVFP4 || shared->format == FFMOE_FMT_BF16 || shared->format == FFMOE_FMT_FP8_CHANNEL,
                  FFMOE_ERR_UNSUPPORTED, "unknown shared expert format %d", shared->format);
       const int gran = shared->format == FFMOE_FMT_FP8_BLOCK128 ? 128 : 64;
@@ -328,7 +354,7 @@ int prefill_impl(const ffmoe_expert_table* table, const ffmoe_prefill* args, int
     for (int i = 0; i < 6; ++i) {
       const bool scale_entry = i % 2 == 1;
       if (scale_entry && shared->format == FFMOE_FMT_BF16) continue;  // BF16 weights carry no scales
-      FF_REQUIRE(shared->slot[i] != 0 && shared->slot[i] % (scale_entry ? (shared->format == FFMOE_FMT_FP8_BLOCK128 ? 4 : 2) : 16) == 0, FFMOE_ERR_ALIGN,
+      FF_REQUIRE(shared->slot[i] != 0 && shared->slot[i] % (scale_entry ? (shared->format == FFMOE_FMT_FP8_BLOCK128 ? 4 : (mx ? 1 : 2)) : 16) == 0, FFMOE_ERR_ALIGN,
                  "shared expert slot[%d] is NULL or misaligned", i);
     }
   }
@@ -363,9 +389,48 @@ int prefill_impl(const ffmoe_expert_table* table, const ffmoe_prefill* args, int
     hipLaunchKernelGGL(k_prefill_fill, dim3(E), dim3(256), 0, stream, lt, b, (long long)A);
     FF_TRY(ff_launch_status());
     // activations -> E4M3 + per-128 scales
-    if (!a16) FF_TRY(ffmoe_quant_fp8_f32_128(args->x, s + l.xq, (float*)(s + l.sx), R, H, stream_));
+    if (mx) FF_TRY(ffmoe_act_quant_e8m0(args->x, s + l.xq, s + l.sx, R, H, stream_));  // E4M3 codes + one E8M0 byte per 32
+    else if (!a16) FF_TRY(ffmoe_quant_fp8_f32_128(args->x, s + l.xq, (float*)(s + l.sx), R, H, stream_));
   }
   const unsigned blocks = ((unsigned)num_cus_p() * 2u) & ~7u;
+  if (mx) {
+    MxParams p{};
+    p.slots = table->slots; p.groups = b.groups; p.perm = b.perm; p.top_k = K; p.limit = args->swiglu_limit;
+    if (stages & 2) {
+      p.a_codes = s + l.xq; p.a_scales = s + l.sx; p.units = b.units0; p.unit_total = b.totals + 0;
+      p.weights = (const float*)args->weights; p.out = (uint16_t*)(s + l.act); p.K = H; p.N = I;
+      FF_TRY((launch_mx<0, 1>(p, mf, blocks, stream)));
+    }
+    if (stages & 4) FF_TRY(ffmoe_act_quant_e8m0(s + l.act, s + l.aq, s + l.sa, int(A), I, stream_));
+    if (stages & 8) {
+      p.a_codes = s + l.aq; p.a_scales = s + l.sa; p.units = b.units1; p.unit_total = b.totals + 1;
+      p.weights = nullptr; p.out = (uint16_t*)args->contributions; p.done = args->done; p.K = I; p.N = H;
+      FF_TRY((launch_mx<1, 1>(p, mf, blocks, stream)));
+    }
+    if (shared) {
+      const int smf = R > 32 ? 4 : R > 16 ? 2 : 1;
+      const int stm = 16 * smf;
+      const uint32_t sgroups = uint32_t((R + stm - 1) / stm);
+      MxParams q{};
+      q.rows_total = R; q.top_k = 1; q.limit = args->swiglu_limit;
+      if (stages & 2) {
+        q.a_codes = s + l.xq; q.a_scales = s + l.sx;
+        q.w0_codes = shared->slot[0]; q.w0_scales = shared->slot[1]; q.w1_codes = shared->slot[2]; q.w1_scales = shared->slot[3];
+        q.total_units = sgroups * uint32_t((SI + 127) / 128);
+        q.out = (uint16_t*)(s + l.sh_act); q.K = H; q.N = SI;
+        FF_TRY((launch_mx<0, 0>(q, smf, std::min<unsigned>(blocks, (q.total_units + 7u) & ~7u), stream)));
+      }
+      if (stages & 4) FF_TRY(ffmoe_act_quant_e8m0(s + l.sh_act, s + l.sh_aq, s + l.sh_sa, R, SI, stream_));
+      if (stages & 8) {
+        q.a_codes = s + l.sh_aq; q.a_scales = s + l.sh_sa;
+        q.w0_codes = shared->slot[4]; q.w0_scales = shared->slot[5]; q.w1_codes = 0; q.w1_scales = 0;
+        q.total_units = sgroups * uint32_t((H + 255) / 256);
+        q.out = (uint16_t*)args->shared_out; q.K = SI; q.N = H;
+        FF_TRY((launch_mx<2, 0>(q, smf, std::min<unsigned>(blocks, (q.total_units + 7u) & ~7u), stream)));
+      }
+    }
+    return 0;
+  }
   if (a16) {
     // BF16 activations end to end: x -> (gate/up + SwiGLU) -> act -> (down x routing weight) -> contributions
     W16Params p{};

@@ -388,12 +388,20 @@ int ffmoe_combine_residual(const void* contributions, const void* routed_in, con
  * computes for its per-channel FP8 and BF16 experts (moe_gemm_w8a16 and the BF16 grouped GEMM,
  * kernels/moe_prefill.cu:157-350, whose summation order is bounded by tolerance only), with the decode path's SwiGLU
  * roundings and routing-weight boundaries; hidden and inter multiples of 64 (128 for block FP8).
+ * FFMOE_FMT_E2M1_E8M0 tables with act_mode FFMOE_ACT_E4M3_E8M0_32 run the W4A8 contract of ffmoe_decode_contribute_e8m0
+ * for a cohort on the MX matrix cores (v_mfma_scale_f32_16x16x128_f8f6f4 takes E2M1 / E4M3 operands with E8M0 scales
+ * per 32 columns as they are): x is quantized per 32, gate/up dots are rounded to BF16, clamped SwiGLU x the f32
+ * routing weight (routed_weight = FFMOE_WEIGHT_BEFORE_DOWN_F32, weights_f32 = 1, swiglu_limit > 0) gives the BF16
+ * activations, they are quantized per 32 again, and the down dots are stored as BF16 contributions; the shared expert
+ * must be FFMOE_FMT_E4M3_E8M0_32. Same operands and stage boundaries as the exact entry, but the matrix core adds
+ * the products in FP32 in its own order: this is the tolerance-checked variant (kernels/moe_ffn.cu:398-867 is the
+ * contract; the reference has no cohort kernel for it). hidden, inter multiples of 128; rows * top_k <= 65535.
  * Assignments whose id is out of range, whose expert is not valid or whose active flag is 0 contribute nothing and
  * keep done = 0.
  */
 typedef struct ffmoe_prefill {
   int rows, top_k;
-  int act_mode;            /* FFMOE_ACT_FP8_BLOCK128 or FFMOE_ACT_BF16 */
+  int act_mode;            /* FFMOE_ACT_FP8_BLOCK128, FFMOE_ACT_BF16, or FFMOE_ACT_E4M3_E8M0_32 (E2M1/E8M0 tables) */
   int swiglu; float swiglu_limit;
   int routed_weight;
   int weights_f32;

@@ -7,8 +7,8 @@ import torch
 
 import oracle as orc
 from flyingfish_amd import capi, synth
-from flyingfish_amd.ops import E8m0DecodeOps, ExpertTable
-from helpers import bits
+from flyingfish_amd.ops import E8m0DecodeOps, ExpertTable, PrefillOps
+from helpers import assert_close_bf16, bits
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda"
@@ -106,6 +106,62 @@ def test_e8m0_experts_seeded_sweep(seed, exact):
         for c in range(top_k):
             assert np.array_equal(got[r, c], ffn(1, xb[r], *ref[int(ids[r, c])], limit, float(wt[r, c]))), (r, c)
         assert np.array_equal(got_sh[r], ffn(0, xb[r], *sh_ref, limit, 1.0)), r
+
+
+def _down_exact(packed, act_bits, down, sdown):
+    """The contract's down projection of one BF16 activation row: quantize per 32, exact dots, BF16."""
+    hq, hs = orc.act_quant_e8m0(act_bits[None, :])
+    return np.array([orc.scaled_dot_exact(packed, down[d], sdown[d] if packed else sdown[d // 32], hq[0], hs[0])[1]
+                     for d in range(down.shape[0])], dtype=np.uint16)
+
+
+@pytest.mark.parametrize("rows,top_k,experts,hidden,inter,shared_inter", [(40, 3, 6, 256, 128, 128), (130, 2, 3, 384, 256, 128), (5, 4, 9, 128, 128, 256)])
+def test_e8m0_prefill_on_the_mx_matrix_cores(rows, top_k, experts, hidden, inter, shared_inter):
+    """Cohorts of the W4A8 / W8A8 contract through ffmoe_prefill_contribute: the same quantized operands and stage
+    boundaries as the exact decode entry, the dots on v_mfma_scale_f32_16x16x128_f8f6f4 (block scales applied by the
+    matrix core, FP32 accumulation in its own order). Checked per stage against the exact oracle: activations, then the
+    down projection of the device's own activations."""
+    limit = 7.0
+    routed, ref, sh_table, sh_ref = _tables(experts, hidden, inter, shared_inter, 500 + rows)
+    x = rand_bf16((rows, hidden), 1.0, 510 + rows)
+    g = synth.generator(520 + rows)
+    ids = torch.stack([torch.randperm(experts, generator=g)[:top_k] for _ in range(rows)]).to(torch.int32)
+    wt = torch.rand((rows, top_k), generator=g) * 0.5 + 0.05
+    active = torch.ones((rows, top_k), dtype=torch.int32)
+    active[1, 0] = 0
+    op = PrefillOps(routed, rows, top_k, swiglu=capi.SWIGLU_CLAMPED_ONCE, swiglu_limit=limit, routed_weight=capi.WEIGHT_BEFORE_DOWN_F32,
+                    weights_f32=True, shared=sh_table.shared_struct(0), act_mode=capi.ACT_E4M3_E8M0_32)
+    op.contributions.zero_()
+    got = op.contribute(x.to(DEV), ids.to(DEV), wt.to(DEV), active=active.to(DEV))
+    torch.cuda.synchronize()
+    assert np.array_equal(op.done.cpu().numpy() != 0, active.numpy() != 0)
+    v = op.scratch_views()
+    n_live = int(active.sum())
+    assert int(v["totals"][3].item()) == n_live
+    perm = v["perm"].cpu().numpy()[:n_live]
+    act = bits(v["act"])[:n_live]
+    g2 = bits(got).reshape(rows * top_k, -1)
+    xb = bits(x)
+    flat_ids, flat_w = ids.reshape(-1).numpy(), wt.reshape(-1).numpy()
+    want_act = np.zeros_like(act)
+    want_down = np.zeros((n_live, hidden), dtype=np.uint16)
+    want_full = np.zeros((n_live, hidden), dtype=np.uint16)
+    for pos, a in enumerate(perm):
+        m = ref[int(flat_ids[a])]
+        want_full[pos], want_act[pos] = orc.expert_ffn_e8m0(1, xb[a // top_k], *m, limit, float(flat_w[a]), return_act=True)
+        want_down[pos] = _down_exact(1, act[pos], m[4], m[5])
+    assert_close_bf16(act, want_act, "activations", max_ulp=3)
+    assert_close_bf16(g2[perm], want_down, "down projection of the device activations")
+    assert orc.rel_l2(g2[perm], want_full) <= 5e-2
+    assert not g2[np.flatnonzero(active.reshape(-1).numpy() == 0)].any()
+    so, sh_act = bits(op.shared_out), bits(v["sh_act"])
+    want_sa = np.zeros_like(sh_act)
+    want_sd = np.zeros_like(so)
+    for r in range(rows):
+        want_sa[r] = orc.expert_ffn_e8m0(0, xb[r], *sh_ref, limit, 1.0, return_act=True)[1]
+        want_sd[r] = _down_exact(0, sh_act[r], sh_ref[4], sh_ref[5])
+    assert_close_bf16(sh_act, want_sa, "shared activations", max_ulp=3)
+    assert_close_bf16(so, want_sd, "shared down projection of the device activations")
 
 
 def test_e8m0_entry_checks_its_contract():
