@@ -121,6 +121,13 @@ def test_prefill_contract_violations_are_reported_before_launch():
     assert call(t=odd, scratch_bytes=16) == capi.ERR_SCRATCH
     bad = capi.ExpertTable(capi.FMT_FP8_BLOCK128, 64, 2048, 1400, 16 << 20, None, None)
     assert call(t=bad) == capi.ERR_SHAPE
+    mx = capi.ExpertTable(capi.FMT_E2M1_E8M0, 64, 2048, 1280, 16 << 20, None, None)
+    mx_ok = dict(act_mode=capi.ACT_E4M3_E8M0_32, routed_weight=capi.WEIGHT_BEFORE_DOWN_F32, swiglu=capi.SWIGLU_CLAMPED_ONCE, swiglu_limit=7.0)
+    assert call(t=mx) == capi.ERR_UNSUPPORTED and "E4M3_E8M0_32" in capi.last_error()        # FP8 block activations
+    assert call(t=mx, **{**mx_ok, "routed_weight": capi.WEIGHT_AFTER_DOWN_BF16}) == capi.ERR_UNSUPPORTED
+    assert call(t=mx, **{**mx_ok, "swiglu_limit": 0.0}) == capi.ERR_SHAPE
+    assert call(t=mx, **{**mx_ok, "rows": 16384, "top_k": 8}) == capi.ERR_SHAPE and "65535" in capi.last_error()
+    assert call(t=mx, scratch_bytes=64, **mx_ok) == capi.ERR_SCRATCH
     assert L.ffmoe_prefill_contribute_stage(ctypes.byref(table), ctypes.byref(_prefill_args()), 7, None) == capi.ERR_SHAPE
     assert L.ffmoe_prefill_scratch_bytes(0, 8, 256, 7168, 2048, 0) == 0
     need = L.ffmoe_prefill_scratch_bytes(4096, 8, 256, 7168, 2048, 0)
