@@ -53,9 +53,18 @@ __global__ __launch_bounds__(256, 2) void k_mx_grouped(const MxParams p) {
   constexpr int TILE = TM * 128 + TM * 4;  // codes + the K block's four scale bytes per row
   constexpr int WL = PACKED ? 1 : 2;        // 16-byte loads per lane, fragment and K block
   __shared__ __attribute__((aligned(16))) uint8_t tile[2][TILE];
+  // E2M1 experts request their weights row-contiguously (4 lanes per 64-byte row segment, the four
+  // scale bytes of the row as one word) and turn them into operand order through a wave-private LDS buffer, as
+  // k_w16_grouped does: requested in operand order, every lane touches a line of its own for 16 bytes, and once more
+  // for one scale byte. LDS operations of one wave execute in order, so no wait sits between the writes and the reads.
+  constexpr bool TW = PACKED != 0;
+  __shared__ __attribute__((aligned(16))) uint8_t wstage[TW ? 4 : 1][TW ? 4 : 1][TW ? 1024 : 16];
+  __shared__ uint32_t sstage[TW ? 4 : 1][TW ? 4 : 1][TW ? 16 : 1];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = uni(tid >> 6);
   const int K = p.K, N = p.N, KB = K >> 7, SB = K >> 5;
+  const int wr_off = (lane >> 2) * 64 + (((lane & 3) ^ ((lane >> 4) & 3)) << 4);
+  const int rd_off = (lane & 15) * 64 + (((lane >> 4) ^ ((lane >> 2) & 3)) << 4);
   const uint32_t total = p.unit_total ? uint32_t(uni(int(load_global<uint32_t>(p.unit_total)))) : p.total_units;
   const int ntiles = (N + gemm_tile_cols<MODE>() - 1) / gemm_tile_cols<MODE>();
   const int q4 = lane >> 4;  // this lane's scale block inside a K block
@@ -99,10 +108,16 @@ __global__ __launch_bounds__(256, 2) void k_mx_grouped(const MxParams p) {
 #pragma unroll
     for (int f = 0; f < 4; ++f) {
       col0[f] = MODE == 0 ? t * 128 + wave * 32 + (f & 1) * 16 : t * 256 + wave * 64 + f * 16;
-      const int row = min(col0[f], N - 16) + (lane & 15);
       const int which = MODE == 0 ? f >> 1 : 0;
-      wrow[f] = reinterpret_cast<const uint8_t*>(wc[which]) + (PACKED ? size_t(row) * (K >> 1) + q4 * 16 : size_t(row) * K + q4 * 16);
-      srow[f] = reinterpret_cast<const uint8_t*>(ws[which]) + size_t(PACKED ? row : row >> 5) * SB + q4;
+      if (TW) {  // row lane / 4 of the fragment, 16-byte piece lane % 4; the row's scale word
+        const int row = min(col0[f], N - 16) + (lane >> 2);
+        wrow[f] = reinterpret_cast<const uint8_t*>(wc[which]) + size_t(row) * (K >> 1) + (lane & 3) * 16;
+        srow[f] = reinterpret_cast<const uint8_t*>(ws[which]) + size_t(row) * SB;
+      } else {
+        const int row = min(col0[f], N - 16) + (lane & 15);
+        wrow[f] = reinterpret_cast<const uint8_t*>(wc[which]) + (PACKED ? size_t(row) * (K >> 1) + q4 * 16 : size_t(row) * K + q4 * 16);
+        srow[f] = reinterpret_cast<const uint8_t*>(ws[which]) + size_t(PACKED ? row : row >> 5) * SB + q4;
+      }
     }
 
     const uint8_t* tsrc[CPT];
@@ -139,7 +154,7 @@ __global__ __launch_bounds__(256, 2) void k_mx_grouped(const MxParams p) {
       for (int f = 0; f < 4; ++f) {
 #pragma unroll
         for (int l = 0; l < WL; ++l) w[s][f][l] = load16(wrow[f] + kb * (PACKED ? 64u : 128u) + 64u * l);
-        wsc[s][f] = uint32_t(load_global<uint8_t>(srow[f] + kb * 4u));
+        wsc[s][f] = TW ? load_global<uint32_t>(srow[f] + kb * 4u) : uint32_t(load_global<uint8_t>(srow[f] + kb * 4u));
       }
     }
     u32x4 tv[CPT];
@@ -173,6 +188,26 @@ __global__ __launch_bounds__(256, 2) void k_mx_grouped(const MxParams p) {
         const int kb = kbo + s;
         if (kb < KB) {
           const uint8_t* tb = tile[kb & 1];
+          u32x4 wt[4];       // first 16 bytes of the four fragments in operand order
+          uint32_t st[4];    // this lane's weight scale byte
+#pragma unroll
+          for (int f = 0; f < 4; ++f) { wt[f] = w[s][f][0]; st[f] = wsc[s][f]; }
+          if constexpr (TW) {
+            uint8_t* wl = &wstage[wave][0][0];
+            uint32_t* sl = &sstage[wave][0][0];
+#pragma unroll
+            for (int f = 0; f < 4; ++f) {
+              *reinterpret_cast<u32x4*>(wl + f * 1024 + wr_off) = w[s][f][0];
+              if ((lane & 3) == 0) sl[f * 16 + (lane >> 2)] = wsc[s][f];
+            }
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int f = 0; f < 4; ++f) {
+              wt[f] = *reinterpret_cast<const u32x4*>(wl + f * 1024 + rd_off);
+              st[f] = (sl[f * 16 + (lane & 15)] >> (8 * q4)) & 0xffu;
+            }
+            __builtin_amdgcn_wave_barrier();
+          }
 #pragma unroll
           for (int m = 0; m < MF; ++m) {
             const u32x4 lo = *reinterpret_cast<const u32x4*>(tb + tlo[m]);
@@ -183,10 +218,10 @@ __global__ __launch_bounds__(256, 2) void k_mx_grouped(const MxParams p) {
 #pragma unroll
             for (int f = 0; f < 4; ++f) {
               v8i wf;
-              if (PACKED) wf = v8i{int(w[s][f][0][0]), int(w[s][f][0][1]), int(w[s][f][0][2]), int(w[s][f][0][3]), 0, 0, 0, 0};
-              else wf = v8i{int(w[s][f][0][0]), int(w[s][f][0][1]), int(w[s][f][0][2]), int(w[s][f][0][3]),
+              if (PACKED) wf = v8i{int(wt[f][0]), int(wt[f][1]), int(wt[f][2]), int(wt[f][3]), 0, 0, 0, 0};
+              else wf = v8i{int(wt[f][0]), int(wt[f][1]), int(wt[f][2]), int(wt[f][3]),
                             int(w[s][f][WL - 1][0]), int(w[s][f][WL - 1][1]), int(w[s][f][WL - 1][2]), int(w[s][f][WL - 1][3])};
-              acc[m][f] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, tok, acc[m][f], PACKED ? 4 : 0, 0, 0, int(wsc[s][f]), 0, sx);
+              acc[m][f] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, tok, acc[m][f], PACKED ? 4 : 0, 0, 0, int(st[f]), 0, sx);
             }
           }
 #pragma unroll
@@ -204,7 +239,7 @@ __global__ __launch_bounds__(256, 2) void k_mx_grouped(const MxParams p) {
             for (int f = 0; f < 4; ++f) {
 #pragma unroll
               for (int l = 0; l < WL; ++l) w[s][f][l] = load16(wrow[f] + kw * (PACKED ? 64u : 128u) + 64u * l);
-              wsc[s][f] = uint32_t(load_global<uint8_t>(srow[f] + kw * 4u));
+              wsc[s][f] = TW ? load_global<uint32_t>(srow[f] + kw * 4u) : uint32_t(load_global<uint8_t>(srow[f] + kw * 4u));
             }
           }
         }
