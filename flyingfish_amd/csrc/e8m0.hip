@@ -33,8 +33,8 @@ extern "C" __attribute__((visibility("default"))) uint64_t ffmoe_e8m0_scratch_by
 extern "C" __attribute__((visibility("default"))) int ffmoe_act_quant_e8m0(const void* x, void* codes, void* scales, int rows, int k, void* stream) {
   FF_REQUIRE(x && codes && scales, FFMOE_ERR_NULL, "x/codes/scales is NULL");
   FF_REQUIRE(rows >= 1 && rows <= 65535 && k >= 32 && k % 32 == 0, FFMOE_ERR_SHAPE, "rows=%d k=%d: k must be a positive multiple of 32", rows, k);
-  FF_PTR2(x);
-  hipLaunchKernelGGL(k_act_quant_e8m0, dim3((k / 32 + 7) / 8, rows), dim3(256), 0, (hipStream_t)stream, (const uint16_t*)x, k, (uint8_t*)codes, k,
+  FF_PTR16(x); FF_PTR_ALIGNED(codes, 8);
+  hipLaunchKernelGGL(k_act_quant_e8m0, dim3((k / 32 + 63) / 64, rows), dim3(256), 0, (hipStream_t)stream, (const uint16_t*)x, k, (uint8_t*)codes, k,
                      (uint8_t*)scales, k / 32, k, (const uint32_t*)nullptr);
   return ff_launch_status();
 }
@@ -88,17 +88,17 @@ extern "C" __attribute__((visibility("default"))) int ffmoe_decode_contribute_e8
   uint32_t* live = (uint32_t*)(sc + l.live);
   hipStream_t st = (hipStream_t)stream;
   const int S = R * K + R;
-  hipLaunchKernelGGL(k_act_quant_e8m0, dim3((H / 32 + 7) / 8, R), dim3(256), 0, st, p.x, H, sc + l.xq, H, sc + l.xs, H / 32, H, (const uint32_t*)nullptr);
+  hipLaunchKernelGGL(k_act_quant_e8m0, dim3((H / 32 + 63) / 64, R), dim3(256), 0, st, p.x, H, sc + l.xq, H, sc + l.xs, H / 32, H, (const uint32_t*)nullptr);
   hipLaunchKernelGGL(k_e8m0_live, dim3((S + 255) / 256), dim3(256), 0, st, p, live);
   if (exact) hipLaunchKernelGGL((k_e8m0_stage<0>), dim3((imax + 7) / 8, R, K + 1), dim3(256), size_t(H / 32) * 33 * 4, st, q);
   else hipLaunchKernelGGL((k_e8m0_stage_f32<0>), dim3((imax + 7) / 8, R, K + 1), dim3(256), size_t(H) * 4 + size_t(H / 32) * 4, st, q);
   FF_TRY(ff_launch_status());
   // every live down-input row is quantized over imax elements (a shorter row leaves its tail unused)
   if (K > 0)
-    hipLaunchKernelGGL(k_act_quant_e8m0, dim3((I / 32 + 7) / 8, R * K), dim3(256), 0, st, p.h, imax, sc + l.hq, imax, sc + l.hs, imax / 32, I,
+    hipLaunchKernelGGL(k_act_quant_e8m0, dim3((I / 32 + 63) / 64, R * K), dim3(256), 0, st, p.h, imax, sc + l.hq, imax, sc + l.hs, imax / 32, I,
                        (const uint32_t*)live);
   if (shared)
-    hipLaunchKernelGGL(k_act_quant_e8m0, dim3((SI / 32 + 7) / 8, R), dim3(256), 0, st, p.h + size_t(R) * K * imax, imax,
+    hipLaunchKernelGGL(k_act_quant_e8m0, dim3((SI / 32 + 63) / 64, R), dim3(256), 0, st, p.h + size_t(R) * K * imax, imax,
                        sc + l.hq + size_t(R) * K * imax, imax, sc + l.hs + size_t(R) * K * (imax / 32), imax / 32, SI, (const uint32_t*)(live + R * K));
   if (exact) hipLaunchKernelGGL((k_e8m0_stage<1>), dim3((H + 7) / 8, R, K + 1), dim3(256), size_t(imax / 32) * 33 * 4, st, q);
   else hipLaunchKernelGGL((k_e8m0_stage_f32<1>), dim3((H + 7) / 8, R, K + 1), dim3(256), size_t(imax) * 4 + size_t(imax / 32) * 4, st, q);

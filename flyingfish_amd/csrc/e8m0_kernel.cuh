@@ -57,27 +57,38 @@ __device__ __forceinline__ uint16_t bf16_round_f64(double value) {
 }
 
 // One 32-element activation-quant group per half wave, a lane per element (q38_contract.cuh:153-170):
-// grid (ceil(groups / 8), rows_to_quantize), block 256. `live` (optional) marks the rows to quantize.
+// grid (ceil(groups / 64), rows_to_quantize), block 256: four lanes per group of 32, eight elements each (one 16-byte
+// load, one 8-byte store). `live` (optional) marks the rows to quantize.
 __global__ __launch_bounds__(256) void k_act_quant_e8m0(const uint16_t* __restrict__ x, int x_stride, uint8_t* __restrict__ codes,
                                                         int c_stride, uint8_t* __restrict__ scales, int s_stride, int k,
                                                         const uint32_t* __restrict__ live) {
   const int row = blockIdx.y;
   if (live && live[row] == 0u) return;
   const int groups = k >> 5;
-  const int group = blockIdx.x * 8 + (threadIdx.x >> 5);
-  if (group >= groups) return;
-  const int lane = threadIdx.x & 31;
-  const float value = bf16_to_f32(x[size_t(row) * x_stride + size_t(group) * 32 + lane]);
-  float amax = fabsf(value);
+  const int group = blockIdx.x * 64 + (threadIdx.x >> 2);
+  if (group >= groups) return;  // the four lanes of a group leave together
+  const int part = threadIdx.x & 3;
+  const u32x4 w = load16(x + size_t(row) * x_stride + size_t(group) * 32 + part * 8);
+  float v[8];
 #pragma unroll
-  for (int off = 16; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 32));
+  for (int q = 0; q < 4; ++q) { v[2 * q] = bf16lo(w[q]); v[2 * q + 1] = bf16hi(w[q]); }
+  float amax = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[i]));
+  amax = fmaxf(amax, __shfl_xor(amax, 1, 4));
+  amax = fmaxf(amax, __shfl_xor(amax, 2, 4));
   amax = fmaxf(amax, 1e-4f);
   const uint32_t qb = __float_as_uint(__fmul_rn(amax, 1.0f / 448.0f));
   int exponent = int((qb >> 23) & 0xffu) - 127 + ((qb & 0x7fffffu) != 0u ? 1 : 0);
   exponent = exponent < -127 ? -127 : (exponent > 127 ? 127 : exponent);  // the reference traps outside this range
   const float scale = __uint_as_float(uint32_t(exponent + 127) << 23);
-  codes[size_t(row) * c_stride + size_t(group) * 32 + lane] = e4m3_encode(fminf(448.0f, fmaxf(-448.0f, __fdiv_rn(value, scale))));
-  if (lane == 0) scales[size_t(row) * s_stride + group] = uint8_t(exponent + 127);
+  uint32_t out[2] = {0u, 0u};
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+    out[i >> 2] |= uint32_t(e4m3_encode(fminf(448.0f, fmaxf(-448.0f, __fdiv_rn(v[i], scale))))) << (8 * (i & 3));
+  const u32x2 o = {out[0], out[1]};
+  *reinterpret_cast<u32x2*>(codes + size_t(row) * c_stride + size_t(group) * 32 + part * 8) = o;
+  if (part == 0) scales[size_t(row) * s_stride + group] = uint8_t(exponent + 127);
 }
 
 // liveness of every activation slot (rows * top_k routed choices, then one per token row for the shared expert)
