@@ -37,7 +37,7 @@ def parse():
                          "widening = the formats and fused steps next to the path (per-channel FP8 / BF16 experts, Lane16 / Lane8 orders, "
                          "combine + residual); linear = config 2 (standalone FP8 block skinny linear, M = 1, 4, 16, 64)")
     ap.add_argument("--batch", type=int, default=None, help="tokens per step (decode: 1, 8, 64; prefill: 4096)")
-    ap.add_argument("--format", choices=["fp8", "nvfp4"], default="fp8",
+    ap.add_argument("--format", choices=["fp8", "nvfp4", "e2m1"], default="fp8",
                     help="routed-expert format: fp8 = config 3 (shared expert FP8 too); nvfp4 = config 4 (NVFP4 routed experts, "
                          "BF16 shared expert, quoted at --batch 32)")
     ap.add_argument("--experts", type=int, default=256)
@@ -62,6 +62,16 @@ def build_layer(args, torch, capi, ops, synth, make_tokens=True):
     H, I, E, K = 7168, 2048, args.experts, 8
     dev = "cuda"
     nvfp4 = args.format == "nvfp4"
+    if args.format == "e2m1":  # E2M1 codes with one E8M0 scale per 32 columns (the W4A8 contract); prefill cohorts only
+        assert not make_tokens, "--format e2m1 is a prefill workload"
+        table = ops.ExpertTable.allocate(capi.FMT_E2M1_E8M0, E, H, I, dev)
+        for e in range(E):
+            v = table.expert_views(e)
+            for i, shape in enumerate([(I, H), (I, H), (H, I)]):
+                codes, scales = synth.quant_e2m1_e8m0(synth.normal(shape, 0.02, args.seed * 100003 + e * 3 + i, device=dev))
+                v[2 * i].copy_(codes)
+                v[2 * i + 1].copy_(scales)
+        return table, None, None, (H, I, E, K)
     if nvfp4:
         table = ops.ExpertTable.allocate(capi.FMT_NVFP4, E, H, I, dev)
         shared_table = ops.ExpertTable.allocate(capi.FMT_BF16, 1, H, I, dev)
@@ -188,9 +198,14 @@ def prefill_main(args, torch, capi, ops, synth):
     logits = (pop.log()[None, :] - (-u.log()).log()).to(torch.float32).to(dev)
     x = synth.normal((R, H), 1.0, args.seed + 5000, device=dev, dtype=torch.bfloat16)
     bias = torch.zeros(E, dtype=torch.float32, device=dev)
-    a16 = args.prefill_act == "bf16" or args.format == "nvfp4"
-    pre = ops.PrefillOps(table, R, K, swiglu=capi.SWIGLU_TWICE, weights_f32=True, act_mode=capi.ACT_BF16 if a16 else capi.ACT_FP8_BLOCK128)
-    peak = MFMA_BF16_PEAK_TFLOPS if a16 else MFMA_FP8_PEAK_TFLOPS
+    mx = args.format == "e2m1"
+    a16 = not mx and (args.prefill_act == "bf16" or args.format == "nvfp4")
+    if mx:
+        pre = ops.PrefillOps(table, R, K, swiglu=capi.SWIGLU_CLAMPED_ONCE, swiglu_limit=7.0, routed_weight=capi.WEIGHT_BEFORE_DOWN_F32,
+                             weights_f32=True, act_mode=capi.ACT_E4M3_E8M0_32)
+    else:
+        pre = ops.PrefillOps(table, R, K, swiglu=capi.SWIGLU_TWICE, weights_f32=True, act_mode=capi.ACT_BF16 if a16 else capi.ACT_FP8_BLOCK128)
+    peak = MFMA_BF16_PEAK_TFLOPS if a16 else MFMA_FP8_PEAK_TFLOPS  # an E2M1 x E4M3 instruction runs at the 8-bit rate
     ids = torch.empty((R, K), dtype=torch.int32, device=dev)
     wts = torch.empty((R, K), dtype=torch.float32, device=dev)
     y = torch.empty((R, H), dtype=torch.bfloat16, device=dev)
@@ -233,11 +248,13 @@ def prefill_main(args, torch, capi, ops, synth):
         "metric": "moe_prefill_ms", "value": ms, "unit": "ms/cohort", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
         "dtype": ("%s weights dequantized to bf16 x bf16 activations, f32 accumulate" % args.format) if a16 else
+                 "fp4_e2m1 weights x fp8_e4m3 activations, e8m0 scales per 32 applied by the matrix core, f32 accumulate" if mx else
                  "fp8_e4m3 weights x fp8_e4m3 activations (per-128 f32 scales), f32 accumulate", "data": "synthetic",
-        "config": {"workload": ("DeepSeek-V3-shape %s MoE prefill, %d tokens, Zipf s=1.1" % (args.format.upper(), R)) if a16 else
+        "config": {"workload": ("DeepSeek-V3-shape %s MoE prefill, %d tokens, Zipf s=1.1" % (args.format.upper(), R)) if (a16 or mx) else
                                "DeepSeek-V3-shape FP8 MoE prefill (BASELINE config 5), %d tokens, Zipf s=1.1" % R,
                    "hidden": H, "intermediate": I, "experts": E, "top_k": K,
-                   "act_mode": "FFMOE_ACT_BF16 (W*A16 on the BF16 matrix cores)" if a16 else "FFMOE_ACT_FP8_BLOCK128 (W8A8)",
+                   "act_mode": "FFMOE_ACT_BF16 (W*A16 on the BF16 matrix cores)" if a16 else
+                               "FFMOE_ACT_E4M3_E8M0_32 (W4A8 on the MX matrix cores)" if mx else "FFMOE_ACT_FP8_BLOCK128 (W8A8)",
                    "tokens": R, "experts_touched": touched, "max_rows_per_expert": int(counts.max()), "min_rows_per_expert": int(counts.min())},
         "tokens_per_s": R / (ms * 1e-3),
         "routed_tflop": flop_total / 1e12,
@@ -245,12 +262,12 @@ def prefill_main(args, torch, capi, ops, synth):
         "cohort_mfma_frac": flop_total / (ms * 1e-3) / 1e12 / peak,
         "weight_bytes_once": touched * per,
         "cohort_weight_gbps": touched * per / (ms * 1e-3) / 1e9,
-        "roofline": {"kernel": ("ffmoe::k_w16_grouped<F, MF, 0, P>" if a16 else "ffmoe::k_w8a8_grouped<MF, 0, P>") + " (gate/up grouped GEMM + SwiGLU)", "bound": "mfma",
+        "roofline": {"kernel": ("ffmoe::k_w16_grouped<F, MF, 0, P>" if a16 else "ffmoe::k_mx_grouped<MF, 0, 1, P>" if mx else "ffmoe::k_w8a8_grouped<MF, 0, P>") + " (gate/up grouped GEMM + SwiGLU)", "bound": "mfma",
                      "achieved": flop0 / (k0_avg * 1e-3) / 1e12, "peak": peak, "unit": "TFLOP/s",
                      "frac": flop0 / (k0_avg * 1e-3) / 1e12 / peak, "traffic": None,
                      "flop_per_launch": flop0, "avg_ms": k0_avg, "min_ms": k0[0],
                      "weight_bytes_once": touched * per * 2 // 3, "weight_gbps": touched * per * 2 / 3 / (k0_avg * 1e-3) / 1e9},
-        "down_kernel": {"kernel": "ffmoe::k_w16_grouped<F, MF, 1, P>" if a16 else "ffmoe::k_w8a8_grouped<MF, 1, P>", "avg_ms": k1_avg, "min_ms": k1[0],
+        "down_kernel": {"kernel": "ffmoe::k_w16_grouped<F, MF, 1, P>" if a16 else "ffmoe::k_mx_grouped<MF, 1, 1, P>" if mx else "ffmoe::k_w8a8_grouped<MF, 1, P>", "avg_ms": k1_avg, "min_ms": k1[0],
                         "tflops": A * 2.0 * H * I / (k1_avg * 1e-3) / 1e12},
     }
     print(json.dumps(out))
