@@ -105,6 +105,11 @@ struct W16<FmtNvfp4> {
   }
 };
 
+// four consecutive scale bytes of an NVFP4 row; the scale array is only 2-byte aligned by contract
+__device__ __forceinline__ uint32_t nv_scale4(const uint8_t* p) {
+  return uint32_t(load_global<uint16_t>(p)) | (uint32_t(load_global<uint16_t>(p + 2)) << 16);
+}
+
 // formats whose dequantization needs the row (a per-row scale or the global scale)
 template <class F> struct W16NeedsRow { static constexpr bool value = false; };
 template <> struct W16NeedsRow<FmtFp8Channel> { static constexpr bool value = true; };
@@ -144,6 +149,12 @@ __global__ __launch_bounds__(256, 2) void k_w16_grouped(const W16Params p) {
   constexpr int CPT = (CHUNKS + 255) / 256;
   constexpr int TILE = TM * 128;
   constexpr bool TR = W16Transpose<F>::value;
+  // NVFP4: a row's K block is 32 code bytes and 4 scale bytes. Two lanes request one row's codes (32 rows = two
+  // fragments per instruction), the scale bytes of a row come as one word, and both are turned into operand order
+  // (8 code bytes and one scale byte per lane) through wave-private LDS, like the FP8 formats below.
+  constexpr bool NVT = std::is_same<F, FmtNvfp4>::value;
+  __shared__ __attribute__((aligned(16))) uint8_t nstage[NVT ? 4 : 1][NVT ? 2 : 1][NVT ? 1024 : 16];  // [wave][row pair of fragments][32 rows x 32 B]
+  __shared__ uint32_t nscale[NVT ? 4 : 1][NVT ? 2 : 1][NVT ? 32 : 1];
   __shared__ __attribute__((aligned(16))) uint8_t tile[2][TILE];
   __shared__ __attribute__((aligned(16))) uint8_t wstage[TR ? 4 : 1][TR ? 4 : 1][TR ? 1024 : 16];  // [wave][fragment][16 rows x 64 B]
   const int tid = threadIdx.x, lane = tid & 63;
@@ -220,6 +231,20 @@ __global__ __launch_bounds__(256, 2) void k_w16_grouped(const W16Params p) {
       }
     }
 
+    const uint8_t* ncod[2] = {nullptr, nullptr};
+    const uint8_t* nscl[2] = {nullptr, nullptr};
+    if constexpr (NVT) {
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {  // fragments 2j and 2j + 1 are 32 consecutive rows of one matrix
+        const int which = MODE == 0 ? j : 0;
+        const int row = min(col0[2 * j], N - 32) + (lane >> 1);
+        ncod[j] = reinterpret_cast<const uint8_t*>(wc[which]) + size_t(row) * (K >> 1) + (lane & 1) * 16;
+        nscl[j] = reinterpret_cast<const uint8_t*>(ws[which]) + size_t(row) * (K >> 4);
+      }
+    }
+    u32x4 nvc[NVT ? P : 1][2];
+    uint32_t nvs[NVT ? P : 1][2];
+
     // token rows this thread stages
     const uint8_t* tsrc[CPT];
     int tdst[CPT];
@@ -246,8 +271,13 @@ __global__ __launch_bounds__(256, 2) void k_w16_grouped(const W16Params p) {
 #pragma unroll
     for (int s = 0; s < P; ++s) {
       const uint32_t kb = uint32_t(min(s, KB - 1));
+      if constexpr (NVT) {
 #pragma unroll
-      for (int f = 0; f < 4; ++f) W16<F>::load(w[s][f], lrow[f], kb * 64u + wcol);
+        for (int j = 0; j < 2; ++j) { nvc[s][j] = load16(ncod[j] + kb * 32u); nvs[s][j] = nv_scale4(nscl[j] + kb * 4u); }
+      } else {
+#pragma unroll
+        for (int f = 0; f < 4; ++f) W16<F>::load(w[s][f], lrow[f], kb * 64u + wcol);
+      }
     }
     u32x4 tv[CPT];
     {
@@ -282,6 +312,23 @@ __global__ __launch_bounds__(256, 2) void k_w16_grouped(const W16Params p) {
           typename W16<F>::Frag wm[4];
 #pragma unroll
           for (int f = 0; f < 4; ++f) wm[f] = w[s][f];
+          if constexpr (NVT) {
+            uint8_t* nl = &nstage[wave][0][0];
+            uint32_t* ns = &nscale[wave][0][0];
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+              *reinterpret_cast<u32x4*>(nl + j * 1024 + (lane >> 1) * 32 + (lane & 1) * 16) = nvc[s][j];
+              if ((lane & 1) == 0) ns[j * 32 + (lane >> 1)] = nvs[s][j];
+            }
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int f = 0; f < 4; ++f) {
+              const int r32 = (f & 1) * 16 + (lane & 15);
+              wm[f].codes = *reinterpret_cast<const u32x2*>(nl + (f >> 1) * 1024 + r32 * 32 + (lane >> 4) * 8);
+              wm[f].scale = (ns[(f >> 1) * 32 + r32] >> (8 * (lane >> 4))) & 0xffu;
+            }
+            __builtin_amdgcn_wave_barrier();
+          }
           if constexpr (TR) {  // LDS operations of one wave execute in order: no wait between the writes and the reads
             uint8_t* wl = &wstage[wave][0][0];
 #pragma unroll
@@ -322,8 +369,13 @@ __global__ __launch_bounds__(256, 2) void k_w16_grouped(const W16Params p) {
 #pragma unroll
             for (int i = 0; i < CPT; ++i) tv[i] = load16(tsrc[i] + kn * 128u);
             const uint32_t kw = uint32_t(min(kb + P, KB - 1));
+            if constexpr (NVT) {
 #pragma unroll
-            for (int f = 0; f < 4; ++f) W16<F>::load(w[s][f], lrow[f], kw * 64u + wcol);
+              for (int j = 0; j < 2; ++j) { nvc[s][j] = load16(ncod[j] + kw * 32u); nvs[s][j] = nv_scale4(nscl[j] + kw * 4u); }
+            } else {
+#pragma unroll
+              for (int f = 0; f < 4; ++f) W16<F>::load(w[s][f], lrow[f], kw * 64u + wcol);
+            }
           }
         }
       }
