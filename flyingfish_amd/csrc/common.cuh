@@ -242,6 +242,55 @@ __device__ __forceinline__ T load_global(const void* p) {
   return *(const FF_GLOBAL T*)(p);
 }
 __device__ __forceinline__ u32x4 load16(const void* p) { return load_global<u32x4>(p); }
+// A copy of a loaded value that is known to have arrived. The compiler waits for a load where its result is first
+// read; inside a loop it repeats that wait in every iteration when the load was issued before the loop, and because
+// loads retire in order such a wait also drains every younger load in flight. Reading the value once through this
+// copy before the loop keeps the loop free of it.
+// Loads whose waits are placed by hand. The compiler sees an ordinary instruction that defines its result at once, so
+// it places no wait of its own; the caller counts the loads it has issued since (they retire in issue order) and names
+// that count in wait_loads<N>() before the first read. The registers go through the wait as in/out operands, which
+// keeps every read of them behind it. A register that still has such a load in flight must not be left dead (the
+// compiler would reuse it): drain with wait_loads<0>() over all of them before they go out of use.
+__device__ __forceinline__ void load16_async(u32x4& d, const void* p) {
+  asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(d) : "v"(p));
+}
+// The same with a wave-uniform 64-bit base in scalar registers and a 32-bit byte offset per lane: no 64-bit address
+// arithmetic and no address registers per load on the vector side.
+__device__ __forceinline__ void load16_async(u32x4& d, uint64_t base, uint32_t offset) {
+  asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(d) : "v"(offset), "s"(base));
+}
+__device__ __forceinline__ void load4_async(float& d, const void* p) {
+  asm volatile("global_load_dword %0, %1, off" : "=v"(d) : "v"(p));
+}
+template <int N>
+__device__ __forceinline__ void wait_loads(u32x4& a, u32x4& b, u32x4& c, u32x4& d, u32x4& e, u32x4& f, u32x4& g, u32x4& h) {
+  asm volatile("s_waitcnt vmcnt(%8)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d), "+v"(e), "+v"(f), "+v"(g), "+v"(h) : "n"(N));
+}
+template <int N>
+__device__ __forceinline__ void wait_loads(u32x4& a) {
+  asm volatile("s_waitcnt vmcnt(%1)" : "+v"(a) : "n"(N));
+}
+template <int N>
+__device__ __forceinline__ void wait_loads(u32x4& a, u32x4& b) {
+  asm volatile("s_waitcnt vmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N));
+}
+template <int N>
+__device__ __forceinline__ void wait_loads(u32x4& a, float& b) {
+  asm volatile("s_waitcnt vmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N));
+}
+template <int N>
+__device__ __forceinline__ void wait_loads(u32x4& a, u32x4& b, float& c) {
+  asm volatile("s_waitcnt vmcnt(%3)" : "+v"(a), "+v"(b), "+v"(c) : "n"(N));
+}
+template <int N>
+__device__ __forceinline__ void wait_loads(u32x4& a, u32x4& b, u32x4& c, u32x4& d, float& e) {
+  asm volatile("s_waitcnt vmcnt(%5)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d), "+v"(e) : "n"(N));
+}
+__device__ __forceinline__ float landed(float v) {
+  float r;
+  asm volatile("v_mov_b32 %0, %1" : "=v"(r) : "v"(v));
+  return r;
+}
 // f(std::integral_constant<int, 0>{}) ... f(std::integral_constant<int, N - 1>{}): a loop whose index is a constant
 // expression in the body (register arrays indexed by it stay in registers)
 template <int N, int I = 0, class Fn>

@@ -54,6 +54,8 @@ __global__ __launch_bounds__(256, MF <= 4 ? 2 : 1) void k_w8a8_grouped(const Gem
   constexpr int CHUNKS = TM * 8;                    // 16-byte token chunks per K block
   constexpr int CPT = (CHUNKS + 255) / 256;         // chunks a thread moves per K block
   constexpr int TILE = TM * 128 + TM * 4;           // codes + scales
+  constexpr int LPS = CPT + 1 + 8;                  // loads a thread issues per stage: token chunks, token scale, weights
+  static_assert(CPT == 1 || CPT == 2 || CPT == 4, "token chunks per thread");
   __shared__ __attribute__((aligned(16))) uint8_t tile[2][TILE];
   // Weight fragments are requested row-contiguously (8 lanes per 128-byte row segment, 8 rows per instruction) and
   // turned into the operand's lane order (row lane % 16, bytes 32 (lane / 16) .. + 31) through this wave-private
@@ -63,6 +65,7 @@ __global__ __launch_bounds__(256, MF <= 4 ? 2 : 1) void k_w8a8_grouped(const Gem
   // so no wait sits between the writes and the reads.
   // Short groups (MF < 4) are bound by HBM, not by the L1: they keep the direct requests and skip the LDS round trip.
   constexpr bool TW = MF >= 4;
+  static_assert(!TW || P == 2, "the hand-counted waits of the long-group path assume two weight stages");
   __shared__ __attribute__((aligned(16))) uint8_t wstage[TW ? 4 : 1][TW ? 4 : 1][TW ? 2048 : 16];  // [wave][fragment][16 rows x 128 B]
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = uni(tid >> 6);
@@ -114,16 +117,19 @@ __global__ __launch_bounds__(256, MF <= 4 ? 2 : 1) void k_w8a8_grouped(const Gem
     }
     // first output column of fragment f; fragments past N are clamped onto the last 16 rows and dropped at the store
     int col0[4];
-    const uint8_t* wrow[4];
+    // weight addresses: a wave-uniform base per fragment (scalar registers) and one byte offset per lane
+    uint64_t wfrag[4];
 #pragma unroll
     for (int f = 0; f < 4; ++f) {
       col0[f] = MODE == 0 ? t * 128 + wave * 32 + (f & 1) * 16 : t * 256 + wave * 64 + f * 16;
       const int base = min(col0[f], N - 16);
       const uint64_t codes = MODE == 0 ? wc[f >> 1] : wc[0];
-      wrow[f] = TW ? reinterpret_cast<const uint8_t*>(codes) + size_t(base + (lane >> 3)) * K + (lane & 7) * 16  // rows 0..7 of the fragment
-                   : reinterpret_cast<const uint8_t*>(codes) + size_t(base + (lane & 15)) * K + (lane >> 4) * 32;
+      wfrag[f] = uni64(codes + uint64_t(base) * uint64_t(K));
     }
-    const uint32_t wsecond = TW ? 8u * uint32_t(K) : 16u;  // second request of a fragment: rows 8..15, or the lane's next 16 bytes
+    // long groups: 8 lanes per 128-byte row segment, rows 0..7 of the fragment (rows 8..15 with the second request);
+    // short groups: operand order, 32 bytes of row lane % 16 as two requests
+    const uint32_t woff0 = TW ? uint32_t(lane >> 3) * uint32_t(K) + uint32_t(lane & 7) * 16u : uint32_t(lane & 15) * uint32_t(K) + uint32_t(lane >> 4) * 32u;
+    const uint32_t woff1 = woff0 + (TW ? 8u * uint32_t(K) : 16u);
     // block-scale rows: one per wave (its fragments sit inside one 128-row block), lane l keeps K block l (+64)
     const int srow = min(MODE == 0 ? t * 128 + wave * 32 : t * 256 + wave * 64, N - 16) >> 7;
     const float* sw0 = reinterpret_cast<const float*>(ws[0]) + size_t(srow) * KB;
@@ -157,22 +163,49 @@ __global__ __launch_bounds__(256, MF <= 4 ? 2 : 1) void k_w8a8_grouped(const Gem
 #pragma unroll
         for (int r = 0; r < 4; ++r) acc[m][f][r] = 0.0f;
 
-    // prologue: weight fragments of the first P K blocks, token tile 0 into LDS, token tile 1 into registers.
-    // Loads retire in issue order, so anything consumed early must be requested before anything consumed late: in
-    // steady state an iteration first requests token tile kb+2 (written to LDS one iteration later) and then the
-    // weight fragments of K block kb+P, so waiting for the tokens never forces the younger weight loads to land.
+    // block scales of K blocks 0 .. 63, one per lane. They are requested before everything else and made to land
+    // (landed()) outside the K loop: a value still counted as in flight when the loop is entered makes the compiler
+    // wait for it in every iteration, and since loads retire in order that wait drains the whole prefetch queue.
+    float swn0 = load_global<float>(sw0 + min(lane, KB - 1));
+    float swn1 = MODE == 0 ? load_global<float>(sw1 + min(lane, KB - 1)) : 0.0f;
+
+    // Loads inside the K loop are issued and awaited by hand (load16_async / wait_loads): the compiler's own waits are
+    // placed for the path with the fewest loads in flight and drain the queue in every iteration. Per stage a thread
+    // issues LPS loads in a fixed order, so "how many younger loads may still be in flight" is a constant:
+    //   64-row groups and longer (TW), stage kb with register slot s = kb % 2: the operand-order fragments of K block
+    //     kb are read from the wave's transposition buffer; then, spread over the matrix instructions of the row
+    //     fragments (an issue that finds the memory or LDS pipeline full stalls under matrix work of the same
+    //     wave): token tile kb+1 (published at the end of this stage), the weights of K block kb+2 into slot s,
+    //     and slot s^1 (K block kb+1, requested one stage ago) written row-contiguously into the transposition
+    //     buffer for the next stage;
+    //   shorter groups: after the barrier token tile kb+2, then the weights of K block kb+P.
+    // Either way the token tile published in a stage has exactly the eight weight loads issued after it behind it.
+    constexpr int WAIT_W = (P - 1) * LPS;  // short groups: younger loads behind a stage's weights
+    // prologue: weight fragments of the first P K blocks, token tile 0 into LDS, everything landed, then token tile 1
+    // (and for short groups the last weight stage once more, so that tile 1 too has eight loads behind it).
     u32x4 w[P][4][2];
+#define FF_REQUEST_WEIGHTS(s_, kb_, f_)                                   \
+  do {                                                                     \
+    load16_async(w[s_][f_][0], wfrag[f_] + (kb_) * 128u, woff0);           \
+    load16_async(w[s_][f_][1], wfrag[f_] + (kb_) * 128u, woff1);           \
+  } while (0)
+#define FF_DRAIN_WEIGHTS()                                                                                                  \
+  _Pragma("unroll") for (int s_ = 0; s_ < P; ++s_)                                                                          \
+      wait_loads<0>(w[s_][0][0], w[s_][0][1], w[s_][1][0], w[s_][1][1], w[s_][2][0], w[s_][2][1], w[s_][3][0], w[s_][3][1])
 #pragma unroll
     for (int s = 0; s < P; ++s) {
       const uint32_t kb = uint32_t(min(s, KB - 1));
 #pragma unroll
-      for (int f = 0; f < 4; ++f) {
-        w[s][f][0] = load16(wrow[f] + kb * 128u);
-        w[s][f][1] = load16(wrow[f] + kb * 128u + wsecond);
-      }
+      for (int f = 0; f < 4; ++f) FF_REQUEST_WEIGHTS(s, kb, f);
     }
     u32x4 tv[CPT];
     float tsv;
+#define FF_WAIT_TOKENS(n_)                                                    \
+  do {                                                                         \
+    if constexpr (CPT == 1) wait_loads<n_>(tv[0], tsv);                        \
+    else if constexpr (CPT == 2) wait_loads<n_>(tv[0], tv[1], tsv);            \
+    else wait_loads<n_>(tv[0], tv[1], tv[2], tv[3], tsv);                      \
+  } while (0)
     {
 #pragma unroll
       for (int i = 0; i < CPT; ++i) {
@@ -180,52 +213,67 @@ __global__ __launch_bounds__(256, MF <= 4 ? 2 : 1) void k_w8a8_grouped(const Gem
         if (stage_chunk) *reinterpret_cast<u32x4*>(&tile[0][tdst[i]]) = v;
       }
       if (tid < TM) *reinterpret_cast<float*>(&tile[0][TM * 128 + tid * 4]) = load_global<float>(ssrc);
-      const uint32_t k1 = uint32_t(min(1, KB - 1));
+      FF_DRAIN_WEIGHTS();
+      if constexpr (TW) {
+        // K block 0 goes into the wave's transposition buffer; stage 0 requests token tile 1 itself
+        uint8_t* wl = &wstage[wave][0][0];
 #pragma unroll
-      for (int i = 0; i < CPT; ++i) tv[i] = load16(tsrc[i] + k1 * 128u);
-      tsv = load_global<float>(ssrc + k1);
+        for (int f = 0; f < 4; ++f) {
+          *reinterpret_cast<u32x4*>(wl + f * 2048 + wr_off) = w[0][f][0];
+          *reinterpret_cast<u32x4*>(wl + f * 2048 + 1024 + wr_off) = w[0][f][1];
+        }
+#pragma unroll
+        for (int i = 0; i < CPT; ++i) tv[i] = u32x4{0u, 0u, 0u, 0u};
+        tsv = 0.0f;
+      } else {
+        const uint32_t k1 = uint32_t(min(1, KB - 1));
+#pragma unroll
+        for (int i = 0; i < CPT; ++i) load16_async(tv[i], tsrc[i] + k1 * 128u);
+        load4_async(tsv, ssrc + k1);
+        const uint32_t kb = uint32_t(min(P - 1, KB - 1));
+#pragma unroll
+        for (int f = 0; f < 4; ++f) FF_REQUEST_WEIGHTS(P - 1, kb, f);
+      }
     }
     __syncthreads();
 
     // LDS addresses of this lane's token fragment pieces (buffer 0)
-    int tlo[MF], thi[MF], tsx[MF];
-#pragma unroll
-    for (int m = 0; m < MF; ++m) {
-      const int trow = 16 * m + (lane & 15);
-      const int q2 = (lane >> 4) * 2;
-      tlo[m] = trow * 128 + (((q2) ^ (trow & 7)) << 4);
-      thi[m] = trow * 128 + (((q2 + 1) ^ (trow & 7)) << 4);
-      tsx[m] = TM * 128 + trow * 4;
-    }
+    // Row fragment m sits 2048 bytes (scales: 64 bytes) behind fragment 0 and keeps its swizzle key (16 m leaves the low
+    // row bits alone), and K block kb sits in buffer kb % 2 = stage % 2 (P is even and the loop advances by P): every
+    // token address is one of three lane values plus a compile-time constant.
+    static_assert(P % 2 == 0, "token buffer = stage parity");
+    const int trow0 = lane & 15, q2 = (lane >> 4) * 2;
+    const int tlo0 = trow0 * 128 + (((q2) ^ (trow0 & 7)) << 4);
+    const int thi0 = trow0 * 128 + (((q2 + 1) ^ (trow0 & 7)) << 4);
+    const int tsx0 = TM * 128 + trow0 * 4;
 
     for (int kb0 = 0; kb0 < KB; kb0 += 64) {
-      // block scales of K blocks kb0 .. kb0+63, one per lane
-      const int kl = min(kb0 + lane, KB - 1);
-      const float swl0 = load_global<float>(sw0 + kl);
-      const float swl1 = MODE == 0 ? load_global<float>(sw1 + kl) : 0.0f;
+      // block scales of K blocks kb0 .. kb0+63, one per lane; the next 64 are requested right away
+      const float swl0 = landed(swn0);
+      const float swl1 = MODE == 0 ? landed(swn1) : 0.0f;
+      if (kb0 + 64 < KB) {
+        const int kl = min(kb0 + 64 + lane, KB - 1);
+        swn0 = load_global<float>(sw0 + kl);
+        if (MODE == 0) swn1 = load_global<float>(sw1 + kl);
+      }
       const int kend = min(KB, kb0 + 64);
       for (int kbo = kb0; kbo < kend; kbo += P) {
 #pragma unroll
         for (int s = 0; s < P; ++s) {
           const int kb = kbo + s;
           if (kb < kend) {
-            const uint8_t* tb = tile[kb & 1];
+            const uint8_t* tb = tile[s & 1];
             const float s0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, swl0), kb - kb0));
             const float s1 = MODE == 0 ? __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, swl1), kb - kb0)) : s0;
             // every row fragment is computed, also the padding of a short group: straight-line code lets the matrix
             // core overlap with the scale fmas, and short groups are bandwidth-bound anyway
             u32x4 wt[4][2];  // the four fragments in operand order
+            uint8_t* wl = &wstage[TW ? wave : 0][0][0];
             if constexpr (!TW) {
+              wait_loads<WAIT_W>(w[s][0][0], w[s][0][1], w[s][1][0], w[s][1][1], w[s][2][0], w[s][2][1], w[s][3][0], w[s][3][1]);
 #pragma unroll
               for (int f = 0; f < 4; ++f) { wt[f][0] = w[s][f][0]; wt[f][1] = w[s][f][1]; }
             } else {
-              uint8_t* wl = &wstage[wave][0][0];
-#pragma unroll
-              for (int f = 0; f < 4; ++f) {
-                *reinterpret_cast<u32x4*>(wl + f * 2048 + wr_off) = w[s][f][0];
-                *reinterpret_cast<u32x4*>(wl + f * 2048 + 1024 + wr_off) = w[s][f][1];
-              }
-              __builtin_amdgcn_wave_barrier();
 #pragma unroll
               for (int f = 0; f < 4; ++f) {
                 wt[f][0] = *reinterpret_cast<const u32x4*>(wl + f * 2048 + rd_lo);
@@ -233,53 +281,92 @@ __global__ __launch_bounds__(256, MF <= 4 ? 2 : 1) void k_w8a8_grouped(const Gem
               }
               __builtin_amdgcn_wave_barrier();
             }
-            v4f pr[MF][4];
-            float sc[MF][2];
+            // Row fragment m's products are folded into the totals while fragment m + 1 is in the matrix core, so two
+            // fragments' worth of product registers are live instead of MF (the scheduling fences keep that order).
+            v4f pr[2][4];
+            float sc[2][2];
 #pragma unroll
-            for (int m = 0; m < MF; ++m) {
-              const u32x4 lo = *reinterpret_cast<const u32x4*>(tb + tlo[m]);
-              const u32x4 hi = *reinterpret_cast<const u32x4*>(tb + thi[m]);
-              const float sx = *reinterpret_cast<const float*>(tb + tsx[m]);
-              const v8i tok = {int(lo[0]), int(lo[1]), int(lo[2]), int(lo[3]), int(hi[0]), int(hi[1]), int(hi[2]), int(hi[3])};
-              sc[m][0] = __fmul_rn(s0, sx);
-              sc[m][1] = __fmul_rn(s1, sx);
+            for (int m = 0; m <= MF; ++m) {
+              if (m < MF) {
+                const u32x4 lo = *reinterpret_cast<const u32x4*>(tb + tlo0 + m * 2048);
+                const u32x4 hi = *reinterpret_cast<const u32x4*>(tb + thi0 + m * 2048);
+                const float sx = *reinterpret_cast<const float*>(tb + tsx0 + m * 64);
+                const v8i tok = {int(lo[0]), int(lo[1]), int(lo[2]), int(lo[3]), int(hi[0]), int(hi[1]), int(hi[2]), int(hi[3])};
+                sc[m & 1][0] = __fmul_rn(s0, sx);
+                sc[m & 1][1] = __fmul_rn(s1, sx);
 #pragma unroll
-              for (int f = 0; f < 4; ++f) {
-                const v8i wf = {int(wt[f][0][0]), int(wt[f][0][1]), int(wt[f][0][2]), int(wt[f][0][3]),
-                                int(wt[f][1][0]), int(wt[f][1][1]), int(wt[f][1][2]), int(wt[f][1][3])};
-                const v4f z = {0.0f, 0.0f, 0.0f, 0.0f};
-                pr[m][f] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, tok, z, 0, 0, 0, 0, 0, 0);
+                for (int f = 0; f < 4; ++f) {
+                  const v8i wf = {int(wt[f][0][0]), int(wt[f][0][1]), int(wt[f][0][2]), int(wt[f][0][3]),
+                                  int(wt[f][1][0]), int(wt[f][1][1]), int(wt[f][1][2]), int(wt[f][1][3])};
+                  const v4f z = {0.0f, 0.0f, 0.0f, 0.0f};
+                  pr[m & 1][f] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, tok, z, 0, 0, 0, 0, 0, 0);
+                }
+                if constexpr (TW) {
+                  const int o = s ^ 1;
+                  if (m == 0) {  // token tile kb+1
+                    const uint32_t kn = uint32_t(min(kb + 1, KB - 1));
+#pragma unroll
+                    for (int i = 0; i < CPT; ++i) load16_async(tv[i], tsrc[i] + kn * 128u);
+                    load4_async(tsv, ssrc + kn);
+                  }
+                  // slot s went into the transposition buffer one stage ago: request K block kb+2 into it. A piece
+                  // of slot s^1 (K block kb+1) has the rest of its own stage's weight loads, this stage's token
+                  // loads and this stage's weight loads so far behind it: CPT + 1 + 8 whichever piece it is
+                  const uint32_t kw = uint32_t(min(kb + 2, KB - 1));
+                  if constexpr (MF == 4) {
+                    FF_REQUEST_WEIGHTS(s, kw, m);
+                    wait_loads<CPT + 1 + 8>(w[o][m][0], w[o][m][1]);
+                    *reinterpret_cast<u32x4*>(wl + m * 2048 + wr_off) = w[o][m][0];
+                    *reinterpret_cast<u32x4*>(wl + m * 2048 + 1024 + wr_off) = w[o][m][1];
+                  } else {
+                    if (m & 1) load16_async(w[s][m >> 1][1], wfrag[m >> 1] + kw * 128u, woff1);
+                    else load16_async(w[s][m >> 1][0], wfrag[m >> 1] + kw * 128u, woff0);
+                    wait_loads<CPT + 1 + 8>(w[o][m >> 1][m & 1]);
+                    *reinterpret_cast<u32x4*>(wl + (m >> 1) * 2048 + (m & 1) * 1024 + wr_off) = w[o][m >> 1][m & 1];
+                  }
+                }
               }
+              if (m > 0) {
+#pragma unroll
+                for (int f = 0; f < 4; ++f)
+#pragma unroll
+                  for (int r = 0; r < 4; ++r)
+                    acc[m - 1][f][r] = __fmaf_rn(pr[(m - 1) & 1][f][r], sc[(m - 1) & 1][(MODE == 0 && f >= 2) ? 1 : 0], acc[m - 1][f][r]);
+              }
+              if constexpr (TW) __builtin_amdgcn_sched_barrier(0);
             }
-#pragma unroll
-            for (int m = 0; m < MF; ++m)
-#pragma unroll
-              for (int f = 0; f < 4; ++f)
-#pragma unroll
-                for (int r = 0; r < 4; ++r) acc[m][f][r] = __fmaf_rn(pr[m][f][r], sc[m][(MODE == 0 && f >= 2) ? 1 : 0], acc[m][f][r]);
-            // publish token tile kb+1 (requested one iteration ago)
+            // publish token tile kb+1
+            FF_WAIT_TOKENS(8);
 #pragma unroll
             for (int i = 0; i < CPT; ++i)
-              if (stage_chunk) *reinterpret_cast<u32x4*>(&tile[(kb & 1) ^ 1][tdst[i]]) = tv[i];
-            if (tid < TM) *reinterpret_cast<float*>(&tile[(kb & 1) ^ 1][TM * 128 + tid * 4]) = tsv;
+              if (stage_chunk) *reinterpret_cast<u32x4*>(&tile[(s & 1) ^ 1][tdst[i]]) = tv[i];
+            if (tid < TM) *reinterpret_cast<float*>(&tile[(s & 1) ^ 1][TM * 128 + tid * 4]) = tsv;
             __syncthreads();
-            // request token tile kb+2, then K block kb+P of the weights into the slot just consumed
-            {
-              const uint32_t kn = uint32_t(min(kb + 2, KB - 1));
+          } else {
+            // a stage past the last K block: its registers still have (clamped) loads in flight and are about to be
+            // requested into again; a register with a load in flight is never left unread
+            wait_loads<0>(w[s][0][0], w[s][0][1], w[s][1][0], w[s][1][1], w[s][2][0], w[s][2][1], w[s][3][0], w[s][3][1]);
+            FF_WAIT_TOKENS(0);
+          }
+          // Short groups: request token tile kb+2 and K block kb+P of the weights into the slot just consumed. The
+          // requests are made also when the stage itself is past the last K block (clamped addresses), so that the
+          // number of loads per stage does not depend on the path.
+          if constexpr (!TW) {
+            const uint32_t kn = uint32_t(min(kb + 2, KB - 1));
 #pragma unroll
-              for (int i = 0; i < CPT; ++i) tv[i] = load16(tsrc[i] + kn * 128u);
-              tsv = load_global<float>(ssrc + kn);
-              const uint32_t kw = uint32_t(min(kb + P, KB - 1));
+            for (int i = 0; i < CPT; ++i) load16_async(tv[i], tsrc[i] + kn * 128u);
+            load4_async(tsv, ssrc + kn);
+            const uint32_t kw = uint32_t(min(kb + P, KB - 1));
 #pragma unroll
-              for (int f = 0; f < 4; ++f) {
-                w[s][f][0] = load16(wrow[f] + kw * 128u);
-                w[s][f][1] = load16(wrow[f] + kw * 128u + wsecond);
-              }
-            }
+            for (int f = 0; f < 4; ++f) FF_REQUEST_WEIGHTS(s, kw, f);
           }
         }
       }
     }
+
+    // The last stages have requested (clamped) data nobody reads: let it land before the registers are reused.
+    FF_DRAIN_WEIGHTS();
+    FF_WAIT_TOKENS(0);
 
     // epilogue
     const int tk = lane & 15, sub = (lane >> 4) * 4;
@@ -332,5 +419,9 @@ __global__ __launch_bounds__(256, MF <= 4 ? 2 : 1) void k_w8a8_grouped(const Gem
     }
   }
 }
+
+#undef FF_REQUEST_WEIGHTS
+#undef FF_DRAIN_WEIGHTS
+#undef FF_WAIT_TOKENS
 
 }  // namespace ffmoe
