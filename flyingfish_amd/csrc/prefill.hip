@@ -191,8 +191,12 @@ int num_cus_p() {
 inline uint64_t up256(uint64_t v) { return (v + 255) & ~uint64_t(255); }
 
 // rows per group for an average of `avg` rows per expert
-int pick_mf(double avg) {
-  if (const char* f = getenv("FFMOE_PREFILL_MF")) return atoi(f);
+// (cap: the largest group a path's kernels are built for, in units of 16 rows; anything else in the variable is ignored)
+int pick_mf(double avg, int cap) {
+  if (const char* f = getenv("FFMOE_PREFILL_MF")) {
+    const int v = atoi(f);
+    if (v == 1 || v == 2 || v == 4 || v == 8) return std::min(v, cap);
+  }
   return avg > 24.0 ? 4 : avg > 12.0 ? 2 : 1;
 }
 
@@ -390,7 +394,7 @@ int prefill_impl(const ffmoe_expert_table* table, const ffmoe_prefill* args, int
   uint8_t* s = (uint8_t*)args->scratch;
   PrefillBook b{(uint32_t*)(s + l.counts), (uint32_t*)(s + l.offsets), (uint32_t*)(s + l.gbase), (uint32_t*)(s + l.totals),
                 (int*)(s + l.perm), (GemmGroup*)(s + l.groups), (u32x2*)(s + l.units0), (u32x2*)(s + l.units1)};
-  const int mf = pick_mf(double(A) / E);
+  const int mf = pick_mf(double(A) / E, (mx || a16) ? 4 : 8);
   const int tm = 16 * mf;
   const int tiles0 = (I + 127) / 128, tiles1 = (H + 255) / 256;
 

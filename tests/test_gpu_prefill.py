@@ -288,6 +288,31 @@ def test_prefill_rows_do_not_depend_on_their_cohort():
         assert np.array_equal(got, ref[lo:lo + n]), "rows %d..%d differ between cohorts" % (lo, lo + n)
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("act_mode", [capi.ACT_FP8_BLOCK128, capi.ACT_BF16])
+def test_prefill_grouping_switches_leave_every_bit_alone(act_mode, monkeypatch):
+    """Rows per group (FFMOE_PREFILL_MF) and the order of the unit list (FFMOE_PREFILL_RGB) decide which block computes
+    what, not what is computed: every setting gives the default run's contributions bit for bit. 700 rows over 6 skewed
+    experts give groups of every length and experts with more row groups than the smallest blockings hold; a group
+    size a path has no kernel for (8 on the BF16 matrix cores) falls back to its largest, an unknown value is ignored."""
+    rows, top_k, experts, hidden, inter = 700, 3, 6, 512, 384
+    table, _ = _make_fp8_table(experts, hidden, inter, 19)
+    ids, w = _routing(rows, top_k, experts, 43, 1.3)
+    x = synth.normal((rows, hidden), 1.0, 44, dtype=torch.bfloat16).cuda()
+    ids_d, w_d = torch.from_numpy(ids).cuda(), torch.from_numpy(w).cuda()
+    op = ops.PrefillOps(table, rows, top_k, act_mode=act_mode)
+    monkeypatch.delenv("FFMOE_PREFILL_MF", raising=False)
+    monkeypatch.delenv("FFMOE_PREFILL_RGB", raising=False)
+    ref = bits(op.contribute(x, ids_d, w_d)).copy()
+    assert np.any(ref != 0)
+    for mf, rgb in [("1", "1"), ("1", "5"), ("2", "3"), ("4", "2"), ("4", "1000000"), ("8", "1"), ("8", "4"), ("3", "0"), ("4", "32")]:
+        monkeypatch.setenv("FFMOE_PREFILL_MF", mf)
+        monkeypatch.setenv("FFMOE_PREFILL_RGB", rgb)
+        op.contributions.zero_()
+        got = bits(op.contribute(x, ids_d, w_d))
+        assert np.array_equal(got, ref), "FFMOE_PREFILL_MF=%s FFMOE_PREFILL_RGB=%s changes the result" % (mf, rgb)
+
+
 def test_prefill_then_combine_layer():
     """contribute -> ordered combine equals the oracle's combine over the oracle's contributions within BF16 noise."""
     rows, top_k, experts, hidden, inter = 32, 4, 8, 256, 128
