@@ -4,6 +4,7 @@
 
 #define FFMOE_DECODE_RG 8              /* rows of one expert served by one pass over its weights */
 #define FFMOE_DECODE_MAX_ASSIGN 4096   /* rows * top_k handled by the single-block grouping kernel */
+#define FFMOE_STATIC_SCRATCH_BYTES (8ull << 20)  /* built-in arena of ffmoe_decode_contribute_static, per GPU */
 
 namespace ffmoe {
 

@@ -313,6 +313,52 @@ extern "C" __attribute__((visibility("default"))) int ffmoe_decode_contribute(co
   return decode_dispatch(table, shared, args, 3, stream);
 }
 
+// ---------------------------------------------------------------------------------------------
+// The same call for callers that cannot allocate (HIP graph capture, serving loops that forbid hipMalloc): the
+// scratch arena is a fixed array in device memory instead of a caller buffer. Every GPU holds its own copy of the
+// array at its own address, looked up once per device with that device current. Nothing in the arena has to start
+// at zero: the grouping kernel writes descriptors and counters before any reader, and the gate/up launch writes every
+// activation row the down launch reads. Calls on one GPU share the array, so calls that overlap in time race.
+static __device__ __align__(256) unsigned char g_static_scratch[FFMOE_STATIC_SCRATCH_BYTES];
+
+static int static_scratch(void** out) {
+  static std::atomic<void*> base[64];
+  int dev = 0;
+  const hipError_t de = hipGetDevice(&dev);
+  if (de != hipSuccess) return ff_fail(int(de), "hipGetDevice failed: %s", hipGetErrorString(de));
+  FF_REQUIRE(dev >= 0 && dev < 64, FFMOE_ERR_UNSUPPORTED, "device ordinal %d is outside the per-device table", dev);
+  void* b = base[dev].load(std::memory_order_acquire);
+  if (!b) {
+    const hipError_t se = hipGetSymbolAddress(&b, HIP_SYMBOL(g_static_scratch));
+    if (se != hipSuccess || !b) {
+      (void)hipGetLastError();
+      return ff_fail(se != hipSuccess ? int(se) : FFMOE_ERR_NULL, "hipGetSymbolAddress(static scratch) failed: %s", hipGetErrorString(se));
+    }
+    base[dev].store(b, std::memory_order_release);
+  }
+  *out = b;
+  return 0;
+}
+
+extern "C" __attribute__((visibility("default"))) uint64_t ffmoe_decode_static_scratch_bytes(void) { return FFMOE_STATIC_SCRATCH_BYTES; }
+
+extern "C" __attribute__((visibility("default"))) int ffmoe_decode_contribute_static(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared,
+                                                                                    const ffmoe_decode* args, void* stream) {
+  FF_REQUIRE(table && args, FFMOE_ERR_NULL, "table/args is NULL");
+  const uint64_t need = ffmoe_decode_scratch_bytes(args->rows, args->top_k > 0 ? args->top_k : 1, table->experts, table->hidden, table->inter,
+                                                   shared ? shared->inter : 0);
+  FF_REQUIRE(need != 0, FFMOE_ERR_SHAPE, "decode rows=%d top_k=%d experts=%d out of range", args->rows, args->top_k, table->experts);
+  FF_REQUIRE(need <= FFMOE_STATIC_SCRATCH_BYTES, FFMOE_ERR_SCRATCH,
+             "this shape needs %llu bytes of scratch, the built-in arena holds %llu: use ffmoe_decode_contribute with a caller arena",
+             (unsigned long long)need, (unsigned long long)FFMOE_STATIC_SCRATCH_BYTES);
+  void* arena = nullptr;
+  FF_TRY(static_scratch(&arena));
+  ffmoe_decode own = *args;
+  own.scratch = arena;
+  own.scratch_bytes = FFMOE_STATIC_SCRATCH_BYTES;
+  return decode_dispatch(table, shared, &own, 3, stream);
+}
+
 extern "C" __attribute__((visibility("default"))) int ffmoe_decode_contribute_stage(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared,
                                              const ffmoe_decode* args, int stage, void* stream) {
   FF_REQUIRE(stage == 0 || stage == 1, FFMOE_ERR_SHAPE, "decode stage %d is neither 0 (gate/up) nor 1 (down)", stage);

@@ -282,6 +282,18 @@ class DecodeOps:
             capi.check(capi.lib().ffmoe_decode_contribute_stage(ctypes.byref(self._table_c), sh, ctypes.byref(d), stage, _stream()))
         return self.contributions, self.shared_out
 
+    def contribute_static(self, x, ids, weights, active=None):
+        """contribute() through ffmoe_decode_contribute_static: the library's built-in per-GPU arena replaces
+        self.scratch (for callers that cannot allocate); results are bit-identical to contribute()."""
+        act_mode, swiglu, limit, rw, wf32 = self.cfg
+        d = capi.Decode(self.rows, self.top_k, act_mode, swiglu, limit, rw, wf32,
+                        x.data_ptr(), ids.data_ptr(), active.data_ptr() if active is not None else None, weights.data_ptr(),
+                        self.contributions.data_ptr(), self.shared_out.data_ptr() if self.shared_out is not None else None,
+                        self.done.data_ptr(), None, 0, None)
+        sh = ctypes.byref(self._shared_c) if self._shared_c is not None else None
+        capi.check(capi.lib().ffmoe_decode_contribute_static(ctypes.byref(self._table_c), sh, ctypes.byref(d), _stream()))
+        return self.contributions, self.shared_out
+
     def contribute_from_logits(self, x, logits, bias, ids, weights, score_mode=capi.NOAUX_SIGMOID, routed_scaling=1.0, n_group=1, topk_group=1):
         """One token: top-k selection inside the gate/up launch; ids / weights (f32) are written. Returns None when the
         shape is outside the fast path (nothing launched)."""

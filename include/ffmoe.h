@@ -194,6 +194,19 @@ uint64_t ffmoe_decode_scratch_bytes(int rows, int top_k, int experts, int hidden
 int ffmoe_decode_contribute(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared,
                             const ffmoe_decode* args, void* stream);
 
+/* ffmoe_decode_contribute for callers that cannot allocate device memory or hand over a scratch arena (code under HIP
+ * graph capture, serving loops and harnesses that forbid hipMalloc). No counterpart in the reference. args->scratch and
+ * args->scratch_bytes are ignored: the arena is a fixed array of ffmoe_decode_static_scratch_bytes() bytes (8 MiB) in
+ * the library's device image, one copy per GPU, held until the process ends. Everything else (arguments, arithmetic,
+ * outputs, errors) is ffmoe_decode_contribute's, and the results are bit-identical to it. A shape whose
+ * ffmoe_decode_scratch_bytes() exceeds the arena is rejected with FFMOE_ERR_SCRATCH and nothing is launched (at the
+ * DeepSeek-V3 dimensions the arena holds up to 128 rows x top-8). The call allocates nothing and clears nothing
+ * (no stage reads arena bytes that an earlier launch of the same call has not written). All calls on one GPU share
+ * that GPU's array: two calls that overlap in time on one GPU (different streams) race. */
+uint64_t ffmoe_decode_static_scratch_bytes(void);
+int ffmoe_decode_contribute_static(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared,
+                                   const ffmoe_decode* args, void* stream);
+
 /* The two launches of the contribution as separate calls, like the reference's gate_up and down launches
  * (src/backend/cuda/moe/decode.rs:486-490 and :513-517): stage 0 = gate/up + SwiGLU into scratch (and the
  * grouping of assignments by expert), stage 1 = down + routing weight from scratch. Stage 0 then stage 1 with the
