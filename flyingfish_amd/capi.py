@@ -22,7 +22,7 @@ ERR_NULL, ERR_ALIGN, ERR_SHAPE, ERR_OVERLAP, ERR_UNSUPPORTED, ERR_SCRATCH = -1, 
 EXPORTS = [
     "ffmoe_last_error", "ffmoe_version",
     "ffmoe_route_logits_bf16", "ffmoe_route_logits_f32", "ffmoe_route_topk", "ffmoe_route_topk_noaux", "ffmoe_route_noaux_decode", "ffmoe_route_decode", "ffmoe_slot_publish", "ffmoe_route_mask",
-    "ffmoe_decode_scratch_bytes", "ffmoe_decode_contribute", "ffmoe_decode_static_scratch_bytes", "ffmoe_decode_contribute_static", "ffmoe_decode_contribute_stage", "ffmoe_decode_finish", "ffmoe_decode_contribute_from_logits", "ffmoe_decode_token_layer", "ffmoe_decode_contribute_form", "ffmoe_e8m0_scratch_bytes", "ffmoe_decode_contribute_e8m0", "ffmoe_act_quant_e8m0",
+    "ffmoe_decode_scratch_bytes", "ffmoe_decode_contribute", "ffmoe_decode_static_scratch_bytes", "ffmoe_decode_contribute_static", "ffmoe_decode_contribute_stage", "ffmoe_decode_finish", "ffmoe_decode_contribute_from_logits", "ffmoe_decode_token_layer", "ffmoe_decode_token_forward", "ffmoe_decode_token_forward_stage", "ffmoe_decode_contribute_form", "ffmoe_e8m0_scratch_bytes", "ffmoe_decode_contribute_e8m0", "ffmoe_act_quant_e8m0",
     "ffmoe_quant_fp8_f32_128", "ffmoe_linear_fp8_block_w8a8", "ffmoe_linear_fp8_block", "ffmoe_linear_nvfp4",
     "ffmoe_gemm_skinny_bf16", "ffmoe_swiglu",
     "ffmoe_shared_scale", "ffmoe_combine",
@@ -103,6 +103,9 @@ def lib():
                                                           P, P, I, F, I, I, P]
         L.ffmoe_decode_token_layer.argtypes = [ctypes.POINTER(ExpertTable), ctypes.POINTER(SharedExpert), ctypes.POINTER(Decode),
                                                P, P, I, F, I, I, P, P, P, I, P]
+        L.ffmoe_decode_token_forward.argtypes = L.ffmoe_decode_token_layer.argtypes
+        L.ffmoe_decode_token_forward_stage.argtypes = [ctypes.POINTER(ExpertTable), ctypes.POINTER(SharedExpert), ctypes.POINTER(Decode),
+                                                       P, P, I, F, I, I, P, P, P, I, I, P]
         L.ffmoe_decode_contribute_form.argtypes = [ctypes.POINTER(ExpertTable), ctypes.POINTER(SharedExpert), ctypes.POINTER(Decode), I, P]
         L.ffmoe_e8m0_scratch_bytes.restype = ctypes.c_uint64
         L.ffmoe_e8m0_scratch_bytes.argtypes = [I, I, I, I, I]

@@ -413,6 +413,74 @@ extern "C" __attribute__((visibility("default"))) int ffmoe_decode_contribute_fr
   return decode_impl(table, shared, args, 3, stream, -1, 0, nullptr, &route);
 }
 
+// One token in two launches: top-k selection in the prologue of the gate/up launch (behind the shared expert's rows,
+// which need no routing), then down + routing weight + ordered combine in one launch.
+static int token_forward(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared, const ffmoe_decode* args, const float* logits,
+                         const float* bias, int score_mode, float routed_scaling, int n_group, int topk_group, const void* scale, void* y,
+                         uint32_t* status, int combine_mode, int stage_mask, void* stream) {
+  FF_REQUIRE(table && args, FFMOE_ERR_NULL, "table/args is NULL");
+  FF_REQUIRE(args->rows == 1, FFMOE_ERR_UNSUPPORTED, "ffmoe_decode_token_forward handles one token row (rows=%d)", args->rows);
+  FF_REQUIRE(args->act_mode == FFMOE_ACT_BF16, FFMOE_ERR_UNSUPPORTED, "ffmoe_decode_token_forward needs FFMOE_ACT_BF16");
+  FF_REQUIRE(!shared || (shared->format == table->format && shared->inter == table->inter), FFMOE_ERR_UNSUPPORTED,
+             "ffmoe_decode_token_forward needs the shared expert in the table's format and width");
+  FF_REQUIRE(combine_mode >= 0 && combine_mode <= FFMOE_COMBINE_ROUTED, FFMOE_ERR_UNSUPPORTED, "unknown combine mode %d", combine_mode);
+  FF_REQUIRE(shared || combine_mode == FFMOE_COMBINE_ROUTED, FFMOE_ERR_SHAPE, "combine mode %d needs a shared expert", combine_mode);
+  FF_REQUIRE(args->weights_f32 == 1 && args->active == nullptr && args->assignment_gen == nullptr, FFMOE_ERR_UNSUPPORTED,
+             "selection inside the gate/up launch writes f32 weights and takes no active mask or epochs");
+  const int E = table->experts, K = args->top_k;
+  FF_REQUIRE(E == 64 || E == 128 || E == 256 || E == 512 || E == 1024, FFMOE_ERR_UNSUPPORTED, "experts=%d is not 64 * 2^n", E);
+  FF_REQUIRE(K >= 1 && K <= 8 && K < E, FFMOE_ERR_UNSUPPORTED, "top_k=%d: the one-token finish holds up to 8 routed choices", K);
+  FF_REQUIRE(score_mode == FFMOE_NOAUX_SIGMOID || score_mode == FFMOE_NOAUX_SQRTSOFTPLUS, FFMOE_ERR_UNSUPPORTED, "unknown score mode %d", score_mode);
+  FF_REQUIRE(routed_scaling > 0.0f && routed_scaling < INFINITY, FFMOE_ERR_SHAPE, "routed_scaling=%g", (double)routed_scaling);
+  FF_REQUIRE(n_group >= 1 && topk_group >= 1 && topk_group <= n_group && E % n_group == 0, FFMOE_ERR_SHAPE, "n_group=%d topk_group=%d", n_group, topk_group);
+  if (n_group > 1) {
+    const int c = E / 64, per = E / n_group;
+    FF_REQUIRE(per % c == 0 && ((per / c) & (per / c - 1)) == 0 && topk_group * per >= K, FFMOE_ERR_UNSUPPORTED,
+               "groups of %d experts do not tile the wave, or the kept groups hold fewer than top_k experts", per);
+  }
+  // rows of the down matrix beyond two 64-lane steps are outside the finish kernel's register buffers
+  {
+    const int epl = table->format == FFMOE_FMT_NVFP4 ? 32 : (table->format == FFMOE_FMT_BF16 ? 8 : 16);
+    FF_REQUIRE((table->inter / epl + 63) / 64 <= 2, FFMOE_ERR_UNSUPPORTED, "inter=%d is beyond the one-token finish's row buffers", table->inter);
+  }
+  FF_PTR4(logits);
+  if (bias) FF_PTR4(bias);
+  FF_PTR16(y);
+  if (combine_mode == FFMOE_COMBINE_GATED) FF_PTR2(scale);
+  if (status) FF_PTR4(status);
+  FF_NO_OVERLAP(y, size_t(table->hidden) * 2, args->scratch, args->scratch_bytes);
+  FF_NO_OVERLAP(y, size_t(table->hidden) * 2, args->x, size_t(table->hidden) * 2);
+  // the shared expert takes part only in the modes that add it
+  const ffmoe_shared_expert* sh = combine_mode == FFMOE_COMBINE_ROUTED ? nullptr : shared;
+  if (stage_mask & 1) {
+    const RouteInline route{logits, bias, score_mode, n_group, topk_group, routed_scaling};
+    FF_TRY(decode_impl(table, sh, args, 1, stream, -1, 0, nullptr, &route));
+  }
+  if (stage_mask & 2) {
+    FinishParams fin{};
+    fin.scale = (const uint16_t*)scale; fin.y = (uint16_t*)y; fin.status = status; fin.mode = combine_mode;
+    FF_TRY(decode_impl(table, sh, args, 0, stream, -1, 0, &fin));
+  }
+  return 0;
+}
+
+extern "C" __attribute__((visibility("default"))) int ffmoe_decode_token_forward(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared,
+                                                                                const ffmoe_decode* args, const float* logits, const float* bias,
+                                                                                int score_mode, float routed_scaling, int n_group, int topk_group,
+                                                                                const void* scale, void* y, uint32_t* status, int combine_mode,
+                                                                                void* stream) {
+  return token_forward(table, shared, args, logits, bias, score_mode, routed_scaling, n_group, topk_group, scale, y, status, combine_mode, 3, stream);
+}
+
+extern "C" __attribute__((visibility("default"))) int ffmoe_decode_token_forward_stage(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared,
+                                                                                      const ffmoe_decode* args, const float* logits, const float* bias,
+                                                                                      int score_mode, float routed_scaling, int n_group, int topk_group,
+                                                                                      const void* scale, void* y, uint32_t* status, int combine_mode,
+                                                                                      int stage, void* stream) {
+  FF_REQUIRE(stage == 0 || stage == 1, FFMOE_ERR_SHAPE, "token forward stage %d is neither 0 (selection + gate/up) nor 1 (down + combine)", stage);
+  return token_forward(table, shared, args, logits, bias, score_mode, routed_scaling, n_group, topk_group, scale, y, status, combine_mode, 1 << stage, stream);
+}
+
 extern "C" __attribute__((visibility("default"))) int ffmoe_decode_token_layer(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared,
                                                                               const ffmoe_decode* args, const float* logits, const float* bias,
                                                                               int score_mode, float routed_scaling, int n_group, int topk_group,

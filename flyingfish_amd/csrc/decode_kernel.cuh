@@ -71,7 +71,6 @@ __device__ __forceinline__ void load_group(const DecodeParams& p, int g, int& ex
 template <class F, int S, int STAGE, int RG, int NR>
 __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
   constexpr int NROWS = STAGE == 0 ? 2 * NR : NR;
-  constexpr int NW = 4;
   extern __shared__ __align__(16) uint8_t xs[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = uni(tid >> 6);
@@ -80,37 +79,21 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
   __shared__ int s_route_ids[FFMOE_MAX_TOP_K];
   __shared__ float s_route_w[FFMOE_MAX_TOP_K];
   const bool inline_route = STAGE == 0 && RG == 1 && p.route.logits != nullptr;
-  if (STAGE == 0 && RG == 1) {
-    if (inline_route) {
-      if (wave == 0)
-        wave_route_dispatch(p.route.logits, p.route.bias, lane, p.experts, p.top_k, p.route.score_mode, p.route.routed_scaling,
-                            p.route.n_group, p.route.topk_group, s_route_ids, s_route_w, 1);
-      __syncthreads();
-      if (blockIdx.x == 0 && tid < p.top_k) {
-        const_cast<int*>(p.ids)[tid] = s_route_ids[tid];
-        reinterpret_cast<float*>(const_cast<void*>(p.weights))[tid] = s_route_w[tid];
-        if (p.done) p.done[tid] = 0u;
-      }
-    }
-  }
+  // With a shared expert the selection hides behind it: its units need no routing, so every block first takes its slice
+  // of the shared expert's rows on waves 1..3 while wave 0 selects, and the routed units follow once the ids are known.
+  const bool shared_first = inline_route && p.has_shared;
   const int n_routed = p.counters ? uni(load_global<int>(p.counters)) : A;
   const int n_shared = p.counters ? uni(load_global<int>(p.counters + 1)) : (p.has_shared ? p.rows : 0);
   // units per group
   const int out_r = (STAGE == 0 ? p.inter : p.hidden) / NR;
   const int out_s = (STAGE == 0 ? p.shared_inter : p.hidden) / NR;
   const long long routed_units = (long long)n_routed * out_r;
-  const long long total = routed_units + (long long)n_shared * out_s;
-  const long long lo = total * blockIdx.x / gridDim.x, hi = total * (blockIdx.x + 1) / gridDim.x;
-  long long u0 = lo;
-  while (u0 < hi) {
-    // group segment containing u0
-    int g, j0, width;
-    if (u0 < routed_units) { g = int(u0 / out_r); j0 = int(u0 % out_r); width = out_r; }
-    else { const long long v = u0 - routed_units; g = n_routed + int(v / out_s); j0 = int(v % out_s); width = out_s; }
-    const long long seg_end = u0 + (width - j0) < hi ? u0 + (width - j0) : hi;
-    const int count = int(seg_end - u0);
+
+  // One segment: `count` units of group g from unit j0 on, split over the waves wv = 0 .. nw-1 (wv < 0: this wave only
+  // takes part in the staging and the barriers).
+  auto segment = [&](int g, int j0, int count, int nw, int wv, const int* inline_ids) {
     int expert, gn, grow[RG], gslot[RG];
-    load_group<RG>(p, g, expert, gn, grow, gslot, inline_route ? s_route_ids : nullptr);
+    load_group<RG>(p, g, expert, gn, grow, gslot, inline_ids);
     const bool shared = expert < 0;
     const int Kg = STAGE == 0 ? p.hidden : (shared ? p.shared_inter : p.inter);
     // the six slot addresses through scalar-friendly paths (kernel argument or global table), never a generic pointer
@@ -153,7 +136,7 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
     const int nchunks = Kg / F::EPL;
     const int nslabs = (nchunks + S * 64 - 1) / (S * 64);
     // this wave's contiguous run of units inside the segment
-    const int w_lo = count * wave / NW, w_hi = count * (wave + 1) / NW;
+    const int w_lo = wv >= 0 ? count * wv / nw : 0, w_hi = wv >= 0 ? count * (wv + 1) / nw : 0;
     const int my_units = gn > 0 ? w_hi - w_lo : 0;
     const int items = my_units * nslabs;
     const int jw = j0 + w_lo;  // first unit of the run
@@ -260,6 +243,36 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
       item_end(items - 1);
       if (my_units & 63) flush(my_units & ~63, my_units & 63);
     }
+  };
+
+  if (STAGE == 0 && RG == 1) {
+    if (shared_first) {
+      // this block's slice of the shared expert (group A: rows == 1), waves 1..3; wave 0 selects meanwhile
+      const int s_lo = int((long long)out_s * blockIdx.x / gridDim.x), s_hi = int((long long)out_s * (blockIdx.x + 1) / gridDim.x);
+      segment(A, s_lo, s_hi - s_lo, 3, wave - 1, nullptr);
+    }
+    if (inline_route) {
+      if (wave == 0)
+        wave_route_dispatch(p.route.logits, p.route.bias, lane, p.experts, p.top_k, p.route.score_mode, p.route.routed_scaling,
+                            p.route.n_group, p.route.topk_group, s_route_ids, s_route_w, 1);
+      __syncthreads();
+      if (blockIdx.x == 0 && tid < p.top_k) {
+        const_cast<int*>(p.ids)[tid] = s_route_ids[tid];
+        reinterpret_cast<float*>(const_cast<void*>(p.weights))[tid] = s_route_w[tid];
+        if (p.done) p.done[tid] = 0u;
+      }
+    }
+  }
+  const long long total = shared_first ? routed_units : routed_units + (long long)n_shared * out_s;
+  const long long lo = total * blockIdx.x / gridDim.x, hi = total * (blockIdx.x + 1) / gridDim.x;
+  long long u0 = lo;
+  while (u0 < hi) {
+    // group segment containing u0
+    int g, j0, width;
+    if (u0 < routed_units) { g = int(u0 / out_r); j0 = int(u0 % out_r); width = out_r; }
+    else { const long long v = u0 - routed_units; g = n_routed + int(v / out_s); j0 = int(v % out_s); width = out_s; }
+    const long long seg_end = u0 + (width - j0) < hi ? u0 + (width - j0) : hi;
+    segment(g, j0, int(seg_end - u0), 4, wave, inline_route ? s_route_ids : nullptr);
     u0 = seg_end;
   }
 }

@@ -3,73 +3,80 @@
 // moe_down / moe_ffn_weight_f32 and moe_combine*, kernels/moe_ffn.cu:211-302,894-908, kernels/moe_combine.cu:51-116,
 // 541-613).
 //
-// A unit is ONE output column d for ALL groups: the wave streams row d of every live expert's down matrix (and of the
-// shared expert's) in combine order, so the per-expert results of a column meet in one lane and the combine needs no
-// second pass over memory: contributions are neither written nor re-read and the combine launch disappears.
-// The groups are visited in the order the combine adds them (ascending expert id, stable; choice order for the
-// accumulate modes), so the parked sums are already in summation order. Per row the dot product is the same chunk ->
-// lane mapping, step order and wave reduction as k_decode_stage, and the rounding boundaries are those of
-// k_decode_stage + k_combine, so y is bit-identical to the three-launch path.
+// A block owns a run of output columns for ALL groups (live choices + shared expert), so the per-expert results of a
+// column meet in the block's LDS and the combine needs no second pass over memory: contributions are neither written
+// nor re-read and the combine launch disappears. Inside the block the work is the down stage's: a unit is NR
+// consecutive rows of one group's down matrix, the units (group-major) are split evenly over the block's waves, each wave
+// streams whole rows one unit ahead. The number of waves per block is chosen by the host so that the units divide
+// evenly. Per row the dot product is the same chunk -> lane mapping, step order and wave reduction as k_decode_stage,
+// and the groups are combined in the order the combine kernel adds them (ascending expert id, stable; choice order for
+// the accumulate modes) with the rounding boundaries of k_decode_stage + k_combine, so y is bit-identical to the
+// three-launch path.
 #pragma once
 #include "decode_kernel.cuh"
+#include <cstdio>
+#include <cstdlib>
 
 namespace ffmoe {
 
-template <class F, int S, int GMAX>
-__global__ __launch_bounds__(256) void k_decode_finish(const FinishParams q) {
+#define FFMOE_FINISH_GROUPS 9  /* 8 routed choices + the shared expert */
+
+template <class F, int S, int NR>
+__global__ __launch_bounds__(1024) void k_decode_finish(const FinishParams q, const int cmax) {
   const DecodeParams& p = q.d;
-  extern __shared__ __align__(16) uint8_t xs[];  // [groups][inter] BF16 activations
-  __shared__ int s_choice[FFMOE_MAX_TOP_K + 1];
+  constexpr int GT = FFMOE_FINISH_GROUPS;
+  extern __shared__ __align__(16) uint8_t xs[];  // [GT][inter] BF16 activations, then [GT][cmax] f32 row sums
+  __shared__ int s_expert[FFMOE_MAX_TOP_K];      // expert of choice c, -1 = not live
+  __shared__ int s_choice[FFMOE_MAX_TOP_K];      // live choices in combine order
   __shared__ int s_groups;
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = uni(tid >> 6);
+  __shared__ uint64_t s_codes[GT], s_scales[GT];
+  __shared__ float s_glob[GT], s_wk[GT];
+  __shared__ int s_slot[GT];
+  const int tid = threadIdx.x, lane = tid & 63, nthreads = blockDim.x;
+  const int wave = uni(tid >> 6), nw = uni(int(blockDim.x >> 6));
   const int K = p.top_k, I = p.inter, H = p.hidden;
+  float* s_part = reinterpret_cast<float*>(xs + size_t(GT) * I * 2);
   const bool ordered = !(q.mode == FFMOE_COMBINE_ACCUM_FP32 || q.mode == FFMOE_COMBINE_ACCUM_BF16);
+  const bool has_shared = p.has_shared != 0;
 
   // live choices in combine order
-  auto is_live = [&](int c) {
-    const int e = p.ids[c];
-    if (p.active && p.active[c] == 0u) return false;
-    if ((unsigned)e >= (unsigned)p.experts || (p.valid && p.valid[e] == 0u)) return false;
-    return !(p.generation && p.assignment_gen && p.generation[e] != p.assignment_gen[c]);
-  };
   if (tid < K) {
-    const int mine = p.ids[tid];
-    const bool live = is_live(tid);
-    if (!live && (!p.active || p.active[tid] != 0u) && q.status && blockIdx.x == 0) atomicOr(q.status, 1u);  // bad expert id
+    const int e = p.ids[tid];
+    bool live = !(p.active && p.active[tid] == 0u);
+    const bool wanted = live;
+    if (live) live = (unsigned)e < (unsigned)p.experts && !(p.valid && p.valid[e] == 0u);
+    if (live && p.generation && p.assignment_gen && p.generation[e] != p.assignment_gen[tid]) live = false;
+    if (wanted && !live && q.status && blockIdx.x == 0) atomicOr(q.status, 1u);  // bad or stale expert id
+    s_expert[tid] = live ? e : -1;
+  }
+  __syncthreads();
+  if (tid < K) {
+    const int mine = s_expert[tid];
     int rank = 0;
     for (int c = 0; c < K; ++c) {
-      const int other = p.ids[c];
+      const int other = s_expert[c];
       const bool before = ordered ? (other < mine || (other == mine && c < tid)) : c < tid;
-      rank += (is_live(c) && before) ? 1 : 0;
+      rank += (other >= 0 && before) ? 1 : 0;
     }
-    if (live) s_choice[rank] = tid;
+    if (mine >= 0) s_choice[rank] = tid;
   }
   if (tid == 0) {
     int total = 0;
-    for (int c = 0; c < K; ++c) total += is_live(c) ? 1 : 0;
-    if (p.has_shared) s_choice[total] = -1;
-    s_groups = total + (p.has_shared ? 1 : 0);
+    for (int c = 0; c < K; ++c) total += s_expert[c] >= 0 ? 1 : 0;
+    s_groups = total;
   }
   __syncthreads();
-  const int ng = uni(s_groups);
-  const int nr = ng - (p.has_shared ? 1 : 0);  // routed groups come first
-  if (ng == 0) {  // nothing contributes: y = 0
-    for (int d = blockIdx.x * 256 + tid; d < H; d += gridDim.x * 256) q.y[d] = 0;
+  const int nr = uni(s_groups);                 // routed groups, in combine order
+  const int G = nr + (has_shared ? 1 : 0);      // group nr = the shared expert
+  if (G == 0) {  // nothing contributes: y = 0
+    for (int d = blockIdx.x * nthreads + tid; d < H; d += gridDim.x * nthreads) q.y[d] = 0;
     return;
   }
-
-  // per-group constants: thread g gathers group g (ids -> slot table, two dependent loads, all groups in parallel) into
-  // LDS; every wave then reads them back as wave-uniform scalars. Entries past the last group repeat it (their loads hit
-  // the same lines, their sums are never used).
-  __shared__ uint64_t s_codes[GMAX], s_scales[GMAX];
-  __shared__ float s_glob[GMAX], s_wk[GMAX];
-  __shared__ int s_slot[GMAX];
-  if (tid < GMAX) {
-    const int gg = tid < ng ? tid : ng - 1;
-    const int c = s_choice[gg];
-    if (c >= 0) {
-      const int e = p.ids[c];
+  // per-group constants: thread g gathers group g (ids -> slot table, two dependent loads, all groups in parallel)
+  if (tid < G) {
+    if (tid < nr) {
+      const int c = s_choice[tid];
+      const int e = s_expert[c];
       s_codes[tid] = p.slots[size_t(e) * 6 + 4];
       s_scales[tid] = p.slots[size_t(e) * 6 + 5];
       s_glob[tid] = p.global_scales ? p.global_scales[size_t(e) * 3 + 2] : 1.0f;
@@ -82,112 +89,113 @@ __global__ __launch_bounds__(256) void k_decode_finish(const FinishParams q) {
     }
   }
   __syncthreads();
-  uint64_t codes[GMAX], scales[GMAX];
-  float glob[GMAX], wk[GMAX];
-  int slot[GMAX];
-#pragma unroll
-  for (int g = 0; g < GMAX; ++g) {
-    codes[g] = uni64(s_codes[g]); scales[g] = uni64(s_scales[g]);
-    glob[g] = unif(s_glob[g]); wk[g] = unif(s_wk[g]);
-    slot[g] = uni(s_slot[g]);
-  }
 
-  // this wave's contiguous run of output columns
+  // this block's columns, its units (group-major: group g, rows b_lo + NR*i ..) and this wave's contiguous run of them
   const int b_lo = int((long long)H * blockIdx.x / gridDim.x), b_hi = int((long long)H * (blockIdx.x + 1) / gridDim.x);
-  const int count = b_hi - b_lo;
-  const int w_lo = count * wave / 4, w_hi = count * (wave + 1) / 4;
-  const int my_units = w_hi - w_lo;
-  const int d0 = b_lo + w_lo;
+  const int C = b_hi - b_lo;
+  const int P = (C + NR - 1) / NR;
+  const int U = G * P;
+  const int u_lo = U * wave / nw, u_hi = U * (wave + 1) / nw;
+  const int my_units = u_hi - u_lo;
   const int nchunks = I / F::EPL;
 
-  typename F::Chunk buf[GMAX][1][S];
-  auto issue = [&](int t, int g, int s) {
+  typename F::Chunk buf[NR][S];
+  auto issue_unit = [&](int u, int s) {
+    const int g = u / P;
+    const int j = b_lo + (u - g * P) * NR;
+    const uint64_t codes = uni64(s_codes[g]), scales = uni64(s_scales[g]);
+    const float glob = unif(s_glob[g]);
     const int chunk = s * 64 + lane;
     const int cc = chunk < nchunks ? chunk : nchunks - 1;
-    F::load(buf[g][0][s], F::row(codes[g], scales[g], glob[g], d0 + t, I), cc);
+#pragma unroll
+    for (int m = 0; m < NR; ++m) {
+      const int row = j + m < b_hi ? j + m : b_hi - 1;  // a ragged last unit repeats the block's last row
+      F::load(buf[m][s], F::row(codes, scales, glob, row, I), cc);
+    }
   };
   if (my_units > 0) {
 #pragma unroll
-    for (int g = 0; g < GMAX; ++g)
-#pragma unroll
-      for (int s = 0; s < S; ++s) issue(0, g, s);
+    for (int s = 0; s < S; ++s) issue_unit(u_lo, s);
   }
   // activations of every group -> LDS, behind the first weight requests
   {
     const int row_words = I >> 3;
-#pragma unroll
-    for (int g = 0; g < GMAX; ++g) {
-      if (g < ng) {
-        u32x4* dst = reinterpret_cast<u32x4*>(xs + size_t(g) * I * 2);
-        const uint16_t* src = p.h + size_t(slot[g]) * p.h_stride;
-        for (int v = tid; v < row_words; v += 256) dst[v] = load16(src + size_t(v) * 8);
-      }
+    for (int g = 0; g < G; ++g) {
+      u32x4* dst = reinterpret_cast<u32x4*>(xs + size_t(g) * I * 2);
+      const uint16_t* src = p.h + size_t(s_slot[g]) * p.h_stride;
+      for (int v = tid; v < row_words; v += nthreads) dst[v] = load16(src + size_t(v) * 8);
     }
   }
   __syncthreads();
-  if (my_units <= 0) return;
-
-  const float sc = (q.mode == FFMOE_COMBINE_GATED) ? bf16_to_f32(q.scale[0]) : 0.0f;
-  float park[GMAX];
-#pragma unroll
-  for (int g = 0; g < GMAX; ++g) park[g] = 0.0f;
-
-  auto flush = [&](int ub, int nu) {
-    if (lane < nu) {
-      float sum = 0.0f, sh = 0.0f;
-#pragma unroll
-      for (int g = 0; g < GMAX; ++g) {
-        if (g < nr) {
-          const float v = __fmul_rn(p.routed_weight == FFMOE_WEIGHT_AFTER_DOWN_BF16 ? bround(park[g]) : park[g], wk[g]);
-          const float c = bround(v);  // the BF16 contribution
-          sum = q.mode == FFMOE_COMBINE_BF16 ? bround(__fadd_rn(sum, c)) : __fadd_rn(sum, c);
-        } else if (g == nr && g < ng) {
-          sh = bround(park[g]);       // the BF16 shared output
-        }
-      }
-      float v;
-      switch (q.mode) {
-        case FFMOE_COMBINE_GATED: v = __fadd_rn(bround(sum), bround(__fmul_rn(sc, sh))); break;
-        case FFMOE_COMBINE_UNGATED:
-        case FFMOE_COMBINE_ACCUM_BF16: v = __fadd_rn(bround(sum), sh); break;
-        case FFMOE_COMBINE_BF16:
-        case FFMOE_COMBINE_ACCUM_FP32: v = __fadd_rn(sum, sh); break;
-        default: v = sum; break;
-      }
-      q.y[d0 + ub + lane] = f32_to_bf16(v);
-    }
-  };
-
   for (int t = 0; t < my_units; ++t) {
-    const int tn = t + 1 < my_units ? t + 1 : t;  // the last unit re-requests its own rows; nothing reads them
-    const int slot_lane = t & 63;
-    float part[GMAX];
+    const int u = u_lo + t;
+    const int un = t + 1 < my_units ? u + 1 : u;  // the last unit re-requests its own rows; nothing reads them
+    const int g = u / P;
+    const int j = b_lo + (u - g * P) * NR;
+    float acc[NR][1];
 #pragma unroll
-    for (int g = 0; g < GMAX; ++g) {
-      float acc[1][1] = {{0.0f}};
+    for (int m = 0; m < NR; ++m) acc[m][0] = 0.0f;
 #pragma unroll
-      for (int s = 0; s < S; ++s) {
-        if (g < ng) step_compute<F, 1, 1, S>(buf[g], s, xs + size_t(g) * I * 2, I, nchunks, s * 64 + lane, 1, acc);
-        issue(tn, g, s);
-      }
-      part[g] = acc[0][0];
+    for (int s = 0; s < S; ++s) {
+      step_compute<F, NR, 1, S>(buf, s, xs + size_t(g) * I * 2, I, nchunks, s * 64 + lane, 1, acc);
+      issue_unit(un, s);
     }
-    // the reductions of the groups are independent chains: issued together they overlap each other's latency
+    float total[NR];
 #pragma unroll
-    for (int g = 0; g < GMAX; ++g) {
-      const float total = wave_sum(part[g]);
-      park[g] = lane == slot_lane ? total : park[g];
+    for (int m = 0; m < NR; ++m) total[m] = wave_sum(acc[m][0]);
+    if (lane == 0) {
+#pragma unroll
+      for (int m = 0; m < NR; ++m)
+        if (j + m < b_hi) s_part[g * cmax + (j - b_lo) + m] = total[m];
     }
-    if (slot_lane == 63) flush(t - 63, 64);
   }
-  if (my_units & 63) flush(my_units & ~63, my_units & 63);
+  __syncthreads();
+  // ordered combine of the block's columns
+  const float sc = (q.mode == FFMOE_COMBINE_GATED) ? bf16_to_f32(q.scale[0]) : 0.0f;
+  for (int col = tid; col < C; col += nthreads) {
+    float sum = 0.0f;
+    for (int g = 0; g < nr; ++g) {
+      const float d = s_part[g * cmax + col];
+      const float v = __fmul_rn(p.routed_weight == FFMOE_WEIGHT_AFTER_DOWN_BF16 ? bround(d) : d, s_wk[g]);
+      const float c = bround(v);  // the BF16 contribution
+      sum = q.mode == FFMOE_COMBINE_BF16 ? bround(__fadd_rn(sum, c)) : __fadd_rn(sum, c);
+    }
+    const float sh = has_shared ? bround(s_part[nr * cmax + col]) : 0.0f;  // the BF16 shared output
+    float v;
+    switch (q.mode) {
+      case FFMOE_COMBINE_GATED: v = __fadd_rn(bround(sum), bround(__fmul_rn(sc, sh))); break;
+      case FFMOE_COMBINE_UNGATED:
+      case FFMOE_COMBINE_ACCUM_BF16: v = __fadd_rn(bround(sum), sh); break;
+      case FFMOE_COMBINE_BF16:
+      case FFMOE_COMBINE_ACCUM_FP32: v = __fadd_rn(sum, sh); break;
+      default: v = sum; break;
+    }
+    q.y[b_lo + col] = f32_to_bf16(v);
+  }
 }
 
-template <class F, int GMAX, int SMAX, int S = 1>
-void launch_finish_steps(int want, const FinishParams& q, int blocks, size_t lds, hipStream_t st) {
+template <class F, int NR, int SMAX, int S = 1>
+void launch_finish_steps(int want, const FinishParams& q, int blocks, int threads, int cmax, size_t lds, hipStream_t st) {
   if constexpr (S <= SMAX) {
-    if (want == S) hipLaunchKernelGGL((k_decode_finish<F, S, GMAX>), dim3(blocks), dim3(256), lds, st, q);
-    else launch_finish_steps<F, GMAX, SMAX, S + 1>(want, q, blocks, lds, st);
+    if (want == S) hipLaunchKernelGGL((k_decode_finish<F, S, NR>), dim3(blocks), dim3(threads), lds, st, q, cmax);
+    else launch_finish_steps<F, NR, SMAX, S + 1>(want, q, blocks, threads, cmax, lds, st);
+  }
+}
+
+// Grid and block size: one block per CU with 8, 12 or 16 waves (the same number on each of the CU's four SIMDs: the
+// dequantization keeps the vector ALUs busy enough that a SIMD with one wave more than its neighbours finishes last;
+// measured at hidden 7168: 8 waves 28.3 us, 9 waves 31.5 us), whichever divides the block's units most evenly (a wave with
+// 6 units against waves with 5 holds the launch for a fifth longer); ties go to fewer waves.
+inline void finish_shape(int columns, int groups, int nr_rows, int cus, int* blocks, int* waves) {
+  *blocks = columns < cus ? columns : cus;
+  const int per_block = (columns + *blocks - 1) / *blocks;
+  const int units = groups * ((per_block + nr_rows - 1) / nr_rows);
+  double best = 1e30;
+  *waves = 8;
+  for (int w = 8; w <= 16; w += 4) {
+    const int busiest = (units + w - 1) / w;
+    const double cost = double(busiest) * w / double(units);
+    if (cost < best - 1e-9) { best = cost; *waves = w; }
   }
 }
 
@@ -196,14 +204,21 @@ void launch_finish_steps(int want, const FinishParams& q, int blocks, size_t lds
 template <class F>
 int launch_finish(const FinishParams& q, hipStream_t st) {
   const DecodeParams& p = q.d;
-  const int groups = p.top_k + (p.has_shared ? 1 : 0);
   const int steps = (p.inter / F::EPL + 63) / 64;
-  if (steps > 2 || groups > 9)
-    return ff_fail(FFMOE_ERR_UNSUPPORTED, "one-token finish holds at most 9 groups and 2 steps per row (groups=%d, steps=%d)", groups, steps);
-  const size_t lds = size_t(groups) * p.inter * 2;
-  const int blocks = decode_num_cus() * 2;
-  if (groups <= 4) launch_finish_steps<F, 4, 2>(steps, q, blocks, lds, st);
-  else launch_finish_steps<F, 9, 2>(steps, q, blocks, lds, st);
+  if (steps > 2 || p.top_k > FFMOE_FINISH_GROUPS - 1)
+    return ff_fail(FFMOE_ERR_UNSUPPORTED, "one-token finish holds at most %d routed groups and 2 steps per row (top_k=%d, steps=%d)",
+                   FFMOE_FINISH_GROUPS - 1, p.top_k, steps);
+  constexpr int NR = 4;
+  int blocks, waves;
+  finish_shape(p.hidden, p.top_k + (p.has_shared ? 1 : 0), NR, decode_num_cus(), &blocks, &waves);
+  if (const char* e = getenv("FFMOE_FINISH_SHAPE")) {  // "blocks,waves": measurement override
+    int b = 0, w = 0;
+    if (sscanf(e, "%d,%d", &b, &w) == 2 && b >= 1 && w >= 1 && w <= 16) { blocks = b; waves = w; }
+  }
+  const int cmax = (p.hidden + blocks - 1) / blocks;
+  const size_t lds = size_t(FFMOE_FINISH_GROUPS) * p.inter * 2 + size_t(FFMOE_FINISH_GROUPS) * cmax * 4;
+  if (lds > 64 * 1024) return ff_fail(FFMOE_ERR_UNSUPPORTED, "one-token finish: %zu bytes of LDS per block", lds);
+  launch_finish_steps<F, NR, 2>(steps, q, blocks, waves * 64, cmax, lds, st);
   return ff_launch_status();
 }
 

@@ -325,6 +325,29 @@ class DecodeOps:
         capi.check(rc)
         return True
 
+    def token_forward(self, x, ids, weights, mode, y, logits, bias=None, status=None, scale=None, score_mode=capi.NOAUX_SIGMOID,
+                      routed_scaling=1.0, n_group=1, topk_group=1, stage=None):
+        """rows == 1, two launches: selection in the prologue of the gate/up launch (ids / weights are outputs), then
+        down + routing weight + ordered combine into y. stage 0 / 1 = one of the launches alone. Returns False (nothing
+        launched) when the shape is outside the fast path."""
+        act_mode, swiglu, limit, rw, wf32 = self.cfg
+        d = capi.Decode(self.rows, self.top_k, act_mode, swiglu, limit, rw, wf32,
+                        x.data_ptr(), ids.data_ptr(), None, weights.data_ptr(),
+                        self.contributions.data_ptr(), self.shared_out.data_ptr() if self.shared_out is not None else None,
+                        self.done.data_ptr(), self.scratch.data_ptr(), self.scratch.numel(), None)
+        sh = ctypes.byref(self._shared_c) if self._shared_c is not None else None
+        L = capi.lib()
+        if stage is None:
+            rc = L.ffmoe_decode_token_forward(ctypes.byref(self._table_c), sh, ctypes.byref(d), _ptr(logits), _ptr(bias), score_mode,
+                                              routed_scaling, n_group, topk_group, _ptr(scale), _ptr(y), _ptr(status), mode, _stream())
+        else:
+            rc = L.ffmoe_decode_token_forward_stage(ctypes.byref(self._table_c), sh, ctypes.byref(d), _ptr(logits), _ptr(bias), score_mode,
+                                                    routed_scaling, n_group, topk_group, _ptr(scale), _ptr(y), _ptr(status), mode, stage, _stream())
+        if rc == capi.ERR_UNSUPPORTED:
+            return False
+        capi.check(rc)
+        return True
+
     def token_layer(self, x, ids, weights, mode, y, status=None, scale=None, logits=None, bias=None, score_mode=capi.NOAUX_SIGMOID,
                     routed_scaling=1.0, n_group=1, topk_group=1, active=None):
         """rows == 1: selection (when logits are given; ids / weights are then outputs), gate/up, down, routing weight and
@@ -570,6 +593,9 @@ class NativeMoe:
         self.fused_finish = False
         # one token: run the top-k selection in the prologue of the gate/up launch (one launch less)
         self.inline_select = True
+        # one token: selection + gate/up, then down + combine (ffmoe_decode_token_forward): three launches per layer with
+        # the logits. contributions / shared_out / done are not written on this path; set False to get them.
+        self.two_launch = True
         # one token: everything after the logits in one resident launch (ffmoe_decode_token_layer). Off by default: on
         # MI355X at the DeepSeek-V3 shape it measured 91 us against 79 us for the three launches it replaces.
         self.one_launch = False
@@ -585,6 +611,13 @@ class NativeMoe:
                                        routed_scaling=scaling, n_group=ng, topk_group=kg):
                 return self.y
             self.one_launch = False
+        if self.rows == 1 and self.two_launch:
+            RouteOps.logits_f32(x, self.router, out=self.logits)
+            mode = self.combine_mode if self.decode.shared_out is not None else capi.COMBINE_ROUTED
+            if self.decode.token_forward(x, self.ids, self.weights, mode, self.y, self.logits, bias=self.bias if self.bias.dim() == 1 else self.bias[0],
+                                         status=self.status, routed_scaling=scaling, n_group=ng, topk_group=kg):
+                return self.y
+            self.two_launch = False
         if self.rows == 1 and self.inline_select:
             # one token: logits launch, then gate/up with the selection in its prologue, down, combine (4 launches)
             RouteOps.logits_f32(x, self.router, out=self.logits)

@@ -282,6 +282,26 @@ int ffmoe_decode_token_layer(const ffmoe_expert_table* table, const ffmoe_shared
                              const float* logits, const float* bias, int score_mode, float routed_scaling, int n_group,
                              int topk_group, const void* scale, void* y, uint32_t* status, int combine_mode, void* stream);
 
+/* One token, everything after the router logits in TWO launches (the default of the host mirror's NativeMoe for one row):
+ * launch 1 = top-k selection (same arithmetic as ffmoe_route_topk_noaux; args->ids and args->weights (f32) are OUTPUTS,
+ * args->done is cleared) in the prologue of the gate/up + SwiGLU launch, hidden behind the shared expert's rows, which
+ * need no routing; launch 2 = ffmoe_decode_finish (down, routing weight and the ordered combine into y [hidden] BF16).
+ * Replaces moe_route_select_noaux, moe_gate_up, moe_down / moe_ffn_weight_f32 and moe_combine* of NativeMoe::run for one
+ * token (src/backend/cuda/moe/decode.rs:1187-1297; kernels/moe_route.cu:315-390, kernels/moe_ffn.cu:98-302,894-908,
+ * kernels/moe_combine.cu:51-116,541-613); ids, weights and y are bit-identical to the separate calls. contributions,
+ * shared_out are not written. Arguments as ffmoe_decode_token_layer; the scratch arena needs no preparation.
+ * FFMOE_ERR_UNSUPPORTED (nothing launched): rows != 1, top_k > 8, experts not 64 * 2^n, a shared expert of another
+ * format or width, an active mask or epochs, or down rows beyond the kernel's register buffers. */
+int ffmoe_decode_token_forward(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared, const ffmoe_decode* args,
+                               const float* logits, const float* bias, int score_mode, float routed_scaling, int n_group,
+                               int topk_group, const void* scale, void* y, uint32_t* status, int combine_mode, void* stream);
+/* One launch of the same call, for timing a kernel alone: stage 0 = selection + gate/up, stage 1 = down + combine
+ * (stage 0 then stage 1 with the same arguments equals ffmoe_decode_token_forward). No counterpart in the reference. */
+int ffmoe_decode_token_forward_stage(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared, const ffmoe_decode* args,
+                                     const float* logits, const float* bias, int score_mode, float routed_scaling, int n_group,
+                                     int topk_group, const void* scale, void* y, uint32_t* status, int combine_mode, int stage,
+                                     void* stream);
+
 /* One-token finish: the down projection of every live choice and of the shared expert, the routing weight and the
  * ordered combine in ONE launch, for rows == 1. Call after ffmoe_decode_contribute_stage(table, shared, args, 0, stream)
  * with the same table / shared / args (the gate/up activations are taken from args->scratch); writes y[hidden] and
@@ -290,8 +310,8 @@ int ffmoe_decode_token_layer(const ffmoe_expert_table* table, const ffmoe_shared
  * moe_combine{,_ungated,_bf16,_accum,_routed} (kernels/moe_ffn.cu:211-302,894-908; kernels/moe_combine.cu:51-116,
  * 541-613) of NativeMoe::run (src/backend/cuda/moe/decode.rs:1187-1297). args->active plays the role of final_active;
  * *status |= 1 when a live choice names an expert that is out of range or not valid.
- * Returns FFMOE_ERR_UNSUPPORTED (nothing launched) when the shape is outside the fast path (rows != 1, more than 9
- * groups, shared expert of another format or width, rows of the down matrix longer than two 64-lane steps): run the
+ * Returns FFMOE_ERR_UNSUPPORTED (nothing launched) when the shape is outside the fast path (rows != 1, top_k > 8,
+ * shared expert of another format or width, rows of the down matrix longer than two 64-lane steps): run the
  * two separate calls then. */
 int ffmoe_decode_finish(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared, const ffmoe_decode* args,
                         const void* scale, void* y, uint32_t* status, int combine_mode, void* stream);

@@ -327,6 +327,7 @@ def test_c3_token_through_native_moe_256_experts_8_groups():
     table, store, shared = _sparse_c3_table(hit, 134)
     layer = ops.NativeMoe(table, shared, router.cuda(), bias.cuda(), 1, K, 2.5, 8, 4, swiglu=capi.SWIGLU_TWICE,
                           routed_weight=capi.WEIGHT_AFTER_DOWN_BF16, combine_mode=capi.COMBINE_UNGATED)
+    layer.two_launch = False  # the separate launches first: they write contributions and shared_out
     print("C3 token through NativeMoe, experts hit", hit, flush=True)
     y = bits(layer.run(x.cuda())).copy()
     torch.cuda.synchronize()
@@ -345,8 +346,8 @@ def test_c3_token_through_native_moe_256_experts_8_groups():
     assert np.all(err <= 3 * (K + 1) * ulp), float(np.max(err / ulp))
     assert orc.rel_l2(y, want_y) <= 4e-3
     # the other launch variants of the same layer: bit-identical y
-    for name, setup in (("separate top-k launch", dict(inline_select=False)), ("fused finish", dict(inline_select=False, fused_finish=True)),
-                        ("one resident launch", dict(one_launch=True))):
+    for name, setup in (("two launches after the logits (default)", dict()), ("separate top-k launch", dict(two_launch=False, inline_select=False)),
+                        ("fused finish", dict(two_launch=False, inline_select=False, fused_finish=True)), ("one resident launch", dict(one_launch=True))):
         other = ops.NativeMoe(table, shared, router.cuda(), bias.cuda(), 1, K, 2.5, 8, 4, swiglu=capi.SWIGLU_TWICE,
                               routed_weight=capi.WEIGHT_AFTER_DOWN_BF16, combine_mode=capi.COMBINE_UNGATED)
         for k_, v_ in setup.items():

@@ -791,6 +791,7 @@ def test_one_token_selection_inside_gate_up_launch(fmt, experts, n_group, topk_g
     for inline in (False, True):
         layer = NativeMoe(table, sh, router, bias, 1, top_k, routed_scaling=2.5, n_group=n_group, topk_group=topk_group)
         layer.inline_select = inline
+        layer.two_launch = False  # this test reads contributions and done, which the two-launch path does not write
         layer.decode.done.fill_(7)  # stale flags: both paths must clear them
         y = bits(layer.run(x)).copy()
         assert layer.inline_select == inline
@@ -813,3 +814,39 @@ def test_selection_inside_gate_up_launch_rejects_batches():
     ids = torch.zeros((2, 2), dtype=torch.int32, device=DEV)
     w = torch.zeros((2, 2), device=DEV)
     assert ops.contribute_from_logits(x, logits, None, ids, w) is None
+
+
+@pytest.mark.parametrize("fmt,hidden,inter", [(capi.FMT_FP8_BLOCK128, 512, 256), (capi.FMT_FP8_BLOCK128, 1280, 2048), (capi.FMT_NVFP4, 512, 256),
+                                              (capi.FMT_FP8_CHANNEL, 256, 512), (capi.FMT_BF16, 512, 256)])
+@pytest.mark.parametrize("experts,n_group,topk_group,top_k", [(64, 1, 1, 3), (256, 8, 4, 8), (128, 4, 2, 5)])
+def test_token_forward_two_launches_equal_the_separate_launches(fmt, hidden, inter, experts, n_group, topk_group, top_k):
+    """ffmoe_decode_token_forward (selection behind the shared expert's rows in the gate/up launch, then down + weight +
+    combine in one launch): ids, weights and y equal the separate launches bit for bit, for every combine mode, with and
+    without a shared expert, over consecutive tokens on one arena."""
+    table = make_table(fmt, 4 + 1, hidden, inter, 161)[0]
+    # experts beyond the four materialised ones reuse their slots (only the arithmetic per slot matters here)
+    slots = table.slots[:4].repeat((experts + 3) // 4, 1)[:experts].contiguous()
+    big = ExpertTable(fmt, experts, hidden, inter, table.storage, slots,
+                      table.global_scales[:4].repeat((experts + 3) // 4, 1)[:experts].contiguous() if table.global_scales is not None else None)
+    sh = table.shared_struct(4)
+    router = rand_bf16((experts, hidden), 0.05, 162).to(DEV)
+    bias = (torch.randn(experts, generator=torch.Generator().manual_seed(163)) * 0.1).to(DEV)
+    for mode, shared in ((capi.COMBINE_BF16, True), (capi.COMBINE_UNGATED, True), (capi.COMBINE_ACCUM_FP32, True), (capi.COMBINE_ROUTED, False)):
+        got = {}
+        for two in (False, True):
+            layer = NativeMoe(big, sh if shared else None, router, bias, 1, top_k, routed_scaling=2.5, n_group=n_group, topk_group=topk_group,
+                              combine_mode=mode)
+            layer.two_launch = two
+            layer.inline_select = False
+            outs = []
+            for step in range(3):
+                x = rand_bf16((1, hidden), 1.0, 165 + step).to(DEV)
+                print("token forward fmt=%d hidden=%d inter=%d experts=%d top_k=%d mode=%d two_launch=%d step=%d" % (fmt, hidden, inter, experts, top_k, mode, two, step), flush=True)
+                y = bits(layer.run(x)).copy()
+                outs.append((layer.ids.cpu().numpy().copy(), layer.weights.cpu().numpy().copy(), y))
+                assert int(layer.status.item()) == 0
+            assert layer.two_launch == two
+            got[two] = outs
+        for a, b in zip(got[False], got[True]):
+            for name, u, v in zip(("ids", "weights", "y"), a, b):
+                assert np.array_equal(u, v), "%s, combine mode %d" % (name, mode)

@@ -73,6 +73,7 @@ def test_token_layer_selects_like_the_separate_launch(fmt, experts, n_group, top
         layer = NativeMoe(table, sh, router, bias, 1, top_k, routed_scaling=2.5, n_group=n_group, topk_group=topk_group)
         layer.one_launch = one_launch
         layer.inline_select = False
+        layer.two_launch = False
         outs = []
         for step in range(4):  # consecutive launches on one scratch arena: each must see only its own activations
             x = rand_bf16((1, hidden), 1.0, 64 + step).to(DEV)
@@ -197,6 +198,7 @@ def test_token_layer_graph_replay_equals_eager():
                       routed_weight=capi.WEIGHT_AFTER_DOWN_BF16)
     xs = [rand_bf16((1, 1024), 1.0, 25 + i).to(DEV) for i in range(3)]
     layer.one_launch = False
+    layer.two_launch = False
     eager = [bits(layer.run(x)).copy() for x in xs]
     layer.one_launch = True
     x_in = xs[0].clone()
