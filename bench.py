@@ -21,10 +21,11 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
 
-# HBM bytes per gate/up launch from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of this script, each scaled by what
-# the same counter reads for a 256 MiB plain copy (--calibrate-copy); measured per workload, keyed by (batch, experts).
-# Summary and commands: profiles/decode_layer_fp8_c3_batch1.hbm_traffic.txt. Other workloads report null.
+# HBM bytes per gate/up launch, not read in the run: FETCH_SIZE and WRITE_SIZE of rocprofv3 --pmc runs of this script, each
+# scaled by what the same counter reads for a 256 MiB plain copy (--calibrate-copy); keyed by (batch, experts). Source of
+# the figure, with the commands: profiles/decode_layer_fp8_c3_batch1.hbm_traffic.txt. Other workloads report null.
 GATE_UP_TRAFFIC_BYTES = {(1, 256): 265007737}
+TRAFFIC_SOURCE = "profiles/decode_layer_fp8_c3_batch1.hbm_traffic.txt"
 
 
 def parse():
@@ -32,10 +33,12 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", choices=["decode", "prefill", "widening", "linear"], default="decode",
+    ap.add_argument("--workload", choices=["decode", "prefill", "widening", "linear", "c1"], default="decode",
                     help="decode = BASELINE config 3 (the headline line); prefill = config 5 (4096 tokens, Zipf s=1.1, FP8 matrix cores); "
                          "widening = the formats and fused steps next to the path (per-channel FP8 / BF16 experts, Lane16 / Lane8 orders, "
-                         "combine + residual); linear = config 2 (standalone FP8 block skinny linear, M = 1, 4, 16, 64)")
+                         "combine + residual); linear = config 2 (standalone FP8 block skinny linear, M = 1, 4, 16, 64); "
+                         "c1 = config 1 (hidden 2048, 64 experts, softmax top-4, intermediate 1408, one token)")
+    ap.add_argument("--no-parity-gate", action="store_true", help="skip the oracle check of one ring slot that precedes the timing")
     ap.add_argument("--batch", type=int, default=None, help="tokens per step (decode: 1, 8, 64; prefill: 4096)")
     ap.add_argument("--format", choices=["fp8", "nvfp4", "e2m1"], default="fp8",
                     help="routed-expert format: fp8 = config 3 (shared expert FP8 too); nvfp4 = config 4 (NVFP4 routed experts, "
@@ -131,6 +134,139 @@ def gate_up_bytes(table, distinct, rows, dims):
     return (distinct * table.weight_bytes_per_expert() + table.shared_bytes) * 2 // 3 + rows * H * 2 + rows * (K + 1) * I * 2
 
 
+def _checkers():
+    """The oracle and the comparison helpers of the test-suite: the checker, never the thing measured."""
+    tests = os.path.join(ROOT, "tests")
+    if tests not in sys.path:
+        sys.path.insert(0, tests)
+    import numpy as np
+    import oracle as orc
+    import helpers
+    return np, orc, helpers
+
+
+def parity_gate_decode(args, torch, capi, ops, table, layer, x, dims):
+    """Oracle check of one ring slot, outside the timed region; raises SystemExit when the layer the timing is about to
+    measure does not match the CPU restatement: router ids and weights bit for bit, every contribution and the shared
+    row at the stage bars of the test-suite (relative L2 <= 1e-3; end to end through both stages <= 4 BF16 steps), y of
+    the timed launch sequence bit-identical to the separate launches and inside the layer bound of the oracle pipeline."""
+    np, orc, hp = _checkers()
+    H, I, E, K = dims
+    rows = min(args.batch, 2)
+    y_timed = hp.bits(layer.run(x)).copy()
+    ids_t, w_t = layer.ids.cpu().numpy().copy(), layer.weights.cpu().numpy().copy()
+    saved = (layer.two_launch, layer.one_launch)
+    layer.two_launch = layer.one_launch = False   # the separate launches write contributions and shared_out
+    y_sep = hp.bits(layer.run(x)).copy()
+    layer.two_launch, layer.one_launch = saved
+    torch.cuda.synchronize()
+    fail = []
+    if not (np.array_equal(y_timed, y_sep) and np.array_equal(ids_t, layer.ids.cpu().numpy())):
+        fail.append("the timed launch sequence and the separate launches disagree")
+    xb = hp.bits(x)
+    lg = orc.route_logits_f32(xb, hp.bits(layer.router))
+    bias = layer.bias.cpu().numpy()
+    oi, ow = orc.route_topk_noaux(lg, bias[None, :] if bias.ndim == 1 else bias, K, 0, 2.5, 8, 4)
+    if not np.array_equal(ids_t, oi):
+        fail.append("router ids differ from the oracle")
+    if not np.array_equal(w_t.view(np.uint32), ow.view(np.uint32)):
+        fail.append("router weights differ from the oracle")
+    got_c, got_s = hp.bits(layer.decode.contributions), hp.bits(layer.decode.shared_out)
+    shared_table = getattr(table, "shared_table", None)
+    eff = {}
+
+    def weights_of(e):
+        if e not in eff:
+            eff[e] = hp.effective_weights(shared_table, 0) if (e == E and shared_table is not None) else hp.effective_weights(table, e)
+        return eff[e]
+    jobs = [(r, c) for r in range(rows) for c in range(K)] + [(r, -1) for r in range(rows)]
+    for e in sorted({int(oi[r, c]) for r in range(rows) for c in range(K)} | {E}):
+        weights_of(e)
+
+    def one(lo, hi):
+        out = []
+        for r, c in jobs[lo:hi]:
+            g, u, d = weights_of(int(oi[r, c]) if c >= 0 else E)
+            out.append(orc.expert_ffn(xb[r], g, u, d, float(ow[r, c]) if c >= 0 else 1.0, orc.TWICE, 0.0, orc.AFTER_DOWN_BF16, orc.LANE8, orc.SILU_DIV,
+                                      apply_weight=c >= 0))
+        return out
+    res = [t for chunk in hp.run_parallel(one, len(jobs), min(16, len(os.sched_getaffinity(0)))) for t in chunk]
+    want_c = np.stack(res[:rows * K]).reshape(rows, K, H)
+    want_s = np.stack(res[rows * K:])
+    stats = {}
+    try:
+        stats["contributions"] = hp.assert_close_bf16(got_c[:rows], want_c, "contributions", max_ulp=4)
+        stats["shared_out"] = hp.assert_close_bf16(got_s[:rows], want_s, "shared expert", max_ulp=4)
+    except AssertionError as exc:
+        fail.append(str(exc))
+    want_y = orc.combine(want_c, want_s, None, oi[:rows], None, orc.COMBINE_UNGATED)
+    terms = np.concatenate([orc.bf16_to_f32(want_c), orc.bf16_to_f32(want_s)[:, None, :], orc.bf16_to_f32(want_y)[:, None, :]], axis=1)
+    ulp = 2.0 ** (np.floor(np.log2(np.maximum(np.max(np.abs(terms), axis=1).astype(np.float64), 1e-30))) - 7)
+    err = np.abs(orc.bf16_to_f32(y_timed[:rows]).astype(np.float64) - orc.bf16_to_f32(want_y).astype(np.float64))
+    y_rel = orc.rel_l2(y_timed[:rows], want_y)
+    if not (np.all(err <= 3 * (K + 1) * ulp) and y_rel <= 4e-3):
+        fail.append("y: %.1f steps of the largest term, relative L2 %.2e" % (float(np.max(err / ulp)), y_rel))
+    if fail:
+        print("bench.py parity gate FAILED: " + "; ".join(fail), file=sys.stderr)
+        sys.exit(3)
+    return {"checked": "ring slot 0, %d token row(s): ids and weights bit-exact, %d contributions + shared rows, y" % (rows, rows * K),
+            "contributions_rel_l2": stats["contributions"][0], "contributions_worst_bf16_steps": stats["contributions"][1],
+            "y_rel_l2": y_rel, "oracle": "oracle/ffmoe_oracle.cpp (scalar, Lane8 form)"}
+
+
+def parity_gate_prefill(args, torch, capi, ops, table, pre, x, ids, wts, dims, a16):
+    """Oracle check of a sample of the cohort, outside the timed region: the assignments at the start, the middle and the
+    end of the segments of the most popular expert, a mid-popular and the least popular one, each stage on the inputs it
+    saw (activations against the oracle's, the down stage against the oracle's down stage on the device's activations)."""
+    np, orc, hp = _checkers()
+    H, I, E, K = dims
+    pre.done.zero_()
+    got = pre.contribute(x, ids, wts)
+    torch.cuda.synchronize()
+    v = pre.scratch_views()
+    n_live = int(v["totals"][3].item())
+    perm = v["perm"].cpu().numpy()[:n_live]
+    offsets = v["offsets"].cpu().numpy()
+    counts = np.diff(offsets)
+    order = np.argsort(-counts, kind="stable")
+    live = [int(e) for e in order if counts[e] > 0]
+    picks = []
+    for e in (live[0], live[len(live) // 2], live[-1]):
+        lo, hi = int(offsets[e]), int(offsets[e + 1])
+        picks += sorted({lo, (lo + hi) // 2, hi - 1})
+    xb = hp.bits(x)
+    flat_ids, flat_w = ids.cpu().numpy().reshape(-1), wts.cpu().numpy().reshape(-1)
+    act = hp.bits(v["act"][torch.tensor(picks, device="cuda")])
+    g2 = hp.bits(got.reshape(pre.rows * K, H)[torch.from_numpy(perm[picks]).cuda().long()])
+    host = {}
+    for e in sorted({int(flat_ids[perm[p]]) for p in picks}):
+        host[e] = hp.effective_weights(table, e) if a16 else hp.host_expert(table, e)
+
+    def one(lo, hi):
+        out = []
+        for i in range(lo, hi):
+            a = int(perm[picks[i]])
+            m, wa = host[int(flat_ids[a])], float(flat_w[a])
+            if a16:
+                _, want_act = orc.expert_ffn(xb[a // K], m[0], m[1], m[2], wa, orc.TWICE, 0.0, orc.AFTER_DOWN_BF16, orc.LANE8, orc.SILU_DIV, return_act=True)
+                d_ref = orc.expert_down(act[i], m[2], 1.0, 0, orc.LANE8, False)
+            else:
+                _, want_act = orc.expert_ffn_w8a8(xb[a // K], *m, wa, orc.TWICE, 0.0, orc.AFTER_DOWN_BF16, return_act=True)
+                d_ref = orc.expert_down_w8a8(act[i], m[4], m[5], apply_weight=False)
+            out.append((want_act, d_ref, wa))
+        return out
+    res = [t for chunk in hp.run_parallel(one, len(picks), min(16, len(os.sched_getaffinity(0)))) for t in chunk]
+    try:
+        a_stats = hp.assert_close_bf16(act, np.stack([t[0] for t in res]), "activations", max_ulp=3)
+        d_stats = hp.assert_weighted_down_close(g2, np.stack([t[1] for t in res]), [t[2] for t in res], "down stage on the device activations")
+    except AssertionError as exc:
+        print("bench.py parity gate FAILED: " + str(exc), file=sys.stderr)
+        sys.exit(3)
+    return {"checked": "%d assignments (first, middle, last of the segments of the most, a mid and the least popular expert), per stage" % len(picks),
+            "activations_rel_l2": a_stats[0], "activations_worst_bf16_steps": a_stats[1], "down_rel_l2": d_stats[0], "down_worst_bf16_steps": d_stats[1],
+            "oracle": "oracle/ffmoe_oracle.cpp (%s)" % ("W*A16, Lane8 form" if a16 else "W8A8 block-128, 32-lane order")}
+
+
 def cpu_baseline(args, torch, table, layer, xs, dims):
     """The reference's CPU expert path (multithreaded port in oracle/cpu_baseline.cpp) on a bounded sample of the
     same workload: the routed + shared experts of a few ring slots, weights copied to host, cold between trials."""
@@ -221,6 +357,9 @@ def prefill_main(args, torch, capi, ops, synth):
         step()
     torch.cuda.synchronize()
     assert int(status.item()) == 0
+    parity = None
+    if not args.no_parity_gate and not mx:
+        parity = parity_gate_prefill(args, torch, capi, ops, table, pre, x, ids, wts, dims, a16)
     t0 = time.perf_counter()
     for _ in range(args.steps):
         step()
@@ -270,6 +409,132 @@ def prefill_main(args, torch, capi, ops, synth):
         "down_kernel": {"kernel": "ffmoe::k_w16_grouped<F, MF, 1, P>" if a16 else "ffmoe::k_mx_grouped<MF, 1, 1, P>" if mx else "ffmoe::k_w8a8_grouped<MF, 1, P>", "avg_ms": k1_avg, "min_ms": k1[0],
                         "tflops": A * 2.0 * H * I / (k1_avg * 1e-3) / 1e12},
     }
+    out["parity"] = parity if parity is not None else ("not gated in bench.py for this format (tests/test_gpu_e8m0.py, tests/test_gpu_fullsize.py)" if mx else None)
+    if not args.no_cpu_baseline and args.format == "fp8":
+        out["cpu_baseline"] = cpu_baseline_prefill(args, torch, table, x, ids, wts, dims)
+    print(json.dumps(out))
+
+
+def cpu_baseline_prefill(args, torch, table, x, ids, wts, dims):
+    """The reference's CPU expert path (W8A16 contract, multithreaded port in oracle/cpu_baseline.cpp) on a bounded
+    sample of the cohort: the assignments of the first 24 token rows (192 expert FFNs), 1 warm-up + 3 timed, median,
+    scaled to the whole cohort by the assignment count."""
+    import numpy as np
+    import oracle as orc
+    H, I, E, K = dims
+    threads = min(orc.cpubase().cpubase_max_threads(), len(os.sched_getaffinity(0)))
+    rows = min(24, x.shape[0])
+    ids_h, w_h = ids[:rows].cpu().numpy(), wts[:rows].cpu().numpy()
+    cache = {}
+
+    def host(e):
+        if e not in cache:
+            cache[e] = tuple(v.cpu().numpy() for v in table.expert_views(e))
+        return cache[e]
+    experts, rws, w, ap = [], [], [], []
+    for r in range(rows):
+        for c in range(K):
+            experts.append(host(int(ids_h[r, c]))); rws.append(r); w.append(float(w_h[r, c])); ap.append(1)
+    x_bits = x[:rows].view(torch.int16).cpu().numpy().view(np.uint16)
+    job = orc.CpuDecodeJob(x_bits, rws, experts, w, ap)
+    times = []
+    for i in range(4):
+        t0 = time.perf_counter()
+        job.run(threads)
+        if i > 0:
+            times.append(time.perf_counter() - t0)
+    times.sort()
+    per = times[len(times) // 2] / (rows * K)
+    total = x.shape[0] * K
+    return {"value": per * total * 1e3, "unit": "ms/cohort", "cores": threads, "kind": "port", "isa": orc.cpubase().cpubase_isa().decode(),
+            "sample": "%d expert FFNs (all %d choices of the first %d token rows), 1 warm-up + %d timed, median, scaled by %d / %d assignments; "
+                      "W8A16 arithmetic of the CPU expert path" % (rows * K, K, rows, len(times), total, rows * K),
+            "tokens_per_s": x.shape[0] / (per * total)}
+
+
+def c1_main(args, torch, capi, ops, synth):
+    """BASELINE config 1: one MoE decode step at the shape of the reference's own CPU-runnable case: 1 token, hidden 2048,
+    64 routed experts (no shared expert), softmax top-4 over BF16 logits, intermediate 1408, FP8 E4M3 experts with
+    128 x 128 f32 block scales. A step = fused BF16-logit route + gate/up + down + routed-only combine on a token from a
+    ring, inputs resident in HBM."""
+    import numpy as np
+    H, I, E, K = 2048, 1408, 64, 4
+    dev = "cuda"
+    table = ops.ExpertTable.allocate(capi.FMT_FP8_BLOCK128, E, H, I, dev)
+    for e in range(E):
+        v = table.expert_views(e)
+        for i, shape in enumerate([(I, H), (I, H), (H, I)]):
+            c, sc = synth.quant_fp8_block(synth.normal(shape, 0.02, args.seed * 100003 + e * 3 + i, device=dev))
+            v[2 * i].copy_(c); v[2 * i + 1].copy_(sc)
+    router = synth.normal((E, H), 0.02, args.seed + 1, device=dev, dtype=torch.bfloat16)
+    xs = [synth.normal((1, H), 1.0, args.seed + 1000 + i, device=dev, dtype=torch.bfloat16) for i in range(args.ring)]
+    dec = ops.DecodeOps(table, None, 1, K, capi.ACT_BF16, capi.SWIGLU_TWICE, 0.0, capi.WEIGHT_AFTER_DOWN_BF16, False)
+    y = torch.empty((1, H), dtype=torch.bfloat16, device=dev)
+    status = torch.zeros(1, dtype=torch.int32, device=dev)
+    logits = torch.empty((1, E), dtype=torch.bfloat16, device=dev)
+    ids = torch.empty((1, K), dtype=torch.int32, device=dev)
+    wts = torch.empty((1, K), dtype=torch.bfloat16, device=dev)
+
+    def step(i):
+        x = xs[i % len(xs)]
+        ops.RouteOps.route(x, router, K, capi.SCORE_SOFTMAX, logits=logits, ids=ids, weights=wts)
+        dec.done.zero_()
+        c, _ = dec.contribute(x, ids, wts)
+        return ops.CombineOps.combine(c, None, ids, capi.COMBINE_ROUTED, done=dec.done, status=status, out=y)
+
+    parity = None
+    if not args.no_parity_gate:
+        np_, orc, hp = _checkers()
+        got_y = hp.bits(step(0)).copy()
+        torch.cuda.synchronize()
+        xb = hp.bits(xs[0])
+        ol = orc.route_logits_bf16(xb, hp.bits(router))
+        oi, ow = orc.route_topk_softmax(ol, K)
+        ok = np.array_equal(hp.bits(logits), ol) and np.array_equal(ids.cpu().numpy(), oi) and np.array_equal(hp.bits(wts), ow)
+        want_c = np.stack([orc.expert_ffn(xb[0], *hp.effective_weights(table, int(oi[0, c])), float(orc.bf16_to_f32(ow)[0, c]), orc.TWICE, 0.0,
+                                          orc.AFTER_DOWN_BF16, orc.LANE8, orc.SILU_DIV) for c in range(K)])[None]
+        try:
+            st = hp.assert_close_bf16(hp.bits(dec.contributions), want_c, "contributions", max_ulp=4)
+            assert ok, "router logits, ids or weights differ from the oracle"
+            assert np.array_equal(got_y, orc.combine(hp.bits(dec.contributions), None, None, oi, None, orc.COMBINE_ROUTED)), "combine"
+        except AssertionError as exc:
+            print("bench.py parity gate FAILED: " + str(exc), file=sys.stderr)
+            sys.exit(3)
+        parity = {"checked": "ring slot 0: BF16 logits, ids and weights bit-exact, 4 contributions, combine bit-exact on the device contributions",
+                  "contributions_rel_l2": st[0], "contributions_worst_bf16_steps": st[1]}
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(args.warmup + i)
+    torch.cuda.synchronize()
+    us = (time.perf_counter() - t0) / args.steps * 1e6
+    per = table.weight_bytes_per_expert()
+    nbytes = K * per + E * H * 2 + H * 2 * (2 + K)
+    # the streaming launches alone (gate/up, then down) with events on the launch stream
+    def timed(stage):
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(8)]
+        for a, b in ev:
+            a.record()
+            for i in range(16):
+                dec.contribute(xs[i % len(xs)], ids, wts, stage=stage)
+            b.record()
+        torch.cuda.synchronize()
+        return sum(a.elapsed_time(b) for a, b in ev) * 1e3 / (8 * 16)
+    k0, k1 = timed(0), timed(1)
+    b0 = K * per * 2 // 3 + H * 2 + K * I * 2
+    out = {"metric": "moe_layer_decode_us", "value": us, "unit": "us/layer", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+           "ms_per_step": us / 1e3, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+           "dtype": "fp8_e4m3 weights, bf16 activations, f32 accumulate", "data": "synthetic",
+           "config": {"workload": "MoE decode step at the reference's CPU-runnable shape (BASELINE config 1), batch 1", "hidden": H, "intermediate": I,
+                      "experts": E, "shared_experts": 0, "top_k": K, "routing": "softmax top-4 over BF16 logits", "ring": len(xs),
+                      "launches_per_layer": "fused BF16-logit route; gate/up; down; combine (+ a done-flag fill)"},
+           "tokens_per_s": 1e6 / us, "layer_bytes": nbytes, "layer_hbm_gbps": nbytes / us / 1e3, "layer_hbm_frac": nbytes / us / 1e3 / HBM_PEAK_GBPS,
+           "roofline": {"kernel": "ffmoe::k_decode_stage<FmtFp8, S, 0, 1, NR> (gate/up + SwiGLU)", "bound": "hbm", "achieved": b0 / k0 / 1e3,
+                        "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": b0 / k0 / 1e3 / HBM_PEAK_GBPS, "traffic": None, "bytes_per_launch": b0,
+                        "avg_us": k0, "launches_timed": 128, "note": "the same 4 experts every launch (34 MB: cache-resident), latency-bound"},
+           "down_kernel": {"avg_us": k1}, "parity": parity}
     print(json.dumps(out))
 
 
@@ -424,6 +689,8 @@ def main():
         return widening_main(args, torch, capi, ops, synth)
     if args.workload == "linear":
         return linear_main(args, torch, capi, ops, synth)
+    if args.workload == "c1":
+        return c1_main(args, torch, capi, ops, synth)
     table, layer, xs, dims = build_layer(args, torch, capi, ops, synth)
     H, I, E, K = dims
     torch.cuda.synchronize()
@@ -443,6 +710,7 @@ def main():
         torch.cuda.synchronize()
         distinct.append(int(torch.unique(layer.ids).numel()))
     assert int(layer.status.item()) == 0, "combine saw a (row, choice) slot that was not contributed exactly once"
+    parity = None if args.no_parity_gate else parity_gate_decode(args, torch, capi, ops, table, layer, xs[0], dims)
 
     graphs = None
     if args.graph:
@@ -477,31 +745,53 @@ def main():
     mean_distinct = sum(used) / len(used)
     bytes_layer = layer_bytes(table, mean_distinct, args.batch, dims)
 
-    # dominant kernel: the gate/up + SwiGLU launch. Route every ring slot once and keep its ids/weights, then time
-    # batches of back-to-back gate/up launches over the ring with events on the launch stream (a batch per event
-    # pair, so the event overhead is amortised and the figure is the kernel's own duration; weights stay cold
-    # because consecutive launches read different experts).
+    # dominant kernel: the gate/up + SwiGLU launch, timed as the layer issues it. One token: the launch with the top-k
+    # selection in its prologue (stage 0 of ffmoe_decode_token_forward) from each ring slot's logits; batches: the plain
+    # gate/up launch from each ring slot's ids. 8 batches of 16 back-to-back launches over the ring with events on the
+    # launch stream (a batch per event pair, so the event overhead is amortised and the figure is the kernel's own
+    # duration; weights stay cold because consecutive launches read different experts), whatever --steps is.
     dec = layer.decode
     routed = []
     for x in xs:
         layer.run(x)
-        routed.append((layer.ids.clone(), layer.weights.clone()))
+        routed.append((layer.ids.clone(), layer.weights.clone(), layer.logits.clone()))
     torch.cuda.synchronize()
-    batch = 16
-    nb = max(1, args.steps // batch)
-    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(nb)]
-    for b_ in range(nb):
-        ev[b_][0].record()
+    token_path = args.batch == 1 and layer.two_launch and not args.one_launch
+    bias1 = layer.bias if layer.bias.dim() == 1 else layer.bias[0]
+
+    def launch(stage, s_):
+        if token_path:
+            ok = dec.token_forward(xs[s_], layer.ids, layer.weights, layer.combine_mode, layer.y, routed[s_][2], bias=bias1, status=layer.status,
+                                   routed_scaling=2.5, n_group=8, topk_group=4, stage=stage)
+            assert ok
+        else:  # stage 1 alone would reuse the previous launch's grouping: time both launches and subtract
+            dec.contribute(xs[s_], routed[s_][0], routed[s_][1], stage=0 if stage == 0 else None)
+
+    def time_stage(stage):
+        batch, nb = 16, 8
         for i in range(batch):
-            s_ = (b_ * batch + i) % len(xs)
-            dec.contribute(xs[s_], routed[s_][0], routed[s_][1], stage=0)
-        ev[b_][1].record()
-    torch.cuda.synchronize()
-    kt = sorted(a.elapsed_time(b) * 1e3 / batch for a, b in ev)  # us per launch
+            launch(stage, i % len(xs))
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(nb)]
+        for b_ in range(nb):
+            ev[b_][0].record()
+            for i in range(batch):
+                launch(stage, (b_ * batch + i) % len(xs))
+            ev[b_][1].record()
+        torch.cuda.synchronize()
+        return sorted(a.elapsed_time(b) * 1e3 / batch for a, b in ev), nb * batch  # us per launch
+
+    kt, launches_timed = time_stage(0)
     k_avg = sum(kt) / len(kt)
     mean_distinct_k = sum(distinct) / len(distinct)
     k_bytes = gate_up_bytes(table, mean_distinct_k, args.batch, dims)
     achieved = k_bytes / (k_avg * 1e-6) / 1e9
+    # second streaming launch: down (+ routing weight; one token: + ordered combine)
+    dt, _ = time_stage(1)
+    if not token_path:
+        dt = sorted(max(t - k_avg, 0.0) for t in dt)
+    d_avg = sum(dt) / len(dt)
+    d_bytes = (mean_distinct_k * table.weight_bytes_per_expert() + table.shared_bytes) // 3 + args.batch * (K + 1) * I * 2 + \
+        (args.batch * H * 2 if token_path else args.batch * (K + 1) * H * 2)
 
     out = {
         "metric": "moe_layer_decode_us", "value": us_per_layer, "unit": "us/layer", "n_gpus": 1,
@@ -515,17 +805,26 @@ def main():
                    "routing": "sigmoid grouped top-8 (8 groups, keep 4), renormalised x2.5",
                    "weights": "E4M3 + f32 128x128 block scales" if args.format == "fp8" else "E2M1 pairs + E4M3 scale per 16 + f32 global",
                    "act_mode": "FFMOE_ACT_BF16 (W8A16)" if args.format == "fp8" else "BF16 activations (W4A16)",
-                   "batch": args.batch, "ring": len(xs), "launch": "eager" if graphs is None else "hip graph per ring slot"},
+                   "batch": args.batch, "ring": len(xs), "launch": "eager" if graphs is None else "hip graph per ring slot",
+                   "launches_per_layer": "router logits; gate/up with the top-k selection in its prologue; down + weight + combine" if token_path else
+                                         "router logits; top-k; grouping; gate/up; down; combine"},
         "tokens_per_s": args.batch / (us_per_layer * 1e-6),
         "distinct_routed_experts": mean_distinct,
         "layer_bytes": bytes_layer,
         "layer_hbm_gbps": bytes_layer / (us_per_layer * 1e-6) / 1e9,
         "layer_hbm_frac": bytes_layer / (us_per_layer * 1e-6) / 1e9 / HBM_PEAK_GBPS,
-        "roofline": {"kernel": "ffmoe::k_decode_stage<%s, S, 0, RG, NR> (gate/up + SwiGLU stage of ffmoe_decode_contribute)" % ("FmtFp8" if args.format == "fp8" else "FmtNvfp4"),
+        "roofline": {"kernel": "ffmoe::k_decode_stage<%s, S, 0, RG, NR> (gate/up + SwiGLU launch%s)" % (
+                         "FmtFp8" if args.format == "fp8" else "FmtNvfp4", ", top-k selection in its prologue, as the layer issues it" if token_path else ""),
                      "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBPS, "traffic": GATE_UP_TRAFFIC_BYTES.get((args.batch, args.experts)) if args.format == "fp8" else None,
+                     "traffic_source": TRAFFIC_SOURCE if (args.format == "fp8" and (args.batch, args.experts) in GATE_UP_TRAFFIC_BYTES) else None,
                      "bytes_per_launch": k_bytes, "avg_us": k_avg, "min_us": kt[0], "median_us": kt[len(kt) // 2],
-                     "launches_timed": nb * batch},
+                     "launches_timed": launches_timed},
+        "down_kernel": {"kernel": ("ffmoe::k_decode_finish<F, S, NR> (down + routing weight + ordered combine)" if token_path else
+                                   "ffmoe::k_decode_stage<F, S, 1, RG, NR> (down + routing weight)"),
+                        "bytes_per_launch": d_bytes, "avg_us": d_avg, "min_us": dt[0], "median_us": dt[len(dt) // 2],
+                        "achieved": d_bytes / (d_avg * 1e-6) / 1e9, "frac": d_bytes / (d_avg * 1e-6) / 1e9 / HBM_PEAK_GBPS},
+        "parity": parity,
     }
     if not args.no_cpu_baseline and args.format == "fp8":
         out["cpu_baseline"] = cpu_baseline(args, torch, table, layer, xs, dims)

@@ -60,7 +60,7 @@ struct FinishParams {
   // the whole token layer in one launch (k_token_layer)
   int whole;              // 0: one-token finish, 1: selection, gate/up, down and combine
   uint32_t* h32;          // [(top_k + 1), d.h_stride] activations as (launch tag << 16 | BF16) words; row top_k = shared expert
-  unsigned int* gen;      // device-wide launch counter: the tag of this launch
+  uint32_t tag;           // 1 .. 65535, the tag of this launch's activation words (host-side launch counter)
   unsigned int* exited;   // blocks that left the kernel; the last one clears it and advances gen
   unsigned int* claims;   // 128 claim counters, 32 words apart: gate/up and down phase of up to 64 grid partitions
   unsigned int spin_limit;

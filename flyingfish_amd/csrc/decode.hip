@@ -26,10 +26,10 @@ int prefill_impl(const ffmoe_expert_table* table, const ffmoe_prefill* args, int
 
 namespace ffmoe {
 
-// Device-side state of the one-launch token layer, zero when the module is loaded: the launch counter whose low 16
-// bits tag the activations of a launch, and 16 slots of {exit counter, 128 claim counters}, every counter on its own
-// 128-byte line. Calls take slots round-robin, so launches in flight on different streams do not share counters.
-// Every launch leaves its slot at zero.
+// Device-side state of the one-launch token layer, zero when the module is loaded: 16 slots of {exit counter, 128 claim
+// counters}, every counter on its own 128-byte line. Calls take slots round-robin and get their activation tag from the
+// same host-side ticket, so launches in flight on different streams share neither counters nor a tag. Every launch
+// leaves its slot at zero.
 #define FFMOE_TOKEN_SLOTS 16
 #define FFMOE_TOKEN_SLOT_WORDS (129 * 32)
 static __device__ __align__(256) unsigned int g_token_state[32 + FFMOE_TOKEN_SLOTS * FFMOE_TOKEN_SLOT_WORDS];
@@ -47,12 +47,11 @@ static bool token_layer_sync(FinishParams* q) {
     }
     base[dev].store(b, std::memory_order_release);
   }
-  static const unsigned int limit = [] {
-    const char* e = getenv("FFMOE_TOKEN_SPIN_LIMIT");
-    return e ? (unsigned int)strtoul(e, nullptr, 10) : 100000u;
-  }();
-  const unsigned int slot = next.fetch_add(1, std::memory_order_relaxed) % FFMOE_TOKEN_SLOTS;
-  q->gen = b;
+  const char* le = getenv("FFMOE_TOKEN_SPIN_LIMIT");  // read per call, so a process can change it
+  const unsigned int limit = le ? (unsigned int)strtoul(le, nullptr, 10) : 100000u;
+  const unsigned int ticket = next.fetch_add(1, std::memory_order_relaxed);
+  const unsigned int slot = ticket % FFMOE_TOKEN_SLOTS;
+  q->tag = 1u + ticket % 65535u;
   q->exited = b + 32 + slot * FFMOE_TOKEN_SLOT_WORDS;
   q->claims = q->exited + 32;
   q->spin_limit = limit;
@@ -140,12 +139,13 @@ extern "C" __attribute__((visibility("default"))) uint64_t ffmoe_decode_scratch_
 }
 
 // layout_k >= 0: the call processes args->top_k choices per row (0 = the shared expert only) but lays the scratch
-// arena out for layout_k choices, so a routed pass and a shared pass of another weight format can share one arena.
+// arena out for layout_k choices and for rows of max(inter, shared inter, arena_shared_inter) activations, so a routed
+// pass and a shared pass of another weight format share one arena with the same row stride and the same offsets.
 // Pass 1 keeps its group descriptors and counters behind those of pass 0: the passes may be issued stage by stage
 // (both gate/up launches, then both down launches), so neither may overwrite the other's grouping.
 static int decode_impl(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared, const ffmoe_decode* args,
                        int stage_mask, void* stream, int layout_k = -1, int pass = 0, const FinishParams* fin = nullptr,
-                       const RouteInline* route = nullptr, int form = -1) {
+                       const RouteInline* route = nullptr, int form = -1, int arena_shared_inter = 0) {
   FF_REQUIRE(table && args, FFMOE_ERR_NULL, "table/args is NULL");
   const int R = args->rows, K = args->top_k, E = table->experts, H = table->hidden, I = table->inter;
   const int LK = layout_k < 0 ? K : layout_k;
@@ -184,7 +184,8 @@ static int decode_impl(const ffmoe_expert_table* table, const ffmoe_shared_exper
     for (int i = 0; i < 6; i += 2)
       FF_REQUIRE(shared->slot[i] != 0 && shared->slot[i] % 16 == 0, FFMOE_ERR_ALIGN, "shared expert slot[%d] is NULL or misaligned", i);
   }
-  const uint64_t need = ffmoe_decode_scratch_bytes(R, LK > 0 ? LK : 1, E, H, I, shared ? SI : 0);
+  const int arena_si = shared ? (SI > arena_shared_inter ? SI : arena_shared_inter) : arena_shared_inter;
+  const uint64_t need = ffmoe_decode_scratch_bytes(R, LK > 0 ? LK : 1, E, H, I, arena_si);
   FF_PTR_ALIGNED(args->scratch, 256);
   FF_REQUIRE(args->scratch_bytes >= need, FFMOE_ERR_SCRATCH, "decode scratch holds %llu bytes, %llu needed",
              (unsigned long long)args->scratch_bytes, (unsigned long long)need);
@@ -206,7 +207,7 @@ static int decode_impl(const ffmoe_expert_table* table, const ffmoe_shared_exper
     FF_NO_OVERLAP(args->done, A * 4, args->scratch, args->scratch_bytes);
   }
 
-  const int imax = I > SI ? I : SI;
+  const int imax = I > arena_si ? I : arena_si;
   const int kmax_lds = H > imax ? H : imax;
   FF_REQUIRE(size_t(kmax_lds) * 2 <= 160 * 1024 / 2, FFMOE_ERR_SHAPE, "row of %d BF16 does not fit the LDS staging", kmax_lds);
 
@@ -299,7 +300,7 @@ static int decode_dispatch(const ffmoe_expert_table* table, const ffmoe_shared_e
     return prefill_impl(table, &pf, (stage_mask & 1 ? 3 : 0) | (stage_mask & 2 ? 12 : 0), stream);
   }
   if (!table || !args || !shared || shared->format == table->format) return decode_impl(table, shared, args, stage_mask, stream);
-  FF_TRY(decode_impl(table, nullptr, args, stage_mask, stream, args->top_k));
+  FF_TRY(decode_impl(table, nullptr, args, stage_mask, stream, args->top_k, 0, nullptr, nullptr, -1, shared->inter));
   ffmoe_expert_table as_shared = *table;
   as_shared.format = shared->format;
   ffmoe_decode only_shared = *args;

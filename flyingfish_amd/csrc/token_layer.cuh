@@ -60,7 +60,7 @@ __global__ __launch_bounds__(256) void k_token_layer(const FinishParams q) {
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = uni(tid >> 6);
   // launch tag, 1 .. 65535: never 0, so a zero-filled arena holds no word that looks valid
-  const uint32_t tag = 1u + uint32_t(uni(int(__hip_atomic_load(q.gen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)))) % 65535u;
+  const uint32_t tag = q.tag;  // chosen by the host per launch: launches in flight on different streams never share one
   const bool ordered = !(q.mode == FFMOE_COMBINE_ACCUM_FP32 || q.mode == FFMOE_COMBINE_ACCUM_BF16);
   const bool select_here = p.route.logits != nullptr;
   const int has_shared = p.has_shared;
@@ -364,10 +364,9 @@ __global__ __launch_bounds__(256) void k_token_layer(const FinishParams q) {
     if (s_gave_up && q.status) atomicOr(q.status, 2u);
     const unsigned int left = __hip_atomic_fetch_add(q.exited, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     s_last = left + 1 == gridDim.x;
-    if (s_last) {  // last block out: clear the claim counters, the next launch gets a new tag
+    if (s_last) {  // last block out: clear the claim counters
       for (int i = 0; i < 128; ++i) __hip_atomic_store(q.claims + i * 32, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       __hip_atomic_store(q.exited, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      __hip_atomic_fetch_add(q.gen, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
   }
   __syncthreads();

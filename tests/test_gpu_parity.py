@@ -350,13 +350,16 @@ def test_decode_seeded_shape_sweep(seed):
             assert_close_bf16(so[None, :], want[None, :], "shared_out row %d" % r, max_ulp=4)
 
 
-@pytest.mark.parametrize("rows,routed_fmt,shared_fmt", [(1, capi.FMT_NVFP4, capi.FMT_BF16), (6, capi.FMT_NVFP4, capi.FMT_BF16),
-                                                        (3, capi.FMT_FP8_BLOCK128, capi.FMT_BF16)])
-def test_decode_shared_expert_in_another_format(rows, routed_fmt, shared_fmt):
-    """BASELINE config 4: NVFP4 routed experts next to a BF16 shared expert (two passes over one scratch arena)."""
+@pytest.mark.parametrize("rows,routed_fmt,shared_fmt,shared_extra", [(1, capi.FMT_NVFP4, capi.FMT_BF16, 0), (6, capi.FMT_NVFP4, capi.FMT_BF16, 0),
+                                                                     (3, capi.FMT_FP8_BLOCK128, capi.FMT_BF16, 0), (9, capi.FMT_NVFP4, capi.FMT_BF16, 8),
+                                                                     (5, capi.FMT_FP8_BLOCK128, capi.FMT_NVFP4, 32), (4, capi.FMT_NVFP4, capi.FMT_BF16, -64)])
+def test_decode_shared_expert_in_another_format(rows, routed_fmt, shared_fmt, shared_extra):
+    """BASELINE config 4: NVFP4 routed experts next to a BF16 shared expert (two passes over one scratch arena). With a
+    shared expert slightly wider (or narrower) than the routed ones both passes must still agree on the arena's row
+    stride and on where the grouping tables sit, also when the stages are issued one by one."""
     experts, hidden, inter, top_k, seed = 6, 1024, 512, 3, 91
     table, ref = make_table(routed_fmt, experts, hidden, inter, seed)
-    stable, sref = make_table(shared_fmt, 1, hidden, inter, seed + 1)
+    stable, sref = make_table(shared_fmt, 1, hidden, inter + shared_extra, seed + 1)
     sh = stable.shared_struct(0)
     x = rand_bf16((rows, hidden), 1.0, seed + 7)
     g = synth.generator(seed + 8)

@@ -248,3 +248,35 @@ def test_cpu_baseline_equals_the_scalar_oracle(threads):
             g, u, d = (orc.dequant_fp8_block(exs[a][i], exs[a][i + 1]) for i in (0, 2, 4))
             ref = orc.expert_ffn(x[rows[a]], g, u, d, w[a], orc.TWICE, 0.0, boundary, orc.LANE16, orc.SILU_RCP, apply_weight=bool(ap[a]))
             assert np.array_equal(ref, out[a])
+
+
+def test_struct_layouts_match_the_c_header(tmp_path):
+    """The ctypes mirrors in flyingfish_amd/capi.py (and with them the #[repr(C)] structs a Rust binding declares) must
+    have the size and field offsets a C compiler gives the structs of include/ffmoe.h (reference: MoeDecode,
+    src/backend/cuda/moe/decode.rs:26-44; MoePrefillContribute, src/backend/cuda/moe/prefill.rs:57-91)."""
+    import ctypes
+    import subprocess
+    structs = {"ffmoe_expert_table": capi.ExpertTable, "ffmoe_shared_expert": capi.SharedExpert, "ffmoe_decode": capi.Decode,
+               "ffmoe_prefill": capi.Prefill}
+    lines = ['#include <stdio.h>', '#include <stddef.h>', '#include "ffmoe.h"', 'int main(void) {']
+    for cname, cls in structs.items():
+        lines.append('  printf("%s size %%zu\\n", sizeof(%s));' % (cname, cname))
+        for field, _ in cls._fields_:
+            lines.append('  printf("%s %s %%zu\\n", offsetof(%s, %s));' % (cname, field, cname, field))
+    lines += ['  return 0;', '}']
+    src = tmp_path / "layout.c"
+    src.write_text("\n".join(lines))
+    exe = tmp_path / "layout"
+    include = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include")
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-I", include, str(src), "-o", str(exe)], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout
+    seen = 0
+    for line in out.splitlines():
+        cname, what, value = line.split()
+        cls = structs[cname]
+        if what == "size":
+            assert ctypes.sizeof(cls) == int(value), "%s: ctypes size %d, C size %s" % (cname, ctypes.sizeof(cls), value)
+        else:
+            assert getattr(cls, what).offset == int(value), "%s.%s: ctypes offset %d, C offset %s" % (cname, what, getattr(cls, what).offset, value)
+        seen += 1
+    assert seen == sum(len(c._fields_) + 1 for c in structs.values())
