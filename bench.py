@@ -148,7 +148,9 @@ def _checkers():
 def parity_gate_decode(args, torch, capi, ops, table, layer, x, dims):
     """Oracle check of one ring slot, outside the timed region; raises SystemExit when the layer the timing is about to
     measure does not match the CPU restatement: router ids and weights bit for bit, every contribution and the shared
-    row at the stage bars of the test-suite (relative L2 <= 1e-3; end to end through both stages <= 4 BF16 steps), y of
+    row end to end through both stages (relative L2 <= 1e-3 over the tensor; element-wise 16 BF16 steps, the loose bound
+    the test-suite uses where a flipped BF16 step of an activation moves a cancelled down output: the per-stage bars of
+    2 steps are held by tests/test_gpu_fullsize.py on the same shapes), y of
     the timed launch sequence bit-identical to the separate launches and inside the layer bound of the oracle pipeline."""
     np, orc, hp = _checkers()
     H, I, E, K = dims
@@ -195,8 +197,8 @@ def parity_gate_decode(args, torch, capi, ops, table, layer, x, dims):
     want_s = np.stack(res[rows * K:])
     stats = {}
     try:
-        stats["contributions"] = hp.assert_close_bf16(got_c[:rows], want_c, "contributions", max_ulp=4)
-        stats["shared_out"] = hp.assert_close_bf16(got_s[:rows], want_s, "shared expert", max_ulp=4)
+        stats["contributions"] = hp.assert_close_bf16(got_c[:rows], want_c, "contributions", max_ulp=16)
+        stats["shared_out"] = hp.assert_close_bf16(got_s[:rows], want_s, "shared expert", max_ulp=16)
     except AssertionError as exc:
         fail.append(str(exc))
     want_y = orc.combine(want_c, want_s, None, oi[:rows], None, orc.COMBINE_UNGATED)

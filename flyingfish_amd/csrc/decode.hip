@@ -22,6 +22,8 @@ int decode_token_layer_bf16(const FinishParams& q, hipStream_t st);
 int decode_token_layer_fp8c(const FinishParams& q, hipStream_t st);
 int decode_form_launch(int fmt, int form, const DecodeParams& p, int stage_mask, hipStream_t st);
 int prefill_impl(const ffmoe_expert_table* table, const ffmoe_prefill* args, int stages, void* stream);
+int shared_expert_w16(const ffmoe_shared_expert* shared, const void* x, int R, int H, int swiglu, float limit, void* act, void* shared_out,
+                      int stage_mask, void* stream_);
 }  // namespace ffmoe
 
 namespace ffmoe {
@@ -134,7 +136,9 @@ extern "C" __attribute__((visibility("default"))) uint64_t ffmoe_decode_scratch_
   const uint64_t groups = (max_groups * sizeof(GroupDesc) + 255) & ~uint64_t(255);
   // FFMOE_ACT_FP8_BLOCK128 runs on the grouped matrix-core path, which lays the arena out differently
   const uint64_t w8a8 = ffmoe_prefill_scratch_bytes(rows, top_k, experts, hidden, inter, shared_inter);
-  const uint64_t own = h + groups + 256;
+  // a shared expert served by the matrix-core path (large batches) keeps its activations behind the decode arena
+  const uint64_t shared_act = shared_inter > 0 ? ((uint64_t(rows) * shared_inter * 2 + 255) & ~uint64_t(255)) : 0;
+  const uint64_t own = h + groups + 256 + shared_act;
   return own > w8a8 ? own : w8a8;
 }
 
@@ -298,6 +302,58 @@ static int decode_dispatch(const ffmoe_expert_table* table, const ffmoe_shared_e
     pf.contributions = args->contributions; pf.done = args->done; pf.scratch = args->scratch; pf.scratch_bytes = args->scratch_bytes;
     pf.shared = shared; pf.shared_out = args->shared_out; pf.assignment_gen = args->assignment_gen;
     return prefill_impl(table, &pf, (stage_mask & 1 ? 3 : 0) | (stage_mask & 2 ? 12 : 0), stream);
+  }
+  // Row counts from which the matrix-core cohort kernels take over for block-FP8 experts (same effective weights and BF16
+  // boundaries, the dot products in the matrix instruction's FP32 order instead of the wave's): the whole batch at
+  // FFMOE_DECODE_COHORT_ROWS (per layer at hidden 7168 / 256 experts: 64 rows 2.00 against 2.40 ms on the streaming kernels,
+  // 48 rows 1.81 against 2.00, 32 rows 1.51 against 1.55, 8 rows 0.65 against 0.54 ms), below that a block-FP8 shared expert
+  // alone from FFMOE_DECODE_SHARED_COHORT_ROWS on (it has every row: streamed once instead of once per row group that fits
+  // LDS; 16 rows 0.935 against 0.964 ms; a BF16 shared expert next to NVFP4 experts measured slower there, 1.88 against
+  // 1.80 ms at 32 rows, and stays on the streaming kernels).
+  // (0 switches a rule off; read at every call)
+  const char* ce = getenv("FFMOE_DECODE_COHORT_ROWS");
+  const char* se = getenv("FFMOE_DECODE_SHARED_COHORT_ROWS");
+  const int cohort_rows = ce ? atoi(ce) : 32, shared_rows = se ? atoi(se) : 16;
+  if (table && args && args->act_mode == FFMOE_ACT_BF16 && args->rows > 1) {
+    const int fmt = table->format, H = table->hidden, I = table->inter, R = args->rows;
+    auto on_matrix_cores = [&](int f, int inter) {
+      const int gran = f == FFMOE_FMT_FP8_BLOCK128 ? 128 : 64;
+      return (f == FFMOE_FMT_FP8_BLOCK128 || f == FFMOE_FMT_NVFP4 || f == FFMOE_FMT_BF16 || f == FFMOE_FMT_FP8_CHANNEL) && H % gran == 0 && inter % gran == 0 &&
+             H >= gran && inter >= gran;
+    };
+    const bool shared_ok = !shared || on_matrix_cores(shared->format, shared->inter);
+    if (cohort_rows > 0 && R >= cohort_rows && fmt == FFMOE_FMT_FP8_BLOCK128 && args->top_k >= 1 && on_matrix_cores(fmt, I) && shared_ok) {
+      ffmoe_prefill pf{};
+      pf.rows = args->rows; pf.top_k = args->top_k; pf.act_mode = FFMOE_ACT_BF16;
+      pf.swiglu = args->swiglu; pf.swiglu_limit = args->swiglu_limit; pf.routed_weight = args->routed_weight; pf.weights_f32 = args->weights_f32;
+      pf.x = args->x; pf.ids = args->ids; pf.active = args->active; pf.weights = args->weights;
+      pf.contributions = args->contributions; pf.done = args->done; pf.scratch = args->scratch; pf.scratch_bytes = args->scratch_bytes;
+      pf.shared = shared; pf.shared_out = args->shared_out; pf.assignment_gen = args->assignment_gen;
+      return prefill_impl(table, &pf, (stage_mask & 1 ? 3 : 0) | (stage_mask & 2 ? 12 : 0), stream);
+    }
+    if (shared && shared_rows > 0 && R >= shared_rows && args->top_k >= 1 && shared_ok && shared->format == FFMOE_FMT_FP8_BLOCK128) {
+      // routed choices on the streaming kernels, the shared expert on the matrix cores with its activations behind the arena
+      FF_TRY(decode_impl(table, nullptr, args, stage_mask, stream, args->top_k, 0, nullptr, nullptr, -1, shared->inter));
+      const int SI = shared->inter;
+      FF_REQUIRE(SI >= 64, FFMOE_ERR_SHAPE, "shared inter=%d", SI);
+      FF_PTR16(args->shared_out);
+      for (int i = 0; i < 6; i += 2)
+        FF_REQUIRE(shared->slot[i] != 0 && shared->slot[i] % 16 == 0, FFMOE_ERR_ALIGN, "shared expert slot[%d] is NULL or misaligned", i);
+      const size_t xb = size_t(R) * H * 2;
+      FF_NO_OVERLAP(args->shared_out, xb, args->x, xb);
+      FF_NO_OVERLAP(args->shared_out, xb, args->contributions, size_t(R) * args->top_k * H * 2);
+      FF_NO_OVERLAP(args->shared_out, xb, args->scratch, args->scratch_bytes);
+      const uint64_t act_bytes = (uint64_t(R) * SI * 2 + 255) & ~uint64_t(255);
+      const uint64_t need = ffmoe_decode_scratch_bytes(R, args->top_k, table->experts, H, I, SI);
+      FF_REQUIRE(args->scratch_bytes >= need, FFMOE_ERR_SCRATCH, "decode scratch holds %llu bytes, %llu needed", (unsigned long long)args->scratch_bytes,
+                 (unsigned long long)need);
+      // the last act_bytes of what ffmoe_decode_scratch_bytes asks for lie behind everything decode_impl lays out
+      const uint64_t A = uint64_t(R) * args->top_k, imax = uint64_t(I > SI ? I : SI);
+      const uint64_t own = (((A + R) * imax * 2 + 255) & ~uint64_t(255)) + (((A + R + 2) * sizeof(GroupDesc) + 255) & ~uint64_t(255)) + 256;
+      uint8_t* act = (uint8_t*)args->scratch + own;
+      FF_REQUIRE(own + act_bytes <= args->scratch_bytes, FFMOE_ERR_SCRATCH, "decode scratch too small for the shared expert's activations");
+      return shared_expert_w16(shared, args->x, R, H, args->swiglu, args->swiglu_limit, act, args->shared_out, stage_mask, stream);
+    }
   }
   if (!table || !args || !shared || shared->format == table->format) return decode_impl(table, shared, args, stage_mask, stream);
   FF_TRY(decode_impl(table, nullptr, args, stage_mask, stream, args->top_k, 0, nullptr, nullptr, -1, shared->inter));

@@ -304,6 +304,40 @@ extern "C" __attribute__((visibility("default"))) uint64_t ffmoe_prefill_scratch
 
 namespace ffmoe {
 int prefill_impl(const ffmoe_expert_table* table, const ffmoe_prefill* args, int stages, void* stream_);
+
+// The always-on expert over all rows in the decode path's W*A16 arithmetic on the BF16 matrix cores, as one dense group
+// per 16 .. 64 rows: the weights stream once however many rows there are. act [rows, shared inter] BF16 holds the SwiGLU
+// activations between the two launches; stage_mask bit 0 = gate/up + SwiGLU, bit 1 = down. Arguments are checked by the
+// callers.
+int shared_expert_w16(const ffmoe_shared_expert* shared, const void* x, int R, int H, int swiglu, float limit, void* act, void* shared_out,
+                      int stage_mask, void* stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  const int SI = shared->inter;
+  const unsigned blocks = ((unsigned)num_cus_p() * 2u) & ~7u;
+  const int smf = R > 32 ? 4 : R > 16 ? 2 : 1;
+  const int stm = 16 * smf;
+  const uint32_t sgroups = uint32_t((R + stm - 1) / stm);
+  W16Params q{};
+  q.rows_total = R; q.top_k = 1;
+  q.swiglu = swiglu; q.limit = limit;
+  if (stage_mask & 1) {
+    q.a = (const uint16_t*)x;
+    q.w0_codes = shared->slot[0]; q.w0_scales = shared->slot[1]; q.w1_codes = shared->slot[2]; q.w1_scales = shared->slot[3];
+    q.g0 = shared->global_scales[0]; q.g1 = shared->global_scales[1];
+    q.total_units = sgroups * uint32_t((SI + 127) / 128);
+    q.out = (uint16_t*)act; q.K = H; q.N = SI;
+    FF_TRY(launch_w16_fmt<0>(shared->format, q, smf, std::min<unsigned>(blocks, (q.total_units + 7u) & ~7u), stream));
+  }
+  if (stage_mask & 2) {
+    q.a = (const uint16_t*)act;
+    q.w0_codes = shared->slot[4]; q.w0_scales = shared->slot[5]; q.w1_codes = 0; q.w1_scales = 0;
+    q.g0 = shared->global_scales[2]; q.g1 = q.g0;
+    q.total_units = sgroups * uint32_t((H + 255) / 256);
+    q.out = (uint16_t*)shared_out; q.K = SI; q.N = H;
+    FF_TRY(launch_w16_fmt<2>(shared->format, q, smf, std::min<unsigned>(blocks, (q.total_units + 7u) & ~7u), stream));
+  }
+  return 0;
+}
 }
 extern "C" __attribute__((visibility("default"))) int ffmoe_prefill_contribute(const ffmoe_expert_table* table, const ffmoe_prefill* args, void* stream) {
   return prefill_impl(table, args, 15, stream);
@@ -464,30 +498,9 @@ int prefill_impl(const ffmoe_expert_table* table, const ffmoe_prefill* args, int
       p.out = (uint16_t*)args->contributions; p.done = args->done; p.weights = args->weights; p.K = I; p.N = H;
       FF_TRY(launch_w16_fmt<1>(table->format, p, mf, blocks, stream));
     }
-    if (shared) {
-      const int smf = R > 32 ? 4 : R > 16 ? 2 : 1;
-      const int stm = 16 * smf;
-      const uint32_t sgroups = uint32_t((R + stm - 1) / stm);
-      W16Params q{};
-      q.rows_total = R; q.top_k = 1;
-      q.swiglu = args->swiglu; q.limit = args->swiglu_limit;
-      if (stages & 2) {
-        q.a = (const uint16_t*)args->x;
-        q.w0_codes = shared->slot[0]; q.w0_scales = shared->slot[1]; q.w1_codes = shared->slot[2]; q.w1_scales = shared->slot[3];
-        q.g0 = shared->global_scales[0]; q.g1 = shared->global_scales[1];
-        q.total_units = sgroups * uint32_t((SI + 127) / 128);
-        q.out = (uint16_t*)(s + l.sh_act); q.K = H; q.N = SI;
-        FF_TRY(launch_w16_fmt<0>(shared->format, q, smf, std::min<unsigned>(blocks, (q.total_units + 7u) & ~7u), stream));
-      }
-      if (stages & 8) {
-        q.a = (const uint16_t*)(s + l.sh_act);
-        q.w0_codes = shared->slot[4]; q.w0_scales = shared->slot[5]; q.w1_codes = 0; q.w1_scales = 0;
-        q.g0 = shared->global_scales[2]; q.g1 = q.g0;
-        q.total_units = sgroups * uint32_t((H + 255) / 256);
-        q.out = (uint16_t*)args->shared_out; q.K = SI; q.N = H;
-        FF_TRY(launch_w16_fmt<2>(shared->format, q, smf, std::min<unsigned>(blocks, (q.total_units + 7u) & ~7u), stream));
-      }
-    }
+    if (shared)
+      FF_TRY(shared_expert_w16(shared, args->x, R, H, args->swiglu, args->swiglu_limit, s + l.sh_act, args->shared_out,
+                               (stages & 2 ? 1 : 0) | (stages & 8 ? 2 : 0), stream_));
     return 0;
   }
   GemmParams p{};

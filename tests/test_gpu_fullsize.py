@@ -212,11 +212,14 @@ def _cpubase_contributions(table, x_bits, ids, wts, shared_e, boundary):
 
 
 @pytest.mark.parametrize("rows", [8, 33])
-def test_decode_fp8_full_width_beyond_the_lds_row_budget(rows):
-    """Hidden 7168 with 8 and 33 rows: a block's LDS holds 4 token rows at this width, so the shared expert is served in
-    several row groups and a popular expert in more than one. Every contribution and shared row against the CPU port
-    (Lane16), three of them also against the scalar oracle."""
+def test_decode_fp8_full_width_beyond_the_lds_row_budget(rows, monkeypatch):
+    """Hidden 7168 with 8 and 33 rows on the streaming kernels: a block's LDS holds 4 token rows at this width, so the
+    shared expert is served in several row groups and a popular expert in more than one. Every contribution and shared
+    row against the CPU port (Lane16), three of them also against the scalar oracle. (The rule that hands the shared
+    expert of larger batches to the matrix-core kernels is switched off here and checked end to end below.)"""
     experts, top_k = 6, 4
+    monkeypatch.setenv("FFMOE_DECODE_COHORT_ROWS", "0")
+    monkeypatch.setenv("FFMOE_DECODE_SHARED_COHORT_ROWS", "0")
     table = make_table_on_device(capi.FMT_FP8_BLOCK128, experts + 1, H, I, 111)
     sh = table.shared_struct(experts)
     table.experts = experts
@@ -262,6 +265,20 @@ def test_decode_fp8_full_width_beyond_the_lds_row_budget(rows):
         ge, ue, de = effective_weights(table, int(ids[r, c]))
         want = orc.expert_ffn(xb[r], ge, ue, de, float(wt[r, c]), orc.TWICE, 0.0, orc.AFTER_DOWN_BF16, orc.LANE8, orc.SILU_DIV)
         assert_close_bf16(got_c[r, c][None, :], want[None, :], "contribution (%d, %d) vs the scalar oracle" % (r, c), max_ulp=4)
+    # the default dispatch of the same batch (from 16 rows the shared expert, from 32 rows the whole batch on the matrix
+    # cores): same bars end to end
+    monkeypatch.delenv("FFMOE_DECODE_COHORT_ROWS")
+    monkeypatch.delenv("FFMOE_DECODE_SHARED_COHORT_ROWS")
+    op.contributions.zero_(); op.shared_out.zero_()
+    c2, s2 = op.contribute(x.cuda(), ids.cuda(), wt.cuda())
+    torch.cuda.synchronize()
+    if rows < 16:
+        assert np.array_equal(bits(c2), got_c) and np.array_equal(bits(s2), got_s), "small batches stay on the streaming kernels"
+    # on the matrix cores the two stages compose as in test_prefill_w16_full_width (each stage inside its bar there): the
+    # relative-L2 bar on the tensor, element-wise a loose bound for cancelled outputs
+    loose = 16 if rows >= 32 else 4
+    assert_close_bf16(bits(c2), want_c, "contributions of the default dispatch vs the CPU port, end to end", max_ulp=loose)
+    assert_close_bf16(bits(s2), want_s, "shared_out of the default dispatch vs the CPU port, end to end", max_ulp=16 if rows >= 16 else 4)
 
 
 def test_decode_nvfp4_full_width_batched():
@@ -357,3 +374,45 @@ def test_c3_token_through_native_moe_256_experts_8_groups():
         torch.cuda.synchronize()
         assert np.array_equal(other.ids.cpu().numpy(), oi)
         assert np.array_equal(y2, y), name
+
+
+def test_decode_fp8_full_width_64_rows_on_the_cohort_path(monkeypatch):
+    """64 rows at hidden 7168: ffmoe_decode_contribute hands the whole batch to the matrix-core cohort kernels (every expert
+    streamed once, the shared expert as one 64-row group). Same effective weights and BF16 boundaries as the streaming
+    kernels: contributions and shared rows against the CPU port end to end, and bit-identical rows whether 64 or 48 rows
+    are in the batch (rows do not depend on their cohort on this path either)."""
+    experts, top_k, rows = 6, 4, 64
+    monkeypatch.delenv("FFMOE_DECODE_COHORT_ROWS", raising=False)
+    monkeypatch.delenv("FFMOE_DECODE_SHARED_COHORT_ROWS", raising=False)
+    monkeypatch.delenv("FFMOE_PREFILL_MF", raising=False)
+    table = make_table_on_device(capi.FMT_FP8_BLOCK128, experts + 1, H, I, 141)
+    sh = table.shared_struct(experts)
+    table.experts = experts
+    g = synth.generator(142)
+    x = synth.normal((rows, H), 1.0, 143).to(torch.bfloat16)
+    ids = torch.stack([torch.randperm(experts, generator=g)[:top_k] for _ in range(rows)]).to(torch.int32)
+    wt = torch.rand((rows, top_k), generator=g) * 0.5 + 0.05
+    op = ops.DecodeOps(table, sh, rows, top_k, capi.ACT_BF16, capi.SWIGLU_TWICE, 0.0, capi.WEIGHT_AFTER_DOWN_BF16, weights_f32=True)
+    op.contributions.zero_()
+    print("full-width decode rows=64 (cohort path)", flush=True)
+    contrib, shared_out = op.contribute(x.cuda(), ids.cuda(), wt.cuda())
+    torch.cuda.synchronize()
+    assert int(op.done.sum().item()) == rows * top_k
+    got_c, got_s = bits(contrib).copy(), bits(shared_out).copy()
+    want_c, want_s, _ = _cpubase_contributions(table, bits(x), ids.numpy(), wt.numpy(), experts, orc.AFTER_DOWN_BF16)
+    # the stages of this path are held to their bars in test_prefill_w16_full_width; end to end the relative-L2 bar on the
+    # tensor and a loose element-wise bound for cancelled outputs, as there
+    r_, worst_ = assert_close_bf16(got_c, want_c, "contributions vs the CPU port, end to end", max_ulp=16)
+    print("contributions end to end: relative L2 %.2e, worst %.1f steps" % (r_, worst_), flush=True)
+    assert_close_bf16(got_s, want_s, "shared_out vs the CPU port, end to end", max_ulp=16)
+    part = ops.DecodeOps(table, sh, 48, top_k, capi.ACT_BF16, capi.SWIGLU_TWICE, 0.0, capi.WEIGHT_AFTER_DOWN_BF16, weights_f32=True)
+    c2, s2 = part.contribute(x[8:56].contiguous().cuda(), ids[8:56].contiguous().cuda(), wt[8:56].contiguous().cuda())
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(c2), got_c[8:56]) and np.array_equal(bits(s2), got_s[8:56]), "rows depend on their cohort"
+    # the streaming kernels on the same batch (rules switched off): within the same bars of the cohort path's result
+    monkeypatch.setenv("FFMOE_DECODE_COHORT_ROWS", "0")
+    monkeypatch.setenv("FFMOE_DECODE_SHARED_COHORT_ROWS", "0")
+    c3, s3 = op.contribute(x.cuda(), ids.cuda(), wt.cuda())
+    torch.cuda.synchronize()
+    assert_close_bf16(bits(c3), want_c, "streaming kernels vs the CPU port, end to end", max_ulp=16)
+    assert_close_bf16(bits(s3), want_s, "streaming kernels, shared_out", max_ulp=16)
