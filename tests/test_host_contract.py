@@ -59,7 +59,11 @@ def test_decode_contract_violations_are_reported_before_launch():
     assert call(x=None) == capi.ERR_NULL
     assert call(x=(1 << 20) + 8) == capi.ERR_ALIGN
     assert call(top_k=40) == capi.ERR_SHAPE
-    assert call(rows=4096) == capi.ERR_SHAPE and "prefill" in capi.last_error()
+    # block-FP8 batches of 32 rows and more go to the cohort kernels, which take any row count (here: too small an arena);
+    # the streaming kernels of the other formats keep their limit of 4096 assignments per call
+    assert call(rows=4096) == capi.ERR_SCRATCH
+    nv_rows = capi.ExpertTable(capi.FMT_NVFP4, 64, 2048, 1408, 16 << 20, None, 32 << 20)
+    assert call(t=nv_rows, rows=4096, scratch_bytes=1 << 30, contributions=1 << 40) == capi.ERR_SHAPE and "prefill" in capi.last_error()
     assert call(scratch_bytes=16) == capi.ERR_SCRATCH
     assert call(contributions=1 << 20) == capi.ERR_OVERLAP
     assert call(act_mode=2) == capi.ERR_UNSUPPORTED
