@@ -569,6 +569,26 @@ def linear_main(args, torch, capi, ops, synth):
             us = e0.elapsed_time(e1) * 1e3 / (reps * ring)
             nbytes = n * k + 4 * ((n + 127) // 128) * ((k + 127) // 128) + 2 * m * (k + n)
             rows["k%d_n%d_m%d" % (k, n, m)] = {"us": us, "gbps": nbytes / us / 1e3, "hbm_frac": nbytes / us / 1e3 / HBM_PEAK_GBPS}
+        # steady state of M = 1: eight linears of the ring per launch (ffmoe_linear_fp8_block_batch), the start-up of a
+        # launch paid once per batch; the ring is walked in three batches per repetition
+        for m in (1, 4):
+            x = synth.normal((m, k), 1.0, args.seed + m, device=dev, dtype=torch.bfloat16)
+            ys = [torch.empty((m, n), dtype=torch.bfloat16, device=dev) for _ in range(ring)]
+            batches = [ops.Fp8Ops.linear_batch_items(ws[b:b + 8], [x] * 8, ys[b:b + 8]) for b in range(0, ring, 8)]
+            for it in batches:
+                ops.Fp8Ops.linear_batch(it, m, n, k)
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            reps = max(1, args.steps // ring)
+            e0.record()
+            for _ in range(reps):
+                for it in batches:
+                    ops.Fp8Ops.linear_batch(it, m, n, k)
+            e1.record()
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) * 1e3 / (reps * ring)
+            nbytes = n * k + 4 * ((n + 127) // 128) * ((k + 127) // 128) + 2 * m * (k + n)
+            rows["k%d_n%d_m%d_batch8" % (k, n, m)] = {"us_per_linear": us, "gbps": nbytes / us / 1e3, "hbm_frac": nbytes / us / 1e3 / HBM_PEAK_GBPS}
     head = rows["k7168_n2048_m16"]
     out = {"metric": "fp8_block_linear_us", "value": head["us"], "unit": "us/call", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
            "ms_per_step": head["us"] * 1e-3, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,

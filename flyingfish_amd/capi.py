@@ -23,7 +23,7 @@ EXPORTS = [
     "ffmoe_last_error", "ffmoe_version",
     "ffmoe_route_logits_bf16", "ffmoe_route_logits_f32", "ffmoe_route_topk", "ffmoe_route_topk_noaux", "ffmoe_route_noaux_decode", "ffmoe_route_decode", "ffmoe_slot_publish", "ffmoe_route_mask",
     "ffmoe_decode_scratch_bytes", "ffmoe_decode_contribute", "ffmoe_decode_static_scratch_bytes", "ffmoe_decode_contribute_static", "ffmoe_decode_contribute_stage", "ffmoe_decode_finish", "ffmoe_decode_contribute_from_logits", "ffmoe_decode_token_layer", "ffmoe_decode_token_forward", "ffmoe_decode_token_forward_stage", "ffmoe_decode_contribute_form", "ffmoe_e8m0_scratch_bytes", "ffmoe_decode_contribute_e8m0", "ffmoe_act_quant_e8m0",
-    "ffmoe_quant_fp8_f32_128", "ffmoe_linear_fp8_block_w8a8", "ffmoe_linear_fp8_block", "ffmoe_linear_nvfp4",
+    "ffmoe_quant_fp8_f32_128", "ffmoe_linear_fp8_block_w8a8", "ffmoe_linear_fp8_block", "ffmoe_linear_fp8_block_batch", "ffmoe_linear_nvfp4",
     "ffmoe_gemm_skinny_bf16", "ffmoe_swiglu",
     "ffmoe_shared_scale", "ffmoe_combine",
     "ffmoe_combine_residual", "ffmoe_prefill_scratch_bytes", "ffmoe_prefill_contribute", "ffmoe_prefill_contribute_stage",
@@ -94,6 +94,7 @@ def lib():
         L.ffmoe_quant_fp8_f32_128.argtypes = [P, P, P, I, I, P]
         L.ffmoe_linear_fp8_block_w8a8.argtypes = [P, P, P, P, P, I, I, I, P]
         L.ffmoe_linear_fp8_block.argtypes = [P, P, P, P, I, I, I, I, P, U64, P]
+        L.ffmoe_linear_fp8_block_batch.argtypes = [P, I, I, I, I, P]
         L.ffmoe_linear_nvfp4.argtypes = [P, P, P, P, P, I, I, I, P]
         L.ffmoe_gemm_skinny_bf16.argtypes = [P, P, P, I, I, I, P]
         L.ffmoe_swiglu.argtypes = [P, P, P, I, I, I, F, P]

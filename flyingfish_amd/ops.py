@@ -533,6 +533,17 @@ class Fp8Ops:
         return y
 
     @staticmethod
+    def linear_batch_items(weights, xs, ys):
+        """Device descriptor array for linear_batch: weights = [(codes, scales), ...], xs / ys = matching BF16 tensors."""
+        rows = [[c.data_ptr(), s.data_ptr(), x.data_ptr(), y.data_ptr()] for (c, s), x, y in zip(weights, xs, ys)]
+        return torch.tensor(rows, dtype=torch.int64).to(xs[0].device)
+
+    @staticmethod
+    def linear_batch(items, m, n, k):
+        """All items (descriptor array from linear_batch_items) in one launch; m <= 4 activation rows each."""
+        capi.check(capi.lib().ffmoe_linear_fp8_block_batch(_ptr(items), items.shape[0], m, n, k, _stream()))
+
+    @staticmethod
     def linear_w8a8(w_codes, w_scales, x_codes, x_scales, out=None):
         n, k = w_codes.shape
         m = x_codes.shape[0]

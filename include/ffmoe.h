@@ -358,6 +358,17 @@ int ffmoe_linear_fp8_block_w8a8(const void* w_codes, const float* w_scales, cons
 int ffmoe_linear_fp8_block(const void* w_codes, const float* w_scales, const void* x, void* y,
                            int m, int n, int k, int act_mode, void* scratch, uint64_t scratch_bytes, void* stream);
 
+/* Several independent block-FP8 skinny linears of one shape in ONE launch, W8A16 arithmetic (act_mode FFMOE_ACT_BF16 of
+ * ffmoe_linear_fp8_block): the projections a decoder layer applies side by side (the reference plans them one
+ * Fp8BlockPlan each, src/linear_plan.rs, src/backend/cuda/linear.rs:571-660, and launches fp8_gemv_bf16 /
+ * fp8_skinny_bf16_mM per projection, kernels/fp8_linear.cu:353-511; it has no batched launch). A 14.7 MB matrix streams for
+ * about 2.3 us on this GPU against 2 - 3 us of launch start-up, so single calls cannot pass ~40 % of the HBM rate;
+ * a batch pays the start-up once. `items` is a DEVICE array of `count` descriptors (device addresses of codes [n,k],
+ * f32 block scales, x [m,k] BF16, y [m,n] BF16), caller-owned like a slot table; 1 <= m <= 4. Every item's y is
+ * bit-identical to its own ffmoe_linear_fp8_block call. Items must not alias each other's outputs. */
+typedef struct ffmoe_linear_item { uint64_t w_codes, w_scales, x, y; } ffmoe_linear_item;
+int ffmoe_linear_fp8_block_batch(const ffmoe_linear_item* items, int count, int m, int n, int k, void* stream);
+
 /* Replaces NvFp4Ops::gemm (linear.rs:488-551; kernels/nvfp4_linear.cu:50-252): W4A16,
  * w = bf16(e2m1 * (e4m3(scale) * global)). global_scale is a device pointer to one f32. k % 16 == 0. Up to 16 rows
  * run the direct kernel (the reference's host mirror order); more rows with k % 128 == 0 and n % 16 == 0 the BF16

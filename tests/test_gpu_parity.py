@@ -853,3 +853,25 @@ def test_token_forward_two_launches_equal_the_separate_launches(fmt, hidden, int
         for a, b in zip(got[False], got[True]):
             for name, u, v in zip(("ids", "weights", "y"), a, b):
                 assert np.array_equal(u, v), "%s, combine mode %d" % (name, mode)
+
+
+@pytest.mark.parametrize("m", [1, 3, 4])
+@pytest.mark.parametrize("k,n,count", [(7168, 200, 5), (2048, 384, 3), (640, 72, 9)])
+def test_linear_fp8_block_batch_equals_single_calls(m, k, n, count):
+    """ffmoe_linear_fp8_block_batch: several linears of one shape in one launch, every item bit-identical to its own
+    ffmoe_linear_fp8_block call (whose parity with the oracle test_linear_fp8_block_w8a16 holds)."""
+    weights, xs, ys, want = [], [], [], []
+    for i in range(count):
+        c, sc = synth.quant_fp8_block(synth.normal((n, k), 0.02, 700 + 10 * i + m))
+        weights.append((c.to(DEV), sc.to(DEV)))
+        xs.append(rand_bf16((m, k), 1.0, 800 + 10 * i + m).to(DEV))
+        ys.append(torch.zeros((m, n), dtype=torch.bfloat16, device=DEV))
+        want.append(bits(Fp8Ops.linear(weights[-1][0], weights[-1][1], xs[-1])).copy())
+    items = Fp8Ops.linear_batch_items(weights, xs, ys)
+    print("batched linear m=%d k=%d n=%d count=%d" % (m, k, n, count), flush=True)
+    Fp8Ops.linear_batch(items, m, n, k)
+    torch.cuda.synchronize()
+    for i in range(count):
+        assert np.array_equal(bits(ys[i]), want[i]), "item %d differs from its single call" % i
+    with pytest.raises(capi.FfmoeError):
+        Fp8Ops.linear_batch(items, 5, n, k)  # more than 4 rows per item: single calls (matrix-core path)
