@@ -12,7 +12,7 @@ LIB_PATH = os.path.join(_HERE, "libffmoe.so")
 FMT_FP8_BLOCK128, FMT_NVFP4, FMT_BF16, FMT_FP8_CHANNEL, FMT_E2M1_E8M0, FMT_E4M3_E8M0_32 = 0, 1, 2, 3, 4, 5
 FORM_LANE16, FORM_LANE8 = 0, 1
 ACT_BF16, ACT_FP8_BLOCK128, ACT_E4M3_E8M0_32, ACT_E4M3_E8M0_32_F32 = 0, 1, 2, 3
-SWIGLU_TWICE, SWIGLU_ONCE, SWIGLU_CLAMPED_TWICE, SWIGLU_CLAMPED_ONCE = 0, 1, 2, 3
+SWIGLU_TWICE, SWIGLU_ONCE, SWIGLU_CLAMPED_TWICE, SWIGLU_CLAMPED_ONCE, SWIGLU_GELU_TWICE = 0, 1, 2, 3, 4
 WEIGHT_AFTER_DOWN_BF16, WEIGHT_BEFORE_CONTRIBUTION_BF16, WEIGHT_BEFORE_DOWN_F32 = 0, 1, 2
 SCORE_SOFTMAX, SCORE_SIGMOID = 0, 1
 NOAUX_SIGMOID, NOAUX_SQRTSOFTPLUS = 0, 1

@@ -134,6 +134,30 @@ __device__ __forceinline__ float sigmoid1(float l) {
   return __fdiv_rn(1.0f, __fadd_rn(1.0f, det_expf(-l)));
 }
 
+// tanhf from the same operations as det_expf: odd Taylor polynomial through x^11 below 0.3, 1 - 2 / (exp(2|x|) + 1)
+// above, +-1 beyond 9; within 3 ulp of the exact function.
+__device__ __forceinline__ float det_tanhf(float x) {
+  const float a = fabsf(x);
+  if (a < 0.3f) {
+    const float z = __fmul_rn(x, x);
+    float p = -8.8632355e-3f;
+    p = __fmaf_rn(p, z, 2.1869488e-2f);
+    p = __fmaf_rn(p, z, -5.3968254e-2f);
+    p = __fmaf_rn(p, z, 1.3333334e-1f);
+    p = __fmaf_rn(p, z, -3.3333334e-1f);
+    return __fmaf_rn(__fmul_rn(x, z), p, x);
+  }
+  float t = 1.0f;
+  if (!(a > 9.0f)) t = __fsub_rn(1.0f, __fdiv_rn(2.0f, __fadd_rn(det_expf(__fmul_rn(2.0f, a)), 1.0f)));
+  return copysignf(t, x);
+}
+// tanh form of GELU with one rounding per operation (src/cpu/expert_ffn.rs:87-91 of the reference)
+__device__ __forceinline__ float gelu_tanh(float g) {
+  const float cube = __fmul_rn(__fmul_rn(g, g), g);
+  const float inner = __fmul_rn(0.7978846f, __fadd_rn(g, __fmul_rn(0.044715f, cube)));
+  return __fmul_rn(__fmul_rn(0.5f, g), __fadd_rn(1.0f, det_tanhf(inner)));
+}
+
 // SwiGLU with the BF16 rounding boundary selected by `mode` (FFMOE_SWIGLU_*): returns BF16 bits.
 // SiLU = g / (1 + exp(-g)) as in the production decode kernels of the reference.
 // SiLU as x * sigmoid(x) with the two-branch sigmoid of the reference's dense activation kernels
@@ -155,12 +179,41 @@ __device__ __forceinline__ uint16_t swiglu_bf16_two_branch(float g, float u, int
 }
 
 __device__ __forceinline__ uint16_t swiglu_bf16(float g, float u, int mode, float limit) {
-  if (mode >= 2) {
-    g = fminf(g, limit);
-    u = fminf(fmaxf(u, -limit), limit);
+  // mode 4 (FFMOE_SWIGLU_GELU_TWICE) is bf16(bf16(gelu_tanh(g)) * u) without a clamp; it is written out here so that it shares
+  // the one expf of the SiLU forms
+  const bool gelu = mode == 4;
+  float inner = 0.0f, arg;
+  if (gelu) {
+    const float cube = __fmul_rn(__fmul_rn(g, g), g);
+    inner = __fmul_rn(0.7978846f, __fadd_rn(g, __fmul_rn(0.044715f, cube)));
+    arg = __fmul_rn(2.0f, fabsf(inner));
+  } else {
+    if (mode >= 2) {
+      g = fminf(g, limit);
+      u = fminf(fmaxf(u, -limit), limit);
+    }
+    arg = -g;
   }
-  const float act = __fdiv_rn(g, __fadd_rn(1.0f, det_expf(-g)));
-  const float prod = (mode == 0 || mode == 2) ? __fmul_rn(bround(act), u) : __fmul_rn(act, u);
+  const float den = __fadd_rn(det_expf(arg), 1.0f);
+  float act;
+  if (gelu) {
+    const float a = fabsf(inner);
+    float t = a > 9.0f ? 1.0f : __fsub_rn(1.0f, __fdiv_rn(2.0f, den));
+    t = copysignf(t, inner);
+    if (a < 0.3f) {
+      const float z = __fmul_rn(inner, inner);
+      float q = -8.8632355e-3f;
+      q = __fmaf_rn(q, z, 2.1869488e-2f);
+      q = __fmaf_rn(q, z, -5.3968254e-2f);
+      q = __fmaf_rn(q, z, 1.3333334e-1f);
+      q = __fmaf_rn(q, z, -3.3333334e-1f);
+      t = __fmaf_rn(__fmul_rn(inner, z), q, inner);
+    }
+    act = __fmul_rn(__fmul_rn(0.5f, g), __fadd_rn(1.0f, t));
+  } else {
+    act = __fdiv_rn(g, den);
+  }
+  const float prod = (mode == 0 || mode == 2 || gelu) ? __fmul_rn(bround(act), u) : __fmul_rn(act, u);
   return f32_to_bf16(prod);
 }
 

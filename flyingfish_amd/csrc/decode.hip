@@ -169,8 +169,8 @@ static int decode_impl(const ffmoe_expert_table* table, const ffmoe_shared_exper
              "hidden=%d inter=%d must be positive multiples of %d for this format", H, I, gran);
   FF_REQUIRE(args->act_mode == FFMOE_ACT_BF16, FFMOE_ERR_UNSUPPORTED,
              "decode act_mode %d is not implemented (only FFMOE_ACT_BF16)", args->act_mode);
-  FF_REQUIRE(args->swiglu >= 0 && args->swiglu <= 3, FFMOE_ERR_UNSUPPORTED, "unknown SwiGLU mode %d", args->swiglu);
-  if (args->swiglu >= 2)
+  FF_REQUIRE(args->swiglu >= 0 && args->swiglu <= FFMOE_SWIGLU_GELU_TWICE, FFMOE_ERR_UNSUPPORTED, "unknown SwiGLU mode %d", args->swiglu);
+  if (args->swiglu == FFMOE_SWIGLU_CLAMPED_TWICE || args->swiglu == FFMOE_SWIGLU_CLAMPED_ONCE)
     FF_REQUIRE(args->swiglu_limit > 0.0f && args->swiglu_limit < INFINITY, FFMOE_ERR_SHAPE, "invalid SwiGLU limit %g",
                (double)args->swiglu_limit);
   FF_REQUIRE(args->routed_weight == 0 || args->routed_weight == 1, FFMOE_ERR_UNSUPPORTED, "unknown routed-weight boundary %d",

@@ -118,6 +118,7 @@ __device__ __forceinline__ float form_dot(const uint8_t* xs, const FormRow<F>& r
 
 // SwiGLU with the reference's SiLU per form (see the file comment)
 __device__ __forceinline__ uint16_t form_swiglu(float g, float u, int mode, float limit, bool reciprocal) {
+  if (mode == FFMOE_SWIGLU_GELU_TWICE) return f32_to_bf16(__fmul_rn(bround(gelu_tanh(g)), u));
   if (mode >= 2) {
     g = fminf(g, limit);
     u = fminf(fmaxf(u, -limit), limit);

@@ -470,8 +470,8 @@ extern "C" __attribute__((visibility("default"))) int ffmoe_gemm_skinny_bf16(con
 
 extern "C" __attribute__((visibility("default"))) int ffmoe_swiglu(const void* gate, const void* up, void* y, int rows, int width, int mode, float limit, void* stream) {
   FF_REQUIRE(rows >= 1 && width >= 8 && width % 8 == 0, FFMOE_ERR_SHAPE, "swiglu rows=%d width=%d (width must be a positive multiple of 8)", rows, width);
-  FF_REQUIRE(mode >= 0 && mode <= 3, FFMOE_ERR_UNSUPPORTED, "unknown SwiGLU mode %d", mode);
-  if (mode >= 2) FF_REQUIRE(limit > 0.0f && limit < INFINITY, FFMOE_ERR_SHAPE, "invalid SwiGLU limit %g", (double)limit);
+  FF_REQUIRE(mode >= 0 && mode <= FFMOE_SWIGLU_GELU_TWICE, FFMOE_ERR_UNSUPPORTED, "unknown SwiGLU mode %d", mode);
+  if (mode == FFMOE_SWIGLU_CLAMPED_TWICE || mode == FFMOE_SWIGLU_CLAMPED_ONCE) FF_REQUIRE(limit > 0.0f && limit < INFINITY, FFMOE_ERR_SHAPE, "invalid SwiGLU limit %g", (double)limit);
   FF_PTR16(gate); FF_PTR16(up); FF_PTR16(y);
   const size_t bytes = size_t(rows) * width * 2;
   FF_NO_OVERLAP(y, bytes, gate, bytes);

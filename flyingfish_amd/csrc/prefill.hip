@@ -379,8 +379,10 @@ int prefill_impl(const ffmoe_expert_table* table, const ffmoe_prefill* args, int
   else
     FF_REQUIRE(H >= 128 && H % 128 == 0 && I >= 128 && I % 128 == 0, FFMOE_ERR_SHAPE, "hidden=%d and inter=%d must be multiples of 128", H, I);
   if (a16 && table->format == FFMOE_FMT_NVFP4) FF_PTR4(table->global_scales);
-  FF_REQUIRE(args->swiglu >= 0 && args->swiglu <= 3, FFMOE_ERR_UNSUPPORTED, "unknown SwiGLU mode %d", args->swiglu);
-  if (args->swiglu >= 2) FF_REQUIRE(args->swiglu_limit > 0.0f && args->swiglu_limit < INFINITY, FFMOE_ERR_SHAPE, "invalid SwiGLU limit %g", (double)args->swiglu_limit);
+  FF_REQUIRE(args->swiglu >= 0 && args->swiglu <= FFMOE_SWIGLU_GELU_TWICE, FFMOE_ERR_UNSUPPORTED, "unknown SwiGLU mode %d", args->swiglu);
+  FF_REQUIRE(args->swiglu != FFMOE_SWIGLU_GELU_TWICE || a16, FFMOE_ERR_UNSUPPORTED,
+             "FFMOE_SWIGLU_GELU_TWICE needs act_mode FFMOE_ACT_BF16 (the FP8-activation kernels implement the SiLU forms only)");
+  if (args->swiglu == FFMOE_SWIGLU_CLAMPED_TWICE || args->swiglu == FFMOE_SWIGLU_CLAMPED_ONCE) FF_REQUIRE(args->swiglu_limit > 0.0f && args->swiglu_limit < INFINITY, FFMOE_ERR_SHAPE, "invalid SwiGLU limit %g", (double)args->swiglu_limit);
   if (!mx)
     FF_REQUIRE(args->routed_weight == FFMOE_WEIGHT_AFTER_DOWN_BF16 || args->routed_weight == FFMOE_WEIGHT_BEFORE_CONTRIBUTION_BF16,
                FFMOE_ERR_UNSUPPORTED, "unknown routed_weight %d", args->routed_weight);

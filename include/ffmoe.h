@@ -61,6 +61,12 @@ extern "C" {
 #define FFMOE_SWIGLU_ONCE           1  /* a = bf16(silu(g) * u) */
 #define FFMOE_SWIGLU_CLAMPED_TWICE  2  /* g = min(g,L), u = clamp(u,+-L), then TWICE */
 #define FFMOE_SWIGLU_CLAMPED_ONCE   3
+/* a = bf16(bf16(gelu(g)) * u), gelu(g) = 0.5 g (1 + tanh(0.7978846 (g + 0.044715 g^3))) in FP32 with one rounding per
+   operation and no clamp (SwigluRounding::GeluTwice, src/cpu/expert_ffn.rs:65,87-91,110-113; kernels/act.cu:16-22).
+   The reference takes tanh from libm or the CUDA math library; this library uses one fixed FP32 tanh within 3 ulp of
+   the exact function. Not available with FFMOE_ACT_FP8_BLOCK128 (the reference binds it to BF16 experts only,
+   src/backend/cuda/engine_diffusion.rs:1135-1141). */
+#define FFMOE_SWIGLU_GELU_TWICE     4
 
 /* routed-weight boundary (src/model_spec.rs:70-75) */
 #define FFMOE_WEIGHT_AFTER_DOWN_BF16          0  /* c = bf16(bf16(d) * w) */

@@ -15,7 +15,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "libffmoe_oracle.so")
 _BASE_PATH = os.path.join(_HERE, "libffmoe_cpubase.so")
 
-TWICE, ONCE, CLAMPED_TWICE, CLAMPED_ONCE = 0, 1, 2, 3
+TWICE, ONCE, CLAMPED_TWICE, CLAMPED_ONCE, GELU_TWICE = 0, 1, 2, 3, 4
 AFTER_DOWN_BF16, BEFORE_CONTRIBUTION_BF16 = 0, 1
 LANE16, LANE8, F64 = 0, 1, 2
 SILU_DIV, SILU_RCP, SILU_SIGMOID2 = 0, 1, 2
@@ -99,6 +99,21 @@ def expf(x):
     x = _c(x, np.float32)
     out = np.empty_like(x)
     lib().orc_expf_array(_p(x), _p(out), ctypes.c_long(x.size))
+    return out
+
+
+def tanhf(x):
+    x = _c(x, np.float32)
+    out = np.empty_like(x)
+    lib().orc_tanhf_array(_p(x), _p(out), ctypes.c_long(x.size))
+    return out
+
+
+def gelu_tanh(x):
+    """0.5 g (1 + tanh(0.7978846 (g + 0.044715 g^3))) in FP32, one rounding per operation."""
+    x = _c(x, np.float32)
+    out = np.empty_like(x)
+    lib().orc_gelu_tanh_array(_p(x), _p(out), ctypes.c_long(x.size))
     return out
 
 

@@ -11,6 +11,8 @@
 //   * codecs, BF16 rounding, effective weights ............ pinned (exhaustive closed forms, spot values)
 //   * noaux / sigmoid / softmax top-k ...................... pinned (golden router vectors, brute force)
 //   * SwiGLU boundaries ..................................... pinned (golden BF16 bit patterns)
+//   * tanh-GELU with two roundings .......................... pinned up to the last bits of tanh (the same FP32 operation
+//     chain with a correctly rounded tanh, every BF16 gate value; the reference pins no tanh and holds no vectors)
 //   * expert FFN on BF16 / per-channel FP8 weights .......... pinned (FP64 boundary oracle at 0 BF16 steps)
 //   * W8A8 quantizer + block dot ............................ pinned (FP64 gamma bound, wrong-cell mutant)
 //   * NVFP4 / BF16-scale skinny linear orders ............... pinned (closed-form dequant table, FP64 bound)
@@ -20,7 +22,7 @@
 //   * combine variants ...................................... pinned (order-spread constants of the fixture)
 //   * expert FFN composed over 128x128-f32 block scales or
 //     NVFP4 weights, grouped routing with n_group > 1,
-//     FP32-logit dot order, last-bit behaviour of expf ....... parity unpinned (no reference code or vectors)
+//     FP32-logit dot order, last-bit behaviour of expf / tanhf parity unpinned (no reference code or vectors)
 #include <cmath>
 #include <cstdint>
 #include <cstring>
@@ -160,6 +162,25 @@ inline float det_log1pf_unit(float u) {
 
 inline float sigmoid1(float l) { return 1.0f / (1.0f + det_expf(-l)); }  // moe_route.cu:255,330
 
+// tanhf from the same operations: the odd Taylor polynomial through x^11 below 0.3 (truncation < 2e-9 relative),
+// 1 - 2 / (exp(2|x|) + 1) above, +-1 beyond 9. The reference takes tanh from libm (src/cpu/expert_ffn.rs:91) or the
+// CUDA math library (kernels/act.cu:21) and pins neither; the tests hold this one to a few ulp of the exact function.
+inline float det_tanhf(float x) {
+  const float a = std::fabs(x);
+  if (a < 0.3f) {
+    const float z = x * x;
+    float p = -8.8632355e-3f;             // -1382/155925
+    p = std::fmaf(p, z, 2.1869488e-2f);   //  62/2835
+    p = std::fmaf(p, z, -5.3968254e-2f);  // -17/315
+    p = std::fmaf(p, z, 1.3333334e-1f);   //  2/15
+    p = std::fmaf(p, z, -3.3333334e-1f);  // -1/3
+    return std::fmaf(x * z, p, x);
+  }
+  float t = 1.0f;
+  if (!(a > 9.0f)) t = 1.0f - 2.0f / (det_expf(2.0f * a) + 1.0f);
+  return std::copysign(t, x);
+}
+
 // moe_route.cu:332-335 (non-literal form) / moe/reference.rs:73-76
 inline float sqrt_softplus(float l) {
   const float softplus = std::fmax(l, 0.0f) + det_log1pf_unit(det_expf(-std::fabs(l)));
@@ -208,7 +229,7 @@ float dot_form(const float* x, const uint16_t* w, int n, int form) {
   return group_sum8(lanes);
 }
 
-enum Swiglu { TWICE = 0, ONCE = 1, CLAMPED_TWICE = 2, CLAMPED_ONCE = 3 };
+enum Swiglu { TWICE = 0, ONCE = 1, CLAMPED_TWICE = 2, CLAMPED_ONCE = 3, GELU_TWICE = 4 };
 enum Boundary { AFTER_DOWN_BF16 = 0, BEFORE_CONTRIBUTION_BF16 = 1 };
 
 // expert_ffn.rs:58-100 (silu_mul_value) followed by the BF16 store of :103-114.
@@ -223,8 +244,15 @@ inline float silu_kind(float g, int kind) {
   else { const float e = det_expf(g); s = e / (1.0f + e); }
   return g * s;
 }
+// tanh form of GELU, every operation rounded on its own (expert_ffn.rs:87-91; kernels/act.cu:18-22)
+inline float gelu_tanh(float g) {
+  const float cube = (g * g) * g;
+  const float inner = 0.7978846f * (g + 0.044715f * cube);
+  return (0.5f * g) * (1.0f + det_tanhf(inner));
+}
 inline uint16_t silu_mul_bits(uint16_t gate, uint16_t up, int rounding, float limit, int kind) {
   float g = bf16_f32(gate), u = bf16_f32(up);
+  if (rounding == GELU_TWICE) return bf16_rne(bround(gelu_tanh(g)) * u);  // expert_ffn.rs:110-113: no clamp, any form
   if (rounding == CLAMPED_TWICE || rounding == CLAMPED_ONCE) {
     g = std::fmin(g, limit);
     u = std::fmin(std::fmax(u, -limit), limit);
@@ -253,6 +281,8 @@ ORC_API uint16_t orc_bf16_rne(float v) { return bf16_rne(v); }
 ORC_API float orc_expf(float v) { return det_expf(v); }
 ORC_API float orc_log1pf_unit(float v) { return det_log1pf_unit(v); }
 ORC_API void orc_expf_array(const float* x, float* y, long n) { for (long i = 0; i < n; ++i) y[i] = det_expf(x[i]); }
+ORC_API void orc_tanhf_array(const float* x, float* y, long n) { for (long i = 0; i < n; ++i) y[i] = det_tanhf(x[i]); }
+ORC_API void orc_gelu_tanh_array(const float* x, float* y, long n) { for (long i = 0; i < n; ++i) y[i] = gelu_tanh(x[i]); }
 ORC_API void orc_bf16_rne_array(const float* x, uint16_t* y, long n) { for (long i = 0; i < n; ++i) y[i] = bf16_rne(x[i]); }
 
 // src/fp8.rs:138-140 with an f32 scale: bf16(decode(code) * scale).

@@ -51,11 +51,12 @@ def test_decode_fp8_per_channel_experts(rows, shared):
     (512, 256, 1, 2, capi.SWIGLU_TWICE, capi.WEIGHT_AFTER_DOWN_BF16),
     (1024, 384, 5, 3, capi.SWIGLU_ONCE, capi.WEIGHT_BEFORE_CONTRIBUTION_BF16),
     (776, 200, 3, 2, capi.SWIGLU_CLAMPED_TWICE, capi.WEIGHT_AFTER_DOWN_BF16),   # widths that are 8 mod 16: the Lane16 tail
+    (512, 256, 2, 2, capi.SWIGLU_GELU_TWICE, capi.WEIGHT_BEFORE_CONTRIBUTION_BF16),
 ])
 def test_reference_summation_orders_bit_exact(fmt, form, hidden, inter, rows, top_k, rounding, boundary):
     if fmt == capi.FMT_FP8_CHANNEL and (hidden % 16 or inter % 16):
         pytest.skip("per-channel FP8 rows are multiples of 16 codes")
-    experts, limit = 5, (0.05 if rounding >= 2 else 0.0)
+    experts, limit = 5, (0.05 if rounding in (capi.SWIGLU_CLAMPED_TWICE, capi.SWIGLU_CLAMPED_ONCE) else 0.0)
     table, ref, sh, x, ids, wt = _case(fmt, experts, hidden, inter, rows, top_k, 181 + form, True)
     active = torch.ones((rows, top_k), dtype=torch.int32)
     if rows > 1:
@@ -96,8 +97,8 @@ def test_reference_summation_orders_seeded_sweep(seed):
     experts = int(rng.integers(2, 9))
     top_k = int(rng.integers(1, min(6, experts) + 1))
     rows = int(rng.choice([1, 2, 4, 9]))
-    rounding = int(rng.integers(0, 4))
-    limit = float(rng.choice([0.05, 1.0])) if rounding >= 2 else 0.0
+    rounding = int(rng.integers(0, 5))
+    limit = float(rng.choice([0.05, 1.0])) if rounding in (2, 3) else 0.0
     boundary = int(rng.integers(0, 2))
     shared = bool(rng.integers(0, 2))
     print("fmt=%d form=%d hidden=%d inter=%d experts=%d top_k=%d rows=%d rounding=%d limit=%g boundary=%d shared=%d" %

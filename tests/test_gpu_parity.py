@@ -83,12 +83,25 @@ def test_device_swiglu_golden_bits():
     gt, ut = torch.from_numpy(g).to(torch.bfloat16).view(1, 16).to(DEV), torch.from_numpy(u).to(torch.bfloat16).view(1, 16).to(DEV)
     assert bits(swiglu(gt, ut, capi.SWIGLU_CLAMPED_TWICE, fx["limit"]))[0, :n].tolist() == fx["twice"]
     assert bits(swiglu(gt, ut, capi.SWIGLU_CLAMPED_ONCE, fx["limit"]))[0, :n].tolist() == fx["once"]
-    # dense random sweep against the oracle for all four modes
+    # dense random sweep against the oracle for all five modes
     gg, uu = rand_bf16((8, 4096), 3.0, 5), rand_bf16((8, 4096), 3.0, 6)
-    for mode in range(4):
+    for mode in range(5):
         got = bits(swiglu(gg.to(DEV), uu.to(DEV), mode, 2.5))
         want = orc.silu_mul(bits(gg), bits(uu), mode, 2.5, orc.SILU_DIV)
         assert np.array_equal(got, want), mode
+
+
+def test_device_gelu_twice_every_gate_value():
+    """tanh-GELU with two roundings: every BF16 gate pattern (NaNs aside) against the oracle, bit for bit."""
+    gate = np.arange(65536, dtype=np.uint32).astype(np.uint16)
+    keep = np.isfinite(orc.bf16_to_f32(gate))
+    gate = gate[keep][: (int(keep.sum()) // 8) * 8]
+    for seed, scale in ((1, 1.0), (2, 40.0)):
+        up = bits(rand_bf16((1, gate.size), scale, seed))[0]
+        gt = torch.from_numpy(gate.view(np.int16)).view(torch.bfloat16).view(1, -1).to(DEV)
+        ut = torch.from_numpy(up.view(np.int16)).view(torch.bfloat16).view(1, -1).to(DEV)
+        got = bits(swiglu(gt, ut, capi.SWIGLU_GELU_TWICE, 0.0))[0]
+        assert np.array_equal(got, orc.silu_mul(gate, up, orc.GELU_TWICE, 0.0, orc.SILU_DIV))
 
 
 # ------------------------------------------------------------------------------------------------
@@ -276,6 +289,13 @@ def test_decode_fp8_modes_and_active_mask():
     _run_decode(capi.FMT_FP8_BLOCK128, 6, 512, 384, 3, 2, 53, True, capi.SWIGLU_CLAMPED_ONCE, 0.1, capi.WEIGHT_AFTER_DOWN_BF16, True, False)
 
 
+@pytest.mark.parametrize("fmt", [capi.FMT_BF16, capi.FMT_FP8_BLOCK128, capi.FMT_NVFP4, capi.FMT_FP8_CHANNEL])
+@pytest.mark.parametrize("rows", [1, 5])
+def test_decode_gelu_twice(fmt, rows):
+    """SwigluRounding::GeluTwice of the reference (src/cpu/expert_ffn.rs:65,87-91,110-113) on the streaming decode kernels."""
+    _run_decode(fmt, 6, 512, 384, rows, 3, 58 + rows, True, capi.SWIGLU_GELU_TWICE, 0.0, capi.WEIGHT_BEFORE_CONTRIBUTION_BF16, True, False)
+
+
 @pytest.mark.parametrize("rows", [1, 6])
 def test_decode_nvfp4(rows):
     _run_decode(capi.FMT_NVFP4, 6, 1024, 512, rows, 3, 61, True)
@@ -304,8 +324,8 @@ def test_decode_seeded_shape_sweep(seed):
     experts = int(rng.integers(2, 13))
     top_k = int(rng.integers(1, min(8, experts) + 1))
     rows = int(rng.choice([1, 1, 2, 3, 4, 7, 9, 17]))
-    mode = int(rng.integers(0, 4))
-    limit = float(rng.choice([0.03, 0.1, 1.0])) if mode >= 2 else 0.0
+    mode = int(rng.integers(0, 5))
+    limit = float(rng.choice([0.03, 0.1, 1.0])) if mode in (2, 3) else 0.0
     boundary = int(rng.integers(0, 2))
     shared, weights_f32, with_active = bool(rng.integers(0, 2)), bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
     print("fmt=%d hidden=%d inter=%d experts=%d top_k=%d rows=%d mode=%d limit=%g boundary=%d shared=%d f32=%d mask=%d" %

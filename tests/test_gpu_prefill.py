@@ -207,7 +207,7 @@ def test_prefill_seeded_sweep(seed):
     hidden, inter = 128 * int(rng.integers(2, 6)), 128 * int(rng.integers(2, 6))
     skew = float(rng.choice([0.0, 1.1, 3.0]))
     mode = int(rng.integers(0, 4))
-    limit = float(rng.choice([0.5, 10.0])) if mode >= 2 else 0.0
+    limit = float(rng.choice([0.5, 10.0])) if mode in (2, 3) else 0.0
     boundary = int(rng.integers(0, 2))
     print("rows=%d top_k=%d experts=%d hidden=%d inter=%d skew=%g mode=%d limit=%g boundary=%d" %
           (rows, top_k, experts, hidden, inter, skew, mode, limit, boundary), flush=True)
@@ -231,6 +231,27 @@ def test_prefill_w16_matches_the_decode_oracle(fmt, rows, top_k, experts, hidden
     """act_mode FFMOE_ACT_BF16: the decode path's W*A16 arithmetic for whole cohorts on the BF16 matrix cores, every
     expert format. Stage-wise against the oracle of the decode path (the same effective weights; the matrix core's FP32
     accumulation against the reference's FP32 chains): activations, then the down stage on the device's activations."""
+    _check_prefill_w16(fmt, rows, top_k, experts, hidden, inter, skew, shared, capi.SWIGLU_CLAMPED_TWICE, 1.0)
+
+
+@pytest.mark.parametrize("fmt", [capi.FMT_BF16, capi.FMT_FP8_BLOCK128])
+def test_prefill_w16_gelu_twice(fmt):
+    """The tanh-GELU activation with two BF16 roundings on BF16 experts, routing weight before the contribution's
+    rounding: the configuration the reference binds it to (src/backend/cuda/engine_diffusion.rs:1135-1141)."""
+    _check_prefill_w16(fmt, 70, 3, 5, 256, 384, 1.5, True, capi.SWIGLU_GELU_TWICE, 0.0)
+
+
+def test_prefill_w8a8_rejects_gelu_twice():
+    from helpers import make_table
+    table, _ = make_table(capi.FMT_FP8_BLOCK128, 2, 128, 128, 5)
+    with pytest.raises(capi.FfmoeError) as e:
+        op = ops.PrefillOps(table, 4, 1, swiglu=capi.SWIGLU_GELU_TWICE, weights_f32=True)
+        ids = torch.zeros((4, 1), dtype=torch.int32, device="cuda")
+        op.contribute(torch.zeros((4, 128), dtype=torch.bfloat16, device="cuda"), ids, torch.ones((4, 1), device="cuda"))
+    assert e.value.code == capi.ERR_UNSUPPORTED
+
+
+def _check_prefill_w16(fmt, rows, top_k, experts, hidden, inter, skew, shared, mode, limit):
     from helpers import make_table
     if fmt == capi.FMT_FP8_BLOCK128 and (hidden % 128 or inter % 128):
         pytest.skip("128 x 128 block scales")
@@ -242,7 +263,7 @@ def test_prefill_w16_matches_the_decode_oracle(fmt, rows, top_k, experts, hidden
     if rows > 2:
         active[1, 0] = 0
     x = synth.normal((rows, hidden), 1.0, 920 + rows, dtype=torch.bfloat16)
-    mode, limit, boundary = capi.SWIGLU_CLAMPED_TWICE, 1.0, capi.WEIGHT_BEFORE_CONTRIBUTION_BF16
+    boundary = capi.WEIGHT_BEFORE_CONTRIBUTION_BF16
     op = ops.PrefillOps(table, rows, top_k, swiglu=mode, swiglu_limit=limit, routed_weight=boundary, weights_f32=True, shared=sh,
                         act_mode=capi.ACT_BF16)
     op.contributions.zero_()

@@ -117,6 +117,8 @@ def test_prefill_contract_violations_are_reported_before_launch():
     assert call(t=odd16, act_mode=capi.ACT_BF16) == capi.ERR_SHAPE  # multiples of 64 on the BF16 matrix cores
     assert call(top_k=40) == capi.ERR_SHAPE
     assert call(swiglu=2, swiglu_limit=0.0) == capi.ERR_SHAPE
+    assert call(swiglu=capi.SWIGLU_GELU_TWICE) == capi.ERR_UNSUPPORTED and "FFMOE_ACT_BF16" in capi.last_error()  # SiLU forms only on FP8 activations
+    assert call(swiglu=5, act_mode=capi.ACT_BF16) == capi.ERR_UNSUPPORTED
     assert call(routed_weight=capi.WEIGHT_BEFORE_DOWN_F32) == capi.ERR_UNSUPPORTED
     assert call(scratch_bytes=4096) == capi.ERR_SCRATCH
     assert call(scratch=(256 << 20) + 16) == capi.ERR_ALIGN

@@ -165,6 +165,59 @@ def test_expf_accuracy_random_and_edges():
     assert np.all(np.diff(orc.expf(xs)) >= 0)
 
 
+def test_tanh_accuracy_odd_and_saturating():
+    rng = np.random.default_rng(7)
+    x = np.concatenate([np.linspace(-12, 12, 400001), rng.normal(0, 0.2, 200000), 10.0 ** rng.uniform(-30, 0, 20000),
+                        [0.0, 0.3, np.nextafter(np.float32(0.3), np.float32(0)), 9.0, np.nextafter(np.float32(9), np.float32(10)), 50.0]]).astype(np.float32)
+    t = orc.tanhf(x)
+    exact = np.tanh(x.astype(np.float64))
+    ulp = np.spacing(np.abs(exact).astype(np.float32)).astype(np.float64)
+    assert np.max(np.abs(t.astype(np.float64) - exact) / np.maximum(ulp, 1e-45)) <= 3.0
+    nz = x != 0
+    assert np.array_equal(orc.tanhf(-x[nz]).view(np.uint32), (-t[nz]).view(np.uint32)) and np.all(t[~nz] == 0)
+    assert np.all(np.abs(t) <= 1.0) and orc.tanhf(np.float32([50.0, -50.0])).tolist() == [1.0, -1.0]
+    xs = np.sort(rng.uniform(-10, 10, 200000).astype(np.float32))
+    assert np.all(np.diff(orc.tanhf(xs)) >= -2 ** -23)   # monotonic to within the last bit at the switch of methods
+
+
+def test_gelu_tanh_follows_the_reference_operation_order():
+    """src/cpu/expert_ffn.rs:87-91: cube = g*g*g, inner = 0.7978846 (g + 0.044715 cube), 0.5 g (1 + tanh(inner)), every
+    operation rounded to FP32. The same chain in numpy FP32 with a correctly rounded tanh: the two may differ only through
+    the last bits of tanh, i.e. by at most 2^-24 |g| times the 3 ulp of the tanh bound, and the BF16 results agree wherever
+    the value is not the cancelled tail."""
+    gate = np.arange(65536, dtype=np.uint32).astype(np.uint16)
+    g = orc.bf16_to_f32(gate)
+    g = g[np.isfinite(g) & (np.abs(g) < 1e12)]
+    f = np.float32
+    cube = (g * g) * g
+    inner = f(0.7978846) * (g + f(0.044715) * cube)
+    want = (f(0.5) * g) * (f(1) + np.tanh(inner.astype(np.float64)).astype(np.float32))
+    got = orc.gelu_tanh(g)
+    assert np.all(np.abs(got.astype(np.float64) - want) <= 3 * 2.0 ** -24 * np.abs(g))
+    assert np.mean(got == want) > 0.99
+    big = np.abs(want) >= 2.0 ** -16
+    assert np.array_equal(orc.f32_to_bf16(got[big]), orc.f32_to_bf16(want[big]))
+    # a dropped cubic term, a missing 0.5 or the erf form are all far outside this
+    assert abs(float(got[g == 1.0][0]) - 0.8411919906082768) < 1e-7
+    assert abs(float(got[g == -1.0][0]) + 0.15880800939172324) < 1e-7
+    assert np.all(got[g == 0.0] == 0.0)
+
+
+def test_gelu_twice_rounds_twice_and_ignores_the_clamp():
+    # src/cpu/expert_ffn.rs:110-113: g = bf16(gelu(gate)); bf16(g * up); no clamp for this mode (:72-73)
+    rng = np.random.default_rng(11)
+    gate = orc.f32_to_bf16(rng.normal(0, 2.0, 50000).astype(np.float32))
+    up = orc.f32_to_bf16(rng.normal(0, 2.0, 50000).astype(np.float32))
+    got = orc.silu_mul(gate, up, orc.GELU_TWICE, 0.0, orc.SILU_DIV)
+    inner = orc.bf16_to_f32(orc.f32_to_bf16(orc.gelu_tanh(orc.bf16_to_f32(gate))))
+    assert np.array_equal(got, orc.f32_to_bf16(inner * orc.bf16_to_f32(up)))
+    once = orc.f32_to_bf16(orc.gelu_tanh(orc.bf16_to_f32(gate)) * orc.bf16_to_f32(up))
+    assert np.any(got != once)   # the inner rounding is visible
+    for kind in (orc.SILU_DIV, orc.SILU_RCP, orc.SILU_SIGMOID2):
+        assert np.array_equal(got, orc.silu_mul(gate, up, orc.GELU_TWICE, 0.5, kind))   # neither the limit nor the SiLU form enter
+    assert np.any(got != orc.silu_mul(gate, up, orc.TWICE, 0.0, orc.SILU_DIV))
+
+
 def test_log1p_unit_accuracy():
     L = orc.lib()
     rng = np.random.default_rng(5)
