@@ -304,16 +304,19 @@ static int decode_dispatch(const ffmoe_expert_table* table, const ffmoe_shared_e
     return prefill_impl(table, &pf, (stage_mask & 1 ? 3 : 0) | (stage_mask & 2 ? 12 : 0), stream);
   }
   // Row counts from which the matrix-core cohort kernels take over for block-FP8 experts (same effective weights and BF16
-  // boundaries, the dot products in the matrix instruction's FP32 order instead of the wave's): the whole batch at
-  // FFMOE_DECODE_COHORT_ROWS (per layer at hidden 7168 / 256 experts: 64 rows 2.00 against 2.40 ms on the streaming kernels,
-  // 48 rows 1.81 against 2.00, 32 rows 1.51 against 1.55, 8 rows 0.65 against 0.54 ms), below that a block-FP8 shared expert
-  // alone from FFMOE_DECODE_SHARED_COHORT_ROWS on (it has every row: streamed once instead of once per row group that fits
-  // LDS; 16 rows 0.935 against 0.964 ms; a BF16 shared expert next to NVFP4 experts measured slower there, 1.88 against
-  // 1.80 ms at 32 rows, and stays on the streaming kernels).
+  // boundaries, the dot products in the matrix instruction's FP32 order instead of the wave's). The whole batch goes there
+  // from FFMOE_DECODE_COHORT_ROWS on: 8 when the shared expert rides in the routed launches (same format and width, or no
+  // shared expert), 32 when it needs launches of its own, a few dozen blocks each. Per layer at hidden 7168 / 256 experts
+  // with a riding shared expert, cohort against streaming kernels: 4 rows 311 / 313 us, 8 rows 548 / 554, 12 rows 747 / 769,
+  // 16 rows 886 / 939, 24 rows 1166 / 1279, 32 rows 1397 / 1550, 64 rows 1886 / 2402; 2 rows 230 / 166. Below that a
+  // block-FP8 shared expert alone from FFMOE_DECODE_SHARED_COHORT_ROWS on (it has every row: streamed once instead of once
+  // per row group that fits LDS; a BF16 shared expert next to NVFP4 experts measured slower there, 1.88 against 1.80 ms at
+  // 32 rows, and stays on the streaming kernels).
   // (0 switches a rule off; read at every call)
   const char* ce = getenv("FFMOE_DECODE_COHORT_ROWS");
   const char* se = getenv("FFMOE_DECODE_SHARED_COHORT_ROWS");
-  const int cohort_rows = ce ? atoi(ce) : 32, shared_rows = se ? atoi(se) : 16;
+  const bool rides = !shared || (table && shared->format == table->format && shared->inter == table->inter);
+  const int cohort_rows = ce ? atoi(ce) : (rides ? 8 : 32), shared_rows = se ? atoi(se) : 16;
   if (table && args && args->act_mode == FFMOE_ACT_BF16 && args->rows > 1) {
     const int fmt = table->format, H = table->hidden, I = table->inter, R = args->rows;
     auto on_matrix_cores = [&](int f, int inter) {

@@ -54,10 +54,16 @@ __global__ __launch_bounds__(256) void k_prefill_count(const LiveTest t, uint32_
 
 // exclusive scans over experts (row offsets and group offsets), group descriptors and the two unit lists
 // (kernels/moe_prefill.cu:421-472; unit order = expert, column tile, row group, so neighbours share weights)
-__global__ __launch_bounds__(1024) void k_prefill_plan(PrefillBook b, int experts, int tm, int tiles0, int tiles1, int rgb) {
-  __shared__ uint32_t s_rows[1025], s_groups[1025], s_tmp[1024];
+// shared_rows > 0 appends the always-on expert as groups of expert id `experts` over rows 0 .. shared_rows - 1, their units
+// behind the routed ones (column tile outermost, so the row groups of a tile are neighbours and share its weights in L2):
+// the launches that run the routed experts then run the shared one as well.
+struct PlanShared { uint32_t rows[1025], groups[1025], tmp[1024]; };
+__device__ __forceinline__ void prefill_plan_body(PlanShared& sh, const PrefillBook& b, int experts, int tm, int tiles0, int tiles1, int rgb,
+                                                  int shared_rows, uint32_t c) {
+  uint32_t* s_rows = sh.rows;
+  uint32_t* s_groups = sh.groups;
+  uint32_t* s_tmp = sh.tmp;
   const int tid = threadIdx.x;
-  const uint32_t c = tid < experts ? b.counts[tid] : 0u;
   const uint32_t g = (c + tm - 1) / tm;
   // Hillis-Steele inclusive scans
   uint32_t vr = c, vg = g;
@@ -82,7 +88,13 @@ __global__ __launch_bounds__(1024) void k_prefill_plan(PrefillBook b, int expert
   if (tid < experts) { b.offsets[tid] = s_rows[tid]; b.gbase[tid] = s_groups[tid]; }
   if (tid == 0) { b.offsets[experts] = s_rows[experts]; b.gbase[experts] = s_groups[experts]; }
   const uint32_t G = s_groups[experts];
-  if (tid == 0) { b.totals[0] = G * tiles0; b.totals[1] = G * tiles1; b.totals[2] = G; b.totals[3] = s_rows[experts]; }
+  const uint32_t GS = shared_rows > 0 ? uint32_t((shared_rows + tm - 1) / tm) : 0u;
+  if (tid == 0) { b.totals[0] = (G + GS) * tiles0; b.totals[1] = (G + GS) * tiles1; b.totals[2] = G; b.totals[3] = s_rows[experts]; }
+  for (uint32_t q = tid; q < GS; q += 1024) {
+    GemmGroup gd;
+    gd.expert = experts; gd.start = int(q) * tm; gd.n = min(tm, shared_rows - int(q) * tm); gd.pad = 0;
+    b.groups[G + q] = gd;
+  }
   // group descriptors
   for (uint32_t q = tid; q < G; q += 1024) {
     int lo = 0, hi = experts;  // last e with s_groups[e] <= q
@@ -112,7 +124,46 @@ __global__ __launch_bounds__(1024) void k_prefill_plan(PrefillBook b, int expert
       const uint32_t rb = min(uint32_t(rgb), ge - j * uint32_t(rgb));
       { const u32x2 e2 = {s_groups[lo] + j * uint32_t(rgb) + w % rb, w / rb}; units[u] = e2; }
     }
+    for (uint32_t v = tid; v < GS * tiles; v += 1024) { const u32x2 e2 = {G + v % GS, v / GS}; units[G * tiles + v] = e2; }
   }
+}
+
+__global__ __launch_bounds__(1024) void k_prefill_plan(PrefillBook b, int experts, int tm, int tiles0, int tiles1, int rgb, int shared_rows) {
+  __shared__ PlanShared sh;
+  prefill_plan_body(sh, b, experts, tm, tiles0, tiles1, rgb, shared_rows, int(threadIdx.x) < experts ? b.counts[threadIdx.x] : 0u);
+}
+
+// Small cohorts (at most FFMOE_BOOK_SMALL_MAX assignments, one per thread): count, plan and stable fill in ONE launch of one
+// block, instead of four launches that each cost a launch more than they compute. The ids of the live assignments are kept
+// in LDS; an assignment's place in its expert's segment is the number of earlier assignments of that expert.
+constexpr int FFMOE_BOOK_SMALL_MAX = 1024;
+__global__ __launch_bounds__(1024) void k_prefill_book_small(const LiveTest lt, PrefillBook b, int A, int experts, int tm, int tiles0, int tiles1,
+                                                             int rgb, int shared_rows) {
+  __shared__ PlanShared sh;
+  __shared__ uint32_t s_cnt[1024];
+  __shared__ __attribute__((aligned(16))) int s_id[FFMOE_BOOK_SMALL_MAX];
+  const int tid = threadIdx.x;
+  s_cnt[tid] = 0u;
+  __syncthreads();
+  int my = -1;  // thread a holds assignment a (A <= 1024 = the block)
+  if (tid < A) {
+    int id;
+    if (assignment_live(lt, tid, id)) { my = id; atomicAdd(&s_cnt[id], 1u); }
+  }
+  s_id[tid] = my;
+  __syncthreads();
+  const uint32_t c = tid < experts ? s_cnt[tid] : 0u;
+  if (tid < experts) b.counts[tid] = c;
+  prefill_plan_body(sh, b, experts, tm, tiles0, tiles1, rgb, shared_rows, c);
+  // position inside the expert's segment = number of earlier assignments of the same expert; every thread walks the same
+  // LDS words (broadcast reads), four at a time
+  uint32_t rank = 0;
+  const int upto = (A + 3) & ~3;
+  for (int q = 0; q < upto; q += 4) {
+    const int4 v = *reinterpret_cast<const int4*>(&s_id[q]);
+    rank += uint32_t(v.x == my && q < tid) + uint32_t(v.y == my && q + 1 < tid) + uint32_t(v.z == my && q + 2 < tid) + uint32_t(v.w == my && q + 3 < tid);
+  }
+  if (my >= 0) b.perm[sh.rows[my] + rank] = tid;
 }
 
 // stable fill: block e lists its assignments in ascending assignment order (the reference permutes with an atomic
@@ -253,7 +304,7 @@ struct PrefillLayout {
 PrefillLayout prefill_layout(int rows, int top_k, int experts, int hidden, int inter, int shared_inter) {
   PrefillLayout l{};
   const uint64_t A = uint64_t(rows) * top_k;
-  l.max_groups = uint64_t(experts) + (A + 15) / 16;
+  l.max_groups = uint64_t(experts) + (A + 15) / 16 + (shared_inter > 0 ? (uint64_t(rows) + 15) / 16 : 0);
   uint64_t off = 0;
   auto take = [&](uint64_t bytes) { const uint64_t at = off; off += up256(bytes); return at; };
   l.xq = take(uint64_t(rows) * hidden);
@@ -318,7 +369,7 @@ int shared_expert_w16(const ffmoe_shared_expert* shared, const void* x, int R, i
   const int stm = 16 * smf;
   const uint32_t sgroups = uint32_t((R + stm - 1) / stm);
   W16Params q{};
-  q.rows_total = R; q.top_k = 1;
+  q.rows_total = R; q.top_k = 1; q.shared_expert = -1;
   q.swiglu = swiglu; q.limit = limit;
   if (stage_mask & 1) {
     q.a = (const uint16_t*)x;
@@ -433,13 +484,28 @@ int prefill_impl(const ffmoe_expert_table* table, const ffmoe_prefill* args, int
   const int mf = pick_mf(double(A) / E, (mx || a16) ? 4 : 8);
   const int tm = 16 * mf;
   const int tiles0 = (I + 127) / 128, tiles1 = (H + 255) / 256;
+  // A shared expert of the routed experts' format and width rides in the routed launches as further row groups (W*A16
+  // cohorts): on its own it is a few dozen blocks per launch, which at small cohorts take longer than the routed experts'
+  // thousands. FFMOE_PREFILL_SHARED_RIDE=0 keeps it in launches of its own (the results are the same bits either way).
+  bool ride = a16 && shared && shared->format == table->format && SI == I;
+  if (const char* f = getenv("FFMOE_PREFILL_SHARED_RIDE")) ride = ride && atoi(f) != 0;
 
   if (stages & 1) {
-    hipLaunchKernelGGL(k_prefill_zero, dim3((E + 255) / 256), dim3(256), 0, stream, b.counts, E, b.totals);
     const LiveTest lt{args->ids, args->active, table->valid, table->generation, args->assignment_gen, E};
-    hipLaunchKernelGGL(k_prefill_count, dim3((unsigned)((A + 255) / 256)), dim3(256), 0, stream, lt, b.counts, (long long)A);
-    hipLaunchKernelGGL(k_prefill_plan, dim3(1), dim3(1024), 0, stream, b, E, tm, tiles0, tiles1, pick_rgb());
-    hipLaunchKernelGGL(k_prefill_fill, dim3(E), dim3(256), 0, stream, lt, b, (long long)A);
+    // up to this many assignments one launch does the bookkeeping (measured at 256 experts: 64 assignments 10 us against
+    // 21 us for the four launches, 512 assignments 31 against 29 us); FFMOE_PREFILL_BOOK_SMALL overrides the limit
+    // (0: the four launches at any size, at most FFMOE_BOOK_SMALL_MAX)
+    int small_max = 256;
+    if (const char* f = getenv("FFMOE_PREFILL_BOOK_SMALL")) small_max = std::max(0, std::min(atoi(f), FFMOE_BOOK_SMALL_MAX));
+    const bool small = A <= size_t(small_max);
+    if (small) {
+      hipLaunchKernelGGL(k_prefill_book_small, dim3(1), dim3(1024), 0, stream, lt, b, int(A), E, tm, tiles0, tiles1, pick_rgb(), ride ? R : 0);
+    } else {
+      hipLaunchKernelGGL(k_prefill_zero, dim3((E + 255) / 256), dim3(256), 0, stream, b.counts, E, b.totals);
+      hipLaunchKernelGGL(k_prefill_count, dim3((unsigned)((A + 255) / 256)), dim3(256), 0, stream, lt, b.counts, (long long)A);
+      hipLaunchKernelGGL(k_prefill_plan, dim3(1), dim3(1024), 0, stream, b, E, tm, tiles0, tiles1, pick_rgb(), ride ? R : 0);
+      hipLaunchKernelGGL(k_prefill_fill, dim3(E), dim3(256), 0, stream, lt, b, (long long)A);
+    }
     FF_TRY(ff_launch_status());
     // activations -> E4M3 + per-128 scales
     if (mx) FF_TRY(ffmoe_act_quant_e8m0(args->x, s + l.xq, s + l.sx, R, H, stream_));  // E4M3 codes + one E8M0 byte per 32
@@ -490,17 +556,24 @@ int prefill_impl(const ffmoe_expert_table* table, const ffmoe_prefill* args, int
     p.slots = table->slots; p.global_scales = table->format == FFMOE_FMT_NVFP4 ? table->global_scales : nullptr;
     p.groups = b.groups; p.perm = b.perm; p.top_k = K;
     p.swiglu = args->swiglu; p.limit = args->swiglu_limit; p.routed_weight = args->routed_weight; p.weights_f32 = args->weights_f32;
+    p.shared_expert = ride ? E : -1;
+    if (ride) {
+      for (int i = 0; i < 6; ++i) p.sh_w[i] = shared->slot[i];
+      for (int i = 0; i < 3; ++i) p.sh_g[i] = shared->global_scales[i];
+    }
     if (stages & 2) {
       p.a = (const uint16_t*)args->x; p.units = b.units0; p.unit_total = b.totals + 0;
       p.out = (uint16_t*)(s + l.act); p.K = H; p.N = I;
+      p.a_sh = (const uint16_t*)args->x; p.out_sh = (uint16_t*)(s + l.sh_act);
       FF_TRY(launch_w16_fmt<0>(table->format, p, mf, blocks, stream));
     }
     if (stages & 8) {
       p.a = (const uint16_t*)(s + l.act); p.units = b.units1; p.unit_total = b.totals + 1;
       p.out = (uint16_t*)args->contributions; p.done = args->done; p.weights = args->weights; p.K = I; p.N = H;
+      p.a_sh = (const uint16_t*)(s + l.sh_act); p.out_sh = (uint16_t*)args->shared_out;
       FF_TRY(launch_w16_fmt<1>(table->format, p, mf, blocks, stream));
     }
-    if (shared)
+    if (shared && !ride)
       FF_TRY(shared_expert_w16(shared, args->x, R, H, args->swiglu, args->swiglu_limit, s + l.sh_act, args->shared_out,
                                (stages & 2 ? 1 : 0) | (stages & 8 ? 2 : 0), stream_));
     return 0;

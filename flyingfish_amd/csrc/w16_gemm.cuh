@@ -140,6 +140,14 @@ struct W16Params {
   int rows_total;
   int K, N, top_k, weights_f32, swiglu, routed_weight;
   float limit;
+  // Groups whose expert id is shared_expert (>= 0) are the always-on expert riding in the routed launch: weights from
+  // sh_w / sh_g (gate, up, down: codes and scales; NVFP4 global scales), token rows are the rows themselves (no
+  // permutation) read from a_sh, results go to out_sh[row] as plain BF16 (no routing weight, no done flag).
+  int shared_expert;
+  uint64_t sh_w[6];
+  float sh_g[3];
+  const uint16_t* a_sh;
+  uint16_t* out_sh;
 };
 
 template <class F, int MF, int MODE, int P>
@@ -190,7 +198,13 @@ __global__ __launch_bounds__(256, 2) void k_w16_grouped(const W16Params p) {
     }
     uint64_t wc[2], ws[2];
     float gl[2] = {p.g0, p.g1};
-    if (p.slots) {
+    const bool ride = p.groups && expert == p.shared_expert;  // wave-uniform
+    if (ride) {
+      wc[0] = MODE == 0 ? p.sh_w[0] : p.sh_w[4]; ws[0] = MODE == 0 ? p.sh_w[1] : p.sh_w[5];
+      wc[1] = MODE == 0 ? p.sh_w[2] : p.sh_w[4]; ws[1] = MODE == 0 ? p.sh_w[3] : p.sh_w[5];
+      gl[0] = MODE == 0 ? p.sh_g[0] : p.sh_g[2];
+      gl[1] = MODE == 0 ? p.sh_g[1] : p.sh_g[2];
+    } else if (p.slots) {
       const uint64_t* sl = p.slots + size_t(expert) * 6;
       if (MODE == 0) {
         wc[0] = uni64(load_global<uint64_t>(sl + 0)); ws[0] = uni64(load_global<uint64_t>(sl + 1));
@@ -253,8 +267,8 @@ __global__ __launch_bounds__(256, 2) void k_w16_grouped(const W16Params p) {
       const int q = min(tid + 256 * i, CHUNKS - 1);
       const int m = q >> 3, c = q & 7;
       const int pos = start + min(m, n - 1);
-      const int row = MODE == 0 && p.perm ? load_global<int>(p.perm + pos) / p.top_k : pos;
-      tsrc[i] = reinterpret_cast<const uint8_t*>(p.a) + size_t(row) * K * 2 + c * 16;
+      const int row = MODE == 0 && p.perm && !ride ? load_global<int>(p.perm + pos) / p.top_k : pos;
+      tsrc[i] = reinterpret_cast<const uint8_t*>(ride ? p.a_sh : p.a) + size_t(row) * K * 2 + c * 16;
       tdst[i] = m * 128 + ((c ^ (m & 7)) << 4);
     }
     const bool stage_chunk = CHUNKS >= 256 || tid < CHUNKS;
@@ -402,13 +416,14 @@ __global__ __launch_bounds__(256, 2) void k_w16_grouped(const W16Params p) {
                 o[h] = lo | (hi << 16);
               }
               const u32x2 v = {o[0], o[1]};
-              *reinterpret_cast<u32x2*>(p.out + size_t(pos) * N + col) = v;
+              *reinterpret_cast<u32x2*>((ride ? p.out_sh : p.out) + size_t(pos) * N + col) = v;
             }
           }
         } else {
-          const int a = (MODE == 1 && p.perm) ? load_global<int>(p.perm + pos) : pos;
+          const int a = (MODE == 1 && p.perm && !ride) ? load_global<int>(p.perm + pos) : pos;
+          const bool weighted = MODE == 1 && p.weights && !ride;
           float rw = 1.0f;
-          if (MODE == 1 && p.weights)
+          if (weighted)
             rw = p.weights_f32 ? load_global<float>(reinterpret_cast<const float*>(p.weights) + a)
                                : bf16_to_f32(load_global<uint16_t>(reinterpret_cast<const uint16_t*>(p.weights) + a));
 #pragma unroll
@@ -418,16 +433,16 @@ __global__ __launch_bounds__(256, 2) void k_w16_grouped(const W16Params p) {
               float v[4];
 #pragma unroll
               for (int r = 0; r < 4; ++r) {
-                if (MODE == 1 && p.weights)
+                if (weighted)
                   v[r] = p.routed_weight == FFMOE_WEIGHT_AFTER_DOWN_BF16 ? __fmul_rn(bround(acc[m][f][r]), rw) : __fmul_rn(acc[m][f][r], rw);
                 else
                   v[r] = acc[m][f][r];
               }
               const u32x2 o = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
-              *reinterpret_cast<u32x2*>(p.out + size_t(a) * N + col) = o;
+              *reinterpret_cast<u32x2*>((ride ? p.out_sh : p.out) + size_t(a) * N + col) = o;
             }
           }
-          if (MODE == 1 && p.done && t == 0 && wave == 0 && lane < 16) p.done[a] = 1u;
+          if (MODE == 1 && p.done && !ride && t == 0 && wave == 0 && lane < 16) p.done[a] = 1u;
         }
       }
     }

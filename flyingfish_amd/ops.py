@@ -455,7 +455,7 @@ class PrefillOps:
         take("perm", A * 4, torch.int32, (A,))
         if self._shared_c is not None:
             SI = self._shared_c.inter
-            max_groups = E + (A + 15) // 16
+            max_groups = E + (A + 15) // 16 + (R + 15) // 16
             take("groups", max_groups * 16, torch.uint8, (max_groups * 16,))
             take("units0", max_groups * (-(-I // 128)) * 8, torch.uint8, (-1,))
             take("units1", max_groups * (-(-H // 256)) * 8, torch.uint8, (-1,))

@@ -20,6 +20,14 @@ def rand_bf16(shape, std, seed):
     return synth.normal(shape, std, seed).to(torch.bfloat16)
 
 
+@pytest.fixture(autouse=True)
+def _streaming_decode_kernels(monkeypatch):
+    """The decode tests of this module check the streaming kernels stage by stage (they read the activations out of that
+    path's arena): block-FP8 batches of 8 rows and more, which the library would hand to the matrix-core cohort kernels,
+    stay on them here. The cohort dispatch has its own tests (test_gpu_prefill.py, test_gpu_fullsize.py)."""
+    monkeypatch.setenv("FFMOE_DECODE_COHORT_ROWS", "0")
+
+
 # ------------------------------------------------------------------------------------------------
 # codecs through the product path
 def test_device_e4m3_decode_all_codes():

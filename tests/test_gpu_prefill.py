@@ -383,6 +383,75 @@ def test_prefill_grouping_switches_leave_every_bit_alone(act_mode, monkeypatch):
         assert np.array_equal(got, ref), "FFMOE_PREFILL_MF=%s FFMOE_PREFILL_RGB=%s changes the result" % (mf, rgb)
 
 
+@pytest.mark.parametrize("fmt", [capi.FMT_FP8_BLOCK128, capi.FMT_NVFP4, capi.FMT_BF16, capi.FMT_FP8_CHANNEL])
+@pytest.mark.parametrize("rows,mf", [(70, "1"), (70, "4"), (9, "2"), (150, "2")])
+def test_prefill_shared_expert_rides_in_the_routed_launches_bitwise(fmt, rows, mf, monkeypatch):
+    """W*A16 cohorts: a shared expert of the routed experts' format and width is appended to the routed launches as
+    row groups of its own. Its outputs, its activations and the routed contributions are the bits of the separate
+    launches (FFMOE_PREFILL_SHARED_RIDE=0), whatever the group size and with rows that do not fill the last group."""
+    from helpers import make_table
+    top_k, experts, hidden, inter = 3, 5, 256, 384
+    table, _ = make_table(fmt, experts + 1, hidden, inter, 300 + rows)
+    sh = table.shared_struct(experts)
+    table.experts = experts
+    ids, w = _routing(rows, top_k, experts, 310 + rows, 1.2)
+    x = synth.normal((rows, hidden), 1.0, 320 + rows, dtype=torch.bfloat16).cuda()
+    ids_d, w_d = torch.from_numpy(ids).cuda(), torch.from_numpy(w).cuda()
+    monkeypatch.setenv("FFMOE_PREFILL_MF", mf)
+    out = {}
+    for ride in ("0", "1"):
+        monkeypatch.setenv("FFMOE_PREFILL_SHARED_RIDE", ride)
+        op = ops.PrefillOps(table, rows, top_k, swiglu=capi.SWIGLU_TWICE, routed_weight=capi.WEIGHT_AFTER_DOWN_BF16, weights_f32=True,
+                            shared=sh, act_mode=capi.ACT_BF16)
+        op.contributions.zero_(); op.shared_out.zero_(); op.scratch.zero_()
+        got = op.contribute(x, ids_d, w_d)
+        torch.cuda.synchronize()
+        v = op.scratch_views()
+        out[ride] = (bits(got).copy(), bits(op.shared_out).copy(), bits(v["sh_act"]).copy(), op.done.cpu().numpy().copy())
+    assert np.any(out["0"][1] != 0) and np.any(out["0"][2] != 0)
+    for a, b, what in zip(out["0"], out["1"], ("contributions", "shared_out", "shared activations", "done")):
+        assert np.array_equal(a, b), what
+
+
+@pytest.mark.parametrize("rows,top_k,experts", [(1, 1, 3), (37, 4, 9), (128, 8, 70), (341, 3, 5)])
+def test_prefill_single_launch_bookkeeping_equals_the_four_launches(rows, top_k, experts, monkeypatch):
+    """Small cohorts (by default up to 256 assignments, here forced up to the kernel's 1024) are counted, planned and listed
+    by one block in one launch. Segment offsets,
+    the stable permutation, group descriptors, both unit lists and the totals are those of the count / plan / fill
+    launches (FFMOE_PREFILL_BOOK_SMALL=0), with inactive, invalid and out-of-range assignments in the input."""
+    hidden, inter = 128, 128
+    table, _ = _make_fp8_table(experts, hidden, inter, 77)
+    ids, w = _routing(rows, top_k, experts, 500 + rows, 1.4)
+    ids = ids.copy()
+    active = (np.random.default_rng(rows).random(ids.shape) > 0.2).astype(np.uint32)
+    if rows > 1:
+        ids[rows // 2, 0] = experts + 3   # out of range: skipped
+        ids[rows - 1, top_k - 1] = -1
+    valid = torch.ones(experts, dtype=torch.int32)
+    valid[experts // 2] = 0
+    table.valid = valid.cuda()
+    x = synth.normal((rows, hidden), 1.0, 510 + rows, dtype=torch.bfloat16).cuda()
+    ids_d, w_d, act_d = torch.from_numpy(ids).cuda(), torch.from_numpy(w).cuda(), torch.from_numpy(active).cuda()
+    seen = {}
+    for small in ("0", "1024"):
+        monkeypatch.setenv("FFMOE_PREFILL_BOOK_SMALL", small)
+        op = ops.PrefillOps(table, rows, top_k, weights_f32=True)
+        op.scratch.zero_(); op.contributions.zero_()
+        got = op.contribute(x, ids_d, w_d, active=act_d)
+        torch.cuda.synchronize()
+        v = op.scratch_views()
+        live = int(v["totals"][3].item())
+        seen[small] = dict(totals=v["totals"].cpu().numpy().copy(), counts=v["counts"].cpu().numpy().copy(), offsets=v["offsets"].cpu().numpy().copy(),
+                           gbase=v["gbase"].cpu().numpy().copy(), perm=v["perm"].cpu().numpy()[:live].copy(), out=bits(got).copy(),
+                           done=op.done.cpu().numpy().copy())
+    for k in seen["0"]:
+        assert np.array_equal(seen["0"][k], seen["1024"][k]), k
+    flat = ids.reshape(-1)
+    keep = (active.reshape(-1) != 0) & (flat >= 0) & (flat < experts) & (flat != experts // 2)
+    want = sorted(np.flatnonzero(keep).tolist(), key=lambda a: (flat[a], a))
+    assert seen["1024"]["perm"].tolist() == want
+
+
 def test_prefill_then_combine_layer():
     """contribute -> ordered combine equals the oracle's combine over the oracle's contributions within BF16 noise."""
     rows, top_k, experts, hidden, inter = 32, 4, 8, 256, 128
