@@ -45,11 +45,25 @@ __device__ __forceinline__ bool assignment_live(const LiveTest& t, long long a, 
   return true;
 }
 
-// histogram of live assignments per expert (kernels/moe_prefill.cu:364-420)
+// histogram of live assignments per expert (kernels/moe_prefill.cu:364-420): per block in LDS over 1024 assignments, then
+// one global add per expert the block has seen (a global add per assignment serializes on the popular experts' counters)
+constexpr int FFMOE_COUNT_PER_BLOCK = 1024;
 __global__ __launch_bounds__(256) void k_prefill_count(const LiveTest t, uint32_t* __restrict__ counts, long long A) {
-  const long long a = (long long)blockIdx.x * 256 + threadIdx.x;
-  int e;
-  if (a < A && assignment_live(t, a, e)) atomicAdd(counts + e, 1u);
+  __shared__ uint32_t s_hist[FFMOE_MAX_EXPERTS];
+  for (int e = threadIdx.x; e < t.experts; e += 256) s_hist[e] = 0u;
+  __syncthreads();
+  const long long first = (long long)blockIdx.x * FFMOE_COUNT_PER_BLOCK;
+#pragma unroll
+  for (int i = 0; i < FFMOE_COUNT_PER_BLOCK / 256; ++i) {
+    const long long a = first + i * 256 + threadIdx.x;
+    int e;
+    if (a < A && assignment_live(t, a, e)) atomicAdd(&s_hist[e], 1u);
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < t.experts; e += 256) {
+    const uint32_t c = s_hist[e];
+    if (c != 0u) atomicAdd(counts + e, c);
+  }
 }
 
 // exclusive scans over experts (row offsets and group offsets), group descriptors and the two unit lists
@@ -58,8 +72,31 @@ __global__ __launch_bounds__(256) void k_prefill_count(const LiveTest t, uint32_
 // behind the routed ones (column tile outermost, so the row groups of a tile are neighbours and share its weights in L2):
 // the launches that run the routed experts then run the shared one as well.
 struct PlanShared { uint32_t rows[1025], groups[1025], tmp[1024]; };
+
+// unit u of a list with `tiles` column tiles per group -> (group, tile); s_groups = exclusive scan of the experts' group
+// counts, G routed groups, GS groups of the riding shared expert behind them
+__device__ __forceinline__ u32x2 plan_unit(const uint32_t* s_groups, int experts, uint32_t tiles, int rgb, uint32_t G, uint32_t GS, uint32_t u) {
+  if (u >= G * tiles) {
+    const uint32_t v = u - G * tiles;
+    return u32x2{G + v % GS, v / GS};
+  }
+  const uint32_t key = u / tiles;
+  int lo = 0, hi = experts;  // last e with s_groups[e] <= key
+  while (hi - lo > 1) { const int mid = (lo + hi) >> 1; if (s_groups[mid] <= key) lo = mid; else hi = mid; }
+  // An expert's units run over blocks of rgb row groups, inside a block over the column tiles, innermost over the
+  // block's row groups. The blocks of an XCD work on neighbouring units at the same time, so a run of units shares
+  // the weights of a tile among a block's row groups and a row group's token tile among neighbouring tiles.
+  const uint32_t ge = s_groups[lo + 1] - s_groups[lo];
+  const uint32_t v = u - s_groups[lo] * tiles;
+  const uint32_t per = uint32_t(rgb) * tiles;
+  const uint32_t j = min(v / per, ge / uint32_t(rgb));
+  const uint32_t w = v - j * per;
+  const uint32_t rb = min(uint32_t(rgb), ge - j * uint32_t(rgb));
+  return u32x2{s_groups[lo] + j * uint32_t(rgb) + w % rb, w / rb};
+}
+
 __device__ __forceinline__ void prefill_plan_body(PlanShared& sh, const PrefillBook& b, int experts, int tm, int tiles0, int tiles1, int rgb,
-                                                  int shared_rows, uint32_t c) {
+                                                  int shared_rows, uint32_t c, bool with_units) {
   uint32_t* s_rows = sh.rows;
   uint32_t* s_groups = sh.groups;
   uint32_t* s_tmp = sh.tmp;
@@ -106,31 +143,33 @@ __device__ __forceinline__ void prefill_plan_body(PlanShared& sh, const PrefillB
     b.groups[q] = gd;
   }
   // unit lists
+  if (!with_units) return;
   for (int pass = 0; pass < 2; ++pass) {
     const uint32_t tiles = pass == 0 ? tiles0 : tiles1;
     u32x2* units = pass == 0 ? b.units0 : b.units1;
-    for (uint32_t u = tid; u < G * tiles; u += 1024) {
-      const uint32_t key = u / tiles;
-      int lo = 0, hi = experts;
-      while (hi - lo > 1) { const int mid = (lo + hi) >> 1; if (s_groups[mid] <= key) lo = mid; else hi = mid; }
-      // An expert's units run over blocks of rgb row groups, inside a block over the column tiles, innermost over the
-      // block's row groups. The blocks of an XCD work on neighbouring units at the same time, so a run of units shares
-      // the weights of a tile among a block's row groups and a row group's token tile among neighbouring tiles.
-      const uint32_t ge = s_groups[lo + 1] - s_groups[lo];
-      const uint32_t v = u - s_groups[lo] * tiles;
-      const uint32_t per = uint32_t(rgb) * tiles;
-      const uint32_t j = min(v / per, ge / uint32_t(rgb));
-      const uint32_t w = v - j * per;
-      const uint32_t rb = min(uint32_t(rgb), ge - j * uint32_t(rgb));
-      { const u32x2 e2 = {s_groups[lo] + j * uint32_t(rgb) + w % rb, w / rb}; units[u] = e2; }
-    }
-    for (uint32_t v = tid; v < GS * tiles; v += 1024) { const u32x2 e2 = {G + v % GS, v / GS}; units[G * tiles + v] = e2; }
+    for (uint32_t u = tid; u < (G + GS) * tiles; u += 1024) units[u] = plan_unit(s_groups, experts, tiles, rgb, G, GS, u);
   }
 }
 
 __global__ __launch_bounds__(1024) void k_prefill_plan(PrefillBook b, int experts, int tm, int tiles0, int tiles1, int rgb, int shared_rows) {
   __shared__ PlanShared sh;
-  prefill_plan_body(sh, b, experts, tm, tiles0, tiles1, rgb, shared_rows, int(threadIdx.x) < experts ? b.counts[threadIdx.x] : 0u);
+  prefill_plan_body(sh, b, experts, tm, tiles0, tiles1, rgb, shared_rows, int(threadIdx.x) < experts ? b.counts[threadIdx.x] : 0u, false);
+}
+
+// the two unit lists behind k_prefill_plan, one unit per thread over as many blocks as the lists can need (blocks past the
+// device-side totals leave at once): tens of thousands of units are too many for the plan's single block
+__global__ __launch_bounds__(256) void k_prefill_units(PrefillBook b, int experts, int tm, int tiles0, int tiles1, int rgb, int shared_rows) {
+  __shared__ uint32_t s_groups[1025];
+  const uint32_t n0 = b.totals[0], n1 = b.totals[1];
+  const uint32_t u = blockIdx.x * 256u + threadIdx.x;
+  if (blockIdx.x * 256u >= n0 + n1) return;
+  for (int e = threadIdx.x; e <= experts; e += 256) s_groups[e] = b.gbase[e];
+  __syncthreads();
+  if (u >= n0 + n1) return;
+  const uint32_t G = s_groups[experts];
+  const uint32_t GS = shared_rows > 0 ? uint32_t((shared_rows + tm - 1) / tm) : 0u;
+  if (u < n0) b.units0[u] = plan_unit(s_groups, experts, uint32_t(tiles0), rgb, G, GS, u);
+  else b.units1[u - n0] = plan_unit(s_groups, experts, uint32_t(tiles1), rgb, G, GS, u - n0);
 }
 
 // Small cohorts (at most FFMOE_BOOK_SMALL_MAX assignments, one per thread): count, plan and stable fill in ONE launch of one
@@ -154,7 +193,7 @@ __global__ __launch_bounds__(1024) void k_prefill_book_small(const LiveTest lt, 
   __syncthreads();
   const uint32_t c = tid < experts ? s_cnt[tid] : 0u;
   if (tid < experts) b.counts[tid] = c;
-  prefill_plan_body(sh, b, experts, tm, tiles0, tiles1, rgb, shared_rows, c);
+  prefill_plan_body(sh, b, experts, tm, tiles0, tiles1, rgb, shared_rows, c, true);
   // position inside the expert's segment = number of earlier assignments of the same expert; every thread walks the same
   // LDS words (broadcast reads), four at a time
   uint32_t rank = 0;
@@ -167,27 +206,77 @@ __global__ __launch_bounds__(1024) void k_prefill_book_small(const LiveTest lt, 
 }
 
 // stable fill: block e lists its assignments in ascending assignment order (the reference permutes with an atomic
-// cursor, kernels/moe_prefill.cu:475-510; per-row results make the order irrelevant, a fixed one keeps runs repeatable)
+// cursor, kernels/moe_prefill.cu:475-510; per-row results make the order irrelevant, a fixed one keeps runs repeatable).
+// Each of the four waves owns a contiguous quarter of the assignments: it counts its hits, the block exchanges the four
+// counts once, and the wave walks its quarter again writing positions - no block-wide step per 256 assignments. The
+// per-assignment words are all loaded unconditionally (independent, coalesced requests: one memory latency per 2048
+// assignments of a wave), and while a quarter has at most 8192 assignments a lane keeps its 128 hit bits in registers, so
+// the second walk reads nothing.
 __global__ __launch_bounds__(256) void k_prefill_fill(const LiveTest lt, PrefillBook b, long long A) {
   __shared__ uint32_t s_wave[4];
   const int e = blockIdx.x;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const uint32_t cnt = b.counts[e];
   if (cnt == 0u) return;
+  const bool gens = lt.generation && lt.assignment_gen;
+  const uint64_t gen_e = gens ? lt.generation[e] : 0ull;
+  const long long quarter = ((A + 255) / 256) * 64;  // a multiple of 64, four of them cover A
+  const long long lo = quarter * wave, hi = lo + quarter < A ? lo + quarter : A;
+  // 32 assignments of this lane starting at a0: bit j = assignment a0 + 64 j + lane is a live choice of expert e
+  // (the conditions of assignment_live; the expert's valid flag is implied by its non-zero count)
+  auto hits32 = [&](long long a0) {
+    int id[32];
+    uint32_t act[32];
+    uint64_t ag[32];
+#pragma unroll
+    for (int j = 0; j < 32; ++j) {
+      const long long a = a0 + 64 * j + lane;
+      const bool in = a < hi;
+      id[j] = in ? lt.ids[a] : -1;
+      act[j] = (in && lt.active) ? lt.active[a] : 1u;
+      ag[j] = (in && gens) ? lt.assignment_gen[a] : gen_e;
+    }
+    uint32_t bits = 0;
+#pragma unroll
+    for (int j = 0; j < 32; ++j) bits |= uint32_t(id[j] == e && act[j] != 0u && ag[j] == gen_e) << j;
+    return bits;
+  };
+  const bool cached = quarter <= 8192;
+  uint32_t keep[4] = {0u, 0u, 0u, 0u};
+  uint32_t mine = 0;
+  {
+    int w = 0;
+    for (long long a0 = lo; a0 < hi; a0 += 2048, ++w) {
+      const uint32_t bits = hits32(a0);
+      if (cached) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) keep[q] = w == q ? bits : keep[q];
+      }
+#pragma unroll
+      for (int j = 0; j < 32; ++j) mine += __popcll(__ballot((bits >> j) & 1u));
+    }
+  }
+  if (lane == 0) s_wave[wave] = mine;
+  __syncthreads();
   uint32_t run = b.offsets[e];
-  for (long long a0 = 0; a0 < A; a0 += 256) {
-    const long long a = a0 + tid;
-    int id;
-    const bool hit = a < A && assignment_live(lt, a, id) && id == e;
-    const uint64_t mask = __ballot(hit);
-    const uint32_t before = __popcll(mask & ((uint64_t(1) << lane) - 1));
-    if (lane == 0) s_wave[wave] = __popcll(mask);
-    __syncthreads();
-    uint32_t base = run;
-    for (int w = 0; w < wave; ++w) base += s_wave[w];
-    if (hit) b.perm[base + before] = int(a);
-    run += s_wave[0] + s_wave[1] + s_wave[2] + s_wave[3];
-    __syncthreads();
+  for (int w = 0; w < wave; ++w) run += s_wave[w];
+  int w = 0;
+  for (long long a0 = lo; a0 < hi; a0 += 2048, ++w) {
+    uint32_t bits;
+    if (cached) {
+      bits = keep[0];
+#pragma unroll
+      for (int q = 1; q < 4; ++q) bits = w == q ? keep[q] : bits;
+    } else {
+      bits = hits32(a0);
+    }
+#pragma unroll
+    for (int j = 0; j < 32; ++j) {
+      const bool h = (bits >> j) & 1u;
+      const uint64_t mask = __ballot(h);
+      if (h) b.perm[run + __popcll(mask & ((uint64_t(1) << lane) - 1))] = int(a0 + 64 * j + lane);
+      run += __popcll(mask);
+    }
   }
 }
 
@@ -502,8 +591,10 @@ int prefill_impl(const ffmoe_expert_table* table, const ffmoe_prefill* args, int
       hipLaunchKernelGGL(k_prefill_book_small, dim3(1), dim3(1024), 0, stream, lt, b, int(A), E, tm, tiles0, tiles1, pick_rgb(), ride ? R : 0);
     } else {
       hipLaunchKernelGGL(k_prefill_zero, dim3((E + 255) / 256), dim3(256), 0, stream, b.counts, E, b.totals);
-      hipLaunchKernelGGL(k_prefill_count, dim3((unsigned)((A + 255) / 256)), dim3(256), 0, stream, lt, b.counts, (long long)A);
+      hipLaunchKernelGGL(k_prefill_count, dim3((unsigned)((A + FFMOE_COUNT_PER_BLOCK - 1) / FFMOE_COUNT_PER_BLOCK)), dim3(256), 0, stream, lt, b.counts, (long long)A);
       hipLaunchKernelGGL(k_prefill_plan, dim3(1), dim3(1024), 0, stream, b, E, tm, tiles0, tiles1, pick_rgb(), ride ? R : 0);
+      const uint64_t max_units = l.max_groups * uint64_t(tiles0 + tiles1);
+      hipLaunchKernelGGL(k_prefill_units, dim3((unsigned)((max_units + 255) / 256)), dim3(256), 0, stream, b, E, tm, tiles0, tiles1, pick_rgb(), ride ? R : 0);
       hipLaunchKernelGGL(k_prefill_fill, dim3(E), dim3(256), 0, stream, lt, b, (long long)A);
     }
     FF_TRY(ff_launch_status());
