@@ -75,7 +75,7 @@ struct PlanShared { uint32_t rows[1025], groups[1025], tmp[1024]; };
 
 // unit u of a list with `tiles` column tiles per group -> (group, tile); s_groups = exclusive scan of the experts' group
 // counts, G routed groups, GS groups of the riding shared expert behind them
-__device__ __forceinline__ u32x2 plan_unit(const uint32_t* s_groups, int experts, uint32_t tiles, int rgb, uint32_t G, uint32_t GS, uint32_t u) {
+__device__ __forceinline__ u32x2 plan_unit(const uint32_t* s_groups, int experts, uint32_t tiles, int rgb, int tgb, uint32_t G, uint32_t GS, uint32_t u) {
   if (u >= G * tiles) {
     const uint32_t v = u - G * tiles;
     return u32x2{G + v % GS, v / GS};
@@ -83,20 +83,25 @@ __device__ __forceinline__ u32x2 plan_unit(const uint32_t* s_groups, int experts
   const uint32_t key = u / tiles;
   int lo = 0, hi = experts;  // last e with s_groups[e] <= key
   while (hi - lo > 1) { const int mid = (lo + hi) >> 1; if (s_groups[mid] <= key) lo = mid; else hi = mid; }
-  // An expert's units run over blocks of rgb row groups, inside a block over the column tiles, innermost over the
-  // block's row groups. The blocks of an XCD work on neighbouring units at the same time, so a run of units shares
-  // the weights of a tile among a block's row groups and a row group's token tile among neighbouring tiles.
+  // An expert's units run over blocks of rgb row groups, inside a row block over blocks of tgb column tiles, inside those
+  // over the tiles, innermost over the row groups. The blocks of an XCD work on neighbouring units at the same time (64 of
+  // them with two blocks per CU), so a window of rgb x tgb units fetches rgb token tiles and tgb weight tiles into that
+  // XCD's L2 and shares each among tgb resp. rgb blocks.
   const uint32_t ge = s_groups[lo + 1] - s_groups[lo];
   const uint32_t v = u - s_groups[lo] * tiles;
   const uint32_t per = uint32_t(rgb) * tiles;
-  const uint32_t j = min(v / per, ge / uint32_t(rgb));
+  const uint32_t j = min(v / per, (ge - 1u) / uint32_t(rgb));
   const uint32_t w = v - j * per;
   const uint32_t rb = min(uint32_t(rgb), ge - j * uint32_t(rgb));
-  return u32x2{s_groups[lo] + j * uint32_t(rgb) + w % rb, w / rb};
+  const uint32_t tg = min(uint32_t(tgb), tiles);
+  const uint32_t per2 = rb * tg;
+  const uint32_t q = min(w / per2, (tiles - 1u) / tg);
+  const uint32_t w2 = w - q * per2;
+  return u32x2{s_groups[lo] + j * uint32_t(rgb) + w2 % rb, q * tg + w2 / rb};
 }
 
 __device__ __forceinline__ void prefill_plan_body(PlanShared& sh, const PrefillBook& b, int experts, int tm, int tiles0, int tiles1, int rgb,
-                                                  int shared_rows, uint32_t c, bool with_units) {
+                                                  int tgb, int shared_rows, uint32_t c, bool with_units) {
   uint32_t* s_rows = sh.rows;
   uint32_t* s_groups = sh.groups;
   uint32_t* s_tmp = sh.tmp;
@@ -147,18 +152,18 @@ __device__ __forceinline__ void prefill_plan_body(PlanShared& sh, const PrefillB
   for (int pass = 0; pass < 2; ++pass) {
     const uint32_t tiles = pass == 0 ? tiles0 : tiles1;
     u32x2* units = pass == 0 ? b.units0 : b.units1;
-    for (uint32_t u = tid; u < (G + GS) * tiles; u += 1024) units[u] = plan_unit(s_groups, experts, tiles, rgb, G, GS, u);
+    for (uint32_t u = tid; u < (G + GS) * tiles; u += 1024) units[u] = plan_unit(s_groups, experts, tiles, rgb, tgb, G, GS, u);
   }
 }
 
-__global__ __launch_bounds__(1024) void k_prefill_plan(PrefillBook b, int experts, int tm, int tiles0, int tiles1, int rgb, int shared_rows) {
+__global__ __launch_bounds__(1024) void k_prefill_plan(PrefillBook b, int experts, int tm, int tiles0, int tiles1, int rgb, int tgb, int shared_rows) {
   __shared__ PlanShared sh;
-  prefill_plan_body(sh, b, experts, tm, tiles0, tiles1, rgb, shared_rows, int(threadIdx.x) < experts ? b.counts[threadIdx.x] : 0u, false);
+  prefill_plan_body(sh, b, experts, tm, tiles0, tiles1, rgb, tgb, shared_rows, int(threadIdx.x) < experts ? b.counts[threadIdx.x] : 0u, false);
 }
 
 // the two unit lists behind k_prefill_plan, one unit per thread over as many blocks as the lists can need (blocks past the
 // device-side totals leave at once): tens of thousands of units are too many for the plan's single block
-__global__ __launch_bounds__(256) void k_prefill_units(PrefillBook b, int experts, int tm, int tiles0, int tiles1, int rgb, int shared_rows) {
+__global__ __launch_bounds__(256) void k_prefill_units(PrefillBook b, int experts, int tm, int tiles0, int tiles1, int rgb, int tgb, int shared_rows) {
   __shared__ uint32_t s_groups[1025];
   const uint32_t n0 = b.totals[0], n1 = b.totals[1];
   const uint32_t u = blockIdx.x * 256u + threadIdx.x;
@@ -168,8 +173,8 @@ __global__ __launch_bounds__(256) void k_prefill_units(PrefillBook b, int expert
   if (u >= n0 + n1) return;
   const uint32_t G = s_groups[experts];
   const uint32_t GS = shared_rows > 0 ? uint32_t((shared_rows + tm - 1) / tm) : 0u;
-  if (u < n0) b.units0[u] = plan_unit(s_groups, experts, uint32_t(tiles0), rgb, G, GS, u);
-  else b.units1[u - n0] = plan_unit(s_groups, experts, uint32_t(tiles1), rgb, G, GS, u - n0);
+  if (u < n0) b.units0[u] = plan_unit(s_groups, experts, uint32_t(tiles0), rgb, tgb, G, GS, u);
+  else b.units1[u - n0] = plan_unit(s_groups, experts, uint32_t(tiles1), rgb, tgb, G, GS, u - n0);
 }
 
 // Small cohorts (at most FFMOE_BOOK_SMALL_MAX assignments, one per thread): count, plan and stable fill in ONE launch of one
@@ -177,7 +182,7 @@ __global__ __launch_bounds__(256) void k_prefill_units(PrefillBook b, int expert
 // in LDS; an assignment's place in its expert's segment is the number of earlier assignments of that expert.
 constexpr int FFMOE_BOOK_SMALL_MAX = 1024;
 __global__ __launch_bounds__(1024) void k_prefill_book_small(const LiveTest lt, PrefillBook b, int A, int experts, int tm, int tiles0, int tiles1,
-                                                             int rgb, int shared_rows) {
+                                                             int rgb, int tgb, int shared_rows) {
   __shared__ PlanShared sh;
   __shared__ uint32_t s_cnt[1024];
   __shared__ __attribute__((aligned(16))) int s_id[FFMOE_BOOK_SMALL_MAX];
@@ -193,7 +198,7 @@ __global__ __launch_bounds__(1024) void k_prefill_book_small(const LiveTest lt, 
   __syncthreads();
   const uint32_t c = tid < experts ? s_cnt[tid] : 0u;
   if (tid < experts) b.counts[tid] = c;
-  prefill_plan_body(sh, b, experts, tm, tiles0, tiles1, rgb, shared_rows, c, true);
+  prefill_plan_body(sh, b, experts, tm, tiles0, tiles1, rgb, tgb, shared_rows, c, true);
   // position inside the expert's segment = number of earlier assignments of the same expert; every thread walks the same
   // LDS words (broadcast reads), four at a time
   uint32_t rank = 0;
@@ -340,14 +345,25 @@ int pick_mf(double avg, int cap) {
   return avg > 24.0 ? 4 : avg > 12.0 ? 2 : 1;
 }
 
+// column tiles per block of the unit order (k_prefill_plan)
+int pick_tgb() {
+  if (const char* f = getenv("FFMOE_PREFILL_TGB")) return max(1, atoi(f));
+  return 1 << 20;
+}
+
 // row groups of one expert that share a run of units (k_prefill_plan)
 int pick_rgb() {
   if (const char* f = getenv("FFMOE_PREFILL_RGB")) return max(1, atoi(f));
   return 32;  // measured at 4096 tokens, top-8 of 256, Zipf: 32 is 1 to 4 % ahead of unblocked on the gate/up launch (two seeded routings), 8 and below lose
 }
 
+// wide: 64-row groups with eight waves per block (twice the columns per unit and token tile), one block per CU
 template <int MODE>
-int launch_gemm(const GemmParams& p, int mf, unsigned blocks, hipStream_t stream) {
+int launch_gemm(const GemmParams& p, int mf, unsigned blocks, hipStream_t stream, bool wide = false) {
+  if (wide) {
+    hipLaunchKernelGGL((k_w8a8_grouped<4, MODE, 2, 8>), dim3(blocks), dim3(512), 0, stream, p);
+    return ff_launch_status();
+  }
   switch (mf) {
     case 1: hipLaunchKernelGGL((k_w8a8_grouped<1, MODE, 4>), dim3(blocks), dim3(256), 0, stream, p); break;
     case 2: hipLaunchKernelGGL((k_w8a8_grouped<2, MODE, 4>), dim3(blocks), dim3(256), 0, stream, p); break;
@@ -572,7 +588,10 @@ int prefill_impl(const ffmoe_expert_table* table, const ffmoe_prefill* args, int
                 (int*)(s + l.perm), (GemmGroup*)(s + l.groups), (u32x2*)(s + l.units0), (u32x2*)(s + l.units1)};
   const int mf = pick_mf(double(A) / E, (mx || a16) ? 4 : 8);
   const int tm = 16 * mf;
-  const int tiles0 = (I + 127) / 128, tiles1 = (H + 255) / 256;
+  // W8A8 cohorts in 64-row groups: eight waves per block share a token tile (FFMOE_PREFILL_WIDE=0: four, two blocks per CU)
+  bool wide = !a16 && !mx && mf == 4;
+  if (const char* f = getenv("FFMOE_PREFILL_WIDE")) wide = wide && atoi(f) != 0;
+  const int tiles0 = wide ? (I + 255) / 256 : (I + 127) / 128, tiles1 = wide ? (H + 511) / 512 : (H + 255) / 256;
   // A shared expert of the routed experts' format and width rides in the routed launches as further row groups (W*A16
   // cohorts): on its own it is a few dozen blocks per launch, which at small cohorts take longer than the routed experts'
   // thousands. FFMOE_PREFILL_SHARED_RIDE=0 keeps it in launches of its own (the results are the same bits either way).
@@ -588,13 +607,13 @@ int prefill_impl(const ffmoe_expert_table* table, const ffmoe_prefill* args, int
     if (const char* f = getenv("FFMOE_PREFILL_BOOK_SMALL")) small_max = std::max(0, std::min(atoi(f), FFMOE_BOOK_SMALL_MAX));
     const bool small = A <= size_t(small_max);
     if (small) {
-      hipLaunchKernelGGL(k_prefill_book_small, dim3(1), dim3(1024), 0, stream, lt, b, int(A), E, tm, tiles0, tiles1, pick_rgb(), ride ? R : 0);
+      hipLaunchKernelGGL(k_prefill_book_small, dim3(1), dim3(1024), 0, stream, lt, b, int(A), E, tm, tiles0, tiles1, pick_rgb(), pick_tgb(), ride ? R : 0);
     } else {
       hipLaunchKernelGGL(k_prefill_zero, dim3((E + 255) / 256), dim3(256), 0, stream, b.counts, E, b.totals);
       hipLaunchKernelGGL(k_prefill_count, dim3((unsigned)((A + FFMOE_COUNT_PER_BLOCK - 1) / FFMOE_COUNT_PER_BLOCK)), dim3(256), 0, stream, lt, b.counts, (long long)A);
-      hipLaunchKernelGGL(k_prefill_plan, dim3(1), dim3(1024), 0, stream, b, E, tm, tiles0, tiles1, pick_rgb(), ride ? R : 0);
+      hipLaunchKernelGGL(k_prefill_plan, dim3(1), dim3(1024), 0, stream, b, E, tm, tiles0, tiles1, pick_rgb(), pick_tgb(), ride ? R : 0);
       const uint64_t max_units = l.max_groups * uint64_t(tiles0 + tiles1);
-      hipLaunchKernelGGL(k_prefill_units, dim3((unsigned)((max_units + 255) / 256)), dim3(256), 0, stream, b, E, tm, tiles0, tiles1, pick_rgb(), ride ? R : 0);
+      hipLaunchKernelGGL(k_prefill_units, dim3((unsigned)((max_units + 255) / 256)), dim3(256), 0, stream, b, E, tm, tiles0, tiles1, pick_rgb(), pick_tgb(), ride ? R : 0);
       hipLaunchKernelGGL(k_prefill_fill, dim3(E), dim3(256), 0, stream, lt, b, (long long)A);
     }
     FF_TRY(ff_launch_status());
@@ -675,7 +694,7 @@ int prefill_impl(const ffmoe_expert_table* table, const ffmoe_prefill* args, int
   if (stages & 2) {  // gate/up + SwiGLU
     p.a_codes = s + l.xq; p.a_scales = (const float*)(s + l.sx); p.units = b.units0; p.unit_total = b.totals + 0;
     p.out = (uint16_t*)(s + l.act); p.K = H; p.N = I;
-    FF_TRY(launch_gemm<0>(p, mf, blocks, stream));
+    FF_TRY(launch_gemm<0>(p, mf, wide ? blocks / 2 : blocks, stream, wide));
   }
   if (stages & 4) {  // re-quantize the activations of the live rows
     const long long cells = (long long)A * (I / 128);
@@ -686,7 +705,7 @@ int prefill_impl(const ffmoe_expert_table* table, const ffmoe_prefill* args, int
   if (stages & 8) {  // down x routing weight, scattered to contributions[assignment]
     p.a_codes = s + l.aq; p.a_scales = (const float*)(s + l.sa); p.units = b.units1; p.unit_total = b.totals + 1;
     p.out = (uint16_t*)args->contributions; p.done = args->done; p.weights = args->weights; p.K = I; p.N = H;
-    FF_TRY(launch_gemm<1>(p, mf, blocks, stream));
+    FF_TRY(launch_gemm<1>(p, mf, wide ? blocks / 2 : blocks, stream, wide));
   }
   if (shared) {
     // the always-on expert: the same three steps over all rows in their own order (no grouping, no routing weight),

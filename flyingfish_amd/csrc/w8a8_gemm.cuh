@@ -45,14 +45,20 @@ struct GemmParams {
   float limit;
 };
 
-template <int MODE>
-__device__ __forceinline__ constexpr int gemm_tile_cols() { return MODE == 0 ? 128 : 256; }
+// output columns per unit: every wave owns 32 activation columns (gate and up rows) or 64 down columns
+template <int MODE, int NW = 4>
+__device__ __forceinline__ constexpr int gemm_tile_cols() { return (MODE == 0 ? 32 : 64) * NW; }
 
-template <int MF, int MODE, int P>
-__global__ __launch_bounds__(256, MF <= 4 ? 2 : 1) void k_w8a8_grouped(const GemmParams p) {
+// NW waves per block share one token tile in LDS. Blocks drift apart by more than a line lives in an XCD's L2 under the
+// weight stream, so a token tile that two blocks need is fetched twice (the fetch counters show every token read of a
+// cohort as an L2 miss, whatever the unit order); with NW = 8 one block per CU covers twice the columns per token tile
+// and the token traffic halves, at the same number of waves per CU as two blocks of four.
+template <int MF, int MODE, int P, int NW = 4>
+__global__ __launch_bounds__(64 * NW, (NW == 4 && MF <= 4) ? 2 : 1) void k_w8a8_grouped(const GemmParams p) {
   constexpr int TM = 16 * MF;
+  constexpr int NT = 64 * NW;                       // threads per block
   constexpr int CHUNKS = TM * 8;                    // 16-byte token chunks per K block
-  constexpr int CPT = (CHUNKS + 255) / 256;         // chunks a thread moves per K block
+  constexpr int CPT = (CHUNKS + NT - 1) / NT;       // chunks a thread moves per K block
   constexpr int TILE = TM * 128 + TM * 4;           // codes + scales
   constexpr int LPS = CPT + 1 + 8;                  // loads a thread issues per stage: token chunks, token scale, weights
   static_assert(CPT == 1 || CPT == 2 || CPT == 4, "token chunks per thread");
@@ -66,7 +72,7 @@ __global__ __launch_bounds__(256, MF <= 4 ? 2 : 1) void k_w8a8_grouped(const Gem
   // Short groups (MF < 4) are bound by HBM, not by the L1: they keep the direct requests and skip the LDS round trip.
   constexpr bool TW = MF >= 4;
   static_assert(!TW || P == 2, "the hand-counted waits of the long-group path assume two weight stages");
-  __shared__ __attribute__((aligned(16))) uint8_t wstage[TW ? 4 : 1][TW ? 4 : 1][TW ? 2048 : 16];  // [wave][fragment][16 rows x 128 B]
+  __shared__ __attribute__((aligned(16))) uint8_t wstage[TW ? NW : 1][TW ? 4 : 1][TW ? 2048 : 16];  // [wave][fragment][16 rows x 128 B]
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = uni(tid >> 6);
   const int K = p.K, N = p.N, KB = K >> 7;
@@ -74,7 +80,7 @@ __global__ __launch_bounds__(256, MF <= 4 ? 2 : 1) void k_w8a8_grouped(const Gem
   const int rd_lo = (lane & 15) * 128 + (((2 * (lane >> 4)) ^ (lane & 7)) << 4);
   const int rd_hi = (lane & 15) * 128 + (((2 * (lane >> 4) + 1) ^ (lane & 7)) << 4);
   const uint32_t total = p.unit_total ? uint32_t(uni(int(load_global<uint32_t>(p.unit_total)))) : p.total_units;
-  const int ntiles = (N + gemm_tile_cols<MODE>() - 1) / gemm_tile_cols<MODE>();
+  const int ntiles = (N + gemm_tile_cols<MODE, NW>() - 1) / gemm_tile_cols<MODE, NW>();
 
   // Blocks are dealt to the 8 XCDs round-robin, and each XCD has its own L2. The unit list is cut into 8 contiguous
   // spans, one per XCD, and the blocks of an XCD walk their span side by side, so the row groups of one (expert,
@@ -121,7 +127,7 @@ __global__ __launch_bounds__(256, MF <= 4 ? 2 : 1) void k_w8a8_grouped(const Gem
     uint64_t wfrag[4];
 #pragma unroll
     for (int f = 0; f < 4; ++f) {
-      col0[f] = MODE == 0 ? t * 128 + wave * 32 + (f & 1) * 16 : t * 256 + wave * 64 + f * 16;
+      col0[f] = MODE == 0 ? t * (32 * NW) + wave * 32 + (f & 1) * 16 : t * (64 * NW) + wave * 64 + f * 16;
       const int base = min(col0[f], N - 16);
       const uint64_t codes = MODE == 0 ? wc[f >> 1] : wc[0];
       wfrag[f] = uni64(codes + uint64_t(base) * uint64_t(K));
@@ -131,7 +137,7 @@ __global__ __launch_bounds__(256, MF <= 4 ? 2 : 1) void k_w8a8_grouped(const Gem
     const uint32_t woff0 = TW ? uint32_t(lane >> 3) * uint32_t(K) + uint32_t(lane & 7) * 16u : uint32_t(lane & 15) * uint32_t(K) + uint32_t(lane >> 4) * 32u;
     const uint32_t woff1 = woff0 + (TW ? 8u * uint32_t(K) : 16u);
     // block-scale rows: one per wave (its fragments sit inside one 128-row block), lane l keeps K block l (+64)
-    const int srow = min(MODE == 0 ? t * 128 + wave * 32 : t * 256 + wave * 64, N - 16) >> 7;
+    const int srow = min(MODE == 0 ? t * (32 * NW) + wave * 32 : t * (64 * NW) + wave * 64, N - 16) >> 7;
     const float* sw0 = reinterpret_cast<const float*>(ws[0]) + size_t(srow) * KB;
     const float* sw1 = reinterpret_cast<const float*>(ws[1]) + size_t(srow) * KB;
 
@@ -140,14 +146,14 @@ __global__ __launch_bounds__(256, MF <= 4 ? 2 : 1) void k_w8a8_grouped(const Gem
     int tdst[CPT];
 #pragma unroll
     for (int i = 0; i < CPT; ++i) {
-      const int q = min(tid + 256 * i, CHUNKS - 1);
+      const int q = min(tid + NT * i, CHUNKS - 1);
       const int m = q >> 3, c = q & 7;
       const int pos = start + min(m, n - 1);
       const int row = MODE == 0 && p.perm ? load_global<int>(p.perm + pos) / p.top_k : pos;
       tsrc[i] = p.a_codes + size_t(row) * K + c * 16;
       tdst[i] = m * 128 + ((c ^ (m & 7)) << 4);
     }
-    const bool stage_chunk = CHUNKS >= 256 || tid < CHUNKS;
+    const bool stage_chunk = CHUNKS >= NT || tid < CHUNKS;
     const float* ssrc;
     {
       const int pos = start + min(min(tid, TM - 1), n - 1);
@@ -332,6 +338,15 @@ __global__ __launch_bounds__(256, MF <= 4 ? 2 : 1) void k_w8a8_grouped(const Gem
 #pragma unroll
                   for (int r = 0; r < 4; ++r)
                     acc[m - 1][f][r] = __fmaf_rn(pr[(m - 1) & 1][f][r], sc[(m - 1) & 1][(MODE == 0 && f >= 2) ? 1 : 0], acc[m - 1][f][r]);
+                // The fmas have no ordering edge of their own, and instruction selection would emit all of them behind the
+                // last fence of the K block (64 product registers live, the VALU work after the matrix work instead of
+                // under it): an empty statement that reads the totals pins them in front of this fragment's fence.
+                if constexpr (TW) {
+#pragma unroll
+                  for (int f = 0; f < 4; ++f)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) asm volatile("" ::"v"(acc[m - 1][f][r]));
+                }
               }
               if constexpr (TW) __builtin_amdgcn_sched_barrier(0);
             }

@@ -361,7 +361,7 @@ def test_prefill_rows_do_not_depend_on_their_cohort():
 @pytest.mark.gpu
 @pytest.mark.parametrize("act_mode", [capi.ACT_FP8_BLOCK128, capi.ACT_BF16])
 def test_prefill_grouping_switches_leave_every_bit_alone(act_mode, monkeypatch):
-    """Rows per group (FFMOE_PREFILL_MF) and the order of the unit list (FFMOE_PREFILL_RGB) decide which block computes
+    """Rows per group (FFMOE_PREFILL_MF) and the order of the unit list (FFMOE_PREFILL_RGB, FFMOE_PREFILL_TGB) decide which block computes
     what, not what is computed: every setting gives the default run's contributions bit for bit. 700 rows over 6 skewed
     experts give groups of every length and experts with more row groups than the smallest blockings hold; a group
     size a path has no kernel for (8 on the BF16 matrix cores) falls back to its largest, an unknown value is ignored."""
@@ -373,14 +373,23 @@ def test_prefill_grouping_switches_leave_every_bit_alone(act_mode, monkeypatch):
     op = ops.PrefillOps(table, rows, top_k, act_mode=act_mode)
     monkeypatch.delenv("FFMOE_PREFILL_MF", raising=False)
     monkeypatch.delenv("FFMOE_PREFILL_RGB", raising=False)
+    monkeypatch.delenv("FFMOE_PREFILL_TGB", raising=False)
     ref = bits(op.contribute(x, ids_d, w_d)).copy()
     assert np.any(ref != 0)
-    for mf, rgb in [("1", "1"), ("1", "5"), ("2", "3"), ("4", "2"), ("4", "1000000"), ("8", "1"), ("8", "4"), ("3", "0"), ("4", "32")]:
+    for wide in ("0", "1"):   # 64-row groups on the FP8 path: four or eight waves per block
+        monkeypatch.setenv("FFMOE_PREFILL_MF", "4")
+        monkeypatch.setenv("FFMOE_PREFILL_WIDE", wide)
+        op.contributions.zero_()
+        assert np.array_equal(bits(op.contribute(x, ids_d, w_d)), ref), "FFMOE_PREFILL_WIDE=%s changes the result" % wide
+    monkeypatch.delenv("FFMOE_PREFILL_WIDE")
+    for mf, rgb, tgb in [("1", "1", "1"), ("1", "5", "2"), ("2", "3", "1000000"), ("4", "2", "3"), ("4", "1000000", "1"), ("8", "1", "4"),
+                         ("8", "4", "2"), ("3", "0", "0"), ("4", "32", "4"), ("4", "16", "5")]:
         monkeypatch.setenv("FFMOE_PREFILL_MF", mf)
         monkeypatch.setenv("FFMOE_PREFILL_RGB", rgb)
+        monkeypatch.setenv("FFMOE_PREFILL_TGB", tgb)
         op.contributions.zero_()
         got = bits(op.contribute(x, ids_d, w_d))
-        assert np.array_equal(got, ref), "FFMOE_PREFILL_MF=%s FFMOE_PREFILL_RGB=%s changes the result" % (mf, rgb)
+        assert np.array_equal(got, ref), "FFMOE_PREFILL_MF=%s FFMOE_PREFILL_RGB=%s FFMOE_PREFILL_TGB=%s changes the result" % (mf, rgb, tgb)
 
 
 @pytest.mark.parametrize("fmt", [capi.FMT_FP8_BLOCK128, capi.FMT_NVFP4, capi.FMT_BF16, capi.FMT_FP8_CHANNEL])
