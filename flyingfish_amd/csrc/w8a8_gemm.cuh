@@ -253,6 +253,20 @@ __global__ __launch_bounds__(64 * NW, (NW == 4 && MF <= 4) ? 2 : 1) void k_w8a8_
     const int thi0 = trow0 * 128 + (((q2 + 1) ^ (trow0 & 7)) << 4);
     const int tsx0 = TM * 128 + trow0 * 4;
 
+    // 64-row groups keep LDS latency off the matrix core's path: the operand-order weight fragments of a stage are read at
+    // the end of the stage before (behind the token publication and the barrier), and the token fragment of row fragment
+    // m + 1 is read before the matrix instructions of fragment m are issued.
+    constexpr bool PF = TW && MF == 4;
+    u32x4 wt[4][2];  // the four weight fragments in operand order
+    if constexpr (PF) {
+      const uint8_t* wl0 = &wstage[wave][0][0];
+#pragma unroll
+      for (int f = 0; f < 4; ++f) {
+        wt[f][0] = *reinterpret_cast<const u32x4*>(wl0 + f * 2048 + rd_lo);
+        wt[f][1] = *reinterpret_cast<const u32x4*>(wl0 + f * 2048 + rd_hi);
+      }
+      __builtin_amdgcn_wave_barrier();
+    }
     for (int kb0 = 0; kb0 < KB; kb0 += 64) {
       // block scales of K blocks kb0 .. kb0+63, one per lane; the next 64 are requested right away
       const float swl0 = landed(swn0);
@@ -273,13 +287,12 @@ __global__ __launch_bounds__(64 * NW, (NW == 4 && MF <= 4) ? 2 : 1) void k_w8a8_
             const float s1 = MODE == 0 ? __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, swl1), kb - kb0)) : s0;
             // every row fragment is computed, also the padding of a short group: straight-line code lets the matrix
             // core overlap with the scale fmas, and short groups are bandwidth-bound anyway
-            u32x4 wt[4][2];  // the four fragments in operand order
             uint8_t* wl = &wstage[TW ? wave : 0][0][0];
             if constexpr (!TW) {
               wait_loads<WAIT_W>(w[s][0][0], w[s][0][1], w[s][1][0], w[s][1][1], w[s][2][0], w[s][2][1], w[s][3][0], w[s][3][1]);
 #pragma unroll
               for (int f = 0; f < 4; ++f) { wt[f][0] = w[s][f][0]; wt[f][1] = w[s][f][1]; }
-            } else {
+            } else if constexpr (!PF) {
 #pragma unroll
               for (int f = 0; f < 4; ++f) {
                 wt[f][0] = *reinterpret_cast<const u32x4*>(wl + f * 2048 + rd_lo);
@@ -291,12 +304,24 @@ __global__ __launch_bounds__(64 * NW, (NW == 4 && MF <= 4) ? 2 : 1) void k_w8a8_
             // fragments' worth of product registers are live instead of MF (the scheduling fences keep that order).
             v4f pr[2][4];
             float sc[2][2];
+            u32x4 tfl[2], tfh[2];  // token fragment pieces, two row fragments in rotation
+            float tfs[2];
+            if constexpr (PF) {
+              tfl[0] = *reinterpret_cast<const u32x4*>(tb + tlo0);
+              tfh[0] = *reinterpret_cast<const u32x4*>(tb + thi0);
+              tfs[0] = *reinterpret_cast<const float*>(tb + tsx0);
+            }
 #pragma unroll
             for (int m = 0; m <= MF; ++m) {
               if (m < MF) {
-                const u32x4 lo = *reinterpret_cast<const u32x4*>(tb + tlo0 + m * 2048);
-                const u32x4 hi = *reinterpret_cast<const u32x4*>(tb + thi0 + m * 2048);
-                const float sx = *reinterpret_cast<const float*>(tb + tsx0 + m * 64);
+                constexpr int ahead = PF ? 1 : 0;
+                if (!PF || m + 1 < MF) {
+                  tfl[(m + ahead) & 1] = *reinterpret_cast<const u32x4*>(tb + tlo0 + (m + ahead) * 2048);
+                  tfh[(m + ahead) & 1] = *reinterpret_cast<const u32x4*>(tb + thi0 + (m + ahead) * 2048);
+                  tfs[(m + ahead) & 1] = *reinterpret_cast<const float*>(tb + tsx0 + (m + ahead) * 64);
+                }
+                const u32x4 lo = tfl[m & 1], hi = tfh[m & 1];
+                const float sx = tfs[m & 1];
                 const v8i tok = {int(lo[0]), int(lo[1]), int(lo[2]), int(lo[3]), int(hi[0]), int(hi[1]), int(hi[2]), int(hi[3])};
                 sc[m & 1][0] = __fmul_rn(s0, sx);
                 sc[m & 1][1] = __fmul_rn(s1, sx);
@@ -349,6 +374,14 @@ __global__ __launch_bounds__(64 * NW, (NW == 4 && MF <= 4) ? 2 : 1) void k_w8a8_
                 }
               }
               if constexpr (TW) __builtin_amdgcn_sched_barrier(0);
+            }
+            if constexpr (PF) {  // K block kb+1 sits in the transposition buffer by now: its fragments for the next stage
+#pragma unroll
+              for (int f = 0; f < 4; ++f) {
+                wt[f][0] = *reinterpret_cast<const u32x4*>(wl + f * 2048 + rd_lo);
+                wt[f][1] = *reinterpret_cast<const u32x4*>(wl + f * 2048 + rd_hi);
+              }
+              __builtin_amdgcn_wave_barrier();
             }
             // publish token tile kb+1
             FF_WAIT_TOKENS(8);
