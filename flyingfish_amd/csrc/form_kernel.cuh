@@ -183,6 +183,151 @@ __global__ __launch_bounds__(256) void k_decode_form(const DecodeParams p) {
   }
 }
 
+// The same dot product for up to RG activation rows at once: a weight word is loaded once and every row keeps its own
+// accumulators, so each (row, column) result is the chain of form_dot bit for bit. n = live rows (uniform in the block).
+template <class F, int FORM, int RG>
+__device__ __forceinline__ void form_dot_rows(const uint8_t* xs, int xstride, int n, const FormRow<F>& row, int K, int sub, float (&out)[RG]) {
+  float x[8], w[8];
+  if (FORM == FFMOE_FORM_LANE16_) {
+    float acc[RG][8];
+#pragma unroll
+    for (int r = 0; r < RG; ++r)
+#pragma unroll
+      for (int t = 0; t < 8; ++t) acc[r][t] = 0.0f;
+    for (int k0 = 8 * sub; k0 < K; k0 += 16) {
+      row.load8(k0, w);
+#pragma unroll
+      for (int r = 0; r < RG; ++r) {
+        if (r < n) {
+          form_x8(xs + size_t(r) * xstride, k0, x);
+#pragma unroll
+          for (int t = 0; t < 8; ++t) acc[r][t] = __fmaf_rn(x[t], w[t], acc[r][t]);
+        }
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < RG; ++r) {
+      const float half = __fadd_rn(__fadd_rn(__fadd_rn(acc[r][0], acc[r][1]), __fadd_rn(acc[r][2], acc[r][3])),
+                                   __fadd_rn(__fadd_rn(acc[r][4], acc[r][5]), __fadd_rn(acc[r][6], acc[r][7])));
+      const float other = lane_xor(half, 1);
+      out[r] = sub == 0 ? __fadd_rn(half, other) : __fadd_rn(other, half);
+    }
+    return;
+  }
+  float acc[RG];
+#pragma unroll
+  for (int r = 0; r < RG; ++r) acc[r] = 0.0f;
+  for (int k0 = 8 * sub; k0 < K; k0 += 64) {
+    row.load8(k0, w);
+#pragma unroll
+    for (int r = 0; r < RG; ++r) {
+      if (r < n) {
+        form_x8(xs + size_t(r) * xstride, k0, x);
+        float inner = 0.0f;
+#pragma unroll
+        for (int t = 0; t < 8; ++t) inner = __fmaf_rn(x[t], w[t], inner);
+        acc[r] = __fadd_rn(acc[r], inner);
+      }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < RG; ++r) {
+    float a = acc[r];
+    float o = lane_xor(a, 4);
+    a = (sub & 4) ? __fadd_rn(o, a) : __fadd_rn(a, o);
+    o = lane_xor(a, 2);
+    a = (sub & 2) ? __fadd_rn(o, a) : __fadd_rn(a, o);
+    o = lane_xor(a, 1);
+    a = (sub & 1) ? __fadd_rn(o, a) : __fadd_rn(a, o);
+    out[r] = a;
+  }
+}
+
+// Token-sorted form of k_decode_form: grid (ceil(out / ROWS), groups). A block takes one group of up to RG assignments of
+// one expert (k_group_assignments; the shared expert's rows come as groups of their own), stages their activation rows
+// in LDS and streams each weight row once for all of them. The reference's grouped kernels read a weight row once per
+// (row, column) and leave the reuse to the cache (kernels/moe_prefill.cu:13-71); the results are the same bits.
+template <class F, int FORM, int STAGE, int RG>
+__global__ __launch_bounds__(256) void k_decode_form_grouped(const DecodeParams p) {
+  constexpr int LPR = FORM == FFMOE_FORM_LANE16_ ? 2 : 8;
+  constexpr int ROWS = 256 / LPR;
+  extern __shared__ __align__(16) uint8_t xs[];
+  const int tid = threadIdx.x;
+  const int g = blockIdx.y;
+  const int n_routed = uni(load_global<int>(p.counters)), n_shared = uni(load_global<int>(p.counters + 1));
+  if (g >= n_routed + n_shared) return;
+  int expert, gn, grow[RG], gslot[RG];
+  load_group<RG>(p, g, expert, gn, grow, gslot);
+  if (gn == 0) return;
+  const bool is_shared = expert < 0;
+  const int Kg = STAGE == 0 ? p.hidden : (is_shared ? p.shared_inter : p.inter);
+  const int out = STAGE == 0 ? (is_shared ? p.shared_inter : p.inter) : p.hidden;
+  if (int(blockIdx.x) * ROWS >= out) return;
+  const int xstride = Kg * 2;
+#pragma unroll
+  for (int r = 0; r < RG; ++r) {
+    if (r < gn) {
+      const uint16_t* src = STAGE == 0 ? p.x + size_t(grow[r]) * p.hidden : p.h + size_t(gslot[r]) * p.h_stride;
+      u32x4* d4 = reinterpret_cast<u32x4*>(xs + size_t(r) * xstride);
+      for (int v = tid; v < (Kg >> 3); v += 256) d4[v] = load16(src + size_t(v) * 8);
+    }
+  }
+  __syncthreads();
+  const int j = blockIdx.x * ROWS + tid / LPR;
+  const int sub = tid % LPR;
+  if (j >= out) return;
+  uint64_t sl[6];
+#pragma unroll
+  for (int i = 0; i < 6; ++i) sl[i] = is_shared ? p.shared_slot[i] : p.slots[size_t(expert) * 6 + i];
+  if (STAGE == 0) {
+    const FormRow<F> gate(sl[0], sl[1], j, Kg), up(sl[2], sl[3], j, Kg);
+    float gv[RG], uv[RG];
+    form_dot_rows<F, FORM, RG>(xs, xstride, gn, gate, Kg, sub, gv);
+    form_dot_rows<F, FORM, RG>(xs, xstride, gn, up, Kg, sub, uv);
+    const bool reciprocal = FORM == FFMOE_FORM_LANE16_ && (p.swiglu == FFMOE_SWIGLU_TWICE || p.swiglu == FFMOE_SWIGLU_CLAMPED_TWICE);
+    if (sub == 0) {
+#pragma unroll
+      for (int r = 0; r < RG; ++r)
+        if (r < gn) p.h[size_t(gslot[r]) * p.h_stride + j] = form_swiglu(bround(gv[r]), bround(uv[r]), p.swiglu, p.swiglu_limit, reciprocal);
+    }
+  } else {
+    const FormRow<F> down(sl[4], sl[5], j, Kg);
+    float dv[RG];
+    form_dot_rows<F, FORM, RG>(xs, xstride, gn, down, Kg, sub, dv);
+    if (sub == 0) {
+#pragma unroll
+      for (int r = 0; r < RG; ++r) {
+        if (r < gn) {
+          if (is_shared) {
+            p.shared_out[size_t(grow[r]) * p.hidden + j] = f32_to_bf16(dv[r]);
+          } else {
+            const float wk = p.weights_f32 ? reinterpret_cast<const float*>(p.weights)[gslot[r]]
+                                           : bf16_to_f32(reinterpret_cast<const uint16_t*>(p.weights)[gslot[r]]);
+            const float v = __fmul_rn(p.routed_weight == FFMOE_WEIGHT_AFTER_DOWN_BF16 ? bround(dv[r]) : dv[r], wk);
+            p.contributions[size_t(gslot[r]) * p.hidden + j] = f32_to_bf16(v);
+            if (j == 0 && p.done) p.done[gslot[r]] = 1u;
+          }
+        }
+      }
+    }
+  }
+}
+
+template <class F, int FORM, int RG>
+int launch_form_grouped(const DecodeParams& p, unsigned max_groups, int stage_mask, hipStream_t st) {
+  constexpr int ROWS = 256 / (FORM == FFMOE_FORM_LANE16_ ? 2 : 8);
+  const int imax = p.inter > p.shared_inter ? p.inter : p.shared_inter;
+  if (stage_mask & 1) {
+    hipLaunchKernelGGL((k_decode_form_grouped<F, FORM, 0, RG>), dim3((imax + ROWS - 1) / ROWS, max_groups), dim3(256), size_t(RG) * p.hidden * 2, st, p);
+    FF_TRY(ff_launch_status());
+  }
+  if (stage_mask & 2) {
+    hipLaunchKernelGGL((k_decode_form_grouped<F, FORM, 1, RG>), dim3((p.hidden + ROWS - 1) / ROWS, max_groups), dim3(256), size_t(RG) * imax * 2, st, p);
+    FF_TRY(ff_launch_status());
+  }
+  return 0;
+}
+
 template <class F, int FORM>
 int launch_form(const DecodeParams& p, int stage_mask, hipStream_t st) {
   constexpr int ROWS = 256 / (FORM == FFMOE_FORM_LANE16_ ? 2 : 8);

@@ -121,10 +121,9 @@ def test_reference_summation_orders_seeded_sweep(seed):
 
 @pytest.mark.parametrize("form", [capi.FORM_LANE16, capi.FORM_LANE8])
 def test_reference_summation_orders_take_whole_cohorts(form):
-    """More assignments than the streaming decode path groups in one call (600 rows x 8 choices): the reduction-order
-    kernels have no grouping pass, so a prefill cohort runs through the same entry, bit-equal row by row - the
-    arithmetic of the reference's moe_gemm_lane16 pipeline (kernels/moe_prefill.cu:13-71: one 16-lane chain per (row,
-    column), no weight reuse across rows)."""
+    """A prefill cohort (600 rows x 8 choices) through the same entry, bit-equal row by row - the arithmetic of the
+    reference's moe_gemm_lane16 pipeline (kernels/moe_prefill.cu:13-71: one 16-lane chain per (row, column)); here the
+    assignments are sorted by expert and a group of rows shares one pass over the expert's weights."""
     experts, hidden, inter, rows, top_k = 12, 128, 64, 600, 8
     table, ref, sh, x, ids, wt = _case(capi.FMT_BF16, experts, hidden, inter, rows, top_k, 7600 + form, True)
     op = DecodeOps(table, sh, rows, top_k, capi.ACT_BF16, capi.SWIGLU_TWICE, 0.0, capi.WEIGHT_AFTER_DOWN_BF16, True)
@@ -139,6 +138,36 @@ def test_reference_summation_orders_take_whole_cohorts(form):
             assert np.array_equal(got[r, c], want), (r, c)
         assert np.array_equal(got_sh[r], orc.expert_ffn(xb[r], *ref[experts], 1.0, orc.TWICE, 0.0, 0, oform, kind, apply_weight=False)), r
     assert int(op.done.sum().item()) == rows * top_k
+
+
+@pytest.mark.parametrize("fmt", [capi.FMT_BF16, capi.FMT_FP8_CHANNEL])
+@pytest.mark.parametrize("form", [capi.FORM_LANE16, capi.FORM_LANE8])
+@pytest.mark.parametrize("rows,hidden,inter", [(70, 784, 208), (9, 4608, 512), (2, 256, 128)])
+def test_token_sorted_form_kernels_equal_one_block_per_choice(fmt, form, rows, hidden, inter, monkeypatch):
+    """Rows of one expert share a pass over its weights (groups of 8, or as many rows as fit LDS: 4 at hidden 4608):
+    contributions, shared output and done flags are the bits of the kernels that run one block per (row, choice)
+    (FFMOE_FORM_GROUPED=0), with masked, invalid and out-of-range choices in the batch and widths that are 8 mod 16."""
+    experts, top_k = 5, 3
+    table, ref, sh, x, ids, wt = _case(fmt, experts, hidden, inter, rows, top_k, 8100 + rows + form, True)
+    ids = ids.clone()
+    active = (torch.rand((rows, top_k), generator=synth.generator(8200 + rows)) > 0.25).to(torch.int32)
+    ids[rows - 1, 0] = experts + 2
+    valid = torch.ones(experts, dtype=torch.int32)
+    valid[1] = 0
+    table.valid = valid.to(DEV)
+    out = {}
+    for grouped in ("0", "1"):
+        monkeypatch.setenv("FFMOE_FORM_GROUPED", grouped)
+        op = DecodeOps(table, sh, rows, top_k, capi.ACT_BF16, capi.SWIGLU_CLAMPED_TWICE, 0.7, capi.WEIGHT_BEFORE_CONTRIBUTION_BF16, True)
+        op.contributions.zero_(); op.shared_out.zero_(); op.done.zero_()
+        contrib, shared_out = op.contribute(x.to(DEV), ids.to(DEV), wt.to(DEV), active.to(DEV), form=form)
+        torch.cuda.synchronize()
+        out[grouped] = (bits(contrib).copy(), bits(shared_out).copy(), op.done.cpu().numpy().copy())
+    assert np.any(out["0"][0] != 0) and np.any(out["0"][1] != 0)
+    for a, b, what in zip(out["0"], out["1"], ("contributions", "shared_out", "done")):
+        assert np.array_equal(a, b), what
+    live = (active.numpy() != 0) & (ids.numpy() < experts) & (ids.numpy() != 1)
+    assert np.array_equal(out["1"][2].reshape(rows, top_k) != 0, live)
 
 
 def test_form_entry_rejects_other_formats():
