@@ -374,7 +374,11 @@ int launch_gemm(const GemmParams& p, int mf, unsigned blocks, hipStream_t stream
 }
 
 template <class F, int MODE>
-int launch_w16(const W16Params& p, int mf, unsigned blocks, hipStream_t stream) {
+int launch_w16(const W16Params& p, int mf, unsigned blocks, hipStream_t stream, bool wide = false) {
+  if (wide) {  // 64-row groups, eight waves per block, one block per CU
+    hipLaunchKernelGGL((k_w16_grouped<F, 4, MODE, 2, 8>), dim3(blocks), dim3(512), 0, stream, p);
+    return ff_launch_status();
+  }
   switch (mf) {
     case 1: hipLaunchKernelGGL((k_w16_grouped<F, 1, MODE, 2>), dim3(blocks), dim3(256), 0, stream, p); break;
     case 2: hipLaunchKernelGGL((k_w16_grouped<F, 2, MODE, 2>), dim3(blocks), dim3(256), 0, stream, p); break;
@@ -383,12 +387,12 @@ int launch_w16(const W16Params& p, int mf, unsigned blocks, hipStream_t stream) 
   return ff_launch_status();
 }
 template <int MODE>
-int launch_w16_fmt(int format, const W16Params& p, int mf, unsigned blocks, hipStream_t stream) {
+int launch_w16_fmt(int format, const W16Params& p, int mf, unsigned blocks, hipStream_t stream, bool wide = false) {
   switch (format) {
-    case FFMOE_FMT_FP8_BLOCK128: return launch_w16<FmtFp8, MODE>(p, mf, blocks, stream);
-    case FFMOE_FMT_NVFP4: return launch_w16<FmtNvfp4, MODE>(p, mf, blocks, stream);
-    case FFMOE_FMT_FP8_CHANNEL: return launch_w16<FmtFp8Channel, MODE>(p, mf, blocks, stream);
-    default: return launch_w16<FmtBf16, MODE>(p, mf, blocks, stream);
+    case FFMOE_FMT_FP8_BLOCK128: return launch_w16<FmtFp8, MODE>(p, mf, blocks, stream, wide);
+    case FFMOE_FMT_NVFP4: return launch_w16<FmtNvfp4, MODE>(p, mf, blocks, stream, wide);
+    case FFMOE_FMT_FP8_CHANNEL: return launch_w16<FmtFp8Channel, MODE>(p, mf, blocks, stream, wide);
+    default: return launch_w16<FmtBf16, MODE>(p, mf, blocks, stream, wide);
   }
 }
 
@@ -588,8 +592,8 @@ int prefill_impl(const ffmoe_expert_table* table, const ffmoe_prefill* args, int
                 (int*)(s + l.perm), (GemmGroup*)(s + l.groups), (u32x2*)(s + l.units0), (u32x2*)(s + l.units1)};
   const int mf = pick_mf(double(A) / E, (mx || a16) ? 4 : 8);
   const int tm = 16 * mf;
-  // W8A8 cohorts in 64-row groups: eight waves per block share a token tile (FFMOE_PREFILL_WIDE=0: four, two blocks per CU)
-  bool wide = !a16 && !mx && mf == 4;
+  // W8A8 and W*A16 cohorts in 64-row groups: eight waves per block share a token tile (FFMOE_PREFILL_WIDE=0: four, two blocks per CU)
+  bool wide = !mx && mf == 4;
   if (const char* f = getenv("FFMOE_PREFILL_WIDE")) wide = wide && atoi(f) != 0;
   const int tiles0 = wide ? (I + 255) / 256 : (I + 127) / 128, tiles1 = wide ? (H + 511) / 512 : (H + 255) / 256;
   // A shared expert of the routed experts' format and width rides in the routed launches as further row groups (W*A16
@@ -675,13 +679,13 @@ int prefill_impl(const ffmoe_expert_table* table, const ffmoe_prefill* args, int
       p.a = (const uint16_t*)args->x; p.units = b.units0; p.unit_total = b.totals + 0;
       p.out = (uint16_t*)(s + l.act); p.K = H; p.N = I;
       p.a_sh = (const uint16_t*)args->x; p.out_sh = (uint16_t*)(s + l.sh_act);
-      FF_TRY(launch_w16_fmt<0>(table->format, p, mf, blocks, stream));
+      FF_TRY(launch_w16_fmt<0>(table->format, p, mf, wide ? blocks / 2 : blocks, stream, wide));
     }
     if (stages & 8) {
       p.a = (const uint16_t*)(s + l.act); p.units = b.units1; p.unit_total = b.totals + 1;
       p.out = (uint16_t*)args->contributions; p.done = args->done; p.weights = args->weights; p.K = I; p.N = H;
       p.a_sh = (const uint16_t*)(s + l.sh_act); p.out_sh = (uint16_t*)args->shared_out;
-      FF_TRY(launch_w16_fmt<1>(table->format, p, mf, blocks, stream));
+      FF_TRY(launch_w16_fmt<1>(table->format, p, mf, wide ? blocks / 2 : blocks, stream, wide));
     }
     if (shared && !ride)
       FF_TRY(shared_expert_w16(shared, args->x, R, H, args->swiglu, args->swiglu_limit, s + l.sh_act, args->shared_out,

@@ -150,21 +150,23 @@ struct W16Params {
   uint16_t* out_sh;
 };
 
-template <class F, int MF, int MODE, int P>
-__global__ __launch_bounds__(256, 2) void k_w16_grouped(const W16Params p) {
+// NW waves per block share one token tile (see k_w8a8_grouped): eight for 64-row groups of a cohort, one block per CU.
+template <class F, int MF, int MODE, int P, int NW = 4>
+__global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void k_w16_grouped(const W16Params p) {
+  constexpr int NT = 64 * NW;
   constexpr int TM = 16 * MF;
   constexpr int CHUNKS = TM * 8;             // 16-byte token chunks per K block (64 BF16 columns = 128 bytes per row)
-  constexpr int CPT = (CHUNKS + 255) / 256;
+  constexpr int CPT = (CHUNKS + NT - 1) / NT;
   constexpr int TILE = TM * 128;
   constexpr bool TR = W16Transpose<F>::value;
   // NVFP4: a row's K block is 32 code bytes and 4 scale bytes. Two lanes request one row's codes (32 rows = two
   // fragments per instruction), the scale bytes of a row come as one word, and both are turned into operand order
   // (8 code bytes and one scale byte per lane) through wave-private LDS, like the FP8 formats below.
   constexpr bool NVT = std::is_same<F, FmtNvfp4>::value;
-  __shared__ __attribute__((aligned(16))) uint8_t nstage[NVT ? 4 : 1][NVT ? 2 : 1][NVT ? 1024 : 16];  // [wave][row pair of fragments][32 rows x 32 B]
-  __shared__ uint32_t nscale[NVT ? 4 : 1][NVT ? 2 : 1][NVT ? 32 : 1];
+  __shared__ __attribute__((aligned(16))) uint8_t nstage[NVT ? NW : 1][NVT ? 2 : 1][NVT ? 1024 : 16];  // [wave][row pair of fragments][32 rows x 32 B]
+  __shared__ uint32_t nscale[NVT ? NW : 1][NVT ? 2 : 1][NVT ? 32 : 1];
   __shared__ __attribute__((aligned(16))) uint8_t tile[2][TILE];
-  __shared__ __attribute__((aligned(16))) uint8_t wstage[TR ? 4 : 1][TR ? 4 : 1][TR ? 1024 : 16];  // [wave][fragment][16 rows x 64 B]
+  __shared__ __attribute__((aligned(16))) uint8_t wstage[TR ? NW : 1][TR ? 4 : 1][TR ? 1024 : 16];  // [wave][fragment][16 rows x 64 B]
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = uni(tid >> 6);
   const int K = p.K, N = p.N, KB = K >> 6;
@@ -173,7 +175,7 @@ __global__ __launch_bounds__(256, 2) void k_w16_grouped(const W16Params p) {
   const int wr_off = (lane >> 2) * 64 + (((lane & 3) ^ ((lane >> 4) & 3)) << 4);
   const int rd_off = (lane & 15) * 64 + (((lane >> 4) ^ ((lane >> 2) & 3)) << 4);
   const uint32_t total = p.unit_total ? uint32_t(uni(int(load_global<uint32_t>(p.unit_total)))) : p.total_units;
-  const int ntiles = (N + gemm_tile_cols<MODE>() - 1) / gemm_tile_cols<MODE>();
+  const int ntiles = (N + gemm_tile_cols<MODE, NW>() - 1) / gemm_tile_cols<MODE, NW>();
 
   // one contiguous span of the unit list per XCD (see k_w8a8_grouped)
   const uint32_t xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3, per_xcd = gridDim.x >> 3;
@@ -227,7 +229,7 @@ __global__ __launch_bounds__(256, 2) void k_w16_grouped(const W16Params p) {
     typename W16<F>::Row wrow[4];
 #pragma unroll
     for (int f = 0; f < 4; ++f) {
-      col0[f] = MODE == 0 ? t * 128 + wave * 32 + (f & 1) * 16 : t * 256 + wave * 64 + f * 16;
+      col0[f] = MODE == 0 ? t * (32 * NW) + wave * 32 + (f & 1) * 16 : t * (64 * NW) + wave * 64 + f * 16;
       const int base = min(col0[f], N - 16);
       const int which = MODE == 0 ? f >> 1 : 0;
       wrow[f] = W16<F>::row(wc[which], ws[which], gl[which], base + (lane & 15), K);
@@ -264,14 +266,14 @@ __global__ __launch_bounds__(256, 2) void k_w16_grouped(const W16Params p) {
     int tdst[CPT];
 #pragma unroll
     for (int i = 0; i < CPT; ++i) {
-      const int q = min(tid + 256 * i, CHUNKS - 1);
+      const int q = min(tid + NT * i, CHUNKS - 1);
       const int m = q >> 3, c = q & 7;
       const int pos = start + min(m, n - 1);
       const int row = MODE == 0 && p.perm && !ride ? load_global<int>(p.perm + pos) / p.top_k : pos;
       tsrc[i] = reinterpret_cast<const uint8_t*>(ride ? p.a_sh : p.a) + size_t(row) * K * 2 + c * 16;
       tdst[i] = m * 128 + ((c ^ (m & 7)) << 4);
     }
-    const bool stage_chunk = CHUNKS >= 256 || tid < CHUNKS;
+    const bool stage_chunk = CHUNKS >= NT || tid < CHUNKS;
 
     v4f acc[MF][4];
 #pragma unroll
