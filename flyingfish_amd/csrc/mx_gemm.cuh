@@ -45,11 +45,13 @@ struct MxParams {
 
 // PACKED 1: E2M1 codes [N, K / 2] (low nibble = even column), E8M0 scales [N, K / 32]
 // PACKED 0: E4M3 codes [N, K], E8M0 scales [N / 32, K / 32]
-template <int MF, int MODE, int PACKED, int P>
-__global__ __launch_bounds__(256, 2) void k_mx_grouped(const MxParams p) {
+// NW waves per block share one token tile (see k_w8a8_grouped): eight for 64-row groups of a cohort, one block per CU.
+template <int MF, int MODE, int PACKED, int P, int NW = 4>
+__global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void k_mx_grouped(const MxParams p) {
   constexpr int TM = 16 * MF;
+  constexpr int NT = 64 * NW;
   constexpr int CHUNKS = TM * 8;
-  constexpr int CPT = (CHUNKS + 255) / 256;
+  constexpr int CPT = (CHUNKS + NT - 1) / NT;
   constexpr int TILE = TM * 128 + TM * 4;  // codes + the K block's four scale bytes per row
   constexpr int WL = PACKED ? 1 : 2;        // 16-byte loads per lane, fragment and K block
   __shared__ __attribute__((aligned(16))) uint8_t tile[2][TILE];
@@ -58,15 +60,15 @@ __global__ __launch_bounds__(256, 2) void k_mx_grouped(const MxParams p) {
   // k_w16_grouped does: requested in operand order, every lane touches a line of its own for 16 bytes, and once more
   // for one scale byte. LDS operations of one wave execute in order, so no wait sits between the writes and the reads.
   constexpr bool TW = PACKED != 0;
-  __shared__ __attribute__((aligned(16))) uint8_t wstage[TW ? 4 : 1][TW ? 4 : 1][TW ? 1024 : 16];
-  __shared__ uint32_t sstage[TW ? 4 : 1][TW ? 4 : 1][TW ? 16 : 1];
+  __shared__ __attribute__((aligned(16))) uint8_t wstage[TW ? NW : 1][TW ? 4 : 1][TW ? 1024 : 16];
+  __shared__ uint32_t sstage[TW ? NW : 1][TW ? 4 : 1][TW ? 16 : 1];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = uni(tid >> 6);
   const int K = p.K, N = p.N, KB = K >> 7, SB = K >> 5;
   const int wr_off = (lane >> 2) * 64 + (((lane & 3) ^ ((lane >> 4) & 3)) << 4);
   const int rd_off = (lane & 15) * 64 + (((lane >> 4) ^ ((lane >> 2) & 3)) << 4);
   const uint32_t total = p.unit_total ? uint32_t(uni(int(load_global<uint32_t>(p.unit_total)))) : p.total_units;
-  const int ntiles = (N + gemm_tile_cols<MODE>() - 1) / gemm_tile_cols<MODE>();
+  const int ntiles = (N + gemm_tile_cols<MODE, NW>() - 1) / gemm_tile_cols<MODE, NW>();
   const int q4 = lane >> 4;  // this lane's scale block inside a K block
 
   const uint32_t xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3, per_xcd = gridDim.x >> 3;
@@ -107,7 +109,7 @@ __global__ __launch_bounds__(256, 2) void k_mx_grouped(const MxParams p) {
     const uint8_t* srow[4];   // this lane's scale byte of K block 0
 #pragma unroll
     for (int f = 0; f < 4; ++f) {
-      col0[f] = MODE == 0 ? t * 128 + wave * 32 + (f & 1) * 16 : t * 256 + wave * 64 + f * 16;
+      col0[f] = MODE == 0 ? t * (32 * NW) + wave * 32 + (f & 1) * 16 : t * (64 * NW) + wave * 64 + f * 16;
       const int which = MODE == 0 ? f >> 1 : 0;
       if (TW) {  // row lane / 4 of the fragment, 16-byte piece lane % 4; the row's scale word
         const int row = min(col0[f], N - 16) + (lane >> 2);
@@ -124,14 +126,14 @@ __global__ __launch_bounds__(256, 2) void k_mx_grouped(const MxParams p) {
     int tdst[CPT];
 #pragma unroll
     for (int i = 0; i < CPT; ++i) {
-      const int q = min(tid + 256 * i, CHUNKS - 1);
+      const int q = min(tid + NT * i, CHUNKS - 1);
       const int m = q >> 3, c = q & 7;
       const int pos = start + min(m, n - 1);
       const int row = MODE == 0 && p.perm ? load_global<int>(p.perm + pos) / p.top_k : pos;
       tsrc[i] = p.a_codes + size_t(row) * K + c * 16;
       tdst[i] = m * 128 + ((c ^ (m & 7)) << 4);
     }
-    const bool stage_chunk = CHUNKS >= 256 || tid < CHUNKS;
+    const bool stage_chunk = CHUNKS >= NT || tid < CHUNKS;
     const uint8_t* ssrc;
     {
       const int pos = start + min(min(tid, TM - 1), n - 1);

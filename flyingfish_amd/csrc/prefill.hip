@@ -397,7 +397,11 @@ int launch_w16_fmt(int format, const W16Params& p, int mf, unsigned blocks, hipS
 }
 
 template <int MODE, int PACKED>
-int launch_mx(const MxParams& p, int mf, unsigned blocks, hipStream_t stream) {
+int launch_mx(const MxParams& p, int mf, unsigned blocks, hipStream_t stream, bool wide = false) {
+  if (wide) {
+    hipLaunchKernelGGL((k_mx_grouped<4, MODE, PACKED, 2, 8>), dim3(blocks), dim3(512), 0, stream, p);
+    return ff_launch_status();
+  }
   switch (mf) {
     case 1: hipLaunchKernelGGL((k_mx_grouped<1, MODE, PACKED, 2>), dim3(blocks), dim3(256), 0, stream, p); break;
     case 2: hipLaunchKernelGGL((k_mx_grouped<2, MODE, PACKED, 2>), dim3(blocks), dim3(256), 0, stream, p); break;
@@ -592,8 +596,8 @@ int prefill_impl(const ffmoe_expert_table* table, const ffmoe_prefill* args, int
                 (int*)(s + l.perm), (GemmGroup*)(s + l.groups), (u32x2*)(s + l.units0), (u32x2*)(s + l.units1)};
   const int mf = pick_mf(double(A) / E, (mx || a16) ? 4 : 8);
   const int tm = 16 * mf;
-  // W8A8 and W*A16 cohorts in 64-row groups: eight waves per block share a token tile (FFMOE_PREFILL_WIDE=0: four, two blocks per CU)
-  bool wide = !mx && mf == 4;
+  // W8A8, W*A16 and MX cohorts in 64-row groups: eight waves per block share a token tile (FFMOE_PREFILL_WIDE=0: four, two blocks per CU)
+  bool wide = mf == 4;
   if (const char* f = getenv("FFMOE_PREFILL_WIDE")) wide = wide && atoi(f) != 0;
   const int tiles0 = wide ? (I + 255) / 256 : (I + 127) / 128, tiles1 = wide ? (H + 511) / 512 : (H + 255) / 256;
   // A shared expert of the routed experts' format and width rides in the routed launches as further row groups (W*A16
@@ -632,13 +636,13 @@ int prefill_impl(const ffmoe_expert_table* table, const ffmoe_prefill* args, int
     if (stages & 2) {
       p.a_codes = s + l.xq; p.a_scales = s + l.sx; p.units = b.units0; p.unit_total = b.totals + 0;
       p.weights = (const float*)args->weights; p.out = (uint16_t*)(s + l.act); p.K = H; p.N = I;
-      FF_TRY((launch_mx<0, 1>(p, mf, blocks, stream)));
+      FF_TRY((launch_mx<0, 1>(p, mf, wide ? blocks / 2 : blocks, stream, wide)));
     }
     if (stages & 4) FF_TRY(ffmoe_act_quant_e8m0(s + l.act, s + l.aq, s + l.sa, int(A), I, stream_));
     if (stages & 8) {
       p.a_codes = s + l.aq; p.a_scales = s + l.sa; p.units = b.units1; p.unit_total = b.totals + 1;
       p.weights = nullptr; p.out = (uint16_t*)args->contributions; p.done = args->done; p.K = I; p.N = H;
-      FF_TRY((launch_mx<1, 1>(p, mf, blocks, stream)));
+      FF_TRY((launch_mx<1, 1>(p, mf, wide ? blocks / 2 : blocks, stream, wide)));
     }
     if (shared) {
       const int smf = R > 32 ? 4 : R > 16 ? 2 : 1;
