@@ -498,18 +498,38 @@ def c1_main(args, torch, capi, ops, synth):
     ids = torch.empty((1, K), dtype=torch.int32, device=dev)
     wts = torch.empty((1, K), dtype=torch.bfloat16, device=dev)
 
-    def step(i):
+    def step_separate(i):
         x = xs[i % len(xs)]
         ops.RouteOps.route(x, router, K, capi.SCORE_SOFTMAX, logits=logits, ids=ids, weights=wts)
         dec.done.zero_()
         c, _ = dec.contribute(x, ids, wts)
         return ops.CombineOps.combine(c, None, ids, capi.COMBINE_ROUTED, done=dec.done, status=status, out=y)
 
+    fused = [True]  # down + routing weight + ordered combine in one launch (ffmoe_decode_finish) where the shape allows it
+
+    def step(i):
+        if not fused[0]:
+            return step_separate(i)
+        x = xs[i % len(xs)]
+        ops.RouteOps.route(x, router, K, capi.SCORE_SOFTMAX, logits=logits, ids=ids, weights=wts)
+        dec.contribute(x, ids, wts, stage=0)
+        if dec.finish(x, ids, wts, capi.COMBINE_ROUTED, y, status=status):
+            return y
+        fused[0] = False
+        return step_separate(i)
+
+    step(0)
+    torch.cuda.synchronize()
     parity = None
     if not args.no_parity_gate:
         np_, orc, hp = _checkers()
-        got_y = hp.bits(step(0)).copy()
+        y_fused = hp.bits(step(0)).copy()
         torch.cuda.synchronize()
+        got_y = hp.bits(step_separate(0)).copy()
+        torch.cuda.synchronize()
+        if not np.array_equal(y_fused, got_y):
+            print("bench.py parity gate FAILED: the fused down + combine launch differs from the separate launches", file=sys.stderr)
+            sys.exit(3)
         xb = hp.bits(xs[0])
         ol = orc.route_logits_bf16(xb, hp.bits(router))
         oi, ow = orc.route_topk_softmax(ol, K)
@@ -553,7 +573,8 @@ def c1_main(args, torch, capi, ops, synth):
            "dtype": "fp8_e4m3 weights, bf16 activations, f32 accumulate", "data": "synthetic",
            "config": {"workload": "MoE decode step at the reference's CPU-runnable shape (BASELINE config 1), batch 1", "hidden": H, "intermediate": I,
                       "experts": E, "shared_experts": 0, "top_k": K, "routing": "softmax top-4 over BF16 logits", "ring": len(xs),
-                      "launches_per_layer": "fused BF16-logit route; gate/up; down; combine (+ a done-flag fill)"},
+                      "launches_per_layer": "fused BF16-logit route; gate/up; down + combine" if fused[0] else
+                                            "fused BF16-logit route; gate/up; down; combine (+ a done-flag fill)"},
            "tokens_per_s": 1e6 / us, "layer_bytes": nbytes, "layer_hbm_gbps": nbytes / us / 1e3, "layer_hbm_frac": nbytes / us / 1e3 / HBM_PEAK_GBPS,
            "roofline": {"kernel": "ffmoe::k_decode_stage<FmtFp8, S, 0, 1, NR> (gate/up + SwiGLU)", "bound": "hbm", "achieved": b0 / k0 / 1e3,
                         "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": b0 / k0 / 1e3 / HBM_PEAK_GBPS, "traffic": None, "bytes_per_launch": b0,
