@@ -49,6 +49,37 @@ def test_prefill_w8a8_full_width_every_group_size(monkeypatch):
         op.contributions.zero_()
         again = bits(op.contribute(x_d, ids_d, w_d))
         assert np.array_equal(again, ref), "FFMOE_PREFILL_MF=%s changes the result at 56 / 16 K blocks" % mf
+    monkeypatch.delenv("FFMOE_PREFILL_MF")
+    monkeypatch.setenv("FFMOE_PREFILL_WIDE", "0")   # 64-row groups with four waves per block instead of eight
+    op.contributions.zero_()
+    assert np.array_equal(bits(op.contribute(x_d, ids_d, w_d)), ref), "FFMOE_PREFILL_WIDE=0 changes the result"
+
+
+def test_prefill_w8a8_cohort_beyond_64_k_blocks(monkeypatch):
+    """A contraction of 66 K blocks (hidden 8448) through the grouped kernels: the block scales are held 64 K blocks at a
+    time and re-armed inside the K loop. Stage-wise against the oracle on every 11th row, and every kernel variant bit for
+    bit against the default one."""
+    experts, rows, top_k, hidden, inter = 2, 150, 1, 8448, 256
+    for k in ("FFMOE_PREFILL_MF", "FFMOE_PREFILL_RGB", "FFMOE_PREFILL_WIDE"):
+        monkeypatch.delenv(k, raising=False)
+    table = make_table_on_device(capi.FMT_FP8_BLOCK128, experts, hidden, inter, 171)
+    host = [host_expert(table, e) for e in range(experts)]
+    ids, w = _routing(rows, top_k, experts, 172, 0.5)
+    x = synth.normal((rows, hidden), 1.0, 173, dtype=torch.bfloat16)
+    op = ops.PrefillOps(table, rows, top_k, swiglu=capi.SWIGLU_TWICE, weights_f32=True)
+    x_d, ids_d, w_d = x.cuda(), torch.from_numpy(ids).cuda(), torch.from_numpy(w).cuda()
+    print("W8A8 cohort at 66 K blocks, default grouping", flush=True)
+    got = op.contribute(x_d, ids_d, w_d)
+    torch.cuda.synchronize()
+    ref = bits(got).copy()
+    _check_prefill(op, host, bits(x), ids, w, orc.TWICE, 0.0, orc.AFTER_DOWN_BF16, np.ones_like(ids, dtype=bool), got, table,
+                   row_step=11, threads=THREADS)
+    for mf, wide in (("4", "0"), ("1", "1"), ("2", "1"), ("8", "1")):
+        monkeypatch.setenv("FFMOE_PREFILL_MF", mf)
+        monkeypatch.setenv("FFMOE_PREFILL_WIDE", wide)
+        print("W8A8 cohort at 66 K blocks, FFMOE_PREFILL_MF=%s FFMOE_PREFILL_WIDE=%s" % (mf, wide), flush=True)
+        op.contributions.zero_()
+        assert np.array_equal(bits(op.contribute(x_d, ids_d, w_d)), ref), (mf, wide)
 
 
 @pytest.mark.parametrize("m", [3, 40, 70, 130])
