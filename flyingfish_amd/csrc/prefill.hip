@@ -337,11 +337,16 @@ inline uint64_t up256(uint64_t v) { return (v + 255) & ~uint64_t(255); }
 
 // rows per group for an average of `avg` rows per expert
 // (cap: the largest group a path's kernels are built for, in units of 16 rows; anything else in the variable is ignored)
-int pick_mf(double avg, int cap) {
+int pick_mf(double avg, int cap, bool w8a8 = false) {
   if (const char* f = getenv("FFMOE_PREFILL_MF")) {
     const int v = atoi(f);
     if (v == 1 || v == 2 || v == 4 || v == 8) return std::min(v, cap);
   }
+  // W8A8: the 64-row kernel with eight waves per block is ahead at every cohort size measured (top-8 of 256 experts at
+  // hidden 7168, 32 / 128 / 512 / 2048 tokens: 0.74 / 1.42 / 2.04 / 2.65 ms against 0.77 / 1.54 / 2.30 / 4.17 ms with 32-row
+  // groups and 0.77 / 1.55 / 2.71 / 6.79 ms with 16-row groups). The W*A16 and MX kernels dequantize per row group
+  // and keep the short groups for short segments (64 rows, 16-row groups: 1.89 ms, 64-row groups: 2.17 ms).
+  if (w8a8) return 4;
   return avg > 24.0 ? 4 : avg > 12.0 ? 2 : 1;
 }
 
@@ -594,7 +599,7 @@ int prefill_impl(const ffmoe_expert_table* table, const ffmoe_prefill* args, int
   uint8_t* s = (uint8_t*)args->scratch;
   PrefillBook b{(uint32_t*)(s + l.counts), (uint32_t*)(s + l.offsets), (uint32_t*)(s + l.gbase), (uint32_t*)(s + l.totals),
                 (int*)(s + l.perm), (GemmGroup*)(s + l.groups), (u32x2*)(s + l.units0), (u32x2*)(s + l.units1)};
-  const int mf = pick_mf(double(A) / E, (mx || a16) ? 4 : 8);
+  const int mf = pick_mf(double(A) / E, (mx || a16) ? 4 : 8, !mx && !a16);
   const int tm = 16 * mf;
   // W8A8, W*A16 and MX cohorts in 64-row groups: eight waves per block share a token tile (FFMOE_PREFILL_WIDE=0: four, two blocks per CU)
   bool wide = mf == 4;
