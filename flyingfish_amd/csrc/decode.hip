@@ -140,7 +140,15 @@ extern "C" __attribute__((visibility("default"))) uint64_t ffmoe_decode_scratch_
   // a shared expert served by the matrix-core path (large batches) keeps its activations behind the decode arena
   const uint64_t shared_act = shared_inter > 0 ? ((uint64_t(rows) * shared_inter * 2 + 255) & ~uint64_t(255)) : 0;
   const uint64_t own = h + groups + 256 + shared_act;
-  return own > w8a8 ? own : w8a8;
+  uint64_t need = own > w8a8 ? own : w8a8;
+  // a cohort of routed experts on the matrix cores with a shared expert of another format on the streaming kernels: the
+  // shared pass gets an arena of its own behind the cohort's, so the two may also be issued stage by stage
+  if (shared_inter > 0) {
+    const uint64_t routed = ffmoe_prefill_scratch_bytes(rows, top_k, experts, hidden, inter, 0);
+    const uint64_t mixed = routed + (top_k == 1 ? need : ffmoe_decode_scratch_bytes(rows, 1, experts, hidden, inter, shared_inter));
+    if (top_k > 1 && mixed > need) need = mixed;
+  }
+  return need;
 }
 
 // layout_k >= 0: the call processes args->top_k choices per row (0 = the shared expert only) but lays the scratch
@@ -333,11 +341,18 @@ static int decode_dispatch(const ffmoe_expert_table* table, const ffmoe_shared_e
   // block-FP8 shared expert alone from FFMOE_DECODE_SHARED_COHORT_ROWS on (it has every row: streamed once instead of once
   // per row group that fits LDS; a BF16 shared expert next to NVFP4 experts measured slower there, 1.88 against 1.80 ms at
   // 32 rows, and stays on the streaming kernels).
+  // NVFP4 experts whose rows are whole 128-byte lines of codes (hidden and inter multiples of 256) take the line-wise
+  // cohort kernel from FFMOE_DECODE_COHORT_ROWS on as well; next to them a shared expert of another format stays on the
+  // streaming kernels up to FFMOE_DECODE_SHARED_STREAM_ROWS rows (a launch of its own on the matrix cores is a few dozen
+  // blocks) and gets an arena of its own behind the cohort's.
   // (0 switches a rule off; read at every call)
   const char* ce = getenv("FFMOE_DECODE_COHORT_ROWS");
   const char* se = getenv("FFMOE_DECODE_SHARED_COHORT_ROWS");
+  const char* te = getenv("FFMOE_DECODE_SHARED_STREAM_ROWS");
   const bool rides = !shared || (table && shared->format == table->format && shared->inter == table->inter);
-  const int cohort_rows = ce ? atoi(ce) : (rides ? 8 : 32), shared_rows = se ? atoi(se) : 16;
+  const bool nv_lines = table && table->format == FFMOE_FMT_NVFP4 && table->hidden % 256 == 0 && table->inter % 256 == 0;
+  const int cohort_rows = ce ? atoi(ce) : (rides || nv_lines ? 8 : 32), shared_rows = se ? atoi(se) : 16;
+  const int stream_rows = te ? atoi(te) : 32;
   if (table && args && args->act_mode == FFMOE_ACT_BF16 && args->rows > 1) {
     const int fmt = table->format, H = table->hidden, I = table->inter, R = args->rows;
     auto on_matrix_cores = [&](int f, int inter) {
@@ -346,14 +361,30 @@ static int decode_dispatch(const ffmoe_expert_table* table, const ffmoe_shared_e
              H >= gran && inter >= gran;
     };
     const bool shared_ok = !shared || on_matrix_cores(shared->format, shared->inter);
-    if (cohort_rows > 0 && R >= cohort_rows && fmt == FFMOE_FMT_FP8_BLOCK128 && args->top_k >= 1 && on_matrix_cores(fmt, I) && shared_ok) {
+    const bool shared_streams = nv_lines && shared && !rides && R <= stream_rows && args->top_k > 1;
+    if (cohort_rows > 0 && R >= cohort_rows && (fmt == FFMOE_FMT_FP8_BLOCK128 || nv_lines) && args->top_k >= 1 && on_matrix_cores(fmt, I) &&
+        (shared_ok || shared_streams)) {
       ffmoe_prefill pf{};
       pf.rows = args->rows; pf.top_k = args->top_k; pf.act_mode = FFMOE_ACT_BF16;
       pf.swiglu = args->swiglu; pf.swiglu_limit = args->swiglu_limit; pf.routed_weight = args->routed_weight; pf.weights_f32 = args->weights_f32;
       pf.x = args->x; pf.ids = args->ids; pf.active = args->active; pf.weights = args->weights;
       pf.contributions = args->contributions; pf.done = args->done; pf.scratch = args->scratch; pf.scratch_bytes = args->scratch_bytes;
-      pf.shared = shared; pf.shared_out = args->shared_out; pf.assignment_gen = args->assignment_gen;
-      return prefill_impl(table, &pf, (stage_mask & 1 ? 3 : 0) | (stage_mask & 2 ? 12 : 0), stream);
+      pf.shared = shared_streams ? nullptr : shared; pf.shared_out = args->shared_out; pf.assignment_gen = args->assignment_gen;
+      if (!shared_streams) return prefill_impl(table, &pf, (stage_mask & 1 ? 3 : 0) | (stage_mask & 2 ? 12 : 0), stream);
+      const uint64_t routed = ffmoe_prefill_scratch_bytes(R, args->top_k, table->experts, H, I, 0);
+      FF_REQUIRE(args->scratch_bytes >= ffmoe_decode_scratch_bytes(R, args->top_k, table->experts, H, I, shared->inter), FFMOE_ERR_SCRATCH,
+                 "decode scratch holds %llu bytes, %llu needed", (unsigned long long)args->scratch_bytes,
+                 (unsigned long long)ffmoe_decode_scratch_bytes(R, args->top_k, table->experts, H, I, shared->inter));
+      pf.scratch_bytes = routed;
+      FF_TRY(prefill_impl(table, &pf, (stage_mask & 1 ? 3 : 0) | (stage_mask & 2 ? 12 : 0), stream));
+      ffmoe_expert_table as_shared = *table;
+      as_shared.format = shared->format;
+      ffmoe_decode only_shared = *args;
+      only_shared.top_k = 0;
+      only_shared.done = nullptr;
+      only_shared.scratch = (uint8_t*)args->scratch + routed;
+      only_shared.scratch_bytes = args->scratch_bytes - routed;
+      return decode_impl(&as_shared, shared, &only_shared, stage_mask, stream, 0, 0);
     }
     if (shared && shared_rows > 0 && R >= shared_rows && args->top_k >= 1 && shared_ok && shared->format == FFMOE_FMT_FP8_BLOCK128) {
       // routed choices on the streaming kernels, the shared expert on the matrix cores with its activations behind the arena

@@ -380,6 +380,17 @@ int launch_gemm(const GemmParams& p, int mf, unsigned blocks, hipStream_t stream
 
 template <class F, int MODE>
 int launch_w16(const W16Params& p, int mf, unsigned blocks, hipStream_t stream, bool wide = false) {
+  if constexpr (std::is_same<F, FmtNvfp4>::value) {
+    // rows of whole 128-byte code lines: the line-wise kernel (FFMOE_PREFILL_NVFP4_LINES=0 keeps the per-K-block one)
+    const char* le = getenv("FFMOE_PREFILL_NVFP4_LINES");
+    if (p.K % 256 == 0 && !(le && atoi(le) == 0)) {
+      if (wide) hipLaunchKernelGGL((k_w16_nvfp4_lines<4, MODE, 1, 8>), dim3(blocks), dim3(512), 0, stream, p);
+      else if (mf == 1) hipLaunchKernelGGL((k_w16_nvfp4_lines<1, MODE, 2>), dim3(blocks), dim3(256), 0, stream, p);
+      else if (mf == 2) hipLaunchKernelGGL((k_w16_nvfp4_lines<2, MODE, 2>), dim3(blocks), dim3(256), 0, stream, p);
+      else hipLaunchKernelGGL((k_w16_nvfp4_lines<4, MODE, 1>), dim3(blocks), dim3(256), 0, stream, p);
+      return ff_launch_status();
+    }
+  }
   if (wide) {  // 64-row groups, eight waves per block, one block per CU
     hipLaunchKernelGGL((k_w16_grouped<F, 4, MODE, 2, 8>), dim3(blocks), dim3(512), 0, stream, p);
     return ff_launch_status();
@@ -576,7 +587,7 @@ int prefill_impl(const ffmoe_expert_table* table, const ffmoe_prefill* args, int
     for (int i = 0; i < 6; ++i) {
       const bool scale_entry = i % 2 == 1;
       if (scale_entry && shared->format == FFMOE_FMT_BF16) continue;  // BF16 weights carry no scales
-      FF_REQUIRE(shared->slot[i] != 0 && shared->slot[i] % (scale_entry ? (shared->format == FFMOE_FMT_FP8_BLOCK128 ? 4 : (mx ? 1 : 2)) : 16) == 0, FFMOE_ERR_ALIGN,
+      FF_REQUIRE(shared->slot[i] != 0 && shared->slot[i] % (scale_entry ? (shared->format == FFMOE_FMT_FP8_BLOCK128 || shared->format == FFMOE_FMT_NVFP4 ? 4 : (mx ? 1 : 2)) : 16) == 0, FFMOE_ERR_ALIGN,
                  "shared expert slot[%d] is NULL or misaligned", i);
     }
   }

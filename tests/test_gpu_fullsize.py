@@ -313,7 +313,8 @@ def test_decode_fp8_full_width_beyond_the_lds_row_budget(rows, monkeypatch):
 
 
 def test_decode_nvfp4_full_width_batched():
-    """C4 dimensions, 9 rows: NVFP4 routed experts with a BF16 shared expert (two passes over one arena) at hidden 7168."""
+    """C4 dimensions, 9 rows: NVFP4 routed experts with a BF16 shared expert (a cohort pass and a streaming pass, an arena
+    each) at hidden 7168."""
     experts, top_k, rows = 4, 3, 9
     table = make_table_on_device(capi.FMT_NVFP4, experts, H, I, 121)
     sh_table = make_table_on_device(capi.FMT_BF16, 1, H, I, 122)
@@ -341,9 +342,12 @@ def test_decode_nvfp4_full_width_batched():
                 out.append(orc.expert_ffn(xb[r], *sref, 1.0, orc.TWICE, 0.0, 0, orc.LANE8, orc.SILU_DIV, apply_weight=False))
         return out
     res = [t for chunk in run_parallel(one, len(jobs), THREADS) for t in chunk]
+    # 9 rows: the routed choices run on the line-wise cohort kernel (both stages on the matrix cores compose as in
+    # test_prefill_w16_full_width: the relative-L2 bar on the row, element-wise a loose bound for cancelled outputs), the
+    # shared expert on the streaming kernels
     for (r, c), want in zip(jobs, res):
         if c >= 0:
-            assert_close_bf16(got[r, c][None, :], want[None, :], "contribution (%d, %d)" % (r, c))
+            assert_close_bf16(got[r, c][None, :], want[None, :], "contribution (%d, %d)" % (r, c), max_ulp=16)
         else:
             assert_close_bf16(got_s[r][None, :], want[None, :], "shared_out row %d" % r)
 

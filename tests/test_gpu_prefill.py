@@ -422,6 +422,89 @@ def test_prefill_shared_expert_rides_in_the_routed_launches_bitwise(fmt, rows, m
         assert np.array_equal(a, b), what
 
 
+@pytest.mark.parametrize("rows,mf,hidden,inter", [(70, "1", 512, 256), (70, "4", 256, 768), (9, "2", 1024, 256), (150, "2", 256, 512), (200, "wide", 768, 512)])
+def test_prefill_nvfp4_line_kernel_equals_the_k_block_kernel_bitwise(rows, mf, hidden, inter, monkeypatch):
+    """NVFP4 experts whose rows are whole 128-byte code lines (K a multiple of 256) go through a kernel that moves whole
+    lines four K blocks at a time, two sets ahead. Same operands into the same matrix instructions in the same order:
+    contributions, activations and the riding shared expert's outputs are the bits of the per-K-block kernel
+    (FFMOE_PREFILL_NVFP4_LINES=0), for every group size, one set per contraction (K = 256), an odd number of sets
+    (K = 768) and rows that do not fill the last group."""
+    from helpers import make_table
+    top_k, experts = 3, 5
+    table, _ = make_table(capi.FMT_NVFP4, experts + 1, hidden, inter, 700 + rows)
+    sh = table.shared_struct(experts)
+    table.experts = experts
+    ids, w = _routing(rows, top_k, experts, 710 + rows, 1.2)
+    x = synth.normal((rows, hidden), 1.0, 720 + rows, dtype=torch.bfloat16).cuda()
+    ids_d, w_d = torch.from_numpy(ids).cuda(), torch.from_numpy(w).cuda()
+    if mf == "wide":
+        monkeypatch.setenv("FFMOE_PREFILL_MF", "4")
+    else:
+        monkeypatch.setenv("FFMOE_PREFILL_MF", mf)
+        monkeypatch.setenv("FFMOE_PREFILL_WIDE", "0")
+    out = {}
+    for lines in ("0", "1"):
+        monkeypatch.setenv("FFMOE_PREFILL_NVFP4_LINES", lines)
+        op = ops.PrefillOps(table, rows, top_k, swiglu=capi.SWIGLU_TWICE, routed_weight=capi.WEIGHT_AFTER_DOWN_BF16, weights_f32=True,
+                            shared=sh, act_mode=capi.ACT_BF16)
+        op.contributions.zero_(); op.shared_out.zero_(); op.scratch.zero_()
+        print("rows=%d mf=%s hidden=%d inter=%d lines=%s" % (rows, mf, hidden, inter, lines), flush=True)
+        got = op.contribute(x, ids_d, w_d)
+        torch.cuda.synchronize()
+        v = op.scratch_views()
+        out[lines] = (bits(got).copy(), bits(op.shared_out).copy(), bits(v["act"]).copy(), op.done.cpu().numpy().copy())
+    assert np.any(out["0"][0] != 0) and np.any(out["0"][1] != 0) and int(out["0"][3].sum()) == rows * top_k
+    for a, b, what in zip(out["0"], out["1"], ("contributions", "shared_out", "activations", "done")):
+        assert np.array_equal(a, b), what
+
+
+@pytest.mark.parametrize("rows", [8, 16, 32, 33])
+def test_decode_nvfp4_cohort_with_a_streaming_shared_expert_of_another_format(rows, monkeypatch):
+    """ffmoe_decode_contribute, NVFP4 experts with whole code lines and a BF16 shared expert, 8 rows and more: the routed
+    choices run on the line-wise cohort kernel (the bits of ffmoe_prefill_contribute in the W*A16 arithmetic), the shared
+    expert on the streaming kernels in an arena of its own behind the cohort's (the bits of the all-streaming dispatch) -
+    in one call and issued stage by stage. Beyond 32 rows the shared expert moves to the matrix cores as well."""
+    from helpers import make_table
+    top_k, experts, hidden, inter = 3, 6, 256, 512
+    table, _ = make_table(capi.FMT_NVFP4, experts, hidden, inter, 800 + rows)
+    sh_table, _ = make_table(capi.FMT_BF16, 1, hidden, inter, 801 + rows)
+    sh = sh_table.shared_struct(0)
+    ids, w = _routing(rows, top_k, experts, 810 + rows, 1.0)
+    x = synth.normal((rows, hidden), 1.0, 820 + rows, dtype=torch.bfloat16).cuda()
+    ids_d, w_d = torch.from_numpy(ids).cuda(), torch.from_numpy(w).cuda()
+    monkeypatch.delenv("FFMOE_DECODE_COHORT_ROWS", raising=False)
+    monkeypatch.delenv("FFMOE_DECODE_SHARED_STREAM_ROWS", raising=False)
+
+    def run(stagewise):
+        op = ops.DecodeOps(table, sh, rows, top_k, capi.ACT_BF16, capi.SWIGLU_TWICE, 0.0, capi.WEIGHT_AFTER_DOWN_BF16, weights_f32=True)
+        op.contributions.zero_(); op.shared_out.zero_(); op.scratch.zero_()
+        if stagewise:
+            op.contribute(x, ids_d, w_d, stage=0)
+            c, so = op.contribute(x, ids_d, w_d, stage=1)
+        else:
+            c, so = op.contribute(x, ids_d, w_d)
+        torch.cuda.synchronize()
+        return bits(c).copy(), bits(so).copy()
+    got_c, got_s = run(False)
+    st_c, st_s = run(True)
+    assert np.array_equal(got_c, st_c) and np.array_equal(got_s, st_s), "stage by stage = one call"
+    monkeypatch.setenv("FFMOE_DECODE_COHORT_ROWS", "0")
+    str_c, str_s = run(False)
+    if rows <= 32:
+        assert np.array_equal(got_s, str_s), "shared expert: the streaming kernels' bits"
+    else:
+        assert np.any(got_s != str_s)
+        assert_close_bf16(got_s, str_s, "shared expert on the matrix cores vs streaming", max_ulp=16)
+    assert np.any(got_c != str_c), "the routed choices did not move to the cohort kernels"
+    pre = ops.PrefillOps(table, rows, top_k, swiglu=capi.SWIGLU_TWICE, routed_weight=capi.WEIGHT_AFTER_DOWN_BF16, weights_f32=True,
+                         act_mode=capi.ACT_BF16)
+    want = pre.contribute(x, ids_d, w_d)
+    torch.cuda.synchronize()
+    assert np.array_equal(got_c, bits(want)), "routed choices: the cohort kernels' bits"
+    # and inside the end-to-end bar of the matrix-core path against the streaming kernels
+    assert_close_bf16(got_c.reshape(rows * top_k, hidden), str_c.reshape(rows * top_k, hidden), "cohort vs streaming contributions", max_ulp=16)
+
+
 @pytest.mark.parametrize("rows,top_k,experts", [(1, 1, 3), (37, 4, 9), (128, 8, 70), (341, 3, 5)])
 def test_prefill_single_launch_bookkeeping_equals_the_four_launches(rows, top_k, experts, monkeypatch):
     """Small cohorts (by default up to 256 assignments, here forced up to the kernel's 1024) are counted, planned and listed
