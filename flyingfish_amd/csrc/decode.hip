@@ -343,8 +343,9 @@ static int decode_dispatch(const ffmoe_expert_table* table, const ffmoe_shared_e
   // 32 rows, and stays on the streaming kernels).
   // NVFP4 experts whose rows are whole 128-byte lines of codes (hidden and inter multiples of 256) take the line-wise
   // cohort kernel from FFMOE_DECODE_COHORT_ROWS on as well; next to them a shared expert of another format stays on the
-  // streaming kernels up to FFMOE_DECODE_SHARED_STREAM_ROWS rows (a launch of its own on the matrix cores is a few dozen
-  // blocks) and gets an arena of its own behind the cohort's.
+  // streaming kernels up to FFMOE_DECODE_SHARED_STREAM_ROWS = 24 rows and runs on one-wave blocks on the matrix cores
+  // beyond (BF16 next to NVFP4 experts at hidden 7168, streaming against matrix cores: 16 rows 725 / 736 us per layer, 32 rows
+  // 1123 / 1109, 64 rows 1524 / 1489) and gets an arena of its own behind the cohort's.
   // (0 switches a rule off; read at every call)
   const char* ce = getenv("FFMOE_DECODE_COHORT_ROWS");
   const char* se = getenv("FFMOE_DECODE_SHARED_COHORT_ROWS");
@@ -352,7 +353,7 @@ static int decode_dispatch(const ffmoe_expert_table* table, const ffmoe_shared_e
   const bool rides = !shared || (table && shared->format == table->format && shared->inter == table->inter);
   const bool nv_lines = table && table->format == FFMOE_FMT_NVFP4 && table->hidden % 256 == 0 && table->inter % 256 == 0;
   const int cohort_rows = ce ? atoi(ce) : (rides || nv_lines ? 8 : 32), shared_rows = se ? atoi(se) : 16;
-  const int stream_rows = te ? atoi(te) : 32;
+  const int stream_rows = te ? atoi(te) : 24;
   if (table && args && args->act_mode == FFMOE_ACT_BF16 && args->rows > 1) {
     const int fmt = table->format, H = table->hidden, I = table->inter, R = args->rows;
     auto on_matrix_cores = [&](int f, int inter) {

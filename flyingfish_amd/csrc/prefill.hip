@@ -378,12 +378,17 @@ int launch_gemm(const GemmParams& p, int mf, unsigned blocks, hipStream_t stream
   return ff_launch_status();
 }
 
+// read at every call
+bool nvfp4_lines_enabled() {
+  const char* le = getenv("FFMOE_PREFILL_NVFP4_LINES");
+  return !(le && atoi(le) == 0);
+}
+
 template <class F, int MODE>
 int launch_w16(const W16Params& p, int mf, unsigned blocks, hipStream_t stream, bool wide = false) {
   if constexpr (std::is_same<F, FmtNvfp4>::value) {
     // rows of whole 128-byte code lines: the line-wise kernel (FFMOE_PREFILL_NVFP4_LINES=0 keeps the per-K-block one)
-    const char* le = getenv("FFMOE_PREFILL_NVFP4_LINES");
-    if (p.K % 256 == 0 && !(le && atoi(le) == 0)) {
+    if (p.K % 256 == 0 && nvfp4_lines_enabled()) {
       if (wide) hipLaunchKernelGGL((k_w16_nvfp4_lines<4, MODE, 1, 8>), dim3(blocks), dim3(512), 0, stream, p);
       else if (mf == 1) hipLaunchKernelGGL((k_w16_nvfp4_lines<1, MODE, 2>), dim3(blocks), dim3(256), 0, stream, p);
       else if (mf == 2) hipLaunchKernelGGL((k_w16_nvfp4_lines<2, MODE, 2>), dim3(blocks), dim3(256), 0, stream, p);
@@ -410,6 +415,22 @@ int launch_w16_fmt(int format, const W16Params& p, int mf, unsigned blocks, hipS
     case FFMOE_FMT_FP8_CHANNEL: return launch_w16<FmtFp8Channel, MODE>(p, mf, blocks, stream, wide);
     default: return launch_w16<FmtBf16, MODE>(p, mf, blocks, stream, wide);
   }
+}
+
+// One wave per block and a quarter of the tile's columns: for one dense group over few rows (the always-on expert), whose
+// four-wave tiles would be a few dozen blocks on 256 CUs. Block-FP8 and BF16 weights.
+template <int MODE>
+bool launch_w16_narrow(int format, const W16Params& p, int mf, unsigned blocks, hipStream_t stream) {
+#define FF_NARROW(F_)                                                                                              \
+  switch (mf) {                                                                                                    \
+    case 1: hipLaunchKernelGGL((k_w16_grouped<F_, 1, MODE, 2, 1>), dim3(blocks), dim3(64), 0, stream, p); break;   \
+    case 2: hipLaunchKernelGGL((k_w16_grouped<F_, 2, MODE, 2, 1>), dim3(blocks), dim3(64), 0, stream, p); break;   \
+    default: hipLaunchKernelGGL((k_w16_grouped<F_, 4, MODE, 2, 1>), dim3(blocks), dim3(64), 0, stream, p); break;  \
+  }
+  if (format == FFMOE_FMT_BF16) { FF_NARROW(FmtBf16) return true; }
+  if (format == FFMOE_FMT_FP8_BLOCK128) { FF_NARROW(FmtFp8) return true; }
+#undef FF_NARROW
+  return false;
 }
 
 template <int MODE, int PACKED>
@@ -500,13 +521,24 @@ int shared_expert_w16(const ffmoe_shared_expert* shared, const void* x, int R, i
   W16Params q{};
   q.rows_total = R; q.top_k = 1; q.shared_expert = -1;
   q.swiglu = swiglu; q.limit = limit;
+  // fewer four-wave tiles than CUs: one-wave blocks over a quarter of the columns each (FFMOE_PREFILL_SHARED_NARROW=0
+  // keeps the four-wave tiles; same bits)
+  const char* ne = getenv("FFMOE_PREFILL_SHARED_NARROW");
+  const bool may_narrow = (shared->format == FFMOE_FMT_BF16 || shared->format == FFMOE_FMT_FP8_BLOCK128) && !(ne && atoi(ne) == 0);
+  const unsigned nblocks = ((unsigned)num_cus_p() * 8u) & ~7u;
   if (stage_mask & 1) {
     q.a = (const uint16_t*)x;
     q.w0_codes = shared->slot[0]; q.w0_scales = shared->slot[1]; q.w1_codes = shared->slot[2]; q.w1_scales = shared->slot[3];
     q.g0 = shared->global_scales[0]; q.g1 = shared->global_scales[1];
     q.total_units = sgroups * uint32_t((SI + 127) / 128);
     q.out = (uint16_t*)act; q.K = H; q.N = SI;
-    FF_TRY(launch_w16_fmt<0>(shared->format, q, smf, std::min<unsigned>(blocks, (q.total_units + 7u) & ~7u), stream));
+    if (may_narrow && q.total_units < (unsigned)num_cus_p()) {
+      q.total_units = sgroups * uint32_t((SI + 31) / 32);
+      launch_w16_narrow<0>(shared->format, q, smf, std::min<unsigned>(nblocks, (q.total_units + 7u) & ~7u), stream);
+      FF_TRY(ff_launch_status());
+    } else {
+      FF_TRY(launch_w16_fmt<0>(shared->format, q, smf, std::min<unsigned>(blocks, (q.total_units + 7u) & ~7u), stream));
+    }
   }
   if (stage_mask & 2) {
     q.a = (const uint16_t*)act;
@@ -514,7 +546,13 @@ int shared_expert_w16(const ffmoe_shared_expert* shared, const void* x, int R, i
     q.g0 = shared->global_scales[2]; q.g1 = q.g0;
     q.total_units = sgroups * uint32_t((H + 255) / 256);
     q.out = (uint16_t*)shared_out; q.K = SI; q.N = H;
-    FF_TRY(launch_w16_fmt<2>(shared->format, q, smf, std::min<unsigned>(blocks, (q.total_units + 7u) & ~7u), stream));
+    if (may_narrow && q.total_units < (unsigned)num_cus_p()) {
+      q.total_units = sgroups * uint32_t((H + 63) / 64);
+      launch_w16_narrow<2>(shared->format, q, smf, std::min<unsigned>(nblocks, (q.total_units + 7u) & ~7u), stream);
+      FF_TRY(ff_launch_status());
+    } else {
+      FF_TRY(launch_w16_fmt<2>(shared->format, q, smf, std::min<unsigned>(blocks, (q.total_units + 7u) & ~7u), stream));
+    }
   }
   return 0;
 }

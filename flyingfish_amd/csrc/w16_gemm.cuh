@@ -279,9 +279,10 @@ __device__ __forceinline__ void w16_store(const v4f (&acc)[MF][4], const W16Para
   }
 }
 
-// NW waves per block share one token tile (see k_w8a8_grouped): eight for 64-row groups of a cohort, one block per CU.
-template <class F, int MF, int MODE, int P, int NW = 4>
-__global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void k_w16_grouped(const W16Params p) {
+// One unit of the grouped W*A16 GEMM, run by the NW waves of a block: a group of at most 16 MF token rows of one expert x
+// one tile of output columns, over the whole contraction. The LDS buffers are the function's own.
+template <class F, int MF, int MODE, int P, int NW>
+__device__ __forceinline__ void w16_unit_run(const W16Params& p, const W16Unit& un_) {
   constexpr int NT = 64 * NW;
   constexpr int TM = 16 * MF;
   constexpr int CHUNKS = TM * 8;             // 16-byte token chunks per K block (64 BF16 columns = 128 bytes per row)
@@ -303,8 +304,228 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void k_w16_grouped(const 
   // lane / 16); pieces are XOR-swizzled by (row / 4) % 4 so that the 16 rows of a read fall into distinct banks
   const int wr_off = (lane >> 2) * 64 + (((lane & 3) ^ ((lane >> 4) & 3)) << 4);
   const int rd_off = (lane & 15) * 64 + (((lane >> 4) ^ ((lane >> 2) & 3)) << 4);
+  const int expert = un_.expert, start = un_.start, n = un_.n, t = un_.t;
+  const bool ride = un_.ride;  // wave-uniform
+  const uint64_t wc[2] = {un_.wc[0], un_.wc[1]}, ws[2] = {un_.ws[0], un_.ws[1]};
+  const float gl[2] = {un_.gl[0], un_.gl[1]};
+  (void)expert;
+  // weight rows of this lane's four fragments; fragments past N are clamped onto the last 16 rows and dropped at the store
+  int col0[4];
+  typename W16<F>::Row wrow[4];
+#pragma unroll
+  for (int f = 0; f < 4; ++f) {
+    col0[f] = MODE == 0 ? t * (32 * NW) + wave * 32 + (f & 1) * 16 : t * (64 * NW) + wave * 64 + f * 16;
+    const int base = min(col0[f], N - 16);
+    const int which = MODE == 0 ? f >> 1 : 0;
+    wrow[f] = W16<F>::row(wc[which], ws[which], gl[which], base + (lane & 15), K);
+  }
+  const uint32_t wcol = TR ? 0u : uint32_t(lane >> 4) * 16u;  // this lane's 16 columns inside a K block
+  typename W16<F>::Row lrow[4];  // what the loads address: the operand's row, or the row-contiguous pattern
+#pragma unroll
+  for (int f = 0; f < 4; ++f) {
+    if constexpr (TR) {
+      const int which = MODE == 0 ? f >> 1 : 0;
+      lrow[f] = W16<F>::row(wc[which], ws[which], gl[which], min(col0[f], N - 16) + (lane >> 2), K);
+      lrow[f].codes += (lane & 3) * 16;
+    } else {
+      lrow[f] = wrow[f];
+    }
+  }
+
+  const uint8_t* ncod[2] = {nullptr, nullptr};
+  const uint8_t* nscl[2] = {nullptr, nullptr};
+  if constexpr (NVT) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {  // fragments 2j and 2j + 1 are 32 consecutive rows of one matrix
+      const int which = MODE == 0 ? j : 0;
+      const int row = min(col0[2 * j], N - 32) + (lane >> 1);
+      ncod[j] = reinterpret_cast<const uint8_t*>(wc[which]) + size_t(row) * (K >> 1) + (lane & 1) * 16;
+      nscl[j] = reinterpret_cast<const uint8_t*>(ws[which]) + size_t(row) * (K >> 4);
+    }
+  }
+  u32x4 nvc[NVT ? P : 1][2];
+  uint32_t nvs[NVT ? P : 1][2];  // the four scale bytes of a row's K block (K is a multiple of 64: a whole aligned word)
+
+  // token rows this thread stages
+  const uint8_t* tsrc[CPT];
+  int tdst[CPT];
+#pragma unroll
+  for (int i = 0; i < CPT; ++i) {
+    const int q = min(tid + NT * i, CHUNKS - 1);
+    const int m = q >> 3, c = q & 7;
+    const int pos = start + min(m, n - 1);
+    const int row = MODE == 0 && p.perm && !ride ? load_global<int>(p.perm + pos) / p.top_k : pos;
+    tsrc[i] = reinterpret_cast<const uint8_t*>(ride ? p.a_sh : p.a) + size_t(row) * K * 2 + c * 16;
+    tdst[i] = m * 128 + ((c ^ (m & 7)) << 4);
+  }
+  const bool stage_chunk = CHUNKS >= NT || tid < CHUNKS;
+
+  v4f acc[MF][4];
+#pragma unroll
+  for (int m = 0; m < MF; ++m)
+#pragma unroll
+    for (int f = 0; f < 4; ++f) acc[m][f] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+
+  // Loads inside the K loop are issued and awaited by hand (load16_async / wait_vm / pin, see k_w8a8_grouped): the
+  // compiler's own waits drain the queue at the top of every stage, which leaves one stage of lead whatever P is. A
+  // thread issues its loads in a fixed order - per stage the token chunks of tile kb+2, then the weights of K block kb+P
+  // into the slot just consumed - so the weights of a stage have the P-1 later stages' loads behind them and a token
+  // tile the weight loads of its own stage.
+  constexpr int WL = NVT ? 4 : 4 * W16<F>::LOADS;  // weight loads per stage
+  constexpr int LPS = CPT + WL;
+  typename W16<F>::Frag w[P][4];
+#define FF_W16_REQUEST(s_, kb_)                                                              \
+  do {                                                                                        \
+  if constexpr (NVT) {                                                                      \
+    _Pragma("unroll") for (int j_ = 0; j_ < 2; ++j_) {                                      \
+      load16_async(nvc[s_][j_], ncod[j_] + (kb_) * 32u);                                    \
+      load4_async(nvs[s_][j_], nscl[j_] + (kb_) * 4u);                                      \
+    }                                                                                       \
+  } else {                                                                                  \
+    _Pragma("unroll") for (int f_ = 0; f_ < 4; ++f_) W16<F>::load(w[s_][f_], lrow[f_], (kb_) * 64u + wcol); \
+  }                                                                                         \
+  } while (0)
+#define FF_W16_PIN(s_)                                                                        \
+  do {                                                                                        \
+  if constexpr (NVT) {                                                                      \
+    _Pragma("unroll") for (int j_ = 0; j_ < 2; ++j_) { pin(nvc[s_][j_]); pin(nvs[s_][j_]); } \
+  } else {                                                                                  \
+    _Pragma("unroll") for (int f_ = 0; f_ < 4; ++f_) W16<F>::pin(w[s_][f_]);                \
+  }                                                                                         \
+  } while (0)
+  // prologue: weights of the first P K blocks, token tile 0 into LDS, everything landed; then token tile 1 and the
+  // last weight stage once more, so that tile 1 too has a stage's weight loads behind it
+#pragma unroll
+  for (int s = 0; s < P; ++s) FF_W16_REQUEST(s, uint32_t(min(s, KB - 1)));
+  u32x4 tv[CPT];
+  {
+#pragma unroll
+    for (int i = 0; i < CPT; ++i) {
+      const u32x4 v = load16(tsrc[i]);
+      if (stage_chunk) *reinterpret_cast<u32x4*>(&tile[0][tdst[i]]) = v;
+    }
+    wait_vm<0>();
+#pragma unroll
+    for (int s = 0; s < P; ++s) FF_W16_PIN(s);
+    const uint32_t k1 = uint32_t(min(1, KB - 1));
+#pragma unroll
+    for (int i = 0; i < CPT; ++i) load16_async(tv[i], tsrc[i] + k1 * 128u);
+    FF_W16_REQUEST(P - 1, uint32_t(min(P - 1, KB - 1)));
+  }
+  __syncthreads();
+
+  // LDS addresses of this lane's token operands: row (16 m + lane % 16), columns 16 (lane / 16) .. + 15 = chunks 2q, 2q + 1
+  int tlo[MF], thi[MF];
+#pragma unroll
+  for (int m = 0; m < MF; ++m) {
+    const int trow = 16 * m + (lane & 15);
+    const int q2 = (lane >> 4) * 2;
+    tlo[m] = trow * 128 + (((q2) ^ (trow & 7)) << 4);
+    thi[m] = trow * 128 + (((q2 + 1) ^ (trow & 7)) << 4);
+  }
+
+  for (int kbo = 0; kbo < KB; kbo += P) {
+#pragma unroll
+    for (int s = 0; s < P; ++s) {
+      const int kb = kbo + s;
+      if (kb < KB) {
+        const uint8_t* tb = tile[kb & 1];
+        w16_bf16x8 a0[4], a1[4];
+        typename W16<F>::Frag wm[4];
+        wait_vm<(P - 1) * LPS>();
+        FF_W16_PIN(s);
+#pragma unroll
+        for (int f = 0; f < 4; ++f) wm[f] = w[s][f];
+        if constexpr (NVT) {
+          uint8_t* nl = &nstage[wave][0][0];
+          uint32_t* ns = &nscale[wave][0][0];
+#pragma unroll
+          for (int j = 0; j < 2; ++j) {
+            *reinterpret_cast<u32x4*>(nl + j * 1024 + (lane >> 1) * 32 + (lane & 1) * 16) = nvc[s][j];
+            if ((lane & 1) == 0) ns[j * 32 + (lane >> 1)] = nvs[s][j];
+          }
+          __builtin_amdgcn_wave_barrier();
+#pragma unroll
+          for (int f = 0; f < 4; ++f) {
+            const int r32 = (f & 1) * 16 + (lane & 15);
+            wm[f].codes = *reinterpret_cast<const u32x2*>(nl + (f >> 1) * 1024 + r32 * 32 + (lane >> 4) * 8);
+            wm[f].scale = (ns[(f >> 1) * 32 + r32] >> (8 * (lane >> 4))) & 0xffu;
+          }
+          __builtin_amdgcn_wave_barrier();
+        }
+        if constexpr (TR) {  // LDS operations of one wave execute in order: no wait between the writes and the reads
+          uint8_t* wl = &wstage[wave][0][0];
+#pragma unroll
+          for (int f = 0; f < 4; ++f) *reinterpret_cast<u32x4*>(wl + f * 1024 + wr_off) = w[s][f].codes;
+          __builtin_amdgcn_wave_barrier();
+#pragma unroll
+          for (int f = 0; f < 4; ++f) wm[f].codes = *reinterpret_cast<const u32x4*>(wl + f * 1024 + rd_off);
+          __builtin_amdgcn_wave_barrier();
+        }
+#pragma unroll
+        for (int f = 0; f < 4; ++f) {
+          uint32_t wd[8];
+          if constexpr (W16NeedsRow<F>::value) W16<F>::dequant(wm[f], wrow[f], wd);
+          else W16<F>::dequant(wm[f], wd);
+          const u32x4 x0 = {wd[0], wd[1], wd[2], wd[3]}, x1 = {wd[4], wd[5], wd[6], wd[7]};
+          a0[f] = __builtin_bit_cast(w16_bf16x8, x0);
+          a1[f] = __builtin_bit_cast(w16_bf16x8, x1);
+        }
+#pragma unroll
+        for (int m = 0; m < MF; ++m) {
+          const u32x4 lo = *reinterpret_cast<const u32x4*>(tb + tlo[m]);
+          const u32x4 hi = *reinterpret_cast<const u32x4*>(tb + thi[m]);
+          const w16_bf16x8 b0 = __builtin_bit_cast(w16_bf16x8, lo), b1 = __builtin_bit_cast(w16_bf16x8, hi);
+#pragma unroll
+          for (int f = 0; f < 4; ++f) {
+            acc[m][f] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0[f], b0, acc[m][f], 0, 0, 0);
+            acc[m][f] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1[f], b1, acc[m][f], 0, 0, 0);
+          }
+        }
+        // publish token tile kb+1 (requested one stage ago, the weight loads of that stage behind it)
+        wait_vm<WL>();
+#pragma unroll
+        for (int i = 0; i < CPT; ++i) {
+          pin(tv[i]);
+          if (stage_chunk) *reinterpret_cast<u32x4*>(&tile[(kb & 1) ^ 1][tdst[i]]) = tv[i];
+        }
+        __syncthreads();
+      } else {
+        // a stage past the last K block: its registers still have (clamped) loads in flight and are about to be
+        // requested into again; a register with a load in flight is never left unread
+        wait_vm<0>();
+        FF_W16_PIN(s);
+#pragma unroll
+        for (int i = 0; i < CPT; ++i) pin(tv[i]);
+      }
+      // request token tile kb+2, then K block kb+P of the weights into the slot just consumed; also past the last K
+      // block (clamped addresses), so that the number of loads per stage does not depend on the path
+      {
+        const uint32_t kn = uint32_t(min(kb + 2, KB - 1));
+#pragma unroll
+        for (int i = 0; i < CPT; ++i) load16_async(tv[i], tsrc[i] + kn * 128u);
+        FF_W16_REQUEST(s, uint32_t(min(kb + P, KB - 1)));
+      }
+    }
+  }
+  // the last stages have requested (clamped) data nobody reads: let it land before the registers are reused
+  wait_vm<0>();
+#pragma unroll
+  for (int s = 0; s < P; ++s) FF_W16_PIN(s);
+#pragma unroll
+  for (int i = 0; i < CPT; ++i) pin(tv[i]);
+#undef FF_W16_REQUEST
+#undef FF_W16_PIN
+
+  w16_store<MF, MODE>(acc, p, ride, start, n, t, col0, wave, lane);
+}
+
+// NW waves per block share one token tile (see k_w8a8_grouped): eight for 64-row groups of a cohort, one block per CU.
+template <class F, int MF, int MODE, int P, int NW = 4>
+__global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void k_w16_grouped(const W16Params p) {
+  constexpr int TM = 16 * MF;
   const uint32_t total = p.unit_total ? uint32_t(uni(int(load_global<uint32_t>(p.unit_total)))) : p.total_units;
-  const int ntiles = (N + gemm_tile_cols<MODE, NW>() - 1) / gemm_tile_cols<MODE, NW>();
+  const int ntiles = (p.N + gemm_tile_cols<MODE, NW>() - 1) / gemm_tile_cols<MODE, NW>();
 
   // one contiguous span of the unit list per XCD (see k_w8a8_grouped)
   const uint32_t xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3, per_xcd = gridDim.x >> 3;
@@ -312,220 +533,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void k_w16_grouped(const 
   const uint32_t span_end = min(total, (xcd + 1u) * span);
   for (uint32_t u = xcd * span + slot; u < span_end; u += per_xcd) {
     const W16Unit un_ = w16_unit<MODE>(p, u, ntiles, TM);
-    const int expert = un_.expert, start = un_.start, n = un_.n, t = un_.t;
-    const bool ride = un_.ride;  // wave-uniform
-    const uint64_t wc[2] = {un_.wc[0], un_.wc[1]}, ws[2] = {un_.ws[0], un_.ws[1]};
-    const float gl[2] = {un_.gl[0], un_.gl[1]};
-    (void)expert;
-    // weight rows of this lane's four fragments; fragments past N are clamped onto the last 16 rows and dropped at the store
-    int col0[4];
-    typename W16<F>::Row wrow[4];
-#pragma unroll
-    for (int f = 0; f < 4; ++f) {
-      col0[f] = MODE == 0 ? t * (32 * NW) + wave * 32 + (f & 1) * 16 : t * (64 * NW) + wave * 64 + f * 16;
-      const int base = min(col0[f], N - 16);
-      const int which = MODE == 0 ? f >> 1 : 0;
-      wrow[f] = W16<F>::row(wc[which], ws[which], gl[which], base + (lane & 15), K);
-    }
-    const uint32_t wcol = TR ? 0u : uint32_t(lane >> 4) * 16u;  // this lane's 16 columns inside a K block
-    typename W16<F>::Row lrow[4];  // what the loads address: the operand's row, or the row-contiguous pattern
-#pragma unroll
-    for (int f = 0; f < 4; ++f) {
-      if constexpr (TR) {
-        const int which = MODE == 0 ? f >> 1 : 0;
-        lrow[f] = W16<F>::row(wc[which], ws[which], gl[which], min(col0[f], N - 16) + (lane >> 2), K);
-        lrow[f].codes += (lane & 3) * 16;
-      } else {
-        lrow[f] = wrow[f];
-      }
-    }
-
-    const uint8_t* ncod[2] = {nullptr, nullptr};
-    const uint8_t* nscl[2] = {nullptr, nullptr};
-    if constexpr (NVT) {
-#pragma unroll
-      for (int j = 0; j < 2; ++j) {  // fragments 2j and 2j + 1 are 32 consecutive rows of one matrix
-        const int which = MODE == 0 ? j : 0;
-        const int row = min(col0[2 * j], N - 32) + (lane >> 1);
-        ncod[j] = reinterpret_cast<const uint8_t*>(wc[which]) + size_t(row) * (K >> 1) + (lane & 1) * 16;
-        nscl[j] = reinterpret_cast<const uint8_t*>(ws[which]) + size_t(row) * (K >> 4);
-      }
-    }
-    u32x4 nvc[NVT ? P : 1][2];
-    uint32_t nvs[NVT ? P : 1][2];  // the four scale bytes of a row's K block (K is a multiple of 64: a whole aligned word)
-
-    // token rows this thread stages
-    const uint8_t* tsrc[CPT];
-    int tdst[CPT];
-#pragma unroll
-    for (int i = 0; i < CPT; ++i) {
-      const int q = min(tid + NT * i, CHUNKS - 1);
-      const int m = q >> 3, c = q & 7;
-      const int pos = start + min(m, n - 1);
-      const int row = MODE == 0 && p.perm && !ride ? load_global<int>(p.perm + pos) / p.top_k : pos;
-      tsrc[i] = reinterpret_cast<const uint8_t*>(ride ? p.a_sh : p.a) + size_t(row) * K * 2 + c * 16;
-      tdst[i] = m * 128 + ((c ^ (m & 7)) << 4);
-    }
-    const bool stage_chunk = CHUNKS >= NT || tid < CHUNKS;
-
-    v4f acc[MF][4];
-#pragma unroll
-    for (int m = 0; m < MF; ++m)
-#pragma unroll
-      for (int f = 0; f < 4; ++f) acc[m][f] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
-
-    // Loads inside the K loop are issued and awaited by hand (load16_async / wait_vm / pin, see k_w8a8_grouped): the
-    // compiler's own waits drain the queue at the top of every stage, which leaves one stage of lead whatever P is. A
-    // thread issues its loads in a fixed order - per stage the token chunks of tile kb+2, then the weights of K block kb+P
-    // into the slot just consumed - so the weights of a stage have the P-1 later stages' loads behind them and a token
-    // tile the weight loads of its own stage.
-    constexpr int WL = NVT ? 4 : 4 * W16<F>::LOADS;  // weight loads per stage
-    constexpr int LPS = CPT + WL;
-    typename W16<F>::Frag w[P][4];
-#define FF_W16_REQUEST(s_, kb_)                                                              \
-  do {                                                                                        \
-    if constexpr (NVT) {                                                                      \
-      _Pragma("unroll") for (int j_ = 0; j_ < 2; ++j_) {                                      \
-        load16_async(nvc[s_][j_], ncod[j_] + (kb_) * 32u);                                    \
-        load4_async(nvs[s_][j_], nscl[j_] + (kb_) * 4u);                                      \
-      }                                                                                       \
-    } else {                                                                                  \
-      _Pragma("unroll") for (int f_ = 0; f_ < 4; ++f_) W16<F>::load(w[s_][f_], lrow[f_], (kb_) * 64u + wcol); \
-    }                                                                                         \
-  } while (0)
-#define FF_W16_PIN(s_)                                                                        \
-  do {                                                                                        \
-    if constexpr (NVT) {                                                                      \
-      _Pragma("unroll") for (int j_ = 0; j_ < 2; ++j_) { pin(nvc[s_][j_]); pin(nvs[s_][j_]); } \
-    } else {                                                                                  \
-      _Pragma("unroll") for (int f_ = 0; f_ < 4; ++f_) W16<F>::pin(w[s_][f_]);                \
-    }                                                                                         \
-  } while (0)
-    // prologue: weights of the first P K blocks, token tile 0 into LDS, everything landed; then token tile 1 and the
-    // last weight stage once more, so that tile 1 too has a stage's weight loads behind it
-#pragma unroll
-    for (int s = 0; s < P; ++s) FF_W16_REQUEST(s, uint32_t(min(s, KB - 1)));
-    u32x4 tv[CPT];
-    {
-#pragma unroll
-      for (int i = 0; i < CPT; ++i) {
-        const u32x4 v = load16(tsrc[i]);
-        if (stage_chunk) *reinterpret_cast<u32x4*>(&tile[0][tdst[i]]) = v;
-      }
-      wait_vm<0>();
-#pragma unroll
-      for (int s = 0; s < P; ++s) FF_W16_PIN(s);
-      const uint32_t k1 = uint32_t(min(1, KB - 1));
-#pragma unroll
-      for (int i = 0; i < CPT; ++i) load16_async(tv[i], tsrc[i] + k1 * 128u);
-      FF_W16_REQUEST(P - 1, uint32_t(min(P - 1, KB - 1)));
-    }
-    __syncthreads();
-
-    // LDS addresses of this lane's token operands: row (16 m + lane % 16), columns 16 (lane / 16) .. + 15 = chunks 2q, 2q + 1
-    int tlo[MF], thi[MF];
-#pragma unroll
-    for (int m = 0; m < MF; ++m) {
-      const int trow = 16 * m + (lane & 15);
-      const int q2 = (lane >> 4) * 2;
-      tlo[m] = trow * 128 + (((q2) ^ (trow & 7)) << 4);
-      thi[m] = trow * 128 + (((q2 + 1) ^ (trow & 7)) << 4);
-    }
-
-    for (int kbo = 0; kbo < KB; kbo += P) {
-#pragma unroll
-      for (int s = 0; s < P; ++s) {
-        const int kb = kbo + s;
-        if (kb < KB) {
-          const uint8_t* tb = tile[kb & 1];
-          w16_bf16x8 a0[4], a1[4];
-          typename W16<F>::Frag wm[4];
-          wait_vm<(P - 1) * LPS>();
-          FF_W16_PIN(s);
-#pragma unroll
-          for (int f = 0; f < 4; ++f) wm[f] = w[s][f];
-          if constexpr (NVT) {
-            uint8_t* nl = &nstage[wave][0][0];
-            uint32_t* ns = &nscale[wave][0][0];
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
-              *reinterpret_cast<u32x4*>(nl + j * 1024 + (lane >> 1) * 32 + (lane & 1) * 16) = nvc[s][j];
-              if ((lane & 1) == 0) ns[j * 32 + (lane >> 1)] = nvs[s][j];
-            }
-            __builtin_amdgcn_wave_barrier();
-#pragma unroll
-            for (int f = 0; f < 4; ++f) {
-              const int r32 = (f & 1) * 16 + (lane & 15);
-              wm[f].codes = *reinterpret_cast<const u32x2*>(nl + (f >> 1) * 1024 + r32 * 32 + (lane >> 4) * 8);
-              wm[f].scale = (ns[(f >> 1) * 32 + r32] >> (8 * (lane >> 4))) & 0xffu;
-            }
-            __builtin_amdgcn_wave_barrier();
-          }
-          if constexpr (TR) {  // LDS operations of one wave execute in order: no wait between the writes and the reads
-            uint8_t* wl = &wstage[wave][0][0];
-#pragma unroll
-            for (int f = 0; f < 4; ++f) *reinterpret_cast<u32x4*>(wl + f * 1024 + wr_off) = w[s][f].codes;
-            __builtin_amdgcn_wave_barrier();
-#pragma unroll
-            for (int f = 0; f < 4; ++f) wm[f].codes = *reinterpret_cast<const u32x4*>(wl + f * 1024 + rd_off);
-            __builtin_amdgcn_wave_barrier();
-          }
-#pragma unroll
-          for (int f = 0; f < 4; ++f) {
-            uint32_t wd[8];
-            if constexpr (W16NeedsRow<F>::value) W16<F>::dequant(wm[f], wrow[f], wd);
-            else W16<F>::dequant(wm[f], wd);
-            const u32x4 x0 = {wd[0], wd[1], wd[2], wd[3]}, x1 = {wd[4], wd[5], wd[6], wd[7]};
-            a0[f] = __builtin_bit_cast(w16_bf16x8, x0);
-            a1[f] = __builtin_bit_cast(w16_bf16x8, x1);
-          }
-#pragma unroll
-          for (int m = 0; m < MF; ++m) {
-            const u32x4 lo = *reinterpret_cast<const u32x4*>(tb + tlo[m]);
-            const u32x4 hi = *reinterpret_cast<const u32x4*>(tb + thi[m]);
-            const w16_bf16x8 b0 = __builtin_bit_cast(w16_bf16x8, lo), b1 = __builtin_bit_cast(w16_bf16x8, hi);
-#pragma unroll
-            for (int f = 0; f < 4; ++f) {
-              acc[m][f] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0[f], b0, acc[m][f], 0, 0, 0);
-              acc[m][f] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1[f], b1, acc[m][f], 0, 0, 0);
-            }
-          }
-          // publish token tile kb+1 (requested one stage ago, the weight loads of that stage behind it)
-          wait_vm<WL>();
-#pragma unroll
-          for (int i = 0; i < CPT; ++i) {
-            pin(tv[i]);
-            if (stage_chunk) *reinterpret_cast<u32x4*>(&tile[(kb & 1) ^ 1][tdst[i]]) = tv[i];
-          }
-          __syncthreads();
-        } else {
-          // a stage past the last K block: its registers still have (clamped) loads in flight and are about to be
-          // requested into again; a register with a load in flight is never left unread
-          wait_vm<0>();
-          FF_W16_PIN(s);
-#pragma unroll
-          for (int i = 0; i < CPT; ++i) pin(tv[i]);
-        }
-        // request token tile kb+2, then K block kb+P of the weights into the slot just consumed; also past the last K
-        // block (clamped addresses), so that the number of loads per stage does not depend on the path
-        {
-          const uint32_t kn = uint32_t(min(kb + 2, KB - 1));
-#pragma unroll
-          for (int i = 0; i < CPT; ++i) load16_async(tv[i], tsrc[i] + kn * 128u);
-          FF_W16_REQUEST(s, uint32_t(min(kb + P, KB - 1)));
-        }
-      }
-    }
-    // the last stages have requested (clamped) data nobody reads: let it land before the registers are reused
-    wait_vm<0>();
-#pragma unroll
-    for (int s = 0; s < P; ++s) FF_W16_PIN(s);
-#pragma unroll
-    for (int i = 0; i < CPT; ++i) pin(tv[i]);
-#undef FF_W16_REQUEST
-#undef FF_W16_PIN
-
-    w16_store<MF, MODE>(acc, p, ride, start, n, t, col0, wave, lane);
+    w16_unit_run<F, MF, MODE, P, NW>(p, un_);
   }
 }
 

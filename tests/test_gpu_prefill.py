@@ -422,6 +422,37 @@ def test_prefill_shared_expert_rides_in_the_routed_launches_bitwise(fmt, rows, m
         assert np.array_equal(a, b), what
 
 
+@pytest.mark.parametrize("fmt", [capi.FMT_FP8_BLOCK128, capi.FMT_BF16])
+@pytest.mark.parametrize("rows", [9, 24, 40, 70])
+def test_prefill_shared_expert_on_one_wave_blocks_bitwise(fmt, rows, monkeypatch):
+    """W*A16 cohorts: a shared expert in launches of its own whose four-wave tiles would not fill the CUs runs on one-wave
+    blocks over a quarter of the columns each. Every output element sees the same matrix instructions in the same order:
+    shared_out and the shared activations are the bits of the four-wave launches (FFMOE_PREFILL_SHARED_NARROW=0)."""
+    from helpers import make_table
+    top_k, experts, hidden, inter = 2, 4, 256, 384
+    table, _ = make_table(fmt, experts + 1, hidden, inter, 900 + rows)
+    sh = table.shared_struct(experts)
+    table.experts = experts
+    ids, w = _routing(rows, top_k, experts, 910 + rows, 0.5)
+    x = synth.normal((rows, hidden), 1.0, 920 + rows, dtype=torch.bfloat16).cuda()
+    ids_d, w_d = torch.from_numpy(ids).cuda(), torch.from_numpy(w).cuda()
+    monkeypatch.setenv("FFMOE_PREFILL_SHARED_RIDE", "0")
+    out = {}
+    for narrow in ("0", "1"):
+        monkeypatch.setenv("FFMOE_PREFILL_SHARED_NARROW", narrow)
+        op = ops.PrefillOps(table, rows, top_k, swiglu=capi.SWIGLU_TWICE, routed_weight=capi.WEIGHT_AFTER_DOWN_BF16, weights_f32=True,
+                            shared=sh, act_mode=capi.ACT_BF16)
+        op.contributions.zero_(); op.shared_out.zero_(); op.scratch.zero_()
+        print("fmt=%d rows=%d narrow=%s" % (fmt, rows, narrow), flush=True)
+        got = op.contribute(x, ids_d, w_d)
+        torch.cuda.synchronize()
+        v = op.scratch_views()
+        out[narrow] = (bits(got).copy(), bits(op.shared_out).copy(), bits(v["sh_act"]).copy())
+    assert np.any(out["0"][1] != 0) and np.any(out["0"][2] != 0)
+    for a, b, what in zip(out["0"], out["1"], ("contributions", "shared_out", "shared activations")):
+        assert np.array_equal(a, b), what
+
+
 @pytest.mark.parametrize("rows,mf,hidden,inter", [(70, "1", 512, 256), (70, "4", 256, 768), (9, "2", 1024, 256), (150, "2", 256, 512), (200, "wide", 768, 512)])
 def test_prefill_nvfp4_line_kernel_equals_the_k_block_kernel_bitwise(rows, mf, hidden, inter, monkeypatch):
     """NVFP4 experts whose rows are whole 128-byte code lines (K a multiple of 256) go through a kernel that moves whole
@@ -458,22 +489,23 @@ def test_prefill_nvfp4_line_kernel_equals_the_k_block_kernel_bitwise(rows, mf, h
         assert np.array_equal(a, b), what
 
 
-@pytest.mark.parametrize("rows", [8, 16, 32, 33])
-def test_decode_nvfp4_cohort_with_a_streaming_shared_expert_of_another_format(rows, monkeypatch):
+@pytest.mark.parametrize("rows", [8, 16, 64, 65])
+@pytest.mark.parametrize("shared_inter", [256, 512])
+def test_decode_nvfp4_cohort_with_a_bf16_shared_expert(rows, shared_inter, monkeypatch):
     """ffmoe_decode_contribute, NVFP4 experts with whole code lines and a BF16 shared expert, 8 rows and more: the routed
-    choices run on the line-wise cohort kernel (the bits of ffmoe_prefill_contribute in the W*A16 arithmetic), the shared
-    expert on the streaming kernels in an arena of its own behind the cohort's (the bits of the all-streaming dispatch) -
-    in one call and issued stage by stage. Beyond 32 rows the shared expert moves to the matrix cores as well."""
+    choices run on the line-wise cohort kernel (the bits of ffmoe_prefill_contribute in the W*A16 arithmetic); the shared
+    expert stays on the streaming kernels in an arena of its own behind the cohort's (the bits of the all-streaming
+    dispatch) up to 24 rows and moves to the matrix cores beyond - in one call and issued stage by stage."""
     from helpers import make_table
     top_k, experts, hidden, inter = 3, 6, 256, 512
     table, _ = make_table(capi.FMT_NVFP4, experts, hidden, inter, 800 + rows)
-    sh_table, _ = make_table(capi.FMT_BF16, 1, hidden, inter, 801 + rows)
+    sh_table, _ = make_table(capi.FMT_BF16, 1, hidden, shared_inter, 801 + rows)
     sh = sh_table.shared_struct(0)
     ids, w = _routing(rows, top_k, experts, 810 + rows, 1.0)
     x = synth.normal((rows, hidden), 1.0, 820 + rows, dtype=torch.bfloat16).cuda()
     ids_d, w_d = torch.from_numpy(ids).cuda(), torch.from_numpy(w).cuda()
-    monkeypatch.delenv("FFMOE_DECODE_COHORT_ROWS", raising=False)
-    monkeypatch.delenv("FFMOE_DECODE_SHARED_STREAM_ROWS", raising=False)
+    for name in ("FFMOE_DECODE_COHORT_ROWS", "FFMOE_DECODE_SHARED_STREAM_ROWS", "FFMOE_PREFILL_SHARED_RIDE"):
+        monkeypatch.delenv(name, raising=False)
 
     def run(stagewise):
         op = ops.DecodeOps(table, sh, rows, top_k, capi.ACT_BF16, capi.SWIGLU_TWICE, 0.0, capi.WEIGHT_AFTER_DOWN_BF16, weights_f32=True)
@@ -485,16 +517,13 @@ def test_decode_nvfp4_cohort_with_a_streaming_shared_expert_of_another_format(ro
             c, so = op.contribute(x, ids_d, w_d)
         torch.cuda.synchronize()
         return bits(c).copy(), bits(so).copy()
+    print("rows=%d shared_inter=%d" % (rows, shared_inter), flush=True)
     got_c, got_s = run(False)
     st_c, st_s = run(True)
     assert np.array_equal(got_c, st_c) and np.array_equal(got_s, st_s), "stage by stage = one call"
     monkeypatch.setenv("FFMOE_DECODE_COHORT_ROWS", "0")
     str_c, str_s = run(False)
-    if rows <= 32:
-        assert np.array_equal(got_s, str_s), "shared expert: the streaming kernels' bits"
-    else:
-        assert np.any(got_s != str_s)
-        assert_close_bf16(got_s, str_s, "shared expert on the matrix cores vs streaming", max_ulp=16)
+    monkeypatch.delenv("FFMOE_DECODE_COHORT_ROWS")
     assert np.any(got_c != str_c), "the routed choices did not move to the cohort kernels"
     pre = ops.PrefillOps(table, rows, top_k, swiglu=capi.SWIGLU_TWICE, routed_weight=capi.WEIGHT_AFTER_DOWN_BF16, weights_f32=True,
                          act_mode=capi.ACT_BF16)
@@ -503,6 +532,11 @@ def test_decode_nvfp4_cohort_with_a_streaming_shared_expert_of_another_format(ro
     assert np.array_equal(got_c, bits(want)), "routed choices: the cohort kernels' bits"
     # and inside the end-to-end bar of the matrix-core path against the streaming kernels
     assert_close_bf16(got_c.reshape(rows * top_k, hidden), str_c.reshape(rows * top_k, hidden), "cohort vs streaming contributions", max_ulp=16)
+    if rows <= 24:
+        assert np.array_equal(got_s, str_s), "shared expert: the streaming kernels' bits"
+    else:
+        assert np.any(got_s != str_s)
+        assert_close_bf16(got_s, str_s, "shared expert on the matrix cores vs streaming", max_ulp=16)
 
 
 @pytest.mark.parametrize("rows,top_k,experts", [(1, 1, 3), (37, 4, 9), (128, 8, 70), (341, 3, 5)])
