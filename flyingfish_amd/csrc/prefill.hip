@@ -418,7 +418,8 @@ int launch_w16_fmt(int format, const W16Params& p, int mf, unsigned blocks, hipS
 }
 
 // One wave per block and a quarter of the tile's columns: for one dense group over few rows (the always-on expert), whose
-// four-wave tiles would be a few dozen blocks on 256 CUs. Block-FP8 and BF16 weights.
+// four-wave tiles would be a few dozen blocks on 256 CUs (a lone wave per CU is bound by the one-stage lead of its token
+// tile, not by its weight loads: four K blocks ahead measured the same as two). Block-FP8 and BF16 weights.
 template <int MODE>
 bool launch_w16_narrow(int format, const W16Params& p, int mf, unsigned blocks, hipStream_t stream) {
 #define FF_NARROW(F_)                                                                                              \
