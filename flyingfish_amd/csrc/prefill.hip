@@ -386,6 +386,15 @@ bool nvfp4_lines_enabled() {
 
 template <class F, int MODE>
 int launch_w16(const W16Params& p, int mf, unsigned blocks, hipStream_t stream, bool wide = false) {
+  if constexpr (std::is_same<F, FmtFp8>::value) {
+    // 16- and 32-row groups (decode batches): whole 128-byte code lines per request (FFMOE_PREFILL_FP8_LINES=0 keeps the
+    // per-K-block kernel; same bits). 64-row groups keep the per-K-block kernel: two sets ahead do not fit their registers
+    const char* le = getenv("FFMOE_PREFILL_FP8_LINES");
+    if (!(le && atoi(le) == 0) && !wide && mf == 1) {
+      hipLaunchKernelGGL((k_w16_fp8_lines<1, MODE, 2>), dim3(blocks), dim3(256), 0, stream, p);
+      return ff_launch_status();
+    }
+  }
   if constexpr (std::is_same<F, FmtNvfp4>::value) {
     // rows of whole 128-byte code lines: the line-wise kernel (FFMOE_PREFILL_NVFP4_LINES=0 keeps the per-K-block one)
     if (p.K % 256 == 0 && nvfp4_lines_enabled()) {

@@ -115,6 +115,10 @@ struct W16<FmtNvfp4> {
 __device__ __forceinline__ void load4_async(uint32_t& d, const void* p) {
   asm volatile("global_load_dword %0, %1, off" : "=v"(d) : "v"(p));
 }
+// load16_async with the streaming hint: the line is the first the L2 gives up again
+__device__ __forceinline__ void load16_async_nt(u32x4& d, uint64_t base, uint32_t offset) {
+  asm volatile("global_load_dwordx4 %0, %1, %2 nt" : "=v"(d) : "v"(offset), "s"(base));
+}
 // At most N of the loads issued so far may still be in flight behind this point. A register is read only after it went
 // through a pin() behind the wait that covers its load (volatile statements keep their order).
 template <int N>
@@ -124,6 +128,7 @@ __device__ __forceinline__ void wait_vm() {
 }
 __device__ __forceinline__ void pin(u32x4& v) { asm volatile("" : "+v"(v)); }
 __device__ __forceinline__ void pin(uint32_t& v) { asm volatile("" : "+v"(v)); }
+__device__ __forceinline__ void pin(float& v) { asm volatile("" : "+v"(v)); }
 
 // formats whose dequantization needs the row (a per-row scale or the global scale)
 template <class F> struct W16NeedsRow { static constexpr bool value = false; };
@@ -555,6 +560,13 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void k_w16_nvfp4_lines(co
   constexpr int CPT = (CHUNKS + NT - 1) / NT;
   constexpr int TILE = TM * 128;
   constexpr int WL = 9;                      // weight loads per set of four K blocks
+  // Short groups (the cohorts of a decode batch) see an expert's codes once: they are requested with the streaming hint,
+  // so that the 128-byte lines of scale bytes, which a row comes back to for eight sets, outlive them in L2 (FETCH_SIZE
+  // 1.28 -> 1.08 x the algorithmic bytes in gate/up, C4 batch 32: 1107 -> 1065 us per layer). It takes whole-line
+  // requests: on the per-K-block kernels, whose requests leave half a line or more for the next K block, the same hint
+  // doubles the traffic (block FP8, batch 64: 1861 -> 2622 us). The 64-row groups of a prefill cohort share an expert's
+  // codes through L2 and keep the plain requests.
+  constexpr bool STREAM = MF <= 2;
   constexpr int U = 4 * P;                   // stages per trip of the K loop
   __shared__ __attribute__((aligned(16))) uint8_t cstage[NW][2][4096];  // [wave][pair of fragments][32 rows x 128 B]
   __shared__ __attribute__((aligned(16))) uint8_t sstage[NW][1024];     // [wave][64 rows x 16 scale bytes]
@@ -624,7 +636,10 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void k_w16_nvfp4_lines(co
 #define FF_NV_REQUEST(s_, sb_)                                                                          \
   do {                                                                                                   \
     _Pragma("unroll") for (int j_ = 0; j_ < 2; ++j_)                                                     \
-      _Pragma("unroll") for (int i_ = 0; i_ < 4; ++i_) load16_async(nvc[s_][j_][i_], ncod[j_] + uint32_t(i_) * rstep + (sb_) * 128u, coff); \
+      _Pragma("unroll") for (int i_ = 0; i_ < 4; ++i_) {                                                 \
+        if constexpr (STREAM) load16_async_nt(nvc[s_][j_][i_], ncod[j_] + uint32_t(i_) * rstep + (sb_) * 128u, coff); \
+        else load16_async(nvc[s_][j_][i_], ncod[j_] + uint32_t(i_) * rstep + (sb_) * 128u, coff);        \
+      }                                                                                                  \
     load16_async(nvs[s_], nscl + (sb_) * 16u);                                                           \
   } while (0)
 #define FF_NV_PIN(s_)                                                                                    \
@@ -729,6 +744,210 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void k_w16_nvfp4_lines(co
 #pragma unroll
           for (int i = 0; i < CPT; ++i) load16_async(tv[(st + 1) & 1][i], tsrc[i] + kt * 128u);
           if (q == 0) FF_NV_REQUEST(s, uint32_t(min((kb >> 2) + P, SB - 1)));
+        }
+      });
+    }
+    wait_vm<0>();
+#pragma unroll
+    for (int s = 0; s < P; ++s) FF_NV_PIN(s);
+#pragma unroll
+    for (int i = 0; i < CPT; ++i) { pin(tv[0][i]); pin(tv[1][i]); }
+#undef FF_NV_REQUEST
+#undef FF_NV_PIN
+
+    w16_store<MF, MODE>(acc, p, ride, start, n, t, col0, wave, lane);
+  }
+}
+
+// Block-FP8 experts the same way: 128 columns of a row are one 128-byte line, a set is two K blocks, and the block scale of a
+// pair of fragments and a set is one float (a pair's 32 rows lie inside one 128-row block). Bit-identical to
+// k_w16_grouped<FmtFp8>, whose requests take half a line per K block and rely on L2 for the other half.
+template <int MF, int MODE, int P, int NW = 4>
+__global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void k_w16_fp8_lines(const W16Params p) {
+  using F = FmtFp8;
+  constexpr int NT = 64 * NW;
+  constexpr int TM = 16 * MF;
+  constexpr int CHUNKS = TM * 8;
+  constexpr int CPT = (CHUNKS + NT - 1) / NT;
+  constexpr int TILE = TM * 128;
+  constexpr int WL = 10;                     // weight loads per set of two K blocks: eight of codes, two block scales
+  // 16-row groups (the cohorts of a decode batch) see an expert's codes once: streaming hint on their whole-line requests
+  constexpr bool STREAM = MF == 1;
+  constexpr int U = 2 * P;                   // stages per trip of the K loop
+  __shared__ __attribute__((aligned(16))) uint8_t cstage[NW][2][4096];  // [wave][pair of fragments][32 rows x 128 B]
+  __shared__ __attribute__((aligned(16))) uint8_t tile[2][TILE];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = uni(tid >> 6);
+  const int K = p.K, N = p.N, KB = K >> 6, SB = K >> 7;
+  const uint32_t total = p.unit_total ? uint32_t(uni(int(load_global<uint32_t>(p.unit_total)))) : p.total_units;
+  const int ntiles = (N + gemm_tile_cols<MODE, NW>() - 1) / gemm_tile_cols<MODE, NW>();
+  // LDS image: a request i of a pair holds rows 8 i + lane / 8, piece lane % 8; an operand read of K block q takes the
+  // 16 bytes of row (16 (f % 2) + lane % 16) at 64 q + 16 (lane / 16)
+  const int wr_off = (lane >> 3) * 128 + (((lane & 7) ^ ((lane >> 4) & 3)) << 4);   // + 1024 i, swizzle key (4 i + lane / 16) % 8
+  const int rd_row = lane & 15, rd_key = rd_row >> 1;  // the swizzle key (row / 2) % 8 is the same for both fragments of a pair
+
+  const uint32_t xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3, per_xcd = gridDim.x >> 3;
+  const uint32_t span = (total + 7u) >> 3;
+  const uint32_t span_end = min(total, (xcd + 1u) * span);
+  for (uint32_t u = xcd * span + slot; u < span_end; u += per_xcd) {
+    const W16Unit un_ = w16_unit<MODE>(p, u, ntiles, TM);
+    const int start = un_.start, n = un_.n, t = un_.t;
+    const bool ride = un_.ride;  // wave-uniform
+    int col0[4];
+#pragma unroll
+    for (int f = 0; f < 4; ++f) col0[f] = MODE == 0 ? t * (32 * NW) + wave * 32 + (f & 1) * 16 : t * (64 * NW) + wave * 64 + f * 16;
+    // fragments 2 j and 2 j + 1 are 32 consecutive rows of one matrix
+    // code addresses: a wave-uniform base per pair (scalar registers) and one byte offset per lane
+    uint64_t ncod[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int which = MODE == 0 ? j : 0;
+      ncod[j] = uni64(un_.wc[which] + uint64_t(min(col0[2 * j], N - 32)) * uint64_t(K));
+    }
+    const uint32_t coff = uint32_t(lane >> 3) * uint32_t(K) + uint32_t(lane & 7) * 16u;
+    const uint32_t rstep = uint32_t(K) * 8u;  // eight rows of codes
+    // block scales: one per pair of fragments (32 rows inside one 128-row block) and set (128 columns)
+    const float* nscl[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int which = MODE == 0 ? j : 0;
+      nscl[j] = reinterpret_cast<const float*>(un_.ws[which]) + size_t(min(col0[2 * j], N - 32) >> 7) * size_t(SB);
+    }
+    u32x4 nvc[P][2][4];
+    float nvs[P][2];
+
+    const uint8_t* tsrc[CPT];
+    int tdst[CPT];
+#pragma unroll
+    for (int i = 0; i < CPT; ++i) {
+      const int q = min(tid + NT * i, CHUNKS - 1);
+      const int m = q >> 3, c = q & 7;
+      const int pos = start + min(m, n - 1);
+      const int row = MODE == 0 && p.perm && !ride ? load_global<int>(p.perm + pos) / p.top_k : pos;
+      tsrc[i] = reinterpret_cast<const uint8_t*>(ride ? p.a_sh : p.a) + size_t(row) * K * 2 + c * 16;
+      tdst[i] = m * 128 + ((c ^ (m & 7)) << 4);
+    }
+    const bool stage_chunk = CHUNKS >= NT || tid < CHUNKS;
+
+    v4f acc[MF][4];
+#pragma unroll
+    for (int m = 0; m < MF; ++m)
+#pragma unroll
+      for (int f = 0; f < 4; ++f) acc[m][f] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+
+#define FF_NV_REQUEST(s_, sb_)                                                                          \
+  do {                                                                                                   \
+    _Pragma("unroll") for (int j_ = 0; j_ < 2; ++j_)                                                     \
+      _Pragma("unroll") for (int i_ = 0; i_ < 4; ++i_) {                                                 \
+        if constexpr (STREAM) load16_async_nt(nvc[s_][j_][i_], ncod[j_] + uint32_t(i_) * rstep + (sb_) * 128u, coff); \
+        else load16_async(nvc[s_][j_][i_], ncod[j_] + uint32_t(i_) * rstep + (sb_) * 128u, coff);        \
+      }                                                                                                  \
+    _Pragma("unroll") for (int j_ = 0; j_ < 2; ++j_) load4_async(nvs[s_][j_], nscl[j_] + (sb_));            \
+  } while (0)
+#define FF_NV_PIN(s_)                                                                                    \
+  do {                                                                                                   \
+    _Pragma("unroll") for (int j_ = 0; j_ < 2; ++j_)                                                     \
+      _Pragma("unroll") for (int i_ = 0; i_ < 4; ++i_) pin(nvc[s_][j_][i_]);                             \
+    _Pragma("unroll") for (int j_ = 0; j_ < 2; ++j_) pin(nvs[s_][j_]);                                     \
+  } while (0)
+    // prologue: the first P weight sets and token tile 0, everything landed; then token tile 1, the last set once more
+    // (a tile has one set's loads and the next tile behind it when it is published) and token tile 2
+#pragma unroll
+    for (int s = 0; s < P; ++s) FF_NV_REQUEST(s, uint32_t(min(s, SB - 1)));
+    u32x4 tv[2][CPT];
+    {
+#pragma unroll
+      for (int i = 0; i < CPT; ++i) {
+        const u32x4 v = load16(tsrc[i]);
+        if (stage_chunk) *reinterpret_cast<u32x4*>(&tile[0][tdst[i]]) = v;
+      }
+      wait_vm<0>();
+#pragma unroll
+      for (int s = 0; s < P; ++s) FF_NV_PIN(s);
+      const uint32_t k1 = uint32_t(min(1, KB - 1)), k2 = uint32_t(min(2, KB - 1));
+#pragma unroll
+      for (int i = 0; i < CPT; ++i) load16_async(tv[1][i], tsrc[i] + k1 * 128u);
+      FF_NV_REQUEST(P - 1, uint32_t(min(P - 1, SB - 1)));
+#pragma unroll
+      for (int i = 0; i < CPT; ++i) load16_async(tv[0][i], tsrc[i] + k2 * 128u);
+    }
+    __syncthreads();
+
+    int tlo[MF], thi[MF];
+#pragma unroll
+    for (int m = 0; m < MF; ++m) {
+      const int trow = 16 * m + (lane & 15);
+      const int q2 = (lane >> 4) * 2;
+      tlo[m] = trow * 128 + (((q2) ^ (trow & 7)) << 4);
+      thi[m] = trow * 128 + (((q2 + 1) ^ (trow & 7)) << 4);
+    }
+    uint8_t* cl = &cstage[wave][0][0];
+    float sc_set[2] = {0.0f, 0.0f};  // block scales of the set at work (its register slot is requested into again after the set's first K block)
+
+    for (int kbo = 0; kbo < KB; kbo += U) {
+      static_for<U>([&](auto st_) {
+        constexpr int st = decltype(st_)::value;
+        const int kb = kbo + st;
+        constexpr int q = st & 1, s = st >> 1;  // K block inside its set, register slot of the set
+        if (kb < KB) {
+          if (q == 0) {
+            // the set was requested 2 P stages ago: behind it the token loads of 2 P - 1 stages and P - 1 later sets
+            wait_vm<(2 * P - 1) * CPT + (P - 1) * WL>();
+            FF_NV_PIN(s);
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+              for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(cl + j * 4096 + i * 1024 + (wr_off ^ ((i & 1) << 6))) = nvc[s][j][i];
+            sc_set[0] = nvs[s][0];
+            sc_set[1] = nvs[s][1];
+          }
+          const uint8_t* tb = tile[st & 1];
+          w16_bf16x8 a0[4], a1[4];
+#pragma unroll
+          for (int f = 0; f < 4; ++f) {
+            typename W16<F>::Frag wm;
+            const int row = (f & 1) * 16 + rd_row;
+            const int piece = 4 * q + (lane >> 4);
+            wm.codes = *reinterpret_cast<const u32x4*>(cl + (f >> 1) * 4096 + row * 128 + ((piece ^ rd_key) << 4));
+            wm.scale = sc_set[f >> 1];
+            uint32_t wd[8];
+            W16<F>::dequant(wm, wd);
+            const u32x4 x0 = {wd[0], wd[1], wd[2], wd[3]}, x1 = {wd[4], wd[5], wd[6], wd[7]};
+            a0[f] = __builtin_bit_cast(w16_bf16x8, x0);
+            a1[f] = __builtin_bit_cast(w16_bf16x8, x1);
+          }
+#pragma unroll
+          for (int m = 0; m < MF; ++m) {
+            const u32x4 lo = *reinterpret_cast<const u32x4*>(tb + tlo[m]);
+            const u32x4 hi = *reinterpret_cast<const u32x4*>(tb + thi[m]);
+            const w16_bf16x8 b0 = __builtin_bit_cast(w16_bf16x8, lo), b1 = __builtin_bit_cast(w16_bf16x8, hi);
+#pragma unroll
+            for (int f = 0; f < 4; ++f) {
+              acc[m][f] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0[f], b0, acc[m][f], 0, 0, 0);
+              acc[m][f] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1[f], b1, acc[m][f], 0, 0, 0);
+            }
+          }
+          // publish token tile kb+1: requested two stages ago, behind it tile kb+2 and the one set the two stages requested
+          wait_vm<CPT + WL>();
+#pragma unroll
+          for (int i = 0; i < CPT; ++i) {
+            pin(tv[(st + 1) & 1][i]);
+            if (stage_chunk) *reinterpret_cast<u32x4*>(&tile[(st + 1) & 1][tdst[i]]) = tv[(st + 1) & 1][i];
+          }
+          __syncthreads();
+        } else {
+          // past the last K block: registers with (clamped) loads in flight are about to be requested into again
+          wait_vm<0>();
+#pragma unroll
+          for (int ss = 0; ss < P; ++ss) FF_NV_PIN(ss);
+#pragma unroll
+          for (int i = 0; i < CPT; ++i) { pin(tv[0][i]); pin(tv[1][i]); }
+        }
+        {
+          const uint32_t kt = uint32_t(min(kb + 3, KB - 1));
+#pragma unroll
+          for (int i = 0; i < CPT; ++i) load16_async(tv[(st + 1) & 1][i], tsrc[i] + kt * 128u);
+          if (q == 0) FF_NV_REQUEST(s, uint32_t(min((kb >> 1) + P, SB - 1)));
         }
       });
     }

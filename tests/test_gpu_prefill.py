@@ -453,16 +453,20 @@ def test_prefill_shared_expert_on_one_wave_blocks_bitwise(fmt, rows, monkeypatch
         assert np.array_equal(a, b), what
 
 
-@pytest.mark.parametrize("rows,mf,hidden,inter", [(70, "1", 512, 256), (70, "4", 256, 768), (9, "2", 1024, 256), (150, "2", 256, 512), (200, "wide", 768, 512)])
-def test_prefill_nvfp4_line_kernel_equals_the_k_block_kernel_bitwise(rows, mf, hidden, inter, monkeypatch):
-    """NVFP4 experts whose rows are whole 128-byte code lines (K a multiple of 256) go through a kernel that moves whole
-    lines four K blocks at a time, two sets ahead. Same operands into the same matrix instructions in the same order:
-    contributions, activations and the riding shared expert's outputs are the bits of the per-K-block kernel
-    (FFMOE_PREFILL_NVFP4_LINES=0), for every group size, one set per contraction (K = 256), an odd number of sets
-    (K = 768) and rows that do not fill the last group."""
+@pytest.mark.parametrize("fmt,switch", [(capi.FMT_NVFP4, "FFMOE_PREFILL_NVFP4_LINES"), (capi.FMT_FP8_BLOCK128, "FFMOE_PREFILL_FP8_LINES")])
+@pytest.mark.parametrize("rows,mf,hidden,inter", [(70, "1", 512, 256), (70, "4", 256, 768), (9, "2", 1024, 256), (150, "2", 256, 512), (200, "wide", 768, 512),
+                                                  (33, "1", 384, 640)])
+def test_prefill_line_kernels_equal_the_k_block_kernel_bitwise(fmt, switch, rows, mf, hidden, inter, monkeypatch):
+    """NVFP4 experts whose rows are whole 128-byte code lines (K a multiple of 256) and block-FP8 experts (K a multiple of
+    128) go through kernels that move whole lines, several K blocks at a time and two sets ahead. Same operands into the
+    same matrix instructions in the same order: contributions, activations and the riding shared expert's outputs are the
+    bits of the per-K-block kernel (the switch = 0), for every group size, one set per contraction, odd numbers of sets
+    and rows that do not fill the last group."""
+    if fmt == capi.FMT_NVFP4 and (hidden % 256 or inter % 256):
+        pytest.skip("the per-K-block kernel serves these contractions either way")
     from helpers import make_table
     top_k, experts = 3, 5
-    table, _ = make_table(capi.FMT_NVFP4, experts + 1, hidden, inter, 700 + rows)
+    table, _ = make_table(fmt, experts + 1, hidden, inter, 700 + rows)
     sh = table.shared_struct(experts)
     table.experts = experts
     ids, w = _routing(rows, top_k, experts, 710 + rows, 1.2)
@@ -475,11 +479,11 @@ def test_prefill_nvfp4_line_kernel_equals_the_k_block_kernel_bitwise(rows, mf, h
         monkeypatch.setenv("FFMOE_PREFILL_WIDE", "0")
     out = {}
     for lines in ("0", "1"):
-        monkeypatch.setenv("FFMOE_PREFILL_NVFP4_LINES", lines)
+        monkeypatch.setenv(switch, lines)
         op = ops.PrefillOps(table, rows, top_k, swiglu=capi.SWIGLU_TWICE, routed_weight=capi.WEIGHT_AFTER_DOWN_BF16, weights_f32=True,
                             shared=sh, act_mode=capi.ACT_BF16)
         op.contributions.zero_(); op.shared_out.zero_(); op.scratch.zero_()
-        print("rows=%d mf=%s hidden=%d inter=%d lines=%s" % (rows, mf, hidden, inter, lines), flush=True)
+        print("fmt=%d rows=%d mf=%s hidden=%d inter=%d lines=%s" % (fmt, rows, mf, hidden, inter, lines), flush=True)
         got = op.contribute(x, ids_d, w_d)
         torch.cuda.synchronize()
         v = op.scratch_views()
