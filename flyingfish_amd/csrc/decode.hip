@@ -334,15 +334,14 @@ static int decode_dispatch(const ffmoe_expert_table* table, const ffmoe_shared_e
   }
   // Row counts from which the matrix-core cohort kernels take over for block-FP8 experts (same effective weights and BF16
   // boundaries, the dot products in the matrix instruction's FP32 order instead of the wave's). The whole batch goes there
-  // from FFMOE_DECODE_COHORT_ROWS on: 8 when the shared expert rides in the routed launches (same format and width, or no
+  // from FFMOE_DECODE_COHORT_ROWS on: 4 when the shared expert rides in the routed launches (same format and width, or no
   // shared expert), 32 when it needs launches of its own, a few dozen blocks each. Per layer at hidden 7168 / 256 experts
-  // with a riding shared expert, cohort against streaming kernels: 4 rows 311 / 313 us, 8 rows 548 / 554, 12 rows 747 / 769,
-  // 16 rows 886 / 939, 24 rows 1166 / 1279, 32 rows 1397 / 1550, 64 rows 1886 / 2402; 2 rows 230 / 166. Below that a
-  // block-FP8 shared expert alone from FFMOE_DECODE_SHARED_COHORT_ROWS on (it has every row: streamed once instead of once
-  // per row group that fits LDS; a BF16 shared expert next to NVFP4 experts measured slower there, 1.88 against 1.80 ms at
-  // 32 rows, and stays on the streaming kernels).
+  // with a riding shared expert, cohort (whole-line kernel) against streaming kernels: 2 rows 200 / 166 us, 3 rows 236 / 235,
+  // 4 rows 277 / 313, 6 rows 368 / 433, 8 rows 485 / 554, 16 rows 810 / 939, 32 rows 1278 / 1550, 64 rows 1730 / 2402. Below
+  // that a block-FP8 shared expert alone from FFMOE_DECODE_SHARED_COHORT_ROWS on (it has every row: streamed once instead of
+  // once per row group that fits LDS).
   // NVFP4 experts whose rows are whole 128-byte lines of codes (hidden and inter multiples of 256) take the line-wise
-  // cohort kernel from FFMOE_DECODE_COHORT_ROWS on as well; next to them a shared expert of another format stays on the
+  // cohort kernel from FFMOE_DECODE_COHORT_ROWS on as well (4 rows 266 / 282 us, 6 rows 352 / 406); next to them a shared expert of another format stays on the
   // streaming kernels up to FFMOE_DECODE_SHARED_STREAM_ROWS = 24 rows and runs on one-wave blocks on the matrix cores
   // beyond (BF16 next to NVFP4 experts at hidden 7168, streaming against matrix cores: 16 rows 725 / 736 us per layer, 32 rows
   // 1123 / 1109, 64 rows 1524 / 1489) and gets an arena of its own behind the cohort's.
@@ -352,7 +351,7 @@ static int decode_dispatch(const ffmoe_expert_table* table, const ffmoe_shared_e
   const char* te = getenv("FFMOE_DECODE_SHARED_STREAM_ROWS");
   const bool rides = !shared || (table && shared->format == table->format && shared->inter == table->inter);
   const bool nv_lines = table && table->format == FFMOE_FMT_NVFP4 && table->hidden % 256 == 0 && table->inter % 256 == 0;
-  const int cohort_rows = ce ? atoi(ce) : (rides || nv_lines ? 8 : 32), shared_rows = se ? atoi(se) : 16;
+  const int cohort_rows = ce ? atoi(ce) : (rides || nv_lines ? 4 : 32), shared_rows = se ? atoi(se) : 16;
   const int stream_rows = te ? atoi(te) : 24;
   if (table && args && args->act_mode == FFMOE_ACT_BF16 && args->rows > 1) {
     const int fmt = table->format, H = table->hidden, I = table->inter, R = args->rows;
