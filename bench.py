@@ -850,6 +850,12 @@ def main():
     k_avg = sum(kt) / len(kt)
     mean_distinct_k = sum(distinct) / len(distinct)
     k_bytes = gate_up_bytes(table, mean_distinct_k, args.batch, dims)
+    # one token, shared expert in another format than the routed experts: stage 0 of the token path is three launches -
+    # the shared expert's gate/up (top-k selection in its prologue) and down, then the routed gate/up - so the shared
+    # expert's down matrix and its output row count here and not in the finish
+    mixed_token = token_path and args.format == "nvfp4"
+    shared_down = table.shared_bytes // 3 + I * 2 + H * 2 if mixed_token else 0
+    k_bytes += shared_down
     achieved = k_bytes / (k_avg * 1e-6) / 1e9
     # second streaming launch: down (+ routing weight; one token: + ordered combine)
     dt, _ = time_stage(1)
@@ -857,7 +863,7 @@ def main():
         dt = sorted(max(t - k_avg, 0.0) for t in dt)
     d_avg = sum(dt) / len(dt)
     d_bytes = (mean_distinct_k * table.weight_bytes_per_expert() + table.shared_bytes) // 3 + args.batch * (K + 1) * I * 2 + \
-        (args.batch * H * 2 if token_path else args.batch * (K + 1) * H * 2)
+        (args.batch * H * 2 if token_path else args.batch * (K + 1) * H * 2) - (shared_down - H * 2 if mixed_token else 0)
 
     out = {
         "metric": "moe_layer_decode_us", "value": us_per_layer, "unit": "us/layer", "n_gpus": 1,
@@ -872,14 +878,18 @@ def main():
                    "weights": "E4M3 + f32 128x128 block scales" if args.format == "fp8" else "E2M1 pairs + E4M3 scale per 16 + f32 global",
                    "act_mode": "FFMOE_ACT_BF16 (W8A16)" if args.format == "fp8" else "BF16 activations (W4A16)",
                    "batch": args.batch, "ring": len(xs), "launch": "eager" if graphs is None else "hip graph per ring slot",
-                   "launches_per_layer": "router logits; gate/up with the top-k selection in its prologue; down + weight + combine" if token_path else
+                   "launches_per_layer": ("router logits; shared expert gate/up with the top-k selection in its prologue; shared expert down; "
+                                          "routed gate/up; routed down + weight + combine with the shared row") if mixed_token else
+                                         "router logits; gate/up with the top-k selection in its prologue; down + weight + combine" if token_path else
                                          "router logits; top-k; grouping; gate/up; down; combine"},
         "tokens_per_s": args.batch / (us_per_layer * 1e-6),
         "distinct_routed_experts": mean_distinct,
         "layer_bytes": bytes_layer,
         "layer_hbm_gbps": bytes_layer / (us_per_layer * 1e-6) / 1e9,
         "layer_hbm_frac": bytes_layer / (us_per_layer * 1e-6) / 1e9 / HBM_PEAK_GBPS,
-        "roofline": {"kernel": "ffmoe::k_decode_stage<%s, S, 0, RG, NR> (gate/up + SwiGLU launch%s)" % (
+        "roofline": {"kernel": ("ffmoe::k_decode_stage<FmtBf16, S, 0|1, 1, NR> x 2 + k_decode_stage<FmtNvfp4, S, 0, 1, NR> (the three launches in front of the "
+                                "finish, as the layer issues them: shared expert gate/up with the top-k selection in its prologue, shared expert down, routed "
+                                "gate/up + SwiGLU)") if mixed_token else "ffmoe::k_decode_stage<%s, S, 0, RG, NR> (gate/up + SwiGLU launch%s)" % (
                          "FmtFp8" if args.format == "fp8" else "FmtNvfp4", ", top-k selection in its prologue, as the layer issues it" if token_path else ""),
                      "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBPS, "traffic": GATE_UP_TRAFFIC_BYTES.get((args.batch, args.experts)) if args.format == "fp8" else None,

@@ -23,6 +23,7 @@ struct RouteInline {
   const float* bias;    // [experts] or NULL
   int score_mode, n_group, topk_group;
   float routed_scaling;
+  int select_k;         // choices to select; 0: the launch's own top_k (a shared-expert-only launch has top_k = 0)
 };
 
 struct DecodeParams {
@@ -57,6 +58,8 @@ struct FinishParams {
   uint16_t* y;            // [hidden]
   uint32_t* status;       // |= 1 when a live choice names an expert that is out of range or not valid
   int mode;               // FFMOE_COMBINE_*
+  const uint16_t* shared_ready;  // [hidden] BF16 output of a shared expert that other launches computed (another format or
+                                 // width than the table's), or NULL: the finish computes d.has_shared's expert itself
   // the whole token layer in one launch (k_token_layer)
   int whole;              // 0: one-token finish, 1: selection, gate/up, down and combine
   uint32_t* h32;          // [(top_k + 1), d.h_stride] activations as (launch tag << 16 | BF16) words; row top_k = shared expert

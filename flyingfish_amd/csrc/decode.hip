@@ -225,7 +225,7 @@ static int decode_impl(const ffmoe_expert_table* table, const ffmoe_shared_exper
   FF_REQUIRE(size_t(kmax_lds) * 2 <= 160 * 1024 / 2, FFMOE_ERR_SHAPE, "row of %d BF16 does not fit the LDS staging", kmax_lds);
 
   DecodeParams p;
-  p.route = route ? *route : RouteInline{nullptr, nullptr, 0, 1, 1, 1.0f};
+  p.route = route ? *route : RouteInline{nullptr, nullptr, 0, 1, 1, 1.0f, 0};
   p.rows = R; p.top_k = K; p.experts = E; p.hidden = H; p.inter = I; p.shared_inter = SI;
   p.has_shared = shared ? 1 : 0;
   p.swiglu = args->swiglu; p.swiglu_limit = args->swiglu_limit; p.routed_weight = args->routed_weight;
@@ -533,8 +533,6 @@ static int token_forward(const ffmoe_expert_table* table, const ffmoe_shared_exp
   FF_REQUIRE(table && args, FFMOE_ERR_NULL, "table/args is NULL");
   FF_REQUIRE(args->rows == 1, FFMOE_ERR_UNSUPPORTED, "ffmoe_decode_token_forward handles one token row (rows=%d)", args->rows);
   FF_REQUIRE(args->act_mode == FFMOE_ACT_BF16, FFMOE_ERR_UNSUPPORTED, "ffmoe_decode_token_forward needs FFMOE_ACT_BF16");
-  FF_REQUIRE(!shared || (shared->format == table->format && shared->inter == table->inter), FFMOE_ERR_UNSUPPORTED,
-             "ffmoe_decode_token_forward needs the shared expert in the table's format and width");
   FF_REQUIRE(combine_mode >= 0 && combine_mode <= FFMOE_COMBINE_ROUTED, FFMOE_ERR_UNSUPPORTED, "unknown combine mode %d", combine_mode);
   FF_REQUIRE(shared || combine_mode == FFMOE_COMBINE_ROUTED, FFMOE_ERR_SHAPE, "combine mode %d needs a shared expert", combine_mode);
   FF_REQUIRE(args->weights_f32 == 1 && args->active == nullptr && args->assignment_gen == nullptr, FFMOE_ERR_UNSUPPORTED,
@@ -564,15 +562,36 @@ static int token_forward(const ffmoe_expert_table* table, const ffmoe_shared_exp
   FF_NO_OVERLAP(y, size_t(table->hidden) * 2, args->x, size_t(table->hidden) * 2);
   // the shared expert takes part only in the modes that add it
   const ffmoe_shared_expert* sh = combine_mode == FFMOE_COMBINE_ROUTED ? nullptr : shared;
-  if (stage_mask & 1) {
-    const RouteInline route{logits, bias, score_mode, n_group, topk_group, routed_scaling};
-    FF_TRY(decode_impl(table, sh, args, 1, stream, -1, 0, nullptr, &route));
+  const RouteInline route{logits, bias, score_mode, n_group, topk_group, routed_scaling};
+  FinishParams fin{};
+  fin.scale = (const uint16_t*)scale; fin.y = (uint16_t*)y; fin.status = status; fin.mode = combine_mode;
+  if (sh && !(sh->format == table->format && sh->inter == table->inter)) {
+    // A shared expert of another format or width (BF16 next to NVFP4 experts) cannot share the routed launches: its
+    // two launches run with the kernels of its own format (second pass of the arena, as in ffmoe_decode_contribute) and
+    // leave the BF16 row in shared_out, which the finish adds where its own shared group's row would go - the same
+    // value, rounded at the same boundary. The selection runs in the prologue of the shared expert's gate/up launch
+    // (wave 0 of every block, next to the three waves that stream the shared rows), so the routed gate/up launch starts
+    // with its ids in memory. Five launches per layer with the logits instead of seven.
+    if (stage_mask & 1) {
+      ffmoe_expert_table as_shared = *table;
+      as_shared.format = sh->format;
+      ffmoe_decode only_shared = *args;
+      only_shared.top_k = 0;
+      RouteInline select = route;
+      select.select_k = K;
+      FF_TRY(decode_impl(&as_shared, sh, &only_shared, 3, stream, K, 1, nullptr, &select));
+      FF_TRY(decode_impl(table, nullptr, args, 1, stream, K, 0, nullptr, nullptr, -1, sh->inter));
+    }
+    if (stage_mask & 2) {
+      FF_PTR16(args->shared_out);
+      FF_NO_OVERLAP(y, size_t(table->hidden) * 2, args->shared_out, size_t(table->hidden) * 2);
+      fin.shared_ready = (const uint16_t*)args->shared_out;
+      FF_TRY(decode_impl(table, nullptr, args, 0, stream, K, 0, &fin, nullptr, -1, sh->inter));
+    }
+    return 0;
   }
-  if (stage_mask & 2) {
-    FinishParams fin{};
-    fin.scale = (const uint16_t*)scale; fin.y = (uint16_t*)y; fin.status = status; fin.mode = combine_mode;
-    FF_TRY(decode_impl(table, sh, args, 0, stream, -1, 0, &fin));
-  }
+  if (stage_mask & 1) FF_TRY(decode_impl(table, sh, args, 1, stream, -1, 0, nullptr, &route));
+  if (stage_mask & 2) FF_TRY(decode_impl(table, sh, args, 0, stream, -1, 0, &fin));
   return 0;
 }
 

@@ -78,6 +78,9 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
   // one token, selection in the prologue: wave 0 selects into LDS, block 0 publishes ids, weights and clean done flags
   __shared__ int s_route_ids[FFMOE_MAX_TOP_K];
   __shared__ float s_route_w[FFMOE_MAX_TOP_K];
+  // NVFP4: the split dot's constants per scale code, one table per matrix of the segment (gate, up | down)
+  constexpr bool NV = std::is_same<F, FmtNvfp4>::value;
+  __shared__ u32x2 s_lut[NV ? 2 * FmtNvfp4::LUT_ENTRIES : 1];
   const bool inline_route = STAGE == 0 && RG == 1 && p.route.logits != nullptr;
   // With a shared expert the selection hides behind it: its units need no routing, so every block first takes its slice
   // of the shared expert's rows on waves 1..3 while wave 0 selects, and the routed units follow once the ids are known.
@@ -168,6 +171,10 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
           for (int v = tid; v < row_words; v += 256) d4[v] = load16(src + base + size_t(v) * 8);
         }
       }
+      if constexpr (NV) {
+        FmtNvfp4::build_lut(s_lut, global[0], tid, 256);
+        if (STAGE == 0) FmtNvfp4::build_lut(s_lut + FmtNvfp4::LUT_ENTRIES, global[1], tid, 256);
+      }
     }
     __syncthreads();
     if (items > 0) {
@@ -212,7 +219,7 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
       };
       auto compute_step = [&](int t, int s) {
         const int chunk = (t % nslabs) * (S * 64) + s * 64 + lane;
-        step_compute<F, NROWS, RG, S>(buf, s, xs, Kg, nchunks, chunk, gn, acc);
+        step_compute<F, NROWS, RG, S, NV>(buf, s, xs, Kg, nchunks, chunk, gn, acc, s_lut, s_lut + (NV ? FmtNvfp4::LUT_ENTRIES : 0), NR);
       };
       auto item_end = [&](int t) {
         const int unit = t / nslabs;
@@ -252,11 +259,12 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
       segment(A, s_lo, s_hi - s_lo, 3, wave - 1, nullptr);
     }
     if (inline_route) {
+      const int select_k = p.route.select_k > 0 ? p.route.select_k : p.top_k;
       if (wave == 0)
-        wave_route_dispatch(p.route.logits, p.route.bias, lane, p.experts, p.top_k, p.route.score_mode, p.route.routed_scaling,
+        wave_route_dispatch(p.route.logits, p.route.bias, lane, p.experts, select_k, p.route.score_mode, p.route.routed_scaling,
                             p.route.n_group, p.route.topk_group, s_route_ids, s_route_w, 1);
       __syncthreads();
-      if (blockIdx.x == 0 && tid < p.top_k) {
+      if (blockIdx.x == 0 && tid < select_k) {
         const_cast<int*>(p.ids)[tid] = s_route_ids[tid];
         reinterpret_cast<float*>(const_cast<void*>(p.weights))[tid] = s_route_w[tid];
         if (p.done) p.done[tid] = 0u;

@@ -32,6 +32,9 @@ __global__ __launch_bounds__(1024) void k_decode_finish(const FinishParams q, co
   __shared__ uint64_t s_codes[GT], s_scales[GT];
   __shared__ float s_glob[GT], s_wk[GT];
   __shared__ int s_slot[GT];
+  // NVFP4: the split dot's constants per scale code, one table per group's down matrix
+  constexpr bool NV = std::is_same<F, FmtNvfp4>::value;
+  __shared__ u32x2 s_lut[NV ? GT * FmtNvfp4::LUT_ENTRIES : 1];
   const int tid = threadIdx.x, lane = tid & 63, nthreads = blockDim.x;
   const int wave = uni(tid >> 6), nw = uni(int(blockDim.x >> 6));
   const int K = p.top_k, I = p.inter, H = p.hidden;
@@ -68,7 +71,7 @@ __global__ __launch_bounds__(1024) void k_decode_finish(const FinishParams q, co
   __syncthreads();
   const int nr = uni(s_groups);                 // routed groups, in combine order
   const int G = nr + (has_shared ? 1 : 0);      // group nr = the shared expert
-  if (G == 0) {  // nothing contributes: y = 0
+  if (G == 0 && !q.shared_ready) {  // nothing contributes: y = 0
     for (int d = blockIdx.x * nthreads + tid; d < H; d += gridDim.x * nthreads) q.y[d] = 0;
     return;
   }
@@ -118,6 +121,9 @@ __global__ __launch_bounds__(1024) void k_decode_finish(const FinishParams q, co
     for (int s = 0; s < S; ++s) issue_unit(u_lo, s);
   }
   // activations of every group -> LDS, behind the first weight requests
+  if constexpr (NV) {
+    for (int g = 0; g < G; ++g) FmtNvfp4::build_lut(s_lut + g * FmtNvfp4::LUT_ENTRIES, s_glob[g], tid, nthreads);
+  }
   {
     const int row_words = I >> 3;
     for (int g = 0; g < G; ++g) {
@@ -137,7 +143,7 @@ __global__ __launch_bounds__(1024) void k_decode_finish(const FinishParams q, co
     for (int m = 0; m < NR; ++m) acc[m][0] = 0.0f;
 #pragma unroll
     for (int s = 0; s < S; ++s) {
-      step_compute<F, NR, 1, S>(buf, s, xs + size_t(g) * I * 2, I, nchunks, s * 64 + lane, 1, acc);
+      step_compute<F, NR, 1, S, NV>(buf, s, xs + size_t(g) * I * 2, I, nchunks, s * 64 + lane, 1, acc, s_lut + (NV ? g * FmtNvfp4::LUT_ENTRIES : 0));
       issue_unit(un, s);
     }
     float total[NR];
@@ -160,7 +166,8 @@ __global__ __launch_bounds__(1024) void k_decode_finish(const FinishParams q, co
       const float c = bround(v);  // the BF16 contribution
       sum = q.mode == FFMOE_COMBINE_BF16 ? bround(__fadd_rn(sum, c)) : __fadd_rn(sum, c);
     }
-    const float sh = has_shared ? bround(s_part[nr * cmax + col]) : 0.0f;  // the BF16 shared output
+    // the BF16 shared output: this launch's own down row, or the row other launches left in memory
+    const float sh = q.shared_ready ? bf16_to_f32(q.shared_ready[b_lo + col]) : (has_shared ? bround(s_part[nr * cmax + col]) : 0.0f);
     float v;
     switch (q.mode) {
       case FFMOE_COMBINE_GATED: v = __fadd_rn(bround(sum), bround(__fmul_rn(sc, sh))); break;
@@ -217,7 +224,8 @@ int launch_finish(const FinishParams& q, hipStream_t st) {
   }
   const int cmax = (p.hidden + blocks - 1) / blocks;
   const size_t lds = size_t(FFMOE_FINISH_GROUPS) * p.inter * 2 + size_t(FFMOE_FINISH_GROUPS) * cmax * 4;
-  if (lds > 64 * 1024) return ff_fail(FFMOE_ERR_UNSUPPORTED, "one-token finish: %zu bytes of LDS per block", lds);
+  const size_t tables = std::is_same<F, FmtNvfp4>::value ? size_t(FFMOE_FINISH_GROUPS) * FmtNvfp4::LUT_ENTRIES * 8 : 0;  // static, next to lds
+  if (lds + tables + 512 > 64 * 1024) return ff_fail(FFMOE_ERR_UNSUPPORTED, "one-token finish: %zu bytes of LDS per block", lds + tables);
   launch_finish_steps<F, NR, 2>(steps, q, blocks, waves * 64, cmax, lds, st);
   return ff_launch_status();
 }

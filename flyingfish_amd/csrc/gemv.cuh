@@ -127,6 +127,39 @@ struct FmtNvfp4 {
       for (int i = 0; i < 4; ++i) o.u[4 * q + i] = o.m[4 * q + i] & 0xffbfffbfu;
     }
   }
+  // The pair (c1, c2) depends on the scale code and the matrix's global scale alone: a table of the 256 codes per
+  // matrix in LDS (entry 256 = zeros, for a masked lane) replaces the dozen instructions per group of 16 by one
+  // 8-byte LDS read. Same formulas, same values.
+  static constexpr int LUT_ENTRIES = 257;
+  static __device__ __forceinline__ void build_lut(u32x2* lut, float global, int tid, int nthreads) {
+    for (int i = tid; i < LUT_ENTRIES; i += nthreads) {
+      const float s = __fmul_rn(e4m3x2_to_f32<false>(uint32_t(i & 255)).x, i < 256 ? global : 0.0f);
+      const float b1 = bround(s), b15 = bround(__fmul_rn(1.5f, s));
+      u32x2 e;
+      e.x = __float_as_uint(__fsub_rn(__fmul_rn(3.0f, b1), __fmul_rn(2.0f, b15)));
+      e.y = __float_as_uint(__fmul_rn(2.0f, __fsub_rn(b15, b1)));
+      lut[i] = e;
+    }
+  }
+  static __device__ __forceinline__ void split_lut(const Chunk& c, Split& o, bool valid, const u32x2* lut) {
+#pragma unroll
+    for (int g = 0; g < 2; ++g) {
+      const uint32_t code = (c.scales >> (8 * g)) & 0xffu;
+      const u32x2 e = lut[valid ? code : 256u];
+      o.c1[g] = __uint_as_float(e.x);
+      o.c2[g] = __uint_as_float(e.y);
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const uint32_t d = c.codes[q];
+      o.m[4 * q + 0] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(d, 1.0f, 0));
+      o.m[4 * q + 1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(d, 1.0f, 1));
+      o.m[4 * q + 2] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(d, 1.0f, 2));
+      o.m[4 * q + 3] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(d, 1.0f, 3));
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o.u[4 * q + i] = o.m[4 * q + i] & 0xffbfffbfu;
+    }
+  }
 };
 
 struct FmtBf16 {
@@ -151,16 +184,23 @@ struct FmtBf16 {
 // One step: this lane's 16-byte chunk of NROWS weight rows against the n activation rows in LDS. The activation
 // chunk is read once and used for every weight row. Straight-line code: a chunk past the end of the row is
 // masked (zero weights), never branched around, so the waits on the prefetched registers stay precise.
-template <class F, int NROWS, int RG, int S>
+// NVFP4 with scale tables in LDS (FmtNvfp4::build_lut): weight rows 0 .. lut_rows-1 use lut0, the rest lut1.
+template <class F, int NROWS, int RG, int S, bool LUT = false>
 __device__ __forceinline__ void step_compute(const typename F::Chunk (&c)[NROWS][S], int s, const uint8_t* xs, int K, int nchunks,
-                                             int chunk, int n, float (&acc)[NROWS][RG]) {
+                                             int chunk, int n, float (&acc)[NROWS][RG], const u32x2* lut0 = nullptr,
+                                             const u32x2* lut1 = nullptr, int lut_rows = NROWS) {
   const bool valid = chunk < nchunks;
   const int cl = valid ? chunk : 0;  // keep the LDS read in range
   if constexpr (std::is_same<F, FmtNvfp4>::value) {
     // two groups of 16 per chunk, each with its own pair of constants (see FmtNvfp4::split)
     FmtNvfp4::Split w[NROWS];
+    if constexpr (LUT) {
 #pragma unroll
-    for (int m = 0; m < NROWS; ++m) FmtNvfp4::split(c[m][s], w[m], valid);
+      for (int m = 0; m < NROWS; ++m) FmtNvfp4::split_lut(c[m][s], w[m], valid, m < lut_rows ? lut0 : lut1);
+    } else {
+#pragma unroll
+      for (int m = 0; m < NROWS; ++m) FmtNvfp4::split(c[m][s], w[m], valid);
+    }
 #pragma unroll
     for (int r = 0; r < RG; ++r) {
       if (RG == 1 || r < n) {

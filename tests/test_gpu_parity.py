@@ -883,6 +883,43 @@ def test_token_forward_two_launches_equal_the_separate_launches(fmt, hidden, int
                 assert np.array_equal(u, v), "%s, combine mode %d" % (name, mode)
 
 
+@pytest.mark.parametrize("fmt,shared_fmt,hidden,inter,shared_inter", [(capi.FMT_NVFP4, capi.FMT_BF16, 512, 256, 256), (capi.FMT_NVFP4, capi.FMT_BF16, 256, 512, 128),
+                                                                     (capi.FMT_FP8_BLOCK128, capi.FMT_BF16, 256, 256, 384), (capi.FMT_FP8_BLOCK128, capi.FMT_FP8_BLOCK128, 256, 256, 512)])
+@pytest.mark.parametrize("experts,n_group,topk_group,top_k", [(64, 1, 1, 3), (256, 8, 4, 8)])
+def test_token_forward_with_a_shared_expert_of_another_format_or_width(fmt, shared_fmt, hidden, inter, shared_inter, experts, n_group, topk_group, top_k):
+    """ffmoe_decode_token_forward next to a shared expert that cannot share the routed launches (BF16 next to NVFP4 experts,
+    or another width): the shared expert's own two launches leave its BF16 row in shared_out and the finish adds that row.
+    ids, weights and y equal the separate launches bit for bit, for every combine mode, over consecutive tokens."""
+    table = make_table(fmt, 4, hidden, inter, 171)[0]
+    slots = table.slots[:4].repeat((experts + 3) // 4, 1)[:experts].contiguous()
+    big = ExpertTable(fmt, experts, hidden, inter, table.storage, slots,
+                      table.global_scales[:4].repeat((experts + 3) // 4, 1)[:experts].contiguous() if table.global_scales is not None else None)
+    sh_table = make_table(shared_fmt, 1, hidden, shared_inter, 172)[0]
+    sh = sh_table.shared_struct(0)
+    router = rand_bf16((experts, hidden), 0.05, 173).to(DEV)
+    bias = (torch.randn(experts, generator=torch.Generator().manual_seed(174)) * 0.1).to(DEV)
+    for mode in (capi.COMBINE_BF16, capi.COMBINE_UNGATED, capi.COMBINE_ACCUM_FP32, capi.COMBINE_ACCUM_BF16):
+        got = {}
+        for two in (False, True):
+            layer = NativeMoe(big, sh, router, bias, 1, top_k, routed_scaling=2.5, n_group=n_group, topk_group=topk_group, combine_mode=mode)
+            layer.two_launch = two
+            layer.inline_select = False
+            outs = []
+            for step in range(3):
+                x = rand_bf16((1, hidden), 1.0, 175 + step).to(DEV)
+                print("token forward fmt=%d shared fmt=%d hidden=%d inter=%d shared inter=%d experts=%d top_k=%d mode=%d two_launch=%d step=%d"
+                      % (fmt, shared_fmt, hidden, inter, shared_inter, experts, top_k, mode, two, step), flush=True)
+                y = bits(layer.run(x)).copy()
+                outs.append((layer.ids.cpu().numpy().copy(), layer.weights.cpu().numpy().copy(), y))
+                assert int(layer.status.item()) == 0
+            assert layer.two_launch == two, "the two-launch path refused the layer"
+            got[two] = outs
+        for a, b in zip(got[False], got[True]):
+            for name, u, v in zip(("ids", "weights", "y"), a, b):
+                assert np.array_equal(u, v), "%s, combine mode %d" % (name, mode)
+        assert np.any(got[True][0][2] != 0)
+
+
 @pytest.mark.parametrize("m", [1, 3, 4])
 @pytest.mark.parametrize("k,n,count", [(7168, 200, 5), (2048, 384, 3), (640, 72, 9)])
 def test_linear_fp8_block_batch_equals_single_calls(m, k, n, count):
