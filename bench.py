@@ -863,7 +863,7 @@ def main():
         dt = sorted(max(t - k_avg, 0.0) for t in dt)
     d_avg = sum(dt) / len(dt)
     d_bytes = (mean_distinct_k * table.weight_bytes_per_expert() + table.shared_bytes) // 3 + args.batch * (K + 1) * I * 2 + \
-        (args.batch * H * 2 if token_path else args.batch * (K + 1) * H * 2) - (shared_down - H * 2 if mixed_token else 0)
+        (args.batch * H * 2 if token_path else args.batch * (K + 1) * H * 2) - (shared_down - 2 * H * 2 if mixed_token else 0)  # mixed: the finish reads the shared row instead of a down matrix
 
     out = {
         "metric": "moe_layer_decode_us", "value": us_per_layer, "unit": "us/layer", "n_gpus": 1,

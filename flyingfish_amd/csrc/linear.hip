@@ -35,6 +35,10 @@ __global__ __launch_bounds__(256) void k_linear(const LinearParams p) {
   const int my_units = w_hi - w_lo;
   const int items = my_units * nslabs;
   const int jw = int(lo) + w_lo;
+  // NVFP4: the split dot's constants per scale code (one global scale per matrix); the first barrier below publishes it
+  constexpr bool NV = std::is_same<F, FmtNvfp4>::value;
+  __shared__ u32x2 s_lut[NV ? FmtNvfp4::LUT_ENTRIES : 1];
+  if constexpr (NV) FmtNvfp4::build_lut(s_lut, global, tid, 256);
   for (int r0 = 0; r0 < p.m; r0 += RG) {
     const int n = p.m - r0 < RG ? p.m - r0 : RG;
     typename F::Chunk buf[1][S];
@@ -60,7 +64,7 @@ __global__ __launch_bounds__(256) void k_linear(const LinearParams p) {
       for (int r = 0; r < RG; ++r) acc[0][r] = 0.0f;
       auto compute_step = [&](int t, int s) {
         const int chunk = (t % nslabs) * (S * 64) + s * 64 + lane;
-        step_compute<F, 1, RG, S>(buf, s, xs, K, nchunks, chunk, n, acc);
+        step_compute<F, 1, RG, S, NV>(buf, s, xs, K, nchunks, chunk, n, acc, s_lut);
       };
       auto item_end = [&](int t) {
         if (t % nslabs != nslabs - 1) return;
