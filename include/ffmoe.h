@@ -296,13 +296,18 @@ int ffmoe_decode_token_layer(const ffmoe_expert_table* table, const ffmoe_shared
  * token (src/backend/cuda/moe/decode.rs:1187-1297; kernels/moe_route.cu:315-390, kernels/moe_ffn.cu:98-302,894-908,
  * kernels/moe_combine.cu:51-116,541-613); ids, weights and y are bit-identical to the separate calls. contributions,
  * shared_out are not written. Arguments as ffmoe_decode_token_layer; the scratch arena needs no preparation.
- * FFMOE_ERR_UNSUPPORTED (nothing launched): rows != 1, top_k > 8, experts not 64 * 2^n, a shared expert of another
- * format or width, an active mask or epochs, or down rows beyond the kernel's register buffers. */
+ * A shared expert of another format or width than the table's (BF16 next to NVFP4 experts) cannot share the routed
+ * launches: its gate/up and down launches run first with the kernels of its own format (the selection then sits in the
+ * prologue of ITS gate/up launch), args->shared_out receives its BF16 row and the finish adds that row - four launches,
+ * the same bits.
+ * FFMOE_ERR_UNSUPPORTED (nothing launched): rows != 1, top_k > 8, experts not 64 * 2^n, an active mask or epochs, or
+ * down rows beyond the kernel's register buffers. */
 int ffmoe_decode_token_forward(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared, const ffmoe_decode* args,
                                const float* logits, const float* bias, int score_mode, float routed_scaling, int n_group,
                                int topk_group, const void* scale, void* y, uint32_t* status, int combine_mode, void* stream);
 /* One launch of the same call, for timing a kernel alone: stage 0 = selection + gate/up, stage 1 = down + combine
- * (stage 0 then stage 1 with the same arguments equals ffmoe_decode_token_forward). No counterpart in the reference. */
+ * (stage 0 then stage 1 with the same arguments equals ffmoe_decode_token_forward; with a shared expert of another
+ * format or width stage 0 also holds that expert's two launches). No counterpart in the reference. */
 int ffmoe_decode_token_forward_stage(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared, const ffmoe_decode* args,
                                      const float* logits, const float* bias, int score_mode, float routed_scaling, int n_group,
                                      int topk_group, const void* scale, void* y, uint32_t* status, int combine_mode, int stage,
