@@ -61,6 +61,7 @@ __device__ __forceinline__ float logit_block_sum(float acc, float* s_part) {
   return total;
 }
 
+constexpr int LOGIT_ROWS = 8;  // token rows per block
 constexpr int LOGIT_PF = 4;  // vectors per thread held in registers: covers hidden <= 8192 in one batch
 
 __device__ __forceinline__ void logits_f32_rows(const uint16_t* __restrict__ x, const uint16_t* __restrict__ router,
@@ -75,8 +76,58 @@ __device__ __forceinline__ void logits_f32_rows(const uint16_t* __restrict__ x, 
 #pragma unroll
     for (int i = 0; i < LOGIT_PF; ++i) {
       const int v = tid + 256 * i;
-      wv[i] = load16(wr + size_t(v < words ? v : tid) * 8);
+      wv[i] = load16(wr + size_t(v < words ? v : words - 1) * 8);
     }
+  }
+  if (one_batch && r1 - r0 <= LOGIT_ROWS) {
+    // The router row stays in registers; the next token row is requested while this one is multiplied, and the block-wide
+    // sums of all the block's rows share one barrier (same products, same order, same tree per row).
+    u32x4 xv[LOGIT_PF], xn[LOGIT_PF];
+    float accs[LOGIT_ROWS];
+#pragma unroll
+    for (int i = 0; i < LOGIT_PF; ++i) {
+      const int v = tid + 256 * i;
+      xn[i] = load16(x + size_t(r0) * hidden + size_t(v < words ? v : words - 1) * 8);
+    }
+#pragma unroll
+    for (int k = 0; k < LOGIT_ROWS; ++k) {
+      accs[k] = 0.0f;
+      if (r0 + k < r1) {
+#pragma unroll
+        for (int i = 0; i < LOGIT_PF; ++i) xv[i] = xn[i];
+        if (r0 + k + 1 < r1) {
+#pragma unroll
+          for (int i = 0; i < LOGIT_PF; ++i) {
+            const int v = tid + 256 * i;
+            xn[i] = load16(x + size_t(r0 + k + 1) * hidden + size_t(v < words ? v : words - 1) * 8);
+          }
+        }
+        float acc = 0.0f;
+#pragma unroll
+        for (int i = 0; i < LOGIT_PF; ++i) {
+          if (tid + 256 * i < words) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              acc = __fmaf_rn(bf16lo(xv[i][q]), bf16lo(wv[i][q]), acc);
+              acc = __fmaf_rn(bf16hi(xv[i][q]), bf16hi(wv[i][q]), acc);
+            }
+          }
+        }
+        accs[k] = acc;
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < LOGIT_ROWS; ++k) {
+      if (r0 + k < r1) {
+        const float w = wave_sum(accs[k]);
+        if ((tid & 63) == 0) s_part[4 * k + (tid >> 6)] = w;
+      }
+    }
+    __syncthreads();
+    if (tid < r1 - r0)
+      logits[size_t(r0 + tid) * experts + e] =
+          __fadd_rn(__fadd_rn(s_part[4 * tid], s_part[4 * tid + 1]), __fadd_rn(s_part[4 * tid + 2], s_part[4 * tid + 3]));
+    return;
   }
   for (int r = r0; r < r1; ++r) {
     const uint16_t* xr = x + size_t(r) * hidden;
@@ -87,13 +138,13 @@ __device__ __forceinline__ void logits_f32_rows(const uint16_t* __restrict__ x, 
 #pragma unroll
         for (int i = 0; i < LOGIT_PF; ++i) {
           const int v = v0 + 256 * i;
-          wv[i] = load16(wr + size_t(v < words ? v : tid) * 8);
+          wv[i] = load16(wr + size_t(v < words ? v : words - 1) * 8);
         }
       }
 #pragma unroll
       for (int i = 0; i < LOGIT_PF; ++i) {
         const int v = v0 + 256 * i;
-        xv[i] = load16(xr + size_t(v < words ? v : tid) * 8);
+        xv[i] = load16(xr + size_t(v < words ? v : words - 1) * 8);
       }
 #pragma unroll
       for (int i = 0; i < LOGIT_PF; ++i) {
@@ -111,11 +162,9 @@ __device__ __forceinline__ void logits_f32_rows(const uint16_t* __restrict__ x, 
   }
 }
 
-constexpr int LOGIT_ROWS = 8;  // token rows per block
-
 __global__ __launch_bounds__(256) void k_route_logits_f32(const uint16_t* __restrict__ x, const uint16_t* __restrict__ router,
                                                           float* __restrict__ logits, int rows, int experts, int hidden) {
-  __shared__ float s_part[4];
+  __shared__ float s_part[4 * LOGIT_ROWS];
   const int r0 = blockIdx.y * LOGIT_ROWS;
   const int r1 = r0 + LOGIT_ROWS < rows ? r0 + LOGIT_ROWS : rows;
   logits_f32_rows(x, router, logits, blockIdx.x, r0, r1, experts, hidden, s_part);
