@@ -352,7 +352,13 @@ static int decode_dispatch(const ffmoe_expert_table* table, const ffmoe_shared_e
   const bool rides = !shared || (table && shared->format == table->format && shared->inter == table->inter);
   const bool nv_lines = table && table->format == FFMOE_FMT_NVFP4 && table->hidden % 256 == 0 && table->inter % 256 == 0;
   const int cohort_rows = ce ? atoi(ce) : (rides || nv_lines ? 4 : 32), shared_rows = se ? atoi(se) : 16;
-  const int stream_rows = te ? atoi(te) : 24;
+  // a BF16 shared expert that the split-contraction kernel takes (dense_splitk.cuh) leaves the streaming kernels with the
+  // routed choices, at 4 rows: hidden 7168 next to NVFP4 experts, 4 / 8 / 16 / 24 rows: 249 / 413 / 665 / 859 us per layer
+  // against 263 / 434 / 691 / 917 with the shared expert streaming
+  const char* ke = getenv("FFMOE_SHARED_SPLITK");
+  const bool shared_splits = table && shared && shared->format == FFMOE_FMT_BF16 && !(ke && atoi(ke) == 0) && table->hidden % 256 == 0 &&
+                             shared->inter % 256 == 0;
+  const int stream_rows = te ? atoi(te) : (shared_splits ? 0 : 24);
   if (table && args && args->act_mode == FFMOE_ACT_BF16 && args->rows > 1) {
     const int fmt = table->format, H = table->hidden, I = table->inter, R = args->rows;
     auto on_matrix_cores = [&](int f, int inter) {

@@ -12,6 +12,7 @@
 #include "w8a8_gemm.cuh"
 #include "w16_gemm.cuh"
 #include "mx_gemm.cuh"
+#include "dense_splitk.cuh"
 #include "api.h"
 #include <algorithm>
 #include <cstdlib>
@@ -536,6 +537,38 @@ int shared_expert_w16(const ffmoe_shared_expert* shared, const void* x, int R, i
   const char* ne = getenv("FFMOE_PREFILL_SHARED_NARROW");
   const bool may_narrow = (shared->format == FFMOE_FMT_BF16 || shared->format == FFMOE_FMT_FP8_BLOCK128) && !(ne && atoi(ne) == 0);
   const unsigned nblocks = ((unsigned)num_cus_p() * 8u) & ~7u;
+  // A BF16 expert over so few rows that the grouped kernels would give it fewer tiles than CUs: blocks of eight waves that
+  // split the contraction (dense_splitk.cuh; FFMOE_SHARED_SPLITK=0 keeps the grouped kernels). Hidden 7168 / intermediate
+  // 2048, 32 rows: 62 + 19 us on one-wave tiles.
+  const char* se = getenv("FFMOE_SHARED_SPLITK");
+  const bool splitk = shared->format == FFMOE_FMT_BF16 && !(se && atoi(se) == 0) && H % 256 == 0 && SI % 256 == 0 &&
+                      sgroups * uint32_t((SI + 127) / 128) < (unsigned)num_cus_p();
+  if (splitk) {
+    // 8 activation columns (gate + up rows in one fragment) or 16 output columns per block; tiles of half that size, for
+    // twice the blocks, measured slower (32 rows: 52 + 34 against 32 + 20 us): every block reads the whole token panel
+    const int mft = R > 32 ? 4 : 2;
+    const unsigned gy = unsigned((R + 16 * mft - 1) / (16 * mft));
+    DenseParams d{};
+    d.rows = R; d.swiglu = swiglu; d.limit = limit;
+    if (stage_mask & 1) {
+      d.x = (const uint16_t*)x; d.w0 = (const uint16_t*)shared->slot[0]; d.w1 = (const uint16_t*)shared->slot[2];
+      d.out = (uint16_t*)act; d.K = H; d.N = SI;
+      const dim3 grid(unsigned(SI / 8), gy);
+      if (mft == 4) hipLaunchKernelGGL((k_dense_bf16_splitk<0, 4, 8>), grid, dim3(512), 0, stream, d);
+      else hipLaunchKernelGGL((k_dense_bf16_splitk<0, 2, 8>), grid, dim3(512), 0, stream, d);
+      FF_TRY(ff_launch_status());
+    }
+    if (stage_mask & 2) {
+      d.x = (const uint16_t*)act; d.w0 = (const uint16_t*)shared->slot[4]; d.w1 = nullptr;
+      d.out = (uint16_t*)shared_out; d.K = SI; d.N = H;
+      // two fragments = 32 output columns per block (32 rows at hidden 7168: 15.2 us against 20.6 with one and 20.7 with four)
+      const dim3 grid(unsigned(H / 32), gy);
+      if (mft == 4) hipLaunchKernelGGL((k_dense_bf16_splitk<2, 4, 16, 2>), grid, dim3(512), 0, stream, d);
+      else hipLaunchKernelGGL((k_dense_bf16_splitk<2, 2, 16, 2>), grid, dim3(512), 0, stream, d);
+      FF_TRY(ff_launch_status());
+    }
+    return 0;
+  }
   if (stage_mask & 1) {
     q.a = (const uint16_t*)x;
     q.w0_codes = shared->slot[0]; q.w0_scales = shared->slot[1]; q.w1_codes = shared->slot[2]; q.w1_scales = shared->slot[3];

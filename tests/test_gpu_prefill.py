@@ -437,6 +437,7 @@ def test_prefill_shared_expert_on_one_wave_blocks_bitwise(fmt, rows, monkeypatch
     x = synth.normal((rows, hidden), 1.0, 920 + rows, dtype=torch.bfloat16).cuda()
     ids_d, w_d = torch.from_numpy(ids).cuda(), torch.from_numpy(w).cuda()
     monkeypatch.setenv("FFMOE_PREFILL_SHARED_RIDE", "0")
+    monkeypatch.setenv("FFMOE_SHARED_SPLITK", "0")  # the grouped kernels, also where the split-contraction kernel would take a BF16 expert
     out = {}
     for narrow in ("0", "1"):
         monkeypatch.setenv("FFMOE_PREFILL_SHARED_NARROW", narrow)
@@ -451,6 +452,48 @@ def test_prefill_shared_expert_on_one_wave_blocks_bitwise(fmt, rows, monkeypatch
     assert np.any(out["0"][1] != 0) and np.any(out["0"][2] != 0)
     for a, b, what in zip(out["0"], out["1"], ("contributions", "shared_out", "shared activations")):
         assert np.array_equal(a, b), what
+
+
+@pytest.mark.parametrize("rows,hidden,inter", [(9, 256, 256), (25, 512, 256), (32, 1792, 512), (33, 256, 768), (64, 768, 256), (65, 512, 512), (130, 256, 256)])
+@pytest.mark.parametrize("mode,limit", [(capi.SWIGLU_TWICE, 0.0), (capi.SWIGLU_CLAMPED_ONCE, 3.0), (capi.SWIGLU_GELU_TWICE, 0.0)])
+def test_prefill_bf16_shared_expert_on_the_split_contraction_kernel(rows, hidden, inter, mode, limit, monkeypatch):
+    """A BF16 shared expert over so few rows that the grouped kernels would give it fewer tiles than CUs runs on blocks whose
+    eight waves split the contraction (hidden and intermediate size multiples of 256). Per stage against the oracle at the
+    north-star bar: activations from x, the down rows from the kernel's own activations; end to end at the composed bar,
+    and next to the grouped kernels' results (FFMOE_SHARED_SPLITK=0)."""
+    from helpers import make_table
+    top_k, experts = 2, 3
+    table, ref = make_table(capi.FMT_BF16, experts + 1, hidden, inter, 930 + rows)
+    sh = table.shared_struct(experts)
+    table.experts = experts
+    ids, w = _routing(rows, top_k, experts, 940 + rows, 0.5)
+    x = synth.normal((rows, hidden), 1.0, 950 + rows, dtype=torch.bfloat16)
+    monkeypatch.setenv("FFMOE_PREFILL_SHARED_RIDE", "0")
+    out = {}
+    for split in ("0", "1"):
+        monkeypatch.setenv("FFMOE_SHARED_SPLITK", split)
+        op = ops.PrefillOps(table, rows, top_k, swiglu=mode, swiglu_limit=limit, routed_weight=capi.WEIGHT_AFTER_DOWN_BF16, weights_f32=True,
+                            shared=sh, act_mode=capi.ACT_BF16)
+        op.contributions.zero_(); op.shared_out.zero_(); op.scratch.zero_()
+        print("rows=%d hidden=%d inter=%d mode=%d split=%s" % (rows, hidden, inter, mode, split), flush=True)
+        got = op.contribute(x.cuda(), torch.from_numpy(ids).cuda(), torch.from_numpy(w).cuda())
+        torch.cuda.synchronize()
+        v = op.scratch_views()
+        out[split] = (bits(got).copy(), bits(op.shared_out).copy(), bits(v["sh_act"]).copy())
+    assert np.array_equal(out["0"][0], out["1"][0]), "the routed choices do not depend on the shared expert's kernel"
+    so, sh_act = out["1"][1], out["1"][2]
+    ge, ue, de = ref[experts]
+    xb = bits(x)
+    want_sh = np.zeros_like(so)
+    for r in range(rows):
+        want, want_act = orc.expert_ffn(xb[r], ge, ue, de, 1.0, mode, limit, 0, orc.LANE8, orc.SILU_DIV, apply_weight=False, return_act=True)
+        assert_close_bf16(sh_act[r][None, :], want_act[None, :], "shared activations row %d" % r)
+        assert_close_bf16(so[r][None, :], orc.expert_down(sh_act[r], de, 1.0, 0, orc.LANE8, False)[None, :], "shared down row %d" % r)
+        want_sh[r] = want
+    assert_close_bf16(so, want_sh, "shared_out, end to end", max_ulp=16)
+    # (the two kernels' FP32 sums differ in order only, which moves a BF16 result about once in 2^15 elements: no bitwise
+    # difference can be demanded of shapes this small)
+    assert_close_bf16(sh_act, out["0"][2], "shared activations against the grouped kernels", max_ulp=4)
 
 
 @pytest.mark.parametrize("fmt,switch", [(capi.FMT_NVFP4, "FFMOE_PREFILL_NVFP4_LINES"), (capi.FMT_FP8_BLOCK128, "FFMOE_PREFILL_FP8_LINES")])
@@ -508,7 +551,7 @@ def test_decode_nvfp4_cohort_with_a_bf16_shared_expert(rows, shared_inter, monke
     ids, w = _routing(rows, top_k, experts, 810 + rows, 1.0)
     x = synth.normal((rows, hidden), 1.0, 820 + rows, dtype=torch.bfloat16).cuda()
     ids_d, w_d = torch.from_numpy(ids).cuda(), torch.from_numpy(w).cuda()
-    for name in ("FFMOE_DECODE_COHORT_ROWS", "FFMOE_DECODE_SHARED_STREAM_ROWS", "FFMOE_PREFILL_SHARED_RIDE"):
+    for name in ("FFMOE_DECODE_COHORT_ROWS", "FFMOE_DECODE_SHARED_STREAM_ROWS", "FFMOE_PREFILL_SHARED_RIDE", "FFMOE_SHARED_SPLITK"):
         monkeypatch.delenv(name, raising=False)
 
     def run(stagewise):
@@ -536,11 +579,16 @@ def test_decode_nvfp4_cohort_with_a_bf16_shared_expert(rows, shared_inter, monke
     assert np.array_equal(got_c, bits(want)), "routed choices: the cohort kernels' bits"
     # and inside the end-to-end bar of the matrix-core path against the streaming kernels
     assert_close_bf16(got_c.reshape(rows * top_k, hidden), str_c.reshape(rows * top_k, hidden), "cohort vs streaming contributions", max_ulp=16)
+    # the BF16 shared expert (hidden and width multiples of 256): blocks that split the contraction at every cohort size
+    assert_close_bf16(got_s, str_s, "shared expert on the matrix cores vs streaming", max_ulp=16)
+    # without that kernel it stays on the streaming kernels up to 24 rows (their bits) and moves to the grouped kernels beyond
+    monkeypatch.setenv("FFMOE_SHARED_SPLITK", "0")
+    _, old_s = run(False)
+    monkeypatch.delenv("FFMOE_SHARED_SPLITK")
     if rows <= 24:
-        assert np.array_equal(got_s, str_s), "shared expert: the streaming kernels' bits"
+        assert np.array_equal(old_s, str_s), "shared expert: the streaming kernels' bits"
     else:
-        assert np.any(got_s != str_s)
-        assert_close_bf16(got_s, str_s, "shared expert on the matrix cores vs streaming", max_ulp=16)
+        assert_close_bf16(old_s, str_s, "shared expert on the grouped kernels vs streaming", max_ulp=16)
 
 
 @pytest.mark.parametrize("rows,top_k,experts", [(1, 1, 3), (37, 4, 9), (128, 8, 70), (341, 3, 5)])
