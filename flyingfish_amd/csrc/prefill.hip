@@ -183,7 +183,7 @@ __global__ __launch_bounds__(256) void k_prefill_units(PrefillBook b, int expert
 // in LDS; an assignment's place in its expert's segment is the number of earlier assignments of that expert.
 constexpr int FFMOE_BOOK_SMALL_MAX = 1024;
 __global__ __launch_bounds__(1024) void k_prefill_book_small(const LiveTest lt, PrefillBook b, int A, int experts, int tm, int tiles0, int tiles1,
-                                                             int rgb, int tgb, int shared_rows) {
+                                                             int rgb, int tgb, int shared_rows, int with_units) {
   __shared__ PlanShared sh;
   __shared__ uint32_t s_cnt[1024];
   __shared__ __attribute__((aligned(16))) int s_id[FFMOE_BOOK_SMALL_MAX];
@@ -199,7 +199,7 @@ __global__ __launch_bounds__(1024) void k_prefill_book_small(const LiveTest lt, 
   __syncthreads();
   const uint32_t c = tid < experts ? s_cnt[tid] : 0u;
   if (tid < experts) b.counts[tid] = c;
-  prefill_plan_body(sh, b, experts, tm, tiles0, tiles1, rgb, tgb, shared_rows, c, true);
+  prefill_plan_body(sh, b, experts, tm, tiles0, tiles1, rgb, tgb, shared_rows, c, with_units != 0);
   // position inside the expert's segment = number of earlier assignments of the same expert; every thread walks the same
   // LDS words (broadcast reads), four at a time
   uint32_t rank = 0;
@@ -712,7 +712,17 @@ int prefill_impl(const ffmoe_expert_table* table, const ffmoe_prefill* args, int
     if (const char* f = getenv("FFMOE_PREFILL_BOOK_SMALL")) small_max = std::max(0, std::min(atoi(f), FFMOE_BOOK_SMALL_MAX));
     const bool small = A <= size_t(small_max);
     if (small) {
-      hipLaunchKernelGGL(k_prefill_book_small, dim3(1), dim3(1024), 0, stream, lt, b, int(A), E, tm, tiles0, tiles1, pick_rgb(), pick_tgb(), ride ? R : 0);
+      // The unit lists are one entry per (row group, column tile): thousands of entries even for a few hundred assignments
+      // (32 rows, top-8 of 256 at hidden 7168: 7260), too many for the one block - from 2048 possible units on they are
+      // written by a launch of their own over as many blocks as they need (FFMOE_PREFILL_BOOK_UNITS overrides the bound)
+      const uint64_t max_units = l.max_groups * uint64_t(tiles0 + tiles1);
+      uint64_t own_launch_from = 2048;
+      if (const char* f = getenv("FFMOE_PREFILL_BOOK_UNITS")) own_launch_from = uint64_t(std::max(0, atoi(f)));
+      const bool split_units = max_units >= own_launch_from;
+      hipLaunchKernelGGL(k_prefill_book_small, dim3(1), dim3(1024), 0, stream, lt, b, int(A), E, tm, tiles0, tiles1, pick_rgb(), pick_tgb(), ride ? R : 0,
+                         split_units ? 0 : 1);
+      if (split_units)
+        hipLaunchKernelGGL(k_prefill_units, dim3((unsigned)((max_units + 255) / 256)), dim3(256), 0, stream, b, E, tm, tiles0, tiles1, pick_rgb(), pick_tgb(), ride ? R : 0);
     } else {
       hipLaunchKernelGGL(k_prefill_zero, dim3((E + 255) / 256), dim3(256), 0, stream, b.counts, E, b.totals);
       hipLaunchKernelGGL(k_prefill_count, dim3((unsigned)((A + FFMOE_COUNT_PER_BLOCK - 1) / FFMOE_COUNT_PER_BLOCK)), dim3(256), 0, stream, lt, b.counts, (long long)A);
