@@ -108,25 +108,33 @@ __device__ __forceinline__ void prefill_plan_body(PlanShared& sh, const PrefillB
   uint32_t* s_tmp = sh.tmp;
   const int tid = threadIdx.x;
   const uint32_t g = (c + tm - 1) / tm;
-  // Hillis-Steele inclusive scans
+  // Inclusive scans of the row and group counts over the block's 1024 threads: inside each wave by six cross-lane steps,
+  // then the sixteen wave totals by the first wave, two barriers for both scans (forty barrier pairs as a block-wide
+  // Hillis-Steele scan, which was most of this block's time)
   uint32_t vr = c, vg = g;
-  s_tmp[tid] = vr; __syncthreads();
-  for (int off = 1; off < 1024; off <<= 1) {
-    const uint32_t add = tid >= off ? s_tmp[tid - off] : 0u;
-    __syncthreads();
-    vr += add; s_tmp[tid] = vr;
-    __syncthreads();
+  const int lane = tid & 63, wv = tid >> 6;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const uint32_t ar = uint32_t(__builtin_amdgcn_ds_bpermute(((lane - off) & 63) << 2, int(vr)));
+    const uint32_t ag = uint32_t(__builtin_amdgcn_ds_bpermute(((lane - off) & 63) << 2, int(vg)));
+    if (lane >= off) { vr += ar; vg += ag; }
   }
-  s_rows[tid + 1] = vr; if (tid == 0) s_rows[0] = 0u;
+  if (lane == 63) { s_tmp[wv] = vr; s_tmp[16 + wv] = vg; }
   __syncthreads();
-  s_tmp[tid] = vg; __syncthreads();
-  for (int off = 1; off < 1024; off <<= 1) {
-    const uint32_t add = tid >= off ? s_tmp[tid - off] : 0u;
-    __syncthreads();
-    vg += add; s_tmp[tid] = vg;
-    __syncthreads();
+  if (wv == 0) {
+    uint32_t tr = lane < 16 ? s_tmp[lane] : 0u, tg = lane < 16 ? s_tmp[16 + lane] : 0u;
+#pragma unroll
+    for (int off = 1; off < 16; off <<= 1) {
+      const uint32_t ar = uint32_t(__builtin_amdgcn_ds_bpermute(((lane - off) & 63) << 2, int(tr)));
+      const uint32_t ag = uint32_t(__builtin_amdgcn_ds_bpermute(((lane - off) & 63) << 2, int(tg)));
+      if (lane >= off) { tr += ar; tg += ag; }
+    }
+    if (lane < 16) { s_tmp[32 + lane] = tr; s_tmp[48 + lane] = tg; }  // inclusive totals of waves 0 .. lane
   }
-  s_groups[tid + 1] = vg; if (tid == 0) s_groups[0] = 0u;
+  __syncthreads();
+  if (wv > 0) { vr += s_tmp[32 + wv - 1]; vg += s_tmp[48 + wv - 1]; }
+  s_rows[tid + 1] = vr; s_groups[tid + 1] = vg;
+  if (tid == 0) { s_rows[0] = 0u; s_groups[0] = 0u; }
   __syncthreads();
   if (tid < experts) { b.offsets[tid] = s_rows[tid]; b.gbase[tid] = s_groups[tid]; }
   if (tid == 0) { b.offsets[experts] = s_rows[experts]; b.gbase[experts] = s_groups[experts]; }
@@ -203,7 +211,7 @@ __global__ __launch_bounds__(1024) void k_prefill_book_small(const LiveTest lt, 
   // position inside the expert's segment = number of earlier assignments of the same expert; every thread walks the same
   // LDS words (broadcast reads), four at a time
   uint32_t rank = 0;
-  const int upto = (A + 3) & ~3;
+  const int upto = my >= 0 ? (tid + 3) & ~3 : 0;  // only earlier assignments count, and only live ones look
   for (int q = 0; q < upto; q += 4) {
     const int4 v = *reinterpret_cast<const int4*>(&s_id[q]);
     rank += uint32_t(v.x == my && q < tid) + uint32_t(v.y == my && q + 1 < tid) + uint32_t(v.z == my && q + 2 < tid) + uint32_t(v.w == my && q + 3 < tid);
