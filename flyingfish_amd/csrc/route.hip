@@ -8,43 +8,75 @@ namespace ffmoe {
 
 // ---------------------------------------------------------------------------------------------
 // logits[r,e] = bf16(fma chain over k ascending). One lane owns one (row, expert) chain
-// (kernels/moe_route.cu:392-403, :536-544). The chain is latency-bound by definition; the lane
-// keeps 8 x 16-byte router words in flight so the dependent fma sequence never waits on memory.
-__global__ __launch_bounds__(64) void k_route_logits_bf16(const uint16_t* __restrict__ x, const uint16_t* __restrict__ router,
-                                                          uint16_t* __restrict__ logits, int rows, int experts, int hidden) {
-  const int e = blockIdx.x * 64 + threadIdx.x;
+// (kernels/moe_route.cu:392-403, :536-544): 2 * hidden dependent fmas, serial by contract. What the lane must not also
+// do is fetch its router row itself - 64 lanes reading 16 bytes each of 64 different rows is 64 cache lines per load
+// instruction, and that, not the chain, was the kernel's time (22.8 us for 64 experts x 2048). A block is four waves: all
+// of them move the router tile of 64 experts x 256 columns and the token row's 256 columns through LDS with coalesced
+// requests (32 lanes per 512-byte row segment), one chunk ahead, and wave 0 runs the 64 chains out of LDS (rows padded by
+// 16 bytes, so the 16 lanes of a quarter wave read 16 different LDS slots).
+constexpr int LOGIT_CHUNK = 256;                      // columns per chunk
+constexpr int LOGIT_ROW_BYTES = LOGIT_CHUNK * 4 + 16;  // a row of the tile as FP32, padded by one 16-byte slot
+__global__ __launch_bounds__(256) void k_route_logits_bf16(const uint16_t* __restrict__ x, const uint16_t* __restrict__ router,
+                                                           uint16_t* __restrict__ logits, int rows, int experts, int hidden) {
+  // 64 router rows + the token row, widened to FP32 by the waves that move them: the chain wave's instruction stream is
+  // then one LDS read per four elements and operand plus the fmas themselves, no unpacking in front of every fma
+  __shared__ __attribute__((aligned(16))) uint8_t tile[2][65 * LOGIT_ROW_BYTES];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int e0 = blockIdx.x * 64;
   const int row = blockIdx.y;
-  const bool live = e < experts;
-  const int words = hidden >> 3;
-  const u32x4* wr = reinterpret_cast<const u32x4*>(router + size_t(live ? e : 0) * hidden);
-  const u32x4* xr = reinterpret_cast<const u32x4*>(x + size_t(row) * hidden);
+  const int words = hidden >> 3;                          // 16-byte pieces (8 columns) per row
+  const int chunks = (words + 31) >> 5;
+  // piece (r, q) of a chunk for i = 0 .. 7: r = (tid + 256 i) / 32, q = (tid + 256 i) % 32; thread tid < 32 also moves piece tid
+  // of the token row. Pieces past the end of the row repeat its last piece; nothing multiplies them.
+  u32x4 regs[8], xreg;
+  auto request = [&](int c) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int idx = tid + 256 * i;
+      const int r = idx >> 5, q = idx & 31;
+      const int er = min(e0 + r, experts - 1);
+      const int piece = min(32 * c + q, words - 1);
+      regs[i] = load16(router + size_t(er) * hidden + size_t(piece) * 8);
+    }
+    if (tid < 32) xreg = load16(x + size_t(row) * hidden + size_t(min(32 * c + tid, words - 1)) * 8);
+  };
+  auto widen = [&](uint8_t* dst, const u32x4& v) {
+    const u32x4 lo = {__float_as_uint(bf16lo(v[0])), __float_as_uint(bf16hi(v[0])), __float_as_uint(bf16lo(v[1])), __float_as_uint(bf16hi(v[1]))};
+    const u32x4 hi = {__float_as_uint(bf16lo(v[2])), __float_as_uint(bf16hi(v[2])), __float_as_uint(bf16lo(v[3])), __float_as_uint(bf16hi(v[3]))};
+    *reinterpret_cast<u32x4*>(dst) = lo;
+    *reinterpret_cast<u32x4*>(dst + 16) = hi;
+  };
+  auto publish = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int idx = tid + 256 * i;
+      widen(&tile[buf][(idx >> 5) * LOGIT_ROW_BYTES + (idx & 31) * 32], regs[i]);
+    }
+    if (tid < 32) widen(&tile[buf][64 * LOGIT_ROW_BYTES + tid * 32], xreg);
+  };
+  request(0);
+  publish(0);
+  __syncthreads();
   float acc = 0.0f;
-  constexpr int PF = 8;
-  int c = 0;
-  for (; c + PF <= words; c += PF) {
-    u32x4 wv[PF];
+  for (int c = 0; c < chunks; ++c) {
+    if (c + 1 < chunks) request(c + 1);
+    if (wave == 0) {
+      const uint8_t* wrow = &tile[c & 1][lane * LOGIT_ROW_BYTES];
+      const uint8_t* xrow = &tile[c & 1][64 * LOGIT_ROW_BYTES];
+      const int nquads = 2 * min(32, words - 32 * c);  // groups of four columns
+      // (reading a batch of groups ahead of the previous batch's fmas by hand measured slower than the compiler's order)
+#pragma unroll 8
+      for (int q = 0; q < nquads; ++q) {
+        const u32x4 wv = *reinterpret_cast<const u32x4*>(wrow + q * 16);
+        const u32x4 xv = *reinterpret_cast<const u32x4*>(xrow + q * 16);
 #pragma unroll
-    for (int p = 0; p < PF; ++p) wv[p] = wr[c + p];
-#pragma unroll
-    for (int p = 0; p < PF; ++p) {
-      const u32x4 xv = xr[c + p];
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        acc = __fmaf_rn(bf16lo(xv[q]), bf16lo(wv[p][q]), acc);
-        acc = __fmaf_rn(bf16hi(xv[q]), bf16hi(wv[p][q]), acc);
+        for (int j = 0; j < 4; ++j) acc = __fmaf_rn(__uint_as_float(xv[j]), __uint_as_float(wv[j]), acc);
       }
     }
+    if (c + 1 < chunks) publish((c + 1) & 1);
+    __syncthreads();
   }
-  for (; c < words; ++c) {
-    const u32x4 wv = wr[c];
-    const u32x4 xv = xr[c];
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      acc = __fmaf_rn(bf16lo(xv[q]), bf16lo(wv[q]), acc);
-      acc = __fmaf_rn(bf16hi(xv[q]), bf16hi(wv[q]), acc);
-    }
-  }
-  if (live) logits[size_t(row) * experts + e] = f32_to_bf16(acc);
+  if (wave == 0 && e0 + lane < experts) logits[size_t(row) * experts + e0 + lane] = f32_to_bf16(acc);
 }
 
 // FP32 logits. One block of 256 threads per expert: thread p chains the 8-element vectors p, p+256, ... in ascending
@@ -359,7 +391,7 @@ extern "C" __attribute__((visibility("default"))) int ffmoe_route_logits_bf16(co
   FF_PTR16(x); FF_PTR16(router); FF_PTR16(logits);
   FF_NO_OVERLAP(logits, size_t(rows) * experts * 2, x, size_t(rows) * hidden * 2);
   FF_NO_OVERLAP(logits, size_t(rows) * experts * 2, router, size_t(experts) * hidden * 2);
-  hipLaunchKernelGGL(k_route_logits_bf16, dim3((experts + 63) / 64, rows), dim3(64), 0, (hipStream_t)stream,
+  hipLaunchKernelGGL(k_route_logits_bf16, dim3((experts + 63) / 64, rows), dim3(256), 0, (hipStream_t)stream,
                      (const uint16_t*)x, (const uint16_t*)router, (uint16_t*)logits, rows, experts, hidden);
   return ff_launch_status();
 }
