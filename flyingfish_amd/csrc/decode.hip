@@ -12,6 +12,8 @@ int decode_launch_fp8(const DecodeParams& p, int rg, int stage_mask, hipStream_t
 int decode_launch_nvfp4(const DecodeParams& p, int rg, int stage_mask, hipStream_t st);
 int decode_launch_bf16(const DecodeParams& p, int rg, int stage_mask, hipStream_t st);
 int decode_launch_fp8c(const DecodeParams& p, int rg, int stage_mask, hipStream_t st);
+bool decode_gate_up_nvfp4_bf16_shared_available(int hidden);
+int decode_gate_up_nvfp4_bf16_shared(const DecodeParams& p, hipStream_t st);
 int decode_finish_fp8(const FinishParams& q, hipStream_t st);
 int decode_finish_nvfp4(const FinishParams& q, hipStream_t st);
 int decode_finish_bf16(const FinishParams& q, hipStream_t st);
@@ -158,7 +160,7 @@ extern "C" __attribute__((visibility("default"))) uint64_t ffmoe_decode_scratch_
 // (both gate/up launches, then both down launches), so neither may overwrite the other's grouping.
 static int decode_impl(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared, const ffmoe_decode* args,
                        int stage_mask, void* stream, int layout_k = -1, int pass = 0, const FinishParams* fin = nullptr,
-                       const RouteInline* route = nullptr, int form = -1, int arena_shared_inter = 0) {
+                       const RouteInline* route = nullptr, int form = -1, int arena_shared_inter = 0, bool mixed_gate_up = false) {
   FF_REQUIRE(table && args, FFMOE_ERR_NULL, "table/args is NULL");
   const int R = args->rows, K = args->top_k, E = table->experts, H = table->hidden, I = table->inter;
   const int LK = layout_k < 0 ? K : layout_k;
@@ -189,8 +191,9 @@ static int decode_impl(const ffmoe_expert_table* table, const ffmoe_shared_exper
   if (fmt == FFMOE_FMT_NVFP4 && K > 0) FF_PTR4(table->global_scales);
   int SI = I;
   if (shared) {
-    FF_REQUIRE(shared->format == fmt, FFMOE_ERR_UNSUPPORTED, "shared expert format %d differs from the table format %d",
-               shared->format, fmt);
+    // mixed_gate_up: NVFP4 experts and a BF16 shared expert in one gate/up launch (one token, selection in the prologue)
+    FF_REQUIRE(shared->format == fmt || (mixed_gate_up && fmt == FFMOE_FMT_NVFP4 && shared->format == FFMOE_FMT_BF16 && route && stage_mask == 1),
+               FFMOE_ERR_UNSUPPORTED, "shared expert format %d differs from the table format %d", shared->format, fmt);
     SI = shared->inter;
     FF_REQUIRE(SI >= gran && SI % gran == 0, FFMOE_ERR_SHAPE, "shared inter=%d must be a positive multiple of %d", SI, gran);
     FF_PTR16(args->shared_out);
@@ -307,6 +310,7 @@ static int decode_impl(const ffmoe_expert_table* table, const ffmoe_shared_exper
       default: return decode_finish_bf16(q, st);
     }
   }
+  if (mixed_gate_up) return decode_gate_up_nvfp4_bf16_shared(p, st);
   switch (fmt) {
     case FFMOE_FMT_FP8_BLOCK128: return decode_launch_fp8(p, rg, stage_mask, st);
     case FFMOE_FMT_NVFP4: return decode_launch_nvfp4(p, rg, stage_mask, st);
@@ -583,10 +587,19 @@ static int token_forward(const ffmoe_expert_table* table, const ffmoe_shared_exp
       as_shared.format = sh->format;
       ffmoe_decode only_shared = *args;
       only_shared.top_k = 0;
-      RouteInline select = route;
-      select.select_k = K;
-      FF_TRY(decode_impl(&as_shared, sh, &only_shared, 3, stream, K, 1, nullptr, &select));
-      FF_TRY(decode_impl(table, nullptr, args, 1, stream, K, 0, nullptr, nullptr, -1, sh->inter));
+      const char* me = getenv("FFMOE_DECODE_MIXED_GATE_UP");
+      if (table->format == FFMOE_FMT_NVFP4 && sh->format == FFMOE_FMT_BF16 && !(me && atoi(me) == 0) &&
+          decode_gate_up_nvfp4_bf16_shared_available(table->hidden)) {
+        // the shared expert's gate/up rows as every block's first slice of the routed gate/up launch, in BF16, next to the
+        // selection; only its down launch is its own: four launches with the logits (FFMOE_DECODE_MIXED_GATE_UP=0: five)
+        FF_TRY(decode_impl(table, sh, args, 1, stream, K, 0, nullptr, &route, -1, sh->inter, true));
+        FF_TRY(decode_impl(&as_shared, sh, &only_shared, 2, stream, K, 1));
+      } else {
+        RouteInline select = route;
+        select.select_k = K;
+        FF_TRY(decode_impl(&as_shared, sh, &only_shared, 3, stream, K, 1, nullptr, &select));
+        FF_TRY(decode_impl(table, nullptr, args, 1, stream, K, 0, nullptr, nullptr, -1, sh->inter));
+      }
     }
     if (stage_mask & 2) {
       FF_PTR16(args->shared_out);

@@ -68,7 +68,13 @@ __device__ __forceinline__ void load_group(const DecodeParams& p, int g, int& ex
 // matrix is in flight at all times and the first requests of a segment go out before the activations are even
 // staged. Reduced sums of up to 64 units are parked one per lane; the epilogue (SwiGLU or weighting, BF16
 // rounding, store) runs once per 64 units with coalesced stores.
-template <class F, int S, int STAGE, int RG, int NR>
+// FSH / SSH: format and steps of the shared expert's rows when they differ from the routed experts' (one token with the
+// selection in the prologue: every block takes its slice of the shared expert first, in that expert's own format, so a
+// BF16 shared expert next to NVFP4 experts needs no gate/up launch of its own). Everything else runs as F / S.
+template <class FF_, int SS_>
+struct SegmentKind { using fmt = FF_; static constexpr int steps = SS_; };
+
+template <class F, int S, int STAGE, int RG, int NR, class FSH = F, int SSH = S>
 __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
   constexpr int NROWS = STAGE == 0 ? 2 * NR : NR;
   extern __shared__ __align__(16) uint8_t xs[];
@@ -79,7 +85,7 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
   __shared__ int s_route_ids[FFMOE_MAX_TOP_K];
   __shared__ float s_route_w[FFMOE_MAX_TOP_K];
   // NVFP4: the split dot's constants per scale code, one table per matrix of the segment (gate, up | down)
-  constexpr bool NV = std::is_same<F, FmtNvfp4>::value;
+  constexpr bool NV = std::is_same<F, FmtNvfp4>::value || std::is_same<FSH, FmtNvfp4>::value;
   __shared__ u32x2 s_lut[NV ? 2 * FmtNvfp4::LUT_ENTRIES : 1];
   const bool inline_route = STAGE == 0 && RG == 1 && p.route.logits != nullptr;
   // With a shared expert the selection hides behind it: its units need no routing, so every block first takes its slice
@@ -94,7 +100,10 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
 
   // One segment: `count` units of group g from unit j0 on, split over the waves wv = 0 .. nw-1 (wv < 0: this wave only
   // takes part in the staging and the barriers).
-  auto segment = [&](int g, int j0, int count, int nw, int wv, const int* inline_ids) {
+  auto segment = [&](auto kind, int g, int j0, int count, int nw, int wv, const int* inline_ids) {
+    using FF = typename decltype(kind)::fmt;
+    constexpr int SS = decltype(kind)::steps;
+    constexpr bool NVF = std::is_same<FF, FmtNvfp4>::value;
     int expert, gn, grow[RG], gslot[RG];
     load_group<RG>(p, g, expert, gn, grow, gslot, inline_ids);
     const bool shared = expert < 0;
@@ -136,27 +145,27 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
                               : bf16_to_f32(uint16_t(uni(int(load_global<uint16_t>(reinterpret_cast<const uint16_t*>(p.weights) + gslot[r])))));
       }
     }
-    const int nchunks = Kg / F::EPL;
-    const int nslabs = (nchunks + S * 64 - 1) / (S * 64);
+    const int nchunks = Kg / FF::EPL;
+    const int nslabs = (nchunks + SS * 64 - 1) / (SS * 64);
     // this wave's contiguous run of units inside the segment
     const int w_lo = wv >= 0 ? count * wv / nw : 0, w_hi = wv >= 0 ? count * (wv + 1) / nw : 0;
     const int my_units = gn > 0 ? w_hi - w_lo : 0;
     const int items = my_units * nslabs;
     const int jw = j0 + w_lo;  // first unit of the run
-    typename F::Chunk buf[NROWS][S];
+    typename FF::Chunk buf[NROWS][SS];
     auto issue_step = [&](int t, int s) {
       const int j = (jw + t / nslabs) * NR;  // first output row of the unit
-      const int chunk = (t % nslabs) * (S * 64) + s * 64 + lane;
+      const int chunk = (t % nslabs) * (SS * 64) + s * 64 + lane;
       const int cc = chunk < nchunks ? chunk : nchunks - 1;
 #pragma unroll
       for (int m = 0; m < NROWS; ++m) {
         const int mat = m / NR;
-        F::load(buf[m][s], F::row(codes[mat], scales[mat], global[mat], j + (m % NR), Kg), cc);
+        FF::load(buf[m][s], FF::row(codes[mat], scales[mat], global[mat], j + (m % NR), Kg), cc);
       }
     };
     if (items > 0) {
 #pragma unroll
-      for (int s = 0; s < S; ++s) issue_step(0, s);
+      for (int s = 0; s < SS; ++s) issue_step(0, s);
     }
     // activations of the group -> LDS (row r at r*Kg*2), behind the first weight requests
     __syncthreads();  // the previous segment's readers are done with xs
@@ -171,7 +180,7 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
           for (int v = tid; v < row_words; v += 256) d4[v] = load16(src + base + size_t(v) * 8);
         }
       }
-      if constexpr (NV) {
+      if constexpr (NVF) {
         FmtNvfp4::build_lut(s_lut, global[0], tid, 256);
         if (STAGE == 0) FmtNvfp4::build_lut(s_lut + FmtNvfp4::LUT_ENTRIES, global[1], tid, 256);
       }
@@ -218,8 +227,8 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
         }
       };
       auto compute_step = [&](int t, int s) {
-        const int chunk = (t % nslabs) * (S * 64) + s * 64 + lane;
-        step_compute<F, NROWS, RG, S, NV>(buf, s, xs, Kg, nchunks, chunk, gn, acc, s_lut, s_lut + (NV ? FmtNvfp4::LUT_ENTRIES : 0), NR);
+        const int chunk = (t % nslabs) * (SS * 64) + s * 64 + lane;
+        step_compute<FF, NROWS, RG, SS, NVF>(buf, s, xs, Kg, nchunks, chunk, gn, acc, s_lut, s_lut + (NVF ? FmtNvfp4::LUT_ENTRIES : 0), NR);
       };
       auto item_end = [&](int t) {
         const int unit = t / nslabs;
@@ -239,14 +248,14 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
       };
       for (int t = 0; t + 1 < items; ++t) {
 #pragma unroll
-        for (int s = 0; s < S; ++s) {
+        for (int s = 0; s < SS; ++s) {
           compute_step(t, s);
           issue_step(t + 1, s);
         }
         item_end(t);
       }
 #pragma unroll
-      for (int s = 0; s < S; ++s) compute_step(items - 1, s);
+      for (int s = 0; s < SS; ++s) compute_step(items - 1, s);
       item_end(items - 1);
       if (my_units & 63) flush(my_units & ~63, my_units & 63);
     }
@@ -256,7 +265,7 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
     if (shared_first) {
       // this block's slice of the shared expert (group A: rows == 1), waves 1..3; wave 0 selects meanwhile
       const int s_lo = int((long long)out_s * blockIdx.x / gridDim.x), s_hi = int((long long)out_s * (blockIdx.x + 1) / gridDim.x);
-      segment(A, s_lo, s_hi - s_lo, 3, wave - 1, nullptr);
+      segment(SegmentKind<FSH, SSH>{}, A, s_lo, s_hi - s_lo, 3, wave - 1, nullptr);
     }
     if (inline_route) {
       const int select_k = p.route.select_k > 0 ? p.route.select_k : p.top_k;
@@ -280,7 +289,7 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
     if (u0 < routed_units) { g = int(u0 / out_r); j0 = int(u0 % out_r); width = out_r; }
     else { const long long v = u0 - routed_units; g = n_routed + int(v / out_s); j0 = int(v % out_s); width = out_s; }
     const long long seg_end = u0 + (width - j0) < hi ? u0 + (width - j0) : hi;
-    segment(g, j0, int(seg_end - u0), 4, wave, inline_route ? s_route_ids : nullptr);
+    segment(SegmentKind<F, S>{}, g, j0, int(seg_end - u0), 4, wave, inline_route ? s_route_ids : nullptr);
     u0 = seg_end;
   }
 }
