@@ -299,7 +299,8 @@ int ffmoe_decode_token_layer(const ffmoe_expert_table* table, const ffmoe_shared
  * A shared expert of another format or width than the table's (BF16 next to NVFP4 experts) cannot share the routed
  * launches: its gate/up and down launches run first with the kernels of its own format (the selection then sits in the
  * prologue of ITS gate/up launch), args->shared_out receives its BF16 row and the finish adds that row - four launches,
- * the same bits.
+ * the same bits. (NVFP4 experts next to a BF16 shared expert at hidden 2048 / 4096 / 7168 / 8192: the shared gate/up rows run
+ * inside the routed gate/up launch, in BF16, and only the shared down launch is its own - three launches.)
  * FFMOE_ERR_UNSUPPORTED (nothing launched): rows != 1, top_k > 8, experts not 64 * 2^n, an active mask or epochs, or
  * down rows beyond the kernel's register buffers. */
 int ffmoe_decode_token_forward(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared, const ffmoe_decode* args,
