@@ -588,8 +588,12 @@ static int token_forward(const ffmoe_expert_table* table, const ffmoe_shared_exp
       ffmoe_decode only_shared = *args;
       only_shared.top_k = 0;
       const char* me = getenv("FFMOE_DECODE_MIXED_GATE_UP");
-      if (table->format == FFMOE_FMT_NVFP4 && sh->format == FFMOE_FMT_BF16 && !(me && atoi(me) == 0) &&
-          decode_gate_up_nvfp4_bf16_shared_available(table->hidden)) {
+      if (sh->format == table->format && !(me && atoi(me) == 0)) {
+        // same format, another width: the gate/up launch takes shared rows of any width as it is; only the finish cannot
+        FF_TRY(decode_impl(table, sh, args, 1, stream, K, 0, nullptr, &route, -1, sh->inter));
+        FF_TRY(decode_impl(&as_shared, sh, &only_shared, 2, stream, K, 1));
+      } else if (table->format == FFMOE_FMT_NVFP4 && sh->format == FFMOE_FMT_BF16 && !(me && atoi(me) == 0) &&
+                 decode_gate_up_nvfp4_bf16_shared_available(table->hidden)) {
         // the shared expert's gate/up rows as every block's first slice of the routed gate/up launch, in BF16, next to the
         // selection; only its down launch is its own: four launches with the logits (FFMOE_DECODE_MIXED_GATE_UP=0: five)
         FF_TRY(decode_impl(table, sh, args, 1, stream, K, 0, nullptr, &route, -1, sh->inter, true));
