@@ -116,6 +116,11 @@ __device__ __forceinline__ void logits_f32_rows(const uint16_t* __restrict__ x, 
     // sums of all the block's rows share one barrier (same products, same order, same tree per row).
     u32x4 xv[LOGIT_PF], xn[LOGIT_PF];
     float accs[LOGIT_ROWS];
+    float wf[LOGIT_PF][8];  // the router row widened once, not once per token row
+#pragma unroll
+    for (int i = 0; i < LOGIT_PF; ++i)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) { wf[i][2 * q] = bf16lo(wv[i][q]); wf[i][2 * q + 1] = bf16hi(wv[i][q]); }
 #pragma unroll
     for (int i = 0; i < LOGIT_PF; ++i) {
       const int v = tid + 256 * i;
@@ -140,8 +145,8 @@ __device__ __forceinline__ void logits_f32_rows(const uint16_t* __restrict__ x, 
           if (tid + 256 * i < words) {
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-              acc = __fmaf_rn(bf16lo(xv[i][q]), bf16lo(wv[i][q]), acc);
-              acc = __fmaf_rn(bf16hi(xv[i][q]), bf16hi(wv[i][q]), acc);
+              acc = __fmaf_rn(bf16lo(xv[i][q]), wf[i][2 * q], acc);
+              acc = __fmaf_rn(bf16hi(xv[i][q]), wf[i][2 * q + 1], acc);
             }
           }
         }
