@@ -65,8 +65,8 @@ __global__ __launch_bounds__(1024) void k_decode_finish(const FinishParams q, co
   using B0 = std::integral_constant<int, 0>;
   using B1 = std::integral_constant<int, 1>;
   // The shared expert's down matrix is a kernel argument, the routed ones are two dependent loads away (ids, then the slot
-  // table): wave w < P takes unit w of the shared expert as its first unit and requests it before anything else, so the
-  // first weights are on their way while the block finds out which experts were chosen.
+  // table): the shared expert's units w, w + nw, ... < P are wave w's first units, and it requests the first of them before
+  // anything else, so the first weights are on their way while the block finds out which experts were chosen.
   const bool first_shared = has_shared && wave < P;
   if (first_shared) {
 #pragma unroll
@@ -124,15 +124,15 @@ __global__ __launch_bounds__(1024) void k_decode_finish(const FinishParams q, co
   }
   __syncthreads();
 
-  // this wave's units: the shared expert's unit `wave` first (waves below P), then a contiguous run of the routed groups'
+  // this wave's units: the shared expert's units wave, wave + nw, ... first, then a contiguous run of the routed groups'
   // units (group-major: group g, rows b_lo + NR * i ..). Which wave computes a unit does not change its result.
   const int Ur = nr * P;
   const int r_lo = Ur * wave / nw, r_hi = Ur * (wave + 1) / nw;
-  const int lead = first_shared ? 1 : 0;
+  const int lead = first_shared ? (P - wave + nw - 1) / nw : 0;  // shared units of this wave
   const int my_units = lead + (r_hi - r_lo);
   auto unit_of = [&](int t, int& g, int& i) {  // units past the run name its last unit again; nothing reads those requests
     const int tc = t < my_units ? t : my_units - 1;
-    if (first_shared && tc == 0) { g = nr; i = wave; return; }
+    if (tc < lead) { g = nr; i = wave + tc * nw; return; }
     const int r = r_lo + tc - lead;
     g = r / P;
     i = r - g * P;

@@ -416,6 +416,8 @@ def test_decode_shared_expert_in_another_format(rows, routed_fmt, shared_fmt, sh
     (capi.FMT_FP8_BLOCK128, 1024, 384, 4, False),    # routed only
     (capi.FMT_NVFP4, 1024, 512, 6, True),
     (capi.FMT_BF16, 1024, 256, 2, True),
+    (capi.FMT_FP8_BLOCK128, 9216, 256, 2, True),     # 36 columns per block on 256 CUs: 9 shared units for 8 waves
+    (capi.FMT_FP8_BLOCK128, 16384, 128, 1, True),    # 64 columns per block: 16 shared units
 ])
 def test_decode_finish_equals_down_plus_combine(fmt, hidden, inter, top_k, shared):
     """One-token finish (one launch) against the separate down and combine launches: bit-identical y in every
@@ -451,6 +453,28 @@ def test_decode_finish_equals_down_plus_combine(fmt, hidden, inter, top_k, share
             torch.cuda.synchronize()
             assert int(status.item()) == 0
             assert np.array_equal(bits(y), bits(want)), "mode %d active %s" % (mode, with_active)
+
+
+@pytest.mark.parametrize("shape", ["16,8", "128,8", "7,12", "3,16"])
+def test_decode_finish_shape_override_keeps_the_bits(shape, monkeypatch):
+    """FFMOE_FINISH_SHAPE = "blocks,waves" changes the launch shape only: also where a block holds more shared-expert
+    units than it has waves (16 blocks of 64 columns = 16 units on 8 waves), y stays what the separate launches give."""
+    experts, hidden, inter, top_k, seed = 6, 1024, 256, 3, 131
+    table, _ = make_table(capi.FMT_FP8_BLOCK128, experts + 1, hidden, inter, seed)
+    sh = table.shared_struct(experts)
+    table.experts = experts
+    x = rand_bf16((1, hidden), 1.0, seed + 1).to(DEV)
+    ids = torch.tensor([[4, 0, 3]], dtype=torch.int32, device=DEV)
+    wt = torch.tensor([[0.4, 0.25, 0.35]], device=DEV)
+    op = DecodeOps(table, sh, 1, top_k, capi.ACT_BF16, capi.SWIGLU_TWICE, 0.0, capi.WEIGHT_AFTER_DOWN_BF16, True)
+    contrib, shared_out = op.contribute(x, ids, wt)
+    want = CombineOps.combine(contrib, shared_out, ids, capi.COMBINE_UNGATED, done=op.done)
+    monkeypatch.setenv("FFMOE_FINISH_SHAPE", shape)
+    y = torch.full((1, hidden), 7.0, dtype=torch.bfloat16, device=DEV)
+    op.contribute(x, ids, wt, stage=0)
+    assert op.finish(x, ids, wt, capi.COMBINE_UNGATED, y)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(y), bits(want))
 
 
 def test_decode_finish_flags_bad_expert_and_declines_unsupported_shapes():
