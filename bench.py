@@ -60,14 +60,21 @@ def parse():
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                     help="also run one plain device copy of this many MiB (a known-size kernel that scales the "
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
+    ap.add_argument("--no-secondary", action="store_true", help="headline run: skip the other configurations (config 3 at 8 and 64 tokens, "
+                    "config 4, config 5) that the default line carries under `secondary`")
     ap.add_argument("--seed", type=int, default=20251)
     return ap.parse_args()
 
 
-def build_layer(args, torch, capi, ops, synth, make_tokens=True):
+def build_layer(args, torch, capi, ops, synth, make_tokens=True, prebuilt=None):
+    """The expert table of --format (seeded weights, quantized on the device) and, for decode, the layer and its token ring.
+    prebuilt = (table, shared) of an earlier call with the same format, experts and seed: the weights are not drawn again."""
     H, I, E, K = 7168, 2048, args.experts, 8
     dev = "cuda"
     nvfp4 = args.format == "nvfp4"
+    if prebuilt is not None:
+        table, shared = prebuilt
+        return (table, None, None, (H, I, E, K)) if not make_tokens else _layer_and_ring(args, torch, capi, ops, synth, table, shared, (H, I, E, K))
     if args.format == "e2m1":  # E2M1 codes with one E8M0 scale per 32 columns (the W4A8 contract); prefill cohorts only
         assert not make_tokens, "--format e2m1 is a prefill workload"
         table = ops.ExpertTable.allocate(capi.FMT_E2M1_E8M0, E, H, I, dev)
@@ -111,8 +118,15 @@ def build_layer(args, torch, capi, ops, synth, make_tokens=True):
         shared = table.shared_struct(E)
         table.experts = E
         table.shared_bytes = table.weight_bytes_per_expert()
+    table.shared_struct_kept = shared
     if not make_tokens:
         return table, None, None, (H, I, E, K)
+    return _layer_and_ring(args, torch, capi, ops, synth, table, shared, (H, I, E, K))
+
+
+def _layer_and_ring(args, torch, capi, ops, synth, table, shared, dims):
+    H, I, E, K = dims
+    dev = "cuda"
     router = synth.normal((E, H), 0.02, args.seed + 1, device=dev, dtype=torch.bfloat16)
     bias = torch.zeros(E, dtype=torch.float32, device=dev)
     layer = ops.NativeMoe(table, shared, router, bias, args.batch, K, routed_scaling=2.5, n_group=8, topk_group=4,
@@ -120,7 +134,7 @@ def build_layer(args, torch, capi, ops, synth, make_tokens=True):
     layer.inline_select = not args.separate_topk
     layer.one_launch = args.one_launch
     xs = [synth.normal((args.batch, H), 1.0, args.seed + 1000 + i, device=dev, dtype=torch.bfloat16) for i in range(args.ring)]
-    return table, layer, xs, (H, I, E, K)
+    return table, layer, xs, dims
 
 
 def layer_bytes(table, distinct, rows, dims):
@@ -161,9 +175,9 @@ def rewarm(torch, step, seconds=0.1):
 def parity_gate_decode(args, torch, capi, ops, table, layer, x, dims):
     """Oracle check of one ring slot, outside the timed region; raises SystemExit when the layer the timing is about to
     measure does not match the CPU restatement: router ids and weights bit for bit, every contribution and the shared
-    row end to end through both stages (relative L2 <= 1e-3 over the tensor; element-wise 16 BF16 steps, the loose bound
-    the test-suite uses where a flipped BF16 step of an activation moves a cancelled down output: the per-stage bars of
-    2 steps are held by tests/test_gpu_fullsize.py on the same shapes), y of
+    row end to end through both stages (relative L2 <= 1e-3 over the tensor; element-wise at most 5e-3 of the elements
+    beyond 2 BF16 steps and none beyond 16, the bound the test-suite uses where a flipped BF16 step of an activation moves
+    a cancelled down output: the per-stage bars of 2 steps are held by tests/test_gpu_fullsize.py on the same shapes), y of
     the timed launch sequence bit-identical to the separate launches and inside the layer bound of the oracle pipeline."""
     np, orc, hp = _checkers()
     H, I, E, K = dims
@@ -210,8 +224,8 @@ def parity_gate_decode(args, torch, capi, ops, table, layer, x, dims):
     want_s = np.stack(res[rows * K:])
     stats = {}
     try:
-        stats["contributions"] = hp.assert_close_bf16(got_c[:rows], want_c, "contributions", max_ulp=16)
-        stats["shared_out"] = hp.assert_close_bf16(got_s[:rows], want_s, "shared expert", max_ulp=16)
+        stats["contributions"] = hp.assert_close_with_rare_outliers(got_c[:rows], want_c, "contributions", loose=16, rare=5e-3)
+        stats["shared_out"] = hp.assert_close_with_rare_outliers(got_s[:rows], want_s, "shared expert", loose=16, rare=5e-3)
     except AssertionError as exc:
         fail.append(str(exc))
     want_y = orc.combine(want_c, want_s, None, oi[:rows], None, orc.COMBINE_UNGATED)
@@ -226,6 +240,7 @@ def parity_gate_decode(args, torch, capi, ops, table, layer, x, dims):
         sys.exit(3)
     return {"checked": "ring slot 0, %d token row(s): ids and weights bit-exact, %d contributions + shared rows, y" % (rows, rows * K),
             "contributions_rel_l2": stats["contributions"][0], "contributions_worst_bf16_steps": stats["contributions"][1],
+            "contributions_share_beyond_2_steps": stats["contributions"][2],
             "y_rel_l2": y_rel, "oracle": "oracle/ffmoe_oracle.cpp (scalar, Lane8 form)"}
 
 
@@ -250,6 +265,7 @@ def parity_gate_prefill(args, torch, capi, ops, table, pre, x, ids, wts, dims, a
         lo, hi = int(offsets[e]), int(offsets[e + 1])
         picks += sorted({lo, (lo + hi) // 2, hi - 1})
     xb = hp.bits(x)
+    xq, sx = (None, None) if a16 else orc.quant_act_fp8_128(xb)
     flat_ids, flat_w = ids.cpu().numpy().reshape(-1), wts.cpu().numpy().reshape(-1)
     act = hp.bits(v["act"][torch.tensor(picks, device="cuda")])
     g2 = hp.bits(got.reshape(pre.rows * K, H)[torch.from_numpy(perm[picks]).cuda().long()])
@@ -262,18 +278,22 @@ def parity_gate_prefill(args, torch, capi, ops, table, pre, x, ids, wts, dims, a
         for i in range(lo, hi):
             a = int(perm[picks[i]])
             m, wa = host[int(flat_ids[a])], float(flat_w[a])
+            t = a // K
             if a16:
-                _, want_act = orc.expert_ffn(xb[a // K], m[0], m[1], m[2], wa, orc.TWICE, 0.0, orc.AFTER_DOWN_BF16, orc.LANE8, orc.SILU_DIV, return_act=True)
+                g_ref, u_ref = orc.linear_skinny(m[0], xb[t:t + 1], 2)[0], orc.linear_skinny(m[1], xb[t:t + 1], 2)[0]
                 d_ref = orc.expert_down(act[i], m[2], 1.0, 0, orc.LANE8, False)
             else:
-                _, want_act = orc.expert_ffn_w8a8(xb[a // K], *m, wa, orc.TWICE, 0.0, orc.AFTER_DOWN_BF16, return_act=True)
+                g_ref = orc.linear_fp8_block_w8a8(m[0], m[1], xq[t:t + 1], sx[t:t + 1])[0]
+                u_ref = orc.linear_fp8_block_w8a8(m[2], m[3], xq[t:t + 1], sx[t:t + 1])[0]
                 d_ref = orc.expert_down_w8a8(act[i], m[4], m[5], apply_weight=False)
-            out.append((want_act, d_ref, wa))
+            out.append((g_ref, u_ref, d_ref, wa))
         return out
     res = [t for chunk in hp.run_parallel(one, len(picks), min(16, len(os.sched_getaffinity(0)))) for t in chunk]
     try:
-        a_stats = hp.assert_close_bf16(act, np.stack([t[0] for t in res]), "activations", max_ulp=3)
-        d_stats = hp.assert_weighted_down_close(g2, np.stack([t[1] for t in res]), [t[2] for t in res], "down stage on the device activations")
+        # activations: within 2 steps of SwiGLU(gate, up) of the oracle, further only where a gate / up one step off explains it
+        a_stats = hp.assert_swiglu_close(act, np.stack([t[0] for t in res]), np.stack([t[1] for t in res]), orc.TWICE, 0.0,
+                                         orc.SILU_DIV if a16 else orc.SILU_SIGMOID2, "activations")
+        d_stats = hp.assert_weighted_down_close(g2, np.stack([t[2] for t in res]), [t[3] for t in res], "down stage on the device activations")
     except AssertionError as exc:
         print("bench.py parity gate FAILED: " + str(exc), file=sys.stderr)
         sys.exit(3)
@@ -331,14 +351,14 @@ MFMA_FP8_PEAK_TFLOPS = 5000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 
 
-def prefill_main(args, torch, capi, ops, synth):
+def prefill_main(args, torch, capi, ops, synth, prebuilt=None):
     """BASELINE config 5: R tokens routed top-8 over 256 experts with Zipf(s=1.1) popularity (seeded router logits =
     log popularity under a seeded expert permutation + Gumbel noise, so the top-8 is a draw without replacement),
     grouped W8A8 GEMMs on the FP8 matrix cores, routed-only ordered combine. A step = top-k selection from the logits
     + prefill contribute + combine on inputs resident in HBM."""
     import math
     R = args.batch
-    table, layer, _, dims = build_layer(args, torch, capi, ops, synth, make_tokens=False)
+    table, layer, _, dims = build_layer(args, torch, capi, ops, synth, make_tokens=False, prebuilt=prebuilt)
     H, I, E, K = dims
     dev = "cuda"
     g = torch.Generator(device="cpu").manual_seed(args.seed + 77)
@@ -435,7 +455,7 @@ def prefill_main(args, torch, capi, ops, synth):
     out["parity"] = parity if parity is not None else ("not gated in bench.py for this format (tests/test_gpu_e8m0.py, tests/test_gpu_fullsize.py)" if mx else None)
     if not args.no_cpu_baseline and args.format == "fp8":
         out["cpu_baseline"] = cpu_baseline_prefill(args, torch, table, x, ids, wts, dims)
-    print(json.dumps(out))
+    return out
 
 
 def cpu_baseline_prefill(args, torch, table, x, ids, wts, dims):
@@ -580,7 +600,7 @@ def c1_main(args, torch, capi, ops, synth):
                         "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": b0 / k0 / 1e3 / HBM_PEAK_GBPS, "traffic": None, "bytes_per_launch": b0,
                         "avg_us": k0, "launches_timed": 128, "note": "the same 4 experts every launch (34 MB: cache-resident), latency-bound"},
            "down_kernel": {"avg_us": k1}, "parity": parity}
-    print(json.dumps(out))
+    return out
 
 
 def linear_main(args, torch, capi, ops, synth):
@@ -640,7 +660,7 @@ def linear_main(args, torch, capi, ops, synth):
            "roofline": {"kernel": "ffmoe::k_linear_mfma<FmtFp8, TR> (more than 4 rows) / ffmoe::k_linear<FmtFp8, S, RG>", "bound": "hbm",
                         "achieved": head["gbps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": head["hbm_frac"], "traffic": None},
            "cases": rows}
-    print(json.dumps(out))
+    return out
 
 
 def widening_main(args, torch, capi, ops, synth):
@@ -729,34 +749,12 @@ def widening_main(args, torch, capi, ops, synth):
                                   "experts (streaming and Lane16 / Lane8 orders), fused combine + residual",
                       "hidden": H, "intermediate": I, "experts_resident": E + 1, "top_k": K, "shared_experts": 1},
            "rows": rows}
-    print(json.dumps(out))
+    return out
 
 
-def main():
-    args = parse()
-    if args.batch is None:
-        args.batch = 1 if args.workload == "decode" else 4096
-    if args.gpus != 1:
-        print("bench.py measures one GPU: this build has no multi-GPU path; "
-              "run with --gpus 1", file=sys.stderr)
-        sys.exit(2)
-    import torch
-    from flyingfish_amd import capi, ops, synth
-    if not torch.cuda.is_available():
-        print("bench.py needs a GPU", file=sys.stderr)
-        sys.exit(1)
-    capi.lib()  # fail loudly when the HIP library is missing
-    if args.workload == "prefill":
-        if args.steps == 200 and args.warmup == 20:
-            args.steps, args.warmup = 10, 2
-        return prefill_main(args, torch, capi, ops, synth)
-    if args.workload == "widening":
-        return widening_main(args, torch, capi, ops, synth)
-    if args.workload == "linear":
-        return linear_main(args, torch, capi, ops, synth)
-    if args.workload == "c1":
-        return c1_main(args, torch, capi, ops, synth)
-    table, layer, xs, dims = build_layer(args, torch, capi, ops, synth)
+def decode_main(args, torch, capi, ops, synth, prebuilt=None):
+    """BASELINE configs 3 and 4: the decode layer at --batch tokens. Returns the line and the table it drew."""
+    table, layer, xs, dims = build_layer(args, torch, capi, ops, synth, prebuilt=prebuilt)
     H, I, E, K = dims
     torch.cuda.synchronize()
 
@@ -767,7 +765,6 @@ def main():
         dst.copy_(src)  # reads and writes exactly calibrate_copy MiB
         torch.cuda.synchronize()
         del src, dst
-
     # distinct experts per ring slot (measured from the ids)
     distinct = []
     for x in xs:
@@ -778,6 +775,11 @@ def main():
     parity = None if args.no_parity_gate else parity_gate_decode(args, torch, capi, ops, table, layer, xs[0], dims)
 
     graphs = None
+    if args.graph and args.one_launch:
+        # the one-launch layer tells its activations from an earlier launch's by a per-launch tag that is a kernel argument:
+        # a captured launch would replay one tag for ever
+        print("bench.py: --graph cannot be combined with --one-launch (ffmoe_decode_token_layer must not be captured)", file=sys.stderr)
+        sys.exit(2)
     if args.graph:
         graphs = []
         side = torch.cuda.Stream()
@@ -904,6 +906,86 @@ def main():
     }
     if not args.no_cpu_baseline and args.format == "fp8":
         out["cpu_baseline"] = cpu_baseline(args, torch, table, layer, xs, dims)
+    return out, table
+
+
+def _brief_decode(out):
+    """The figures of a decode line that the one-line summary of the other configurations keeps."""
+    return {"workload": out["config"]["workload"], "us": out["value"], "steps": out["steps"], "distinct_routed_experts": out["distinct_routed_experts"],
+            "bytes": out["layer_bytes"], "gbps": out["layer_hbm_gbps"], "frac": out["layer_hbm_frac"], "bound": "hbm",
+            "gate_up": {"kernel": out["roofline"]["kernel"], "us": out["roofline"]["avg_us"], "bytes": out["roofline"]["bytes_per_launch"],
+                        "frac": out["roofline"]["frac"]},
+            "down": {"kernel": out["down_kernel"]["kernel"], "us": out["down_kernel"]["avg_us"], "bytes": out["down_kernel"]["bytes_per_launch"],
+                     "frac": out["down_kernel"]["frac"]},
+            "parity": out["parity"]}
+
+
+def secondary(args, torch, capi, ops, synth, fp8_table):
+    """The other configurations the metric names, measured after the headline's timed region in the same process and each
+    behind its own oracle gate: config 3 at 8 and 64 tokens, config 5 (prefill on the FP8 matrix cores, with its CPU
+    baseline sample) on the headline's expert table, config 4 (NVFP4 routed experts + BF16 shared expert) at 32 tokens and
+    one token on a table of its own. Fewer steps than the stand-alone runs of the same workloads (--batch, --format,
+    --workload prefill), the same measurement otherwise."""
+    import copy
+    sec = {}
+    fp8 = (fp8_table, fp8_table.shared_struct_kept)
+    for batch, steps in ((8, 60), (64, 24)):
+        a = copy.copy(args)
+        a.batch, a.ring, a.steps, a.warmup, a.calibrate_copy, a.no_cpu_baseline = batch, 16, steps, 4, 0, True
+        out, _ = decode_main(a, torch, capi, ops, synth, prebuilt=fp8)
+        sec["c3_fp8_batch%d" % batch] = _brief_decode(out)
+    a = copy.copy(args)
+    a.workload, a.batch, a.steps, a.warmup, a.prefill_act = "prefill", 4096, 6, 2, "fp8"
+    out = prefill_main(a, torch, capi, ops, synth, prebuilt=fp8)
+    sec["c5_fp8_prefill_4096"] = {
+        "workload": out["config"]["workload"], "ms": out["value"], "steps": out["steps"], "flop": out["routed_tflop"] * 1e12, "tflops": out["cohort_tflops"],
+        "frac": out["cohort_mfma_frac"], "bound": "mfma", "peak_tflops": MFMA_FP8_PEAK_TFLOPS, "weight_gbps_once": out["cohort_weight_gbps"],
+        "experts_touched": out["config"]["experts_touched"], "max_rows_per_expert": out["config"]["max_rows_per_expert"],
+        "gate_up": {"kernel": out["roofline"]["kernel"], "ms": out["roofline"]["avg_ms"], "flop": out["roofline"]["flop_per_launch"], "frac": out["roofline"]["frac"]},
+        "down": {"kernel": out["down_kernel"]["kernel"], "ms": out["down_kernel"]["avg_ms"], "tflops": out["down_kernel"]["tflops"],
+                 "frac": out["down_kernel"]["tflops"] / MFMA_FP8_PEAK_TFLOPS},
+        "parity": out["parity"], "cpu_baseline": out.get("cpu_baseline")}
+    del out
+    nv = None
+    for batch, steps, ring in ((32, 24, 16), (1, 100, 64)):
+        a = copy.copy(args)
+        a.format, a.batch, a.ring, a.steps, a.warmup, a.calibrate_copy, a.no_cpu_baseline = "nvfp4", batch, ring, steps, 4, 0, True
+        out, t = decode_main(a, torch, capi, ops, synth, prebuilt=nv)
+        nv = (t, t.shared_struct_kept)
+        sec["c4_nvfp4_batch%d" % batch] = _brief_decode(out)
+    return sec
+
+
+def main():
+    args = parse()
+    if args.batch is None:
+        args.batch = 1 if args.workload == "decode" else 4096
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path; "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from flyingfish_amd import capi, ops, synth
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(1)
+    capi.lib()  # fail loudly when the HIP library is missing
+    if args.workload == "prefill":
+        if args.steps == 200 and args.warmup == 20:
+            args.steps, args.warmup = 10, 2
+        out = prefill_main(args, torch, capi, ops, synth)
+    elif args.workload == "widening":
+        out = widening_main(args, torch, capi, ops, synth)
+    elif args.workload == "linear":
+        out = linear_main(args, torch, capi, ops, synth)
+    elif args.workload == "c1":
+        out = c1_main(args, torch, capi, ops, synth)
+    else:
+        out, table = decode_main(args, torch, capi, ops, synth)
+        # the headline line (config 3, one token) also carries the rest of the metric, measured after its own timed region
+        headline = args.format == "fp8" and args.batch == 1 and args.experts == 256 and not (args.one_launch or args.separate_topk or args.graph)
+        if headline and not args.no_secondary:
+            out["secondary"] = secondary(args, torch, capi, ops, synth, table)
     print(json.dumps(out))
 
 

@@ -433,15 +433,21 @@ class PrefillOps:
         """The arena regions a caller may inspect after contribute(): same offsets as prefill_layout() in
         csrc/prefill.hip (every region rounded up to 256 bytes). act[pos] is the BF16 SwiGLU output of the assignment
         perm[pos]; offsets[e]..offsets[e+1] is expert e's segment; totals[3] is the number of live assignments."""
-        t = self.table
-        R, K, E, H, I = self.rows, self.top_k, t.experts, t.hidden, t.inter
+        return PrefillOps.arena_views(self.scratch, self.table, self.rows, self.top_k, self._shared_c)
+
+    @staticmethod
+    def arena_views(scratch, table, rows, top_k, shared):
+        """scratch_views() of any arena a cohort call laid out, e.g. the scratch of a DecodeOps whose batch
+        ffmoe_decode_contribute handed to the cohort kernels."""
+        t = table
+        R, K, E, H, I = rows, top_k, t.experts, t.hidden, t.inter
         A = R * K
         off = 0
         out = {}
 
         def take(name, nbytes, dtype, shape):
             nonlocal off
-            out[name] = self.scratch[off:off + nbytes].view(dtype).view(shape)
+            out[name] = scratch[off:off + nbytes].view(dtype).view(shape)
             off += (nbytes + 255) // 256 * 256
         take("xq", R * H, torch.uint8, (R, H))
         take("sx", R * (H // 128) * 4, torch.float32, (R, H // 128))
@@ -453,8 +459,8 @@ class PrefillOps:
         take("gbase", (E + 1) * 4, torch.int32, (E + 1,))
         take("totals", 16, torch.int32, (4,))
         take("perm", A * 4, torch.int32, (A,))
-        if self._shared_c is not None:
-            SI = self._shared_c.inter
+        if shared is not None:
+            SI = shared.inter
             max_groups = E + (A + 15) // 16 + (R + 15) // 16
             take("groups", max_groups * 16, torch.uint8, (max_groups * 16,))
             take("units0", max_groups * (-(-I // 128)) * 8, torch.uint8, (-1,))

@@ -208,7 +208,10 @@ int ffmoe_decode_contribute(const ffmoe_expert_table* table, const ffmoe_shared_
  * ffmoe_decode_scratch_bytes() exceeds the arena is rejected with FFMOE_ERR_SCRATCH and nothing is launched (at the
  * DeepSeek-V3 dimensions the arena holds up to 128 rows x top-8). The call allocates nothing and clears nothing
  * (no stage reads arena bytes that an earlier launch of the same call has not written). All calls on one GPU share
- * that GPU's array: two calls that overlap in time on one GPU (different streams) race. */
+ * that GPU's array: two calls that overlap in time on one GPU (different streams) race. Under HIP graph capture: make
+ * the first call on each GPU outside capture (it looks the array's address up with hipGetSymbolAddress, which may load
+ * the code object), and note that the environment switches that pick the kernels (FFMOE_DECODE_COHORT_ROWS and the
+ * like) are read when the call is made, i.e. at capture, not at replay. */
 uint64_t ffmoe_decode_static_scratch_bytes(void);
 int ffmoe_decode_contribute_static(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared,
                                    const ffmoe_decode* args, void* stream);
@@ -281,8 +284,11 @@ int ffmoe_decode_contribute_from_logits(const ffmoe_expert_table* table, const f
  * contributions, shared_out and done are not written. Bit 0 of *status is set for
  * a live choice naming an expert that is out of range or not valid (its contribution is skipped), bit 1 if a block
  * gave up waiting for another (y is then not valid; happens only when the grid cannot be resident at once, e.g. two
- * such launches running concurrently on one GPU, each holding part of the CUs). FFMOE_ERR_UNSUPPORTED (nothing
- * launched): rows != 1, a shape outside the kernel's register buffers, or a shared expert of another format; use
+ * such launches running concurrently on one GPU, each holding part of the CUs; FFMOE_TOKEN_SPIN_LIMIT, read at every
+ * call, sets the number of polls a block makes before it gives up, default 100000). Do not capture this call into a
+ * HIP graph: the tag is a kernel argument drawn from a host-side counter at call time, so every replay of a captured
+ * launch would carry the same tag and could take a late word of the replay before for its own. FFMOE_ERR_UNSUPPORTED
+ * (nothing launched): rows != 1, a shape outside the kernel's register buffers, or a shared expert of another format; use
  * the separate calls then. */
 int ffmoe_decode_token_layer(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared, const ffmoe_decode* args,
                              const float* logits, const float* bias, int score_mode, float routed_scaling, int n_group,

@@ -206,6 +206,25 @@ def assert_close_or_explained(got_bits, want_bits, candidates, what, max_ulp=2, 
     return r, float(steps.max())
 
 
+OUTLIER_STATS = []  # (what, relative L2, worst steps, share beyond strict, allowed share, loose) of every call, for the run's summary
+
+
+def assert_close_with_rare_outliers(got_bits, want_bits, what, strict=2, loose=16, rare=1e-3, rel=1e-3):
+    """A bar for values behind TWO composed stages, where the north-star bar holds per stage but an element can move
+    further end to end (a BF16 step of an activation shifts every down output a little, and a cancelled output by several
+    of its own steps): relative L2 <= rel over the tensor, no element beyond `loose` steps, and - what a kernel that is
+    genuinely a step or two worse would fail - at most a fraction `rare` of the elements beyond `strict` steps.
+    Returns (relative L2, worst steps, fraction beyond strict)."""
+    r = orc.rel_l2(got_bits, want_bits)
+    assert r <= rel, "%s: relative L2 %.3e > %.1e" % (what, r, rel)
+    steps = _bf16_steps(got_bits, want_bits)
+    worst, frac = float(steps.max()), float(np.mean(steps > strict))
+    OUTLIER_STATS.append((what, r, worst, frac, rare, loose))
+    assert worst <= loose, "%s: %.2f BF16 steps > %d" % (what, worst, loose)
+    assert frac <= rare, "%s: %.2e of the elements beyond %d steps (allowed %.1e; worst %.1f)" % (what, frac, strict, rare, worst)
+    return r, worst, frac
+
+
 def assert_weighted_down_close(got_bits, down_ref_bits, weights, what, max_ulp=2, rel=1e-3):
     """Routing weight applied after the BF16 cast of the down output: c = bf16(bf16(d) * w), rows [n, H] with one weight
     each. The bar is on d: c must lie within max_ulp steps / rel of bf16(d_ref * w), and an element further away must be

@@ -8,9 +8,15 @@ import torch
 import oracle as orc
 from flyingfish_amd import capi, synth
 from flyingfish_amd.ops import E8m0DecodeOps, ExpertTable, PrefillOps
-from helpers import assert_close_bf16, bits
+from helpers import assert_close_with_rare_outliers, assert_close_bf16, bits
 
 pytestmark = pytest.mark.gpu
+# Values behind two composed stages (end to end) or behind a twice-rounded product (activations of the matrix-core paths):
+# the per-stage bars are 2 steps; here the relative-L2 bar holds on the tensor, no element lies beyond a loose bound, and
+# the share of elements beyond 2 steps must stay below these (small shapes: a cancelled output behind one activation that
+# rounded the other way moves by several of its own steps).
+E2E_RARE = 2e-2
+ACT_RARE = 5e-3
 DEV = "cuda"
 
 
@@ -150,7 +156,7 @@ def test_e8m0_prefill_on_the_mx_matrix_cores(rows, top_k, experts, hidden, inter
         m = ref[int(flat_ids[a])]
         want_full[pos], want_act[pos] = orc.expert_ffn_e8m0(1, xb[a // top_k], *m, limit, float(flat_w[a]), return_act=True)
         want_down[pos] = _down_exact(1, act[pos], m[4], m[5])
-    assert_close_bf16(act, want_act, "activations", max_ulp=3)
+    assert_close_with_rare_outliers(act, want_act, "activations", loose=3, rare=ACT_RARE)
     assert_close_bf16(g2[perm], want_down, "down projection of the device activations")
     assert orc.rel_l2(g2[perm], want_full) <= 5e-2
     assert not g2[np.flatnonzero(active.reshape(-1).numpy() == 0)].any()
@@ -160,7 +166,7 @@ def test_e8m0_prefill_on_the_mx_matrix_cores(rows, top_k, experts, hidden, inter
     for r in range(rows):
         want_sa[r] = orc.expert_ffn_e8m0(0, xb[r], *sh_ref, limit, 1.0, return_act=True)[1]
         want_sd[r] = _down_exact(0, sh_act[r], sh_ref[4], sh_ref[5])
-    assert_close_bf16(sh_act, want_sa, "shared activations", max_ulp=3)
+    assert_close_with_rare_outliers(sh_act, want_sa, "shared activations", loose=3, rare=ACT_RARE)
     assert_close_bf16(so, want_sd, "shared down projection of the device activations")
 
 

@@ -12,12 +12,18 @@ import torch
 
 import oracle as orc
 from flyingfish_amd import capi, ops, synth
-from helpers import assert_close_bf16, assert_swiglu_close, assert_weighted_down_close, bits, effective_weights, host_expert, make_table_on_device, run_parallel
+from helpers import assert_close_bf16, assert_close_with_rare_outliers, assert_swiglu_close, assert_weighted_down_close, bits, effective_weights, host_expert, make_table_on_device, run_parallel
 from test_gpu_prefill import _check_prefill, _routing
 
 pytestmark = pytest.mark.gpu
 H, I = 7168, 2048
 THREADS = 12
+# end to end through both stages on the matrix-core paths: the largest share of elements further than two BF16 steps from
+# the scalar oracle (measured 0 .. 2e-3 at these shapes; cancelled outputs behind activations that rounded the other way)
+E2E_RARE = 5e-3
+# activations of the MX cohort path against the exact oracle's: a twice-rounded product of gate / up values one step off
+# can sit three steps away; such elements must stay rare
+ACT_RARE = 5e-3
 
 
 def test_prefill_w8a8_full_width_every_group_size(monkeypatch):
@@ -132,20 +138,23 @@ def test_prefill_w16_full_width(fmt, monkeypatch):
         for pos in check[lo:hi]:
             a = int(perm[pos])
             ge, ue, de = ref[int(ids.reshape(-1)[a])]
-            want, want_act = orc.expert_ffn(xb[a // top_k], ge, ue, de, float(w.reshape(-1)[a]), mode, limit, boundary, orc.LANE8, orc.SILU_DIV, return_act=True)
-            out.append((pos, a, want, want_act, orc.expert_down(act[pos], de, 1.0, boundary, orc.LANE8, False)))
+            want = orc.expert_ffn(xb[a // top_k], ge, ue, de, float(w.reshape(-1)[a]), mode, limit, boundary, orc.LANE8, orc.SILU_DIV)
+            xr = xb[a // top_k][None, :]
+            out.append((pos, a, want, orc.linear_skinny(ge, xr, 2)[0], orc.linear_skinny(ue, xr, 2)[0], orc.expert_down(act[pos], de, 1.0, boundary, orc.LANE8, False)))
         return out
-    e2e_got, e2e_want, acts, want_acts, downs, wts_ = [], [], [], [], [], []
+    e2e_got, e2e_want, acts, g_refs, u_refs, downs, wts_ = [], [], [], [], [], [], []
     for chunk in run_parallel(one, len(check), THREADS):
-        for pos, a, want, want_act, down_ref in chunk:
-            acts.append(act[pos]); want_acts.append(want_act); downs.append(down_ref); wts_.append(float(w.reshape(-1)[a]))
+        for pos, a, want, g_ref, u_ref, down_ref in chunk:
+            acts.append(act[pos]); g_refs.append(g_ref); u_refs.append(u_ref); downs.append(down_ref); wts_.append(float(w.reshape(-1)[a]))
             e2e_got.append(g2[a]); e2e_want.append(want)
-    assert_close_bf16(np.stack(acts), np.stack(want_acts), "activations", max_ulp=3)
+    # each stage at the bar on its own inputs: activations within 2 steps of SwiGLU(gate, up) from FP64 accumulation, an
+    # element further away only if a gate / up one step off explains it bit for bit
+    assert_swiglu_close(np.stack(acts), np.stack(g_refs), np.stack(u_refs), mode, limit, orc.SILU_DIV, "activations vs SwiGLU of the FP64-accumulated gate / up")
     assert_weighted_down_close(np.stack(e2e_got), np.stack(downs), wts_, "down stage on the device activations")
     # end to end the two stages compose (a flipped BF16 step of an activation moves every down output a little): the
-    # relative-L2 bar on the checked tensor, element-wise a loose bound
-    r_, worst_ = assert_close_bf16(np.stack(e2e_got), np.stack(e2e_want), "contributions, end to end", max_ulp=16)
-    print("end to end: relative L2 %.2e, worst %.1f steps" % (r_, worst_), flush=True)
+    # relative-L2 bar on the checked tensor, few elements beyond two steps, none beyond a loose bound
+    r_, worst_, frac_ = assert_close_with_rare_outliers(np.stack(e2e_got), np.stack(e2e_want), "contributions, end to end", rare=E2E_RARE)
+    print("end to end: relative L2 %.2e, worst %.1f steps, %.2e beyond 2 steps" % (r_, worst_, frac_), flush=True)
     ge, ue, de = ref[experts]
     rows_sh = [0, 15, 16, 63, 64, rows - 1]
 
@@ -202,7 +211,7 @@ def test_prefill_mx_full_width(monkeypatch):
         return out
     for chunk in run_parallel(one, len(check), THREADS):
         for pos, a, full, want_act, want_down in chunk:
-            assert_close_bf16(act[pos][None, :], want_act[None, :], "activations of assignment %d" % a, max_ulp=3)
+            assert_close_with_rare_outliers(act[pos][None, :], want_act[None, :], "activations of assignment %d" % a, loose=3, rare=ACT_RARE)
             assert_close_bf16(g2[a][None, :], want_down[None, :], "down projection of the device activations, assignment %d" % a)
     rows_sh = [0, 33, rows - 1]
 
@@ -210,7 +219,7 @@ def test_prefill_mx_full_width(monkeypatch):
         return [(r, orc.expert_ffn_e8m0(0, xb[r], *sh_ref, limit, 1.0, return_act=True)[1], _down_exact(0, sh_act[r], sh_ref[4], sh_ref[5])) for r in rows_sh[lo:hi]]
     for chunk in run_parallel(shared_rows, len(rows_sh), THREADS):
         for r, want_act, want_down in chunk:
-            assert_close_bf16(sh_act[r][None, :], want_act[None, :], "shared activations row %d" % r, max_ulp=3)
+            assert_close_with_rare_outliers(sh_act[r][None, :], want_act[None, :], "shared activations row %d" % r, loose=3, rare=ACT_RARE)
             assert_close_bf16(so[r][None, :], want_down[None, :], "shared down projection row %d" % r)
     for mf in ("1", "2"):
         monkeypatch.setenv("FFMOE_PREFILL_MF", mf)
@@ -307,9 +316,26 @@ def test_decode_fp8_full_width_beyond_the_lds_row_budget(rows, monkeypatch):
         assert np.array_equal(bits(c2), got_c) and np.array_equal(bits(s2), got_s), "small batches stay on the streaming kernels"
     # on the matrix cores the two stages compose as in test_prefill_w16_full_width (each stage inside its bar there): the
     # relative-L2 bar on the tensor, element-wise a loose bound for cancelled outputs
-    loose = 16 if rows >= 4 else 4
-    assert_close_bf16(bits(c2), want_c, "contributions of the default dispatch vs the CPU port, end to end", max_ulp=loose)
-    assert_close_bf16(bits(s2), want_s, "shared_out of the default dispatch vs the CPU port, end to end", max_ulp=loose)
+    if rows >= 4:
+        # stage by stage as above: the cohort launches leave their activations in the prefill arena
+        v = ops.PrefillOps.arena_views(op.scratch, table, rows, top_k, sh)
+        perm2 = v["perm"].cpu().numpy()[:A]
+        act2 = np.empty((A + rows, I), dtype=np.uint16)
+        act2[perm2] = bits(v["act"])[:A]
+        act2[A:] = bits(v["sh_act"])
+        assert_swiglu_close(act2, np.stack([t[0] for t in res]), np.stack([t[1] for t in res]), orc.TWICE, 0.0, orc.SILU_DIV,
+                            "cohort path: activations vs SwiGLU of the FP64-accumulated gate / up")
+
+        def downs(lo, hi):
+            return [orc.expert_down(act2[r * top_k + c if c >= 0 else A + r], eff[int(ids[r, c])][2] if c >= 0 else eff[experts][2], 1.0, 0, orc.LANE8, False)
+                    for r, c in jobs[lo:hi]]
+        d2 = np.stack([t for chunk in run_parallel(downs, len(jobs), THREADS) for t in chunk])
+        assert_weighted_down_close(bits(c2).reshape(A, -1), d2[:A], wt.numpy().reshape(-1), "cohort path: down stage on the device activations")
+        assert_close_bf16(bits(s2), d2[A:], "cohort path: shared down stage on the device activations")
+    for name, got_, want_ in (("contributions", bits(c2), want_c), ("shared_out", bits(s2), want_s)):
+        r_, worst_, frac_ = assert_close_with_rare_outliers(got_, want_, name + " of the default dispatch vs the CPU port, end to end",
+                                                            loose=16 if rows >= 4 else 4, rare=E2E_RARE)
+        print("default dispatch, %s end to end: relative L2 %.2e, worst %.1f steps, %.2e beyond 2 steps" % (name, r_, worst_, frac_), flush=True)
 
 
 def test_decode_nvfp4_full_width_batched():
@@ -347,7 +373,7 @@ def test_decode_nvfp4_full_width_batched():
     # shared expert on the streaming kernels
     for (r, c), want in zip(jobs, res):
         if c >= 0:
-            assert_close_bf16(got[r, c][None, :], want[None, :], "contribution (%d, %d)" % (r, c), max_ulp=16)
+            assert_close_with_rare_outliers(got[r, c][None, :], want[None, :], "contribution (%d, %d)" % (r, c), rare=E2E_RARE)
         else:
             assert_close_bf16(got_s[r][None, :], want[None, :], "shared_out row %d" % r)
 
@@ -437,9 +463,9 @@ def test_decode_fp8_full_width_64_rows_on_the_cohort_path(monkeypatch):
     want_c, want_s, _ = _cpubase_contributions(table, bits(x), ids.numpy(), wt.numpy(), experts, orc.AFTER_DOWN_BF16)
     # the stages of this path are held to their bars in test_prefill_w16_full_width; end to end the relative-L2 bar on the
     # tensor and a loose element-wise bound for cancelled outputs, as there
-    r_, worst_ = assert_close_bf16(got_c, want_c, "contributions vs the CPU port, end to end", max_ulp=16)
-    print("contributions end to end: relative L2 %.2e, worst %.1f steps" % (r_, worst_), flush=True)
-    assert_close_bf16(got_s, want_s, "shared_out vs the CPU port, end to end", max_ulp=16)
+    r_, worst_, frac_ = assert_close_with_rare_outliers(got_c, want_c, "contributions vs the CPU port, end to end", rare=E2E_RARE)
+    print("contributions end to end: relative L2 %.2e, worst %.1f steps, %.2e beyond 2 steps" % (r_, worst_, frac_), flush=True)
+    assert_close_with_rare_outliers(got_s, want_s, "shared_out vs the CPU port, end to end", rare=E2E_RARE)
     part = ops.DecodeOps(table, sh, 48, top_k, capi.ACT_BF16, capi.SWIGLU_TWICE, 0.0, capi.WEIGHT_AFTER_DOWN_BF16, weights_f32=True)
     c2, s2 = part.contribute(x[8:56].contiguous().cuda(), ids[8:56].contiguous().cuda(), wt[8:56].contiguous().cuda())
     torch.cuda.synchronize()
@@ -449,5 +475,82 @@ def test_decode_fp8_full_width_64_rows_on_the_cohort_path(monkeypatch):
     monkeypatch.setenv("FFMOE_DECODE_SHARED_COHORT_ROWS", "0")
     c3, s3 = op.contribute(x.cuda(), ids.cuda(), wt.cuda())
     torch.cuda.synchronize()
-    assert_close_bf16(bits(c3), want_c, "streaming kernels vs the CPU port, end to end", max_ulp=16)
-    assert_close_bf16(bits(s3), want_s, "streaming kernels, shared_out", max_ulp=16)
+    assert_close_with_rare_outliers(bits(c3), want_c, "streaming kernels vs the CPU port, end to end", loose=4, rare=E2E_RARE)
+    assert_close_with_rare_outliers(bits(s3), want_s, "streaming kernels, shared_out", loose=4, rare=E2E_RARE)
+
+
+def test_prefill_c5_full_scale_bookkeeping_and_sampled_assignments():
+    """BASELINE config 5 at its real size: 4096 tokens x top-8 over 256 experts with Zipf(s = 1.1) popularity - 32,768
+    assignments through the multi-block count / plan / unit-list / stable-fill launches and both grouped GEMMs. The
+    bookkeeping is checked exactly (every assignment once, inside its expert's segment, ascending within it - the
+    invariants of kernels/moe_prefill.cu:495-499 and src/backend/cuda/moe/prefill_tests.rs:652-700 - counts, offsets,
+    totals, every done flag set once); 16 assignments at the start, middle and end of the segments of the most popular,
+    mid-popular and least popular experts are checked stage by stage against the oracle. Only the six experts those
+    assignments hit are materialised (44 MB each); every other slot points at a spare expert, so all 32,768 rows still
+    stream real weights."""
+    E, K, R = 256, 8, 4096
+    rng = np.random.default_rng(20251)
+    pop = np.empty(E)
+    pop[rng.permutation(E)] = np.arange(1, E + 1, dtype=np.float64) ** -1.1
+    logits = np.log(pop)[None, :] - np.log(-np.log(rng.uniform(1e-12, 1.0 - 1e-12, size=(R, E))))   # Gumbel: a draw without replacement
+    ids = np.argsort(-logits, axis=1, kind="stable")[:, :K].astype(np.int32)
+    w = rng.uniform(0.05, 1.0, size=(R, K)).astype(np.float32)
+    counts = np.bincount(ids.reshape(-1), minlength=E)
+    order = np.argsort(-counts, kind="stable")
+    live = [int(e) for e in order if counts[e] > 0]
+    assert counts.max() > 2000 and counts.min() < 64 and len(live) >= 250, (counts.max(), counts.min(), len(live))
+    hit = [live[0], live[1], live[len(live) // 2], live[len(live) // 2 + 1], live[-2], live[-1]]
+    table, store, _ = _sparse_c3_table(hit, 151)
+    host = {e: host_expert(store, i) for i, e in enumerate(hit)}
+    x = synth.normal((R, H), 1.0, 152, dtype=torch.bfloat16)
+    op = ops.PrefillOps(table, R, K, swiglu=capi.SWIGLU_TWICE, weights_f32=True)
+    print("C5 full scale: %d assignments, rows per expert max %d min %d, %d experts touched" % (R * K, counts.max(), counts.min(), len(live)), flush=True)
+    got = op.contribute(x.cuda(), torch.from_numpy(ids).cuda(), torch.from_numpy(w).cuda())
+    torch.cuda.synchronize()
+    # bookkeeping, exactly
+    v = op.scratch_views()
+    A = R * K
+    assert v["totals"].cpu().numpy()[3] == A
+    assert np.array_equal(v["counts"].cpu().numpy(), counts)
+    offsets = v["offsets"].cpu().numpy()
+    assert np.array_equal(offsets, np.concatenate([[0], np.cumsum(counts)]))
+    perm = v["perm"].cpu().numpy()[:A]
+    assert np.array_equal(np.sort(perm), np.arange(A)), "every assignment exactly once"
+    flat_ids = ids.reshape(-1)
+    assert np.array_equal(flat_ids[perm], np.repeat(np.arange(E), counts)), "every position inside its expert's segment"
+    inner = np.ones(A, dtype=bool)
+    inner[offsets[1:-1][offsets[1:-1] < A]] = False
+    inner[0] = False
+    assert np.all((np.diff(perm) > 0)[inner[1:]]), "ascending assignment index within a segment"
+    assert np.array_equal(op.done.cpu().numpy(), np.ones((R, K), dtype=np.int32)), "done set once per assignment"
+    # sampled assignments, stage by stage
+    picks = []
+    for e in hit:
+        lo, hi = int(offsets[e]), int(offsets[e + 1])
+        picks += sorted({lo, (lo + hi) // 2, hi - 1})
+    picks = picks[:16]
+    xb = bits(x)
+    xq, sx = orc.quant_act_fp8_128(xb)
+    assert np.array_equal(v["xq"].cpu().numpy(), xq) and np.array_equal(v["sx"].cpu().numpy().view(np.uint32), sx.view(np.uint32)), "activation quantizer"
+    act = bits(v["act"][torch.tensor(picks, device="cuda")])
+    g2 = bits(got.reshape(A, H)[torch.from_numpy(perm[picks]).cuda().long()])
+    flat_w = w.reshape(-1)
+
+    def one(lo, hi):
+        out = []
+        for i in range(lo, hi):
+            a = int(perm[picks[i]])
+            m, t = host[int(flat_ids[a])], a // K
+            out.append((orc.linear_fp8_block_w8a8(m[0], m[1], xq[t:t + 1], sx[t:t + 1])[0], orc.linear_fp8_block_w8a8(m[2], m[3], xq[t:t + 1], sx[t:t + 1])[0],
+                        orc.expert_down_w8a8(act[i], m[4], m[5], apply_weight=False), float(flat_w[a])))
+        return out
+    res = [t for chunk in run_parallel(one, len(picks), THREADS) for t in chunk]
+    assert_swiglu_close(act, np.stack([t[0] for t in res]), np.stack([t[1] for t in res]), orc.TWICE, 0.0, orc.SILU_SIGMOID2,
+                        "activations of the sampled assignments")
+    assert_weighted_down_close(g2, np.stack([t[2] for t in res]), [t[3] for t in res], "down stage of the sampled assignments on the device activations")
+    # a second cohort through the same arena after clearing done: same bits (nothing in the arena has to start at zero)
+    first = bits(got.reshape(A, H)[torch.from_numpy(perm[picks]).cuda().long()]).copy()
+    op.done.zero_()
+    again = op.contribute(x.cuda(), torch.from_numpy(ids).cuda(), torch.from_numpy(w).cuda())
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(again.reshape(A, H)[torch.from_numpy(perm[picks]).cuda().long()]), first)

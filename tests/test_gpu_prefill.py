@@ -11,9 +11,15 @@ import torch
 
 import oracle as orc
 from flyingfish_amd import capi, ops, synth
-from helpers import assert_close_bf16, assert_weighted_down_close, bf16_tensor, bits
+from helpers import assert_close_with_rare_outliers, assert_swiglu_close, assert_close_bf16, assert_weighted_down_close, bf16_tensor, bits
 
 pytestmark = pytest.mark.gpu
+# Values behind two composed stages (end to end) or behind a twice-rounded product (activations of the matrix-core paths):
+# the per-stage bars are 2 steps; here the relative-L2 bar holds on the tensor, no element lies beyond a loose bound, and
+# the share of elements beyond 2 steps must stay below these (small shapes: a cancelled output behind one activation that
+# rounded the other way moves by several of its own steps).
+E2E_RARE = 2e-2
+ACT_RARE = 5e-3
 
 
 def _fp8_matrix(n, k, seed, std=0.02):
@@ -155,14 +161,19 @@ def _check_prefill(op, host, x_bits, ids, w, swiglu, limit, boundary, live, got,
             g, sg, u, su, d, sd = host[int(flat_ids[a])]
             wa = float(w.reshape(-1)[a])
             full, oact = orc.expert_ffn_w8a8(x_bits[a // top_k], g, sg, u, su, d, sd, wa, swiglu, limit, boundary, return_act=True)
-            out.append((orc.expert_down_w8a8(act[p_], d, sd, wa, boundary), full, oact, orc.expert_down_w8a8(act[p_], d, sd, apply_weight=False), wa))
+            t_ = a // top_k
+            out.append((orc.expert_down_w8a8(act[p_], d, sd, wa, boundary), full, oact, orc.expert_down_w8a8(act[p_], d, sd, apply_weight=False), wa,
+                        orc.linear_fp8_block_w8a8(g, sg, xq_o[t_:t_ + 1], sx_o[t_:t_ + 1])[0], orc.linear_fp8_block_w8a8(u, su, xq_o[t_:t_ + 1], sx_o[t_:t_ + 1])[0]))
         return out
     res = [t for chunk in run_parallel(down_and_full, len(checked), threads) for t in chunk]
     want_down = np.stack([t[0] for t in res])
     want_full = np.stack([t[1] for t in res])
     want_act = np.stack([t[2] for t in res])
     a_idx = perm[checked]
-    assert_close_bf16(act[checked], want_act, "prefill activations", max_ulp=3)
+    # activations against the oracle's: within 2 steps, an element further away only if it is bit for bit the SwiGLU of a
+    # gate and an up value one step from the oracle's (which the gate / up bar allows) - and such elements are rare
+    assert np.array_equal(want_act, orc.silu_mul(np.stack([t[5] for t in res]), np.stack([t[6] for t in res]), swiglu, limit, kind))
+    assert_swiglu_close(act[checked], np.stack([t[5] for t in res]), np.stack([t[6] for t in res]), swiglu, limit, kind, "prefill activations")
     if boundary == orc.AFTER_DOWN_BF16:
         assert_weighted_down_close(g2[a_idx], np.stack([t[3] for t in res]), [t[4] for t in res], "prefill contributions from the device activations")
     else:
@@ -288,7 +299,7 @@ def _check_prefill_w16(fmt, rows, top_k, experts, hidden, inter, skew, shared, m
         want_full[a] = want
     # end to end the two stages compose (a flipped BF16 step of an activation moves a cancelled down output by several of
     # its own steps at these widths): the relative-L2 bar on the whole tensor, element-wise a loose bound
-    assert_close_bf16(g2[perm], want_full[perm], "contributions, end to end", max_ulp=16)
+    assert_close_with_rare_outliers(g2[perm], want_full[perm], "contributions, end to end", rare=E2E_RARE)
     dead = np.flatnonzero(active.reshape(-1) == 0)
     assert not g2[dead].any()
     if shared:
@@ -301,7 +312,7 @@ def _check_prefill_w16(fmt, rows, top_k, experts, hidden, inter, skew, shared, m
             assert_close_bf16(sh_act[r][None, :], want_act[None, :], "shared activations row %d" % r)
             assert_close_bf16(so[r][None, :], orc.expert_down(sh_act[r], de, 1.0, 0, orc.LANE8, False)[None, :], "shared down row %d" % r)
             want_sh[r] = want
-        assert_close_bf16(so, want_sh, "shared_out, end to end", max_ulp=16)
+        assert_close_with_rare_outliers(so, want_sh, "shared_out, end to end", rare=E2E_RARE)
 
 
 def test_prefill_skips_inactive_invalid_and_out_of_range():
@@ -490,7 +501,7 @@ def test_prefill_bf16_shared_expert_on_the_split_contraction_kernel(rows, hidden
         assert_close_bf16(sh_act[r][None, :], want_act[None, :], "shared activations row %d" % r)
         assert_close_bf16(so[r][None, :], orc.expert_down(sh_act[r], de, 1.0, 0, orc.LANE8, False)[None, :], "shared down row %d" % r)
         want_sh[r] = want
-    assert_close_bf16(so, want_sh, "shared_out, end to end", max_ulp=16)
+    assert_close_with_rare_outliers(so, want_sh, "shared_out, end to end", rare=E2E_RARE)
     # (the two kernels' FP32 sums differ in order only, which moves a BF16 result about once in 2^15 elements: no bitwise
     # difference can be demanded of shapes this small)
     assert_close_bf16(sh_act, out["0"][2], "shared activations against the grouped kernels", max_ulp=4)
@@ -578,9 +589,9 @@ def test_decode_nvfp4_cohort_with_a_bf16_shared_expert(rows, shared_inter, monke
     torch.cuda.synchronize()
     assert np.array_equal(got_c, bits(want)), "routed choices: the cohort kernels' bits"
     # and inside the end-to-end bar of the matrix-core path against the streaming kernels
-    assert_close_bf16(got_c.reshape(rows * top_k, hidden), str_c.reshape(rows * top_k, hidden), "cohort vs streaming contributions", max_ulp=16)
+    assert_close_with_rare_outliers(got_c.reshape(rows * top_k, hidden), str_c.reshape(rows * top_k, hidden), "cohort vs streaming contributions", rare=E2E_RARE)
     # the BF16 shared expert (hidden and width multiples of 256): blocks that split the contraction at every cohort size
-    assert_close_bf16(got_s, str_s, "shared expert on the matrix cores vs streaming", max_ulp=16)
+    assert_close_with_rare_outliers(got_s, str_s, "shared expert on the matrix cores vs streaming", rare=E2E_RARE)
     # without that kernel it stays on the streaming kernels up to 24 rows (their bits) and moves to the grouped kernels beyond
     monkeypatch.setenv("FFMOE_SHARED_SPLITK", "0")
     _, old_s = run(False)
@@ -588,7 +599,7 @@ def test_decode_nvfp4_cohort_with_a_bf16_shared_expert(rows, shared_inter, monke
     if rows <= 24:
         assert np.array_equal(old_s, str_s), "shared expert: the streaming kernels' bits"
     else:
-        assert_close_bf16(old_s, str_s, "shared expert on the grouped kernels vs streaming", max_ulp=16)
+        assert_close_with_rare_outliers(old_s, str_s, "shared expert on the grouped kernels vs streaming", rare=E2E_RARE)
 
 
 @pytest.mark.parametrize("rows,top_k,experts", [(1, 1, 3), (37, 4, 9), (128, 8, 70), (341, 3, 5)])
@@ -673,7 +684,7 @@ def test_prefill_shared_expert(rows):
     g, sg, u, su, d, sd = host[experts]
     want = _oracle_shared_w8a8(host[experts], bits(x), orc.TWICE, 0.0)
     want_act = np.stack([a for _, a in want])
-    assert_close_bf16(sh_act, want_act, "shared activations", max_ulp=3)
+    assert_close_with_rare_outliers(sh_act, want_act, "shared activations", loose=3, rare=ACT_RARE)
     want_out = np.stack([orc.expert_down_w8a8(sh_act[r], d, sd, apply_weight=False) for r in range(rows)])
     assert_close_bf16(bits(op.shared_out), want_out, "shared_out from the device activations")
 

@@ -220,3 +220,45 @@ def test_token_layer_graph_replay_equals_eager():
         torch.cuda.synchronize()
         assert np.array_equal(bits(layer.y), eager[it % 3]), "replay %d" % it
     assert int(layer.status.item()) == 0
+
+
+def test_token_layer_bounded_wait_gives_up_and_the_next_launch_recovers(monkeypatch):
+    """The grid-wide hand-over of the one-launch layer is a bounded wait: with FFMOE_TOKEN_SPIN_LIMIT=0 (read at every call) a
+    block that finds activations of other blocks missing on its first look gives up, sets bit 1 of the status word and
+    still leaves the kernel; the last block out hands the arena and the claim counters back clean. Whether any block has
+    to give up is a matter of timing, so both outcomes are accepted for the forced call - status 0 with the right y, or
+    status 2 - and the launches that follow (default limit, same arena, same stream) must give the separate launches' bits."""
+    experts, hidden, inter, top_k, seed = 12, 2048, 1024, 8, 211
+    table, _ = make_table(capi.FMT_FP8_BLOCK128, experts + 1, hidden, inter, seed)
+    sh = table.shared_struct(experts)
+    table.experts = experts
+    op = DecodeOps(table, sh, 1, top_k, capi.ACT_BF16, capi.SWIGLU_TWICE, 0.0, capi.WEIGHT_AFTER_DOWN_BF16, True)
+    g = synth.generator(seed + 1)
+    gave_up = 0
+    for trial in range(6):
+        x = rand_bf16((1, hidden), 1.0, seed + 10 + trial).to(DEV)
+        ids = torch.randperm(experts, generator=g)[:top_k].to(torch.int32).view(1, top_k).to(DEV)
+        wt = (torch.rand((1, top_k), generator=g) * 0.5 + 0.05).to(DEV)
+        op.done.zero_()
+        contrib, shared_out = op.contribute(x, ids, wt)
+        want = bits(CombineOps.combine(contrib, shared_out, ids, capi.COMBINE_UNGATED, done=op.done)).copy()
+        y = torch.full((1, hidden), 7.0, dtype=torch.bfloat16, device=DEV)
+        status = torch.zeros(1, dtype=torch.int32, device=DEV)
+        monkeypatch.setenv("FFMOE_TOKEN_SPIN_LIMIT", "0")
+        print("one-launch layer, spin limit 0, trial %d" % trial, flush=True)
+        assert op.token_layer(x, ids, wt, capi.COMBINE_UNGATED, y, status=status)
+        torch.cuda.synchronize()
+        st = int(status.item())
+        assert st in (0, 2), st
+        if st == 0:
+            assert np.array_equal(bits(y), want), "no block gave up, so y must be right"
+        gave_up += st == 2
+        monkeypatch.delenv("FFMOE_TOKEN_SPIN_LIMIT")
+        for again in range(2):
+            y.fill_(7.0)
+            status.zero_()
+            assert op.token_layer(x, ids, wt, capi.COMBINE_UNGATED, y, status=status)
+            torch.cuda.synchronize()
+            assert int(status.item()) == 0
+            assert np.array_equal(bits(y), want), "launch %d after a forced give-up" % again
+    print("forced give-ups: %d of 6 launches" % gave_up, flush=True)

@@ -82,3 +82,42 @@ def test_static_scratch_rejects_oversize_and_reports_its_size():
     assert rc == capi.ERR_SCRATCH and "built-in arena" in capi.last_error()
     torch.cuda.synchronize()
     assert bool((contrib == 7.0).all()), "a rejected call must not launch anything"
+
+
+@pytest.mark.parametrize("rows,top_k", [(1, 4), (9, 3)])
+def test_static_scratch_call_replays_from_a_hip_graph(rows, top_k):
+    """The caller this entry point is for: one ffmoe_decode_contribute_static call captured into a HIP graph (after a first
+    call outside capture, which looks the array's address up) and replayed with new inputs in the same buffers. Every
+    replay, with eager work and synchronisations in between, must give the eager ffmoe_decode_contribute bits."""
+    experts, hidden, inter = 8, 1024, 512
+    table, _ = make_table(capi.FMT_FP8_BLOCK128, experts + 1, hidden, inter, 981)
+    sh = table.shared_struct(experts)
+    table.experts = experts
+    g = synth.generator(982)
+    x = synth.normal((rows, hidden), 1.0, 983).to(torch.bfloat16).to(DEV)
+    ids = torch.stack([torch.randperm(experts, generator=g)[:top_k] for _ in range(rows)]).to(torch.int32).to(DEV)
+    wt = (torch.rand((rows, top_k), generator=g) * 0.5 + 0.05).to(DEV)
+    eager = DecodeOps(table, sh, rows, top_k, capi.ACT_BF16, capi.SWIGLU_TWICE, 0.0, capi.WEIGHT_AFTER_DOWN_BF16, weights_f32=True)
+    op = DecodeOps(table, sh, rows, top_k, capi.ACT_BF16, capi.SWIGLU_TWICE, 0.0, capi.WEIGHT_AFTER_DOWN_BF16, weights_f32=True)
+    op.contribute_static(x, ids, wt)   # first call on this GPU outside capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    print("capturing ffmoe_decode_contribute_static rows=%d top_k=%d" % (rows, top_k), flush=True)
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            op.contribute_static(x, ids, wt)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    for replay in range(4):
+        x.copy_(synth.normal((rows, hidden), 1.0, 990 + replay).to(torch.bfloat16))
+        ids.copy_(torch.stack([torch.randperm(experts, generator=g)[:top_k] for _ in range(rows)]).to(torch.int32))
+        op.contributions.zero_(); op.shared_out.zero_(); op.done.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        c, s = eager.contribute(x, ids, wt)
+        torch.cuda.synchronize()
+        assert np.array_equal(bits(op.contributions), bits(c)) and np.array_equal(bits(op.shared_out), bits(s)), "replay %d" % replay
+        assert bool((op.done != 0).all())
