@@ -15,8 +15,8 @@ pytestmark = pytest.mark.gpu
 # the per-stage bars are 2 steps; here the relative-L2 bar holds on the tensor, no element lies beyond a loose bound, and
 # the share of elements beyond 2 steps must stay below these (small shapes: a cancelled output behind one activation that
 # rounded the other way moves by several of its own steps).
-E2E_RARE = 2e-2
-ACT_RARE = 5e-3
+E2E_RARE = 5e-3
+ACT_RARE = 2e-3
 DEV = "cuda"
 
 
