@@ -828,11 +828,14 @@ def decode_main(args, torch, capi, ops, synth, prebuilt=None):
     bias1 = layer.bias if layer.bias.dim() == 1 else layer.bias[0]
 
     def launch(stage, s_):
+        # the second launch alone would not be the launch the layer issues (one token: it starts from the record of the live
+        # choices that the gate/up launch of the same call leaves; batches: from that call's grouping): time both launches
+        # and subtract the first
         if token_path:
             ok = dec.token_forward(xs[s_], layer.ids, layer.weights, layer.combine_mode, layer.y, routed[s_][2], bias=bias1, status=layer.status,
-                                   routed_scaling=2.5, n_group=8, topk_group=4, stage=stage)
+                                   routed_scaling=2.5, n_group=8, topk_group=4, stage=0 if stage == 0 else None)
             assert ok
-        else:  # stage 1 alone would reuse the previous launch's grouping: time both launches and subtract
+        else:
             dec.contribute(xs[s_], routed[s_][0], routed[s_][1], stage=0 if stage == 0 else None)
 
     def time_stage(stage):
@@ -861,8 +864,7 @@ def decode_main(args, torch, capi, ops, synth, prebuilt=None):
     achieved = k_bytes / (k_avg * 1e-6) / 1e9
     # second streaming launch: down (+ routing weight; one token: + ordered combine)
     dt, _ = time_stage(1)
-    if not token_path:
-        dt = sorted(max(t - k_avg, 0.0) for t in dt)
+    dt = sorted(max(t - k_avg, 0.0) for t in dt)
     d_avg = sum(dt) / len(dt)
     d_bytes = (mean_distinct_k * table.weight_bytes_per_expert() + table.shared_bytes) // 3 + args.batch * (K + 1) * I * 2 + \
         (args.batch * H * 2 if token_path else args.batch * (K + 1) * H * 2) - (shared_down - 2 * H * 2 if mixed_token else 0)  # mixed: the finish reads the shared row instead of a down matrix

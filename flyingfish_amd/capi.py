@@ -6,7 +6,8 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libffmoe.so")
+# FFMOE_LIBRARY names another build of the same library (A/B measurements of two builds in one session)
+LIB_PATH = os.environ.get("FFMOE_LIBRARY") or os.path.join(_HERE, "libffmoe.so")
 
 # enums of include/ffmoe.h
 FMT_FP8_BLOCK128, FMT_NVFP4, FMT_BF16, FMT_FP8_CHANNEL, FMT_E2M1_E8M0, FMT_E4M3_E8M0_32 = 0, 1, 2, 3, 4, 5

@@ -16,6 +16,19 @@ struct GroupDesc {
   int pad[2];
 };
 
+// What the one-token finish needs to know about the live choices, in combine order, resolved by the gate/up launch that
+// selected them (block 0, right behind the selection): the finish then starts from one load of this record instead of the
+// chain ids -> slot table, and ranks nothing.
+#define FFMOE_FINISH_ROUTED 8
+struct FinishDesc {
+  int n;       // live routed groups
+  int bad;     // 1: a selected expert is out of range or not valid (the finish reports it in its status word)
+  int pad[2];
+  uint64_t codes[FFMOE_FINISH_ROUTED], scales[FFMOE_FINISH_ROUTED];  // down matrix of group g
+  float glob[FFMOE_FINISH_ROUTED], wk[FFMOE_FINISH_ROUTED];          // its global scale (NVFP4) and routing weight
+  int slot[FFMOE_FINISH_ROUTED];                                     // its choice index = activation row
+};
+
 // Top-k selection inside the gate/up kernel (one token row): every block selects from the FP32 logits in its prologue,
 // block 0 publishes ids and weights for the later launches. logits == NULL: ids and weights are inputs.
 struct RouteInline {
@@ -24,6 +37,8 @@ struct RouteInline {
   int score_mode, n_group, topk_group;
   float routed_scaling;
   int select_k;         // choices to select; 0: the launch's own top_k (a shared-expert-only launch has top_k = 0)
+  FinishDesc* finish_desc;  // block 0 also resolves the live choices for the finish launch of the same call, or NULL
+  int finish_ordered;       // their order: 1 ascending expert id (stable), 0 choice order (the accumulate combine modes)
 };
 
 struct DecodeParams {
@@ -58,6 +73,7 @@ struct FinishParams {
   uint16_t* y;            // [hidden]
   uint32_t* status;       // |= 1 when a live choice names an expert that is out of range or not valid
   int mode;               // FFMOE_COMBINE_*
+  const FinishDesc* desc;  // the live choices as the gate/up launch of the same call resolved them, or NULL: from ids
   const uint16_t* shared_ready;  // [hidden] BF16 output of a shared expert that other launches computed (another format or
                                  // width than the table's), or NULL: the finish computes d.has_shared's expert itself
   // the whole token layer in one launch (k_token_layer)

@@ -160,7 +160,8 @@ extern "C" __attribute__((visibility("default"))) uint64_t ffmoe_decode_scratch_
 // (both gate/up launches, then both down launches), so neither may overwrite the other's grouping.
 static int decode_impl(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared, const ffmoe_decode* args,
                        int stage_mask, void* stream, int layout_k = -1, int pass = 0, const FinishParams* fin = nullptr,
-                       const RouteInline* route = nullptr, int form = -1, int arena_shared_inter = 0, bool mixed_gate_up = false) {
+                       const RouteInline* route = nullptr, int form = -1, int arena_shared_inter = 0, bool mixed_gate_up = false,
+                       bool finish_record = false) {
   FF_REQUIRE(table && args, FFMOE_ERR_NULL, "table/args is NULL");
   const int R = args->rows, K = args->top_k, E = table->experts, H = table->hidden, I = table->inter;
   const int LK = layout_k < 0 ? K : layout_k;
@@ -288,10 +289,15 @@ static int decode_impl(const ffmoe_expert_table* table, const ffmoe_shared_exper
   } else {
     p.groups = nullptr;
     p.counters = nullptr;
+    // one row: the group tables are unused, and the gate/up launch with the selection in its prologue leaves the record
+    // of the live choices there for the finish launch of the same call
+    if (finish_record) p.route.finish_desc = (FinishDesc*)(sc + hbytes);
   }
   if (fin) {
     FinishParams q = *fin;
     q.d = p;
+    q.d.route.finish_desc = nullptr;
+    q.desc = finish_record && rg == 1 ? (const FinishDesc*)(sc + hbytes) : nullptr;
     if (q.whole) {
       if (!token_layer_sync(&q)) return ff_fail(FFMOE_ERR_UNSUPPORTED, "one-launch token layer: no device counters on this device");
       q.h32 = (uint32_t*)sc;
@@ -613,8 +619,14 @@ static int token_forward(const ffmoe_expert_table* table, const ffmoe_shared_exp
     }
     return 0;
   }
-  if (stage_mask & 1) FF_TRY(decode_impl(table, sh, args, 1, stream, -1, 0, nullptr, &route));
-  if (stage_mask & 2) FF_TRY(decode_impl(table, sh, args, 0, stream, -1, 0, &fin));
+  // both launches in one call: block 0 of the gate/up launch resolves the live choices (combine order, down matrices,
+  // routing weights) for the finish, which then starts from that record instead of the chain ids -> slot table. A stage
+  // issued alone works from ids and weights in memory, as ffmoe_decode_finish does.
+  const bool record = stage_mask == 3 && K <= FFMOE_FINISH_ROUTED;
+  RouteInline route_rec = route;
+  route_rec.finish_ordered = !(combine_mode == FFMOE_COMBINE_ACCUM_FP32 || combine_mode == FFMOE_COMBINE_ACCUM_BF16);
+  if (stage_mask & 1) FF_TRY(decode_impl(table, sh, args, 1, stream, -1, 0, nullptr, &route_rec, -1, 0, false, record));
+  if (stage_mask & 2) FF_TRY(decode_impl(table, sh, args, 0, stream, -1, 0, &fin, nullptr, -1, 0, false, record));
   return 0;
 }
 

@@ -278,6 +278,31 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
         reinterpret_cast<float*>(const_cast<void*>(p.weights))[tid] = s_route_w[tid];
         if (p.done) p.done[tid] = 0u;
       }
+      // the finish launch of the same call: live choices in combine order with their down matrices resolved
+      if (blockIdx.x == 0 && p.route.finish_desc && tid < 64) {
+        FinishDesc* fd = p.route.finish_desc;
+        const int mine = tid < select_k ? s_route_ids[tid] : -1;
+        const bool in_range = tid < select_k && (unsigned)mine < (unsigned)p.experts;
+        const bool live = in_range && !(p.valid && p.valid[mine] == 0u);
+        const unsigned long long lives = __ballot(live);
+        int rank = 0;
+        for (int c = 0; c < select_k; ++c) {
+          const int other = s_route_ids[c];
+          const bool before = p.route.finish_ordered ? (other < mine || (other == mine && c < tid)) : c < tid;
+          rank += (((lives >> c) & 1ull) && before) ? 1 : 0;
+        }
+        if (live && rank < FFMOE_FINISH_ROUTED) {
+          fd->codes[rank] = p.slots[size_t(mine) * 6 + 4];
+          fd->scales[rank] = p.slots[size_t(mine) * 6 + 5];
+          fd->glob[rank] = p.global_scales ? p.global_scales[size_t(mine) * 3 + 2] : 1.0f;
+          fd->wk[rank] = s_route_w[tid];
+          fd->slot[rank] = tid;
+        }
+        if (tid == 0) {
+          fd->n = __builtin_popcountll(lives);
+          fd->bad = __builtin_popcountll(lives) != select_k ? 1 : 0;
+        }
+      }
     }
   }
   const long long total = shared_first ? routed_units : routed_units + (long long)n_shared * out_s;

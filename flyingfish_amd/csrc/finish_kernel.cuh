@@ -72,55 +72,103 @@ __global__ __launch_bounds__(1024) void k_decode_finish(const FinishParams q, co
 #pragma unroll
     for (int s = 0; s < S; ++s) issue_rows(B0{}, uni64(p.shared_slot[4]), uni64(p.shared_slot[5]), unif(p.shared_global[2]), wave, s);
   }
-
-  // live choices in combine order
-  if (tid < K) {
-    const int e = p.ids[tid];
-    bool live = !(p.active && p.active[tid] == 0u);
-    const bool wanted = live;
-    if (live) live = (unsigned)e < (unsigned)p.experts && !(p.valid && p.valid[e] == 0u);
-    if (live && p.generation && p.assignment_gen && p.generation[e] != p.assignment_gen[tid]) live = false;
-    if (wanted && !live && q.status && blockIdx.x == 0) atomicOr(q.status, 1u);  // bad or stale expert id
-    s_expert[tid] = live ? e : -1;
+  // Activations: row c of the arena belongs to choice c, row K to the shared expert, whichever experts were chosen, so
+  // all K + 1 rows are requested right here, in front of everything that depends on the ids, and go to LDS in arena
+  // order (a group finds its row through s_slot). Rows of choices that turn out not to be live are never read.
+  constexpr int HV = 8;  // 16-byte words per thread: (K + 1) * inter * 2 <= 64 KiB of LDS over >= 512 threads
+  const int row_words = I >> 3;
+  const int h_rows = K + (has_shared ? 1 : 0);
+  const int h_words = h_rows * row_words;
+  u32x4 hv[HV];
+#pragma unroll
+  for (int i = 0; i < HV; ++i) {
+    const int v = tid + i * nthreads;
+    const int vc = v < h_words ? v : 0;
+    const int row = vc / row_words;
+    hv[i] = load16(p.h + size_t(row) * p.h_stride + size_t(vc - row * row_words) * 8);
   }
-  __syncthreads();
-  if (tid < K) {
-    const int mine = s_expert[tid];
-    int rank = 0;
-    for (int c = 0; c < K; ++c) {
-      const int other = s_expert[c];
-      const bool before = ordered ? (other < mine || (other == mine && c < tid)) : c < tid;
-      rank += (other >= 0 && before) ? 1 : 0;
+  auto stage_activations = [&]() {
+    u32x4* dst = reinterpret_cast<u32x4*>(xs);
+#pragma unroll
+    for (int i = 0; i < HV; ++i) {
+      const int v = tid + i * nthreads;
+      if (v < h_words) dst[v] = hv[i];
     }
-    if (mine >= 0) s_choice[rank] = tid;
+    for (int v = tid + HV * nthreads; v < h_words; v += nthreads) {  // blocks below 512 threads with long rows
+      const int row = v / row_words;
+      dst[v] = load16(p.h + size_t(row) * p.h_stride + size_t(v - row * row_words) * 8);
+    }
+  };
+
+  int nr_;
+  if (q.desc) {
+    // the gate/up launch of the same call has resolved the live choices: one record instead of ids -> slot table
+    if (tid < FFMOE_FINISH_ROUTED) {
+      s_codes[tid] = q.desc->codes[tid]; s_scales[tid] = q.desc->scales[tid];
+      s_glob[tid] = q.desc->glob[tid]; s_wk[tid] = q.desc->wk[tid]; s_slot[tid] = q.desc->slot[tid];
+    }
+    if (tid == 0) {
+      s_groups = q.desc->n;
+      if (q.desc->bad && q.status && blockIdx.x == 0) atomicOr(q.status, 1u);
+    }
+    __syncthreads();
+    nr_ = uni(s_groups);
+    if (tid == 0 && has_shared) {
+      s_codes[nr_] = p.shared_slot[4]; s_scales[nr_] = p.shared_slot[5]; s_glob[nr_] = p.shared_global[2];
+      s_wk[nr_] = 1.0f;
+      s_slot[nr_] = K;
+    }
+  } else {
+    // live choices in combine order
+    if (tid < K) {
+      const int e = p.ids[tid];
+      bool live = !(p.active && p.active[tid] == 0u);
+      const bool wanted = live;
+      if (live) live = (unsigned)e < (unsigned)p.experts && !(p.valid && p.valid[e] == 0u);
+      if (live && p.generation && p.assignment_gen && p.generation[e] != p.assignment_gen[tid]) live = false;
+      if (wanted && !live && q.status && blockIdx.x == 0) atomicOr(q.status, 1u);  // bad or stale expert id
+      s_expert[tid] = live ? e : -1;
+    }
+    __syncthreads();
+    if (tid < K) {
+      const int mine = s_expert[tid];
+      int rank = 0;
+      for (int c = 0; c < K; ++c) {
+        const int other = s_expert[c];
+        const bool before = ordered ? (other < mine || (other == mine && c < tid)) : c < tid;
+        rank += (other >= 0 && before) ? 1 : 0;
+      }
+      if (mine >= 0) s_choice[rank] = tid;
+    }
+    if (tid == 0) {
+      int total = 0;
+      for (int c = 0; c < K; ++c) total += s_expert[c] >= 0 ? 1 : 0;
+      s_groups = total;
+    }
+    __syncthreads();
+    nr_ = uni(s_groups);
+    // per-group constants: thread g gathers group g (ids -> slot table, two dependent loads, all groups in parallel)
+    if (tid < nr_ + (has_shared ? 1 : 0)) {
+      if (tid < nr_) {
+        const int c = s_choice[tid];
+        const int e = s_expert[c];
+        s_codes[tid] = p.slots[size_t(e) * 6 + 4];
+        s_scales[tid] = p.slots[size_t(e) * 6 + 5];
+        s_glob[tid] = p.global_scales ? p.global_scales[size_t(e) * 3 + 2] : 1.0f;
+        s_wk[tid] = p.weights_f32 ? reinterpret_cast<const float*>(p.weights)[c] : bf16_to_f32(reinterpret_cast<const uint16_t*>(p.weights)[c]);
+        s_slot[tid] = c;
+      } else {
+        s_codes[tid] = p.shared_slot[4]; s_scales[tid] = p.shared_slot[5]; s_glob[tid] = p.shared_global[2];
+        s_wk[tid] = 1.0f;
+        s_slot[tid] = K;  // rows == 1: the shared expert's activations follow the K routed slots
+      }
+    }
   }
-  if (tid == 0) {
-    int total = 0;
-    for (int c = 0; c < K; ++c) total += s_expert[c] >= 0 ? 1 : 0;
-    s_groups = total;
-  }
-  __syncthreads();
-  const int nr = uni(s_groups);                 // routed groups, in combine order
+  const int nr = nr_;                           // routed groups, in combine order
   const int G = nr + (has_shared ? 1 : 0);      // group nr = the shared expert
   if (G == 0 && !q.shared_ready) {  // nothing contributes: y = 0
     for (int d = blockIdx.x * nthreads + tid; d < H; d += gridDim.x * nthreads) q.y[d] = 0;
     return;
-  }
-  // per-group constants: thread g gathers group g (ids -> slot table, two dependent loads, all groups in parallel)
-  if (tid < G) {
-    if (tid < nr) {
-      const int c = s_choice[tid];
-      const int e = s_expert[c];
-      s_codes[tid] = p.slots[size_t(e) * 6 + 4];
-      s_scales[tid] = p.slots[size_t(e) * 6 + 5];
-      s_glob[tid] = p.global_scales ? p.global_scales[size_t(e) * 3 + 2] : 1.0f;
-      s_wk[tid] = p.weights_f32 ? reinterpret_cast<const float*>(p.weights)[c] : bf16_to_f32(reinterpret_cast<const uint16_t*>(p.weights)[c]);
-      s_slot[tid] = c;
-    } else {
-      s_codes[tid] = p.shared_slot[4]; s_scales[tid] = p.shared_slot[5]; s_glob[tid] = p.shared_global[2];
-      s_wk[tid] = 1.0f;
-      s_slot[tid] = K;  // rows == 1: the shared expert's activations follow the K routed slots
-    }
   }
   __syncthreads();
 
@@ -152,29 +200,23 @@ __global__ __launch_bounds__(1024) void k_decode_finish(const FinishParams q, co
       for (int s = 0; s < S; ++s) issue_unit(B1{}, 1, s);
     }
   }
-  // activations of every group -> LDS, behind the first weight requests
+  // NVFP4: the split dot's constants of every group's down matrix; then the activations, which were requested first
   if constexpr (NV) {
     for (int g = 0; g < G; ++g) FmtNvfp4::build_lut(s_lut + g * FmtNvfp4::LUT_ENTRIES, s_glob[g], tid, nthreads);
   }
-  {
-    const int row_words = I >> 3;
-    for (int g = 0; g < G; ++g) {
-      u32x4* dst = reinterpret_cast<u32x4*>(xs + size_t(g) * I * 2);
-      const uint16_t* src = p.h + size_t(s_slot[g]) * p.h_stride;
-      for (int v = tid; v < row_words; v += nthreads) dst[v] = load16(src + size_t(v) * 8);
-    }
-  }
+  stage_activations();
   __syncthreads();
   auto unit = [&](auto which, int t) {
     constexpr int b_ = decltype(which)::value;
     int g, i;
     unit_of(t, g, i);
+    const int arow = uni(s_slot[g]);  // the group's activation row in LDS (arena order)
     float acc[NR][1];
 #pragma unroll
     for (int m = 0; m < NR; ++m) acc[m][0] = 0.0f;
 #pragma unroll
     for (int s = 0; s < S; ++s) {
-      step_compute<F, NR, 1, S, NV>(buf[b_], s, xs + size_t(g) * I * 2, I, nchunks, s * 64 + lane, 1, acc, s_lut + (NV ? g * FmtNvfp4::LUT_ENTRIES : 0));
+      step_compute<F, NR, 1, S, NV>(buf[b_], s, xs + size_t(arow) * I * 2, I, nchunks, s * 64 + lane, 1, acc, s_lut + (NV ? g * FmtNvfp4::LUT_ENTRIES : 0));
       issue_unit(which, t + NB, s);
     }
     float total[NR];
