@@ -21,8 +21,10 @@ namespace ffmoe {
 
 #define FFMOE_FINISH_GROUPS 9  /* 8 routed choices + the shared expert */
 
-template <class F, int S, int NR>
-__global__ __launch_bounds__(1024) void k_decode_finish(const FinishParams q, const int cmax) {
+// MAXT: the largest block the instantiation is launched with. Blocks of eight waves (the usual shape) are compiled for two
+// waves per SIMD, i.e. with the whole register file of 256 registers per lane; 12 and 16 waves need the 128-register build.
+template <class F, int S, int NR, int MAXT = 1024>
+__global__ __launch_bounds__(MAXT) void k_decode_finish(const FinishParams q, const int cmax) {
   const DecodeParams& p = q.d;
   constexpr int GT = FFMOE_FINISH_GROUPS;
   extern __shared__ __align__(16) uint8_t xs[];  // [GT][inter] BF16 activations, then [GT][cmax] f32 row sums
@@ -48,7 +50,9 @@ __global__ __launch_bounds__(1024) void k_decode_finish(const FinishParams q, co
   const int P = (C + NR - 1) / NR;  // units per group
   const int nchunks = I / F::EPL;
   // One register buffer per wave: as soon as step s of a unit has been consumed, step s of the wave's next unit is requested
-  // into the same registers (a second buffer, two units ahead, measured the same: 28.1 against 28.3 us at hidden 7168).
+  // into the same registers. A second buffer, two units ahead, is slower for both formats measured (FP8 at hidden 7168:
+  // 28.5 against 27.0 us, more requests in flight than the memory system takes; NVFP4: 24.1 against 22.1 us, its units
+  // are bound by the conversion work, not by requests in flight).
   constexpr int NB = 1;
   typename F::Chunk buf[NB][NR][S];
   auto issue_rows = [&](auto which, uint64_t codes, uint64_t scales, float glob, int i, int s) {
@@ -263,7 +267,10 @@ __global__ __launch_bounds__(1024) void k_decode_finish(const FinishParams q, co
 template <class F, int NR, int SMAX, int S = 1>
 void launch_finish_steps(int want, const FinishParams& q, int blocks, int threads, int cmax, size_t lds, hipStream_t st) {
   if constexpr (S <= SMAX) {
-    if (want == S) hipLaunchKernelGGL((k_decode_finish<F, S, NR>), dim3(blocks), dim3(threads), lds, st, q, cmax);
+    if (want == S) {
+      if (threads <= 512) hipLaunchKernelGGL((k_decode_finish<F, S, NR, 512>), dim3(blocks), dim3(threads), lds, st, q, cmax);
+      else hipLaunchKernelGGL((k_decode_finish<F, S, NR, 1024>), dim3(blocks), dim3(threads), lds, st, q, cmax);
+    }
     else launch_finish_steps<F, NR, SMAX, S + 1>(want, q, blocks, threads, cmax, lds, st);
   }
 }
@@ -301,6 +308,8 @@ int launch_finish(const FinishParams& q, hipStream_t st) {
     int b = 0, w = 0;
     if (sscanf(e, "%d,%d", &b, &w) == 2 && b >= 1 && w >= 1 && w <= 16) { blocks = b; waves = w; }
   }
+  // NVFP4 rows of two steps hold their split-dot operands in more registers than the 128 of a 12- or 16-wave block
+  if (std::is_same<F, FmtNvfp4>::value && steps == 2 && waves > 8) waves = 8;
   const int cmax = (p.hidden + blocks - 1) / blocks;
   const size_t lds = size_t(FFMOE_FINISH_GROUPS) * p.inter * 2 + size_t(FFMOE_FINISH_GROUPS) * cmax * 4;
   const size_t tables = std::is_same<F, FmtNvfp4>::value ? size_t(FFMOE_FINISH_GROUPS) * FmtNvfp4::LUT_ENTRIES * 8 : 0;  // static, next to lds
