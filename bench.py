@@ -424,6 +424,26 @@ def prefill_main(args, torch, capi, ops, synth, prebuilt=None):
     k0_avg, k1_avg = sum(k0) / len(k0), sum(k1) / len(k1)
     flop0 = A * 4.0 * H * I
     per = table.weight_bytes_per_expert()
+    # side pass in front of the cohort, reported apart from it: the FP32 router logits of all R rows (the cohort itself
+    # starts from seeded logits), R x E x H multiply-adds on the vector ALUs in the oracle's summation order
+    router = synth.normal((E, H), 0.02, args.seed + 1, device=dev, dtype=torch.bfloat16)
+    lg_out = torch.empty((R, E), dtype=torch.float32, device=dev)
+    for _ in range(2):
+        ops.RouteOps.logits_f32(x, router, out=lg_out)
+    evl = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(5)]
+    for a, b in evl:
+        a.record(); ops.RouteOps.logits_f32(x, router, out=lg_out); b.record()
+    torch.cuda.synchronize()
+    lg_ms = sorted(a.elapsed_time(b) for a, b in evl)[len(evl) // 2]
+    lg_parity = None
+    if not args.no_parity_gate:
+        _, orc_, hp_ = _checkers()
+        sample = [0, R // 2, R - 1]
+        want_lg = orc_.route_logits_f32(hp_.bits(x[sample]), hp_.bits(router))
+        if not (lg_out[sample].cpu().numpy().view("uint32") == want_lg.view("uint32")).all():
+            print("bench.py parity gate FAILED: router logits differ from the oracle", file=sys.stderr)
+            sys.exit(3)
+        lg_parity = "rows %s bit-exact against the oracle" % sample
     out = {
         "metric": "moe_prefill_ms", "value": ms, "unit": "ms/cohort", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
@@ -452,6 +472,10 @@ def prefill_main(args, torch, capi, ops, synth, prebuilt=None):
         "down_kernel": {"kernel": "ffmoe::k_w16_grouped<F, MF, 1, P>" if a16 else "ffmoe::k_mx_grouped<MF, 1, 1, P>" if mx else "ffmoe::k_w8a8_grouped<MF, 1, P>", "avg_ms": k1_avg, "min_ms": k1[0],
                         "tflops": A * 2.0 * H * I / (k1_avg * 1e-3) / 1e12},
     }
+    out["router_logits"] = {"kernel": "ffmoe::k_route_logits_f32_rows (FP32 logits of all token rows, vector ALUs, the oracle's summation order)",
+                            "ms": lg_ms, "flop": 2.0 * R * E * H, "tflops": 2.0 * R * E * H / (lg_ms * 1e-3) / 1e12,
+                            "frac_of_fp32_vector_peak": 2.0 * R * E * H / (lg_ms * 1e-3) / 1e12 / 157.3, "parity": lg_parity,
+                            "note": "side pass, not part of `value`: the cohort starts from seeded logits (BASELINE config 5)"}
     out["parity"] = parity if parity is not None else ("not gated in bench.py for this format (tests/test_gpu_e8m0.py, tests/test_gpu_fullsize.py)" if mx else None)
     if not args.no_cpu_baseline and args.format == "fp8":
         out["cpu_baseline"] = cpu_baseline_prefill(args, torch, table, x, ids, wts, dims)

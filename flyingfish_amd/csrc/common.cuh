@@ -278,6 +278,69 @@ __device__ __forceinline__ void wave_argmax(float& v, int& id) {
   id = __builtin_amdgcn_readlane(id, 63);
 }
 
+// 64 values per lane in, one value per lane out: lane L ends with the sum over the wave's 64 lanes of value
+// bitrev6(L), added in the adjacent-pair tree (lanes 2i and 2i+1, then pairs of pairs, ...), i.e. bit for bit what
+// wave_sum gives for that value. At every level the two partners split the values they still hold: each keeps one half,
+// sends the other and adds what it receives, so level k moves 64 / 2^k values instead of 64 - about 200 instructions
+// where 64 calls of wave_sum take 1600. Levels 1-4 exchange inside a row of 16 lanes on the DPP path, levels 5 and 6
+// with the row and half-wave swaps of gfx950.
+// v_permlane16_swap_b32 a, b: lanes 16-31 and 48-63 of a trade places with lanes 0-15 and 32-47 of b;
+// v_permlane32_swap_b32 a, b: lanes 32-63 of a trade places with lanes 0-31 of b. Both operands are read and written,
+// which is stated here operand by operand (the compiler's own builtins for the two instructions lost the second result in
+// this toolchain: the sum of the two results came out as twice the first). The idle cycles in front and behind are
+// the wait states the compiler would insert between vector ALU writes and these cross-lane reads.
+__device__ __forceinline__ void swap_rows16(float& a, float& b) {
+  asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+}
+__device__ __forceinline__ void swap_halves32(float& a, float& b) {
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+}
+constexpr int DPP_ROW_SHL4 = 0x104, DPP_ROW_SHR4 = 0x114, DPP_ROW_SHL8 = 0x108, DPP_ROW_SHR8 = 0x118;
+__device__ __forceinline__ float wave_reduce_scatter64(float (&a)[64], int lane) {
+  const bool b0 = lane & 1, b1 = lane & 2, b2 = lane & 4, b3 = lane & 8;
+  float c[32];
+#pragma unroll
+  for (int j = 0; j < 32; ++j) {  // partner lane ^ 1; a lane with bit 0 set keeps the upper half
+    const float send = b0 ? a[j] : a[j + 32], keep = b0 ? a[j + 32] : a[j];
+    c[j] = __fadd_rn(keep, dpp_or<DPP_QUAD_SWAP1, 0xf>(0.0f, send));
+  }
+  float d[16];
+#pragma unroll
+  for (int j = 0; j < 16; ++j) {  // lane ^ 2
+    const float send = b1 ? c[j] : c[j + 16], keep = b1 ? c[j + 16] : c[j];
+    d[j] = __fadd_rn(keep, dpp_or<DPP_QUAD_SWAP2, 0xf>(0.0f, send));
+  }
+  float e[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {  // lane ^ 4: banks 0 and 2 of a row read four lanes up, banks 1 and 3 four lanes down
+    const float send = b2 ? d[j] : d[j + 8], keep = b2 ? d[j + 8] : d[j];
+    float got = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, send), DPP_ROW_SHL4, 0xf, 0x5, false));
+    got = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, got), __builtin_bit_cast(int, send), DPP_ROW_SHR4, 0xf, 0xa, false));
+    e[j] = __fadd_rn(keep, got);
+  }
+  float f[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {  // lane ^ 8: banks 0 and 1 read eight lanes up, banks 2 and 3 eight lanes down
+    const float send = b3 ? e[j] : e[j + 4], keep = b3 ? e[j + 4] : e[j];
+    float got = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, send), DPP_ROW_SHL8, 0xf, 0x3, false));
+    got = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, got), __builtin_bit_cast(int, send), DPP_ROW_SHR8, 0xf, 0xc, false));
+    f[j] = __fadd_rn(keep, got);
+  }
+  // lane ^ 16: the odd rows of the first operand trade places with the even rows of the second, after which an even-row
+  // lane holds both partners' copies of the first value and an odd-row lane both copies of the second
+  float g[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    float lo = f[j], hi = f[j + 2];
+    swap_rows16(lo, hi);
+    g[j] = __fadd_rn(lo, hi);
+  }
+  // lane ^ 32: the same with the two halves of the wave
+  swap_halves32(g[0], g[1]);
+  return __fadd_rn(g[0], g[1]);
+}
+__device__ __forceinline__ int bitrev6(int v) { return int(__builtin_bitreverse32(unsigned(v)) >> 26); }
+
 // Wave-uniform copies of values every lane already agrees on: they move to scalar registers, so addresses built
 // from them use a scalar base.
 __device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }

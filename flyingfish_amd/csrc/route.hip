@@ -3,6 +3,8 @@
 #include "common.cuh"
 #include "route_select.cuh"
 #include "api.h"
+#include <stdlib.h>
+#include <algorithm>
 
 namespace ffmoe {
 
@@ -207,6 +209,81 @@ __global__ __launch_bounds__(256) void k_route_logits_f32(const uint16_t* __rest
   logits_f32_rows(x, router, logits, blockIdx.x, r0, r1, experts, hidden, s_part);
 }
 
+// FP32 logits for many token rows (a prefill cohort: 4096 x 256 x 7168 is 15 GFLOP, and with eight rows per pass over a
+// router row the kernel above re-reads the 3.67 MB router 512 times). Same products, same order, same tree per logit
+// as k_route_logits_f32: partial chain p (0 .. 255) walks the 16-byte vectors p, p + 256, ... element by element, the
+// 256 partials meet in the adjacent-pair tree. A block owns a tile of ME experts, whose router rows stay in LDS as BF16
+// for the whole launch, and a run of token rows; it is TEAMS teams of 256 threads, thread t of a team = chain t. A
+// team takes MR rows at a time: per vector it widens its slice of the MR rows once (registers) and walks the ME
+// experts out of LDS, MR x 8 fmas per 16-byte LDS read, so the widening costs a fifth of the fmas. Row chunks map to
+// XCDs (block index mod 8), so the blocks that read the same token rows at about the same time share an L2.
+constexpr int LG_ME = 8, LG_MR = 8, LG_TEAMS = 3;
+
+__global__ __launch_bounds__(256 * LG_TEAMS) void k_route_logits_f32_rows(const uint16_t* __restrict__ x, const uint16_t* __restrict__ router,
+                                                                           float* __restrict__ logits, int rows, int experts, int hidden,
+                                                                           int row_chunks) {
+  extern __shared__ __align__(16) uint8_t lg_lds[];
+  const int tid = threadIdx.x, team = uni(tid >> 8), t = tid & 255, lane = tid & 63, wave_in_team = uni((tid >> 6) & 3);
+  const int words = hidden >> 3;
+  const int nvec = (words + 255) >> 8;  // vectors per chain
+  u32x4* wl = reinterpret_cast<u32x4*>(lg_lds);                                   // [ME][words] router tile
+  float* part = reinterpret_cast<float*>(lg_lds + size_t(LG_ME) * words * 16);   // [TEAMS][4 waves][MR * ME]
+  const int chunk = blockIdx.x % row_chunks, etile = blockIdx.x / row_chunks;
+  const int e0 = etile * LG_ME;
+  const int per_chunk = (rows + row_chunks - 1) / row_chunks;
+  const int r_lo = chunk * per_chunk, r_hi = min(rows, r_lo + per_chunk);
+  for (int v = tid; v < LG_ME * words; v += 256 * LG_TEAMS) {
+    const int e = v / words, w = v - e * words;
+    wl[v] = load16(router + size_t(min(e0 + e, experts - 1)) * hidden + size_t(w) * 8);
+  }
+  __syncthreads();
+  for (int rb = r_lo; rb < r_hi; rb += LG_MR * LG_TEAMS) {  // uniform trip count over the block: the barriers below are block-wide
+    const int r0 = rb + team * LG_MR;
+    float acc[LG_MR * LG_ME];
+#pragma unroll
+    for (int j = 0; j < LG_MR * LG_ME; ++j) acc[j] = 0.0f;
+    for (int i = 0; i < nvec; ++i) {
+      const int v = t + 256 * i;
+      if (v < words) {  // a chain that ends early skips the step: its lanes are switched off, its sums stay as they are
+        float xf[LG_MR][8];
+#pragma unroll
+        for (int r = 0; r < LG_MR; ++r) {
+          const int row = min(r0 + r, rows - 1);
+          const u32x4 xv = load16(x + size_t(row) * hidden + size_t(v) * 8);
+#pragma unroll
+          for (int q = 0; q < 4; ++q) { xf[r][2 * q] = bf16lo(xv[q]); xf[r][2 * q + 1] = bf16hi(xv[q]); }
+        }
+#pragma unroll
+        for (int e = 0; e < LG_ME; ++e) {
+          const u32x4 wv = wl[e * words + v];
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const float w0 = bf16lo(wv[q]), w1 = bf16hi(wv[q]);
+#pragma unroll
+            for (int r = 0; r < LG_MR; ++r) acc[r * LG_ME + e] = __fmaf_rn(xf[r][2 * q], w0, acc[r * LG_ME + e]);
+#pragma unroll
+            for (int r = 0; r < LG_MR; ++r) acc[r * LG_ME + e] = __fmaf_rn(xf[r][2 * q + 1], w1, acc[r * LG_ME + e]);
+          }
+        }
+      }
+    }
+    // the adjacent-pair tree over the 256 chains: the 64 lanes of a wave (lane L ends with the sum of value bitrev6(L)),
+    // then the team's four waves
+    float* mine = part + (team * 4 + wave_in_team) * (LG_MR * LG_ME);
+    static_assert(LG_MR * LG_ME == 64, "one value per lane");
+    const float wsum = wave_reduce_scatter64(acc, lane);
+    mine[bitrev6(lane)] = wsum;
+    __syncthreads();
+    if (t < LG_MR * LG_ME) {
+      const int r = t / LG_ME, e = t - r * LG_ME;
+      const float* pt = part + team * 4 * (LG_MR * LG_ME) + t;
+      const float total = __fadd_rn(__fadd_rn(pt[0], pt[LG_MR * LG_ME]), __fadd_rn(pt[2 * LG_MR * LG_ME], pt[3 * LG_MR * LG_ME]));
+      if (r0 + r < r_hi && e0 + e < experts) logits[size_t(r0 + r) * experts + e0 + e] = total;
+    }
+    __syncthreads();
+  }
+}
+
 // ---------------------------------------------------------------------------------------------
 // Selection by rank. The reference runs top_k rounds of a block-wide arg-max under (score desc, id asc)
 // (kernels/moe_route.cu:205-235); that order is total, so the r-th pick is the candidate with exactly r
@@ -383,6 +460,15 @@ __global__ __launch_bounds__(64) void k_route_topk_noaux_wave(const float* __res
 
 using namespace ffmoe;
 
+static int decode_cus() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0, n = 0;
+    cus = (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) ? n : 256;
+  }
+  return cus;
+}
+
 static int check_route_dims(int rows, int experts, int hidden) {
   FF_REQUIRE(rows >= 1 && experts >= 1 && experts <= FFMOE_MAX_EXPERTS, FFMOE_ERR_SHAPE,
              "router rows=%d experts=%d outside [1, %d]", rows, experts, FFMOE_MAX_EXPERTS);
@@ -407,6 +493,28 @@ extern "C" __attribute__((visibility("default"))) int ffmoe_route_logits_f32(con
   FF_PTR16(x); FF_PTR16(router); FF_PTR4(logits);
   FF_NO_OVERLAP(logits, size_t(rows) * experts * 4, x, size_t(rows) * hidden * 2);
   FF_NO_OVERLAP(logits, size_t(rows) * experts * 4, router, size_t(experts) * hidden * 2);
+  // Many rows: the kernel that keeps a tile of router rows in LDS (from FFMOE_ROUTE_LOGITS_TILE_ROWS rows on, default 96 - 15.8 against 18.4 us there at 256 x 7168, 13.2 against 15.5 us at 64 rows;
+  // 0 = never), when the tile and the partial sums fit. Same bits either way.
+  {
+    static const int tile_rows = [] { const char* e = getenv("FFMOE_ROUTE_LOGITS_TILE_ROWS"); return e ? atoi(e) : 96; }();
+    const size_t lds = size_t(LG_ME) * hidden * 2 + size_t(LG_TEAMS) * 4 * LG_MR * LG_ME * 4;
+    if (tile_rows > 0 && rows >= tile_rows && lds <= 150 * 1024) {
+      static int lds_ok = -1;
+      if (lds_ok < 0)
+        lds_ok = hipFuncSetAttribute(reinterpret_cast<const void*>(k_route_logits_f32_rows), hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024) == hipSuccess ? 1 : 0;
+      if (lds_ok == 1) {
+        const int etiles = (experts + LG_ME - 1) / LG_ME;
+        // a block takes LG_MR * LG_TEAMS rows per pass and one block fits a CU: as many row chunks as keep the grid within
+        // one round of blocks, eight (one per XCD) for a cohort
+        const int per_pass = LG_MR * LG_TEAMS;
+        const int max_chunks = std::max(1, decode_cus() / etiles);
+        const int row_chunks = std::max(1, std::min(max_chunks, (rows + per_pass - 1) / per_pass));
+        hipLaunchKernelGGL(k_route_logits_f32_rows, dim3(unsigned(etiles) * unsigned(row_chunks)), dim3(256 * LG_TEAMS), lds, (hipStream_t)stream,
+                           (const uint16_t*)x, (const uint16_t*)router, logits, rows, experts, hidden, row_chunks);
+        return ff_launch_status();
+      }
+    }
+  }
   FF_REQUIRE((rows + LOGIT_ROWS - 1) / LOGIT_ROWS <= 65535, FFMOE_ERR_SHAPE, "too many rows (%d) for one logits launch", rows);
   hipLaunchKernelGGL(k_route_logits_f32, dim3(experts, (rows + LOGIT_ROWS - 1) / LOGIT_ROWS), dim3(256), 0, (hipStream_t)stream,
                      (const uint16_t*)x, (const uint16_t*)router, logits, rows, experts, hidden);

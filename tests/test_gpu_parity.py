@@ -121,7 +121,9 @@ def test_route_logits_bf16_bit_exact(rows, experts, hidden):
     assert np.array_equal(got, orc.route_logits_bf16(bits(x), bits(w)))
 
 
-@pytest.mark.parametrize("rows,experts,hidden", [(1, 256, 7168), (9, 64, 2048), (5, 33, 520)])
+@pytest.mark.parametrize("rows,experts,hidden", [(1, 256, 7168), (9, 64, 2048), (5, 33, 520),
+                                                 # from 96 rows on: the kernel that keeps a tile of router rows in LDS
+                                                 (300, 256, 7168), (96, 8, 2048), (97, 33, 520), (203, 50, 4104), (1000, 9, 8), (128, 256, 7168)])
 def test_route_logits_f32_bit_exact_and_close_to_f64(rows, experts, hidden):
     x, w = rand_bf16((rows, hidden), 1.0, 13), rand_bf16((experts, hidden), 0.02, 14)
     got = RouteOps.logits_f32(x.to(DEV), w.to(DEV)).cpu().numpy()
