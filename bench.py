@@ -49,8 +49,9 @@ def parse():
     ap.add_argument("--experts", type=int, default=256)
     ap.add_argument("--ring", type=int, default=64, help="distinct token batches cycled through")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--prefill-act", choices=["fp8", "bf16"], default="fp8", help="prefill: W8A8 on the FP8 matrix cores (block-FP8 "
-                    "experts) or the decode path's W*A16 arithmetic on the BF16 matrix cores (any --format)")
+    ap.add_argument("--prefill-act", choices=["auto", "fp8", "bf16"], default="auto", help="prefill: fp8 = FP8 activations on the FP8 matrix "
+                    "cores (W8A8 for block-FP8 experts; W4A8 for --format nvfp4, whose weights are rounded to E4M3 inside the kernel); "
+                    "bf16 = the decode path's W*A16 arithmetic on the BF16 matrix cores (any --format); auto = fp8 for --format fp8, bf16 for nvfp4")
     ap.add_argument("--one-launch", action="store_true", help="one token: selection, gate/up, down and combine in the one resident "
                     "launch (ffmoe_decode_token_layer) instead of launches of their own")
     ap.add_argument("--separate-topk", action="store_true", help="one token: run the top-k selection as a launch of its own "
@@ -272,6 +273,11 @@ def parity_gate_prefill(args, torch, capi, ops, table, pre, x, ids, wts, dims, a
     host = {}
     for e in sorted({int(flat_ids[perm[p]]) for p in picks}):
         host[e] = hp.effective_weights(table, e) if a16 else hp.host_expert(table, e)
+        if not a16 and table.format == capi.FMT_NVFP4:  # W4A8: the oracle's E4M3 derivation of the NVFP4 weights, then W8A8
+            m, d8 = host[e], []
+            for i in range(3):
+                d8 += list(orc.nvfp4_to_fp8_block(m[2 * i], m[2 * i + 1], float(table.global_scales[e, i].item())))
+            host[e] = d8
 
     def one(lo, hi):
         out = []
@@ -370,8 +376,9 @@ def prefill_main(args, torch, capi, ops, synth, prebuilt=None):
     x = synth.normal((R, H), 1.0, args.seed + 5000, device=dev, dtype=torch.bfloat16)
     bias = torch.zeros(E, dtype=torch.float32, device=dev)
     mx = args.format == "e2m1"
-    a16 = not mx and (args.prefill_act == "bf16" or args.format == "nvfp4")
-    default_cohort = not mx and not a16 and R == 4096 and E == 256 and args.seed == 20251  # the cohort the committed profile measured
+    a16 = not mx and (args.prefill_act == "bf16" or (args.format == "nvfp4" and args.prefill_act != "fp8"))
+    w4a8 = not mx and not a16 and args.format == "nvfp4"
+    default_cohort = not mx and not a16 and args.format == "fp8" and R == 4096 and E == 256 and args.seed == 20251  # the cohort the committed profile measured
     if mx:
         pre = ops.PrefillOps(table, R, K, swiglu=capi.SWIGLU_CLAMPED_ONCE, swiglu_limit=7.0, routed_weight=capi.WEIGHT_BEFORE_DOWN_F32,
                              weights_f32=True, act_mode=capi.ACT_E4M3_E8M0_32)
@@ -448,13 +455,15 @@ def prefill_main(args, torch, capi, ops, synth, prebuilt=None):
         "metric": "moe_prefill_ms", "value": ms, "unit": "ms/cohort", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
         "dtype": ("%s weights dequantized to bf16 x bf16 activations, f32 accumulate" % args.format) if a16 else
+                 "nvfp4 weights rounded to fp8_e4m3 in the kernel x fp8_e4m3 activations (per-128 f32 scales), f32 accumulate" if w4a8 else
                  "fp4_e2m1 weights x fp8_e4m3 activations, e8m0 scales per 32 applied by the matrix core, f32 accumulate" if mx else
                  "fp8_e4m3 weights x fp8_e4m3 activations (per-128 f32 scales), f32 accumulate", "data": "synthetic",
-        "config": {"workload": ("DeepSeek-V3-shape %s MoE prefill, %d tokens, Zipf s=1.1" % (args.format.upper(), R)) if (a16 or mx) else
+        "config": {"workload": ("DeepSeek-V3-shape %s MoE prefill, %d tokens, Zipf s=1.1" % (args.format.upper(), R)) if (a16 or mx or w4a8) else
                                "DeepSeek-V3-shape FP8 MoE prefill (BASELINE config 5), %d tokens, Zipf s=1.1" % R,
                    "hidden": H, "intermediate": I, "experts": E, "top_k": K,
                    "act_mode": "FFMOE_ACT_BF16 (W*A16 on the BF16 matrix cores)" if a16 else
-                               "FFMOE_ACT_E4M3_E8M0_32 (W4A8 on the MX matrix cores)" if mx else "FFMOE_ACT_FP8_BLOCK128 (W8A8)",
+                               "FFMOE_ACT_E4M3_E8M0_32 (W4A8 on the MX matrix cores)" if mx else
+                               "FFMOE_ACT_FP8_BLOCK128 on NVFP4 experts (W4A8 on the FP8 matrix cores)" if w4a8 else "FFMOE_ACT_FP8_BLOCK128 (W8A8)",
                    "tokens": R, "experts_touched": touched, "max_rows_per_expert": int(counts.max()), "min_rows_per_expert": int(counts.min())},
         "tokens_per_s": R / (ms * 1e-3),
         "routed_tflop": flop_total / 1e12,
@@ -961,7 +970,7 @@ def secondary(args, torch, capi, ops, synth, fp8_table):
         out, _ = decode_main(a, torch, capi, ops, synth, prebuilt=fp8)
         sec["c3_fp8_batch%d" % batch] = _brief_decode(out)
     a = copy.copy(args)
-    a.workload, a.batch, a.steps, a.warmup, a.prefill_act = "prefill", 4096, 6, 2, "fp8"
+    a.workload, a.batch, a.steps, a.warmup, a.prefill_act = "prefill", 4096, 6, 2, "auto"
     out = prefill_main(a, torch, capi, ops, synth, prebuilt=fp8)
     sec["c5_fp8_prefill_4096"] = {
         "workload": out["config"]["workload"], "ms": out["value"], "steps": out["steps"], "flop": out["routed_tflop"] * 1e12, "tflops": out["cohort_tflops"],

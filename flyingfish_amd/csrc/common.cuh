@@ -378,8 +378,15 @@ __device__ __forceinline__ void load16_async(u32x4& d, uint64_t base, uint32_t o
 __device__ __forceinline__ void load4_async(float& d, const void* p) {
   asm volatile("global_load_dword %0, %1, off" : "=v"(d) : "v"(p));
 }
+__device__ __forceinline__ void load4_async(float& d, uint64_t base, uint32_t offset) {
+  asm volatile("global_load_dword %0, %1, %2" : "=v"(d) : "v"(offset), "s"(base));
+}
 template <int N>
 __device__ __forceinline__ void wait_loads(u32x4& a, u32x4& b, u32x4& c, u32x4& d, u32x4& e, u32x4& f, u32x4& g, u32x4& h) {
+  asm volatile("s_waitcnt vmcnt(%8)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d), "+v"(e), "+v"(f), "+v"(g), "+v"(h) : "n"(N));
+}
+template <int N>
+__device__ __forceinline__ void wait_loads(u32x4& a, u32x4& b, u32x4& c, u32x4& d, float& e, float& f, float& g, float& h) {
   asm volatile("s_waitcnt vmcnt(%8)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d), "+v"(e), "+v"(f), "+v"(g), "+v"(h) : "n"(N));
 }
 template <int N>

@@ -373,7 +373,11 @@ int pick_rgb() {
 
 // wide: 64-row groups with eight waves per block (twice the columns per unit and token tile), one block per CU
 template <int MODE>
-int launch_gemm(const GemmParams& p, int mf, unsigned blocks, hipStream_t stream, bool wide = false) {
+int launch_gemm(const GemmParams& p, int mf, unsigned blocks, hipStream_t stream, bool wide = false, bool nv = false) {
+  if (nv) {  // NVFP4 weights turned into E4M3 on their way through LDS: the eight-wave 64-row kernel only
+    hipLaunchKernelGGL((k_w8a8_grouped<4, MODE, 2, 8, true>), dim3(blocks), dim3(512), 0, stream, p);
+    return ff_launch_status();
+  }
   if (wide) {
     hipLaunchKernelGGL((k_w8a8_grouped<4, MODE, 2, 8>), dim3(blocks), dim3(512), 0, stream, p);
     return ff_launch_status();
@@ -638,8 +642,13 @@ int prefill_impl(const ffmoe_expert_table* table, const ffmoe_prefill* args, int
     FF_REQUIRE(table->format == FFMOE_FMT_FP8_BLOCK128 || table->format == FFMOE_FMT_NVFP4 || table->format == FFMOE_FMT_BF16 || table->format == FFMOE_FMT_FP8_CHANNEL,
                FFMOE_ERR_UNSUPPORTED, "unknown expert format %d", table->format);
   else
-    FF_REQUIRE(table->format == FFMOE_FMT_FP8_BLOCK128, FFMOE_ERR_UNSUPPORTED, "the W8A8 prefill runs on the FP8 matrix cores and takes FFMOE_FMT_FP8_BLOCK128 experts only (format %d)", table->format);
+    FF_REQUIRE(table->format == FFMOE_FMT_FP8_BLOCK128 || table->format == FFMOE_FMT_NVFP4, FFMOE_ERR_UNSUPPORTED,
+               "FP8 activations on the FP8 matrix cores take FFMOE_FMT_FP8_BLOCK128 experts (W8A8) or FFMOE_FMT_NVFP4 experts (W4A8) (format %d)", table->format);
   }
+  // W4A8: NVFP4 experts with FP8 activations. Each weight becomes E4M3 inside the kernel (E2M1 value x E4M3 scale / 8,
+  // rounded to nearest even), the matrix's global scale x 8 takes the place of the block scales
+  const bool nv = !mx && !a16 && table->format == FFMOE_FMT_NVFP4;
+  if (nv) FF_PTR4(table->global_scales);
   const int E = table->experts, H = table->hidden, I = table->inter, R = args->rows, K = args->top_k;
   FF_REQUIRE(E >= 1 && E <= FFMOE_MAX_EXPERTS, FFMOE_ERR_SHAPE, "experts=%d out of range", E);
   FF_REQUIRE(R >= 1 && K >= 1 && K <= FFMOE_MAX_TOP_K && (long long)R * K <= 0x3fffffffLL, FFMOE_ERR_SHAPE, "rows=%d top_k=%d out of range", R, K);
@@ -669,7 +678,8 @@ int prefill_impl(const ffmoe_expert_table* table, const ffmoe_prefill* args, int
       const int gran = shared->format == FFMOE_FMT_FP8_BLOCK128 ? 128 : 64;
       FF_REQUIRE(SI >= gran && SI % gran == 0 && H % gran == 0, FFMOE_ERR_SHAPE, "shared inter=%d and hidden=%d must be multiples of %d", SI, H, gran);
     } else {
-      FF_REQUIRE(shared->format == FFMOE_FMT_FP8_BLOCK128, FFMOE_ERR_UNSUPPORTED, "the W8A8 prefill needs an FFMOE_FMT_FP8_BLOCK128 shared expert (format %d)", shared->format);
+      FF_REQUIRE(shared->format == FFMOE_FMT_FP8_BLOCK128 || (nv && shared->format == FFMOE_FMT_NVFP4), FFMOE_ERR_UNSUPPORTED,
+                 "with FP8 activations the shared expert is FFMOE_FMT_FP8_BLOCK128, or FFMOE_FMT_NVFP4 next to NVFP4 experts (format %d)", shared->format);
       FF_REQUIRE(SI >= 128 && SI % 128 == 0, FFMOE_ERR_SHAPE, "shared inter=%d must be a positive multiple of 128", SI);
     }
     FF_PTR16(args->shared_out);
@@ -699,11 +709,11 @@ int prefill_impl(const ffmoe_expert_table* table, const ffmoe_prefill* args, int
   uint8_t* s = (uint8_t*)args->scratch;
   PrefillBook b{(uint32_t*)(s + l.counts), (uint32_t*)(s + l.offsets), (uint32_t*)(s + l.gbase), (uint32_t*)(s + l.totals),
                 (int*)(s + l.perm), (GemmGroup*)(s + l.groups), (u32x2*)(s + l.units0), (u32x2*)(s + l.units1)};
-  const int mf = pick_mf(double(A) / E, (mx || a16) ? 4 : 8, !mx && !a16);
+  const int mf = nv ? 4 : pick_mf(double(A) / E, (mx || a16) ? 4 : 8, !mx && !a16);
   const int tm = 16 * mf;
   // W8A8, W*A16 and MX cohorts in 64-row groups: eight waves per block share a token tile (FFMOE_PREFILL_WIDE=0: four, two blocks per CU)
   bool wide = mf == 4;
-  if (const char* f = getenv("FFMOE_PREFILL_WIDE")) wide = wide && atoi(f) != 0;
+  if (const char* f = getenv("FFMOE_PREFILL_WIDE")) wide = (wide && atoi(f) != 0) || nv;
   const int tiles0 = wide ? (I + 255) / 256 : (I + 127) / 128, tiles1 = wide ? (H + 511) / 512 : (H + 255) / 256;
   // A shared expert of the routed experts' format and width rides in the routed launches as further row groups (W*A16
   // cohorts): on its own it is a few dozen blocks per launch, which at small cohorts take longer than the routed experts'
@@ -813,11 +823,12 @@ int prefill_impl(const ffmoe_expert_table* table, const ffmoe_prefill* args, int
   }
   GemmParams p{};
   p.slots = table->slots; p.groups = b.groups; p.perm = b.perm; p.top_k = K;
+  p.global_scales = nv ? table->global_scales : nullptr;
   p.swiglu = args->swiglu; p.limit = args->swiglu_limit; p.routed_weight = args->routed_weight; p.weights_f32 = args->weights_f32;
   if (stages & 2) {  // gate/up + SwiGLU
     p.a_codes = s + l.xq; p.a_scales = (const float*)(s + l.sx); p.units = b.units0; p.unit_total = b.totals + 0;
     p.out = (uint16_t*)(s + l.act); p.K = H; p.N = I;
-    FF_TRY(launch_gemm<0>(p, mf, wide ? blocks / 2 : blocks, stream, wide));
+    FF_TRY(launch_gemm<0>(p, mf, wide ? blocks / 2 : blocks, stream, wide, nv));
   }
   if (stages & 4) {  // re-quantize the activations of the live rows
     const long long cells = (long long)A * (I / 128);
@@ -828,32 +839,35 @@ int prefill_impl(const ffmoe_expert_table* table, const ffmoe_prefill* args, int
   if (stages & 8) {  // down x routing weight, scattered to contributions[assignment]
     p.a_codes = s + l.aq; p.a_scales = (const float*)(s + l.sa); p.units = b.units1; p.unit_total = b.totals + 1;
     p.out = (uint16_t*)args->contributions; p.done = args->done; p.weights = args->weights; p.K = I; p.N = H;
-    FF_TRY(launch_gemm<1>(p, mf, wide ? blocks / 2 : blocks, stream, wide));
+    FF_TRY(launch_gemm<1>(p, mf, wide ? blocks / 2 : blocks, stream, wide, nv));
   }
   if (shared) {
     // the always-on expert: the same three steps over all rows in their own order (no grouping, no routing weight),
     // as the reference runs it on the block-FP8 path (src/backend/cuda/moe/decode.rs:1187-1297)
-    const int smf = R > 32 ? 4 : R > 16 ? 2 : 1;
+    const bool snv = shared->format == FFMOE_FMT_NVFP4;  // its weights through the same conversion: 64-row groups, eight waves
+    const int smf = snv ? 4 : (R > 32 ? 4 : R > 16 ? 2 : 1);
     const int stm = 16 * smf;
     const uint32_t sgroups = uint32_t((R + stm - 1) / stm);
     GemmParams q{};
+    q.w0_global = shared->global_scales[0]; q.w1_global = shared->global_scales[1];
     q.rows_total = R; q.top_k = 1;
     q.swiglu = args->swiglu; q.limit = args->swiglu_limit;
     if (stages & 2) {
       q.a_codes = s + l.xq; q.a_scales = (const float*)(s + l.sx);
       q.w0_codes = shared->slot[0]; q.w0_scales = shared->slot[1]; q.w1_codes = shared->slot[2]; q.w1_scales = shared->slot[3];
-      q.total_units = sgroups * uint32_t((SI + 127) / 128);
+      q.total_units = sgroups * uint32_t(snv ? (SI + 255) / 256 : (SI + 127) / 128);
       q.out = (uint16_t*)(s + l.sh_act); q.K = H; q.N = SI;
-      FF_TRY(launch_gemm<0>(q, smf, std::min<unsigned>(blocks, (q.total_units + 7u) & ~7u), stream));
+      FF_TRY(launch_gemm<0>(q, smf, std::min<unsigned>(snv ? blocks / 2 : blocks, (q.total_units + 7u) & ~7u), stream, false, snv));
     }
     if (stages & 4)
       FF_TRY(ffmoe_quant_fp8_f32_128(s + l.sh_act, s + l.sh_aq, (float*)(s + l.sh_sa), R, SI, stream_));
     if (stages & 8) {
       q.a_codes = s + l.sh_aq; q.a_scales = (const float*)(s + l.sh_sa);
       q.w0_codes = shared->slot[4]; q.w0_scales = shared->slot[5]; q.w1_codes = 0; q.w1_scales = 0;
-      q.total_units = sgroups * uint32_t((H + 255) / 256);
+      q.w0_global = shared->global_scales[2];
+      q.total_units = sgroups * uint32_t(snv ? (H + 511) / 512 : (H + 255) / 256);
       q.out = (uint16_t*)args->shared_out; q.K = SI; q.N = H;
-      FF_TRY(launch_gemm<2>(q, smf, std::min<unsigned>(blocks, (q.total_units + 7u) & ~7u), stream));
+      FF_TRY(launch_gemm<2>(q, smf, std::min<unsigned>(snv ? blocks / 2 : blocks, (q.total_units + 7u) & ~7u), stream, false, snv));
     }
   }
   return 0;

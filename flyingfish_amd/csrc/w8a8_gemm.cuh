@@ -31,6 +31,8 @@ struct GemmParams {
   const uint8_t* a_codes;    // activation codes [*, K]
   const float* a_scales;     // activation scales [*, K/128]
   const uint64_t* slots;     // [E, 6] expert table, or NULL: the four addresses below
+  const float* global_scales;  // NVFP4 experts: [E, 3] f32 (gate, up, down), with slots
+  float w0_global, w1_global;  // NVFP4 experts without a table: the global scales of w0 / w1
   uint64_t w0_codes, w0_scales, w1_codes, w1_scales;  // MODE 0: gate, up; MODE 1/2: w0 only
   const GemmGroup* groups;   // NULL: rows split arithmetically into groups of TM (single matrix)
   const u32x2* units;       // (group, tile) per unit, or NULL with groups == NULL
@@ -53,7 +55,14 @@ __device__ __forceinline__ constexpr int gemm_tile_cols() { return (MODE == 0 ? 
 // weight stream, so a token tile that two blocks need is fetched twice (the fetch counters show every token read of a
 // cohort as an L2 miss, whatever the unit order); with NW = 8 one block per CU covers twice the columns per token tile
 // and the token traffic halves, at the same number of waves per CU as two blocks of four.
-template <int MF, int MODE, int P, int NW = 4>
+//
+// NV: the weights are NVFP4 (two E2M1 codes per byte, one E4M3 scale per 16 columns, an f32 per matrix). A fragment's
+// 16 rows x 128 columns are requested as 64 bytes of codes per row (four lanes) and the row's eight scale bytes, turned
+// into E4M3 on the way into the wave's transposition buffer - code value x scale / 8, rounded to nearest even, which
+// 6 x 448 / 8 = 336 keeps inside E4M3 - and from there on the kernel is the block-FP8 one with 8 x global as every
+// block's scale. That rounding is the arithmetic of this mode (a weight rounded twice, where the BF16-activation paths
+// round it once): its CPU restatement derives the same E4M3 codes and runs the block-FP8 W8A8 oracle on them.
+template <int MF, int MODE, int P, int NW = 4, bool NV = false>
 __global__ __launch_bounds__(64 * NW, (NW == 4 && MF <= 4) ? 2 : 1) void k_w8a8_grouped(const GemmParams p) {
   constexpr int TM = 16 * MF;
   constexpr int NT = 64 * NW;                       // threads per block
@@ -72,6 +81,7 @@ __global__ __launch_bounds__(64 * NW, (NW == 4 && MF <= 4) ? 2 : 1) void k_w8a8_
   // Short groups (MF < 4) are bound by HBM, not by the L1: they keep the direct requests and skip the LDS round trip.
   constexpr bool TW = MF >= 4;
   static_assert(!TW || P == 2, "the hand-counted waits of the long-group path assume two weight stages");
+  static_assert(!NV || MF == 4, "NVFP4 weights take the 64-row path, whose weights pass through LDS");
   __shared__ __attribute__((aligned(16))) uint8_t wstage[TW ? NW : 1][TW ? 4 : 1][TW ? 2048 : 16];  // [wave][fragment][16 rows x 128 B]
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = uni(tid >> 6);
@@ -121,6 +131,17 @@ __global__ __launch_bounds__(64 * NW, (NW == 4 && MF <= 4) ? 2 : 1) void k_w8a8_
       wc[0] = p.w0_codes; ws[0] = p.w0_scales;
       wc[1] = MODE == 0 ? p.w1_codes : p.w0_codes; ws[1] = MODE == 0 ? p.w1_scales : p.w0_scales;
     }
+    float nvg[2] = {1.0f, 1.0f};  // NV: 8 x the matrix's global scale stands in for every block scale
+    if constexpr (NV) {
+      if (p.slots) {
+        const float* gl = p.global_scales + size_t(expert) * 3;
+        nvg[0] = unif(load_global<float>(gl + (MODE == 0 ? 0 : 2)));
+        nvg[1] = MODE == 0 ? unif(load_global<float>(gl + 1)) : nvg[0];
+      } else {
+        nvg[0] = p.w0_global; nvg[1] = MODE == 0 ? p.w1_global : p.w0_global;
+      }
+      nvg[0] = __fmul_rn(nvg[0], 8.0f); nvg[1] = __fmul_rn(nvg[1], 8.0f);
+    }
     // first output column of fragment f; fragments past N are clamped onto the last 16 rows and dropped at the store
     int col0[4];
     // weight addresses: a wave-uniform base per fragment (scalar registers) and one byte offset per lane
@@ -130,16 +151,26 @@ __global__ __launch_bounds__(64 * NW, (NW == 4 && MF <= 4) ? 2 : 1) void k_w8a8_
       col0[f] = MODE == 0 ? t * (32 * NW) + wave * 32 + (f & 1) * 16 : t * (64 * NW) + wave * 64 + f * 16;
       const int base = min(col0[f], N - 16);
       const uint64_t codes = MODE == 0 ? wc[f >> 1] : wc[0];
-      wfrag[f] = uni64(codes + uint64_t(base) * uint64_t(K));
+      wfrag[f] = uni64(codes + uint64_t(base) * uint64_t(NV ? K >> 1 : K));
+    }
+    // NV: the scale bytes of the fragment's rows, [N, K / 16]
+    uint64_t sfrag[4] = {0, 0, 0, 0};
+    if constexpr (NV) {
+#pragma unroll
+      for (int f = 0; f < 4; ++f) sfrag[f] = uni64((MODE == 0 ? ws[f >> 1] : ws[0]) + uint64_t(min(col0[f], N - 16)) * uint64_t(K >> 4));
     }
     // long groups: 8 lanes per 128-byte row segment, rows 0..7 of the fragment (rows 8..15 with the second request);
     // short groups: operand order, 32 bytes of row lane % 16 as two requests
-    const uint32_t woff0 = TW ? uint32_t(lane >> 3) * uint32_t(K) + uint32_t(lane & 7) * 16u : uint32_t(lane & 15) * uint32_t(K) + uint32_t(lane >> 4) * 32u;
-    const uint32_t woff1 = woff0 + (TW ? 8u * uint32_t(K) : 16u);
+    // NV: four lanes per row of 64 code bytes, 16 rows per request; a lane's two scale bytes sit in the dword its pair shares
+    const uint32_t woff0 = NV ? uint32_t(lane >> 2) * uint32_t(K >> 1) + uint32_t(lane & 3) * 16u
+                              : TW ? uint32_t(lane >> 3) * uint32_t(K) + uint32_t(lane & 7) * 16u : uint32_t(lane & 15) * uint32_t(K) + uint32_t(lane >> 4) * 32u;
+    const uint32_t woff1 = NV ? uint32_t(lane >> 2) * uint32_t(K >> 4) + uint32_t((lane & 3) >> 1) * 4u : woff0 + (TW ? 8u * uint32_t(K) : 16u);
+    const int nv_wr = ((lane >> 2) & 7) * 128 + (lane >> 5) * 1024;  // NV: this lane's row of the fragment in the buffer
+    const int nv_key = (lane >> 2) & 7, nv_piece = (lane & 3) * 2;
     // block-scale rows: one per wave (its fragments sit inside one 128-row block), lane l keeps K block l (+64)
     const int srow = min(MODE == 0 ? t * (32 * NW) + wave * 32 : t * (64 * NW) + wave * 64, N - 16) >> 7;
-    const float* sw0 = reinterpret_cast<const float*>(ws[0]) + size_t(srow) * KB;
-    const float* sw1 = reinterpret_cast<const float*>(ws[1]) + size_t(srow) * KB;
+    const float* sw0 = reinterpret_cast<const float*>(NV ? uint64_t(p.a_scales) : ws[0]) + (NV ? 0 : size_t(srow) * KB);  // NV: any readable floats, never used
+    const float* sw1 = reinterpret_cast<const float*>(NV ? uint64_t(p.a_scales) : ws[1]) + (NV ? 0 : size_t(srow) * KB);
 
     // token rows this thread stages
     const uint8_t* tsrc[CPT];
@@ -190,14 +221,43 @@ __global__ __launch_bounds__(64 * NW, (NW == 4 && MF <= 4) ? 2 : 1) void k_w8a8_
     // prologue: weight fragments of the first P K blocks, token tile 0 into LDS, everything landed, then token tile 1
     // (and for short groups the last weight stage once more, so that tile 1 too has eight loads behind it).
     u32x4 w[P][4][2];
+    float wsc[P][4];  // NV: the dword with the lane's scale bytes (w[..][1] stays unused)
 #define FF_REQUEST_WEIGHTS(s_, kb_, f_)                                   \
   do {                                                                     \
-    load16_async(w[s_][f_][0], wfrag[f_] + (kb_) * 128u, woff0);           \
-    load16_async(w[s_][f_][1], wfrag[f_] + (kb_) * 128u, woff1);           \
+    if constexpr (NV) {                                                    \
+      load16_async(w[s_][f_][0], wfrag[f_] + (kb_) * 64u, woff0);          \
+      load4_async(wsc[s_][f_], sfrag[f_] + (kb_) * 8u, woff1);             \
+    } else {                                                               \
+      load16_async(w[s_][f_][0], wfrag[f_] + (kb_) * 128u, woff0);         \
+      load16_async(w[s_][f_][1], wfrag[f_] + (kb_) * 128u, woff1);         \
+    }                                                                      \
   } while (0)
 #define FF_DRAIN_WEIGHTS()                                                                                                  \
-  _Pragma("unroll") for (int s_ = 0; s_ < P; ++s_)                                                                          \
-      wait_loads<0>(w[s_][0][0], w[s_][0][1], w[s_][1][0], w[s_][1][1], w[s_][2][0], w[s_][2][1], w[s_][3][0], w[s_][3][1])
+  _Pragma("unroll") for (int s_ = 0; s_ < P; ++s_) {                                                                        \
+    if constexpr (NV) wait_loads<0>(w[s_][0][0], w[s_][1][0], w[s_][2][0], w[s_][3][0], wsc[s_][0], wsc[s_][1], wsc[s_][2], wsc[s_][3]); \
+    else wait_loads<0>(w[s_][0][0], w[s_][0][1], w[s_][1][0], w[s_][1][1], w[s_][2][0], w[s_][2][1], w[s_][3][0], w[s_][3][1]); \
+  }
+    // NV: a landed fragment piece (32 codes and their two scale bytes) as 32 E4M3 bytes into the transposition buffer
+    auto nv_store = [&](uint8_t* frag_base, const u32x4& codes, float scale_word) {
+      const uint32_t sb = __float_as_uint(scale_word) >> (16 * (lane & 1));
+      const f32x2 sc = e4m3x2_to_f32<false>(sb);
+      const float s2[2] = {__fmul_rn(sc.x, 0.125f), __fmul_rn(sc.y, 0.125f)};
+      uint32_t o[8];
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {
+        const float sg = s2[d >> 1];
+        int lo = 0, hi = 0;
+        const f32x2 v0 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(codes[d], 1.0f, 0), v1 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(codes[d], 1.0f, 1);
+        const f32x2 v2 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(codes[d], 1.0f, 2), v3 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(codes[d], 1.0f, 3);
+        lo = __builtin_amdgcn_cvt_pk_fp8_f32(__fmul_rn(v0.x, sg), __fmul_rn(v0.y, sg), lo, false);
+        lo = __builtin_amdgcn_cvt_pk_fp8_f32(__fmul_rn(v1.x, sg), __fmul_rn(v1.y, sg), lo, true);
+        hi = __builtin_amdgcn_cvt_pk_fp8_f32(__fmul_rn(v2.x, sg), __fmul_rn(v2.y, sg), hi, false);
+        hi = __builtin_amdgcn_cvt_pk_fp8_f32(__fmul_rn(v3.x, sg), __fmul_rn(v3.y, sg), hi, true);
+        o[2 * d] = uint32_t(lo); o[2 * d + 1] = uint32_t(hi);
+      }
+      *reinterpret_cast<u32x4*>(frag_base + nv_wr + ((nv_piece ^ nv_key) << 4)) = u32x4{o[0], o[1], o[2], o[3]};
+      *reinterpret_cast<u32x4*>(frag_base + nv_wr + (((nv_piece + 1) ^ nv_key) << 4)) = u32x4{o[4], o[5], o[6], o[7]};
+    };
 #pragma unroll
     for (int s = 0; s < P; ++s) {
       const uint32_t kb = uint32_t(min(s, KB - 1));
@@ -225,8 +285,12 @@ __global__ __launch_bounds__(64 * NW, (NW == 4 && MF <= 4) ? 2 : 1) void k_w8a8_
         uint8_t* wl = &wstage[wave][0][0];
 #pragma unroll
         for (int f = 0; f < 4; ++f) {
-          *reinterpret_cast<u32x4*>(wl + f * 2048 + wr_off) = w[0][f][0];
-          *reinterpret_cast<u32x4*>(wl + f * 2048 + 1024 + wr_off) = w[0][f][1];
+          if constexpr (NV) {
+            nv_store(wl + f * 2048, w[0][f][0], wsc[0][f]);
+          } else {
+            *reinterpret_cast<u32x4*>(wl + f * 2048 + wr_off) = w[0][f][0];
+            *reinterpret_cast<u32x4*>(wl + f * 2048 + 1024 + wr_off) = w[0][f][1];
+          }
         }
 #pragma unroll
         for (int i = 0; i < CPT; ++i) tv[i] = u32x4{0u, 0u, 0u, 0u};
@@ -269,8 +333,8 @@ __global__ __launch_bounds__(64 * NW, (NW == 4 && MF <= 4) ? 2 : 1) void k_w8a8_
     }
     for (int kb0 = 0; kb0 < KB; kb0 += 64) {
       // block scales of K blocks kb0 .. kb0+63, one per lane; the next 64 are requested right away
-      const float swl0 = landed(swn0);
-      const float swl1 = MODE == 0 ? landed(swn1) : 0.0f;
+      const float swl0 = NV ? nvg[0] : landed(swn0);
+      const float swl1 = NV ? nvg[1] : (MODE == 0 ? landed(swn1) : 0.0f);
       if (kb0 + 64 < KB) {
         const int kl = min(kb0 + 64 + lane, KB - 1);
         swn0 = load_global<float>(sw0 + kl);
@@ -344,7 +408,11 @@ __global__ __launch_bounds__(64 * NW, (NW == 4 && MF <= 4) ? 2 : 1) void k_w8a8_
                   // of slot s^1 (K block kb+1) has the rest of its own stage's weight loads, this stage's token
                   // loads and this stage's weight loads so far behind it: CPT + 1 + 8 whichever piece it is
                   const uint32_t kw = uint32_t(min(kb + 2, KB - 1));
-                  if constexpr (MF == 4) {
+                  if constexpr (MF == 4 && NV) {
+                    FF_REQUEST_WEIGHTS(s, kw, m);
+                    wait_loads<CPT + 1 + 8>(w[o][m][0], wsc[o][m]);
+                    nv_store(wl + m * 2048, w[o][m][0], wsc[o][m]);
+                  } else if constexpr (MF == 4) {
                     FF_REQUEST_WEIGHTS(s, kw, m);
                     wait_loads<CPT + 1 + 8>(w[o][m][0], w[o][m][1]);
                     *reinterpret_cast<u32x4*>(wl + m * 2048 + wr_off) = w[o][m][0];
@@ -393,7 +461,8 @@ __global__ __launch_bounds__(64 * NW, (NW == 4 && MF <= 4) ? 2 : 1) void k_w8a8_
           } else {
             // a stage past the last K block: its registers still have (clamped) loads in flight and are about to be
             // requested into again; a register with a load in flight is never left unread
-            wait_loads<0>(w[s][0][0], w[s][0][1], w[s][1][0], w[s][1][1], w[s][2][0], w[s][2][1], w[s][3][0], w[s][3][1]);
+            if constexpr (NV) wait_loads<0>(w[s][0][0], w[s][1][0], w[s][2][0], w[s][3][0], wsc[s][0], wsc[s][1], wsc[s][2], wsc[s][3]);
+            else wait_loads<0>(w[s][0][0], w[s][0][1], w[s][1][0], w[s][1][1], w[s][2][0], w[s][2][1], w[s][3][0], w[s][3][1]);
             FF_WAIT_TOKENS(0);
           }
           // Short groups: request token tile kb+2 and K block kb+P of the weights into the slot just consumed. The

@@ -50,7 +50,8 @@ extern "C" {
 #define FFMOE_ACT_BF16         0  /* W8A16: w = bf16(e4m3(code) * scale), FP32 accumulate against BF16 activations
                                      (src/fp8.rs:138-140, src/cpu/expert_ffn.rs:592-679) */
 #define FFMOE_ACT_FP8_BLOCK128 1  /* W8A8: activations quantized per 128 to E4M3 with an f32 scale, per-128 dot then
-                                     one scale product (kernels/fp8_linear.cu:12-48, kernels/q38_contract.cuh:239-279) */
+                                     one scale product (kernels/fp8_linear.cu:12-48, kernels/q38_contract.cuh:239-279);
+                                     on NVFP4 tables W4A8: the weights rounded to E4M3 first (ffmoe_prefill_contribute) */
 #define FFMOE_ACT_E4M3_E8M0_32  2  /* activations quantized per 32 to E4M3 with a power-of-two (E8M0) scale, exact integer dots
                                      (ffmoe_decode_contribute_e8m0 only) */
 #define FFMOE_ACT_E4M3_E8M0_32_F32 3  /* the same quantizer with the FP32 fma chains and 32-lane order of the reference's
@@ -442,7 +443,14 @@ int ffmoe_combine_residual(const void* contributions, const void* routed_in, con
  * kernels/moe_ffn.cu:870-908), which is how the reference runs block-FP8 prefill (in 16-row chunks).
  * Replaces PrefillOps::prefill_contribute (src/backend/cuda/moe/prefill.rs:1033-1408) and kernels moe_count_scan /
  * moe_permute / moe_gemm_* / silu_mul / moe_scatter_rows (kernels/moe_prefill.cu:364-553).
- * That is act_mode FFMOE_ACT_FP8_BLOCK128 (W8A8): FFMOE_FMT_FP8_BLOCK128 tables only, hidden and inter multiples of 128.
+ * That is act_mode FFMOE_ACT_FP8_BLOCK128 (W8A8) on FFMOE_FMT_FP8_BLOCK128 tables, hidden and inter multiples of 128.
+ * The same act_mode on an FFMOE_FMT_NVFP4 table is W4A8 on the FP8 matrix cores: the kernels turn every NVFP4 weight
+ * into E4M3 on its way through LDS - E2M1 value x E4M3 group scale / 8, rounded to nearest even (6 x 448 / 8 = 336 stays
+ * inside E4M3) - and use 8 x the matrix's f32 global scale where a block-FP8 matrix has its 128 x 128 scales; everything
+ * else (activation quantizer, per-128 dots, SwiGLU, re-quantization, routing weight) is the W8A8 pipeline above. The
+ * second rounding of the weights makes this an arithmetic of its own (the reference's NVFP4 GEMM dequantizes to BF16,
+ * kernels/nvfp4_linear.cu:262-573, and has no FP8 form): results equal, bit for bit, a block-FP8 cohort on those derived
+ * codes. The shared expert may be FFMOE_FMT_FP8_BLOCK128 or FFMOE_FMT_NVFP4 then.
  * act_mode FFMOE_ACT_BF16 runs the cohort in the decode path's W*A16 arithmetic instead: experts of any format
  * (block FP8, NVFP4, per-channel FP8, BF16; the shared expert may have another format than the table) are
  * dequantized in registers to the BF16 effective weights of ffmoe_decode_contribute, activations stay BF16 between

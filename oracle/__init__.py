@@ -146,6 +146,18 @@ def dequant_nvfp4(codes, scales, global_scale):
     return out
 
 
+def nvfp4_to_fp8_block(codes, scales, global_scale):
+    """NVFP4 matrix -> (E4M3 codes [n, k], f32 block scales [n / 128, k / 128]) of the W4A8 mode: every weight rounded to
+    E4M3 as e2m1 x e4m3(scale) / 8, every 128 x 128 block scaled by 8 x global."""
+    c = _c(codes, np.uint8)
+    s = _c(scales, np.uint8)
+    n, k2 = c.shape
+    k = k2 * 2
+    out = np.empty((n, k), dtype=np.uint8)
+    lib().orc_nvfp4_to_e4m3(_p(c), _p(s), n, k, _p(out))
+    return out, np.full(((n + 127) // 128, (k + 127) // 128), np.float32(global_scale) * np.float32(8.0), dtype=np.float32)
+
+
 def quant_weight_fp8_block(w, bn=128, bk=128):
     w = _c(w, np.float32)
     n, k = w.shape

@@ -20,6 +20,8 @@
 //   * E8M0 block-32 contract: activation quantizer, exact
 //     integer dot, repaired BF16 rounding ................... pinned (closed forms, rational arithmetic, tie witness)
 //   * combine variants ...................................... pinned (order-spread constants of the fixture)
+//   * NVFP4 weights re-rounded to E4M3 (W4A8 mode) .......... pinned as a function (rational arithmetic + brute-force nearest
+//     code); the mode itself is this build's definition, the reference has no FP8 form of NVFP4
 //   * expert FFN composed over 128x128-f32 block scales or
 //     NVFP4 weights, grouped routing with n_group > 1,
 //     FP32-logit dot order, last-bit behaviour of expf / tanhf parity unpinned (no reference code or vectors)
@@ -315,6 +317,20 @@ ORC_API void orc_dequant_nvfp4(const uint8_t* codes, const uint8_t* scales, floa
       const uint8_t nib = (c & 1) ? uint8_t(b >> 4) : uint8_t(b & 15u);
       const float s = decode_e4m3(scales[size_t(r) * (k / 16) + c / 16]) * global;
       out[size_t(r) * k + c] = bf16_rne(decode_e2m1(nib) * s);
+    }
+}
+
+// NVFP4 weights as the FP8 matrix cores take them in the W4A8 mode (FP8 activations on NVFP4 experts; the reference's
+// MMA path for NVFP4 dequantizes to BF16 instead, kernels/nvfp4_linear.cu:262-573, and has no FP8 form): each weight is
+// rounded to E4M3 once more, code value x group scale / 8 (6 x 448 / 8 = 336 stays inside E4M3's 448), nearest even by
+// the reference's own encoder (src/fp8.rs:85-121), and 8 x the matrix's global scale is every 128 x 128 block's scale.
+// Defined by this build; the derived codes then go through the block-FP8 W8A8 arithmetic above the reference defines.
+ORC_API void orc_nvfp4_to_e4m3(const uint8_t* codes, const uint8_t* scales, int n, int k, uint8_t* out) {
+  for (int r = 0; r < n; ++r)
+    for (int c = 0; c < k; ++c) {
+      const uint8_t b = codes[size_t(r) * (k / 2) + c / 2];
+      const uint8_t nib = (c & 1) ? uint8_t(b >> 4) : uint8_t(b & 15u);
+      out[size_t(r) * k + c] = encode_e4m3(decode_e2m1(nib) * decode_e4m3(scales[size_t(r) * (k / 16) + c / 16]) * 0.125f);
     }
 }
 

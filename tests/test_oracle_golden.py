@@ -871,3 +871,40 @@ def test_w8a8_one_step_gate_differences_amplify_end_to_end():
         o1 = np.stack([orc.expert_down_w8a8(a1[r], d, sd, 0.5) for r in range(R)])
         spread[frac] = orc.rel_l2(o1, o0)
     assert 1e-3 < spread[0.005] < spread[0.06] < 5e-2, spread
+
+
+def test_nvfp4_weights_re_rounded_to_e4m3_against_rational_arithmetic():
+    """The W4A8 mode's weight: e4m3_rne(e2m1 x e4m3(scale) / 8). Every (code, scale code) pair against exact rational
+    arithmetic and a brute-force search for the nearest E4M3 value (ties to the even code); both zero codes give +0; the
+    largest product, 6 x 448 / 8 = 336, is a tie that goes to 320, inside E4M3's 448; where the product is representable it comes back exactly."""
+    from fractions import Fraction
+    e4m3 = {}
+    for c in range(256):
+        if (c & 0x7f) == 0x7f:
+            continue
+        m, e, sgn = c & 7, (c >> 3) & 15, -1 if c & 0x80 else 1
+        e4m3[c] = sgn * (Fraction(m, 512) if e == 0 else Fraction(8 + m, 8) * Fraction(2) ** (e - 7))
+    mags = [Fraction(0), Fraction(1, 2), Fraction(1), Fraction(3, 2), Fraction(2), Fraction(3), Fraction(4), Fraction(6)]
+    positive = sorted((v, c) for c, v in e4m3.items() if c < 0x80)
+    scale_codes = [c for c in range(256) if (c & 0x7f) != 0x7f and c < 0x80]   # NVFP4 scales are non-negative
+    codes = np.zeros((1, 8), dtype=np.uint8)
+    largest = Fraction(0)
+    for sc in scale_codes:
+        for lo in range(16):
+            codes[0, :] = lo | (((lo + 5) % 16) << 4)
+            got = orc.nvfp4_to_fp8_block(codes, np.array([[sc]], dtype=np.uint8), 1.0)[0][0]
+            for nib, g in ((lo, int(got[0])), ((lo + 5) % 16, int(got[1]))):
+                exact = mags[nib & 7] * e4m3[sc] / 8
+                best = min(positive, key=lambda vc: (abs(vc[0] - exact), vc[1] & 1))   # nearest, ties to the even code
+                want = best[1] | (0x80 if (nib & 8) and exact != 0 and best[0] != 0 else 0)
+                if (nib & 7) == 0:
+                    want = 0
+                elif best[0] == 0 and (nib & 8):
+                    want = 0x80   # a negative value that underflows keeps its sign, as the reference's encoder does
+                assert g == want, (sc, nib, g, want, float(exact))
+                largest = max(largest, abs(e4m3[g]))
+                if exact in e4m3.values():
+                    assert e4m3[g] == (-exact if nib & 8 else exact)
+    assert largest == 320
+    block = orc.nvfp4_to_fp8_block(np.zeros((130, 192), dtype=np.uint8), np.full((130, 24), 0x38, dtype=np.uint8), 0.25)[1]
+    assert block.shape == (2, 3) and np.all(block == np.float32(2.0))
