@@ -68,7 +68,11 @@ def test_decode_contract_violations_are_reported_before_launch():
     assert call(contributions=1 << 20) == capi.ERR_OVERLAP
     assert call(act_mode=2) == capi.ERR_UNSUPPORTED
     nv = capi.ExpertTable(capi.FMT_NVFP4, 64, 2048, 1408, 16 << 20, None, 32 << 20)
-    assert call(t=nv, act_mode=1) == capi.ERR_UNSUPPORTED  # the W8A8 path takes FP8 block experts only
+    # FP8 activations run on block-FP8 experts (W8A8) and NVFP4 experts (W4A8, which needs the global scales), not on BF16 ones
+    bf = capi.ExpertTable(capi.FMT_BF16, 64, 2048, 1408, 16 << 20, None, None)
+    assert call(t=bf, act_mode=1) == capi.ERR_UNSUPPORTED
+    nv_no_globals = capi.ExpertTable(capi.FMT_NVFP4, 64, 2048, 1408, 16 << 20, None, None)
+    assert call(t=nv_no_globals, act_mode=1) == capi.ERR_NULL
     assert call(swiglu=2, swiglu_limit=0.0) == capi.ERR_SHAPE
     assert call(swiglu=7) == capi.ERR_UNSUPPORTED
     bad = capi.ExpertTable(capi.FMT_FP8_BLOCK128, 64, 2000, 1408, 16 << 20, None, None)
@@ -110,7 +114,11 @@ def test_prefill_contract_violations_are_reported_before_launch():
     assert L.ffmoe_prefill_contribute(None, None, None) == capi.ERR_NULL
     assert call(act_mode=capi.ACT_E4M3_E8M0_32) == capi.ERR_UNSUPPORTED
     nv = capi.ExpertTable(capi.FMT_NVFP4, 64, 2048, 1280, 16 << 20, None, 32 << 20)
-    assert call(t=nv) == capi.ERR_UNSUPPORTED and "matrix cores" in capi.last_error()  # W8A8 takes block-FP8 experts only
+    bf = capi.ExpertTable(capi.FMT_BF16, 64, 2048, 1280, 16 << 20, None, None)
+    assert call(t=bf) == capi.ERR_UNSUPPORTED and "matrix cores" in capi.last_error()  # FP8 activations: block-FP8 (W8A8) or NVFP4 (W4A8) experts
+    assert call(t=capi.ExpertTable(capi.FMT_NVFP4, 64, 2048, 1280, 16 << 20, None, None)) == capi.ERR_NULL  # W4A8 needs the global scales
+    bf_shared = capi.SharedExpert(capi.FMT_BF16, 1280)
+    assert call(t=nv, shared=ctypes.pointer(bf_shared), shared_out=512 << 20) == capi.ERR_UNSUPPORTED  # no BF16 shared expert next to FP8 activations
     nv_bare = capi.ExpertTable(capi.FMT_NVFP4, 64, 2048, 1280, 16 << 20, None, None)
     assert call(t=nv_bare, act_mode=capi.ACT_BF16) == capi.ERR_NULL   # W4A16 prefill: the table must bring its global scales
     odd16 = capi.ExpertTable(capi.FMT_BF16, 64, 2048 + 32, 1280, 16 << 20, None, None)
