@@ -16,6 +16,7 @@ bool decode_gate_up_nvfp4_bf16_shared_available(int hidden);
 int decode_gate_up_nvfp4_bf16_shared(const DecodeParams& p, hipStream_t st);
 int decode_finish_fp8(const FinishParams& q, hipStream_t st);
 int decode_finish_nvfp4(const FinishParams& q, hipStream_t st);
+int decode_finish_nvfp4_bf16_shared(const FinishParams& q, hipStream_t st);
 int decode_finish_bf16(const FinishParams& q, hipStream_t st);
 int decode_finish_fp8c(const FinishParams& q, hipStream_t st);
 int decode_token_layer_fp8(const FinishParams& q, hipStream_t st);
@@ -161,7 +162,7 @@ extern "C" __attribute__((visibility("default"))) uint64_t ffmoe_decode_scratch_
 static int decode_impl(const ffmoe_expert_table* table, const ffmoe_shared_expert* shared, const ffmoe_decode* args,
                        int stage_mask, void* stream, int layout_k = -1, int pass = 0, const FinishParams* fin = nullptr,
                        const RouteInline* route = nullptr, int form = -1, int arena_shared_inter = 0, bool mixed_gate_up = false,
-                       bool finish_record = false) {
+                       bool finish_record = false, bool mixed_finish = false) {
   FF_REQUIRE(table && args, FFMOE_ERR_NULL, "table/args is NULL");
   const int R = args->rows, K = args->top_k, E = table->experts, H = table->hidden, I = table->inter;
   const int LK = layout_k < 0 ? K : layout_k;
@@ -193,7 +194,9 @@ static int decode_impl(const ffmoe_expert_table* table, const ffmoe_shared_exper
   int SI = I;
   if (shared) {
     // mixed_gate_up: NVFP4 experts and a BF16 shared expert in one gate/up launch (one token, selection in the prologue)
-    FF_REQUIRE(shared->format == fmt || (mixed_gate_up && fmt == FFMOE_FMT_NVFP4 && shared->format == FFMOE_FMT_BF16 && route && stage_mask == 1),
+    // mixed_finish: the same pair in the one-token finish launch
+    FF_REQUIRE(shared->format == fmt || (mixed_gate_up && fmt == FFMOE_FMT_NVFP4 && shared->format == FFMOE_FMT_BF16 && route && stage_mask == 1) ||
+                   (mixed_finish && fmt == FFMOE_FMT_NVFP4 && shared->format == FFMOE_FMT_BF16 && fin && !fin->whole && R == 1),
                FFMOE_ERR_UNSUPPORTED, "shared expert format %d differs from the table format %d", shared->format, fmt);
     SI = shared->inter;
     FF_REQUIRE(SI >= gran && SI % gran == 0, FFMOE_ERR_SHAPE, "shared inter=%d must be a positive multiple of %d", SI, gran);
@@ -309,6 +312,7 @@ static int decode_impl(const ffmoe_expert_table* table, const ffmoe_shared_exper
         default: return decode_token_layer_bf16(q, st);
       }
     }
+    if (mixed_finish) return decode_finish_nvfp4_bf16_shared(q, st);
     switch (fmt) {
       case FFMOE_FMT_FP8_BLOCK128: return decode_finish_fp8(q, st);
       case FFMOE_FMT_NVFP4: return decode_finish_nvfp4(q, st);
@@ -588,6 +592,14 @@ static int token_forward(const ffmoe_expert_table* table, const ffmoe_shared_exp
     // value, rounded at the same boundary. The selection runs in the prologue of the shared expert's gate/up launch
     // (wave 0 of every block, next to the three waves that stream the shared rows), so the routed gate/up launch starts
     // with its ids in memory. Five launches per layer with the logits instead of seven.
+    // NVFP4 experts and a BF16 shared expert of their width: the finish launch streams the shared expert's down rows too, in
+    // BF16, as every wave's first units - three launches with the logits (FFMOE_DECODE_MIXED_FINISH=0: four)
+    const char* mf = getenv("FFMOE_DECODE_MIXED_FINISH");
+    const char* mg = getenv("FFMOE_DECODE_MIXED_GATE_UP");
+    const int sh_steps = (sh->inter / 8 + 63) / 64;
+    const bool finish_shared = table->format == FFMOE_FMT_NVFP4 && sh->format == FFMOE_FMT_BF16 && sh->inter == table->inter &&
+                               table->inter <= 2048 && (sh_steps == 1 || sh_steps == 2 || sh_steps == 4) && !(mf && atoi(mf) == 0) &&
+                               !(mg && atoi(mg) == 0) && decode_gate_up_nvfp4_bf16_shared_available(table->hidden);
     if (stage_mask & 1) {
       ffmoe_expert_table as_shared = *table;
       as_shared.format = sh->format;
@@ -603,7 +615,7 @@ static int token_forward(const ffmoe_expert_table* table, const ffmoe_shared_exp
         // the shared expert's gate/up rows as every block's first slice of the routed gate/up launch, in BF16, next to the
         // selection; only its down launch is its own: four launches with the logits (FFMOE_DECODE_MIXED_GATE_UP=0: five)
         FF_TRY(decode_impl(table, sh, args, 1, stream, K, 0, nullptr, &route, -1, sh->inter, true));
-        FF_TRY(decode_impl(&as_shared, sh, &only_shared, 2, stream, K, 1));
+        if (!finish_shared) FF_TRY(decode_impl(&as_shared, sh, &only_shared, 2, stream, K, 1));
       } else {
         RouteInline select = route;
         select.select_k = K;
@@ -611,7 +623,9 @@ static int token_forward(const ffmoe_expert_table* table, const ffmoe_shared_exp
         FF_TRY(decode_impl(table, nullptr, args, 1, stream, K, 0, nullptr, nullptr, -1, sh->inter));
       }
     }
-    if (stage_mask & 2) {
+    if ((stage_mask & 2) && finish_shared) {
+      FF_TRY(decode_impl(table, sh, args, 0, stream, K, 0, &fin, nullptr, -1, sh->inter, false, false, true));
+    } else if (stage_mask & 2) {
       FF_PTR16(args->shared_out);
       FF_NO_OVERLAP(y, size_t(table->hidden) * 2, args->shared_out, size_t(table->hidden) * 2);
       fin.shared_ready = (const uint16_t*)args->shared_out;

@@ -5,6 +5,8 @@
 namespace ffmoe {
 int decode_launch_nvfp4(const DecodeParams& p, int rg, int stage_mask, hipStream_t st) { return launch_format<FmtNvfp4>(p, rg, stage_mask, st); }
 int decode_finish_nvfp4(const FinishParams& q, hipStream_t st) { return launch_finish<FmtNvfp4>(q, st); }
+// the same with a BF16 shared expert, whose down rows the finish streams in their own format
+int decode_finish_nvfp4_bf16_shared(const FinishParams& q, hipStream_t st) { return launch_finish<FmtNvfp4>(q, st, true); }
 int decode_token_layer_nvfp4(const FinishParams& q, hipStream_t st) { return launch_token_layer<FmtNvfp4>(q, st); }
 
 // One token, NVFP4 routed experts next to a BF16 shared expert: the gate/up launch with the selection in its prologue

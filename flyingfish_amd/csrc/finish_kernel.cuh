@@ -23,7 +23,10 @@ namespace ffmoe {
 
 // MAXT: the largest block the instantiation is launched with. Blocks of eight waves (the usual shape) are compiled for two
 // waves per SIMD, i.e. with the whole register file of 256 registers per lane; 12 and 16 waves need the 128-register build.
-template <class F, int S, int NR, int MAXT = 1024>
+// FSH / SSH: format and steps per row of the shared expert's down matrix when they differ from the routed experts' (a BF16
+// shared expert next to NVFP4 experts): its units are every wave's first units, streamed and multiplied in their own
+// format, so such a shared expert needs no down launch of its own.
+template <class F, int S, int NR, int MAXT = 1024, class FSH = F, int SSH = S>
 __global__ __launch_bounds__(MAXT) void k_decode_finish(const FinishParams q, const int cmax) {
   const DecodeParams& p = q.d;
   constexpr int GT = FFMOE_FINISH_GROUPS;
@@ -54,7 +57,20 @@ __global__ __launch_bounds__(MAXT) void k_decode_finish(const FinishParams q, co
   // 28.5 against 27.0 us, more requests in flight than the memory system takes; NVFP4: 24.1 against 22.1 us, its units
   // are bound by the conversion work, not by requests in flight).
   constexpr int NB = 1;
+  constexpr bool MIXED = !std::is_same<F, FSH>::value;
   typename F::Chunk buf[NB][NR][S];
+  typename FSH::Chunk sbuf[MIXED ? NR : 1][MIXED ? SSH : 1];  // MIXED: the shared expert's unit in flight
+  const int nchunks_sh = I / FSH::EPL;
+  auto issue_shared_rows = [&](int i, int s) {  // MIXED: step s of the shared expert's unit i
+    const int j = b_lo + i * NR;
+    const int chunk = s * 64 + lane;
+    const int cc = chunk < nchunks_sh ? chunk : nchunks_sh - 1;
+#pragma unroll
+    for (int m = 0; m < NR; ++m) {
+      const int row = j + m < b_hi ? j + m : b_hi - 1;
+      FSH::load(sbuf[MIXED ? m : 0][MIXED ? s : 0], FSH::row(uni64(p.shared_slot[4]), uni64(p.shared_slot[5]), unif(p.shared_global[2]), row, I), cc);
+    }
+  };
   auto issue_rows = [&](auto which, uint64_t codes, uint64_t scales, float glob, int i, int s) {
     constexpr int b_ = decltype(which)::value;
     const int j = b_lo + i * NR;
@@ -73,8 +89,13 @@ __global__ __launch_bounds__(MAXT) void k_decode_finish(const FinishParams q, co
   // anything else, so the first weights are on their way while the block finds out which experts were chosen.
   const bool first_shared = has_shared && wave < P;
   if (first_shared) {
+    if constexpr (MIXED) {
 #pragma unroll
-    for (int s = 0; s < S; ++s) issue_rows(B0{}, uni64(p.shared_slot[4]), uni64(p.shared_slot[5]), unif(p.shared_global[2]), wave, s);
+      for (int s = 0; s < SSH; ++s) issue_shared_rows(wave, s);
+    } else {
+#pragma unroll
+      for (int s = 0; s < S; ++s) issue_rows(B0{}, uni64(p.shared_slot[4]), uni64(p.shared_slot[5]), unif(p.shared_global[2]), wave, s);
+    }
   }
   // Activations: row c of the arena belongs to choice c, row K to the shared expert, whichever experts were chosen, so
   // all K + 1 rows are requested right here, in front of everything that depends on the ids, and go to LDS in arena
@@ -195,9 +216,9 @@ __global__ __launch_bounds__(MAXT) void k_decode_finish(const FinishParams q, co
     issue_rows(which, uni64(s_codes[g]), uni64(s_scales[g]), unif(s_glob[g]), i, s);
   };
   if (my_units > 0) {
-    if (!first_shared) {
+    if (!first_shared || (MIXED && my_units > lead)) {  // MIXED: the first routed unit goes out next to the shared ones, into its own registers
 #pragma unroll
-      for (int s = 0; s < S; ++s) issue_unit(B0{}, 0, s);
+      for (int s = 0; s < S; ++s) issue_unit(B0{}, MIXED ? lead : 0, s);
     }
     if constexpr (NB == 2) {
 #pragma unroll
@@ -206,7 +227,7 @@ __global__ __launch_bounds__(MAXT) void k_decode_finish(const FinishParams q, co
   }
   // NVFP4: the split dot's constants of every group's down matrix; then the activations, which were requested first
   if constexpr (NV) {
-    for (int g = 0; g < G; ++g) FmtNvfp4::build_lut(s_lut + g * FmtNvfp4::LUT_ENTRIES, s_glob[g], tid, nthreads);
+    for (int g = 0; g < (MIXED ? nr : G); ++g) FmtNvfp4::build_lut(s_lut + g * FmtNvfp4::LUT_ENTRIES, s_glob[g], tid, nthreads);
   }
   stage_activations();
   __syncthreads();
@@ -232,7 +253,31 @@ __global__ __launch_bounds__(MAXT) void k_decode_finish(const FinishParams q, co
         if (i * NR + m < C) s_part[g * cmax + i * NR + m] = total[m];
     }
   };
-  for (int t = 0; t < my_units; t += NB) {
+  int t_first = 0;
+  if constexpr (MIXED) {
+    // the shared expert's units of this wave in their own format; the first routed unit is already on its way
+    for (int t = 0; t < lead; ++t) {
+      const int i = wave + t * nw;
+      float acc[NR][1];
+#pragma unroll
+      for (int m = 0; m < NR; ++m) acc[m][0] = 0.0f;
+#pragma unroll
+      for (int s = 0; s < SSH; ++s) {
+        step_compute<FSH, NR, 1, SSH, false>(sbuf, s, xs + size_t(K) * I * 2, I, nchunks_sh, s * 64 + lane, 1, acc);
+        if (t + 1 < lead) issue_shared_rows(i + nw, s);
+      }
+      float total[NR];
+#pragma unroll
+      for (int m = 0; m < NR; ++m) total[m] = wave_sum(acc[m][0]);
+      if (lane == 0) {
+#pragma unroll
+        for (int m = 0; m < NR; ++m)
+          if (i * NR + m < C) s_part[nr * cmax + i * NR + m] = total[m];
+      }
+    }
+    t_first = lead;
+  }
+  for (int t = t_first; t < my_units; t += NB) {
     unit(B0{}, t);
     if constexpr (NB == 2) {
       if (t + 1 < my_units) unit(B1{}, t + 1);
@@ -262,6 +307,12 @@ __global__ __launch_bounds__(MAXT) void k_decode_finish(const FinishParams q, co
     }
     q.y[b_lo + col] = f32_to_bf16(v);
   }
+}
+
+// NVFP4 routed experts next to a BF16 shared expert of the same width: steps per row are (S, SSH) = (inter / 2048, inter / 512)
+template <int S, int SSH>
+void launch_finish_mixed(const FinishParams& q, int blocks, int threads, int cmax, size_t lds, hipStream_t st) {
+  hipLaunchKernelGGL((k_decode_finish<FmtNvfp4, S, 4, 512, FmtBf16, SSH>), dim3(blocks), dim3(threads), lds, st, q, cmax);
 }
 
 template <class F, int NR, int SMAX, int S = 1>
@@ -295,9 +346,12 @@ inline void finish_shape(int columns, int groups, int nr_rows, int cus, int* blo
 // Returns FFMOE_ERR_UNSUPPORTED when the shape is outside what the kernel holds in registers; the caller then runs the
 // separate down and combine launches.
 template <class F>
-int launch_finish(const FinishParams& q, hipStream_t st) {
+int launch_finish(const FinishParams& q, hipStream_t st, bool bf16_shared = false) {
   const DecodeParams& p = q.d;
   const int steps = (p.inter / F::EPL + 63) / 64;
+  const int steps_sh = (p.inter / FmtBf16::EPL + 63) / 64;
+  if (bf16_shared && !(std::is_same<F, FmtNvfp4>::value && steps == 1 && (steps_sh == 1 || steps_sh == 2 || steps_sh == 4) && p.shared_inter == p.inter))
+    return ff_fail(FFMOE_ERR_UNSUPPORTED, "one-token finish with a BF16 shared expert: NVFP4 experts of the same width, at most 2048 columns (inter=%d)", p.inter);
   if (steps > 2 || p.top_k > FFMOE_FINISH_GROUPS - 1)
     return ff_fail(FFMOE_ERR_UNSUPPORTED, "one-token finish holds at most %d routed groups and 2 steps per row (top_k=%d, steps=%d)",
                    FFMOE_FINISH_GROUPS - 1, p.top_k, steps);
@@ -314,6 +368,15 @@ int launch_finish(const FinishParams& q, hipStream_t st) {
   const size_t lds = size_t(FFMOE_FINISH_GROUPS) * p.inter * 2 + size_t(FFMOE_FINISH_GROUPS) * cmax * 4;
   const size_t tables = std::is_same<F, FmtNvfp4>::value ? size_t(FFMOE_FINISH_GROUPS) * FmtNvfp4::LUT_ENTRIES * 8 : 0;  // static, next to lds
   if (lds + tables + 512 > 64 * 1024) return ff_fail(FFMOE_ERR_UNSUPPORTED, "one-token finish: %zu bytes of LDS per block", lds + tables);
+  if (bf16_shared) {
+    if constexpr (std::is_same<F, FmtNvfp4>::value) {
+      waves = 8;  // the instantiation is built for eight-wave blocks
+      if (steps_sh == 4) launch_finish_mixed<1, 4>(q, blocks, waves * 64, cmax, lds, st);
+      else if (steps_sh == 2) launch_finish_mixed<1, 2>(q, blocks, waves * 64, cmax, lds, st);
+      else launch_finish_mixed<1, 1>(q, blocks, waves * 64, cmax, lds, st);
+    }
+    return ff_launch_status();
+  }
   launch_finish_steps<F, NR, 2>(steps, q, blocks, waves * 64, cmax, lds, st);
   return ff_launch_status();
 }

@@ -911,12 +911,16 @@ def test_token_forward_two_launches_equal_the_separate_launches(fmt, hidden, int
 
 @pytest.mark.parametrize("fmt,shared_fmt,hidden,inter,shared_inter", [(capi.FMT_NVFP4, capi.FMT_BF16, 512, 256, 256), (capi.FMT_NVFP4, capi.FMT_BF16, 256, 512, 128),
                                                                      (capi.FMT_NVFP4, capi.FMT_BF16, 2048, 256, 384), (capi.FMT_NVFP4, capi.FMT_BF16, 4096, 128, 128),
+                                                                     (capi.FMT_NVFP4, capi.FMT_BF16, 2048, 1024, 1024), (capi.FMT_NVFP4, capi.FMT_BF16, 4096, 2048, 2048),
+                                                                     (capi.FMT_NVFP4, capi.FMT_BF16, 2048, 1536, 1536),
                                                                      (capi.FMT_FP8_BLOCK128, capi.FMT_BF16, 256, 256, 384), (capi.FMT_FP8_BLOCK128, capi.FMT_FP8_BLOCK128, 256, 256, 512)])
 @pytest.mark.parametrize("experts,n_group,topk_group,top_k", [(64, 1, 1, 3), (256, 8, 4, 8)])
 def test_token_forward_with_a_shared_expert_of_another_format_or_width(fmt, shared_fmt, hidden, inter, shared_inter, experts, n_group, topk_group, top_k):
     """ffmoe_decode_token_forward next to a shared expert that cannot share the routed launches (BF16 next to NVFP4 experts,
     or another width): the shared expert's own two launches leave its BF16 row in shared_out and the finish adds that row;
-    at hidden 2048 and 4096 a BF16 shared expert's gate/up rows run inside the NVFP4 gate/up launch, in BF16.
+    at hidden 2048 and 4096 a BF16 shared expert's gate/up rows run inside the NVFP4 gate/up launch, in BF16, and where its
+    width is the experts' (128, 1024 and 2048 columns here: one, two and four steps per BF16 row; 1536 is three, which keeps
+    the down launch) its down rows run inside the finish launch.
     ids, weights and y equal the separate launches bit for bit, for every combine mode, over consecutive tokens."""
     table = make_table(fmt, 4, hidden, inter, 171)[0]
     slots = table.slots[:4].repeat((experts + 3) // 4, 1)[:experts].contiguous()
