@@ -888,11 +888,13 @@ def decode_main(args, torch, capi, ops, synth, prebuilt=None):
     k_avg = sum(kt) / len(kt)
     mean_distinct_k = sum(distinct) / len(distinct)
     k_bytes = gate_up_bytes(table, mean_distinct_k, args.batch, dims)
-    # one token, shared expert in another format than the routed experts: stage 0 of the token path is three launches -
-    # the shared expert's gate/up (top-k selection in its prologue) and down, then the routed gate/up - so the shared
-    # expert's down matrix and its output row count here and not in the finish
+    # one token, NVFP4 experts next to a BF16 shared expert: the shared expert's rows ride in both launches in BF16 (gate/up
+    # rows as every block's first slice, down rows as every wave's first units of the finish), so the bytes split as for one
+    # format. With that switched off by the environment the shared expert's down launch is its own, in front of the routed
+    # gate/up, and its down matrix and output row count in stage 0.
     mixed_token = token_path and args.format == "nvfp4"
-    shared_down = table.shared_bytes // 3 + I * 2 + H * 2 if mixed_token else 0
+    own_down = mixed_token and (os.environ.get("FFMOE_DECODE_MIXED_FINISH") == "0" or os.environ.get("FFMOE_DECODE_MIXED_GATE_UP") == "0")
+    shared_down = table.shared_bytes // 3 + I * 2 + H * 2 if own_down else 0
     k_bytes += shared_down
     achieved = k_bytes / (k_avg * 1e-6) / 1e9
     # second streaming launch: down (+ routing weight; one token: + ordered combine)
@@ -900,7 +902,29 @@ def decode_main(args, torch, capi, ops, synth, prebuilt=None):
     dt = sorted(max(t - k_avg, 0.0) for t in dt)
     d_avg = sum(dt) / len(dt)
     d_bytes = (mean_distinct_k * table.weight_bytes_per_expert() + table.shared_bytes) // 3 + args.batch * (K + 1) * I * 2 + \
-        (args.batch * H * 2 if token_path else args.batch * (K + 1) * H * 2) - (shared_down - 2 * H * 2 if mixed_token else 0)  # mixed: the finish reads the shared row instead of a down matrix
+        (args.batch * H * 2 if token_path else args.batch * (K + 1) * H * 2) - (shared_down - 2 * H * 2 if own_down else 0)  # own down launch: the finish reads the shared row instead of a down matrix
+
+    fname = "FmtFp8" if args.format == "fp8" else "FmtNvfp4"
+    cohort = not token_path and args.batch >= 4 and not os.environ.get("FFMOE_DECODE_COHORT_ROWS")  # the library's default hand-over to the matrix cores
+    if mixed_token:
+        gate_up_kernel = ("ffmoe::k_decode_stage<FmtNvfp4, S, 0, 1, NR, FmtBf16, SSH> (gate/up + SwiGLU launch: the BF16 shared expert's rows as every "
+                          "block's first slice next to the top-k selection, then the NVFP4 rows%s)" % (
+                              "; with the shared expert's own BF16 down launch behind it" if own_down else ""))
+        down_kernel = ("ffmoe::k_decode_finish<FmtNvfp4, S, NR> (routed down + routing weight + ordered combine with the shared row)" if own_down else
+                       "ffmoe::k_decode_finish<FmtNvfp4, S, NR, 512, FmtBf16, SSH> (down of the BF16 shared expert and of the NVFP4 choices + routing weight + "
+                       "ordered combine)")
+    elif token_path:
+        gate_up_kernel = "ffmoe::k_decode_stage<%s, S, 0, 1, NR> (gate/up + SwiGLU launch, top-k selection in its prologue, as the layer issues it)" % fname
+        down_kernel = "ffmoe::k_decode_finish<%s, S, NR> (down + routing weight + ordered combine)" % fname
+    elif cohort:
+        lines = "k_w16_fp8_lines" if args.format == "fp8" else "k_w16_nvfp4_lines"
+        gate_up_kernel = ("ffmoe::%s<MF, 0, P, NW> (gate/up + SwiGLU of the token cohort on the BF16 matrix cores, each chosen expert's weights streamed "
+                          "once%s)" % (lines, "; the BF16 shared expert's gate/up launch rides in the figure" if args.format != "fp8" else ""))
+        down_kernel = "ffmoe::%s<MF, 1, P, NW> (down + routing weight of the cohort%s)" % (
+            lines, "; with the BF16 shared expert's down launch" if args.format != "fp8" else "")
+    else:
+        gate_up_kernel = "ffmoe::k_decode_stage<%s, S, 0, RG, NR> (gate/up + SwiGLU launch)" % fname
+        down_kernel = "ffmoe::k_decode_stage<%s, S, 1, RG, NR> (down + routing weight)" % fname
 
     out = {
         "metric": "moe_layer_decode_us", "value": us_per_layer, "unit": "us/layer", "n_gpus": 1,
@@ -915,8 +939,8 @@ def decode_main(args, torch, capi, ops, synth, prebuilt=None):
                    "weights": "E4M3 + f32 128x128 block scales" if args.format == "fp8" else "E2M1 pairs + E4M3 scale per 16 + f32 global",
                    "act_mode": "FFMOE_ACT_BF16 (W8A16)" if args.format == "fp8" else "BF16 activations (W4A16)",
                    "batch": args.batch, "ring": len(xs), "launch": "eager" if graphs is None else "hip graph per ring slot",
-                   "launches_per_layer": ("router logits; shared expert gate/up with the top-k selection in its prologue; shared expert down; "
-                                          "routed gate/up; routed down + weight + combine with the shared row") if mixed_token else
+                   "launches_per_layer": ("router logits; gate/up with the top-k selection in its prologue (BF16 shared rows first); shared expert down; "
+                                          "routed down + weight + combine with the shared row") if own_down else
                                          "router logits; gate/up with the top-k selection in its prologue; down + weight + combine" if token_path else
                                          "router logits; top-k; grouping; gate/up; down; combine"},
         "tokens_per_s": args.batch / (us_per_layer * 1e-6),
@@ -924,17 +948,13 @@ def decode_main(args, torch, capi, ops, synth, prebuilt=None):
         "layer_bytes": bytes_layer,
         "layer_hbm_gbps": bytes_layer / (us_per_layer * 1e-6) / 1e9,
         "layer_hbm_frac": bytes_layer / (us_per_layer * 1e-6) / 1e9 / HBM_PEAK_GBPS,
-        "roofline": {"kernel": ("ffmoe::k_decode_stage<FmtBf16, S, 0|1, 1, NR> x 2 + k_decode_stage<FmtNvfp4, S, 0, 1, NR> (the three launches in front of the "
-                                "finish, as the layer issues them: shared expert gate/up with the top-k selection in its prologue, shared expert down, routed "
-                                "gate/up + SwiGLU)") if mixed_token else "ffmoe::k_decode_stage<%s, S, 0, RG, NR> (gate/up + SwiGLU launch%s)" % (
-                         "FmtFp8" if args.format == "fp8" else "FmtNvfp4", ", top-k selection in its prologue, as the layer issues it" if token_path else ""),
+        "roofline": {"kernel": gate_up_kernel,
                      "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBPS, "traffic": GATE_UP_TRAFFIC_BYTES.get((args.batch, args.experts)) if args.format == "fp8" else None,
                      "traffic_source": TRAFFIC_SOURCE if (args.format == "fp8" and (args.batch, args.experts) in GATE_UP_TRAFFIC_BYTES) else None,
                      "bytes_per_launch": k_bytes, "avg_us": k_avg, "min_us": kt[0], "median_us": kt[len(kt) // 2],
                      "launches_timed": launches_timed},
-        "down_kernel": {"kernel": ("ffmoe::k_decode_finish<F, S, NR> (down + routing weight + ordered combine)" if token_path else
-                                   "ffmoe::k_decode_stage<F, S, 1, RG, NR> (down + routing weight)"),
+        "down_kernel": {"kernel": down_kernel,
                         "bytes_per_launch": d_bytes, "avg_us": d_avg, "min_us": dt[0], "median_us": dt[len(dt) // 2],
                         "achieved": d_bytes / (d_avg * 1e-6) / 1e9, "frac": d_bytes / (d_avg * 1e-6) / 1e9 / HBM_PEAK_GBPS},
         "parity": parity,

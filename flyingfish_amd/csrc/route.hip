@@ -12,35 +12,42 @@ namespace ffmoe {
 // logits[r,e] = bf16(fma chain over k ascending). One lane owns one (row, expert) chain
 // (kernels/moe_route.cu:392-403, :536-544): 2 * hidden dependent fmas, serial by contract. What the lane must not also
 // do is fetch its router row itself - 64 lanes reading 16 bytes each of 64 different rows is 64 cache lines per load
-// instruction, and that, not the chain, was the kernel's time (22.8 us for 64 experts x 2048). A block is four waves: all
+// instruction, and that, not the chain, was the kernel's time (22.8 us for 64 experts x 2048). A block is five waves: four
 // of them move the router tile of 64 experts x 256 columns and the token row's 256 columns through LDS with coalesced
-// requests (32 lanes per 512-byte row segment), one chunk ahead, and wave 0 runs the 64 chains out of LDS (rows padded by
-// 16 bytes, so the 16 lanes of a quarter wave read 16 different LDS slots).
+// requests (32 lanes per 512-byte row segment), one chunk ahead, and wave 0 does nothing but run the 64 chains out of LDS
+// (rows padded by 16 bytes, so the 16 lanes of a quarter wave read 16 different LDS slots). A dependent v_fma_f32 takes 8
+// cycles on this machine and 10 with its operands arriving from LDS (2048 of them: 8.6 and 10.5 us), whatever the row
+// stride and whether the token row comes through LDS or scalar registers; the chain wave is kept clear of everything else.
 constexpr int LOGIT_CHUNK = 256;                      // columns per chunk
 constexpr int LOGIT_ROW_BYTES = LOGIT_CHUNK * 4 + 16;  // a row of the tile as FP32, padded by one 16-byte slot
-__global__ __launch_bounds__(256) void k_route_logits_bf16(const uint16_t* __restrict__ x, const uint16_t* __restrict__ router,
+__global__ __launch_bounds__(320) void k_route_logits_bf16(const uint16_t* __restrict__ x, const uint16_t* __restrict__ router,
                                                            uint16_t* __restrict__ logits, int rows, int experts, int hidden) {
   // 64 router rows + the token row, widened to FP32 by the waves that move them: the chain wave's instruction stream is
   // then one LDS read per four elements and operand plus the fmas themselves, no unpacking in front of every fma
   __shared__ __attribute__((aligned(16))) uint8_t tile[2][65 * LOGIT_ROW_BYTES];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int lane = threadIdx.x & 63, wave = uni(int(threadIdx.x >> 6));
+  const int tid = int(threadIdx.x) - 64;                  // index among the 256 moving threads (wave 0: negative, moves nothing)
+  const bool mover = wave != 0;
   const int e0 = blockIdx.x * 64;
   const int row = blockIdx.y;
   const int words = hidden >> 3;                          // 16-byte pieces (8 columns) per row
   const int chunks = (words + 31) >> 5;
   // piece (r, q) of a chunk for i = 0 .. 7: r = (tid + 256 i) / 32, q = (tid + 256 i) % 32; thread tid < 32 also moves piece tid
   // of the token row. Pieces past the end of the row repeat its last piece; nothing multiplies them.
-  u32x4 regs[8], xreg;
-  auto request = [&](int c) {
+  // The movers run two chunks ahead in two register sets (chunk c in set c % 2): a chunk's chains take about 1.3 us, less than a
+  // request that misses the caches.
+  u32x4 regs[2][8], xreg[2];
+  auto request = [&](auto set, int c) {
+    constexpr int S = decltype(set)::value;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const int idx = tid + 256 * i;
       const int r = idx >> 5, q = idx & 31;
       const int er = min(e0 + r, experts - 1);
       const int piece = min(32 * c + q, words - 1);
-      regs[i] = load16(router + size_t(er) * hidden + size_t(piece) * 8);
+      regs[S][i] = load16(router + size_t(er) * hidden + size_t(piece) * 8);
     }
-    if (tid < 32) xreg = load16(x + size_t(row) * hidden + size_t(min(32 * c + tid, words - 1)) * 8);
+    if (tid < 32) xreg[S] = load16(x + size_t(row) * hidden + size_t(min(32 * c + tid, words - 1)) * 8);
   };
   auto widen = [&](uint8_t* dst, const u32x4& v) {
     const u32x4 lo = {__float_as_uint(bf16lo(v[0])), __float_as_uint(bf16hi(v[0])), __float_as_uint(bf16lo(v[1])), __float_as_uint(bf16hi(v[1]))};
@@ -48,25 +55,34 @@ __global__ __launch_bounds__(256) void k_route_logits_bf16(const uint16_t* __res
     *reinterpret_cast<u32x4*>(dst) = lo;
     *reinterpret_cast<u32x4*>(dst + 16) = hi;
   };
-  auto publish = [&](int buf) {
+  auto publish = [&](auto set) {  // chunk c sits in set c % 2 and goes to buffer c % 2
+    constexpr int S = decltype(set)::value;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const int idx = tid + 256 * i;
-      widen(&tile[buf][(idx >> 5) * LOGIT_ROW_BYTES + (idx & 31) * 32], regs[i]);
+      widen(&tile[S][(idx >> 5) * LOGIT_ROW_BYTES + (idx & 31) * 32], regs[S][i]);
     }
-    if (tid < 32) widen(&tile[buf][64 * LOGIT_ROW_BYTES + tid * 32], xreg);
+    if (tid < 32) widen(&tile[S][64 * LOGIT_ROW_BYTES + tid * 32], xreg[S]);
   };
-  request(0);
-  publish(0);
+  using S0 = std::integral_constant<int, 0>;
+  using S1 = std::integral_constant<int, 1>;
+  if (mover) {
+    request(S0{}, 0);
+    if (chunks > 1) request(S1{}, 1);
+    publish(S0{});
+    if (chunks > 2) request(S0{}, 2);
+  }
   __syncthreads();
   float acc = 0.0f;
-  for (int c = 0; c < chunks; ++c) {
-    if (c + 1 < chunks) request(c + 1);
-    if (wave == 0) {
+  // stage c: the chain wave reads buffer c % 2; the movers publish chunk c + 1 into the other buffer and request chunk c + 3
+  auto stage = [&](auto other, int c) {
+    if (mover) {
+      if (c + 1 < chunks) publish(other);
+      if (c + 3 < chunks) request(other, c + 3);
+    } else {
       const uint8_t* wrow = &tile[c & 1][lane * LOGIT_ROW_BYTES];
       const uint8_t* xrow = &tile[c & 1][64 * LOGIT_ROW_BYTES];
       const int nquads = 2 * min(32, words - 32 * c);  // groups of four columns
-      // (reading a batch of groups ahead of the previous batch's fmas by hand measured slower than the compiler's order)
 #pragma unroll 8
       for (int q = 0; q < nquads; ++q) {
         const u32x4 wv = *reinterpret_cast<const u32x4*>(wrow + q * 16);
@@ -75,10 +91,13 @@ __global__ __launch_bounds__(256) void k_route_logits_bf16(const uint16_t* __res
         for (int j = 0; j < 4; ++j) acc = __fmaf_rn(__uint_as_float(xv[j]), __uint_as_float(wv[j]), acc);
       }
     }
-    if (c + 1 < chunks) publish((c + 1) & 1);
     __syncthreads();
+  };
+  for (int c = 0; c < chunks; c += 2) {
+    stage(S1{}, c);
+    if (c + 1 < chunks) stage(S0{}, c + 1);
   }
-  if (wave == 0 && e0 + lane < experts) logits[size_t(row) * experts + e0 + lane] = f32_to_bf16(acc);
+  if (!mover && e0 + lane < experts) logits[size_t(row) * experts + e0 + lane] = f32_to_bf16(acc);
 }
 
 // FP32 logits. One block of 256 threads per expert: thread p chains the 8-element vectors p, p+256, ... in ascending
@@ -482,7 +501,7 @@ extern "C" __attribute__((visibility("default"))) int ffmoe_route_logits_bf16(co
   FF_PTR16(x); FF_PTR16(router); FF_PTR16(logits);
   FF_NO_OVERLAP(logits, size_t(rows) * experts * 2, x, size_t(rows) * hidden * 2);
   FF_NO_OVERLAP(logits, size_t(rows) * experts * 2, router, size_t(experts) * hidden * 2);
-  hipLaunchKernelGGL(k_route_logits_bf16, dim3((experts + 63) / 64, rows), dim3(256), 0, (hipStream_t)stream,
+  hipLaunchKernelGGL(k_route_logits_bf16, dim3((experts + 63) / 64, rows), dim3(320), 0, (hipStream_t)stream,
                      (const uint16_t*)x, (const uint16_t*)router, (uint16_t*)logits, rows, experts, hidden);
   return ff_launch_status();
 }
