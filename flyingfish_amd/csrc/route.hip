@@ -18,10 +18,65 @@ namespace ffmoe {
 // (rows padded by 16 bytes, so the 16 lanes of a quarter wave read 16 different LDS slots). A dependent v_fma_f32 takes 8
 // cycles on this machine and 10 with its operands arriving from LDS (2048 of them: 8.6 and 10.5 us), whatever the row
 // stride and whether the token row comes through LDS or scalar registers; the chain wave is kept clear of everything else.
+__device__ __forceinline__ int rank_of(const float* s_key, int padded, float mine, int e);
+
+// Softmax / sigmoid top-k of at most 64 experts by the wave whose lane e holds expert e's BF16 logit: the arithmetic of
+// k_route_topk for a block of one wave, operation for operation (the softmax denominator as the reference's 32-lane trees
+// and the tree over the two 32-lane sums, selection by rank, weights = score / sum of the picked scores in pick order), with
+// the block-wide exchanges replaced by the wave's own LDS scratch (LDS operations of one wave execute in order).
+// s_key: 64 floats, 16-byte aligned; s_sel / s_selid: FFMOE_MAX_TOP_K entries.
+__device__ __forceinline__ void wave_topk64(float logit, bool live, int lane, int top_k, int score_mode, float* s_key, float* s_sel,
+                                            int* s_selid, int* __restrict__ ids_row, uint16_t* __restrict__ weights_row) {
+  float score;
+  if (score_mode == FFMOE_SCORE_SOFTMAX) {
+    const float m = wave_max(logit);
+    const float ev = live ? det_expf(__fsub_rn(logit, m)) : 0.0f;
+    float v = ev;
+#pragma unroll
+    for (int off = 16; off > 0; off >>= 1) {
+      const float o = __shfl_down(v, off, 32);
+      v = __fadd_rn(v, ((lane & 31) + off < 32) ? o : 0.0f);
+    }
+    const float upper = __shfl(v, 32);  // the second 32-lane group's sum
+    v = lane == 0 ? v : (lane == 1 ? upper : 0.0f);
+#pragma unroll
+    for (int off = 16; off > 0; off >>= 1) {
+      const float o = __shfl_down(v, off, 32);
+      v = __fadd_rn(v, ((lane & 31) + off < 32) ? o : 0.0f);
+    }
+    const float den = __shfl(v, 0);
+    score = live ? __fdiv_rn(ev, den) : -INFINITY;
+  } else {
+    score = live ? sigmoid1(logit) : -INFINITY;
+  }
+  s_key[lane] = score;
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  if (live) {
+    const int rank = rank_of(s_key, 64, score, lane);
+    if (rank < top_k) { s_sel[rank] = score; s_selid[rank] = lane; }
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  if (lane < top_k) {
+    float tsum = 0.0f;
+    for (int r = 0; r < top_k; ++r) tsum = __fadd_rn(tsum, s_sel[r]);
+    const float den = score_mode == FFMOE_SCORE_SOFTMAX ? tsum : __fadd_rn(tsum, 1.0e-20f);
+    ids_row[lane] = s_selid[lane];
+    weights_row[lane] = f32_to_bf16(__fdiv_rn(s_sel[lane], den));
+  }
+}
+
 constexpr int LOGIT_CHUNK = 256;                      // columns per chunk
 constexpr int LOGIT_ROW_BYTES = LOGIT_CHUNK * 4 + 16;  // a row of the tile as FP32, padded by one 16-byte slot
+// SELECT (at most 64 experts, i.e. one block per row): the chain wave goes on to the top-k of its row, whose logits it holds
+// one per lane - the selection launch and the logits' round trip through memory fall away.
+template <bool SELECT>
 __global__ __launch_bounds__(320) void k_route_logits_bf16(const uint16_t* __restrict__ x, const uint16_t* __restrict__ router,
-                                                           uint16_t* __restrict__ logits, int rows, int experts, int hidden) {
+                                                           uint16_t* __restrict__ logits, int rows, int experts, int hidden,
+                                                           int* __restrict__ ids, uint16_t* __restrict__ weights, int top_k, int score_mode) {
   // 64 router rows + the token row, widened to FP32 by the waves that move them: the chain wave's instruction stream is
   // then one LDS read per four elements and operand plus the fmas themselves, no unpacking in front of every fma
   __shared__ __attribute__((aligned(16))) uint8_t tile[2][65 * LOGIT_ROW_BYTES];
@@ -97,7 +152,19 @@ __global__ __launch_bounds__(320) void k_route_logits_bf16(const uint16_t* __res
     stage(S1{}, c);
     if (c + 1 < chunks) stage(S0{}, c + 1);
   }
-  if (!mover && e0 + lane < experts) logits[size_t(row) * experts + e0 + lane] = f32_to_bf16(acc);
+  if (!mover) {
+    const bool live = e0 + lane < experts;
+    const uint16_t lb = f32_to_bf16(acc);
+    if (live) logits[size_t(row) * experts + e0 + lane] = lb;
+    if constexpr (SELECT) {
+      // the tiles are no longer read (every wave is past the last barrier): the head of buffer 0 is the wave's scratch
+      float* s_key = reinterpret_cast<float*>(&tile[0][0]);
+      float* s_sel = s_key + 64;
+      int* s_selid = reinterpret_cast<int*>(s_sel + FFMOE_MAX_TOP_K);
+      wave_topk64(live ? bf16_to_f32(lb) : -INFINITY, live, lane, top_k, score_mode, s_key, s_sel, s_selid, ids + size_t(row) * top_k,
+                  weights + size_t(row) * top_k);
+    }
+  }
 }
 
 // FP32 logits. One block of 256 threads per expert: thread p chains the 8-element vectors p, p+256, ... in ascending
@@ -501,8 +568,8 @@ extern "C" __attribute__((visibility("default"))) int ffmoe_route_logits_bf16(co
   FF_PTR16(x); FF_PTR16(router); FF_PTR16(logits);
   FF_NO_OVERLAP(logits, size_t(rows) * experts * 2, x, size_t(rows) * hidden * 2);
   FF_NO_OVERLAP(logits, size_t(rows) * experts * 2, router, size_t(experts) * hidden * 2);
-  hipLaunchKernelGGL(k_route_logits_bf16, dim3((experts + 63) / 64, rows), dim3(320), 0, (hipStream_t)stream,
-                     (const uint16_t*)x, (const uint16_t*)router, (uint16_t*)logits, rows, experts, hidden);
+  hipLaunchKernelGGL(k_route_logits_bf16<false>, dim3((experts + 63) / 64, rows), dim3(320), 0, (hipStream_t)stream,
+                     (const uint16_t*)x, (const uint16_t*)router, (uint16_t*)logits, rows, experts, hidden, (int*)nullptr, (uint16_t*)nullptr, 0, 0);
   return ff_launch_status();
 }
 
@@ -594,6 +661,24 @@ extern "C" __attribute__((visibility("default"))) int ffmoe_route_topk_noaux(con
 extern "C" __attribute__((visibility("default"))) int ffmoe_route_decode(const void* x, const void* router, void* logits, int* ids, void* weights, int rows,
                                   int experts, int hidden, int top_k, int score, void* stream) {
   FF_TRY(check_topk_dims(rows, experts, top_k, false));
+  // up to 64 experts the wave that runs a row's chains holds all its logits and selects right away: one launch
+  // (FFMOE_ROUTE_FUSED=0: the two launches; same bits)
+  static const bool fused = [] { const char* e = getenv("FFMOE_ROUTE_FUSED"); return !(e && atoi(e) == 0); }();
+  if (fused && experts <= 64) {
+    FF_TRY(check_route_dims(rows, experts, hidden));
+    FF_REQUIRE(score == FFMOE_SCORE_SOFTMAX || score == FFMOE_SCORE_SIGMOID, FFMOE_ERR_UNSUPPORTED, "unknown router score %d", score);
+    FF_PTR16(x); FF_PTR16(router); FF_PTR16(logits); FF_PTR4(ids); FF_PTR2(weights);
+    FF_NO_OVERLAP(logits, size_t(rows) * experts * 2, x, size_t(rows) * hidden * 2);
+    FF_NO_OVERLAP(logits, size_t(rows) * experts * 2, router, size_t(experts) * hidden * 2);
+    FF_NO_OVERLAP(ids, size_t(rows) * top_k * 4, logits, size_t(rows) * experts * 2);
+    FF_NO_OVERLAP(weights, size_t(rows) * top_k * 2, logits, size_t(rows) * experts * 2);
+    FF_NO_OVERLAP(ids, size_t(rows) * top_k * 4, weights, size_t(rows) * top_k * 2);
+    FF_NO_OVERLAP(ids, size_t(rows) * top_k * 4, x, size_t(rows) * hidden * 2);
+    FF_NO_OVERLAP(weights, size_t(rows) * top_k * 2, x, size_t(rows) * hidden * 2);
+    hipLaunchKernelGGL(k_route_logits_bf16<true>, dim3(1, rows), dim3(320), 0, (hipStream_t)stream, (const uint16_t*)x, (const uint16_t*)router,
+                       (uint16_t*)logits, rows, experts, hidden, ids, (uint16_t*)weights, top_k, score);
+    return ff_launch_status();
+  }
   int rc = ffmoe_route_logits_bf16(x, router, logits, rows, experts, hidden, stream);
   if (rc) return rc;
   return ffmoe_route_topk(logits, ids, weights, rows, experts, top_k, score, stream);

@@ -251,6 +251,29 @@ def test_route_decode_fused_c1_shape():
     assert np.array_equal(bits(logits), ol) and np.array_equal(ids.cpu().numpy(), oi) and np.array_equal(bits(wt), ow)
 
 
+@pytest.mark.parametrize("score", [capi.SCORE_SOFTMAX, capi.SCORE_SIGMOID])
+@pytest.mark.parametrize("rows,experts,hidden,top_k", [(1, 64, 2048, 4), (3, 64, 520, 6), (5, 33, 264, 8), (2, 8, 4104, 3), (1, 128, 512, 4)])
+def test_route_decode_one_launch_equals_the_two_launches_and_the_oracle(score, rows, experts, hidden, top_k):
+    """ffmoe_route_decode: up to 64 experts the wave that runs a row's logit chains also selects (one launch); beyond, logits
+    and selection are two launches. Logits, ids and weights bit for bit against the oracle and against the separate calls,
+    with exact ties planted among the router rows (equal rows give equal logits: the lower id wins)."""
+    x, w = rand_bf16((rows, hidden), 1.0, 121 + rows), rand_bf16((experts, hidden), 0.05, 122 + experts)
+    w[experts - 1] = w[1]
+    w[5] = w[2]
+    print("route decode rows=%d experts=%d hidden=%d top_k=%d score=%d" % (rows, experts, hidden, top_k, score), flush=True)
+    ids, wt, logits = RouteOps.route(x.to(DEV), w.to(DEV), top_k, score)
+    torch.cuda.synchronize()
+    ol = orc.route_logits_bf16(bits(x), bits(w))
+    fn = orc.route_topk_softmax if score == capi.SCORE_SOFTMAX else orc.route_topk_sigmoid
+    oi, ow = fn(ol, top_k)
+    assert np.array_equal(bits(logits), ol)
+    assert np.array_equal(ids.cpu().numpy(), oi)
+    assert np.array_equal(bits(wt), ow)
+    l2 = RouteOps.logits_bf16(x.to(DEV), w.to(DEV))
+    i2, w2 = RouteOps.topk(l2, top_k, score)
+    assert torch.equal(l2.view(torch.int16), logits.view(torch.int16)) and torch.equal(i2, ids) and torch.equal(w2.view(torch.int16), wt.view(torch.int16))
+
+
 # ------------------------------------------------------------------------------------------------
 # decode contributions
 def _run_decode(fmt, experts, hidden, inter, rows, top_k, seed, shared, swiglu_mode=capi.SWIGLU_TWICE, limit=0.0,
