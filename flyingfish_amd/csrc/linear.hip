@@ -19,7 +19,8 @@ struct LinearParams {
 // weight row at a time against up to RG activation rows held in LDS; rows beyond RG are served by further
 // passes. One register buffer of S steps per wave: step s of the next item is requested as soon as step s of
 // the current one has been consumed.
-template <class F, int S, int RG>
+// NR: weight rows per unit (they share every activation chunk read from LDS, and NR x S KiB per wave are in flight).
+template <class F, int S, int RG, int NR = 1>
 __global__ __launch_bounds__(256) void k_linear(const LinearParams p) {
   constexpr int NW = 4;
   extern __shared__ __align__(16) uint8_t xs[];
@@ -32,7 +33,8 @@ __global__ __launch_bounds__(256) void k_linear(const LinearParams p) {
   const int nchunks = K / F::EPL;
   const int nslabs = (nchunks + S * 64 - 1) / (S * 64);
   const int w_lo = count * wave / NW, w_hi = count * (wave + 1) / NW;
-  const int my_units = w_hi - w_lo;
+  const int my_rows = w_hi - w_lo;
+  const int my_units = (my_rows + NR - 1) / NR;
   const int items = my_units * nslabs;
   const int jw = int(lo) + w_lo;
   // NVFP4: the split dot's constants per scale code (one global scale per matrix); the first barrier below publishes it
@@ -41,11 +43,14 @@ __global__ __launch_bounds__(256) void k_linear(const LinearParams p) {
   if constexpr (NV) FmtNvfp4::build_lut(s_lut, global, tid, 256);
   for (int r0 = 0; r0 < p.m; r0 += RG) {
     const int n = p.m - r0 < RG ? p.m - r0 : RG;
-    typename F::Chunk buf[1][S];
+    typename F::Chunk buf[NR][S];
     auto issue_step = [&](int t, int s) {
-      const int j = jw + t / nslabs;
       const int chunk = (t % nslabs) * (S * 64) + s * 64 + lane;
-      F::load(buf[0][s], F::row(p.codes, p.scales, global, j, K), chunk < nchunks ? chunk : nchunks - 1);
+#pragma unroll
+      for (int w = 0; w < NR; ++w) {
+        const int jr = (t / nslabs) * NR + w;  // a ragged last unit repeats the wave's last row
+        F::load(buf[w][s], F::row(p.codes, p.scales, global, jw + (jr < my_rows ? jr : my_rows - 1), K), chunk < nchunks ? chunk : nchunks - 1);
+      }
     };
     if (items > 0) {
 #pragma unroll
@@ -59,23 +64,28 @@ __global__ __launch_bounds__(256) void k_linear(const LinearParams p) {
     }
     __syncthreads();
     if (items > 0) {
-      float acc[1][RG];
+      float acc[NR][RG];
 #pragma unroll
-      for (int r = 0; r < RG; ++r) acc[0][r] = 0.0f;
+      for (int w = 0; w < NR; ++w)
+#pragma unroll
+        for (int r = 0; r < RG; ++r) acc[w][r] = 0.0f;
       auto compute_step = [&](int t, int s) {
         const int chunk = (t % nslabs) * (S * 64) + s * 64 + lane;
-        step_compute<F, 1, RG, S, NV>(buf, s, xs, K, nchunks, chunk, n, acc, s_lut);
+        step_compute<F, NR, RG, S, NV>(buf, s, xs, K, nchunks, chunk, n, acc, s_lut, s_lut, NR);
       };
       auto item_end = [&](int t) {
         if (t % nslabs != nslabs - 1) return;
-        const int j = jw + t / nslabs;
 #pragma unroll
-        for (int r = 0; r < RG; ++r) {
-          if (RG == 1 || r < n) {
-            const float total = wave_sum(acc[0][r]);
-            if (lane == r) p.y[size_t(r0 + r) * p.n + j] = f32_to_bf16(total);
+        for (int w = 0; w < NR; ++w) {
+          const int jr = (t / nslabs) * NR + w;
+#pragma unroll
+          for (int r = 0; r < RG; ++r) {
+            if (RG == 1 || r < n) {
+              const float total = wave_sum(acc[w][r]);
+              if (lane == r && jr < my_rows) p.y[size_t(r0 + r) * p.n + jw + jr] = f32_to_bf16(total);
+            }
+            acc[w][r] = 0.0f;
           }
-          acc[0][r] = 0.0f;
         }
       };
       for (int t = 0; t + 1 < items; ++t) {
@@ -106,7 +116,9 @@ struct LinearBatchParams {
   int count, m, n, k;
 };
 
-template <class F, int S, int RG>
+// NR: weight rows per unit. With several activation rows a unit of two weight rows reads every activation chunk from LDS
+// once for both (the LDS pipe, not the weight stream, is what four activation rows per weight row load).
+template <class F, int S, int RG, int NR = 1>
 __global__ __launch_bounds__(256) void k_linear_batch(const LinearBatchParams p) {
   constexpr int NW = 4;
   extern __shared__ __align__(16) uint8_t xs[];
@@ -128,14 +140,18 @@ __global__ __launch_bounds__(256) void k_linear_batch(const LinearBatchParams p)
     uint16_t* y = reinterpret_cast<uint16_t*>(uni64(load_global<uint64_t>(it + 3)));
     const float global = p.global ? unif(load_global<float>(p.global + item)) : 1.0f;
     const int w_lo = count * wave / NW, w_hi = count * (wave + 1) / NW;
-    const int my_units = w_hi - w_lo;
+    const int my_rows = w_hi - w_lo;
+    const int my_units = (my_rows + NR - 1) / NR;
     const int items_w = my_units * nslabs;
     const int jw = j0 + w_lo;
-    typename F::Chunk buf[1][S];
+    typename F::Chunk buf[NR][S];
     auto issue_step = [&](int t, int s) {
-      const int j = jw + t / nslabs;
       const int chunk = (t % nslabs) * (S * 64) + s * 64 + lane;
-      F::load(buf[0][s], F::row(codes, scales, global, j, K), chunk < nchunks ? chunk : nchunks - 1);
+#pragma unroll
+      for (int r = 0; r < NR; ++r) {
+        const int jr = (t / nslabs) * NR + r;  // a ragged last unit repeats the wave's last row
+        F::load(buf[r][s], F::row(codes, scales, global, jw + (jr < my_rows ? jr : my_rows - 1), K), chunk < nchunks ? chunk : nchunks - 1);
+      }
     };
     if (items_w > 0) {
 #pragma unroll
@@ -149,23 +165,28 @@ __global__ __launch_bounds__(256) void k_linear_batch(const LinearBatchParams p)
     }
     __syncthreads();
     if (items_w > 0) {
-      float acc[1][RG];
+      float acc[NR][RG];
 #pragma unroll
-      for (int r = 0; r < RG; ++r) acc[0][r] = 0.0f;
+      for (int w = 0; w < NR; ++w)
+#pragma unroll
+        for (int r = 0; r < RG; ++r) acc[w][r] = 0.0f;
       auto compute_step = [&](int t, int s) {
         const int chunk = (t % nslabs) * (S * 64) + s * 64 + lane;
-        step_compute<F, 1, RG, S>(buf, s, xs, K, nchunks, chunk, p.m, acc);
+        step_compute<F, NR, RG, S>(buf, s, xs, K, nchunks, chunk, p.m, acc);
       };
       auto item_end = [&](int t) {
         if (t % nslabs != nslabs - 1) return;
-        const int j = jw + t / nslabs;
 #pragma unroll
-        for (int r = 0; r < RG; ++r) {
-          if (RG == 1 || r < p.m) {
-            const float sum = wave_sum(acc[0][r]);
-            if (lane == r) y[size_t(r) * N + j] = f32_to_bf16(sum);
+        for (int w = 0; w < NR; ++w) {
+          const int jr = (t / nslabs) * NR + w;
+#pragma unroll
+          for (int r = 0; r < RG; ++r) {
+            if (RG == 1 || r < p.m) {
+              const float sum = wave_sum(acc[w][r]);
+              if (lane == r && jr < my_rows) y[size_t(r) * N + jw + jr] = f32_to_bf16(sum);
+            }
+            acc[w][r] = 0.0f;
           }
-          acc[0][r] = 0.0f;
         }
       };
       for (int t = 0; t + 1 < items_w; ++t) {
@@ -359,9 +380,29 @@ int launch_linear(const LinearParams& p, hipStream_t st) {
   int blocks = num_cus_l() * 2;
   if (blocks > (p.n + 3) / 4) blocks = (p.n + 3) / 4;
   const size_t row = size_t(p.k) * 2;
-  if (p.m > 1 && 8 * row <= 64 * 1024) hipLaunchKernelGGL((k_linear<F, 4, 8>), dim3(blocks), dim3(256), 8 * row, st, p);
-  else if (p.m > 1 && 4 * row <= 64 * 1024) hipLaunchKernelGGL((k_linear<F, 4, 4>), dim3(blocks), dim3(256), 4 * row, st, p);
-  else hipLaunchKernelGGL((k_linear<F, 4, 1>), dim3(blocks), dim3(256), row, st, p);
+  // Weight rows per unit: one. A single call is bound by its start-up, and more rows per unit, which pay in the batched entry,
+  // change nothing or lose here (FFMOE_LINEAR_NR=2 / 4, same bits: M = 1 8.8 us either way, M = 4 at K 7168 11.7 against 9.1 us).
+  // NVFP4, whose split-dot operands of one row take the registers four FP8 rows do, has no other instantiation.
+  constexpr bool one_row_units = std::is_same<F, FmtNvfp4>::value;
+  int nr = 1;
+  if (const char* e = getenv("FFMOE_LINEAR_NR")) { const int v = atoi(e); if (v == 1 || v == 2 || v == 4) nr = v; }
+  auto go = [&](auto rg, auto nrc) {
+    constexpr int RG = decltype(rg)::value, NR = decltype(nrc)::value;
+    hipLaunchKernelGGL((k_linear<F, 4, RG, NR>), dim3(blocks), dim3(256), RG * row, st, p);
+  };
+  auto with_rg = [&](auto rg) {
+    constexpr int RG = decltype(rg)::value;
+    if constexpr (one_row_units) {
+      go(rg, std::integral_constant<int, 1>{});
+    } else {
+      if (nr == 4 && RG == 1) go(std::integral_constant<int, 1>{}, std::integral_constant<int, 4>{});
+      else if (nr >= 2 && RG <= 4) go(rg, std::integral_constant<int, 2>{});
+      else go(rg, std::integral_constant<int, 1>{});
+    }
+  };
+  if (p.m > 4 && 8 * row <= 64 * 1024) with_rg(std::integral_constant<int, 8>{});
+  else if (p.m > 1 && 4 * row <= 64 * 1024) with_rg(std::integral_constant<int, 4>{});
+  else with_rg(std::integral_constant<int, 1>{});
   return ff_launch_status();
 }
 
@@ -424,11 +465,11 @@ extern "C" __attribute__((visibility("default"))) int ffmoe_linear_fp8_block(con
 }
 
 namespace {
-template <class F, int RG, int SMAX, int S = 1>
+template <class F, int RG, int SMAX, int NR, int S = 1>
 void launch_batch_steps(int want, const LinearBatchParams& p, int blocks, size_t lds, hipStream_t st) {
   if constexpr (S <= SMAX) {
-    if (want == S) hipLaunchKernelGGL((k_linear_batch<F, S, RG>), dim3(blocks), dim3(256), lds, st, p);
-    else launch_batch_steps<F, RG, SMAX, S + 1>(want, p, blocks, lds, st);
+    if (want == S) hipLaunchKernelGGL((k_linear_batch<F, S, RG, NR>), dim3(blocks), dim3(256), lds, st, p);
+    else launch_batch_steps<F, RG, SMAX, NR, S + 1>(want, p, blocks, lds, st);
   }
 }
 }  // namespace
@@ -445,13 +486,25 @@ extern "C" __attribute__((visibility("default"))) int ffmoe_linear_fp8_block_bat
   int blocks = num_cus_l() * 2;
   if (blocks > (total + 3) / 4) blocks = int((total + 3) / 4);
   const int steps = (k / 16 + 63) / 64;
-  const int smax = m == 1 ? 8 : 4;
+  int smax = 8;
+  if (const char* e = getenv("FFMOE_LINEAR_BATCH_SMAX")) { const int v = atoi(e); if (v >= 1 && v <= 8) smax = v; }
   const int nslabs = (steps + smax - 1) / smax;
   const int S = (steps + nslabs - 1) / nslabs;
   const size_t lds = size_t(m) * k * 2;
   hipStream_t st = (hipStream_t)stream;
-  if (m == 1) launch_batch_steps<FmtFp8, 1, 8>(S, p, blocks, lds, st);
-  else launch_batch_steps<FmtFp8, 4, 4>(S, p, blocks, lds, st);
+  // Weight rows per unit (bit-identical whatever it is: a row's dot product does not depend on its neighbours). One activation
+  // row: what counts is bytes in flight per wave - two rows of seven steps (14 KB) at K 7168, four rows of two steps (8 KB) at
+  // K 2048 (eight matrices per launch, us per matrix with 1 / 2 / 4 rows per unit: 3.00 / 2.83 / 3.43 and 4.03 / 3.11 / 2.95).
+  // Several activation rows: four weight rows share every activation chunk read from LDS (M = 4: 6.61 / 4.74 / 4.31 and
+  // 7.44 / 5.45 / 4.77 us; with rows of at most four steps per slab, as before, 7.51 and 7.42).
+  int nr = m == 1 ? (steps >= 4 ? 2 : 4) : 4;
+  if (const char* e = getenv("FFMOE_LINEAR_BATCH_NR")) { const int v = atoi(e); if (v == 1 || v == 2 || v == 4) nr = v; }
+  if (m == 1 && nr == 4) launch_batch_steps<FmtFp8, 1, 8, 4>(S, p, blocks, lds, st);
+  else if (m == 1 && nr == 2) launch_batch_steps<FmtFp8, 1, 8, 2>(S, p, blocks, lds, st);
+  else if (m == 1) launch_batch_steps<FmtFp8, 1, 8, 1>(S, p, blocks, lds, st);
+  else if (nr == 4) launch_batch_steps<FmtFp8, 4, 8, 4>(S, p, blocks, lds, st);
+  else if (nr == 2) launch_batch_steps<FmtFp8, 4, 8, 2>(S, p, blocks, lds, st);
+  else launch_batch_steps<FmtFp8, 4, 8, 1>(S, p, blocks, lds, st);
   return ff_launch_status();
 }
 
