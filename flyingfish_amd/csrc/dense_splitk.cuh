@@ -30,7 +30,14 @@ struct DenseParams {
 // MFT token fragments of 16 rows per block; blockIdx.x = column tile of 16, blockIdx.y = row block of 16 * MFT
 // TC output columns per block: MODE 0: 8 (gate rows 0-7, up rows 8-15 of the fragment); MODE 2: 16. (Half of that, the
 // fragment's upper rows repeating the lower ones, also works and is slower: every block reads the whole token panel.)
-template <int MODE, int MFT, int TC, int NA = 1>
+// XL: the token panel goes through LDS. Requested in the instruction's lane order a token load touches 64 lines for 16 bytes
+// each (the 16 lanes of a quarter wave are 16 token rows), and with two or four token fragments per weight fragment those
+// loads, not the weights, were the kernel's time: 31.6 us for the gate/up launch of 32 rows at hidden 7168, 16.6 us with
+// every lane reading one row's bytes (wrong results). A round is one chunk of every wave = 1024 contiguous columns; the
+// block moves the round's 16 MFT x 2 KB of token rows with row-contiguous requests (128 threads per row) into one of two
+// LDS buffers a round ahead, and a lane reads its fragment pieces from there (rows padded by 16 bytes). Same operands into
+// the same instructions in the same order: bit-identical. Needs the dealt chunk order (steps per wave a multiple of CH).
+template <int MODE, int MFT, int TC, int NA = 1, bool XL = false>
 __global__ __launch_bounds__(512, 1) void k_dense_bf16_splitk(const DenseParams p) {
   constexpr int NWV = 8;               // waves = parts of the contraction
   constexpr int CH = 4;                // K steps (of 32) per chunk in flight
@@ -38,7 +45,10 @@ __global__ __launch_bounds__(512, 1) void k_dense_bf16_splitk(const DenseParams 
   static_assert(MODE != 0 || NA == 1, "gate/up blocks hold one fragment");
   constexpr int RR = MODE == 0 ? 2 * TC : TC;  // distinct weight rows of the fragment
   static_assert(RR == 16 || RR == 8, "fragment rows");
-  __shared__ __attribute__((aligned(16))) float red[NWV][NA * MFT][64][4];
+  constexpr int XROWS = 16 * MFT, XRS = 2048 + 16, XBUF = XROWS * XRS;  // XL: token rows, bytes per row and per buffer
+  extern __shared__ __attribute__((aligned(16))) uint8_t xl_lds[];        // XL: two token buffers, then the partial tiles
+  __shared__ __attribute__((aligned(16))) float red_s[XL ? 4 : NWV * NA * MFT * 64 * 4];
+  float* red = XL ? reinterpret_cast<float*>(xl_lds) : red_s;             // [wave][fragment][lane][4]
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = uni(tid >> 6);
   const int K = p.K, N = p.N;
@@ -98,6 +108,63 @@ __global__ __launch_bounds__(512, 1) void k_dense_bf16_splitk(const DenseParams 
       }
     }
   };
+  if constexpr (XL) {
+    // token rows of a round: thread (piece tid % 128, row tid / 128 + 4 k)
+    constexpr int TP = XROWS / 4;
+    u32x4 tv[TP];
+    const int piece = tid & 127, rsub = tid >> 7;
+    auto load_tokens = [&](int r) {
+#pragma unroll
+      for (int k = 0; k < TP; ++k)
+        tv[k] = load16(p.x + size_t(min(m0 + 4 * k + rsub, p.rows - 1)) * K + size_t(r) * 1024 + piece * 8);
+    };
+    auto store_tokens = [&](int r) {
+#pragma unroll
+      for (int k = 0; k < TP; ++k) *reinterpret_cast<u32x4*>(xl_lds + (r & 1) * XBUF + (4 * k + rsub) * XRS + piece * 16) = tv[k];
+    };
+    auto request_w = [&](auto slot_, int s0) {
+      constexpr int s_ = decltype(slot_)::value;
+#pragma unroll
+      for (int j = 0; j < CH; ++j) {
+        const int st = step_k(min(s0 + j, steps - 1));
+#pragma unroll
+        for (int a = 0; a < NA; ++a) wa[s_][j][a] = load16(wr[a] + st);
+      }
+    };
+    auto multiply_l = [&](auto slot_, int r) {
+      constexpr int s_ = decltype(slot_)::value;
+      const uint8_t* tok = xl_lds + (r & 1) * XBUF + i * XRS + (wave * CH) * 64 + 16 * c;
+#pragma unroll
+      for (int j = 0; j < CH; ++j) {
+#pragma unroll
+        for (int m = 0; m < MFT; ++m) {
+          const u32x4 xv = *reinterpret_cast<const u32x4*>(tok + 16 * m * XRS + j * 64);
+#pragma unroll
+          for (int a = 0; a < NA; ++a)
+            acc[a][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(w16_bf16x8, wa[s_][j][a]), __builtin_bit_cast(w16_bf16x8, xv),
+                                                               acc[a][m], 0, 0, 0);
+        }
+      }
+    };
+    const int rounds = steps / CH;
+    load_tokens(0);
+    request_w(std::integral_constant<int, 0>{}, 0);
+    store_tokens(0);
+    if (rounds > 1) load_tokens(1);
+    __syncthreads();
+    auto round = [&](auto slot_, int r) {
+      constexpr int s_ = decltype(slot_)::value;
+      if (r + 1 < rounds) request_w(std::integral_constant<int, s_ ^ 1>{}, (r + 1) * CH);
+      multiply_l(slot_, r);
+      if (r + 1 < rounds) store_tokens(r + 1);
+      if (r + 2 < rounds) load_tokens(r + 2);
+      __syncthreads();
+    };
+    for (int r = 0; r < rounds; r += 2) {
+      round(std::integral_constant<int, 0>{}, r);
+      if (r + 1 < rounds) round(std::integral_constant<int, 1>{}, r + 1);
+    }
+  } else {
   static_for<NBUF - 1>([&](auto ib) { request(ib, decltype(ib)::value * CH); });
   for (int s0 = 0; s0 < steps; s0 += NBUF * CH) {
     static_for<NBUF>([&](auto ib) {
@@ -106,12 +173,13 @@ __global__ __launch_bounds__(512, 1) void k_dense_bf16_splitk(const DenseParams 
       multiply(ib, s0 + b * CH);
     });
   }
+  }
 
   // the eight partial tiles, added in wave order
 #pragma unroll
   for (int a = 0; a < NA; ++a)
 #pragma unroll
-    for (int m = 0; m < MFT; ++m) *reinterpret_cast<v4f*>(&red[wave][a * MFT + m][lane][0]) = acc[a][m];
+    for (int m = 0; m < MFT; ++m) *reinterpret_cast<v4f*>(red + ((wave * (NA * MFT) + a * MFT + m) * 64 + lane) * 4) = acc[a][m];
   __syncthreads();
   // wave m < MFT finishes token fragment m: lane (token i, group c) holds weight rows 4c .. 4c+3 of the fragment. MODE 0:
   // the first TC / 4 groups are gate columns n0 .. n0 + TC - 1 and the next TC / 4 the same columns of up, so a lane of the
@@ -125,12 +193,12 @@ __global__ __launch_bounds__(512, 1) void k_dense_bf16_splitk(const DenseParams 
 #pragma unroll
       for (int a = 0; a < (MODE == 0 ? 2 : 1); ++a) {
         const int src = lane + 4 * TC * a;  // the up rows sit TC rows = TC / 4 lane groups further on
-        const v4f first = *reinterpret_cast<const v4f*>(&red[0][f * MFT + m][src][0]);
+        const v4f first = *reinterpret_cast<const v4f*>(red + ((f * MFT + m) * 64 + src) * 4);
 #pragma unroll
         for (int r = 0; r < 4; ++r) v[a][r] = first[r];
 #pragma unroll
         for (int w = 1; w < NWV; ++w) {
-          const v4f part = *reinterpret_cast<const v4f*>(&red[w][f * MFT + m][src][0]);
+          const v4f part = *reinterpret_cast<const v4f*>(red + ((w * (NA * MFT) + f * MFT + m) * 64 + src) * 4);
 #pragma unroll
           for (int r = 0; r < 4; ++r) v[a][r] = __fadd_rn(v[a][r], part[r]);
         }

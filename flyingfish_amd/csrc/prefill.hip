@@ -562,11 +562,23 @@ int shared_expert_w16(const ffmoe_shared_expert* shared, const void* x, int R, i
     const unsigned gy = unsigned((R + 16 * mft - 1) / (16 * mft));
     DenseParams d{};
     d.rows = R; d.swiglu = swiglu; d.limit = limit;
+    // up to 32 rows the token panel goes through LDS (two buffers of 32 rows x 2 KB, a round ahead); it needs every wave's steps
+    // in whole chunks of four, i.e. contractions that are multiples of 1024 (FFMOE_SPLITK_LDS=0: requested in lane order; same bits)
+    const char* xe = getenv("FFMOE_SPLITK_LDS");
+    constexpr size_t xl_bytes = size_t(2) * 32 * (2048 + 16);
+    static int xl_ok = -1;
+    if (xl_ok < 0) {
+      xl_ok = hipFuncSetAttribute(reinterpret_cast<const void*>(k_dense_bf16_splitk<0, 2, 8, 1, true>), hipFuncAttributeMaxDynamicSharedMemorySize, int(xl_bytes)) == hipSuccess &&
+              hipFuncSetAttribute(reinterpret_cast<const void*>(k_dense_bf16_splitk<2, 2, 16, 2, true>), hipFuncAttributeMaxDynamicSharedMemorySize, int(xl_bytes)) == hipSuccess ? 1 : 0;
+      if (!xl_ok) (void)hipGetLastError();
+    }
+    const bool xl = mft == 2 && xl_ok == 1 && !(xe && atoi(xe) == 0);
     if (stage_mask & 1) {
       d.x = (const uint16_t*)x; d.w0 = (const uint16_t*)shared->slot[0]; d.w1 = (const uint16_t*)shared->slot[2];
       d.out = (uint16_t*)act; d.K = H; d.N = SI;
       const dim3 grid(unsigned(SI / 8), gy);
       if (mft == 4) hipLaunchKernelGGL((k_dense_bf16_splitk<0, 4, 8>), grid, dim3(512), 0, stream, d);
+      else if (xl && H % 1024 == 0) hipLaunchKernelGGL((k_dense_bf16_splitk<0, 2, 8, 1, true>), grid, dim3(512), xl_bytes, stream, d);
       else hipLaunchKernelGGL((k_dense_bf16_splitk<0, 2, 8>), grid, dim3(512), 0, stream, d);
       FF_TRY(ff_launch_status());
     }
@@ -576,6 +588,7 @@ int shared_expert_w16(const ffmoe_shared_expert* shared, const void* x, int R, i
       // two fragments = 32 output columns per block (32 rows at hidden 7168: 15.2 us against 20.6 with one and 20.7 with four)
       const dim3 grid(unsigned(H / 32), gy);
       if (mft == 4) hipLaunchKernelGGL((k_dense_bf16_splitk<2, 4, 16, 2>), grid, dim3(512), 0, stream, d);
+      else if (xl && SI % 1024 == 0) hipLaunchKernelGGL((k_dense_bf16_splitk<2, 2, 16, 2, true>), grid, dim3(512), xl_bytes, stream, d);
       else hipLaunchKernelGGL((k_dense_bf16_splitk<2, 2, 16, 2>), grid, dim3(512), 0, stream, d);
       FF_TRY(ff_launch_status());
     }

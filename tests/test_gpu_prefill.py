@@ -511,6 +511,43 @@ def test_prefill_bf16_shared_expert_on_the_split_contraction_kernel(rows, hidden
     assert_close_bf16(sh_act, out["0"][2], "shared activations against the grouped kernels", max_ulp=4)
 
 
+@pytest.mark.parametrize("rows,hidden,inter", [(4, 1024, 1024), (17, 2048, 1024), (32, 3072, 2048), (25, 1024, 2048), (32, 7168, 2048)])
+def test_prefill_split_contraction_kernel_with_the_token_panel_in_lds_bitwise(rows, hidden, inter, monkeypatch):
+    """Up to 32 rows, contractions that are multiples of 1024: the split-contraction kernel moves its token panel through LDS
+    with row-contiguous requests instead of requesting it in the matrix instruction's lane order. Same operands into the same
+    instructions in the same order: activations and shared output are the bits of the lane-order kernel
+    (FFMOE_SPLITK_LDS=0), whose parity test_prefill_bf16_shared_expert_on_the_split_contraction_kernel holds; the first
+    rows are also checked against the oracle here, since no shape of that test takes this path."""
+    from helpers import make_table
+    top_k, experts = 2, 3
+    table, ref = make_table(capi.FMT_BF16, experts + 1, hidden, inter, 1930 + rows)
+    sh = table.shared_struct(experts)
+    table.experts = experts
+    ids, w = _routing(rows, top_k, experts, 1940 + rows, 0.5)
+    x = synth.normal((rows, hidden), 1.0, 1950 + rows, dtype=torch.bfloat16)
+    monkeypatch.setenv("FFMOE_PREFILL_SHARED_RIDE", "0")
+    monkeypatch.setenv("FFMOE_SHARED_SPLITK", "1")
+    out = {}
+    for lds in ("0", "1"):
+        monkeypatch.setenv("FFMOE_SPLITK_LDS", lds)
+        op = ops.PrefillOps(table, rows, top_k, swiglu=capi.SWIGLU_TWICE, swiglu_limit=0.0, routed_weight=capi.WEIGHT_AFTER_DOWN_BF16, weights_f32=True,
+                            shared=sh, act_mode=capi.ACT_BF16)
+        op.contributions.zero_(); op.shared_out.zero_(); op.scratch.zero_()
+        print("split contraction rows=%d hidden=%d inter=%d token panel in LDS=%s" % (rows, hidden, inter, lds), flush=True)
+        op.contribute(x.cuda(), torch.from_numpy(ids).cuda(), torch.from_numpy(w).cuda())
+        torch.cuda.synchronize()
+        out[lds] = (bits(op.shared_out).copy(), bits(op.scratch_views()["sh_act"]).copy())
+    assert np.array_equal(out["0"][1], out["1"][1]), "shared activations"
+    assert np.array_equal(out["0"][0], out["1"][0]), "shared output"
+    assert np.any(out["1"][0] != 0)
+    ge, ue, de = ref[experts]
+    xb = bits(x)
+    for r in sorted({0, rows // 2, rows - 1}):
+        _, want_act = orc.expert_ffn(xb[r], ge, ue, de, 1.0, capi.SWIGLU_TWICE, 0.0, 0, orc.LANE8, orc.SILU_DIV, apply_weight=False, return_act=True)
+        assert_close_bf16(out["1"][1][r][None, :], want_act[None, :], "shared activations row %d" % r)
+        assert_close_bf16(out["1"][0][r][None, :], orc.expert_down(out["1"][1][r], de, 1.0, 0, orc.LANE8, False)[None, :], "shared down row %d" % r)
+
+
 @pytest.mark.parametrize("fmt,switch", [(capi.FMT_NVFP4, "FFMOE_PREFILL_NVFP4_LINES"), (capi.FMT_FP8_BLOCK128, "FFMOE_PREFILL_FP8_LINES")])
 @pytest.mark.parametrize("rows,mf,hidden,inter", [(70, "1", 512, 256), (70, "4", 256, 768), (9, "2", 1024, 256), (150, "2", 256, 512), (200, "wide", 768, 512),
                                                   (33, "1", 384, 640)])
