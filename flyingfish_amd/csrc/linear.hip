@@ -374,35 +374,36 @@ int num_cus_l() {
   return g_cus_l;
 }
 
+template <class F, int RG, int SMAX, int S = 1>
+void launch_linear_steps(int want, const LinearParams& p, int blocks, size_t lds, hipStream_t st) {
+  if constexpr (S <= SMAX) {
+    if (want == S) hipLaunchKernelGGL((k_linear<F, S, RG, 1>), dim3(blocks), dim3(256), lds, st, p);
+    else launch_linear_steps<F, RG, SMAX, S + 1>(want, p, blocks, lds, st);
+  }
+}
+
 template <class F>
 int launch_linear(const LinearParams& p, hipStream_t st) {
   // rows per pass bounded by 64 KiB of LDS
   int blocks = num_cus_l() * 2;
   if (blocks > (p.n + 3) / 4) blocks = (p.n + 3) / 4;
   const size_t row = size_t(p.k) * 2;
-  // Weight rows per unit: one. A single call is bound by its start-up, and more rows per unit, which pay in the batched entry,
-  // change nothing or lose here (FFMOE_LINEAR_NR=2 / 4, same bits: M = 1 8.8 us either way, M = 4 at K 7168 11.7 against 9.1 us).
-  // NVFP4, whose split-dot operands of one row take the registers four FP8 rows do, has no other instantiation.
-  constexpr bool one_row_units = std::is_same<F, FmtNvfp4>::value;
-  int nr = 1;
-  if (const char* e = getenv("FFMOE_LINEAR_NR")) { const int v = atoi(e); if (v == 1 || v == 2 || v == 4) nr = v; }
-  auto go = [&](auto rg, auto nrc) {
-    constexpr int RG = decltype(rg)::value, NR = decltype(nrc)::value;
-    hipLaunchKernelGGL((k_linear<F, 4, RG, NR>), dim3(blocks), dim3(256), RG * row, st, p);
+  // Steps of a weight row held in flight at once: slabs of at most four, the row cut into equal slabs (K 2048: two steps, no
+  // masked ones). A single call is bound by its start-up - the whole row of seven steps in flight (FFMOE_LINEAR_SMAX=8; same
+  // bits) measures 6.74 against 6.37 us at M = 1, K 7168, and more weight rows per unit, which pay in the batched entry, change
+  // nothing or lose. NVFP4 rows hold their split-dot operands in registers and cannot take more than four.
+  const int steps = (p.k / F::EPL + 63) / 64;
+  constexpr int SMAX = std::is_same<F, FmtNvfp4>::value ? 4 : 8;
+  int smax = 4;
+  if (const char* e = getenv("FFMOE_LINEAR_SMAX")) { const int v = atoi(e); if (v >= 1 && v <= SMAX) smax = v; }
+  auto steps_per_slab = [&](int cap) {  // the row in equal slabs of at most cap steps
+    const int nslabs = (steps + cap - 1) / cap;
+    return (steps + nslabs - 1) / nslabs;
   };
-  auto with_rg = [&](auto rg) {
-    constexpr int RG = decltype(rg)::value;
-    if constexpr (one_row_units) {
-      go(rg, std::integral_constant<int, 1>{});
-    } else {
-      if (nr == 4 && RG == 1) go(std::integral_constant<int, 1>{}, std::integral_constant<int, 4>{});
-      else if (nr >= 2 && RG <= 4) go(rg, std::integral_constant<int, 2>{});
-      else go(rg, std::integral_constant<int, 1>{});
-    }
-  };
-  if (p.m > 4 && 8 * row <= 64 * 1024) with_rg(std::integral_constant<int, 8>{});
-  else if (p.m > 1 && 4 * row <= 64 * 1024) with_rg(std::integral_constant<int, 4>{});
-  else with_rg(std::integral_constant<int, 1>{});
+  const int S = steps_per_slab(smax);
+  if (p.m > 4 && 8 * row <= 64 * 1024) launch_linear_steps<F, 8, 4>(steps_per_slab(smax < 4 ? smax : 4), p, blocks, 8 * row, st);
+  else if (p.m > 1 && 4 * row <= 64 * 1024) launch_linear_steps<F, 4, SMAX>(S, p, blocks, 4 * row, st);
+  else launch_linear_steps<F, 1, SMAX>(S, p, blocks, row, st);
   return ff_launch_status();
 }
 
