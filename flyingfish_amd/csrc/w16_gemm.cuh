@@ -551,8 +551,12 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void k_w16_grouped(const 
 // k_w16_grouped<FmtNvfp4>, results equal bit for bit.
 // Loads per thread and stage, in issue order: the token chunks of tile kb+3 (two tiles are in flight, in two register
 // sets), then, in the first K block of a set, the nine weight loads of the set P ahead.
-template <int MF, int MODE, int P, int NW = 4>
-__global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void k_w16_nvfp4_lines(const W16Params p) {
+// OCC: blocks per CU the kernel is compiled for. With one set of lines ahead (P = 1) the 16-row kernel holds 143 registers and
+// three blocks fit a CU: the conversion work (two VALU instructions per weight) is what bounds NVFP4 cohorts, and a third wave
+// per SIMD keeps the vector ALUs busier than a second set of lines in flight does (C4 layer, 32 tokens: 1022 -> 943 us; 8
+// tokens: 405 -> 362 us). Four blocks would need 128 registers, which spills.
+template <int MF, int MODE, int P, int NW = 4, int OCC = (NW == 4 ? 2 : 1)>
+__global__ __launch_bounds__(64 * NW, OCC) void k_w16_nvfp4_lines(const W16Params p) {
   using F = FmtNvfp4;
   constexpr int NT = 64 * NW;
   constexpr int TM = 16 * MF;
@@ -765,6 +769,9 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void k_w16_nvfp4_lines(co
 template <int MF, int MODE, int P, int NW = 4>
 __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void k_w16_fp8_lines(const W16Params p) {
   using F = FmtFp8;
+  // a set's slot is requested into again after the set's first K block: with a single set the second K block would read the
+  // next set's lines (measured: wrong bits). With two sets the kernel holds 183 - 187 registers, so two blocks per CU it is.
+  static_assert(P >= 2, "the block-FP8 line kernel needs two sets of lines");
   constexpr int NT = 64 * NW;
   constexpr int TM = 16 * MF;
   constexpr int CHUNKS = TM * 8;
