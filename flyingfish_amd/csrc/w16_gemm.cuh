@@ -769,9 +769,11 @@ __global__ __launch_bounds__(64 * NW, OCC) void k_w16_nvfp4_lines(const W16Param
 template <int MF, int MODE, int P, int NW = 4>
 __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void k_w16_fp8_lines(const W16Params p) {
   using F = FmtFp8;
-  // a set's slot is requested into again after the set's first K block: with a single set the second K block would read the
-  // next set's lines (measured: wrong bits). With two sets the kernel holds 183 - 187 registers, so two blocks per CU it is.
-  static_assert(P >= 2, "the block-FP8 line kernel needs two sets of lines");
+  // One set of lines ahead (P = 1, 116 - 121 registers, up to four blocks per CU) comes out of the register allocator with
+  // copies of token registers that have loads in flight at the K loop's back edge (v_mov_b64 of a hand-issued load's
+  // destination: flagged by the check of the generated assembly, and wrong bits on the GPU), with the loads' destinations as
+  // outputs and as in/out operands alike. Not instantiated; with two sets the kernel holds 183 - 187 registers, two blocks per CU.
+  static_assert(P >= 2, "the block-FP8 line kernel with one set of lines is miscompiled (in-flight register copies)");
   constexpr int NT = 64 * NW;
   constexpr int TM = 16 * MF;
   constexpr int CHUNKS = TM * 8;
