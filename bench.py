@@ -987,7 +987,7 @@ def secondary(args, torch, capi, ops, synth, fp8_table):
     import copy
     sec = {}
     fp8 = (fp8_table, fp8_table.shared_struct_kept)
-    for batch, steps in ((8, 60), (64, 24)):
+    for batch, steps in ((8, 60), (64, 32)):
         a = copy.copy(args)
         a.batch, a.ring, a.steps, a.warmup, a.calibrate_copy, a.no_cpu_baseline = batch, 16, steps, 4, 0, True
         out, _ = decode_main(a, torch, capi, ops, synth, prebuilt=fp8)
@@ -1005,7 +1005,7 @@ def secondary(args, torch, capi, ops, synth, fp8_table):
         "parity": out["parity"], "cpu_baseline": out.get("cpu_baseline")}
     del out
     nv = None
-    for batch, steps, ring in ((32, 24, 16), (1, 100, 64)):
+    for batch, steps, ring in ((32, 48, 16), (1, 100, 64)):
         a = copy.copy(args)
         a.format, a.batch, a.ring, a.steps, a.warmup, a.calibrate_copy, a.no_cpu_baseline = "nvfp4", batch, ring, steps, 4, 0, True
         out, t = decode_main(a, torch, capi, ops, synth, prebuilt=nv)
