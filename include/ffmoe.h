@@ -136,7 +136,10 @@ int ffmoe_route_noaux_decode(const void* x, const void* router, const float* bia
                              int n_group, int topk_group, void* stream);
 
 /* Fused decode route: BF16 logits (stored) then softmax/sigmoid top-k.
- * Replaces RouteOps::route / moe_route_decode_bf16 (route.rs:450-499; kernels/moe_route.cu:496-568). */
+ * Replaces RouteOps::route / moe_route_decode_bf16 (route.rs:450-499; kernels/moe_route.cu:496-568). With at most 64
+ * experts it is ONE launch, as in the reference: the wave that runs a row's 64 logit chains holds the row's logits one per
+ * lane and selects right away; with more experts a row's logits come from several blocks and the selection is a launch of
+ * its own. logits, ids and weights are the bits of ffmoe_route_logits_bf16 followed by ffmoe_route_topk either way. */
 int ffmoe_route_decode(const void* x, const void* router, void* logits, int* ids, void* weights,
                        int rows, int experts, int hidden, int top_k, int score, void* stream);
 
