@@ -419,7 +419,7 @@ int launch_w16(const W16Params& p, int mf, unsigned blocks, hipStream_t stream, 
     // rows of whole 128-byte code lines: the line-wise kernel (FFMOE_PREFILL_NVFP4_LINES=0 keeps the per-K-block one)
     if (p.K % 256 == 0 && nvfp4_lines_enabled()) {
       if (wide) hipLaunchKernelGGL((k_w16_nvfp4_lines<4, MODE, 1, 8>), dim3(blocks), dim3(512), 0, stream, p);
-      else if (mf == 1 && lines_three_blocks()) hipLaunchKernelGGL((k_w16_nvfp4_lines<1, MODE, 1, 4, 3>), dim3(blocks * 3 / 2), dim3(256), 0, stream, p);
+      else if (mf == 1 && lines_three_blocks()) hipLaunchKernelGGL((k_w16_nvfp4_lines<1, MODE, 1, 4, 3>), dim3((blocks * 3 / 2 + 7u) & ~7u), dim3(256), 0, stream, p);  // whole blocks per XCD
       else if (mf == 1) hipLaunchKernelGGL((k_w16_nvfp4_lines<1, MODE, 2>), dim3(blocks), dim3(256), 0, stream, p);
       else if (mf == 2) hipLaunchKernelGGL((k_w16_nvfp4_lines<2, MODE, 2>), dim3(blocks), dim3(256), 0, stream, p);
       else hipLaunchKernelGGL((k_w16_nvfp4_lines<4, MODE, 1>), dim3(blocks), dim3(256), 0, stream, p);
