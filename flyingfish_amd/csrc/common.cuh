@@ -51,6 +51,16 @@ __device__ __forceinline__ float e4m3_to_f32(uint8_t code) { return e4m3x2_to_f3
 
 // E4M3 code of a finite value already clamped to [-448, 448], round-to-nearest-even
 // (same function as src/fp8.rs:85-121 of the reference).
+// Four finite values inside +-448 to E4M3 by the hardware conversion (round to nearest even, OCP E4M3 on this GPU): the
+// same codes as e4m3_encode for such values (-0 -> 0x80, subnormals on the m / 512 grid), two instructions instead of four
+// software encodings. The quantizers clamp to +-448 first, so saturation and NaN handling never come into it.
+__device__ __forceinline__ uint32_t e4m3x4_encode_finite(float a, float b, float c, float d) {
+  int w = 0;
+  w = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, w, false);
+  w = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, w, true);
+  return uint32_t(w);
+}
+
 __device__ __forceinline__ uint8_t e4m3_encode(float value) {
   const uint32_t bits = __float_as_uint(value);
   const uint32_t sign = (bits >> 24) & 0x80u;

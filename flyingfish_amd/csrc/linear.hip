@@ -325,12 +325,10 @@ __global__ __launch_bounds__(256) void k_quant_fp8_128(const uint16_t* __restric
   const float scale = __fmul_rn(amax, 1.0f / 448.0f);
   if (sub == 0) scales[cell] = scale;
   const float divisor = fmaxf(scale, 1.0e-12f);
-  uint32_t out[2] = {0, 0};
+  float q[8];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const float q = fminf(448.0f, fmaxf(-448.0f, __fdiv_rn(v[i], divisor)));
-    out[i >> 2] |= uint32_t(e4m3_encode(q)) << (8 * (i & 3));
-  }
+  for (int i = 0; i < 8; ++i) q[i] = fminf(448.0f, fmaxf(-448.0f, __fdiv_rn(v[i], divisor)));
+  const uint32_t out[2] = {e4m3x4_encode_finite(q[0], q[1], q[2], q[3]), e4m3x4_encode_finite(q[4], q[5], q[6], q[7])};
   uint8_t* dst = codes + row * k + first;
   if (first + 8 <= k) {
     u32x2 o = {out[0], out[1]};

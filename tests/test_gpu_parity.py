@@ -80,6 +80,21 @@ def test_device_activation_quantizer_bits():
     codes, scales = Fp8Ops.quantize(bf16_tensor(vals))
     wc, ws = orc.quant_act_fp8_128(vals)
     assert np.array_equal(codes.cpu().numpy(), wc) and np.array_equal(scales.cpu().numpy().view(np.uint32), ws.view(np.uint32))
+    # every finite BF16 value up to 2^20 in magnitude, in two orders (sorted: groups of like-sized values, quotients near the
+    # top of the grid; shuffled: every group holds large values, quotients down to the subnormal codes and zero): the codes come
+    # from the hardware conversion, the oracle's from the reference's software encoder
+    pats = np.arange(65536, dtype=np.uint32).astype(np.uint16)
+    f = (pats.astype(np.uint32) << 16).view(np.float32)
+    keep = pats[np.isfinite(f) & (np.abs(f) <= 2.0 ** 20)]
+    keep = keep[: (keep.size // 1024) * 1024]
+    rng = np.random.default_rng(77)
+    for order in (keep, rng.permutation(keep)):
+        vals = order.reshape(-1, 1024)
+        codes, scales = Fp8Ops.quantize(bf16_tensor(vals))
+        wc, ws = orc.quant_act_fp8_128(vals)
+        assert np.array_equal(scales.cpu().numpy().view(np.uint32), ws.view(np.uint32))
+        assert np.array_equal(codes.cpu().numpy(), wc)
+        assert len(np.unique(wc)) >= 250  # (nearly) the whole code space is exercised
 
 
 def test_device_swiglu_golden_bits():
