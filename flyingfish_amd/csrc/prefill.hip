@@ -409,7 +409,14 @@ int launch_w16(const W16Params& p, int mf, unsigned blocks, hipStream_t stream, 
     // per-K-block kernel; same bits). 64-row groups keep the per-K-block kernel: two sets ahead do not fit their registers
     const char* le = getenv("FFMOE_PREFILL_FP8_LINES");
     if (!(le && atoi(le) == 0) && !wide && mf == 1) {
-      hipLaunchKernelGGL((k_w16_fp8_lines<1, MODE, 2>), dim3(blocks), dim3(256), 0, stream, p);
+      // one set of lines ahead and four blocks per CU for gate/up, three for down (FFMOE_FP8_LINES_OCC=2: two sets ahead, two
+      // blocks; 3 / 4: that many blocks for both launches; same bits). 8 tokens, gate/up | down: 308 | 161 us with two, 299 | 148
+      // with three, 292 | 153 with four blocks; 64 tokens: 1116 | 600, 1080 | 568, 1051 | 569
+      const char* oe = getenv("FFMOE_FP8_LINES_OCC");
+      const int occ = oe ? atoi(oe) : (MODE == 0 ? 4 : 3);
+      if (occ == 3) hipLaunchKernelGGL((k_w16_fp8_lines<1, MODE, 1, 4, 3>), dim3((blocks * 3 / 2 + 7u) & ~7u), dim3(256), 0, stream, p);
+      else if (occ == 4) hipLaunchKernelGGL((k_w16_fp8_lines<1, MODE, 1, 4, 4>), dim3(blocks * 2), dim3(256), 0, stream, p);
+      else hipLaunchKernelGGL((k_w16_fp8_lines<1, MODE, 2>), dim3(blocks), dim3(256), 0, stream, p);
       return ff_launch_status();
     }
   }

@@ -766,14 +766,15 @@ __global__ __launch_bounds__(64 * NW, OCC) void k_w16_nvfp4_lines(const W16Param
 // Block-FP8 experts the same way: 128 columns of a row are one 128-byte line, a set is two K blocks, and the block scale of a
 // pair of fragments and a set is one float (a pair's 32 rows lie inside one 128-row block). Bit-identical to
 // k_w16_grouped<FmtFp8>, whose requests take half a line per K block and rely on L2 for the other half.
-template <int MF, int MODE, int P, int NW = 4>
-__global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void k_w16_fp8_lines(const W16Params p) {
+template <int MF, int MODE, int P, int NW = 4, int OCC = (NW == 4 ? 2 : 1)>
+__global__ __launch_bounds__(64 * NW, OCC) void k_w16_fp8_lines(const W16Params p) {
   using F = FmtFp8;
-  // One set of lines ahead (P = 1, 116 - 121 registers, up to four blocks per CU) comes out of the register allocator with
-  // copies of token registers that have loads in flight at the K loop's back edge (v_mov_b64 of a hand-issued load's
-  // destination: flagged by the check of the generated assembly, and wrong bits on the GPU), with the loads' destinations as
-  // outputs and as in/out operands alike. Not instantiated; with two sets the kernel holds 183 - 187 registers, two blocks per CU.
-  static_assert(P >= 2, "the block-FP8 line kernel with one set of lines is miscompiled (in-flight register copies)");
+  // One set of lines ahead (P = 1): 118 - 123 registers instead of 183 - 187, so three or four blocks fit a CU (OCC; 36 KB of LDS
+  // per block), and more waves per SIMD beat a second set of lines in flight here too (C3 layer, 64 tokens: 1736 -> 1647 us; 8
+  // tokens: 481 -> 461 us). Its K loop covers TWO sets per trip: with one set per trip (two stages) the register allocator
+  // split the token registers' live ranges at the back edge and restored them with v_mov_b64 while their loads were in flight
+  // (flagged by the check of the generated assembly; wrong bits on the GPU, with the loads' destinations as outputs and as
+  // in/out operands alike); with four stages per trip it does not.
   constexpr int NT = 64 * NW;
   constexpr int TM = 16 * MF;
   constexpr int CHUNKS = TM * 8;
@@ -782,7 +783,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void k_w16_fp8_lines(cons
   constexpr int WL = 10;                     // weight loads per set of two K blocks: eight of codes, two block scales
   // 16-row groups (the cohorts of a decode batch) see an expert's codes once: streaming hint on their whole-line requests
   constexpr bool STREAM = MF == 1;
-  constexpr int U = 2 * P;                   // stages per trip of the K loop
+  constexpr int U = P == 1 ? 4 : 2 * P;      // stages per trip of the K loop (one set ahead: two sets per trip)
   __shared__ __attribute__((aligned(16))) uint8_t cstage[NW][2][4096];  // [wave][pair of fragments][32 rows x 128 B]
   __shared__ __attribute__((aligned(16))) uint8_t tile[2][TILE];
   const int tid = threadIdx.x, lane = tid & 63;
@@ -897,7 +898,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void k_w16_fp8_lines(cons
       static_for<U>([&](auto st_) {
         constexpr int st = decltype(st_)::value;
         const int kb = kbo + st;
-        constexpr int q = st & 1, s = st >> 1;  // K block inside its set, register slot of the set
+        constexpr int q = st & 1, s = (st >> 1) % P;  // K block inside its set, register slot of the set
         if (kb < KB) {
           if (q == 0) {
             // the set was requested 2 P stages ago: behind it the token loads of 2 P - 1 stages and P - 1 later sets
