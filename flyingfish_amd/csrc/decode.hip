@@ -348,8 +348,9 @@ static int decode_dispatch(const ffmoe_expert_table* table, const ffmoe_shared_e
   }
   // Row counts from which the matrix-core cohort kernels take over for block-FP8 experts (same effective weights and BF16
   // boundaries, the dot products in the matrix instruction's FP32 order instead of the wave's). The whole batch goes there
-  // from FFMOE_DECODE_COHORT_ROWS on: 4 when the shared expert rides in the routed launches (same format and width, or no
-  // shared expert), 32 when it needs launches of its own, a few dozen blocks each. Per layer at hidden 7168 / 256 experts
+  // from FFMOE_DECODE_COHORT_ROWS on: 3 when a block-FP8 shared expert rides in the routed launches (same format and width, or no
+  // shared expert; with the four-block line kernel: 2 rows 186 / 166 us, 3 rows 220 / 235, 4 rows 264 / 312), 32 when it needs
+  // launches of its own, a few dozen blocks each. Per layer at hidden 7168 / 256 experts
   // with a riding shared expert, cohort (whole-line kernel) against streaming kernels: 2 rows 200 / 166 us, 3 rows 236 / 235,
   // 4 rows 277 / 313, 6 rows 368 / 433, 8 rows 485 / 554, 16 rows 810 / 939, 32 rows 1278 / 1550, 64 rows 1730 / 2402. Below
   // that a block-FP8 shared expert alone from FFMOE_DECODE_SHARED_COHORT_ROWS on (it has every row: streamed once instead of
@@ -365,7 +366,8 @@ static int decode_dispatch(const ffmoe_expert_table* table, const ffmoe_shared_e
   const char* te = getenv("FFMOE_DECODE_SHARED_STREAM_ROWS");
   const bool rides = !shared || (table && shared->format == table->format && shared->inter == table->inter);
   const bool nv_lines = table && table->format == FFMOE_FMT_NVFP4 && table->hidden % 256 == 0 && table->inter % 256 == 0;
-  const int cohort_rows = ce ? atoi(ce) : (rides || nv_lines ? 4 : 32), shared_rows = se ? atoi(se) : 16;
+  const bool fp8_rides = rides && table && table->format == FFMOE_FMT_FP8_BLOCK128;
+  const int cohort_rows = ce ? atoi(ce) : (fp8_rides ? 3 : (rides || nv_lines ? 4 : 32)), shared_rows = se ? atoi(se) : 16;
   // a BF16 shared expert that the split-contraction kernel takes (dense_splitk.cuh) leaves the streaming kernels with the
   // routed choices, at 4 rows: hidden 7168 next to NVFP4 experts, 4 / 8 / 16 / 24 rows: 249 / 413 / 665 / 859 us per layer
   // against 263 / 434 / 691 / 917 with the shared expert streaming
