@@ -105,6 +105,23 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
     constexpr int SS = decltype(kind)::steps;
     constexpr bool NVF = std::is_same<FF, FmtNvfp4>::value;
     int expert, gn, grow[RG], gslot[RG];
+    // One row per call: the slot entries of the choice are requested next to the checks of its id (valid flag, epoch), not
+    // behind them - one round trip to L2 in front of the first weight request instead of two.
+    uint64_t slv[6] = {0, 0, 0, 0, 0, 0};
+    float glv[3] = {1.0f, 1.0f, 1.0f};
+    bool early = false;
+    if (!p.groups && g < A) {
+      const int e = inline_ids ? uni(inline_ids[g]) : uni(load_global<int>(p.ids + g));
+      if ((unsigned)e < (unsigned)p.experts) {
+        early = true;
+#pragma unroll
+        for (int i = 0; i < 6; ++i) slv[i] = load_global<uint64_t>(p.slots + size_t(e) * 6 + i);
+        if (p.global_scales) {
+#pragma unroll
+          for (int i = 0; i < 3; ++i) glv[i] = load_global<float>(p.global_scales + size_t(e) * 3 + i);
+        }
+      }
+    }
     load_group<RG>(p, g, expert, gn, grow, gslot, inline_ids);
     const bool shared = expert < 0;
     const int Kg = STAGE == 0 ? p.hidden : (shared ? p.shared_inter : p.inter);
@@ -117,6 +134,11 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
         for (int i = 0; i < 6; ++i) sl[i] = p.shared_slot[i];
 #pragma unroll
         for (int i = 0; i < 3; ++i) gl3[i] = p.shared_global[i];
+      } else if (early) {
+#pragma unroll
+        for (int i = 0; i < 6; ++i) sl[i] = uni64(slv[i]);
+#pragma unroll
+        for (int i = 0; i < 3; ++i) gl3[i] = unif(glv[i]);
       } else {
 #pragma unroll
         for (int i = 0; i < 6; ++i) sl[i] = uni64(load_global<uint64_t>(p.slots + size_t(expert) * 6 + i));
