@@ -616,6 +616,7 @@ __global__ __launch_bounds__(64 * NW, OCC) void k_w16_nvfp4_lines(const W16Param
       const int row = min(second ? col0[2] : col0[0], N - 32) + (lane & 31);
       nscl = reinterpret_cast<const uint8_t*>(MODE == 0 && second ? un_.ws[1] : un_.ws[0]) + size_t(row) * (K >> 4);
     }
+    const uint8_t* nscl_first = reinterpret_cast<const uint8_t*>(un_.ws[0]);  // one valid line for requests past the last set
     u32x4 nvc[P][2][4], nvs[P];
 
     const uint8_t* tsrc[CPT];
@@ -637,14 +638,22 @@ __global__ __launch_bounds__(64 * NW, OCC) void k_w16_nvfp4_lines(const W16Param
 #pragma unroll
       for (int f = 0; f < 4; ++f) acc[m][f] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
 
-#define FF_NV_REQUEST(s_, sb_)                                                                          \
+    // nx_: the set asked for. Past the last set the requests only keep the hand-counted number of loads per stage constant
+    // and nothing reads them: every one of them then asks for the same line (the first row's last set) instead of the last
+    // set's 64 rows once more - with the streaming hint those lines have left L2 by then and came from HBM a second time,
+    // 32 KB per block and unit (an eighth of a down unit's bytes).
+#define FF_NV_REQUEST(s_, nx_)                                                                          \
   do {                                                                                                   \
+    const bool past_ = P == 1 && int(nx_) >= SB; /* two sets ahead: the last set once more, as before */ \
+    const uint32_t sb_ = uint32_t(min(int(nx_), SB - 1));                                                \
+    const uint32_t rs_ = past_ ? 0u : rstep;                                                             \
+    const uint32_t co_ = past_ ? uint32_t(lane & 7) * 16u : coff;                                        \
     _Pragma("unroll") for (int j_ = 0; j_ < 2; ++j_)                                                     \
       _Pragma("unroll") for (int i_ = 0; i_ < 4; ++i_) {                                                 \
-        if constexpr (STREAM) load16_async_nt(nvc[s_][j_][i_], ncod[j_] + uint32_t(i_) * rstep + (sb_) * 128u, coff); \
-        else load16_async(nvc[s_][j_][i_], ncod[j_] + uint32_t(i_) * rstep + (sb_) * 128u, coff);        \
+        if constexpr (STREAM) load16_async_nt(nvc[s_][j_][i_], ncod[j_] + uint32_t(i_) * rs_ + sb_ * 128u, co_); \
+        else load16_async(nvc[s_][j_][i_], ncod[j_] + uint32_t(i_) * rs_ + sb_ * 128u, co_);             \
       }                                                                                                  \
-    load16_async(nvs[s_], nscl + (sb_) * 16u);                                                           \
+    load16_async(nvs[s_], past_ ? nscl_first : nscl + sb_ * 16u);                                         \
   } while (0)
 #define FF_NV_PIN(s_)                                                                                    \
   do {                                                                                                   \
@@ -654,7 +663,7 @@ __global__ __launch_bounds__(64 * NW, OCC) void k_w16_nvfp4_lines(const W16Param
   } while (0)
     // prologue: the first P weight sets and token tile 0, everything landed; then token tiles 1 and 2
 #pragma unroll
-    for (int s = 0; s < P; ++s) FF_NV_REQUEST(s, uint32_t(min(s, SB - 1)));
+    for (int s = 0; s < P; ++s) FF_NV_REQUEST(s, s);
     u32x4 tv[2][CPT];
     {
 #pragma unroll
@@ -747,7 +756,7 @@ __global__ __launch_bounds__(64 * NW, OCC) void k_w16_nvfp4_lines(const W16Param
           const uint32_t kt = uint32_t(min(kb + 3, KB - 1));
 #pragma unroll
           for (int i = 0; i < CPT; ++i) load16_async(tv[(st + 1) & 1][i], tsrc[i] + kt * 128u);
-          if (q == 0) FF_NV_REQUEST(s, uint32_t(min((kb >> 2) + P, SB - 1)));
+          if (q == 0) FF_NV_REQUEST(s, (kb >> 2) + P);
         }
       });
     }
@@ -845,14 +854,19 @@ __global__ __launch_bounds__(64 * NW, OCC) void k_w16_fp8_lines(const W16Params 
 #pragma unroll
       for (int f = 0; f < 4; ++f) acc[m][f] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
 
-#define FF_NV_REQUEST(s_, sb_)                                                                          \
+    // nx_: the set asked for; past the last set every request asks for one and the same line (see k_w16_nvfp4_lines)
+#define FF_NV_REQUEST(s_, nx_)                                                                          \
   do {                                                                                                   \
+    const bool past_ = P == 1 && int(nx_) >= SB; /* two sets ahead: the last set once more, as before */ \
+    const uint32_t sb_ = uint32_t(min(int(nx_), SB - 1));                                                \
+    const uint32_t rs_ = past_ ? 0u : rstep;                                                             \
+    const uint32_t co_ = past_ ? uint32_t(lane & 7) * 16u : coff;                                        \
     _Pragma("unroll") for (int j_ = 0; j_ < 2; ++j_)                                                     \
       _Pragma("unroll") for (int i_ = 0; i_ < 4; ++i_) {                                                 \
-        if constexpr (STREAM) load16_async_nt(nvc[s_][j_][i_], ncod[j_] + uint32_t(i_) * rstep + (sb_) * 128u, coff); \
-        else load16_async(nvc[s_][j_][i_], ncod[j_] + uint32_t(i_) * rstep + (sb_) * 128u, coff);        \
+        if constexpr (STREAM) load16_async_nt(nvc[s_][j_][i_], ncod[j_] + uint32_t(i_) * rs_ + sb_ * 128u, co_); \
+        else load16_async(nvc[s_][j_][i_], ncod[j_] + uint32_t(i_) * rs_ + sb_ * 128u, co_);             \
       }                                                                                                  \
-    _Pragma("unroll") for (int j_ = 0; j_ < 2; ++j_) load4_async(nvs[s_][j_], nscl[j_] + (sb_));            \
+    _Pragma("unroll") for (int j_ = 0; j_ < 2; ++j_) load4_async(nvs[s_][j_], nscl[j_] + sb_);             \
   } while (0)
 #define FF_NV_PIN(s_)                                                                                    \
   do {                                                                                                   \
@@ -860,10 +874,10 @@ __global__ __launch_bounds__(64 * NW, OCC) void k_w16_fp8_lines(const W16Params 
       _Pragma("unroll") for (int i_ = 0; i_ < 4; ++i_) pin(nvc[s_][j_][i_]);                             \
     _Pragma("unroll") for (int j_ = 0; j_ < 2; ++j_) pin(nvs[s_][j_]);                                     \
   } while (0)
-    // prologue: the first P weight sets and token tile 0, everything landed; then token tile 1, the last set once more
-    // (a tile has one set's loads and the next tile behind it when it is published) and token tile 2
+    // prologue: the first P - 1 weight sets and token tile 0, everything landed; then token tile 1, set P - 1 (a tile has
+    // one set's loads and the next tile behind it when it is published) and token tile 2
 #pragma unroll
-    for (int s = 0; s < P; ++s) FF_NV_REQUEST(s, uint32_t(min(s, SB - 1)));
+    for (int s = 0; s + 1 < P; ++s) FF_NV_REQUEST(s, s);
     u32x4 tv[2][CPT];
     {
 #pragma unroll
@@ -873,11 +887,11 @@ __global__ __launch_bounds__(64 * NW, OCC) void k_w16_fp8_lines(const W16Params 
       }
       wait_vm<0>();
 #pragma unroll
-      for (int s = 0; s < P; ++s) FF_NV_PIN(s);
+      for (int s = 0; s + 1 < P; ++s) FF_NV_PIN(s);
       const uint32_t k1 = uint32_t(min(1, KB - 1)), k2 = uint32_t(min(2, KB - 1));
 #pragma unroll
       for (int i = 0; i < CPT; ++i) load16_async(tv[1][i], tsrc[i] + k1 * 128u);
-      FF_NV_REQUEST(P - 1, uint32_t(min(P - 1, SB - 1)));
+      FF_NV_REQUEST(P - 1, P - 1);
 #pragma unroll
       for (int i = 0; i < CPT; ++i) load16_async(tv[0][i], tsrc[i] + k2 * 128u);
     }
@@ -957,7 +971,7 @@ __global__ __launch_bounds__(64 * NW, OCC) void k_w16_fp8_lines(const W16Params 
           const uint32_t kt = uint32_t(min(kb + 3, KB - 1));
 #pragma unroll
           for (int i = 0; i < CPT; ++i) load16_async(tv[(st + 1) & 1][i], tsrc[i] + kt * 128u);
-          if (q == 0) FF_NV_REQUEST(s, uint32_t(min((kb >> 1) + P, SB - 1)));
+          if (q == 0) FF_NV_REQUEST(s, (kb >> 1) + P);
         }
       });
     }
