@@ -71,11 +71,14 @@ __global__ __launch_bounds__(MAXT) void k_decode_finish(const FinishParams q, co
       FSH::load(sbuf[MIXED ? m : 0][MIXED ? s : 0], FSH::row(uni64(p.shared_slot[4]), uni64(p.shared_slot[5]), unif(p.shared_global[2]), row, I), cc);
     }
   };
-  auto issue_rows = [&](auto which, uint64_t codes, uint64_t scales, float glob, int i, int s) {
+  // spare: a request behind the wave's last unit. It keeps the loop free of branches around its loads and nothing reads it;
+  // every lane then asks for the row's first chunk (one line per load) instead of the unit's rows once more, which, streamed,
+  // have left L2 by then and would come from HBM a second time (an eighth of the launch's bytes).
+  auto issue_rows = [&](auto which, uint64_t codes, uint64_t scales, float glob, int i, int s, bool spare = false) {
     constexpr int b_ = decltype(which)::value;
     const int j = b_lo + i * NR;
     const int chunk = s * 64 + lane;
-    const int cc = chunk < nchunks ? chunk : nchunks - 1;
+    const int cc = spare ? 0 : (chunk < nchunks ? chunk : nchunks - 1);
 #pragma unroll
     for (int m = 0; m < NR; ++m) {
       const int row = j + m < b_hi ? j + m : b_hi - 1;  // a ragged last unit repeats the block's last row
@@ -213,7 +216,7 @@ __global__ __launch_bounds__(MAXT) void k_decode_finish(const FinishParams q, co
   auto issue_unit = [&](auto which, int t, int s) {
     int g, i;
     unit_of(t, g, i);
-    issue_rows(which, uni64(s_codes[g]), uni64(s_scales[g]), unif(s_glob[g]), i, s);
+    issue_rows(which, uni64(s_codes[g]), uni64(s_scales[g]), unif(s_glob[g]), i, s, t >= my_units);
   };
   if (my_units > 0) {
     if (!first_shared || (MIXED && my_units > lead)) {  // MIXED: the first routed unit goes out next to the shared ones, into its own registers
