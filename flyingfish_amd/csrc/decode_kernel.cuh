@@ -100,7 +100,9 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
 
   // One segment: `count` units of group g from unit j0 on, split over the waves wv = 0 .. nw-1 (wv < 0: this wave only
   // takes part in the staging and the barriers).
-  auto segment = [&](auto kind, int g, int j0, int count, int nw, int wv, const int* inline_ids) {
+  // staged: the group's activation row is in LDS already (one token: the routed segments behind the shared slice read the
+  // same token row) - no second copy behind the segment's first weight requests, and without a table to build no barrier
+  auto segment = [&](auto kind, int g, int j0, int count, int nw, int wv, const int* inline_ids, bool staged = false) {
     using FF = typename decltype(kind)::fmt;
     constexpr int SS = decltype(kind)::steps;
     constexpr bool NVF = std::is_same<FF, FmtNvfp4>::value;
@@ -190,13 +192,14 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
       for (int s = 0; s < SS; ++s) issue_step(0, s);
     }
     // activations of the group -> LDS (row r at r*Kg*2), behind the first weight requests
-    __syncthreads();  // the previous segment's readers are done with xs
-    if (gn > 0) {
+    const bool skip_staging = staged && !NVF;  // wave-uniform, block-uniform
+    if (!skip_staging) __syncthreads();  // the previous segment's readers are done with xs
+    if (gn > 0 && !skip_staging) {
       const uint16_t* src = STAGE == 0 ? p.x : p.h;
       const int row_words = Kg >> 3;  // 16-byte words per row
 #pragma unroll
       for (int r = 0; r < RG; ++r) {
-        if (r < gn) {
+        if (r < gn && !staged) {
           const size_t base = STAGE == 0 ? size_t(grow[r]) * p.hidden : size_t(gslot[r]) * p.h_stride;
           u32x4* d4 = reinterpret_cast<u32x4*>(xs + size_t(r) * Kg * 2);
           for (int v = tid; v < row_words; v += 256) d4[v] = load16(src + base + size_t(v) * 8);
@@ -207,7 +210,7 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
         if (STAGE == 0) FmtNvfp4::build_lut(s_lut + FmtNvfp4::LUT_ENTRIES, global[1], tid, 256);
       }
     }
-    __syncthreads();
+    if (!skip_staging) __syncthreads();
     if (items > 0) {
       float acc[NROWS][RG];
       float park[NROWS][RG];  // lane L keeps the sums of unit (batch base + L)
@@ -284,6 +287,19 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
   };
 
   if (STAGE == 0 && RG == 1) {
+    // 256 experts: wave 0 asks for its four logits and biases per lane before anything else of this CU is in the memory
+    // pipeline; asked for behind the shared slice (below) they wait for the waves' first weight rows, which the vector memory
+    // pipeline of the CU serves first (2 - 4 us in front of the selection)
+    constexpr int PC = 4;
+    float pre_l[PC] = {0.0f, 0.0f, 0.0f, 0.0f}, pre_b[PC] = {0.0f, 0.0f, 0.0f, 0.0f};
+    const bool preloaded = inline_route && shared_first && p.experts == 64 * PC;
+    if (preloaded && wave == 0) {
+#pragma unroll
+      for (int j = 0; j < PC; ++j) {
+        pre_l[j] = load_global<float>(p.route.logits + lane * PC + j);
+        if (p.route.bias) pre_b[j] = load_global<float>(p.route.bias + lane * PC + j);
+      }
+    }
     if (shared_first) {
       // this block's slice of the shared expert (group A: rows == 1), waves 1..3; wave 0 selects meanwhile
       const int s_lo = int((long long)out_s * blockIdx.x / gridDim.x), s_hi = int((long long)out_s * (blockIdx.x + 1) / gridDim.x);
@@ -291,7 +307,10 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
     }
     if (inline_route) {
       const int select_k = p.route.select_k > 0 ? p.route.select_k : p.top_k;
-      if (wave == 0)
+      if (wave == 0 && preloaded)
+        wave_route_row_preloaded<PC>(pre_l, pre_b, lane, p.experts, select_k, p.route.score_mode, p.route.routed_scaling, p.route.n_group,
+                                     p.route.topk_group, s_route_ids, s_route_w, 1);
+      else if (wave == 0)
         wave_route_dispatch(p.route.logits, p.route.bias, lane, p.experts, select_k, p.route.score_mode, p.route.routed_scaling,
                             p.route.n_group, p.route.topk_group, s_route_ids, s_route_w, 1);
       __syncthreads();
@@ -336,7 +355,8 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
     if (u0 < routed_units) { g = int(u0 / out_r); j0 = int(u0 % out_r); width = out_r; }
     else { const long long v = u0 - routed_units; g = n_routed + int(v / out_s); j0 = int(v % out_s); width = out_s; }
     const long long seg_end = u0 + (width - j0) < hi ? u0 + (width - j0) : hi;
-    segment(SegmentKind<F, S>{}, g, j0, int(seg_end - u0), 4, wave, inline_route ? s_route_ids : nullptr);
+    segment(SegmentKind<F, S>{}, g, j0, int(seg_end - u0), 4, wave, inline_route ? s_route_ids : nullptr,
+            STAGE == 0 && RG == 1 && shared_first && p.rows == 1 && g < A);
     u0 = seg_end;
   }
 }

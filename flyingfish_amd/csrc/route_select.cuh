@@ -121,6 +121,20 @@ __device__ __forceinline__ void wave_route_row(const float* __restrict__ logits_
   wave_select_noaux<C>(score, select, lane, experts, top_k, routed_scaling, n_group, topk_group, ids_row, weights_row, weights_f32);
 }
 
+// the same with the lane's C logits and biases already in registers (fetched early by the caller)
+template <int C>
+__device__ __forceinline__ void wave_route_row_preloaded(const float (&l)[C], const float (&b)[C], int lane, int experts, int top_k, int score_mode,
+                                                         float routed_scaling, int n_group, int topk_group, int* ids_row, void* weights_row,
+                                                         int weights_f32) {
+  float score[C], select[C];
+#pragma unroll
+  for (int j = 0; j < C; ++j) {
+    score[j] = noaux_score(l[j], score_mode);
+    select[j] = __fadd_rn(score[j], b[j]);
+  }
+  wave_select_noaux<C>(score, select, lane, experts, top_k, routed_scaling, n_group, topk_group, ids_row, weights_row, weights_f32);
+}
+
 __device__ __forceinline__ void wave_route_dispatch(const float* logits_row, const float* bias_row, int lane, int experts,
                                                     int top_k, int score_mode, float routed_scaling, int n_group,
                                                     int topk_group, int* ids_row, void* weights_row, int weights_f32) {
