@@ -34,6 +34,16 @@ __device__ __forceinline__ uint64_t wave_max_u64(uint64_t v) {
   return (uint64_t(hi) << 32) | lo;
 }
 
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
+  v = max(v, uint32_t(dpp_or<DPP_QUAD_SWAP1, 0xf>(int(v), int(v))));
+  v = max(v, uint32_t(dpp_or<DPP_QUAD_SWAP2, 0xf>(int(v), int(v))));
+  v = max(v, uint32_t(dpp_or<DPP_ROW_HALF_MIRROR, 0xf>(int(v), int(v))));
+  v = max(v, uint32_t(dpp_or<DPP_ROW_MIRROR, 0xf>(int(v), int(v))));
+  v = max(v, uint32_t(dpp_or<DPP_ROW_BCAST15, 0xa>(int(v), int(v))));
+  v = max(v, uint32_t(dpp_or<DPP_ROW_BCAST31, 0xc>(int(v), int(v))));
+  return uint32_t(__builtin_amdgcn_readlane(int(v), 63));
+}
+
 // One wave selects for one row. Requires experts == 64 * C and, with groups, experts / n_group a multiple of C whose
 // lane span is a power of two. score[] = unbiased scores, select[] = score + bias of the lane's C candidates.
 template <int C>
@@ -52,12 +62,22 @@ __device__ __forceinline__ void wave_select_noaux(const float (&score)[C], const
       a = fmaxf(a, v);
     }
     const int span = (experts / n_group) / C;  // lanes per group
-    for (int off = 1; off < span; off <<= 1) {
-      const float oa = __shfl_xor(a, off, 64), ob = __shfl_xor(b, off, 64);
+    // Merging the two largest of two disjoint sets of lanes is symmetric, and after a level all lanes of a merged set hold
+    // the same pair, so the partner may be any lane of the neighbouring set: the cross-lane modes of the vector ALU reach
+    // one for sets of up to 8 lanes (pairs, quads, the mirrored half row, the mirrored row); wider sets go through LDS.
+    auto merge = [&](float oa, float ob) {
       const float na = fmaxf(a, oa);
       b = fmaxf(fminf(a, oa), fmaxf(b, ob));
       a = na;
-    }
+    };
+    auto fdpp = [](auto ctrl, float v) {
+      return __builtin_bit_cast(float, dpp_or<decltype(ctrl)::value, 0xf>(__builtin_bit_cast(int, v), __builtin_bit_cast(int, v)));
+    };
+    if (span > 1) merge(fdpp(std::integral_constant<int, DPP_QUAD_SWAP1>{}, a), fdpp(std::integral_constant<int, DPP_QUAD_SWAP1>{}, b));
+    if (span > 2) merge(fdpp(std::integral_constant<int, DPP_QUAD_SWAP2>{}, a), fdpp(std::integral_constant<int, DPP_QUAD_SWAP2>{}, b));
+    if (span > 4) merge(fdpp(std::integral_constant<int, DPP_ROW_HALF_MIRROR>{}, a), fdpp(std::integral_constant<int, DPP_ROW_HALF_MIRROR>{}, b));
+    if (span > 8) merge(fdpp(std::integral_constant<int, DPP_ROW_MIRROR>{}, a), fdpp(std::integral_constant<int, DPP_ROW_MIRROR>{}, b));
+    for (int off = 16; off < span; off <<= 1) merge(__shfl_xor(a, off, 64), __shfl_xor(b, off, 64));
     const float gscore = __fadd_rn(a, b);
     const int g = lane / span;
     // rank of the lane's group among the groups under (score desc, id asc)
@@ -68,13 +88,45 @@ __device__ __forceinline__ void wave_select_noaux(const float (&score)[C], const
     }
     allowed = rank < topk_group;
   }
+  float tsum = 0.0f;
+  float my_w = 0.0f;  // lane r keeps the score of the r-th pick
+  int my_id = 0;
+  // Enough candidates for top_k picks (every sane configuration): a round is the wave maximum of the 32-bit orderable scores
+  // and then the lowest id that has it - the order of the 64-bit keys below (score descending, id ascending: ids ascend
+  // with the lane and inside the lane), in a quarter of the dependent instructions.
+  const int candidates = __builtin_popcountll(__ballot(allowed)) * C;
+  if (candidates >= top_k) {
+    uint32_t k32[C];
+#pragma unroll
+    for (int j = 0; j < C; ++j) k32[j] = allowed ? orderable(select[j]) : 0u;  // 0: below every score, also -inf
+    for (int r = 0; r < top_k; ++r) {
+      uint32_t m = k32[0];
+#pragma unroll
+      for (int j = 1; j < C; ++j) m = max(m, k32[j]);
+      const uint32_t win = wave_max_u32(m);
+      int first = C;
+      float sc = 0.0f;
+#pragma unroll
+      for (int j = C - 1; j >= 0; --j) {
+        const bool hit = k32[j] == win;
+        first = hit ? j : first;
+        sc = hit ? score[j] : sc;
+      }
+      const unsigned long long hits = __ballot(first < C);
+      const int wl = __builtin_ctzll(hits);  // a retired or barred candidate (0) never equals a live maximum
+      const int jw = __builtin_amdgcn_readlane(first, wl);
+      const int id = wl * C + jw;
+#pragma unroll
+      for (int j = 0; j < C; ++j) k32[j] = (lane == wl && j == jw) ? 0u : k32[j];
+      const float wsc = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, sc), wl));
+      tsum = __fadd_rn(tsum, wsc);
+      if (lane == r) { my_w = wsc; my_id = id; }
+    }
+  } else {
   uint64_t key[C];
 #pragma unroll
   for (int j = 0; j < C; ++j)
     key[j] = allowed ? (uint64_t(orderable(select[j])) << 32) | uint32_t(~uint32_t(lane * C + j)) : 0ull;
-  float tsum = 0.0f;
-  float my_w = 0.0f;  // lane r keeps the score of the r-th pick
-  int my_id = 0;
   for (int r = 0; r < top_k; ++r) {
     uint64_t best = key[0];
 #pragma unroll
@@ -91,6 +143,7 @@ __device__ __forceinline__ void wave_select_noaux(const float (&score)[C], const
     const float wsc = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, sc), id / C));
     tsum = __fadd_rn(tsum, wsc);
     if (lane == r) { my_w = wsc; my_id = id; }
+  }
   }
   if (lane < top_k) {
     const float w = __fmul_rn(__fdiv_rn(my_w, __fadd_rn(tsum, 1.0e-20f)), routed_scaling);
