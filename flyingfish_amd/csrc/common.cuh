@@ -368,6 +368,13 @@ __device__ __forceinline__ T load_global(const void* p) {
   return *(const FF_GLOBAL T*)(p);
 }
 __device__ __forceinline__ u32x4 load16(const void* p) { return load_global<u32x4>(p); }
+// A load of a value every lane of the wave wants from the same address (tables written by earlier launches): through the
+// scalar data cache, so it neither queues with the wave's vector requests nor counts against their hand-counted waits.
+#define FF_CONSTANT __attribute__((address_space(4)))
+template <class T>
+__device__ __forceinline__ T load_uniform(const void* p) {
+  return *(const FF_CONSTANT T*)(p);
+}
 // A copy of a loaded value that is known to have arrived. The compiler waits for a load where its result is first
 // read; inside a loop it repeats that wait in every iteration when the load was issued before the loop, and because
 // loads retire in order such a wait also drains every younger load in flight. Reading the value once through this

@@ -98,50 +98,64 @@ __global__ __launch_bounds__(64 * NW, (NW == 4 && MF <= 4) ? 2 : 1) void k_w8a8_
   const uint32_t xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3, per_xcd = gridDim.x >> 3;
   const uint32_t span = (total + 7u) >> 3;
   const uint32_t span_end = min(total, (xcd + 1u) * span);
-  for (uint32_t u = xcd * span + slot; u < span_end; u += per_xcd) {
-
-    int expert, start, n, t;
+  // What a unit is and where its expert's matrices are: unit list -> group record -> slot table, three loads that depend on
+  // each other. They are wave-uniform and go through the scalar cache, and the next unit's chain is walked while this unit's
+  // first weights are on their way (one block of this kernel fills a CU, so nothing else would hide the three round trips
+  // in front of every unit's first weight request).
+  struct UnitDesc { int expert, start, n, t; uint64_t wc[2], ws[2]; float nvg[2]; };
+  auto fetch_unit = [&](uint32_t u) {
+    UnitDesc d;
     if (p.groups) {
-      const u32x2 un = load_global<u32x2>(p.units + u);
-      const int g = uni(int(un.x));
-      t = uni(int(un.y));
+      const u32x2 un = load_uniform<u32x2>(p.units + u);
+      const int g = int(un.x);
+      d.t = int(un.y);
       const int* gd = reinterpret_cast<const int*>(p.groups + g);
-      expert = uni(load_global<int>(gd));
-      start = uni(load_global<int>(gd + 1));
-      n = uni(load_global<int>(gd + 2));
+      d.expert = load_uniform<int>(gd);
+      d.start = load_uniform<int>(gd + 1);
+      d.n = load_uniform<int>(gd + 2);
     } else {
       const int g = int(u) / ntiles;
-      t = int(u) - g * ntiles;
-      expert = 0;
-      start = g * TM;
-      n = min(TM, p.rows_total - start);
+      d.t = int(u) - g * ntiles;
+      d.expert = 0;
+      d.start = g * TM;
+      d.n = min(TM, p.rows_total - d.start);
     }
-
-    // weight fragments of this wave
-    uint64_t wc[2], ws[2];
     if (p.slots) {
-      const uint64_t* sl = p.slots + size_t(expert) * 6;
+      const uint64_t* sl = p.slots + size_t(d.expert) * 6;
       if (MODE == 0) {
-        wc[0] = uni64(load_global<uint64_t>(sl + 0)); ws[0] = uni64(load_global<uint64_t>(sl + 1));
-        wc[1] = uni64(load_global<uint64_t>(sl + 2)); ws[1] = uni64(load_global<uint64_t>(sl + 3));
+        d.wc[0] = load_uniform<uint64_t>(sl + 0); d.ws[0] = load_uniform<uint64_t>(sl + 1);
+        d.wc[1] = load_uniform<uint64_t>(sl + 2); d.ws[1] = load_uniform<uint64_t>(sl + 3);
       } else {
-        wc[0] = wc[1] = uni64(load_global<uint64_t>(sl + 4)); ws[0] = ws[1] = uni64(load_global<uint64_t>(sl + 5));
+        d.wc[0] = d.wc[1] = load_uniform<uint64_t>(sl + 4); d.ws[0] = d.ws[1] = load_uniform<uint64_t>(sl + 5);
       }
     } else {
-      wc[0] = p.w0_codes; ws[0] = p.w0_scales;
-      wc[1] = MODE == 0 ? p.w1_codes : p.w0_codes; ws[1] = MODE == 0 ? p.w1_scales : p.w0_scales;
+      d.wc[0] = p.w0_codes; d.ws[0] = p.w0_scales;
+      d.wc[1] = MODE == 0 ? p.w1_codes : p.w0_codes; d.ws[1] = MODE == 0 ? p.w1_scales : p.w0_scales;
     }
-    float nvg[2] = {1.0f, 1.0f};  // NV: 8 x the matrix's global scale stands in for every block scale
+    d.nvg[0] = d.nvg[1] = 1.0f;  // NV: 8 x the matrix's global scale stands in for every block scale
     if constexpr (NV) {
       if (p.slots) {
-        const float* gl = p.global_scales + size_t(expert) * 3;
-        nvg[0] = unif(load_global<float>(gl + (MODE == 0 ? 0 : 2)));
-        nvg[1] = MODE == 0 ? unif(load_global<float>(gl + 1)) : nvg[0];
+        const float* gl = p.global_scales + size_t(d.expert) * 3;
+        d.nvg[0] = load_uniform<float>(gl + (MODE == 0 ? 0 : 2));
+        d.nvg[1] = MODE == 0 ? load_uniform<float>(gl + 1) : d.nvg[0];
       } else {
-        nvg[0] = p.w0_global; nvg[1] = MODE == 0 ? p.w1_global : p.w0_global;
+        d.nvg[0] = p.w0_global; d.nvg[1] = MODE == 0 ? p.w1_global : p.w0_global;
       }
-      nvg[0] = __fmul_rn(nvg[0], 8.0f); nvg[1] = __fmul_rn(nvg[1], 8.0f);
+      d.nvg[0] = __fmul_rn(d.nvg[0], 8.0f); d.nvg[1] = __fmul_rn(d.nvg[1], 8.0f);
     }
+    return d;
+  };
+  constexpr bool AHEAD = !NV;  // (next to the NVFP4 conversion the chain walked ahead costs scalar registers it does not have: measured slower)
+  const uint32_t u_first = xcd * span + slot;
+  UnitDesc next_unit = {};
+  if (AHEAD && u_first < span_end) next_unit = fetch_unit(u_first);
+  for (uint32_t u = u_first; u < span_end; u += per_xcd) {
+    if (!AHEAD) next_unit = fetch_unit(u);
+    const UnitDesc unit = next_unit;
+    const int expert = unit.expert, start = unit.start, n = unit.n, t = unit.t;
+    (void)expert;
+    const uint64_t wc[2] = {unit.wc[0], unit.wc[1]}, ws[2] = {unit.ws[0], unit.ws[1]};
+    const float nvg[2] = {unit.nvg[0], unit.nvg[1]};
     // first output column of fragment f; fragments past N are clamped onto the last 16 rows and dropped at the store
     int col0[4];
     // weight addresses: a wave-uniform base per fragment (scalar registers) and one byte offset per lane
@@ -279,6 +293,8 @@ __global__ __launch_bounds__(64 * NW, (NW == 4 && MF <= 4) ? 2 : 1) void k_w8a8_
         if (stage_chunk) *reinterpret_cast<u32x4*>(&tile[0][tdst[i]]) = v;
       }
       if (tid < TM) *reinterpret_cast<float*>(&tile[0][TM * 128 + tid * 4]) = load_global<float>(ssrc);
+      // the next unit's descriptor chain, under the round trip of this unit's first weights
+      if (AHEAD && u + per_xcd < span_end) next_unit = fetch_unit(u + per_xcd);
       FF_DRAIN_WEIGHTS();
       if constexpr (TW) {
         // K block 0 goes into the wave's transposition buffer; stage 0 requests token tile 1 itself
