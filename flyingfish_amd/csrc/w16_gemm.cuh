@@ -181,13 +181,13 @@ template <int MODE>
 __device__ __forceinline__ W16Unit w16_unit(const W16Params& p, uint32_t u, int ntiles, int TM) {
   int expert, start, n, t;
   if (p.groups) {
-    const u32x2 un = load_global<u32x2>(p.units + u);
-    const int g = uni(int(un.x));
-    t = uni(int(un.y));
+    const u32x2 un = load_uniform<u32x2>(p.units + u);
+    const int g = int(un.x);
+    t = int(un.y);
     const int* gd = reinterpret_cast<const int*>(p.groups + g);
-    expert = uni(load_global<int>(gd));
-    start = uni(load_global<int>(gd + 1));
-    n = uni(load_global<int>(gd + 2));
+    expert = load_uniform<int>(gd);
+    start = load_uniform<int>(gd + 1);
+    n = load_uniform<int>(gd + 2);
   } else {
     const int g = int(u) / ntiles;
     t = int(u) - g * ntiles;
@@ -206,15 +206,15 @@ __device__ __forceinline__ W16Unit w16_unit(const W16Params& p, uint32_t u, int 
   } else if (p.slots) {
     const uint64_t* sl = p.slots + size_t(expert) * 6;
     if (MODE == 0) {
-      wc[0] = uni64(load_global<uint64_t>(sl + 0)); ws[0] = uni64(load_global<uint64_t>(sl + 1));
-      wc[1] = uni64(load_global<uint64_t>(sl + 2)); ws[1] = uni64(load_global<uint64_t>(sl + 3));
+      wc[0] = load_uniform<uint64_t>(sl + 0); ws[0] = load_uniform<uint64_t>(sl + 1);
+      wc[1] = load_uniform<uint64_t>(sl + 2); ws[1] = load_uniform<uint64_t>(sl + 3);
     } else {
-      wc[0] = wc[1] = uni64(load_global<uint64_t>(sl + 4)); ws[0] = ws[1] = uni64(load_global<uint64_t>(sl + 5));
+      wc[0] = wc[1] = load_uniform<uint64_t>(sl + 4); ws[0] = ws[1] = load_uniform<uint64_t>(sl + 5);
     }
     if (p.global_scales) {
       const float* g3 = p.global_scales + size_t(expert) * 3;
-      gl[0] = unif(load_global<float>(g3 + (MODE == 0 ? 0 : 2)));
-      gl[1] = MODE == 0 ? unif(load_global<float>(g3 + 1)) : gl[0];
+      gl[0] = load_uniform<float>(g3 + (MODE == 0 ? 0 : 2));
+      gl[1] = MODE == 0 ? load_uniform<float>(g3 + 1) : gl[0];
     }
   } else {
     wc[0] = p.w0_codes; ws[0] = p.w0_scales;
