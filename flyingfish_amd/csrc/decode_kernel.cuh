@@ -28,12 +28,12 @@ __device__ __forceinline__ void load_group(const DecodeParams& p, int g, int& ex
                                            const int* inline_ids = nullptr) {
   if (p.groups) {
     const int* gd = reinterpret_cast<const int*>(p.groups + g);
-    expert = uni(load_global<int>(gd));
-    n = uni(load_global<int>(gd + 1));
+    expert = load_uniform<int>(gd);
+    n = load_uniform<int>(gd + 1);
 #pragma unroll
     for (int r = 0; r < RG; ++r) {
-      row[r] = uni(load_global<int>(gd + 2 + r));
-      slot[r] = uni(load_global<int>(gd + 2 + FFMOE_DECODE_RG + r));
+      row[r] = load_uniform<int>(gd + 2 + r);
+      slot[r] = load_uniform<int>(gd + 2 + FFMOE_DECODE_RG + r);
     }
     return;
   }
@@ -42,14 +42,14 @@ __device__ __forceinline__ void load_group(const DecodeParams& p, int g, int& ex
   for (int r = 0; r < RG; ++r) { row[r] = 0; slot[r] = 0; }
   n = 1;
   if (g < A) {
-    expert = inline_ids ? uni(inline_ids[g]) : uni(load_global<int>(p.ids + g));
+    expert = inline_ids ? uni(inline_ids[g]) : load_uniform<int>(p.ids + g);
     row[0] = g / p.top_k;
     slot[0] = g;
-    if (p.active && uni(int(load_global<uint32_t>(p.active + g))) == 0) n = 0;
+    if (p.active && int(load_uniform<uint32_t>(p.active + g)) == 0) n = 0;
     if ((unsigned)expert >= (unsigned)p.experts) n = 0;  // out-of-range id: contribute nothing, done stays 0
-    else if (p.valid && uni(int(load_global<uint32_t>(p.valid + expert))) == 0) n = 0;
+    else if (p.valid && int(load_uniform<uint32_t>(p.valid + expert)) == 0) n = 0;
     else if (p.generation && p.assignment_gen &&
-             uni64(load_global<uint64_t>(p.generation + expert)) != uni64(load_global<uint64_t>(p.assignment_gen + g))) n = 0;  // stale choice
+             load_uniform<uint64_t>(p.generation + expert) != load_uniform<uint64_t>(p.assignment_gen + g)) n = 0;  // stale choice
   } else {
     expert = -1;
     row[0] = g - A;
@@ -113,14 +113,14 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
     float glv[3] = {1.0f, 1.0f, 1.0f};
     bool early = false;
     if (!p.groups && g < A) {
-      const int e = inline_ids ? uni(inline_ids[g]) : uni(load_global<int>(p.ids + g));
+      const int e = inline_ids ? uni(inline_ids[g]) : load_uniform<int>(p.ids + g);
       if ((unsigned)e < (unsigned)p.experts) {
         early = true;
 #pragma unroll
-        for (int i = 0; i < 6; ++i) slv[i] = load_global<uint64_t>(p.slots + size_t(e) * 6 + i);
+        for (int i = 0; i < 6; ++i) slv[i] = load_uniform<uint64_t>(p.slots + size_t(e) * 6 + i);
         if (p.global_scales) {
 #pragma unroll
-          for (int i = 0; i < 3; ++i) glv[i] = load_global<float>(p.global_scales + size_t(e) * 3 + i);
+          for (int i = 0; i < 3; ++i) glv[i] = load_uniform<float>(p.global_scales + size_t(e) * 3 + i);
         }
       }
     }
@@ -143,10 +143,10 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
         for (int i = 0; i < 3; ++i) gl3[i] = unif(glv[i]);
       } else {
 #pragma unroll
-        for (int i = 0; i < 6; ++i) sl[i] = uni64(load_global<uint64_t>(p.slots + size_t(expert) * 6 + i));
+        for (int i = 0; i < 6; ++i) sl[i] = load_uniform<uint64_t>(p.slots + size_t(expert) * 6 + i);
         if (p.global_scales) {
 #pragma unroll
-          for (int i = 0; i < 3; ++i) gl3[i] = unif(load_global<float>(p.global_scales + size_t(expert) * 3 + i));
+          for (int i = 0; i < 3; ++i) gl3[i] = load_uniform<float>(p.global_scales + size_t(expert) * 3 + i);
         }
       }
     }
