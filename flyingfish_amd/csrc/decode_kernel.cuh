@@ -98,11 +98,61 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
   const int out_s = (STAGE == 0 ? p.shared_inter : p.hidden) / NR;
   const long long routed_units = (long long)n_routed * out_r;
 
+  // 256 experts: wave 0 asks for its four logits and biases per lane before anything else of this CU is in the memory
+  // pipeline; asked for behind the shared slice they wait for the waves' first weight rows, which the vector memory
+  // pipeline of the CU serves first (2 - 4 us in front of the selection)
+  constexpr int PC = 4;
+  float pre_l[PC] = {0.0f, 0.0f, 0.0f, 0.0f}, pre_b[PC] = {0.0f, 0.0f, 0.0f, 0.0f};
+  const bool preloaded = STAGE == 0 && RG == 1 && inline_route && shared_first && p.experts == 64 * PC;
+  if (preloaded && wave == 0) {
+    if (((reinterpret_cast<uintptr_t>(p.route.logits) | reinterpret_cast<uintptr_t>(p.route.bias)) & 15) == 0) {
+      // one 16-byte request per lane and array
+      const u32x4 vl = load16(p.route.logits + lane * PC);
+      u32x4 vb = {0u, 0u, 0u, 0u};
+      if (p.route.bias) vb = load16(p.route.bias + lane * PC);
+#pragma unroll
+      for (int j = 0; j < PC; ++j) {
+        const uint32_t lj = vl[j], bj = vb[j];  // a bit cast of the vector element itself reads element 0
+        pre_l[j] = __uint_as_float(lj);
+        pre_b[j] = __uint_as_float(bj);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < PC; ++j) {
+        pre_l[j] = load_global<float>(p.route.logits + lane * PC + j);
+        if (p.route.bias) pre_b[j] = load_global<float>(p.route.bias + lane * PC + j);
+      }
+    }
+  }
+  const int select_k = p.route.select_k > 0 ? p.route.select_k : p.top_k;
+  NoauxState<PC> sel;
+  // The usual router (256 experts in 8 groups of which 4 stay, sigmoid scores, 8 picks) runs a copy of the selection with
+  // these numbers as literals: two thirds of the instructions of the general one (no integer divisions, loops unrolled).
+  const bool usual_router = p.experts == 256 && p.route.n_group == 8 && p.route.topk_group == 4 && select_k == 8 &&
+                            p.route.score_mode == FFMOE_NOAUX_SIGMOID;
+  auto select_preloaded = [&]() {
+    if (usual_router) {
+      wave_route_prepare_preloaded<PC>(sel, pre_l, pre_b, lane, 256, 8, FFMOE_NOAUX_SIGMOID, 8, 4);
+      wave_select_pick<PC>(sel, lane, 8, p.route.routed_scaling, s_route_ids, s_route_w, 1);
+    } else {
+      wave_route_prepare_preloaded<PC>(sel, pre_l, pre_b, lane, p.experts, select_k, p.route.score_mode, p.route.n_group, p.route.topk_group);
+      wave_select_pick<PC>(sel, lane, select_k, p.route.routed_scaling, s_route_ids, s_route_w, 1);
+    }
+  };
+  bool sel_inside = false;  // the selection ran inside the shared slice's staging, in front of its barrier
+  // Wave 0 selects inside the shared slice's staging, between asking for its share of the token row and writing it to LDS:
+  // the slice's first barrier is dropped (nothing has read the token buffer yet; the other waves reach it only once the
+  // memory pipeline has taken their first weight requests, microseconds after entry), so wave 0 asks for its share and
+  // selects while the other waves' shares are still behind their weight rows, and the barrier behind the staging is also the
+  // one behind the selection.
+  constexpr bool EARLY = !NV;
+  const bool select_early = EARLY && preloaded;
+
   // One segment: `count` units of group g from unit j0 on, split over the waves wv = 0 .. nw-1 (wv < 0: this wave only
   // takes part in the staging and the barriers).
   // staged: the group's activation row is in LDS already (one token: the routed segments behind the shared slice read the
   // same token row) - no second copy behind the segment's first weight requests, and without a table to build no barrier
-  auto segment = [&](auto kind, int g, int j0, int count, int nw, int wv, const int* inline_ids, bool staged = false) {
+  auto segment = [&](auto kind, int g, int j0, int count, int nw, int wv, const int* inline_ids, bool staged = false, bool with_select = false) {
     using FF = typename decltype(kind)::fmt;
     constexpr int SS = decltype(kind)::steps;
     constexpr bool NVF = std::is_same<FF, FmtNvfp4>::value;
@@ -193,7 +243,7 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
     }
     // activations of the group -> LDS (row r at r*Kg*2), behind the first weight requests
     const bool skip_staging = staged && !NVF;  // wave-uniform, block-uniform
-    if (!skip_staging) __syncthreads();  // the previous segment's readers are done with xs
+    if (!skip_staging && !with_select) __syncthreads();  // the previous segment's readers are done with xs
     if (gn > 0 && !skip_staging) {
       const uint16_t* src = STAGE == 0 ? p.x : p.h;
       const int row_words = Kg >> 3;  // 16-byte words per row
@@ -202,7 +252,24 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
         if (r < gn && !staged) {
           const size_t base = STAGE == 0 ? size_t(grow[r]) * p.hidden : size_t(gslot[r]) * p.h_stride;
           u32x4* d4 = reinterpret_cast<u32x4*>(xs + size_t(r) * Kg * 2);
-          for (int v = tid; v < row_words; v += 256) d4[v] = load16(src + base + size_t(v) * 8);
+          if (EARLY && RG == 1 && with_select) sel_inside = true;  // block-uniform
+          if (EARLY && RG == 1 && with_select && wave == 0) {
+            // wave 0: its share of the row is asked for (rows of up to 8192 values: held in registers), then it selects,
+            // then the share goes to LDS
+            const bool in_regs = row_words <= 1024;
+            u32x4 st[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              if (in_regs && tid + 256 * i < row_words) st[i] = load16(src + base + size_t(tid + 256 * i) * 8);
+            select_preloaded();
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              if (in_regs && tid + 256 * i < row_words) d4[tid + 256 * i] = st[i];
+            if (!in_regs)
+              for (int v = tid; v < row_words; v += 256) d4[v] = load16(src + base + size_t(v) * 8);
+          } else {
+            for (int v = tid; v < row_words; v += 256) d4[v] = load16(src + base + size_t(v) * 8);
+          }
         }
       }
       if constexpr (NVF) {
@@ -287,33 +354,17 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
   };
 
   if (STAGE == 0 && RG == 1) {
-    // 256 experts: wave 0 asks for its four logits and biases per lane before anything else of this CU is in the memory
-    // pipeline; asked for behind the shared slice (below) they wait for the waves' first weight rows, which the vector memory
-    // pipeline of the CU serves first (2 - 4 us in front of the selection)
-    constexpr int PC = 4;
-    float pre_l[PC] = {0.0f, 0.0f, 0.0f, 0.0f}, pre_b[PC] = {0.0f, 0.0f, 0.0f, 0.0f};
-    const bool preloaded = inline_route && shared_first && p.experts == 64 * PC;
-    if (preloaded && wave == 0) {
-#pragma unroll
-      for (int j = 0; j < PC; ++j) {
-        pre_l[j] = load_global<float>(p.route.logits + lane * PC + j);
-        if (p.route.bias) pre_b[j] = load_global<float>(p.route.bias + lane * PC + j);
-      }
-    }
     if (shared_first) {
       // this block's slice of the shared expert (group A: rows == 1), waves 1..3; wave 0 selects meanwhile
       const int s_lo = int((long long)out_s * blockIdx.x / gridDim.x), s_hi = int((long long)out_s * (blockIdx.x + 1) / gridDim.x);
-      segment(SegmentKind<FSH, SSH>{}, A, s_lo, s_hi - s_lo, 3, wave - 1, nullptr);
+      segment(SegmentKind<FSH, SSH>{}, A, s_lo, s_hi - s_lo, 3, wave - 1, nullptr, false, select_early);
     }
     if (inline_route) {
-      const int select_k = p.route.select_k > 0 ? p.route.select_k : p.top_k;
-      if (wave == 0 && preloaded)
-        wave_route_row_preloaded<PC>(pre_l, pre_b, lane, p.experts, select_k, p.route.score_mode, p.route.routed_scaling, p.route.n_group,
-                                     p.route.topk_group, s_route_ids, s_route_w, 1);
-      else if (wave == 0)
+      if (!EARLY && wave == 0 && preloaded) select_preloaded();
+      else if (wave == 0 && !sel_inside)
         wave_route_dispatch(p.route.logits, p.route.bias, lane, p.experts, select_k, p.route.score_mode, p.route.routed_scaling,
                             p.route.n_group, p.route.topk_group, s_route_ids, s_route_w, 1);
-      __syncthreads();
+      if (!sel_inside) __syncthreads();
       if (blockIdx.x == 0 && tid < select_k) {
         const_cast<int*>(p.ids)[tid] = s_route_ids[tid];
         reinterpret_cast<float*>(const_cast<void*>(p.weights))[tid] = s_route_w[tid];

@@ -34,22 +34,39 @@ __device__ __forceinline__ uint64_t wave_max_u64(uint64_t v) {
   return (uint64_t(hi) << 32) | lo;
 }
 
+// Wave maximum, returned in a scalar register. The cross-lane modes ride on the max itself (the compiler emits a move with
+// the mode and a separate max); the waits the cross-lane reads need behind a vector write are spelled out, the
+// compiler does not look into the block.
 __device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
-  v = max(v, uint32_t(dpp_or<DPP_QUAD_SWAP1, 0xf>(int(v), int(v))));
-  v = max(v, uint32_t(dpp_or<DPP_QUAD_SWAP2, 0xf>(int(v), int(v))));
-  v = max(v, uint32_t(dpp_or<DPP_ROW_HALF_MIRROR, 0xf>(int(v), int(v))));
-  v = max(v, uint32_t(dpp_or<DPP_ROW_MIRROR, 0xf>(int(v), int(v))));
-  v = max(v, uint32_t(dpp_or<DPP_ROW_BCAST15, 0xa>(int(v), int(v))));
-  v = max(v, uint32_t(dpp_or<DPP_ROW_BCAST31, 0xc>(int(v), int(v))));
-  return uint32_t(__builtin_amdgcn_readlane(int(v), 63));
+  uint32_t out;
+  asm volatile(
+      "s_nop 1\n\tv_max_u32_dpp %1, %1, %1 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+      "s_nop 1\n\tv_max_u32_dpp %1, %1, %1 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+      "s_nop 1\n\tv_max_u32_dpp %1, %1, %1 row_half_mirror row_mask:0xf bank_mask:0xf\n\t"
+      "s_nop 1\n\tv_max_u32_dpp %1, %1, %1 row_mirror row_mask:0xf bank_mask:0xf\n\t"
+      "s_nop 1\n\tv_max_u32_dpp %1, %1, %1 row_bcast:15 row_mask:0xa bank_mask:0xf\n\t"
+      "s_nop 1\n\tv_max_u32_dpp %1, %1, %1 row_bcast:31 row_mask:0xc bank_mask:0xf\n\t"
+      "s_nop 1\n\tv_readlane_b32 %0, %1, 63\n\ts_nop 3"
+      : "=s"(out), "+v"(v));
+  return out;
 }
 
-// One wave selects for one row. Requires experts == 64 * C and, with groups, experts / n_group a multiple of C whose
-// lane span is a power of two. score[] = unbiased scores, select[] = score + bias of the lane's C candidates.
+// One wave selects for one row, in two parts so that a caller can do the first before something it has to wait for and the
+// second behind it. Requires experts == 64 * C and, with groups, experts / n_group a multiple of C whose lane span is a
+// power of two. score[] = unbiased scores, select[] = score + bias of the lane's C candidates.
 template <int C>
-__device__ __forceinline__ void wave_select_noaux(const float (&score)[C], const float (&select)[C], int lane, int experts,
-                                                  int top_k, float routed_scaling, int n_group, int topk_group,
-                                                  int* __restrict__ ids_row, void* __restrict__ weights_row, int weights_f32) {
+struct NoauxState {
+  float score[C], select[C];
+  uint32_t key[C];  // heads form: the lane's candidates in pick order, barred and retired ones 0
+  int pos[C];       // the register index (id % C) that goes with key[]
+  bool allowed;     // the lane's group passed the group filter
+  bool heads;       // wave-uniform: enough candidates for top_k picks and few enough per lane to sort them
+};
+
+// Part one: group filter, keys, the lane's candidates sorted.
+template <int C>
+__device__ __forceinline__ void wave_select_prepare(NoauxState<C>& st, int lane, int experts, int top_k, int n_group, int topk_group) {
+  const float (&select)[C] = st.select;
   bool allowed = true;
   if (n_group > 1) {
     // the two largest selection scores of the lane, then of the lanes of its group (values only: the group score
@@ -88,17 +105,71 @@ __device__ __forceinline__ void wave_select_noaux(const float (&score)[C], const
     }
     allowed = rank < topk_group;
   }
+  st.allowed = allowed;
+  const int candidates = __builtin_popcountll(__ballot(allowed)) * C;
+  st.heads = C <= 8 && candidates >= top_k;
+#pragma unroll
+  for (int j = 0; j < C; ++j) { st.key[j] = allowed ? orderable(select[j]) : 0u; st.pos[j] = j; }  // 0: below every score, also -inf
+  if (st.heads) {
+    // The lane's candidates sorted once (score descending, id ascending: exchanges of neighbours only, so equal scores keep
+    // their order).
+#pragma unroll
+    for (int pass = 0; pass < C - 1; ++pass) {
+#pragma unroll
+      for (int i = 0; i < C - 1 - pass; ++i) {
+        const bool sw = st.key[i + 1] > st.key[i];
+        const uint32_t ka = sw ? st.key[i + 1] : st.key[i], kb = sw ? st.key[i] : st.key[i + 1];
+        const int pa = sw ? st.pos[i + 1] : st.pos[i], pb = sw ? st.pos[i] : st.pos[i + 1];
+        st.key[i] = ka; st.key[i + 1] = kb; st.pos[i] = pa; st.pos[i + 1] = pb;
+      }
+    }
+  }
+}
+
+// Part two: top_k rounds, normalized weights, ids and weights written by the lanes 0 .. top_k-1.
+template <int C>
+__device__ __forceinline__ void wave_select_pick(NoauxState<C>& st, int lane, int top_k, float routed_scaling,
+                                                 int* __restrict__ ids_row, void* __restrict__ weights_row, int weights_f32) {
+  const float (&score)[C] = st.score;
+  const float (&select)[C] = st.select;
+  const bool allowed = st.allowed;
   float tsum = 0.0f;
   float my_w = 0.0f;  // lane r keeps the score of the r-th pick
   int my_id = 0;
-  // Enough candidates for top_k picks (every sane configuration): a round is the wave maximum of the 32-bit orderable scores
-  // and then the lowest id that has it - the order of the 64-bit keys below (score descending, id ascending: ids ascend
-  // with the lane and inside the lane), in a quarter of the dependent instructions.
+  // Enough candidates for top_k picks (every sane configuration): rounds on 32-bit orderable scores with "the lowest id that
+  // has the maximum" - the order of the 64-bit keys at the bottom (score descending, id ascending: ids ascend with the lane
+  // and inside the lane).
   const int candidates = __builtin_popcountll(__ballot(allowed)) * C;
-  if (candidates >= top_k) {
-    uint32_t k32[C];
+  if (st.heads) {
+    // A round looks at the lanes' heads only: wave maximum, the lowest lane whose head has it, that lane pops its head.
+    // The picks' scores are fetched once at the end.
+    uint32_t (&key)[C] = st.key;
+    int (&pos)[C] = st.pos;
+    for (int r = 0; r < top_k; ++r) {
+      const uint32_t win = wave_max_u32(key[0]);
+      const int wl = __builtin_ctzll(__ballot(key[0] == win));  // a retired or barred head (0) never equals a live maximum
+      const int id = wl * C + __builtin_amdgcn_readlane(pos[0], wl);
+      const bool me = lane == wl;
 #pragma unroll
-    for (int j = 0; j < C; ++j) k32[j] = allowed ? orderable(select[j]) : 0u;  // 0: below every score, also -inf
+      for (int j = 0; j < C - 1; ++j) {
+        key[j] = me ? key[j + 1] : key[j];
+        pos[j] = me ? pos[j + 1] : pos[j];
+      }
+      key[C - 1] = me ? 0u : key[C - 1];
+      my_id = lane == r ? id : my_id;
+    }
+    // lane r < top_k: the score of pick r sits in lane id / C, register id % C
+#pragma unroll
+    for (int j = 0; j < C; ++j) {
+      const float sj = __shfl(score[j], my_id / C, 64);
+      my_w = (my_id % C) == j ? sj : my_w;
+    }
+    for (int r = 0; r < top_k; ++r)
+      tsum = __fadd_rn(tsum, __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, my_w), r)));
+  } else if (C > 8 && candidates >= top_k) {
+    // more than eight candidates per lane: a round is the wave maximum of the 32-bit orderable scores and then the lowest
+    // id that has it
+    uint32_t (&k32)[C] = st.key;
     for (int r = 0; r < top_k; ++r) {
       uint32_t m = k32[0];
 #pragma unroll
@@ -153,6 +224,17 @@ __device__ __forceinline__ void wave_select_noaux(const float (&score)[C], const
   }
 }
 
+template <int C>
+__device__ __forceinline__ void wave_select_noaux(const float (&score)[C], const float (&select)[C], int lane, int experts,
+                                                  int top_k, float routed_scaling, int n_group, int topk_group,
+                                                  int* __restrict__ ids_row, void* __restrict__ weights_row, int weights_f32) {
+  NoauxState<C> st;
+#pragma unroll
+  for (int j = 0; j < C; ++j) { st.score[j] = score[j]; st.select[j] = select[j]; }
+  wave_select_prepare<C>(st, lane, experts, top_k, n_group, topk_group);
+  wave_select_pick<C>(st, lane, top_k, routed_scaling, ids_row, weights_row, weights_f32);
+}
+
 __device__ __forceinline__ float noaux_score(float l, int score_mode) {
   if (score_mode == FFMOE_NOAUX_SIGMOID) return sigmoid1(l);
   const float softplus = __fadd_rn(fmaxf(l, 0.0f), det_log1pf_unit(det_expf(-fabsf(l))));
@@ -186,6 +268,18 @@ __device__ __forceinline__ void wave_route_row_preloaded(const float (&l)[C], co
     select[j] = __fadd_rn(score[j], b[j]);
   }
   wave_select_noaux<C>(score, select, lane, experts, top_k, routed_scaling, n_group, topk_group, ids_row, weights_row, weights_f32);
+}
+
+// Part one of the same from registers: scores, group filter, sorted candidates (part two is wave_select_pick)
+template <int C>
+__device__ __forceinline__ void wave_route_prepare_preloaded(NoauxState<C>& st, const float (&l)[C], const float (&b)[C], int lane, int experts,
+                                                             int top_k, int score_mode, int n_group, int topk_group) {
+#pragma unroll
+  for (int j = 0; j < C; ++j) {
+    st.score[j] = noaux_score(l[j], score_mode);
+    st.select[j] = __fadd_rn(st.score[j], b[j]);
+  }
+  wave_select_prepare<C>(st, lane, experts, top_k, n_group, topk_group);
 }
 
 __device__ __forceinline__ void wave_route_dispatch(const float* logits_row, const float* bias_row, int lane, int experts,
