@@ -34,6 +34,7 @@ __global__ __launch_bounds__(MAXT) void k_decode_finish(const FinishParams q, co
   __shared__ int s_expert[FFMOE_MAX_TOP_K];      // expert of choice c, -1 = not live
   __shared__ int s_choice[FFMOE_MAX_TOP_K];      // live choices in combine order
   __shared__ int s_groups;
+  __shared__ int s_next;  // the block's next unclaimed routed unit
   __shared__ uint64_t s_codes[GT], s_scales[GT];
   __shared__ float s_glob[GT], s_wk[GT];
   __shared__ int s_slot[GT];
@@ -86,7 +87,6 @@ __global__ __launch_bounds__(MAXT) void k_decode_finish(const FinishParams q, co
     }
   };
   using B0 = std::integral_constant<int, 0>;
-  using B1 = std::integral_constant<int, 1>;
   // The shared expert's down matrix is a kernel argument, the routed ones are two dependent loads away (ids, then the slot
   // table): the shared expert's units w, w + nw, ... < P are wave w's first units, and it requests the first of them before
   // anything else, so the first weights are on their way while the block finds out which experts were chosen.
@@ -137,6 +137,7 @@ __global__ __launch_bounds__(MAXT) void k_decode_finish(const FinishParams q, co
     }
     if (tid == 0) {
       s_groups = q.desc->n;
+      s_next = 0;
       if (q.desc->bad && q.status && blockIdx.x == 0) atomicOr(q.status, 1u);
     }
     __syncthreads();
@@ -172,6 +173,7 @@ __global__ __launch_bounds__(MAXT) void k_decode_finish(const FinishParams q, co
       int total = 0;
       for (int c = 0; c < K; ++c) total += s_expert[c] >= 0 ? 1 : 0;
       s_groups = total;
+      s_next = 0;
     }
     __syncthreads();
     nr_ = uni(s_groups);
@@ -200,32 +202,37 @@ __global__ __launch_bounds__(MAXT) void k_decode_finish(const FinishParams q, co
   }
   __syncthreads();
 
-  // this wave's units: the shared expert's units wave, wave + nw, ... first, then a contiguous run of the routed groups'
-  // units (group-major: group g, rows b_lo + NR * i ..). Which wave computes a unit does not change its result.
+  // This wave's units: the shared expert's units wave, wave + nw, ... < P first (the first of them is on its way since
+  // entry), then routed units claimed one at a time from the block's counter (unit u = rows b_lo + NR * (u % P) .. of
+  // group u / P). The two waves of a SIMD do not run at the same pace - the one placed first issues first and, with equal
+  // shares, is done a fifth earlier - so equal shares leave every SIMD with one wave for the last microseconds. Which wave
+  // computes a unit does not change its result.
   const int Ur = nr * P;
-  const int r_lo = Ur * wave / nw, r_hi = Ur * (wave + 1) / nw;
-  const int lead = first_shared ? (P - wave + nw - 1) / nw : 0;  // shared units of this wave
-  const int my_units = lead + (r_hi - r_lo);
-  auto unit_of = [&](int t, int& g, int& i) {  // units past the run name its last unit again; nothing reads those requests
-    const int tc = t < my_units ? t : my_units - 1;
-    if (tc < lead) { g = nr; i = wave + tc * nw; return; }
-    const int r = r_lo + tc - lead;
-    g = r / P;
-    i = r - g * P;
+  auto claim = [&](int& g, int& i) -> bool {
+    int u = 0;
+    if (lane == 0) u = atomicAdd(&s_next, 1);
+    u = uni(u);
+    if (u >= Ur) return false;
+    g = u / P;
+    i = u - g * P;
+    return true;
   };
-  auto issue_unit = [&](auto which, int t, int s) {
-    int g, i;
-    unit_of(t, g, i);
-    issue_rows(which, uni64(s_codes[g]), uni64(s_scales[g]), unif(s_glob[g]), i, s, t >= my_units);
+  // the unit after (g, i): the wave's next shared unit, else a claim
+  auto next_unit = [&](int& g, int& i) -> bool {
+    if (!MIXED && g == nr && first_shared && i + nw < P) { i += nw; return true; }
+    return claim(g, i);
   };
-  if (my_units > 0) {
-    if (!first_shared || (MIXED && my_units > lead)) {  // MIXED: the first routed unit goes out next to the shared ones, into its own registers
+  auto issue_unit = [&](auto which, int g, int i, int s, bool spare) {
+    issue_rows(which, uni64(s_codes[g]), uni64(s_scales[g]), unif(s_glob[g]), i, s, spare);
+  };
+  // (ug, ui): the unit whose rows are in flight in buf
+  int ug = nr, ui = wave;
+  bool uvalid = first_shared && !MIXED;
+  if (!uvalid) {
+    uvalid = claim(ug, ui);  // MIXED: the first routed unit goes out next to the shared ones, into its own registers
+    if (uvalid) {
 #pragma unroll
-      for (int s = 0; s < S; ++s) issue_unit(B0{}, MIXED ? lead : 0, s);
-    }
-    if constexpr (NB == 2) {
-#pragma unroll
-      for (int s = 0; s < S; ++s) issue_unit(B1{}, 1, s);
+      for (int s = 0; s < S; ++s) issue_unit(B0{}, ug, ui, s, false);
     }
   }
   // NVFP4: the split dot's constants of every group's down matrix; then the activations, which were requested first
@@ -234,31 +241,9 @@ __global__ __launch_bounds__(MAXT) void k_decode_finish(const FinishParams q, co
   }
   stage_activations();
   __syncthreads();
-  auto unit = [&](auto which, int t) {
-    constexpr int b_ = decltype(which)::value;
-    int g, i;
-    unit_of(t, g, i);
-    const int arow = uni(s_slot[g]);  // the group's activation row in LDS (arena order)
-    float acc[NR][1];
-#pragma unroll
-    for (int m = 0; m < NR; ++m) acc[m][0] = 0.0f;
-#pragma unroll
-    for (int s = 0; s < S; ++s) {
-      step_compute<F, NR, 1, S, NV>(buf[b_], s, xs + size_t(arow) * I * 2, I, nchunks, s * 64 + lane, 1, acc, s_lut + (NV ? g * FmtNvfp4::LUT_ENTRIES : 0));
-      issue_unit(which, t + NB, s);
-    }
-    float total[NR];
-#pragma unroll
-    for (int m = 0; m < NR; ++m) total[m] = wave_sum(acc[m][0]);
-    if (lane == 0) {
-#pragma unroll
-      for (int m = 0; m < NR; ++m)
-        if (i * NR + m < C) s_part[g * cmax + i * NR + m] = total[m];
-    }
-  };
-  int t_first = 0;
   if constexpr (MIXED) {
     // the shared expert's units of this wave in their own format; the first routed unit is already on its way
+    const int lead = first_shared ? (P - wave + nw - 1) / nw : 0;
     for (int t = 0; t < lead; ++t) {
       const int i = wave + t * nw;
       float acc[NR][1];
@@ -278,13 +263,29 @@ __global__ __launch_bounds__(MAXT) void k_decode_finish(const FinishParams q, co
           if (i * NR + m < C) s_part[nr * cmax + i * NR + m] = total[m];
       }
     }
-    t_first = lead;
   }
-  for (int t = t_first; t < my_units; t += NB) {
-    unit(B0{}, t);
-    if constexpr (NB == 2) {
-      if (t + 1 < my_units) unit(B1{}, t + 1);
+  while (uvalid) {
+    int ng = ug, ni = ui;
+    const bool nvalid = next_unit(ng, ni);
+    const int arow = uni(s_slot[ug]);  // the group's activation row in LDS (arena order)
+    float acc[NR][1];
+#pragma unroll
+    for (int m = 0; m < NR; ++m) acc[m][0] = 0.0f;
+#pragma unroll
+    for (int s = 0; s < S; ++s) {
+      step_compute<F, NR, 1, S, NV>(buf[0], s, xs + size_t(arow) * I * 2, I, nchunks, s * 64 + lane, 1, acc, s_lut + (NV ? ug * FmtNvfp4::LUT_ENTRIES : 0));
+      // behind the last unit a request that nothing reads keeps the loop free of branches around its loads
+      issue_unit(B0{}, nvalid ? ng : ug, nvalid ? ni : ui, s, !nvalid);
     }
+    float total[NR];
+#pragma unroll
+    for (int m = 0; m < NR; ++m) total[m] = wave_sum(acc[m][0]);
+    if (lane == 0) {
+#pragma unroll
+      for (int m = 0; m < NR; ++m)
+        if (ui * NR + m < C) s_part[ug * cmax + ui * NR + m] = total[m];
+    }
+    ug = ng; ui = ni; uvalid = nvalid;
   }
   __syncthreads();
   // ordered combine of the block's columns
