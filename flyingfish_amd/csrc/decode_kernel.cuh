@@ -140,6 +140,7 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
     }
   };
   bool sel_inside = false;  // the selection ran inside the shared slice's staging, in front of its barrier
+  int slice_first_units = 0;  // > 0 while the block's first routed segment is dealt out: the units of its shared slice
   // Wave 0 selects inside the shared slice's staging, between asking for its share of the token row and writing it to LDS:
   // the slice's first barrier is dropped (nothing has read the token buffer yet; the other waves reach it only once the
   // memory pipeline has taken their first weight requests, microseconds after entry), so wave 0 asks for its share and
@@ -222,7 +223,20 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
     const int nchunks = Kg / FF::EPL;
     const int nslabs = (nchunks + SS * 64 - 1) / (SS * 64);
     // this wave's contiguous run of units inside the segment
-    const int w_lo = wv >= 0 ? count * wv / nw : 0, w_hi = wv >= 0 ? count * (wv + 1) / nw : 0;
+    int w_lo = wv >= 0 ? count * wv / nw : 0, w_hi = wv >= 0 ? count * (wv + 1) / nw : 0;
+    if (slice_first_units > 0 && wv >= 0 && nw == 4) {
+      // the block's first routed segment behind its slice of the shared expert: shares that even out slice units plus
+      // routed units per wave (wave 0 took no slice unit and has been streaming routed rows since the selection, the
+      // wave with two slice units starts last) - 9 / 8 / 8 / 7 units for a slice of 4 and 32 routed units
+      const int all = count + slice_first_units;
+      auto cut = [&](int w) {  // routed units of the waves below w
+        const int slice_below = w == 0 ? 0 : slice_first_units * (w - 1) / 3;
+        const int c = all * w / 4 - slice_below;
+        return c < 0 ? 0 : (c > count ? count : c);
+      };
+      w_lo = cut(wv); w_hi = wv == 3 ? count : cut(wv + 1);
+      if (w_hi < w_lo) w_hi = w_lo;
+    }
     const int my_units = gn > 0 ? w_hi - w_lo : 0;
     const int items = my_units * nslabs;
     const int jw = j0 + w_lo;  // first unit of the run
@@ -358,6 +372,7 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
       // this block's slice of the shared expert (group A: rows == 1), waves 1..3; wave 0 selects meanwhile
       const int s_lo = int((long long)out_s * blockIdx.x / gridDim.x), s_hi = int((long long)out_s * (blockIdx.x + 1) / gridDim.x);
       segment(SegmentKind<FSH, SSH>{}, A, s_lo, s_hi - s_lo, 3, wave - 1, nullptr, false, select_early);
+      if (EARLY && sel_inside) slice_first_units = s_hi - s_lo;
     }
     if (inline_route) {
       if (!EARLY && wave == 0 && preloaded) select_preloaded();
@@ -409,6 +424,7 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
     segment(SegmentKind<F, S>{}, g, j0, int(seg_end - u0), 4, wave, inline_route ? s_route_ids : nullptr,
             STAGE == 0 && RG == 1 && shared_first && p.rows == 1 && g < A);
     u0 = seg_end;
+    slice_first_units = 0;
   }
 }
 
