@@ -87,6 +87,12 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
   // NVFP4: the split dot's constants per scale code, one table per matrix of the segment (gate, up | down)
   constexpr bool NV = std::is_same<F, FmtNvfp4>::value || std::is_same<FSH, FmtNvfp4>::value;
   __shared__ u32x2 s_lut[NV ? 2 * FmtNvfp4::LUT_ENTRIES : 1];
+  // One token with NVFP4 experts: behind the shared slice every wave keeps tables of its own for its routed segments (a wave
+  // builds them with its own lanes, so nothing has to wait for anything) and picks up the selection from a flag of wave 0
+  // instead of a block barrier: a wave starts on its routed rows as soon as it is done with its own slice units.
+  constexpr bool FREE = NV && STAGE == 0 && RG == 1;
+  __shared__ u32x2 s_lut_wave[FREE ? 4 * 2 * FmtNvfp4::LUT_ENTRIES : 1];
+  __shared__ int s_selected;
   const bool inline_route = STAGE == 0 && RG == 1 && p.route.logits != nullptr;
   // With a shared expert the selection hides behind it: its units need no routing, so every block first takes its slice
   // of the shared expert's rows on waves 1..3 while wave 0 selects, and the routed units follow once the ids are known.
@@ -140,6 +146,8 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
     }
   };
   bool sel_inside = false;  // the selection ran inside the shared slice's staging, in front of its barrier
+  const bool free_run = FREE && preloaded && p.rows == 1;  // block-uniform
+  if (free_run && tid == 0) s_selected = 0;  // in front of the slice's barriers; read behind them
   int slice_first_units = 0;  // > 0 while the block's first routed segment is dealt out: the units of its shared slice
   // Wave 0 selects inside the shared slice's staging, between asking for its share of the token row and writing it to LDS:
   // the slice's first barrier is dropped (nothing has read the token buffer yet; the other waves reach it only once the
@@ -256,7 +264,17 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
       for (int s = 0; s < SS; ++s) issue_step(0, s);
     }
     // activations of the group -> LDS (row r at r*Kg*2), behind the first weight requests
-    const bool skip_staging = staged && !NVF;  // wave-uniform, block-uniform
+    const bool own_tables = FREE && NVF && staged && free_run;  // block-uniform
+    const bool skip_staging = staged && (!NVF || own_tables);  // wave-uniform, block-uniform
+    const u32x2* lut = s_lut;
+    if constexpr (FREE && NVF) {
+      if (own_tables && gn > 0) {
+        u32x2* mine = s_lut_wave + wave * 2 * FmtNvfp4::LUT_ENTRIES;
+        FmtNvfp4::build_lut(mine, global[0], lane, 64);
+        FmtNvfp4::build_lut(mine + FmtNvfp4::LUT_ENTRIES, global[1], lane, 64);
+        lut = mine;
+      }
+    }
     if (!skip_staging && !with_select) __syncthreads();  // the previous segment's readers are done with xs
     if (gn > 0 && !skip_staging) {
       const uint16_t* src = STAGE == 0 ? p.x : p.h;
@@ -334,7 +352,7 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
       };
       auto compute_step = [&](int t, int s) {
         const int chunk = (t % nslabs) * (SS * 64) + s * 64 + lane;
-        step_compute<FF, NROWS, RG, SS, NVF>(buf, s, xs, Kg, nchunks, chunk, gn, acc, s_lut, s_lut + (NVF ? FmtNvfp4::LUT_ENTRIES : 0), NR);
+        step_compute<FF, NROWS, RG, SS, NVF>(buf, s, xs, Kg, nchunks, chunk, gn, acc, lut, lut + (NVF ? FmtNvfp4::LUT_ENTRIES : 0), NR);
       };
       auto item_end = [&](int t) {
         const int unit = t / nslabs;
@@ -372,14 +390,21 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
       // this block's slice of the shared expert (group A: rows == 1), waves 1..3; wave 0 selects meanwhile
       const int s_lo = int((long long)out_s * blockIdx.x / gridDim.x), s_hi = int((long long)out_s * (blockIdx.x + 1) / gridDim.x);
       segment(SegmentKind<FSH, SSH>{}, A, s_lo, s_hi - s_lo, 3, wave - 1, nullptr, false, select_early);
-      if (EARLY && sel_inside) slice_first_units = s_hi - s_lo;
+      if ((EARLY && sel_inside) || free_run) slice_first_units = s_hi - s_lo;
     }
     if (inline_route) {
-      if (!EARLY && wave == 0 && preloaded) select_preloaded();
-      else if (wave == 0 && !sel_inside)
+      if (!EARLY && wave == 0 && preloaded) {
+        select_preloaded();
+        if (free_run && lane == 0) s_selected = 1;  // behind the ids and weights: a wave's LDS writes land in program order
+      } else if (wave == 0 && !sel_inside)
         wave_route_dispatch(p.route.logits, p.route.bias, lane, p.experts, select_k, p.route.score_mode, p.route.routed_scaling,
                             p.route.n_group, p.route.topk_group, s_route_ids, s_route_w, 1);
-      if (!sel_inside) __syncthreads();
+      if (free_run) {
+        // bounded by wave 0, which selects right behind the slice's staging barrier
+        while (uni(*reinterpret_cast<volatile int*>(&s_selected)) == 0) __builtin_amdgcn_s_sleep(1);
+      } else if (!sel_inside) {
+        __syncthreads();
+      }
       if (blockIdx.x == 0 && tid < select_k) {
         const_cast<int*>(p.ids)[tid] = s_route_ids[tid];
         reinterpret_cast<float*>(const_cast<void*>(p.weights))[tid] = s_route_w[tid];
