@@ -91,7 +91,7 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
   // builds them with its own lanes, so nothing has to wait for anything) and picks up the selection from a flag of wave 0
   // instead of a block barrier: a wave starts on its routed rows as soon as it is done with its own slice units.
   constexpr bool FREE = NV && STAGE == 0 && RG == 1;
-  __shared__ u32x2 s_lut_wave[FREE ? 4 * 2 * FmtNvfp4::LUT_ENTRIES : 1];
+  __shared__ u32x2 s_lut_wave[FREE && NV ? 4 * 2 * FmtNvfp4::LUT_ENTRIES : 1];
   __shared__ int s_selected;
   const bool inline_route = STAGE == 0 && RG == 1 && p.route.logits != nullptr;
   // With a shared expert the selection hides behind it: its units need no routing, so every block first takes its slice
@@ -154,7 +154,7 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
   // memory pipeline has taken their first weight requests, microseconds after entry), so wave 0 asks for its share and
   // selects while the other waves' shares are still behind their weight rows, and the barrier behind the staging is also the
   // one behind the selection.
-  constexpr bool EARLY = !NV;
+  constexpr bool EARLY = !FREE;
   const bool select_early = EARLY && preloaded;
 
   // One segment: `count` units of group g from unit j0 on, split over the waves wv = 0 .. nw-1 (wv < 0: this wave only
