@@ -87,10 +87,15 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
   // NVFP4: the split dot's constants per scale code, one table per matrix of the segment (gate, up | down)
   constexpr bool NV = std::is_same<F, FmtNvfp4>::value || std::is_same<FSH, FmtNvfp4>::value;
   __shared__ u32x2 s_lut[NV ? 2 * FmtNvfp4::LUT_ENTRIES : 1];
-  // One token with NVFP4 experts: behind the shared slice every wave keeps tables of its own for its routed segments (a wave
-  // builds them with its own lanes, so nothing has to wait for anything) and picks up the selection from a flag of wave 0
-  // instead of a block barrier: a wave starts on its routed rows as soon as it is done with its own slice units.
-  constexpr bool FREE = NV && STAGE == 0 && RG == 1;
+  // One token with the selection in this launch (256 experts, a shared expert): no block barrier behind the slice's first
+  // one. Wave 0 selects as soon as its logits are there and hands the choices over through a flag in LDS; the other waves
+  // stage the token row, compute their slice units and pick the flag up when they are done - a wave starts on its routed
+  // rows as soon as its own slice units are finished. FP8 / BF16 rows: the token row is staged by the three slice waves
+  // alone, counted in s_staged (with wave 0 in that barrier either it waits four microseconds for rows it does not need
+  // before it may select, or the slice waves wait for the selection). NVFP4 rows: every wave keeps split-dot tables of
+  // its own for its routed segments, built with its own lanes, so those segments need no barrier either.
+  constexpr bool FREE = STAGE == 0 && RG == 1;
+  __shared__ int s_staged;  // slice waves whose share of the token row is in LDS
   __shared__ u32x2 s_lut_wave[FREE && NV ? 4 * 2 * FmtNvfp4::LUT_ENTRIES : 1];
   __shared__ int s_selected;
   const bool inline_route = STAGE == 0 && RG == 1 && p.route.logits != nullptr;
@@ -145,23 +150,16 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
       wave_select_pick<PC>(sel, lane, select_k, p.route.routed_scaling, s_route_ids, s_route_w, 1);
     }
   };
-  bool sel_inside = false;  // the selection ran inside the shared slice's staging, in front of its barrier
+  bool slice3_used = false;  // the slice's token row was staged by the three slice waves alone, counted in s_staged
   const bool free_run = FREE && preloaded && p.rows == 1;  // block-uniform
-  if (free_run && tid == 0) s_selected = 0;  // in front of the slice's barriers; read behind them
+  if (free_run && tid == 0) { s_selected = 0; s_staged = 0; }  // in front of the slice's first barrier; read behind it
   int slice_first_units = 0;  // > 0 while the block's first routed segment is dealt out: the units of its shared slice
-  // Wave 0 selects inside the shared slice's staging, between asking for its share of the token row and writing it to LDS:
-  // the slice's first barrier is dropped (nothing has read the token buffer yet; the other waves reach it only once the
-  // memory pipeline has taken their first weight requests, microseconds after entry), so wave 0 asks for its share and
-  // selects while the other waves' shares are still behind their weight rows, and the barrier behind the staging is also the
-  // one behind the selection.
-  constexpr bool EARLY = !FREE;
-  const bool select_early = EARLY && preloaded;
 
   // One segment: `count` units of group g from unit j0 on, split over the waves wv = 0 .. nw-1 (wv < 0: this wave only
   // takes part in the staging and the barriers).
   // staged: the group's activation row is in LDS already (one token: the routed segments behind the shared slice read the
   // same token row) - no second copy behind the segment's first weight requests, and without a table to build no barrier
-  auto segment = [&](auto kind, int g, int j0, int count, int nw, int wv, const int* inline_ids, bool staged = false, bool with_select = false) {
+  auto segment = [&](auto kind, int g, int j0, int count, int nw, int wv, const int* inline_ids, bool staged = false, bool slice_free = false) {
     using FF = typename decltype(kind)::fmt;
     constexpr int SS = decltype(kind)::steps;
     constexpr bool NVF = std::is_same<FF, FmtNvfp4>::value;
@@ -266,6 +264,8 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
     // activations of the group -> LDS (row r at r*Kg*2), behind the first weight requests
     const bool own_tables = FREE && NVF && staged && free_run;  // block-uniform
     const bool skip_staging = staged && (!NVF || own_tables);  // wave-uniform, block-uniform
+    const bool slice3 = FREE && !NV && slice_free && gn == 1;  // block-uniform
+    if (slice3) slice3_used = true;  // block-uniform
     const u32x2* lut = s_lut;
     if constexpr (FREE && NVF) {
       if (own_tables && gn > 0) {
@@ -275,7 +275,7 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
         lut = mine;
       }
     }
-    if (!skip_staging && !with_select) __syncthreads();  // the previous segment's readers are done with xs
+    if (!skip_staging) __syncthreads();  // the previous segment's readers are done with xs
     if (gn > 0 && !skip_staging) {
       const uint16_t* src = STAGE == 0 ? p.x : p.h;
       const int row_words = Kg >> 3;  // 16-byte words per row
@@ -284,21 +284,12 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
         if (r < gn && !staged) {
           const size_t base = STAGE == 0 ? size_t(grow[r]) * p.hidden : size_t(gslot[r]) * p.h_stride;
           u32x4* d4 = reinterpret_cast<u32x4*>(xs + size_t(r) * Kg * 2);
-          if (EARLY && RG == 1 && with_select) sel_inside = true;  // block-uniform
-          if (EARLY && RG == 1 && with_select && wave == 0) {
-            // wave 0: its share of the row is asked for (rows of up to 8192 values: held in registers), then it selects,
-            // then the share goes to LDS
-            const bool in_regs = row_words <= 1024;
-            u32x4 st[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-              if (in_regs && tid + 256 * i < row_words) st[i] = load16(src + base + size_t(tid + 256 * i) * 8);
-            select_preloaded();
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-              if (in_regs && tid + 256 * i < row_words) d4[tid + 256 * i] = st[i];
-            if (!in_regs)
-              for (int v = tid; v < row_words; v += 256) d4[v] = load16(src + base + size_t(v) * 8);
+          if (slice3) {
+            // the three slice waves stage the row; the selecting wave takes no part and does not wait for it here
+            if (wave != 0) {
+              for (int v = tid - 64; v < row_words; v += 192) d4[v] = load16(src + base + size_t(v) * 8);
+              if (lane == 0) atomicAdd(&s_staged, 1);  // behind the wave's writes: its LDS operations land in program order
+            }
           } else {
             for (int v = tid; v < row_words; v += 256) d4[v] = load16(src + base + size_t(v) * 8);
           }
@@ -309,7 +300,12 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
         if (STAGE == 0) FmtNvfp4::build_lut(s_lut + FmtNvfp4::LUT_ENTRIES, global[1], tid, 256);
       }
     }
-    if (!skip_staging) __syncthreads();
+    if (slice3) {
+      // bounded by the other slice waves, which are on their way to the same point
+      if (wave != 0) while (uni(*reinterpret_cast<volatile int*>(&s_staged)) < 3) __builtin_amdgcn_s_sleep(1);
+    } else if (!skip_staging) {
+      __syncthreads();
+    }
     if (items > 0) {
       float acc[NROWS][RG];
       float park[NROWS][RG];  // lane L keeps the sums of unit (batch base + L)
@@ -389,20 +385,22 @@ __global__ __launch_bounds__(256) void k_decode_stage(const DecodeParams p) {
     if (shared_first) {
       // this block's slice of the shared expert (group A: rows == 1), waves 1..3; wave 0 selects meanwhile
       const int s_lo = int((long long)out_s * blockIdx.x / gridDim.x), s_hi = int((long long)out_s * (blockIdx.x + 1) / gridDim.x);
-      segment(SegmentKind<FSH, SSH>{}, A, s_lo, s_hi - s_lo, 3, wave - 1, nullptr, false, select_early);
-      if ((EARLY && sel_inside) || free_run) slice_first_units = s_hi - s_lo;
+      segment(SegmentKind<FSH, SSH>{}, A, s_lo, s_hi - s_lo, 3, wave - 1, nullptr, false, free_run);
+      if (free_run) slice_first_units = s_hi - s_lo;
     }
     if (inline_route) {
-      if (!EARLY && wave == 0 && preloaded) {
+      if (wave == 0 && preloaded) {
         select_preloaded();
         if (free_run && lane == 0) s_selected = 1;  // behind the ids and weights: a wave's LDS writes land in program order
-      } else if (wave == 0 && !sel_inside)
+      } else if (wave == 0)
         wave_route_dispatch(p.route.logits, p.route.bias, lane, p.experts, select_k, p.route.score_mode, p.route.routed_scaling,
                             p.route.n_group, p.route.topk_group, s_route_ids, s_route_w, 1);
       if (free_run) {
         // bounded by wave 0, which selects right behind the slice's staging barrier
         while (uni(*reinterpret_cast<volatile int*>(&s_selected)) == 0) __builtin_amdgcn_s_sleep(1);
-      } else if (!sel_inside) {
+        // the selecting wave took no part in the staging of the slice: the row has to be there before its routed units
+        if (slice3_used && wave == 0) while (uni(*reinterpret_cast<volatile int*>(&s_staged)) < 3) __builtin_amdgcn_s_sleep(1);
+      } else {
         __syncthreads();
       }
       if (blockIdx.x == 0 && tid < select_k) {
