@@ -24,7 +24,7 @@ HBM_PEAK_GBPS = 8000.0
 # HBM bytes per gate/up launch, not read in the run: FETCH_SIZE and WRITE_SIZE of rocprofv3 --pmc runs of this script, each
 # scaled by what the same counter reads for a 256 MiB plain copy (--calibrate-copy); keyed by (batch, experts). Source of
 # the figure, with the commands: profiles/decode_layer_fp8_c3_batch1.hbm_traffic.txt. Other workloads report null.
-GATE_UP_TRAFFIC_BYTES = {(1, 256): 265437700}
+GATE_UP_TRAFFIC_BYTES = {(1, 256): 265451800}
 TRAFFIC_SOURCE = "profiles/decode_layer_fp8_c3_batch1.hbm_traffic.txt"
 # W8A8 gate/up launch of the default prefill cohort (4096 tokens, 256 experts, seed 20251): FETCH_SIZE x 1.99977 + WRITE_SIZE
 PREFILL_GATE_UP_TRAFFIC_BYTES = 9190000000 + 135000000
