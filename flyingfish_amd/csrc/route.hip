@@ -13,11 +13,11 @@ namespace ffmoe {
 // (kernels/moe_route.cu:392-403, :536-544): 2 * hidden dependent fmas, serial by contract. What the lane must not also
 // do is fetch its router row itself - 64 lanes reading 16 bytes each of 64 different rows is 64 cache lines per load
 // instruction, and that, not the chain, was the kernel's time (22.8 us for 64 experts x 2048). A block is five waves: four
-// of them move the router tile of 64 experts x 256 columns and the token row's 256 columns through LDS with coalesced
-// requests (32 lanes per 512-byte row segment), one chunk ahead, and wave 0 does nothing but run the 64 chains out of LDS
-// (rows padded by 16 bytes, so the 16 lanes of a quarter wave read 16 different LDS slots). A dependent v_fma_f32 takes 8
-// cycles on this machine and 10 with its operands arriving from LDS (2048 of them: 8.6 and 10.5 us), whatever the row
-// stride and whether the token row comes through LDS or scalar registers; the chain wave is kept clear of everything else.
+// of them move the router tile of 64 experts x 256 columns through LDS with coalesced requests (32 lanes per 512-byte row
+// segment), one chunk ahead, multiplied by the token's values on the way (see the kernel), and wave 0 does nothing but run
+// the 64 chains out of LDS (rows padded by 16 bytes, so the 16 lanes of a quarter wave read 16 different LDS slots). A
+// dependent FP32 add or fma takes 8 cycles on this machine; fed from LDS the chain runs at 8.7 cycles per element with one
+// operand per element and at 12.1 with two (2048 elements: 7.5 and 10.3 us); the chain wave is kept clear of everything else.
 __device__ __forceinline__ int rank_of(const float* s_key, int padded, float mine, int e);
 
 // Softmax / sigmoid top-k of at most 64 experts by the wave whose lane e holds expert e's BF16 logit: the arithmetic of
@@ -77,9 +77,14 @@ template <bool SELECT>
 __global__ __launch_bounds__(320) void k_route_logits_bf16(const uint16_t* __restrict__ x, const uint16_t* __restrict__ router,
                                                            uint16_t* __restrict__ logits, int rows, int experts, int hidden,
                                                            int* __restrict__ ids, uint16_t* __restrict__ weights, int top_k, int score_mode) {
-  // 64 router rows + the token row, widened to FP32 by the waves that move them: the chain wave's instruction stream is
-  // then one LDS read per four elements and operand plus the fmas themselves, no unpacking in front of every fma
-  __shared__ __attribute__((aligned(16))) uint8_t tile[2][65 * LOGIT_ROW_BYTES];
+  // The waves that move the router tile leave PRODUCTS in LDS: x[k] * w[e][k] of two BF16 values has at most 16 significant
+  // bits and is exact in FP32 unless it falls below the normal range, and then fma(x, w, acc) = acc + product, one rounding
+  // either way. The chain wave's step is one dependent add with one LDS operand per four elements (8.7 cycles per element
+  // against 12.1 for the fma with the token and the router element read separately). A product that is zero or subnormal -
+  // an exact zero in the token or the router, or an underflow - flags its chunk, and the chain wave then runs that chunk
+  // as fmas on the BF16 values themselves: the same bits for every input.
+  __shared__ __attribute__((aligned(16))) uint8_t tile[2][64 * LOGIT_ROW_BYTES];
+  __shared__ int s_inexact[2];
   const int lane = threadIdx.x & 63, wave = uni(int(threadIdx.x >> 6));
   const int tid = int(threadIdx.x) - 64;                  // index among the 256 moving threads (wave 0: negative, moves nothing)
   const bool mover = wave != 0;
@@ -87,9 +92,10 @@ __global__ __launch_bounds__(320) void k_route_logits_bf16(const uint16_t* __res
   const int row = blockIdx.y;
   const int words = hidden >> 3;                          // 16-byte pieces (8 columns) per row
   const int chunks = (words + 31) >> 5;
-  // piece (r, q) of a chunk for i = 0 .. 7: r = (tid + 256 i) / 32, q = (tid + 256 i) % 32; thread tid < 32 also moves piece tid
-  // of the token row. Pieces past the end of the row repeat its last piece; nothing multiplies them.
-  // The movers run two chunks ahead in two register sets (chunk c in set c % 2): a chunk's chains take about 1.3 us, less than a
+  // piece (r, q) of a chunk for i = 0 .. 7: r = (tid + 256 i) / 32, q = (tid + 256 i) % 32 = tid % 32: a thread moves the same
+  // eight columns of eight router rows and needs the token's eight values of those columns. Pieces past the end of the row
+  // repeat its last piece; nothing adds them.
+  // The movers run two chunks ahead in two register sets (chunk c in set c % 2): a chunk's chains take about 0.9 us, less than a
   // request that misses the caches.
   u32x4 regs[2][8], xreg[2];
   auto request = [&](auto set, int c) {
@@ -102,25 +108,38 @@ __global__ __launch_bounds__(320) void k_route_logits_bf16(const uint16_t* __res
       const int piece = min(32 * c + q, words - 1);
       regs[S][i] = load16(router + size_t(er) * hidden + size_t(piece) * 8);
     }
-    if (tid < 32) xreg[S] = load16(x + size_t(row) * hidden + size_t(min(32 * c + tid, words - 1)) * 8);
-  };
-  auto widen = [&](uint8_t* dst, const u32x4& v) {
-    const u32x4 lo = {__float_as_uint(bf16lo(v[0])), __float_as_uint(bf16hi(v[0])), __float_as_uint(bf16lo(v[1])), __float_as_uint(bf16hi(v[1]))};
-    const u32x4 hi = {__float_as_uint(bf16lo(v[2])), __float_as_uint(bf16hi(v[2])), __float_as_uint(bf16lo(v[3])), __float_as_uint(bf16hi(v[3]))};
-    *reinterpret_cast<u32x4*>(dst) = lo;
-    *reinterpret_cast<u32x4*>(dst + 16) = hi;
+    xreg[S] = load16(x + size_t(row) * hidden + size_t(min(32 * c + (tid & 31), words - 1)) * 8);
   };
   auto publish = [&](auto set) {  // chunk c sits in set c % 2 and goes to buffer c % 2
     constexpr int S = decltype(set)::value;
+    float xf[8];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) { xf[2 * j] = bf16lo(xreg[S][j]); xf[2 * j + 1] = bf16hi(xreg[S][j]); }
+    float smallest = INFINITY;  // of the products' magnitudes
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const int idx = tid + 256 * i;
-      widen(&tile[S][(idx >> 5) * LOGIT_ROW_BYTES + (idx & 31) * 32], regs[S][i]);
+      const u32x4 v = regs[S][i];
+      float pr[8];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        pr[2 * j] = __fmul_rn(xf[2 * j], bf16lo(v[j]));
+        pr[2 * j + 1] = __fmul_rn(xf[2 * j + 1], bf16hi(v[j]));
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) smallest = fminf(smallest, fabsf(pr[j]));
+      uint8_t* dst = &tile[S][(idx >> 5) * LOGIT_ROW_BYTES + (idx & 31) * 32];
+      const u32x4 lo = {__float_as_uint(pr[0]), __float_as_uint(pr[1]), __float_as_uint(pr[2]), __float_as_uint(pr[3])};
+      const u32x4 hi = {__float_as_uint(pr[4]), __float_as_uint(pr[5]), __float_as_uint(pr[6]), __float_as_uint(pr[7])};
+      *reinterpret_cast<u32x4*>(dst) = lo;
+      *reinterpret_cast<u32x4*>(dst + 16) = hi;
     }
-    if (tid < 32) widen(&tile[S][64 * LOGIT_ROW_BYTES + tid * 32], xreg[S]);
+    if (smallest < 1.17549435e-38f) s_inexact[S] = 1;  // a zero or a subnormal product
   };
   using S0 = std::integral_constant<int, 0>;
   using S1 = std::integral_constant<int, 1>;
+  if (threadIdx.x < 2) s_inexact[threadIdx.x] = 0;
+  __syncthreads();
   if (mover) {
     request(S0{}, 0);
     if (chunks > 1) request(S1{}, 1);
@@ -135,15 +154,28 @@ __global__ __launch_bounds__(320) void k_route_logits_bf16(const uint16_t* __res
       if (c + 1 < chunks) publish(other);
       if (c + 3 < chunks) request(other, c + 3);
     } else {
-      const uint8_t* wrow = &tile[c & 1][lane * LOGIT_ROW_BYTES];
-      const uint8_t* xrow = &tile[c & 1][64 * LOGIT_ROW_BYTES];
       const int nquads = 2 * min(32, words - 32 * c);  // groups of four columns
+      if (uni(s_inexact[c & 1]) == 0) {
+        const uint8_t* prow = &tile[c & 1][lane * LOGIT_ROW_BYTES];
 #pragma unroll 8
-      for (int q = 0; q < nquads; ++q) {
-        const u32x4 wv = *reinterpret_cast<const u32x4*>(wrow + q * 16);
-        const u32x4 xv = *reinterpret_cast<const u32x4*>(xrow + q * 16);
+        for (int q = 0; q < nquads; ++q) {
+          const u32x4 pv = *reinterpret_cast<const u32x4*>(prow + q * 16);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc = __fmaf_rn(__uint_as_float(xv[j]), __uint_as_float(wv[j]), acc);
+          for (int j = 0; j < 4; ++j) acc = __fadd_rn(acc, __uint_as_float(pv[j]));
+        }
+      } else {
+        // a product of this chunk is not exact (or is an exact zero, which looks the same): the fmas on the values themselves
+        const uint16_t* wr = router + size_t(min(e0 + lane, experts - 1)) * hidden + size_t(c) * LOGIT_CHUNK;
+        const uint16_t* xr = x + size_t(row) * hidden + size_t(c) * LOGIT_CHUNK;
+        for (int q = 0; q < nquads; q += 2) {
+          const u32x4 wv = load16(wr + q * 4), xv = load16(xr + q * 4);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            acc = __fmaf_rn(bf16lo(xv[j]), bf16lo(wv[j]), acc);
+            acc = __fmaf_rn(bf16hi(xv[j]), bf16hi(wv[j]), acc);
+          }
+        }
+        if (lane == 0) s_inexact[c & 1] = 0;  // the buffer's next chunk starts clean (the movers write behind the barrier)
       }
     }
     __syncthreads();

@@ -136,6 +136,26 @@ def test_route_logits_bf16_bit_exact(rows, experts, hidden):
     assert np.array_equal(got, orc.route_logits_bf16(bits(x), bits(w)))
 
 
+def test_route_logits_bf16_bit_exact_with_zero_subnormal_and_underflowing_products():
+    """The kernel chains FP32 products of the BF16 values; a product that is zero or below the normal range sends its chunk
+    of 256 columns through fmas on the values themselves. Planted: exact zeros in the token and in the router, products in
+    the subnormal range, products that underflow to zero, and huge values next to them - bit for bit against the oracle."""
+    rows, experts, hidden = 2, 70, 1032
+    x, w = rand_bf16((rows, hidden), 1.0, 13), rand_bf16((experts, hidden), 0.02, 14)
+    x[0, 5] = 0.0                       # an exact zero in the token: chunk 0 of row 0
+    w[3, 300] = 0.0                     # an exact zero in the router: chunk 1, both rows
+    x[1, 600], w[:, 600] = 2.0 ** -70, (torch.arange(experts, dtype=torch.float32) + 1.0).to(torch.bfloat16) * 2.0 ** -62  # subnormal products
+    x[1, 601], w[:, 601] = 2.0 ** -100, 2.0 ** -90                                                      # underflow to zero
+    x[1, 602], w[:, 602] = -(2.0 ** -120), 2.0 ** -20                                                   # tiny, sign
+    x[0, 800], w[:, 800] = 3.0e38, 1.0e-38                                                              # huge times tiny: normal
+    x[1, 1031], w[7, 1031] = 2.0 ** -64, -(2.0 ** -64)                                                  # last column of the ragged last chunk
+    got = bits(RouteOps.logits_bf16(x.to(DEV), w.to(DEV)))
+    assert np.array_equal(got, orc.route_logits_bf16(bits(x), bits(w)))
+    # and a token row of zeros
+    z = torch.zeros((1, hidden), dtype=torch.bfloat16)
+    assert np.array_equal(bits(RouteOps.logits_bf16(z.to(DEV), w.to(DEV))), orc.route_logits_bf16(bits(z), bits(w)))
+
+
 @pytest.mark.parametrize("rows,experts,hidden", [(1, 256, 7168), (9, 64, 2048), (5, 33, 520),
                                                  # from 96 rows on: the kernel that keeps a tile of router rows in LDS
                                                  (300, 256, 7168), (96, 8, 2048), (97, 33, 520), (203, 50, 4104), (1000, 9, 8), (128, 256, 7168)])
