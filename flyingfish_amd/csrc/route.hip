@@ -570,8 +570,14 @@ __global__ __launch_bounds__(64) void k_route_topk_noaux_wave(const float* __res
   if (done && lane < top_k) done[size_t(row) * top_k + lane] = 0u;  // the contribution of this row starts from a clean slate
   void* wrow = weights_f32 ? (void*)(reinterpret_cast<float*>(weights) + size_t(row) * top_k)
                            : (void*)(reinterpret_cast<uint16_t*>(weights) + size_t(row) * top_k);
-  wave_route_dispatch(logits + size_t(row) * experts, bias ? bias + size_t(row) * bias_row_stride : nullptr, lane, experts, top_k,
-                      score_mode, routed_scaling, n_group, topk_group, ids + size_t(row) * top_k, wrow, weights_f32);
+  const float* brow = bias ? bias + size_t(row) * bias_row_stride : nullptr;
+  // the usual router (256 experts in 8 groups of which 4 stay, sigmoid scores, 8 picks) with its numbers as literals: two
+  // thirds of the general selection's instructions, the same ids and weights
+  if (experts == 256 && top_k == 8 && n_group == 8 && topk_group == 4 && score_mode == FFMOE_NOAUX_SIGMOID)
+    wave_route_row<4>(logits + size_t(row) * 256, brow, lane, 256, 8, FFMOE_NOAUX_SIGMOID, routed_scaling, 8, 4, ids + size_t(row) * 8, wrow, weights_f32);
+  else
+    wave_route_dispatch(logits + size_t(row) * experts, brow, lane, experts, top_k, score_mode, routed_scaling, n_group, topk_group,
+                        ids + size_t(row) * top_k, wrow, weights_f32);
 }
 
 }  // namespace ffmoe
